@@ -1,0 +1,21 @@
+"""Paged / quantized KV-cache attention ops (the hot path of ``areno.accel`` in the reference).
+
+Re-exports the op surface the reference's inference backend imports
+(``areno/accel/__init__.py:17-21`` there) plus this build's two additions.
+"""
+
+from areno_amd.accel.attention import (
+    areno_causal_attention,
+    areno_paged_cache_write,
+    areno_paged_causal_attention_decode,
+    areno_paged_varlen_causal_attention,
+    areno_varlen_causal_attention,
+)
+
+__all__ = [
+    "areno_causal_attention",
+    "areno_paged_cache_write",
+    "areno_paged_causal_attention_decode",
+    "areno_paged_varlen_causal_attention",
+    "areno_varlen_causal_attention",
+]

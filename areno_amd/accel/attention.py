@@ -1,0 +1,265 @@
+"""Python op surface of the paged / quantized KV-cache attention path.
+
+Drop-in for the ops the reference engine imports from ``areno.accel.attention``
+(``areno/engine/layers/attention_backend/infer.py:25`` there):
+
+* ``areno_paged_causal_attention_decode``  (reference ``areno/accel/attention.py:267-314``)
+* ``areno_varlen_causal_attention``        (reference ``areno/accel/attention.py:186-209``)
+* ``areno_causal_attention``               (reference ``areno/accel/attention.py:121-142``; no engine caller)
+
+with the same positional/keyword arguments, defaults (``window_left=None`` -> no window,
+``softmax_scale=None`` -> ``head_dim ** -0.5``, l.17-22 there) and error behaviour
+(non-GPU tensor -> ``RuntimeError``; wrong rank or non-int32 metadata -> ``ValueError``;
+everything else -> ``RuntimeError`` from the extension's checks).  Keyword-only additions, all
+defaulting to the reference behaviour:
+
+* ``k_scale`` / ``v_scale`` on the decode op: per-(token, kv head) scale pools ``[NB, bs, Hkv]``
+  for ``int8`` / ``float8_e4m3fn`` caches; the fused cache append then quantizes ``k_update``/``v_update``.
+* ``areno_paged_cache_write``: the prefill cache store (``_store_prefill_cache``,
+  ``attention_backend/infer.py:245-263`` there) as one quantize-and-scatter kernel.
+* ``areno_paged_varlen_causal_attention``: causal prefill of new queries over paged KV with a cached
+  context (chunked prefill that re-reads earlier chunks).
+
+Everything runs as HIP kernels through ``areno_amd.accel._areno_accel``; there is no Python
+fallback and no autograd (the ops are used under ``torch.inference_mode``).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from areno_amd.accel._extension import extension as _extension
+
+_QUANTIZED = (torch.int8, torch.float8_e4m3fn)
+
+
+def _window_left(window_left: int | None) -> int:
+    return -1 if window_left is None else int(window_left)
+
+
+def _scale(q: torch.Tensor, softmax_scale: float | None) -> float:
+    return float(softmax_scale if softmax_scale is not None else q.shape[-1] ** -0.5)
+
+
+def _all_on_gpu(*tensors: torch.Tensor | None) -> bool:
+    return all(t.is_cuda for t in tensors if t is not None)
+
+
+def _contig(t: torch.Tensor | None) -> torch.Tensor | None:
+    return None if t is None else t.contiguous()
+
+
+def _check_scales(op: str, cache: torch.Tensor, k_scale, v_scale) -> None:
+    if (k_scale is None) != (v_scale is None):
+        raise ValueError(f"{op} expects k_scale and v_scale together")
+    if cache.dtype in _QUANTIZED and k_scale is None:
+        raise ValueError(f"{op} expects k_scale and v_scale for an int8/float8_e4m3fn cache")
+    if cache.dtype not in _QUANTIZED and k_scale is not None:
+        raise ValueError(f"{op} got scales for an unquantized cache")
+    if k_scale is not None and (k_scale.dim() != 3 or v_scale.dim() != 3):
+        raise ValueError(f"{op} expects scales shaped (num_blocks, block_size, kv_heads)")
+
+
+@torch._dynamo.disable
+def areno_paged_causal_attention_decode(
+    q: torch.Tensor,
+    k_update: torch.Tensor,
+    v_update: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    block_table: torch.Tensor,
+    cache_seqlens: torch.Tensor,
+    *,
+    window_left: int | None = None,
+    num_splits: int = 8,
+    softmax_scale: float | None = None,
+    k_scale: torch.Tensor | None = None,
+    v_scale: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Apply single-token paged-cache causal attention to ``(batch, heads, dim)`` Q.
+
+    Appends ``k_update``/``v_update`` at position ``cache_seqlens[b]`` of each sequence
+    (mutating the caches, and the scale pools for quantized caches, in place), then attends
+    over positions ``[0, cache_seqlens[b]]``.  ``num_splits`` is a hint: ``1`` keeps one
+    partial per row, any other value lets the kernel pick fixed-size KV chunks.
+    """
+    op = "areno_paged_causal_attention_decode"
+    if not _all_on_gpu(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, k_scale, v_scale):
+        raise RuntimeError(f"{op} requires CUDA tensors")
+    if q.dim() != 3:
+        raise ValueError(f"{op} expects q shaped (batch, heads, head_dim)")
+    if k_update.dim() != 3 or v_update.dim() != 3:
+        raise ValueError(f"{op} expects k/v updates shaped (batch, kv_heads, head_dim)")
+    if k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise ValueError(f"{op} expects 4D paged cache tensors")
+    if block_table.dim() != 2 or cache_seqlens.dim() != 1:
+        raise ValueError(f"{op} expects block_table 2D and cache_seqlens 1D")
+    if block_table.dtype != torch.int32 or cache_seqlens.dtype != torch.int32:
+        raise ValueError(f"{op} expects int32 block_table and cache_seqlens")
+    _check_scales(op, k_cache, k_scale, v_scale)
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        # a contiguous copy would silently drop the in-place cache append
+        raise ValueError(f"{op} expects contiguous cache tensors (they are updated in place)")
+    if k_scale is not None and not (k_scale.is_contiguous() and v_scale.is_contiguous()):
+        raise ValueError(f"{op} expects contiguous scale tensors (they are updated in place)")
+    ext = _extension()
+    args = (
+        q.contiguous(), k_update.contiguous(), v_update.contiguous(), k_cache, v_cache,
+        block_table.contiguous(), cache_seqlens.contiguous(),
+        _window_left(window_left), int(num_splits), _scale(q, softmax_scale),
+    )  # fmt: skip
+    if k_scale is None:
+        return ext.areno_paged_causal_attention_decode_forward(*args)
+    return ext.areno_paged_causal_attention_decode_forward_scaled(*args, k_scale, v_scale)
+
+
+@torch._dynamo.disable
+def areno_varlen_causal_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    cu_seqlens: torch.Tensor,
+    *,
+    window_left: int | None = None,
+    softmax_scale: float | None = None,
+) -> torch.Tensor:
+    """Apply packed causal attention to flat ``(tokens, heads, head_dim)`` tensors."""
+    op = "areno_varlen_causal_attention"
+    if not _all_on_gpu(q, k, v, cu_seqlens):
+        raise RuntimeError(f"{op} requires CUDA q, k, v, and cu_seqlens tensors")
+    if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
+        raise ValueError(f"{op} expects q/k/v tensors shaped (tokens, heads, head_dim)")
+    if cu_seqlens.dim() != 1 or cu_seqlens.dtype != torch.int32:
+        raise ValueError(f"{op} expects an int32 1D cu_seqlens tensor")
+    if q.shape[0] != k.shape[0] or q.shape[0] != v.shape[0]:
+        raise ValueError(f"{op} token count mismatch")
+    if k.shape[1] != v.shape[1] or q.shape[1] % k.shape[1] != 0:
+        raise ValueError(f"{op} expects q heads to be divisible by kv heads")
+    if q.shape[2] != k.shape[2] or q.shape[2] != v.shape[2]:
+        raise ValueError(f"{op} head dim mismatch")
+    return _extension().areno_varlen_causal_attention_forward(
+        q.contiguous(), k.contiguous(), v.contiguous(), cu_seqlens.contiguous(),
+        _window_left(window_left), _scale(q, softmax_scale),
+    )  # fmt: skip
+
+
+@torch._dynamo.disable
+def areno_causal_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    *,
+    query_start: int = 0,
+    window_left: int | None = None,
+    softmax_scale: float | None = None,
+) -> torch.Tensor:
+    """Apply causal attention to ``(batch, heads, seqlen, head_dim)`` tensors.
+
+    Served by the paged prefill kernel: ``k``/``v`` are viewed as one page per batch row
+    (``block_size = Sk``) and ``query_start`` becomes the cached-context length, so query ``i``
+    sits at position ``query_start + i``.  Requires ``Sk >= query_start + Sq`` (every position a
+    query may see exists as a key).
+    """
+    op = "areno_causal_attention"
+    if not _all_on_gpu(q, k, v):
+        raise RuntimeError(f"{op} requires CUDA q, k, and v tensors")
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError(f"{op} expects q/k/v tensors shaped (batch, heads, seqlen, head_dim)")
+    if q.shape[0] != k.shape[0] or q.shape[0] != v.shape[0]:
+        raise ValueError(f"{op} batch size mismatch")
+    if q.shape[1] != k.shape[1] or q.shape[1] != v.shape[1]:
+        raise ValueError(f"{op} head count mismatch")
+    if q.shape[-1] != k.shape[-1] or q.shape[-1] != v.shape[-1]:
+        raise ValueError(f"{op} head dim mismatch")
+    batch, heads, sq, _ = q.shape
+    sk = k.shape[2]
+    if sk < int(query_start) + sq:
+        raise ValueError(f"{op} needs at least query_start + q_len = {int(query_start) + sq} keys, got {sk}")
+    q_flat = q.transpose(1, 2).reshape(batch * sq, heads, q.shape[-1]).contiguous()
+    k_pool = k.transpose(1, 2).contiguous()  # (batch, Sk, heads, D): one page per row
+    v_pool = v.transpose(1, 2).contiguous()
+    dev = q.device
+    table = torch.arange(batch, device=dev, dtype=torch.int32).view(batch, 1)
+    cu = torch.arange(batch + 1, device=dev, dtype=torch.int32) * sq
+    ctx = torch.full((batch,), int(query_start), device=dev, dtype=torch.int32)
+    out = _extension().areno_paged_varlen_causal_attention_forward(
+        q_flat, k_pool, v_pool, table, cu, ctx, _window_left(window_left), _scale(q, softmax_scale), None, None
+    )
+    return out.view(batch, sq, heads, q.shape[-1]).transpose(1, 2)
+
+
+@torch._dynamo.disable
+def areno_paged_cache_write(
+    k: torch.Tensor,
+    v: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    cache_block_ids: torch.Tensor,
+    cache_block_offsets: torch.Tensor,
+    *,
+    k_scale: torch.Tensor | None = None,
+    v_scale: torch.Tensor | None = None,
+) -> None:
+    """Store packed ``(tokens, kv_heads, head_dim)`` K/V at ``cache[ids[t], offsets[t]]``, quantizing on the way.
+
+    For ``int8`` / ``float8_e4m3fn`` caches each ``(token, kv head)`` row gets its own scale,
+    written to ``k_scale``/``v_scale`` at the same ``(block, slot)``.
+    """
+    op = "areno_paged_cache_write"
+    if not _all_on_gpu(k, v, k_cache, v_cache, cache_block_ids, cache_block_offsets, k_scale, v_scale):
+        raise RuntimeError(f"{op} requires CUDA tensors")
+    if k.dim() != 3 or v.dim() != 3:
+        raise ValueError(f"{op} expects k/v shaped (tokens, kv_heads, head_dim)")
+    if k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise ValueError(f"{op} expects 4D paged cache tensors")
+    if cache_block_ids.dim() != 1 or cache_block_offsets.dim() != 1:
+        raise ValueError(f"{op} expects 1D cache_block_ids and cache_block_offsets")
+    if cache_block_ids.dtype != torch.int64 or cache_block_offsets.dtype != torch.int64:
+        raise ValueError(f"{op} expects int64 cache_block_ids and cache_block_offsets")
+    _check_scales(op, k_cache, k_scale, v_scale)
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError(f"{op} expects contiguous cache tensors (they are updated in place)")
+    if k_scale is not None and not (k_scale.is_contiguous() and v_scale.is_contiguous()):
+        raise ValueError(f"{op} expects contiguous scale tensors (they are updated in place)")
+    _extension().areno_paged_cache_write(
+        k.contiguous(), v.contiguous(), k_cache, v_cache,
+        cache_block_ids.contiguous(), cache_block_offsets.contiguous(), k_scale, v_scale,
+    )  # fmt: skip
+
+
+@torch._dynamo.disable
+def areno_paged_varlen_causal_attention(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    block_table: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    context_lens: torch.Tensor,
+    *,
+    window_left: int | None = None,
+    softmax_scale: float | None = None,
+    k_scale: torch.Tensor | None = None,
+    v_scale: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Causal attention of packed new queries ``(tokens, heads, head_dim)`` over paged KV.
+
+    The new tokens' K/V must already be in the cache.  Query ``i`` of sequence ``s`` sits at
+    absolute position ``context_lens[s] + i`` and sees keys ``[0, context_lens[s] + i]``.
+    """
+    op = "areno_paged_varlen_causal_attention"
+    if not _all_on_gpu(q, k_cache, v_cache, block_table, cu_seqlens_q, context_lens, k_scale, v_scale):
+        raise RuntimeError(f"{op} requires CUDA tensors")
+    if q.dim() != 3:
+        raise ValueError(f"{op} expects q shaped (tokens, heads, head_dim)")
+    if k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise ValueError(f"{op} expects 4D paged cache tensors")
+    if block_table.dim() != 2 or cu_seqlens_q.dim() != 1 or context_lens.dim() != 1:
+        raise ValueError(f"{op} expects block_table 2D, cu_seqlens_q 1D and context_lens 1D")
+    if any(t.dtype != torch.int32 for t in (block_table, cu_seqlens_q, context_lens)):
+        raise ValueError(f"{op} expects int32 block_table, cu_seqlens_q and context_lens")
+    _check_scales(op, k_cache, k_scale, v_scale)
+    return _extension().areno_paged_varlen_causal_attention_forward(
+        q.contiguous(), k_cache.contiguous(), v_cache.contiguous(), block_table.contiguous(),
+        cu_seqlens_q.contiguous(), context_lens.contiguous(), _window_left(window_left), _scale(q, softmax_scale),
+        _contig(k_scale), _contig(v_scale),
+    )  # fmt: skip

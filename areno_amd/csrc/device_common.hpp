@@ -1,0 +1,103 @@
+// Shared device helpers for the gfx950 paged-attention kernels: 16-bit / 8-bit element
+// conversions, wave64 cross-lane primitives and the host-side error plumbing of the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/areno_hip.h"
+
+namespace areno {
+
+constexpr int kWave = 64;
+
+typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) float float2_t;
+typedef __attribute__((ext_vector_type(4))) float float4_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t uint4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t uint2_t;
+
+// ---- scalar conversions ------------------------------------------------------------------
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t bits16) {
+  return __builtin_bit_cast(float, bits16 << 16);
+}
+
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float x) {
+  __bf16 h = static_cast<__bf16>(x);  // round to nearest even
+  return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, h));
+}
+
+__device__ __forceinline__ float f16_bits_to_float(uint32_t bits16) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits16)));
+}
+
+__device__ __forceinline__ uint32_t float_to_f16_bits(float x) {
+  _Float16 h = static_cast<_Float16>(x);
+  return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, h));
+}
+
+// OCP e4m3fn byte -> float (hardware conversion; gfx950 implements the OCP encodings).
+__device__ __forceinline__ float fp8_byte_to_float(uint32_t byte) {
+  return __builtin_amdgcn_cvt_f32_fp8(byte & 0xffu, 0);
+}
+
+// float (already clamped to [-448, 448]) -> OCP e4m3fn byte, round to nearest even.
+__device__ __forceinline__ uint32_t float_to_fp8_byte(float x) {
+  return static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false)) & 0xffu;
+}
+
+// Element `idx` of a row stored with the given dtype, as float.
+__device__ __forceinline__ float load_as_float(const void* base, int64_t idx, int dtype) {
+  switch (dtype) {
+    case ARENO_DT_F32: return static_cast<const float*>(base)[idx];
+    case ARENO_DT_F16: return f16_bits_to_float(static_cast<const uint16_t*>(base)[idx]);
+    case ARENO_DT_BF16: return bf16_bits_to_float(static_cast<const uint16_t*>(base)[idx]);
+    case ARENO_DT_I8: return static_cast<float>(static_cast<const int8_t*>(base)[idx]);
+    default: return fp8_byte_to_float(static_cast<const uint8_t*>(base)[idx]);
+  }
+}
+
+__device__ __forceinline__ void store_from_float(void* base, int64_t idx, int dtype, float x) {
+  switch (dtype) {
+    case ARENO_DT_F32: static_cast<float*>(base)[idx] = x; break;
+    case ARENO_DT_F16: static_cast<uint16_t*>(base)[idx] = static_cast<uint16_t>(float_to_f16_bits(x)); break;
+    default: static_cast<uint16_t*>(base)[idx] = static_cast<uint16_t>(float_to_bf16_bits(x)); break;
+  }
+}
+
+__device__ __forceinline__ float load_scale(const void* base, int64_t idx, int scale_dtype) {
+  return scale_dtype == ARENO_DT_F16 ? f16_bits_to_float(static_cast<const uint16_t*>(base)[idx])
+                                     : static_cast<const float*>(base)[idx];
+}
+
+// ---- wave64 cross-lane -------------------------------------------------------------------
+
+__device__ __forceinline__ float wave_xor(float x, int mask) { return __shfl_xor(x, mask, kWave); }
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) x += wave_xor(x, m);
+  return x;
+}
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) x = fmaxf(x, wave_xor(x, m));
+  return x;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ---- host side ---------------------------------------------------------------------------
+
+void set_error(const char* fmt, ...);
+int fail(int status, const char* fmt, ...);
+int check_launch(const char* what);
+size_t dtype_size(int dtype);
+bool is_quantized(int dtype);
+
+}  // namespace areno

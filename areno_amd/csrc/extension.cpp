@@ -1,0 +1,257 @@
+// PyTorch-ROCm binding of libareno_hip.so: at::Tensor checks -> C ABI (include/areno_hip.h).
+//
+// Mirrors the reference's pybind surface for this path (areno/accel/csrc/extension.cpp:180-184):
+//   areno_paged_causal_attention_decode_forward, areno_varlen_causal_attention_forward
+// with the same TORCH_CHECK contract as its host launchers (areno/accel/csrc/attention.cu:813-861,
+// 926-1020): device / contiguity / rank / dtype / shape agreement, current device guard, launch on the
+// current stream, fresh output tensor, per-call workspace from the caching allocator.  The extra
+// entry points (cache write, paged prefill, scales) are this build's extension of the path.
+
+#include <ATen/ATen.h>
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/extension.h>
+
+#include "../../include/areno_hip.h"
+
+namespace {
+
+int dtype_code(const at::Tensor& t, const char* op, const char* name) {
+  switch (t.scalar_type()) {
+    case at::kFloat: return ARENO_DT_F32;
+    case at::kHalf: return ARENO_DT_F16;
+    case at::kBFloat16: return ARENO_DT_BF16;
+    case at::kChar: return ARENO_DT_I8;
+    case at::kFloat8_e4m3fn: return ARENO_DT_FP8_E4M3;
+    default: TORCH_CHECK(false, op, " ", name, " has unsupported dtype ", t.scalar_type());
+  }
+  return -1;
+}
+
+void check_status(int status, const char* op) {
+  TORCH_CHECK(status == ARENO_OK, op, " failed: ", areno_hip_status_string(status), " (", areno_hip_last_error(), ")");
+}
+
+void* current_stream(const at::Tensor& t) {
+  return static_cast<void*>(c10::hip::getCurrentHIPStream(t.device().index()).stream());
+}
+
+areno_paged_cache describe_cache(const at::Tensor& k_cache, const at::Tensor& v_cache,
+                                 const c10::optional<at::Tensor>& k_scale, const c10::optional<at::Tensor>& v_scale,
+                                 const char* op) {
+  TORCH_CHECK(k_cache.is_cuda(), op, " k_cache must be CUDA");
+  TORCH_CHECK(v_cache.is_cuda(), op, " v_cache must be CUDA");
+  TORCH_CHECK(k_cache.is_contiguous(), op, " k_cache must be contiguous");
+  TORCH_CHECK(v_cache.is_contiguous(), op, " v_cache must be contiguous");
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4, op, " cache tensors must be 4D");
+  TORCH_CHECK(k_cache.scalar_type() == v_cache.scalar_type(), op, " cache dtype mismatch");
+  TORCH_CHECK(k_cache.size(0) == v_cache.size(0) && k_cache.size(1) == v_cache.size(1), op,
+              " cache block shape mismatch");
+  TORCH_CHECK(k_cache.size(2) == v_cache.size(2), op, " cache head mismatch");
+  TORCH_CHECK(k_cache.size(3) == v_cache.size(3), op, " cache head dim mismatch");
+  areno_paged_cache c;
+  c.k = k_cache.data_ptr();
+  c.v = v_cache.data_ptr();
+  c.k_scale = nullptr;
+  c.v_scale = nullptr;
+  c.num_blocks = k_cache.size(0);
+  c.block_size = static_cast<int32_t>(k_cache.size(1));
+  c.kv_heads = static_cast<int32_t>(k_cache.size(2));
+  c.head_dim = static_cast<int32_t>(k_cache.size(3));
+  c.cache_dtype = dtype_code(k_cache, op, "k_cache");
+  c.scale_dtype = ARENO_DT_F32;
+  const bool quantized = c.cache_dtype == ARENO_DT_I8 || c.cache_dtype == ARENO_DT_FP8_E4M3;
+  TORCH_CHECK(quantized == (k_scale.has_value() && v_scale.has_value()), op,
+              " k_scale and v_scale are required for int8/float8_e4m3fn caches and forbidden otherwise");
+  if (quantized) {
+    const at::Tensor& ks = *k_scale;
+    const at::Tensor& vs = *v_scale;
+    TORCH_CHECK(ks.is_cuda() && vs.is_cuda(), op, " scales must be CUDA");
+    TORCH_CHECK(ks.is_contiguous() && vs.is_contiguous(), op, " scales must be contiguous");
+    TORCH_CHECK(ks.scalar_type() == vs.scalar_type(), op, " scale dtype mismatch");
+    TORCH_CHECK(ks.scalar_type() == at::kHalf || ks.scalar_type() == at::kFloat, op, " scales must be fp16 or fp32");
+    TORCH_CHECK(ks.dim() == 3 && vs.dim() == 3, op, " scales must be shaped (num_blocks, block_size, kv_heads)");
+    for (int i = 0; i < 3; ++i) {
+      TORCH_CHECK(ks.size(i) == k_cache.size(i) && vs.size(i) == k_cache.size(i), op, " scale shape mismatch");
+    }
+    c.k_scale = ks.data_ptr();
+    c.v_scale = vs.data_ptr();
+    c.scale_dtype = ks.scalar_type() == at::kHalf ? ARENO_DT_F16 : ARENO_DT_F32;
+  }
+  return c;
+}
+
+at::Tensor paged_decode_forward_impl(at::Tensor q, at::Tensor k_update, at::Tensor v_update, at::Tensor k_cache,
+                                     at::Tensor v_cache, at::Tensor block_table, at::Tensor cache_seqlens,
+                                     int64_t window_left, int64_t num_splits, double softmax_scale,
+                                     c10::optional<at::Tensor> k_scale, c10::optional<at::Tensor> v_scale) {
+  const char* op = "areno_paged_causal_attention_decode";
+  TORCH_CHECK(q.is_cuda(), op, " q must be CUDA");
+  TORCH_CHECK(k_update.is_cuda(), op, " k_update must be CUDA");
+  TORCH_CHECK(v_update.is_cuda(), op, " v_update must be CUDA");
+  TORCH_CHECK(block_table.is_cuda(), op, " block_table must be CUDA");
+  TORCH_CHECK(cache_seqlens.is_cuda(), op, " cache_seqlens must be CUDA");
+  TORCH_CHECK(q.is_contiguous(), op, " q must be contiguous");
+  TORCH_CHECK(k_update.is_contiguous(), op, " k_update must be contiguous");
+  TORCH_CHECK(v_update.is_contiguous(), op, " v_update must be contiguous");
+  TORCH_CHECK(block_table.is_contiguous(), op, " block_table must be contiguous");
+  TORCH_CHECK(cache_seqlens.is_contiguous(), op, " cache_seqlens must be contiguous");
+  TORCH_CHECK(q.dim() == 3, op, " q must be shaped (batch, heads, head_dim)");
+  TORCH_CHECK(k_update.dim() == 3 && v_update.dim() == 3, op, " updates must be 3D");
+  TORCH_CHECK(block_table.dim() == 2, op, " block_table must be 2D");
+  TORCH_CHECK(cache_seqlens.dim() == 1, op, " cache_seqlens must be 1D");
+  const areno_paged_cache cache = describe_cache(k_cache, v_cache, k_scale, v_scale, op);
+  const bool quantized = cache.k_scale != nullptr;
+  if (!quantized) {
+    TORCH_CHECK(q.scalar_type() == k_cache.scalar_type(), op, " dtype mismatch");
+  } else {
+    TORCH_CHECK(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, op,
+                " q must be fp16 or bf16 with a quantized cache");
+  }
+  TORCH_CHECK(k_update.scalar_type() == q.scalar_type() && v_update.scalar_type() == q.scalar_type(), op,
+              " update dtype mismatch");
+  TORCH_CHECK(block_table.scalar_type() == at::kInt, op, " block_table must be int32");
+  TORCH_CHECK(cache_seqlens.scalar_type() == at::kInt, op, " cache_seqlens must be int32");
+  TORCH_CHECK(q.size(0) == block_table.size(0) && q.size(0) == cache_seqlens.size(0), op, " batch mismatch");
+  TORCH_CHECK(k_update.size(0) == q.size(0) && v_update.size(0) == q.size(0), op, " update batch mismatch");
+  TORCH_CHECK(k_update.size(1) == k_cache.size(2) && v_update.size(1) == v_cache.size(2), op, " update head mismatch");
+  TORCH_CHECK(q.size(2) == k_cache.size(3) && q.size(2) == v_cache.size(3), op, " head dim mismatch");
+  TORCH_CHECK(k_update.size(2) == k_cache.size(3) && v_update.size(2) == v_cache.size(3), op,
+              " update head dim mismatch");
+  TORCH_CHECK(q.size(1) % k_cache.size(2) == 0, op, " q heads must be divisible by kv heads");
+  TORCH_CHECK(num_splits >= 1, op, " num_splits must be >= 1");
+
+  const c10::hip::OptionalHIPGuard guard(device_of(q));
+  auto out = at::empty_like(q);
+  if (q.size(0) == 0) return out;
+  const size_t ws_bytes = areno_hip_paged_decode_workspace_bytes(
+      static_cast<int32_t>(q.size(0)), static_cast<int32_t>(q.size(1)), cache.head_dim, cache.block_size,
+      static_cast<int32_t>(block_table.size(1)), static_cast<int32_t>(num_splits));
+  TORCH_CHECK(ws_bytes > 0, op, " invalid shapes for the split-KV workspace");
+  auto workspace = at::empty({static_cast<int64_t>(ws_bytes)}, q.options().dtype(at::kByte));
+  const int status = areno_hip_paged_decode(
+      &cache, q.data_ptr(), k_update.data_ptr(), v_update.data_ptr(), out.data_ptr(), dtype_code(q, op, "q"),
+      static_cast<int32_t>(q.size(0)), static_cast<int32_t>(q.size(1)), block_table.data_ptr<int32_t>(),
+      static_cast<int32_t>(block_table.size(1)), cache_seqlens.data_ptr<int32_t>(), static_cast<int32_t>(window_left),
+      static_cast<int32_t>(num_splits), static_cast<float>(softmax_scale), workspace.data_ptr(), ws_bytes,
+      current_stream(q));
+  check_status(status, op);
+  return out;
+}
+
+// Reference signature (extension.cpp:184 in the reference).
+at::Tensor paged_decode_forward(at::Tensor q, at::Tensor k_update, at::Tensor v_update, at::Tensor k_cache,
+                                at::Tensor v_cache, at::Tensor block_table, at::Tensor cache_seqlens,
+                                int64_t window_left, int64_t num_splits, double softmax_scale) {
+  return paged_decode_forward_impl(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, window_left,
+                                   num_splits, softmax_scale, c10::nullopt, c10::nullopt);
+}
+
+at::Tensor varlen_forward(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor cu_seqlens, int64_t window_left,
+                          double softmax_scale) {
+  const char* op = "areno_varlen_causal_attention";
+  TORCH_CHECK(q.is_cuda(), op, " q must be CUDA");
+  TORCH_CHECK(k.is_cuda(), op, " k must be CUDA");
+  TORCH_CHECK(v.is_cuda(), op, " v must be CUDA");
+  TORCH_CHECK(cu_seqlens.is_cuda(), op, " cu_seqlens must be CUDA");
+  TORCH_CHECK(q.is_contiguous(), op, " q must be contiguous");
+  TORCH_CHECK(k.is_contiguous(), op, " k must be contiguous");
+  TORCH_CHECK(v.is_contiguous(), op, " v must be contiguous");
+  TORCH_CHECK(cu_seqlens.is_contiguous(), op, " cu_seqlens must be contiguous");
+  TORCH_CHECK(q.dim() == 3 && k.dim() == 3 && v.dim() == 3, op, " expects 3D q/k/v");
+  TORCH_CHECK(cu_seqlens.dim() == 1, op, " cu_seqlens must be 1D");
+  TORCH_CHECK(cu_seqlens.scalar_type() == at::kInt, op, " cu_seqlens must be int32");
+  TORCH_CHECK(q.scalar_type() == k.scalar_type() && q.scalar_type() == v.scalar_type(), op, " dtype mismatch");
+  TORCH_CHECK(q.size(0) == k.size(0) && q.size(0) == v.size(0), op, " token count mismatch");
+  TORCH_CHECK(k.size(1) == v.size(1), op, " key/value head mismatch");
+  TORCH_CHECK(q.size(1) % k.size(1) == 0, op, " q heads must be divisible by kv heads");
+  TORCH_CHECK(q.size(2) == k.size(2) && q.size(2) == v.size(2), op, " head dim mismatch");
+  TORCH_CHECK(cu_seqlens.size(0) >= 2, op, " cu_seqlens must contain at least one sequence");
+  const c10::hip::OptionalHIPGuard guard(device_of(q));
+  auto out = at::empty_like(q);
+  const int status = areno_hip_varlen_attention(
+      q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dtype_code(q, op, "q"), q.size(0),
+      static_cast<int32_t>(q.size(1)), static_cast<int32_t>(k.size(1)), static_cast<int32_t>(q.size(2)),
+      cu_seqlens.data_ptr<int32_t>(), static_cast<int32_t>(cu_seqlens.size(0) - 1), static_cast<int32_t>(window_left),
+      static_cast<float>(softmax_scale), current_stream(q));
+  check_status(status, op);
+  return out;
+}
+
+void cache_write(at::Tensor k, at::Tensor v, at::Tensor k_cache, at::Tensor v_cache, at::Tensor block_ids,
+                 at::Tensor block_offsets, c10::optional<at::Tensor> k_scale, c10::optional<at::Tensor> v_scale) {
+  const char* op = "areno_paged_cache_write";
+  TORCH_CHECK(k.is_cuda() && v.is_cuda(), op, " k and v must be CUDA");
+  TORCH_CHECK(block_ids.is_cuda() && block_offsets.is_cuda(), op, " block ids/offsets must be CUDA");
+  TORCH_CHECK(k.is_contiguous() && v.is_contiguous(), op, " k and v must be contiguous");
+  TORCH_CHECK(block_ids.is_contiguous() && block_offsets.is_contiguous(), op, " block ids/offsets must be contiguous");
+  TORCH_CHECK(k.dim() == 3 && v.dim() == 3, op, " expects k/v shaped (tokens, kv_heads, head_dim)");
+  TORCH_CHECK(block_ids.dim() == 1 && block_offsets.dim() == 1, op, " block ids/offsets must be 1D");
+  TORCH_CHECK(block_ids.scalar_type() == at::kLong && block_offsets.scalar_type() == at::kLong, op,
+              " block ids/offsets must be int64");
+  TORCH_CHECK(k.scalar_type() == v.scalar_type(), op, " dtype mismatch");
+  const areno_paged_cache cache = describe_cache(k_cache, v_cache, k_scale, v_scale, op);
+  if (cache.k_scale == nullptr) TORCH_CHECK(k.scalar_type() == k_cache.scalar_type(), op, " dtype mismatch");
+  TORCH_CHECK(k.size(0) == v.size(0) && k.size(0) == block_ids.size(0) && k.size(0) == block_offsets.size(0), op,
+              " token count mismatch");
+  TORCH_CHECK(k.size(1) == k_cache.size(2) && v.size(1) == v_cache.size(2), op, " head mismatch");
+  TORCH_CHECK(k.size(2) == k_cache.size(3) && v.size(2) == v_cache.size(3), op, " head dim mismatch");
+  const c10::hip::OptionalHIPGuard guard(device_of(k));
+  const int status =
+      areno_hip_cache_write(&cache, k.data_ptr(), v.data_ptr(), dtype_code(k, op, "k"), k.size(0),
+                            block_ids.data_ptr<int64_t>(), block_offsets.data_ptr<int64_t>(), current_stream(k));
+  check_status(status, op);
+}
+
+at::Tensor paged_varlen_forward(at::Tensor q, at::Tensor k_cache, at::Tensor v_cache, at::Tensor block_table,
+                                at::Tensor cu_seqlens_q, at::Tensor context_lens, int64_t window_left,
+                                double softmax_scale, c10::optional<at::Tensor> k_scale,
+                                c10::optional<at::Tensor> v_scale) {
+  const char* op = "areno_paged_varlen_causal_attention";
+  TORCH_CHECK(q.is_cuda() && block_table.is_cuda() && cu_seqlens_q.is_cuda() && context_lens.is_cuda(), op,
+              " tensors must be CUDA");
+  TORCH_CHECK(q.is_contiguous() && block_table.is_contiguous() && cu_seqlens_q.is_contiguous() &&
+                  context_lens.is_contiguous(),
+              op, " tensors must be contiguous");
+  TORCH_CHECK(q.dim() == 3, op, " q must be shaped (tokens, heads, head_dim)");
+  TORCH_CHECK(block_table.dim() == 2 && cu_seqlens_q.dim() == 1 && context_lens.dim() == 1, op,
+              " expects block_table 2D, cu_seqlens_q 1D, context_lens 1D");
+  TORCH_CHECK(block_table.scalar_type() == at::kInt && cu_seqlens_q.scalar_type() == at::kInt &&
+                  context_lens.scalar_type() == at::kInt,
+              op, " block_table, cu_seqlens_q and context_lens must be int32");
+  const areno_paged_cache cache = describe_cache(k_cache, v_cache, k_scale, v_scale, op);
+  if (cache.k_scale == nullptr) {
+    TORCH_CHECK(q.scalar_type() == k_cache.scalar_type(), op, " dtype mismatch");
+  } else {
+    TORCH_CHECK(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, op,
+                " q must be fp16 or bf16 with a quantized cache");
+  }
+  TORCH_CHECK(cu_seqlens_q.size(0) >= 2, op, " cu_seqlens_q must contain at least one sequence");
+  TORCH_CHECK(context_lens.size(0) == cu_seqlens_q.size(0) - 1 && block_table.size(0) == context_lens.size(0), op,
+              " sequence count mismatch");
+  TORCH_CHECK(q.size(2) == k_cache.size(3), op, " head dim mismatch");
+  TORCH_CHECK(q.size(1) % k_cache.size(2) == 0, op, " q heads must be divisible by kv heads");
+  const c10::hip::OptionalHIPGuard guard(device_of(q));
+  auto out = at::empty_like(q);
+  const int status = areno_hip_paged_varlen_prefill(
+      &cache, q.data_ptr(), out.data_ptr(), dtype_code(q, op, "q"), q.size(0), static_cast<int32_t>(q.size(1)),
+      static_cast<int32_t>(context_lens.size(0)), block_table.data_ptr<int32_t>(),
+      static_cast<int32_t>(block_table.size(1)), cu_seqlens_q.data_ptr<int32_t>(), context_lens.data_ptr<int32_t>(),
+      static_cast<int32_t>(window_left), static_cast<float>(softmax_scale), current_stream(q));
+  check_status(status, op);
+  return out;
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("areno_paged_causal_attention_decode_forward", &paged_decode_forward,
+        "ARENO paged causal attention decode forward");
+  m.def("areno_varlen_causal_attention_forward", &varlen_forward, "ARENO varlen causal attention forward");
+  m.def("areno_paged_causal_attention_decode_forward_scaled", &paged_decode_forward_impl,
+        "paged decode forward with optional int8/fp8 cache scales");
+  m.def("areno_paged_cache_write", &cache_write, "quantize-and-scatter KV cache write");
+  m.def("areno_paged_varlen_causal_attention_forward", &paged_varlen_forward,
+        "causal varlen prefill over paged (optionally quantized) KV");
+  m.def("abi_version", &areno_hip_abi_version, "C ABI version of libareno_hip.so");
+}

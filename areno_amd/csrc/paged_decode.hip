@@ -1,0 +1,263 @@
+// Host launcher of the paged decode op plus its two small kernels:
+//   decode_split_generic_kernel  -- any dtype / head_dim <= 512 / head ratio; one wave per (chunk, row)
+//   decode_reduce_kernel         -- log-sum-exp merge of the chunk partials (attention.cu:656-702 in the
+//                                   reference), normalise, cast to the query dtype
+// The fast split kernels live in paged_decode_kernels.hpp.
+
+#include "paged_decode_kernels.hpp"
+
+namespace areno {
+
+int validate_paged_cache(const areno_paged_cache* c, const char* op);
+
+namespace {
+
+constexpr int kGenericMaxPerLane = 8;  // head_dim <= 512
+
+__global__ __launch_bounds__(kWave) void decode_split_generic_kernel(DecodeParams p) {
+  const int lane = threadIdx.x;
+  const int row = blockIdx.x;
+  const int c = blockIdx.y;
+  const int b = row / p.q_heads;
+  const int h = row - b * p.q_heads;
+  const int kvh = h / p.group;
+  const int d = p.head_dim;
+
+  const int length = p.cache_seqlens[b] + 1;
+  const int first_allowed = first_allowed_key(length, p.window_left);
+  const int lo = max(c * p.chunk, first_allowed);
+  const int hi = min((c + 1) * p.chunk, length);
+  if (lo >= hi) return;
+
+  float q[kGenericMaxPerLane], acc[kGenericMaxPerLane];
+#pragma unroll
+  for (int e = 0; e < kGenericMaxPerLane; ++e) {
+    const int idx = lane + e * kWave;
+    q[e] = idx < d ? load_as_float(p.q, static_cast<int64_t>(row) * d + idx, p.q_dtype) : 0.0f;
+    acc[e] = 0.0f;
+  }
+  const bool quant = p.cache_dtype == ARENO_DT_I8 || p.cache_dtype == ARENO_DT_FP8_E4M3;
+  float m = kNegInf, l = 0.0f;
+  const int32_t* table_row = p.block_table + static_cast<int64_t>(b) * p.max_blocks;
+  for (int t = lo; t < hi; ++t) {
+    const int col = t / p.block_size;
+    const int slot = t - col * p.block_size;
+    const int64_t blk = table_row[col];
+    const int64_t r = (blk * p.block_size + slot) * p.kv_heads + kvh;
+    float dot = 0.0f;
+    float v[kGenericMaxPerLane];
+#pragma unroll
+    for (int e = 0; e < kGenericMaxPerLane; ++e) {
+      const int idx = lane + e * kWave;
+      if (idx < d) {
+        dot += q[e] * load_as_float(p.k_cache, r * d + idx, p.cache_dtype);
+        v[e] = load_as_float(p.v_cache, r * d + idx, p.cache_dtype);
+      } else {
+        v[e] = 0.0f;
+      }
+    }
+    dot = wave_sum(dot);
+    float ks = 1.0f, vs = 1.0f;
+    if (quant) {
+      ks = load_scale(p.k_scale, r, p.scale_dtype);
+      vs = load_scale(p.v_scale, r, p.scale_dtype);
+    }
+    const float s = dot * ks * p.scale_log2e;
+    const float m_new = fmaxf(m, s);
+    const float alpha = fast_exp2(m - m_new);  // m = -inf on the first key -> 0
+    const float beta = fast_exp2(s - m_new);
+    l = l * alpha + beta;
+    m = m_new;
+    const float bv = beta * vs;
+#pragma unroll
+    for (int e = 0; e < kGenericMaxPerLane; ++e) acc[e] = acc[e] * alpha + bv * v[e];
+  }
+  const int64_t prow = static_cast<int64_t>(row) * p.max_parts + c;
+#pragma unroll
+  for (int e = 0; e < kGenericMaxPerLane; ++e) {
+    const int idx = lane + e * kWave;
+    if (idx < d) p.part_acc[prow * d + idx] = acc[e];
+  }
+  if (lane == 0) {
+    p.part_ml[prow * 2] = m;
+    p.part_ml[prow * 2 + 1] = l;
+  }
+}
+
+constexpr int kReduceRows = 4;
+
+__global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_kernel(DecodeParams p) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int row = blockIdx.x * kReduceRows + (threadIdx.x >> 6);
+  if (row >= p.batch * p.q_heads) return;
+  const int b = row / p.q_heads;
+  const int d = p.head_dim;
+  const int length = p.cache_seqlens[b] + 1;
+  const int first_allowed = first_allowed_key(length, p.window_left);
+  const int c_lo = first_allowed / p.chunk;
+  const int c_hi = (length - 1) / p.chunk;
+
+  float acc[kGenericMaxPerLane];
+#pragma unroll
+  for (int e = 0; e < kGenericMaxPerLane; ++e) acc[e] = 0.0f;
+  float m = kNegInf, l = 0.0f;
+  const int64_t base = static_cast<int64_t>(row) * p.max_parts;
+  for (int c = c_lo; c <= c_hi && c < p.max_parts; ++c) {
+    const float part_m = p.part_ml[(base + c) * 2];
+    const float part_l = p.part_ml[(base + c) * 2 + 1];
+    if (part_l == 0.0f) continue;  // a partial without keys contributes nothing (attention.cu:680-682)
+    const float m_new = fmaxf(m, part_m);
+    const float alpha = fast_exp2(m - m_new);
+    const float beta = fast_exp2(part_m - m_new);
+    const float* part = p.part_acc + (base + c) * d;
+#pragma unroll
+    for (int e = 0; e < kGenericMaxPerLane; ++e) {
+      const int idx = lane + e * kWave;
+      if (idx < d) acc[e] = acc[e] * alpha + part[idx] * beta;
+    }
+    l = l * alpha + part_l * beta;
+    m = m_new;
+  }
+#pragma unroll
+  for (int e = 0; e < kGenericMaxPerLane; ++e) {
+    const int idx = lane + e * kWave;
+    if (idx < d) store_from_float(p.out, static_cast<int64_t>(row) * d + idx, p.q_dtype, acc[e] / l);
+  }
+}
+
+struct Chunking {
+  int chunk;
+  int max_parts;
+};
+
+constexpr int kChunkQuantum = 256;  // multiple of every tile size times the largest token split
+constexpr int kMaxParts = 64;
+
+bool pick_chunking(int64_t block_size, int64_t max_blocks, int num_splits, Chunking* out) {
+  const int64_t max_tokens = block_size * max_blocks;
+  if (max_tokens <= 0 || max_tokens > 0x3fffffffLL) return false;
+  int64_t chunk = kChunkQuantum;
+  if (num_splits == 1) {
+    chunk = (max_tokens + kChunkQuantum - 1) / kChunkQuantum * kChunkQuantum;
+  } else {
+    while ((max_tokens + chunk - 1) / chunk > kMaxParts) chunk *= 2;
+  }
+  out->chunk = static_cast<int>(chunk);
+  out->max_parts = static_cast<int>((max_tokens + chunk - 1) / chunk);
+  return true;
+}
+
+int log2_exact(int x) {
+  if (x <= 0 || (x & (x - 1)) != 0) return -1;
+  int s = 0;
+  while ((1 << s) < x) ++s;
+  return s;
+}
+
+}  // namespace
+}  // namespace areno
+
+extern "C" size_t areno_hip_paged_decode_workspace_bytes(int32_t batch, int32_t q_heads, int32_t head_dim,
+                                                         int32_t block_size, int32_t max_blocks, int32_t num_splits) {
+  areno::Chunking ch;
+  if (batch <= 0 || q_heads <= 0 || head_dim <= 0 || num_splits < 1) return 0;
+  if (!areno::pick_chunking(block_size, max_blocks, num_splits, &ch)) return 0;
+  const size_t rows = static_cast<size_t>(batch) * q_heads * ch.max_parts;
+  const size_t bytes = rows * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
+  return (bytes + 255) / 256 * 256;
+}
+
+extern "C" int areno_hip_paged_decode(const areno_paged_cache* cache, const void* q, const void* k_update,
+                                      const void* v_update, void* out, int32_t q_dtype, int32_t batch,
+                                      int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
+                                      const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
+                                      float softmax_scale, void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace areno;
+  const char* op = "areno_hip_paged_decode";
+  if (int rc = validate_paged_cache(cache, op)) return rc;
+  if (q == nullptr || out == nullptr || block_table == nullptr || cache_seqlens == nullptr)
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: q/out/block_table/cache_seqlens is NULL", op);
+  if ((k_update == nullptr) != (v_update == nullptr))
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: k_update and v_update must both be given or both be NULL", op);
+  if (batch < 0 || batch > 65535 || q_heads <= 0 || max_blocks <= 0)
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: batch/q_heads/max_blocks out of range", op);
+  if (q_heads % cache->kv_heads != 0)
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: q heads must be divisible by kv heads", op);
+  if (num_splits < 1) return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: num_splits must be >= 1", op);
+  if (q_dtype != ARENO_DT_F32 && q_dtype != ARENO_DT_F16 && q_dtype != ARENO_DT_BF16)
+    return fail(ARENO_ERR_UNSUPPORTED, "%s: q must be f32, f16 or bf16", op);
+  if (!is_quantized(cache->cache_dtype) && cache->cache_dtype != q_dtype)
+    return fail(ARENO_ERR_UNSUPPORTED, "%s: q dtype must equal an unquantized cache's dtype", op);
+  if (cache->head_dim > kGenericMaxPerLane * kWave)
+    return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim %d > %d", op, cache->head_dim, kGenericMaxPerLane * kWave);
+  if (batch == 0) return ARENO_OK;
+
+  Chunking ch;
+  if (!pick_chunking(cache->block_size, max_blocks, num_splits, &ch))
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: block_size * max_blocks out of range", op);
+  const size_t need = areno_hip_paged_decode_workspace_bytes(batch, q_heads, cache->head_dim, cache->block_size,
+                                                             max_blocks, num_splits);
+  if (workspace == nullptr || workspace_bytes < need)
+    return fail(ARENO_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", op, need, workspace_bytes);
+
+  if (k_update != nullptr) {
+    if (int rc = areno_hip_cache_write_decode(cache, k_update, v_update, q_dtype, batch, block_table, max_blocks,
+                                              cache_seqlens, stream))
+      return rc;
+  }
+
+  DecodeParams p;
+  p.q = q;
+  p.k_cache = cache->k;
+  p.v_cache = cache->v;
+  p.k_scale = cache->k_scale;
+  p.v_scale = cache->v_scale;
+  p.block_table = block_table;
+  p.cache_seqlens = cache_seqlens;
+  const size_t rows = static_cast<size_t>(batch) * q_heads * ch.max_parts;
+  p.part_ml = static_cast<float*>(workspace);
+  p.part_acc = p.part_ml + rows * 2;
+  p.out = out;
+  p.batch = batch;
+  p.q_heads = q_heads;
+  p.kv_heads = cache->kv_heads;
+  p.head_dim = cache->head_dim;
+  p.block_size = cache->block_size;
+  p.bs_shift = log2_exact(cache->block_size);
+  p.max_blocks = max_blocks;
+  p.window_left = window_left;
+  p.chunk = ch.chunk;
+  p.max_parts = ch.max_parts;
+  p.q_dtype = q_dtype;
+  p.cache_dtype = cache->cache_dtype;
+  p.scale_dtype = cache->scale_dtype;
+  p.group = q_heads / cache->kv_heads;
+  p.heads_per_wg = cache->kv_heads % 4 == 0 ? 4 : (cache->kv_heads % 2 == 0 ? 2 : 1);
+  p.scale_log2e = softmax_scale * kLog2e;
+
+  decode_split_fn fast = nullptr;
+  const bool aligned = (reinterpret_cast<uintptr_t>(cache->k) % 16 == 0) &&
+                       (reinterpret_cast<uintptr_t>(cache->v) % 16 == 0) &&
+                       (reinterpret_cast<uintptr_t>(workspace) % 16 == 0);
+  if (aligned && q_dtype != ARENO_DT_F32) {
+    switch (cache->cache_dtype) {
+      case ARENO_DT_BF16: fast = decode_split_lookup_bf16(p.head_dim, p.group); break;
+      case ARENO_DT_F16: fast = decode_split_lookup_f16(p.head_dim, p.group); break;
+      case ARENO_DT_I8: fast = decode_split_lookup_i8(p.head_dim, p.group); break;
+      case ARENO_DT_FP8_E4M3: fast = decode_split_lookup_fp8(p.head_dim, p.group); break;
+      default: break;
+    }
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (fast != nullptr) {
+    const dim3 grid(ch.max_parts, batch, cache->kv_heads / p.heads_per_wg);
+    hipLaunchKernelGGL(fast, grid, dim3(kDecodeThreads), 0, s, p);
+  } else {
+    const dim3 grid(batch * q_heads, ch.max_parts);
+    hipLaunchKernelGGL(decode_split_generic_kernel, grid, dim3(kWave), 0, s, p);
+  }
+  if (int rc = check_launch(op)) return rc;
+  const int rblocks = (batch * q_heads + kReduceRows - 1) / kReduceRows;
+  hipLaunchKernelGGL(decode_reduce_kernel, dim3(rblocks), dim3(kReduceRows * kWave), 0, s, p);
+  return check_launch(op);
+}

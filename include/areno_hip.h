@@ -1,0 +1,141 @@
+/*
+ * C ABI of libareno_hip.so: the MI355X (gfx950) kernels behind AReno's native paged
+ * KV-cache attention ops.  Plain pointers and sizes only; every pointer named "device"
+ * is a HIP device pointer.  No entry point allocates, synchronises the host or throws:
+ * each returns ARENO_OK (0) or a negative ARENO_ERR_* code and records a message that
+ * areno_hip_last_error() returns (thread-local).  All launches go to `stream`
+ * (a hipStream_t passed as void*; NULL is the null stream) and are legal inside HIP
+ * stream capture.
+ *
+ * Layouts (all contiguous, row-major), as the reference engine allocates them
+ * (areno/models/qwen3/model.py:309-333, areno/engine/runtime/metadata.py:29-45):
+ *   cache pools   k, v            [num_blocks, block_size, kv_heads, head_dim]   cache_dtype
+ *   scale pools   k_scale,v_scale [num_blocks, block_size, kv_heads]             scale_dtype (quantized caches only)
+ *   block_table                   [batch, max_blocks]  int32, entries must be valid block ids
+ *   cache_seqlens                 [batch]              int32, tokens cached before the step
+ */
+#ifndef ARENO_HIP_H
+#define ARENO_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ARENO_HIP_ABI_VERSION 1
+
+enum areno_dtype {
+  ARENO_DT_F32 = 0,
+  ARENO_DT_F16 = 1,
+  ARENO_DT_BF16 = 2,
+  ARENO_DT_I8 = 3,       /* symmetric int8 codes, per (token, kv head) scale */
+  ARENO_DT_FP8_E4M3 = 4  /* OCP e4m3fn codes, per (token, kv head) scale */
+};
+
+enum areno_status {
+  ARENO_OK = 0,
+  ARENO_ERR_INVALID_ARGUMENT = -1, /* null pointer, non-positive size, inconsistent shapes */
+  ARENO_ERR_UNSUPPORTED = -2,      /* dtype / head_dim / head-ratio combination with no kernel */
+  ARENO_ERR_WORKSPACE = -3,        /* workspace pointer null or too small */
+  ARENO_ERR_LAUNCH = -4            /* the HIP runtime refused a launch */
+};
+
+/* The paged pools of one layer.  k_scale/v_scale are NULL unless cache_dtype is I8 or FP8_E4M3. */
+typedef struct areno_paged_cache {
+  void* k;
+  void* v;
+  void* k_scale;
+  void* v_scale;
+  int64_t num_blocks;
+  int32_t block_size;
+  int32_t kv_heads;
+  int32_t head_dim;
+  int32_t cache_dtype; /* enum areno_dtype */
+  int32_t scale_dtype; /* ARENO_DT_F16 or ARENO_DT_F32; ignored for unquantized caches */
+} areno_paged_cache;
+
+int areno_hip_abi_version(void);
+const char* areno_hip_status_string(int status);
+const char* areno_hip_last_error(void);
+
+/*
+ * Prefill cache store: cache[block_ids[t], block_offsets[t], h, :] = quantize(k[t, h, :]) (same for v), and the
+ * row's scale to scale[block_ids[t], block_offsets[t], h] for quantized caches.
+ * Replaces _store_prefill_cache's two index_put_ calls
+ * (areno/engine/layers/attention_backend/infer.py:245-263).
+ *   k, v          device [tokens, kv_heads, head_dim], in_dtype (must equal cache_dtype for unquantized caches)
+ *   block_ids     device [tokens] int64,  block_offsets device [tokens] int64
+ * Rows whose (id, offset) fall outside the pool are skipped.
+ */
+int areno_hip_cache_write(const areno_paged_cache* cache, const void* k, const void* v, int32_t in_dtype,
+                          int64_t tokens, const int64_t* block_ids, const int64_t* block_offsets, void* stream);
+
+/*
+ * Decode cache append: row b goes to cache[block_table[b, L_b / block_size], L_b % block_size] with
+ * L_b = cache_seqlens[b].  Replaces paged_decode_update_kernel (areno/accel/csrc/attention.cu:526-553) and
+ * _store_decode_cache (attention_backend/infer.py:266-288); quantizes when the cache is I8 / FP8.
+ *   k_update, v_update   device [batch, kv_heads, head_dim], in_dtype
+ */
+int areno_hip_cache_write_decode(const areno_paged_cache* cache, const void* k_update, const void* v_update,
+                                 int32_t in_dtype, int32_t batch, const int32_t* block_table, int32_t max_blocks,
+                                 const int32_t* cache_seqlens, void* stream);
+
+/*
+ * Bytes of device workspace areno_hip_paged_decode needs for these shapes (split-KV partials).
+ * num_splits is the caller's hint (the reference passes 8, attention_backend/infer.py:240);
+ * 1 forces a single partial per row, anything else lets the library pick the chunking.
+ * Returns 0 for invalid shapes.
+ */
+size_t areno_hip_paged_decode_workspace_bytes(int32_t batch, int32_t q_heads, int32_t head_dim, int32_t block_size,
+                                              int32_t max_blocks, int32_t num_splits);
+
+/*
+ * Single-token paged causal attention, the whole op of areno_paged_causal_attention_decode_forward_cuda
+ * (areno/accel/csrc/attention.cu:926-1020; pybind name areno_paged_causal_attention_decode_forward,
+ * areno/accel/csrc/extension.cpp:184):
+ *   1. if k_update/v_update are non-NULL, append them (areno_hip_cache_write_decode);
+ *   2. split-KV pass over keys [first_allowed, L_b], first_allowed = max(0, L_b - window_left) when
+ *      window_left >= 0 else 0; query head h reads kv head h / (q_heads / kv_heads);
+ *   3. log-sum-exp merge of the partials, normalise, cast to q_dtype.
+ *   q, out        device [batch, q_heads, head_dim], q_dtype (F16/BF16; F32 with an F32 cache)
+ *   workspace     device, at least areno_hip_paged_decode_workspace_bytes(...) bytes, 256-byte aligned
+ */
+int areno_hip_paged_decode(const areno_paged_cache* cache, const void* q, const void* k_update, const void* v_update,
+                           void* out, int32_t q_dtype, int32_t batch, int32_t q_heads, const int32_t* block_table,
+                           int32_t max_blocks, const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
+                           float softmax_scale, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Packed causal self-attention over new tokens only, GQA without expanding KV:
+ * areno_varlen_causal_attention_forward_cuda (areno/accel/csrc/attention.cu:813-861; pybind name
+ * areno_varlen_causal_attention_forward, extension.cpp:182).  Token t of the sequence starting at
+ * cu_seqlens[s] sees keys [max(cu_seqlens[s], t - window_left), t] (all of [cu_seqlens[s], t] when window_left < 0).
+ *   q, out  device [tokens, q_heads, head_dim];  k, v  device [tokens, kv_heads, head_dim];  all `dtype`
+ *   cu_seqlens  device [num_seqs + 1] int32
+ */
+int areno_hip_varlen_attention(const void* q, const void* k, const void* v, void* out, int32_t dtype, int64_t tokens,
+                               int32_t q_heads, int32_t kv_heads, int32_t head_dim, const int32_t* cu_seqlens,
+                               int32_t num_seqs, int32_t window_left, float softmax_scale, void* stream);
+
+/*
+ * Causal prefill of new queries over paged (optionally quantized) KV; the new tokens' K/V must already be in
+ * the cache (areno_hip_cache_write).  Query i of sequence s sits at absolute position context_lens[s] + i and sees
+ * keys [0, that] (clipped on the left by window_left when >= 0).  No counterpart kernel in the reference (its
+ * chunked prefill never re-reads earlier chunks, areno/engine/data/rollout_state.py:121-172); semantics are those of
+ * _reference_attention with query_start = context_lens[s] (areno/accel/attention.py:25-41).
+ *   q, out        device [tokens, q_heads, head_dim], q_dtype (F16/BF16)
+ *   cu_seqlens_q  device [num_seqs + 1] int32;  context_lens device [num_seqs] int32
+ *   block_table   device [num_seqs, max_blocks] int32
+ */
+int areno_hip_paged_varlen_prefill(const areno_paged_cache* cache, const void* q, void* out, int32_t q_dtype,
+                                   int64_t tokens, int32_t q_heads, int32_t num_seqs, const int32_t* block_table,
+                                   int32_t max_blocks, const int32_t* cu_seqlens_q, const int32_t* context_lens,
+                                   int32_t window_left, float softmax_scale, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ARENO_HIP_H */

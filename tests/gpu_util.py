@@ -1,0 +1,68 @@
+"""Helpers shared by the GPU parity tests (imported only by tests)."""
+
+from __future__ import annotations
+
+import torch
+
+from areno_amd import workloads
+from areno_amd.accel import attention as ops
+from oracle import attention_ref as ar
+from oracle import quant_ref as qr
+
+DEV = "cuda:0"
+BF16_MAX_ABS, BF16_MEAN_ABS = 2e-2, 2e-3  # bf16 / fp16 / fp32 KV vs the fp32 reference
+QUANT_MAX_ABS = 5e-2  # int8 / fp8 KV vs the same reference on the dequantized cache
+
+
+def gpu_quantize(x: torch.Tensor, cache_dtype: torch.dtype):
+    """Quantize ``x (N, Hkv, D)`` with the HIP cache-write kernel (one page per token)."""
+    n, hkv, d = x.shape
+    sdt = torch.float16 if cache_dtype == torch.int8 else torch.float32
+    kc = torch.empty((n, 1, hkv, d), dtype=cache_dtype, device=x.device)
+    vc = torch.empty_like(kc)
+    ks = torch.empty((n, 1, hkv), dtype=sdt, device=x.device)
+    vs = torch.empty_like(ks)
+    ids = torch.arange(n, device=x.device, dtype=torch.int64)
+    ops.areno_paged_cache_write(x, x, kc, vc, ids, torch.zeros_like(ids), k_scale=ks, v_scale=vs)
+    return kc.view(n, hkv, d), ks.view(n, hkv)
+
+
+def dequant_cpu(cache: torch.Tensor, scale: torch.Tensor | None) -> torch.Tensor:
+    c = cache.cpu()
+    if scale is None:
+        return c.float()
+    out = qr.dequantize(c, scale.cpu())
+    # poisoned (never-read) slots carry NaN scales; keep them NaN so a stray read shows up
+    return out
+
+
+def run_decode(w: workloads.DecodeWorkload, *, window_left=None, num_splits=8):
+    return ops.areno_paged_causal_attention_decode(
+        w.q, w.k_update, w.v_update, w.k_cache, w.v_cache, w.block_table, w.cache_seqlens,
+        window_left=window_left, num_splits=num_splits, softmax_scale=w.softmax_scale,
+        k_scale=w.k_scale, v_scale=w.v_scale,
+    )  # fmt: skip
+
+
+def expected_decode(w: workloads.DecodeWorkload, *, window_left=None, rows=None):
+    """Oracle on the post-step cache (dequantized for int8/fp8), optionally on a subset of rows."""
+    kc = dequant_cpu(w.k_cache, w.k_scale)
+    vc = dequant_cpu(w.v_cache, w.v_scale)
+    q, table, lens = w.q.cpu().float(), w.block_table.cpu(), w.cache_seqlens.cpu()
+    if rows is not None:
+        q, table, lens = q[rows], table[rows], lens[rows]
+    return ar.ref_paged_decode(q, kc, vc, table, lens, ar.window_left_arg(window_left), w.softmax_scale)
+
+
+def assert_close(got: torch.Tensor, want: torch.Tensor, max_abs: float, mean_abs: float | None = None, what=""):
+    got = got.detach().cpu().float()
+    assert torch.isfinite(got).all(), f"{what}: non-finite output"
+    err = (got - want.float()).abs()
+    assert err.max().item() <= max_abs, f"{what}: max-abs {err.max().item():.4g} > {max_abs}"
+    if mean_abs is not None:
+        assert err.mean().item() <= mean_abs, f"{what}: mean-abs {err.mean().item():.4g} > {mean_abs}"
+    return err.max().item(), err.mean().item()
+
+
+def tolerances(kv: str):
+    return (QUANT_MAX_ABS, None) if kv in ("int8", "fp8") else (BF16_MAX_ABS, BF16_MEAN_ABS)

@@ -1,0 +1,108 @@
+"""Varlen prefill ops vs the CPU oracle: packed new-token attention (the reference's op) and
+causal prefill over paged, optionally quantized KV with a cached context (this build's extension)."""
+
+import pytest
+import torch
+
+from areno_amd import workloads
+from areno_amd.accel import attention as ops
+from oracle import attention_ref as ar
+from tests.gpu_util import DEV, assert_close, dequant_cpu, gpu_quantize, tolerances
+
+pytestmark = pytest.mark.gpu
+
+
+def _packed(lens, hq, hkv, d, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    t = sum(lens)
+    q, k, v = (torch.randn(t, h, d, generator=g).to(dtype) for h in (hq, hkv, hkv))
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    return q, k, v, cu
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("window_left", [None, 0, 7])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (28, 4, 128), (4, 4, 80)])
+def test_varlen_new_tokens_only(dtype, window_left, hq, hkv, d):
+    q, k, v, cu = _packed([5, 1, 130, 0, 67], hq, hkv, d, dtype)
+    out = ops.areno_varlen_causal_attention(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), window_left=window_left)
+    want = ar.ref_varlen(q, k, v, cu, ar.window_left_arg(window_left), d**-0.5)
+    assert out.dtype == dtype and out.shape == q.shape
+    assert_close(out, want, *tolerances("bf16"), what="varlen")
+
+
+def _expected_prefill(w, window_left=None):
+    kc, vc = dequant_cpu(w.k_cache, w.k_scale), dequant_cpu(w.v_cache, w.v_scale)
+    return ar.ref_paged_varlen_prefill(w.q.cpu().float(), kc, vc, w.block_table.cpu(), w.cu_seqlens_q.cpu(),
+                                       w.context_lens.cpu(), ar.window_left_arg(window_left), w.softmax_scale)  # fmt: skip
+
+
+def _run_prefill(w, window_left=None):
+    return ops.areno_paged_varlen_causal_attention(
+        w.q, w.k_cache, w.v_cache, w.block_table, w.cu_seqlens_q, w.context_lens,
+        window_left=window_left, softmax_scale=w.softmax_scale, k_scale=w.k_scale, v_scale=w.v_scale,
+    )  # fmt: skip
+
+
+@pytest.mark.parametrize("kv", ["bf16", "fp16", "int8", "fp8"])
+@pytest.mark.parametrize("window_left", [None, 33])
+def test_paged_prefill_small(kv, window_left):
+    w = workloads.cfg4_prefill(kv, device=DEV, seqs=5, new_hi=70, ctx_hi=300, quantize_fn=gpu_quantize, seed=5)
+    out = _run_prefill(w, window_left)
+    assert_close(out, _expected_prefill(w, window_left), *tolerances(kv), what=f"paged prefill {kv}")
+
+
+@pytest.mark.parametrize("hq,hkv,d,bs", [(28, 4, 128, 16), (8, 8, 64, 32), (6, 2, 128, 256), (4, 1, 96, 16)])
+def test_paged_prefill_shapes(hq, hkv, d, bs):
+    g = torch.Generator().manual_seed(d + hq)
+    new = torch.tensor([1, 64, 17, 129])
+    ctx = torch.tensor([0, 5, 200, 63])
+    w = workloads.make_prefill_workload("shapes", seed=3, new_lens=new, ctx_lens=ctx, hq=hq, hkv=hkv, d=d, bs=bs,
+                                        kv="bf16", device=DEV)  # fmt: skip
+    assert_close(_run_prefill(w), _expected_prefill(w), *tolerances("bf16"), what="prefill shapes")
+
+
+def test_write_then_prefill_then_decode_are_consistent():
+    """The three ops agree with each other: cache write of the new tokens, prefill with ctx,
+    and n = 1 prefill == decode without append."""
+    w = workloads.cfg4_prefill("fp8", device=DEV, seqs=6, new_hi=40, ctx_hi=200, quantize_fn=gpu_quantize, seed=9)
+    ops.areno_paged_cache_write(w.k_new, w.v_new, w.k_cache, w.v_cache, w.cache_block_ids, w.cache_block_offsets,
+                                k_scale=w.k_scale, v_scale=w.v_scale)  # fmt: skip
+    out = _run_prefill(w)
+    assert_close(out, _expected_prefill(w), *tolerances("fp8"), what="after write")
+    # last query of each sequence == a decode row whose token is already cached: compare through the oracle
+    cu = w.cu_seqlens_q.cpu().long()
+    last = cu[1:] - 1
+    lens = (w.context_lens.cpu().long() + (cu[1:] - cu[:-1]) - 1).int()
+    kc, vc = dequant_cpu(w.k_cache, w.k_scale), dequant_cpu(w.v_cache, w.v_scale)
+    dec = ar.ref_paged_decode(w.q.cpu().float()[last], kc, vc, w.block_table.cpu(), lens, -1, w.softmax_scale)
+    assert_close(out[last.to(DEV)], dec, *tolerances("fp8"), what="prefill last row vs decode oracle")
+
+
+def test_cfg4_reduced():
+    """cfg 4 shape (32/8 heads, D=128, fp8) with the full range of new lengths and a reduced context range."""
+    w = workloads.cfg4_prefill("fp8", device=DEV, seqs=6, new_hi=512, ctx_hi=3000, quantize_fn=gpu_quantize)
+    assert_close(_run_prefill(w), _expected_prefill(w), *tolerances("fp8"), what="cfg4 reduced")
+
+
+def test_dense_causal_attention_wrapper():
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(2, 4, 9, 64, generator=g).bfloat16()
+    k = torch.randn(2, 4, 21, 64, generator=g).bfloat16()
+    v = torch.randn(2, 4, 21, 64, generator=g).bfloat16()
+    out = ops.areno_causal_attention(q.to(DEV), k.to(DEV), v.to(DEV), query_start=12, window_left=6)
+    want = ar.ref_attention(q, k, v, 12, 6, 64**-0.5)
+    assert_close(out, want, *tolerances("bf16"), what="dense")
+
+
+def test_varlen_error_behaviour():
+    q, k, v, cu = _packed([4, 4], 4, 2, 64, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="requires CUDA"):
+        ops.areno_varlen_causal_attention(q, k, v, cu)
+    q, k, v, cu = (t.to(DEV) for t in (q, k, v, cu))
+    with pytest.raises(ValueError, match="int32 1D cu_seqlens"):
+        ops.areno_varlen_causal_attention(q, k, v, cu.long())
+    with pytest.raises(ValueError, match="token count mismatch"):
+        ops.areno_varlen_causal_attention(q, k[:-1], v, cu)
+    with pytest.raises(ValueError, match="divisible by kv heads"):
+        ops.areno_varlen_causal_attention(q[:, :3], k, v, cu)
