@@ -154,8 +154,9 @@ int launch_write(const areno_paged_cache* cache, const void* k, const void* v, i
                  const int64_t* ids, const int64_t* offs, const int32_t* table, int32_t max_blocks,
                  const int32_t* seqlens, void* stream, const char* op) {
   if (int rc = validate_cache(cache, op)) return rc;
-  if (k == nullptr || v == nullptr) return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: k/v pointer is NULL", op);
   if (tokens < 0) return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: negative token count", op);
+  if (tokens > 0 && (k == nullptr || v == nullptr))
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: k/v pointer is NULL", op);
   if (cache->head_dim > kMaxPerLane * kWave)
     return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim %d > %d", op, cache->head_dim, kMaxPerLane * kWave);
   if (in_dtype != ARENO_DT_F32 && in_dtype != ARENO_DT_F16 && in_dtype != ARENO_DT_BF16)

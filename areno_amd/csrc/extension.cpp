@@ -8,8 +8,8 @@
 // entry points (cache write, paged prefill, scales) are this build's extension of the path.
 
 #include <ATen/ATen.h>
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
 
 #include "../../include/areno_hip.h"
@@ -32,8 +32,10 @@ void check_status(int status, const char* op) {
   TORCH_CHECK(status == ARENO_OK, op, " failed: ", areno_hip_status_string(status), " (", areno_hip_last_error(), ")");
 }
 
+// ROCm builds of PyTorch expose HIP devices under the "cuda" device type; these are its own
+// stream / guard accessors for that arrangement.
 void* current_stream(const at::Tensor& t) {
-  return static_cast<void*>(c10::hip::getCurrentHIPStream(t.device().index()).stream());
+  return static_cast<void*>(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream());
 }
 
 areno_paged_cache describe_cache(const at::Tensor& k_cache, const at::Tensor& v_cache,
@@ -121,7 +123,7 @@ at::Tensor paged_decode_forward_impl(at::Tensor q, at::Tensor k_update, at::Tens
   TORCH_CHECK(q.size(1) % k_cache.size(2) == 0, op, " q heads must be divisible by kv heads");
   TORCH_CHECK(num_splits >= 1, op, " num_splits must be >= 1");
 
-  const c10::hip::OptionalHIPGuard guard(device_of(q));
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(q));
   auto out = at::empty_like(q);
   if (q.size(0) == 0) return out;
   const size_t ws_bytes = areno_hip_paged_decode_workspace_bytes(
@@ -167,7 +169,7 @@ at::Tensor varlen_forward(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor c
   TORCH_CHECK(q.size(1) % k.size(1) == 0, op, " q heads must be divisible by kv heads");
   TORCH_CHECK(q.size(2) == k.size(2) && q.size(2) == v.size(2), op, " head dim mismatch");
   TORCH_CHECK(cu_seqlens.size(0) >= 2, op, " cu_seqlens must contain at least one sequence");
-  const c10::hip::OptionalHIPGuard guard(device_of(q));
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(q));
   auto out = at::empty_like(q);
   const int status = areno_hip_varlen_attention(
       q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dtype_code(q, op, "q"), q.size(0),
@@ -196,7 +198,7 @@ void cache_write(at::Tensor k, at::Tensor v, at::Tensor k_cache, at::Tensor v_ca
               " token count mismatch");
   TORCH_CHECK(k.size(1) == k_cache.size(2) && v.size(1) == v_cache.size(2), op, " head mismatch");
   TORCH_CHECK(k.size(2) == k_cache.size(3) && v.size(2) == v_cache.size(3), op, " head dim mismatch");
-  const c10::hip::OptionalHIPGuard guard(device_of(k));
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(k));
   const int status =
       areno_hip_cache_write(&cache, k.data_ptr(), v.data_ptr(), dtype_code(k, op, "k"), k.size(0),
                             block_ids.data_ptr<int64_t>(), block_offsets.data_ptr<int64_t>(), current_stream(k));
@@ -231,7 +233,7 @@ at::Tensor paged_varlen_forward(at::Tensor q, at::Tensor k_cache, at::Tensor v_c
               " sequence count mismatch");
   TORCH_CHECK(q.size(2) == k_cache.size(3), op, " head dim mismatch");
   TORCH_CHECK(q.size(1) % k_cache.size(2) == 0, op, " q heads must be divisible by kv heads");
-  const c10::hip::OptionalHIPGuard guard(device_of(q));
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(q));
   auto out = at::empty_like(q);
   const int status = areno_hip_paged_varlen_prefill(
       &cache, q.data_ptr(), out.data_ptr(), dtype_code(q, op, "q"), q.size(0), static_cast<int32_t>(q.size(1)),

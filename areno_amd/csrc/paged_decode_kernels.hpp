@@ -128,7 +128,10 @@ __device__ __forceinline__ void k_pairs(const uint4_t& r, typename KVTraits<KIND
   using P = typename KVTraits<KIND>::pair_t;
   if constexpr (KIND == KV_BF16 || KIND == KV_F16) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) out[j] = __builtin_bit_cast(P, r[j]);
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t word = r[j];  // copy first: bit_cast straight from a vector-element lvalue reads element 0
+      out[j] = __builtin_bit_cast(P, word);
+    }
   } else if constexpr (KIND == KV_I8) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {

@@ -18,7 +18,7 @@ def _inputs(t, hkv, d, dtype, seed=0):
     x[:, 0] = 0
     if t > 4:
         x[:, 1] *= 1e-9
-        x[:, 2] *= 3e4
+        x[:, 2] *= 3e4 if dtype != torch.float16 else 1e3  # stay finite in fp16: non-finite rows are outside the contract
         x[:, 3, :, 0] = 0.5  # exact halves after scaling exercise round-half-even
     return x[0].to(dtype), x[1].to(dtype)
 
