@@ -1,0 +1,114 @@
+"""ctypes mirror of ``include/areno_hip.h``: calls ``libareno_hip.so`` with raw device pointers.
+
+This is the binding a non-PyTorch host would write; the benchmark and the C-ABI tests use it to drive
+single kernels (stage masks) without going through the torch extension.  Tensors are only used here to
+obtain ``data_ptr()`` and shapes.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from areno_amd.accel._extension import library_path
+
+DT_F32, DT_F16, DT_BF16, DT_I8, DT_FP8_E4M3 = 0, 1, 2, 3, 4
+STAGE_APPEND, STAGE_SPLIT, STAGE_REDUCE, STAGE_ALL = 1, 2, 4, 7
+
+_DTYPE_CODES = {
+    torch.float32: DT_F32,
+    torch.float16: DT_F16,
+    torch.bfloat16: DT_BF16,
+    torch.int8: DT_I8,
+    torch.float8_e4m3fn: DT_FP8_E4M3,
+}
+
+
+class PagedCache(ctypes.Structure):
+    """``struct areno_paged_cache``."""
+
+    _fields_ = [
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("k_scale", ctypes.c_void_p),
+        ("v_scale", ctypes.c_void_p),
+        ("num_blocks", ctypes.c_int64),
+        ("block_size", ctypes.c_int32),
+        ("kv_heads", ctypes.c_int32),
+        ("head_dim", ctypes.c_int32),
+        ("cache_dtype", ctypes.c_int32),
+        ("scale_dtype", ctypes.c_int32),
+    ]
+
+
+_LIB: ctypes.CDLL | None = None
+_P, _I32, _I64, _F, _SZ = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_size_t
+
+
+def lib() -> ctypes.CDLL:
+    global _LIB
+    if _LIB is None:
+        try:
+            handle = ctypes.CDLL(library_path())
+        except OSError as exc:
+            raise RuntimeError(
+                f"libareno_hip.so could not be loaded ({exc}); build it with `python setup.py build_ext --inplace`"
+            ) from exc
+        handle.areno_hip_last_error.restype = ctypes.c_char_p
+        handle.areno_hip_status_string.restype = ctypes.c_char_p
+        handle.areno_hip_paged_decode_workspace_bytes.restype = _SZ
+        handle.areno_hip_paged_decode_workspace_bytes.argtypes = [_I32] * 6
+        handle.areno_hip_cache_write.argtypes = [_P, _P, _P, _I32, _I64, _P, _P, _P]
+        handle.areno_hip_cache_write_decode.argtypes = [_P, _P, _P, _I32, _I32, _P, _I32, _P, _P]
+        decode_args = [_P, _P, _P, _P, _P, _I32, _I32, _I32, _P, _I32, _P, _I32, _I32, _F, _P, _SZ]
+        handle.areno_hip_paged_decode.argtypes = decode_args + [_P]
+        handle.areno_hip_paged_decode_stages.argtypes = decode_args + [_I32, _P]
+        handle.areno_hip_varlen_attention.argtypes = [_P, _P, _P, _P, _I32, _I64, _I32, _I32, _I32, _P, _I32, _I32, _F, _P]
+        handle.areno_hip_paged_varlen_prefill.argtypes = [_P, _P, _P, _I32, _I64, _I32, _I32, _P, _I32, _P, _P, _I32, _F, _P]
+        _LIB = handle
+    return _LIB
+
+
+def check(status: int, op: str) -> None:
+    if status != 0:
+        handle = lib()
+        raise RuntimeError(
+            f"{op} failed: {handle.areno_hip_status_string(status).decode()} ({handle.areno_hip_last_error().decode()})"
+        )
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    return _DTYPE_CODES[t.dtype]
+
+
+def describe_cache(k_cache, v_cache, k_scale=None, v_scale=None) -> PagedCache:
+    nb, bs, hkv, d = k_cache.shape
+    return PagedCache(
+        k_cache.data_ptr(), v_cache.data_ptr(),
+        None if k_scale is None else k_scale.data_ptr(), None if v_scale is None else v_scale.data_ptr(),
+        nb, bs, hkv, d, dtype_code(k_cache),
+        DT_F32 if k_scale is None else dtype_code(k_scale),
+    )  # fmt: skip
+
+
+def current_stream_ptr() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def decode_workspace_bytes(batch, q_heads, head_dim, block_size, max_blocks, num_splits=8) -> int:
+    return int(lib().areno_hip_paged_decode_workspace_bytes(batch, q_heads, head_dim, block_size, max_blocks, num_splits))
+
+
+def paged_decode(cache: PagedCache, q, k_update, v_update, out, block_table, cache_seqlens, workspace, *,
+                 window_left=-1, num_splits=8, softmax_scale=None, stages=STAGE_ALL, stream=None) -> None:  # fmt: skip
+    """``areno_hip_paged_decode_stages`` on raw pointers; ``workspace`` is a uint8 device tensor."""
+    scale = float(softmax_scale if softmax_scale is not None else q.shape[-1] ** -0.5)
+    status = lib().areno_hip_paged_decode_stages(
+        ctypes.byref(cache), q.data_ptr(), None if k_update is None else k_update.data_ptr(),
+        None if v_update is None else v_update.data_ptr(), out.data_ptr(), dtype_code(q), q.shape[0], q.shape[1],
+        block_table.data_ptr(), block_table.shape[1], cache_seqlens.data_ptr(), int(window_left), int(num_splits),
+        scale, workspace.data_ptr(), workspace.numel(), int(stages),
+        current_stream_ptr() if stream is None else stream,
+    )  # fmt: skip
+    check(status, "areno_hip_paged_decode")

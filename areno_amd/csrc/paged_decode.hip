@@ -172,6 +172,17 @@ extern "C" int areno_hip_paged_decode(const areno_paged_cache* cache, const void
                                       int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
                                       const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
                                       float softmax_scale, void* workspace, size_t workspace_bytes, void* stream) {
+  return areno_hip_paged_decode_stages(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table,
+                                       max_blocks, cache_seqlens, window_left, num_splits, softmax_scale, workspace,
+                                       workspace_bytes, ARENO_STAGE_ALL, stream);
+}
+
+extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, const void* q, const void* k_update,
+                                             const void* v_update, void* out, int32_t q_dtype, int32_t batch,
+                                             int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
+                                             const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
+                                             float softmax_scale, void* workspace, size_t workspace_bytes,
+                                             int32_t stages, void* stream) {
   using namespace areno;
   const char* op = "areno_hip_paged_decode";
   if (int rc = validate_paged_cache(cache, op)) return rc;
@@ -200,7 +211,7 @@ extern "C" int areno_hip_paged_decode(const areno_paged_cache* cache, const void
   if (workspace == nullptr || workspace_bytes < need)
     return fail(ARENO_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", op, need, workspace_bytes);
 
-  if (k_update != nullptr) {
+  if (k_update != nullptr && (stages & ARENO_STAGE_APPEND)) {
     if (int rc = areno_hip_cache_write_decode(cache, k_update, v_update, q_dtype, batch, block_table, max_blocks,
                                               cache_seqlens, stream))
       return rc;
@@ -249,7 +260,9 @@ extern "C" int areno_hip_paged_decode(const areno_paged_cache* cache, const void
     }
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (fast != nullptr) {
+  if (!(stages & ARENO_STAGE_SPLIT)) {
+    // skip
+  } else if (fast != nullptr) {
     const dim3 grid(ch.max_parts, batch, cache->kv_heads / p.heads_per_wg);
     hipLaunchKernelGGL(fast, grid, dim3(kDecodeThreads), 0, s, p);
   } else {
@@ -257,6 +270,7 @@ extern "C" int areno_hip_paged_decode(const areno_paged_cache* cache, const void
     hipLaunchKernelGGL(decode_split_generic_kernel, grid, dim3(kWave), 0, s, p);
   }
   if (int rc = check_launch(op)) return rc;
+  if (!(stages & ARENO_STAGE_REDUCE)) return ARENO_OK;
   const int rblocks = (batch * q_heads + kReduceRows - 1) / kReduceRows;
   hipLaunchKernelGGL(decode_reduce_kernel, dim3(rblocks), dim3(kReduceRows * kWave), 0, s, p);
   return check_launch(op);

@@ -1,0 +1,299 @@
+"""Benchmark of the paged decode-attention hot path on one MI355X.
+
+A step is one call of the decode op (fused cache append + split-KV GQA attention + merge) for one layer over
+one batch of synthetic sequences.  The headline workload is the Qwen2.5-7B-like shape (B=64, 28 q heads /
+4 kv heads, D=128, page 16, contexts uniform in [512, 4096]) with a bf16 KV cache; the same shape with an
+int8 cache (quantizing append included) and the fp8 rollout shape are measured too and reported under
+"workloads".  Inputs are resident in HBM before timing starts.  Steps rotate over several copies of the KV
+pools so that the working set exceeds the 256 MB Infinity Cache and the reads really come from HBM.
+
+Prints ONE JSON line.  `value` is microseconds per step measured over exactly `--steps` steps replayed from
+HIP graphs (how the engine runs decode); `roofline` is for the split-KV kernel alone: algorithmic bytes of one
+launch divided by its mean duration measured with events on the launch stream; `cpu_baseline` is the CPU
+oracle timed on the host cores on a stated sample.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+POOL_TARGET_BYTES = 1.3e9  # rotate over at least this much distinct KV
+
+
+def _clone_pools(w, copies):
+    pools = [(w.k_cache, w.v_cache, w.k_scale, w.v_scale)]
+    for _ in range(copies - 1):
+        pools.append(tuple(None if t is None else t.clone() for t in pools[0]))
+    return pools
+
+
+def _gpu_quantize(x, cache_dtype):
+    import torch
+
+    from areno_amd.accel import attention as ops
+
+    n, hkv, d = x.shape
+    sdt = torch.float16 if cache_dtype == torch.int8 else torch.float32
+    kc = torch.empty((n, 1, hkv, d), dtype=cache_dtype, device=x.device)
+    vc = torch.empty_like(kc)
+    ks = torch.empty((n, 1, hkv), dtype=sdt, device=x.device)
+    vs = torch.empty_like(ks)
+    ids = torch.arange(n, device=x.device, dtype=torch.int64)
+    ops.areno_paged_cache_write(x, x, kc, vc, ids, torch.zeros_like(ids), k_scale=ks, v_scale=vs)
+    return kc.view(n, hkv, d), ks.view(n, hkv)
+
+
+def _step(w, pool):
+    from areno_amd.accel import attention as ops
+
+    kc, vc, ks, vs = pool
+    return ops.areno_paged_causal_attention_decode(
+        w.q, w.k_update, w.v_update, kc, vc, w.block_table, w.cache_seqlens,
+        softmax_scale=w.softmax_scale, k_scale=ks, v_scale=vs,
+    )  # fmt: skip
+
+
+def _parity_sample(w, out, rows=4):
+    """Max-abs error of the first rows against the CPU oracle (dequantized cache for int8/fp8)."""
+    from oracle import attention_ref as ar
+    from oracle import quant_ref as qr
+
+    if w.k_scale is None:
+        kc, vc = w.k_cache.cpu().float(), w.v_cache.cpu().float()
+    else:
+        kc, vc = qr.dequantize(w.k_cache.cpu(), w.k_scale.cpu()), qr.dequantize(w.v_cache.cpu(), w.v_scale.cpu())
+    want = ar.ref_paged_decode(
+        w.q[:rows].cpu().float(), kc, vc, w.block_table[:rows].cpu(), w.cache_seqlens[:rows].cpu(), -1, w.softmax_scale
+    )
+    return float((out[:rows].cpu().float() - want).abs().max())
+
+
+def measure_decode(w, steps, warmup, *, kernel_iters=60):
+    """Time the whole op (graph replay and eager) and each kernel of it; returns a dict of numbers."""
+    import torch
+
+    from areno_amd.accel import cabi
+
+    pool_bytes = sum(t.numel() * t.element_size() for t in (w.k_cache, w.v_cache, w.k_scale, w.v_scale) if t is not None)
+    copies = max(2, int(-(-POOL_TARGET_BYTES // pool_bytes)))
+    pools = _clone_pools(w, copies)
+    alg_bytes = w.algorithmic_bytes()
+
+    out = _step(w, pools[0])
+    torch.cuda.synchronize()
+    parity = _parity_sample(w, out)
+
+    # ---- whole op, replayed from HIP graphs (one graph = one pass over all pool copies) --------------
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for pool in pools:
+            _step(w, pool)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+
+    def capture(n):
+        g = torch.cuda.CUDAGraph()
+        keep = []
+        with torch.cuda.graph(g):
+            for i in range(n):
+                keep.append(_step(w, pools[i % copies]))
+        return g, keep
+
+    full, keep_full = capture(copies)
+    rem_n = steps % copies
+    rem, keep_rem = capture(rem_n) if rem_n else (None, None)
+    for _ in range(max(1, -(-warmup // copies))):
+        full.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps // copies):
+        full.replay()
+    if rem is not None:
+        rem.replay()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    us_graph = (t1 - t0) / steps * 1e6
+    # graph replays must reproduce the eager result (checked on the first pool)
+    graph_ok = bool(torch.equal(keep_full[0], out))
+
+    # ---- whole op, eager launches (host launch overhead included) ----------------------------------------
+    for i in range(warmup):
+        _step(w, pools[i % copies])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        _step(w, pools[i % copies])
+    torch.cuda.synchronize()
+    us_eager = (time.perf_counter() - t0) / steps * 1e6
+
+    # ---- per-kernel durations: events on the launch stream around back-to-back launches through the C ABI ---
+    b, hq, hkv, d, bs = w.shape
+    ws_bytes = cabi.decode_workspace_bytes(b, hq, d, bs, w.block_table.shape[1])
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=w.q.device)
+    caches = [cabi.describe_cache(*pool) for pool in pools]
+    out2 = torch.empty_like(w.q)
+
+    def time_stage(stage):
+        def launch(i):
+            cabi.paged_decode(caches[i % copies], w.q, w.k_update, w.v_update, out2, w.block_table, w.cache_seqlens,
+                              workspace, softmax_scale=w.softmax_scale, stages=stage)  # fmt: skip
+
+        for i in range(copies):
+            launch(i)
+        torch.cuda.synchronize()
+        samples = []
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(kernel_iters):
+                launch(i)
+            e1.record()
+            e1.synchronize()
+            samples.append(e0.elapsed_time(e1) * 1e3 / kernel_iters)
+        return statistics.median(samples)
+
+    us_split = time_stage(cabi.STAGE_SPLIT)
+    us_reduce = time_stage(cabi.STAGE_REDUCE)
+    us_append = time_stage(cabi.STAGE_APPEND)
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out), "C-ABI staged run disagrees with the op"
+
+    gbps = alg_bytes / (us_split * 1e-6) / 1e9
+    return {
+        "workload": w.name,
+        "us_per_step": us_graph,
+        "us_per_step_eager": us_eager,
+        "kernel_us": {"append": us_append, "split": us_split, "reduce": us_reduce},
+        "tokens_per_s": w.q.shape[0] / (us_graph * 1e-6),
+        "algorithmic_bytes": alg_bytes,
+        "op_gbps": alg_bytes / (us_graph * 1e-6) / 1e9,
+        "roofline": {
+            "bound": "hbm", "kernel": "decode_split_kernel", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": gbps / HBM_PEAK_GBPS, "traffic": None,
+        },  # fmt: skip
+        "pool_copies": copies,
+        "parity_max_abs_4rows": parity,
+        "graph_replay_matches_eager": graph_ok,
+        "kv_tokens": {"logical": w.logical_tokens, "unique": w.unique_tokens},
+    }
+
+
+def cpu_baseline(w, rows=16, repeats=3):
+    """The CPU oracle (PyTorch restatement of the reference's native path) on the first `rows` sequences."""
+    import torch
+
+    from oracle import attention_ref as ar
+    from oracle import quant_ref as qr
+
+    threads = torch.get_num_threads()
+    if w.k_scale is None:
+        kc, vc = w.k_cache.cpu().float(), w.v_cache.cpu().float()
+    else:
+        kc, vc = qr.dequantize(w.k_cache.cpu(), w.k_scale.cpu()), qr.dequantize(w.v_cache.cpu(), w.v_scale.cpu())
+    q, ku, vu = w.q[:rows].cpu().float(), w.k_update[:rows].cpu().float(), w.v_update[:rows].cpu().float()
+    table, lens = w.block_table[:rows].cpu(), w.cache_seqlens[:rows].cpu()
+
+    def once():
+        ar.ref_decode_update(ku, vu, kc, vc, table, lens)
+        return ar.ref_paged_decode(q, kc, vc, table, lens, -1, w.softmax_scale)
+
+    once()
+    times = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        once()
+        times.append(time.perf_counter() - t0)
+    per_step_us = statistics.median(times) * 1e6 * (w.q.shape[0] / rows)
+    return {
+        "value": per_step_us, "unit": "us/step", "cores": threads, "kind": "port",
+        "sample": f"{rows} of {w.q.shape[0]} sequences of {w.name} (fp32 caches, append + gather + attention), "
+                  f"median of {repeats}, scaled by {w.q.shape[0] / rows:g}",
+    }  # fmt: skip
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3"], default=None, help="measure a single workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(
+            "bench.py measures one GPU: the decode path has no cross-GPU step (sequences and heads shard with no "
+            "exchange), so --gpus above 1 is not a configuration of this benchmark.",
+            file=sys.stderr,
+        )
+        return 2
+
+    import torch
+
+    from areno_amd import workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py needs an AMD GPU (torch.cuda.is_available() is False)", file=sys.stderr)
+        return 2
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+
+    builders = {
+        "cfg1": lambda: workloads.cfg1_qwen7b("bf16", device=dev),
+        "cfg2": lambda: workloads.cfg2_qwen7b_int8(device=dev, quantize_fn=_gpu_quantize),
+        "cfg3": lambda: workloads.cfg3_rollout("fp8", device=dev, quantize_fn=_gpu_quantize),
+    }
+    names = [args.only] if args.only else ["cfg1", "cfg2", "cfg3"]
+    results = {}
+    baseline = None
+    for name in names:
+        w = builders[name]()
+        results[name] = measure_decode(w, args.steps, args.warmup)
+        if name == names[0] and not args.no_cpu:
+            baseline = cpu_baseline(w)
+        del w
+        torch.cuda.empty_cache()
+
+    head = results[names[0]]
+    dtype = {"cfg1": "bf16", "cfg2": "int8", "cfg3": "fp8"}[names[0]]
+    line = {
+        "metric": "paged_decode_attn_us_per_step",
+        "value": head["us_per_step"],
+        "unit": "us/step",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["us_per_step"] / 1e3,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype,
+        "data": "synthetic",
+        "config": {
+            "workload": head["workload"],
+            "shape": "B=64 Hq=28 Hkv=4 D=128 page=16 ctx~U[512,4096]" if names[0] != "cfg3" else "B=256 Hq=32 Hkv=8 D=128",
+            "launch": "HIP graph replay, KV pools rotated over >1.3 GB",
+        },
+        "tokens_per_s": head["tokens_per_s"],
+        "hbm_gbps_op": head["op_gbps"],
+        "roofline": head["roofline"],
+        "cpu_baseline": baseline,
+        "workloads": results,
+        "device": torch.cuda.get_device_name(0),
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -108,6 +108,23 @@ int areno_hip_paged_decode(const areno_paged_cache* cache, const void* q, const 
                            float softmax_scale, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The same op with a stage mask, for profilers and benchmarks that time one kernel at a time:
+ * ARENO_STAGE_APPEND (cache write of the update rows), ARENO_STAGE_SPLIT (split-KV pass into the workspace),
+ * ARENO_STAGE_REDUCE (merge of the workspace partials into `out`).  areno_hip_paged_decode is
+ * stages = ARENO_STAGE_ALL.  No counterpart in the reference, whose launcher always runs its three
+ * kernels (areno/accel/csrc/attention.cu:979-1018).
+ */
+#define ARENO_STAGE_APPEND 1
+#define ARENO_STAGE_SPLIT 2
+#define ARENO_STAGE_REDUCE 4
+#define ARENO_STAGE_ALL 7
+int areno_hip_paged_decode_stages(const areno_paged_cache* cache, const void* q, const void* k_update,
+                                  const void* v_update, void* out, int32_t q_dtype, int32_t batch, int32_t q_heads,
+                                  const int32_t* block_table, int32_t max_blocks, const int32_t* cache_seqlens,
+                                  int32_t window_left, int32_t num_splits, float softmax_scale, void* workspace,
+                                  size_t workspace_bytes, int32_t stages, void* stream);
+
+/*
  * Packed causal self-attention over new tokens only, GQA without expanding KV:
  * areno_varlen_causal_attention_forward_cuda (areno/accel/csrc/attention.cu:813-861; pybind name
  * areno_varlen_causal_attention_forward, extension.cpp:182).  Token t of the sequence starting at
