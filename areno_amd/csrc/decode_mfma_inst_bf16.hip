@@ -1,0 +1,8 @@
+// Instantiates the MFMA split-KV decode kernels for one KV-cache element kind (bf16).
+#include "decode_mfma_kernels.hpp"
+
+namespace areno {
+decode_mfma_fn decode_mfma_lookup_bf16(int head_dim, bool scale16) {
+  return decode_mfma_lookup_impl<KV_BF16>(head_dim, scale16);
+}
+}  // namespace areno

@@ -1,0 +1,562 @@
+// Split-KV GQA paged decode on the matrix cores (gfx950), device code.
+//
+// Why MFMA for a bandwidth-bound op: at 70 % of 8 TB/s every SIMD must consume ~2.3 KV bytes per clock
+// and each int8/fp8 byte needs G = q_heads / kv_heads multiply-adds on the QK^T side and G more on the P.V
+// side.  With G = 7 that is more than the vector ALU can issue even with v_dot2, so the VALU kernel
+// (paged_decode_kernels.hpp) tops out well below the HBM roofline.  Here the G query heads of one KV head
+// form the (zero padded) 16-wide N side of v_mfma_f32_16x16x32 tiles; the vector ALU only dequantizes
+// (<= 0.75 op per element) and runs the softmax.
+//
+// Work decomposition (exactly balanced, no host knowledge of the lengths):
+//   * a sequence contributes ceil(visible_keys / 32) tiles of 32 tokens; every workgroup computes the
+//     prefix sum of tile counts over the batch in LDS and takes an equal share of the global tile range
+//     ("wave piece"), so all waves stream the same number of bytes whatever the length distribution;
+//   * a piece that crosses a sequence boundary emits one partial per sequence it touches, into slot
+//     (piece index + sequence index), which is unique and contiguous per sequence; the reduce kernel merges
+//     the slots of each sequence.
+//   * block = 4 wave64; wave w owns KV head z*HW + w % HW, so with kv_heads >= 4 the four waves of a
+//     workgroup read whole pages ([slot][kv_head][D] is contiguous).  Waves never synchronise after the
+//     prefix sum: each has private LDS tiles.
+// Data path per 32-token tile and wave:
+//   global --16 B/lane coalesced loads--> registers (in flight while the previous tile is computed)
+//          --ds_write_b128--> LDS K tile [32][D*es + 16] and V tile (row padding makes every access below
+//          bank-conflict free)
+//   S^T[token][head] = K . Q^T : A = K rows read straight from LDS (8 consecutive dims per lane), B = Q^T held in
+//          registers for the whole sequence; C puts head = lane % 16, 4 tokens per lane.
+//   online softmax in the log2 domain on C; the per-token K scale multiplies S, the V scale multiplies P.
+//   O^T[dim][head] += V^T . P^T : A = V^T through ds_read_b64_tr_b8 / _tr_b16 (the LDS transpose read gives each
+//          lane 8 tokens of one dim), B = P^T which *is* the C layout of S^T (token order chosen to match), so
+//          no cross-lane movement of P is needed.
+// int8 codes become fp16 by placing (code ^ 0x80) under the exponent byte 0x64 (v_perm): 1152 + code exactly;
+// the offsets are removed algebraically (1152 * sum(q) per head, 1152 * sum(p) per head).  fp8 uses
+// v_cvt_scalef32_pk_f16_fp8 with scale 1 (exact).  bf16 / fp16 caches feed the MFMA directly.
+//
+// Semantics: the reference's split kernel (areno/accel/csrc/attention.cu:555-654) -- keys [first_allowed, L_b],
+// q head h <-> kv head h / G, fp32 accumulation.
+#pragma once
+
+#include <type_traits>
+
+#include "paged_decode_kernels.hpp"
+
+namespace areno {
+
+constexpr int kMfmaMaxBatch = 1024;  // prefix-sum capacity of one workgroup
+constexpr int kTileTokens = 32;
+
+typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) short short4_t;
+typedef __attribute__((ext_vector_type(2))) int int2_t;
+
+struct MfmaDecodeParams {
+  DecodeParams d;      // part_ml / part_acc are indexed [slot][q_head] here
+  int32_t* plan;        // [batch + 1] exclusive prefix sums of tiles per sequence, written by workgroup 0
+  int32_t tok_splits;   // waves of a workgroup that share a KV head (4 / heads_per_wg)
+  int32_t num_pieces;   // gridDim.x * tok_splits
+};
+
+template <int KIND>
+struct MfmaOps;
+
+template <>
+struct MfmaOps<KV_BF16> {
+  using vec8 = bf16x8_t;
+  static __device__ __forceinline__ float4_t mfma(vec8 a, vec8 b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct MfmaOps<KV_F16> {
+  using vec8 = half8_t;
+  static __device__ __forceinline__ float4_t mfma(vec8 a, vec8 b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct MfmaOps<KV_I8> : MfmaOps<KV_F16> {};
+template <>
+struct MfmaOps<KV_FP8> : MfmaOps<KV_F16> {};
+
+typedef __attribute__((address_space(3))) int2_t lds_int2;
+typedef __attribute__((address_space(3))) short4_t lds_short4;
+
+// 8 elements (two dwords of 8-bit codes, or four dwords of 16-bit values) -> one MFMA operand register group
+template <int KIND>
+__device__ __forceinline__ typename MfmaOps<KIND>::vec8 to_operand(const uint32_t* w) {
+  using V = typename MfmaOps<KIND>::vec8;
+  uint4_t r;
+  if constexpr (KIND == KV_BF16 || KIND == KV_F16) {
+    r = uint4_t{w[0], w[1], w[2], w[3]};
+  } else if constexpr (KIND == KV_I8) {  // bytes already flipped to offset binary when staged
+    r[0] = __builtin_amdgcn_perm(kF16Filler, w[0], 0x04010400u);
+    r[1] = __builtin_amdgcn_perm(kF16Filler, w[0], 0x04030402u);
+    r[2] = __builtin_amdgcn_perm(kF16Filler, w[1], 0x04010400u);
+    r[3] = __builtin_amdgcn_perm(kF16Filler, w[1], 0x04030402u);
+  } else {
+    r[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[0], 1.0f, false));
+    r[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[0], 1.0f, true));
+    r[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[1], 1.0f, false));
+    r[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[1], 1.0f, true));
+  }
+  return __builtin_bit_cast(V, r);
+}
+
+template <int KIND>
+__device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
+  using P = typename KVTraits<KIND>::pair_t;
+  return __builtin_bit_cast(uint32_t, make_pair<P>(lo, hi));
+}
+
+// LDS row that holds tile token t of the V tile: the second half is rotated by 4 rows so that the 8 tokens a
+// lane group reads through the transpose load ({4g..4g+3} and {16+4g..16+4g+3}) sit in rows distinct mod 16.
+__device__ __forceinline__ int v_row_of(int t) { return t < 16 ? t : 16 + ((t + 4) & 15); }
+
+// Position of a tile stream inside a wave piece: which sequence, which token of it comes next.
+struct TileCursor {
+  int b;         // sequence
+  int tok;       // first token (position inside the sequence) of the tile
+  int end;       // visible length of the sequence (cache_seqlens[b] + 1)
+  int next_end;  // same for sequence b + 1, fetched one sequence ahead
+};
+
+template <int KIND, int D, bool SCALE16>
+__global__ __launch_bounds__(kDecodeThreads, 2) void decode_mfma_kernel(MfmaDecodeParams mp) {
+  using T = KVTraits<KIND>;
+  using Ops = MfmaOps<KIND>;
+  using V8 = typename Ops::vec8;
+  using Pair = typename T::pair_t;
+  const DecodeParams& p = mp.d;
+  constexpr int ES = T::kBytes;
+  constexpr int EPL = 16 / ES;
+  constexpr int LPT = D / EPL;
+  constexpr int TPL = kWave / LPT;
+  constexpr int TK = kTileTokens;
+  constexpr int NLD = TK / TPL;  // 16-byte loads per lane, per tensor, per tile
+  constexpr int RSK = D * ES + 16;
+  constexpr int RSV = ES == 1 ? D + 16 : 2 * D + 32;
+  constexpr int NS = D / 32;       // QK^T k-slices
+  constexpr int NB = D / 16;       // P.V dim blocks
+  constexpr int WPL = 8 * ES / 4;  // dwords per lane per k-slice of 8 elements
+  constexpr float kPScale = T::kQuant ? 256.0f : 1.0f;
+  constexpr int kWaveLds = TK * RSK + TK * RSV + 2 * TK * 4;
+  static_assert(NLD >= 1 && LPT >= 4 && LPT <= 16, "unsupported head_dim");
+
+  __shared__ __attribute__((aligned(16))) char s_tiles[4][kWaveLds];
+  __shared__ int s_cum[kMfmaMaxBatch + 1];
+  __shared__ int s_wave_tot[4];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int lr = lane & 15;  // MFMA row / column index
+  const int lk = lane >> 4;  // MFMA k group
+  const int grp = lane / LPT;
+  const int dc = lane % LPT;
+
+  // ---- tiles per sequence, exclusive prefix sum over the batch ---------------------------------
+  {
+    int nt[4];
+    int local = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int b = 4 * tid + j;
+      nt[j] = 0;
+      if (b < p.batch) {
+        const int length = p.cache_seqlens[b] + 1;
+        nt[j] = (length - first_allowed_key(length, p.window_left) + TK - 1) / TK;
+      }
+      local += nt[j];
+    }
+    int incl = local;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const int v = __shfl_up(incl, off, kWave);
+      if (lane >= off) incl += v;
+    }
+    if (lane == kWave - 1) s_wave_tot[wave] = incl;
+    __syncthreads();
+    int excl = incl - local;
+    for (int w2 = 0; w2 < wave; ++w2) excl += s_wave_tot[w2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int b = 4 * tid + j;
+      if (b <= p.batch) s_cum[b] = excl;
+      excl += nt[j];
+    }
+    __syncthreads();
+  }
+  const int total_tiles = s_cum[p.batch];
+  if (blockIdx.x == 0 && blockIdx.y == 0) {
+    for (int b = tid; b <= p.batch; b += kDecodeThreads) mp.plan[b] = s_cum[b];
+  }
+
+  const int hw_count = p.heads_per_wg;
+  const int hw = wave % hw_count;
+  const int ts = wave / hw_count;
+  const int kvh = blockIdx.y * hw_count + hw;
+  const int piece = blockIdx.x * mp.tok_splits + ts;
+  const int x0 = static_cast<int>(static_cast<int64_t>(piece) * total_tiles / mp.num_pieces);
+  const int x1 = static_cast<int>(static_cast<int64_t>(piece + 1) * total_tiles / mp.num_pieces);
+  if (x0 >= x1) return;
+
+  // sequence that owns tile x0: largest b with cum[b] <= x0
+  int b_first;
+  {
+    int lo = 0, hi = p.batch;
+    while (lo + 1 < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (s_cum[mid] <= x0) {
+        lo = mid;
+      } else {
+        hi = mid;
+      }
+    }
+    b_first = lo;
+  }
+
+  char* const k_tile = &s_tiles[wave][0];
+  char* const v_tile = k_tile + TK * RSK;
+  float* const ksc = reinterpret_cast<float*>(&s_tiles[wave][TK * RSK + TK * RSV]);
+  float* const vsc = ksc + TK;
+
+  constexpr int64_t row_bytes = static_cast<int64_t>(D) * ES;
+  const int h0 = kvh * p.group;
+  const bool q_is_operand_type = (KIND == KV_BF16 && p.q_dtype == ARENO_DT_BF16) ||
+                                 (KIND != KV_BF16 && p.q_dtype == ARENO_DT_F16);
+
+  auto seq_len = [&](int b) { return b < p.batch ? p.cache_seqlens[b] + 1 : 0; };
+  // move a cursor from tile x to tile x + 1; returns true when that tile starts a new sequence
+  auto advance = [&](TileCursor& c, int x_next) {
+    if (x_next == s_cum[c.b + 1]) {
+      ++c.b;
+      c.end = c.next_end;
+      c.next_end = seq_len(c.b + 1);
+      c.tok = first_allowed_key(c.end, p.window_left);
+      return true;
+    }
+    c.tok += TK;
+    return false;
+  };
+
+  // ---- three cursors: block ids are fetched two tiles ahead, KV one tile ahead of the tile being computed ---
+  TileCursor kv_cur;
+  kv_cur.b = b_first;
+  kv_cur.end = seq_len(b_first);
+  kv_cur.next_end = seq_len(b_first + 1);
+  kv_cur.tok = first_allowed_key(kv_cur.end, p.window_left) + (x0 - s_cum[b_first]) * TK;
+  TileCursor id_cur = kv_cur;
+
+  int ids[NLD];
+  auto issue_id_loads = [&]() {
+    const int32_t* table_row = p.block_table + static_cast<int64_t>(id_cur.b) * p.max_blocks;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int t = min(id_cur.tok + i * TPL + grp, id_cur.end - 1);
+      const int col = p.bs_shift >= 0 ? (t >> p.bs_shift) : (t / p.block_size);
+      ids[i] = table_row[col];
+    }
+  };
+
+  uint4_t kreg[NLD], vreg[NLD];
+  typedef typename std::conditional<SCALE16, uint16_t, float>::type scale_raw_t;
+  scale_raw_t ksreg[NLD], vsreg[NLD];
+  auto issue_kv_loads = [&]() {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int t = min(kv_cur.tok + i * TPL + grp, kv_cur.end - 1);
+      const int slot = p.bs_shift >= 0 ? (t & (p.block_size - 1)) : (t % p.block_size);
+      const int64_t row = (static_cast<int64_t>(ids[i]) * p.block_size + slot) * p.kv_heads + kvh;
+      kreg[i] = load16(p.k_cache, row * row_bytes + dc * 16);
+      vreg[i] = load16(p.v_cache, row * row_bytes + dc * 16);
+      if constexpr (T::kQuant) {
+        ksreg[i] = static_cast<const scale_raw_t*>(p.k_scale)[row];
+        vsreg[i] = static_cast<const scale_raw_t*>(p.v_scale)[row];
+      }
+    }
+  };
+  auto scale_value = [](scale_raw_t raw) -> float {
+    if constexpr (SCALE16) {
+      return static_cast<float>(__builtin_bit_cast(_Float16, raw));
+    } else {
+      return raw;
+    }
+  };
+
+  // Q of a sequence: lane (lr = head, lk) needs dims (D/4)*lk + 8*s + [0, 8) of head h0 + lr, 16 raw bytes per
+  // slice for 16-bit queries; fetched when the KV cursor enters the sequence, converted when compute gets there.
+  uint4_t qraw[NS];
+  auto issue_q_loads = [&](int b) {
+#pragma unroll
+    for (int sl = 0; sl < NS; ++sl) {
+      qraw[sl] = uint4_t{0u, 0u, 0u, 0u};
+      if (lr < p.group) {
+        const int64_t idx = (static_cast<int64_t>(b) * p.q_heads + h0 + lr) * D + (D / 4) * lk + 8 * sl;
+        qraw[sl] = load16(p.q, idx * 2);
+      }
+    }
+  };
+  V8 qop[NS];
+  float qbias = 0.0f;
+  auto adopt_q = [&]() {
+    float qsum = 0.0f;
+#pragma unroll
+    for (int sl = 0; sl < NS; ++sl) {
+      uint4_t w = qraw[sl];
+      if (!q_is_operand_type) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          // the other 16-bit float format: go through fp32 (bf16 query with an fp16 operand, or the reverse)
+          float a, c;
+          if constexpr (KIND == KV_BF16) {
+            a = f16_bits_to_float(w[j] & 0xffffu);
+            c = f16_bits_to_float(w[j] >> 16);
+          } else {
+            a = bf16_bits_to_float(w[j] & 0xffffu);
+            c = bf16_bits_to_float(w[j] >> 16);
+          }
+          w[j] = __builtin_bit_cast(uint32_t, make_pair<Pair>(a, c));
+        }
+      }
+      if constexpr (KIND == KV_I8) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const Pair pr = __builtin_bit_cast(Pair, static_cast<uint32_t>(w[j]));
+          qsum += static_cast<float>(pr.x) + static_cast<float>(pr.y);
+        }
+      }
+      qop[sl] = __builtin_bit_cast(V8, w);
+    }
+    if constexpr (KIND == KV_I8) {
+      qsum += wave_xor(qsum, 16);
+      qsum += wave_xor(qsum, 32);
+      qbias = kI8Offset * qsum;
+    }
+  };
+
+  float4_t acc[NB];
+  float m_run = kNegInf, l_run = 0.0f, p_sum = 0.0f;
+  auto reset_state = [&]() {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    m_run = kNegInf;
+    l_run = 0.0f;
+    p_sum = 0.0f;
+  };
+
+  auto write_partial = [&](int b) {
+    // combine the four k-groups' row sums; every lane of a head ends with the head's totals
+    float l_tot = l_run;
+    l_tot += wave_xor(l_tot, 16);
+    l_tot += wave_xor(l_tot, 32);
+    float off = 0.0f;
+    if constexpr (KIND == KV_I8) {
+      float ps = p_sum;
+      ps += wave_xor(ps, 16);
+      ps += wave_xor(ps, 32);
+      off = kI8Offset * ps;
+    }
+    if (lr < p.group) {
+      const int64_t prow = (static_cast<int64_t>(piece + b)) * p.q_heads + h0 + lr;
+      float* dst = p.part_acc + prow * D + 4 * lk;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        float4_t o = acc[nb];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = (o[j] - off) * (1.0f / kPScale);
+        *reinterpret_cast<float4_t*>(dst + 16 * nb) = o;
+      }
+      if (lk == 0) {
+        p.part_ml[prow * 2] = m_run;
+        p.part_ml[prow * 2 + 1] = l_tot;
+      }
+    }
+  };
+
+  // ---- prologue -------------------------------------------------------------------------------------------
+  issue_id_loads();
+  issue_q_loads(kv_cur.b);
+  issue_kv_loads();  // tile x0 (waits for its ids)
+  if (x0 + 1 < x1) {
+    advance(id_cur, x0 + 1);
+    issue_id_loads();  // ids of tile x0 + 1
+  }
+  int cp_b = kv_cur.b, cp_tok = kv_cur.tok, cp_end = kv_cur.end;
+  adopt_q();
+  reset_state();
+
+  for (int x = x0; x < x1; ++x) {
+    // -- stage the fetched tile into LDS (waits for its loads) ---------------------------------------------
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int t = i * TPL + grp;  // tile-local token
+      uint4_t kk = kreg[i], vv = vreg[i];
+      if constexpr (KIND == KV_I8) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          kk[j] ^= kI8Flip;
+          vv[j] ^= kI8Flip;
+        }
+      }
+      *reinterpret_cast<uint4_t*>(k_tile + t * RSK + dc * 16) = kk;
+      *reinterpret_cast<uint4_t*>(v_tile + v_row_of(t) * RSV + dc * 16) = vv;
+      if (dc == 0) {
+        const bool ok = cp_tok + t < cp_end;
+        if constexpr (T::kQuant) {
+          ksc[t] = ok ? scale_value(ksreg[i]) * p.scale_log2e : kNegInf;
+          vsc[t] = ok ? scale_value(vsreg[i]) * kPScale : 0.0f;
+        } else {
+          ksc[t] = ok ? p.scale_log2e : kNegInf;
+          vsc[t] = ok ? kPScale : 0.0f;
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // -- fetch tile x + 1 (its block ids arrived during the previous iteration) and the ids of tile x + 2 ------
+    bool next_is_new_seq = false;
+    if (x + 1 < x1) {
+      next_is_new_seq = advance(kv_cur, x + 1);
+      if (next_is_new_seq) issue_q_loads(kv_cur.b);
+      issue_kv_loads();
+      if (x + 2 < x1) {
+        advance(id_cur, x + 2);
+        issue_id_loads();
+      }
+    }
+
+    // -- S^T = K . Q^T for the two 16-token groups ------------------------------------------------------------
+    float s[2][4];
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+      float4_t c = {0.0f, 0.0f, 0.0f, 0.0f};
+      const char* krow = k_tile + (16 * tg + lr) * RSK + (D / 4) * ES * lk;
+      uint32_t kw[NS * WPL];
+#pragma unroll
+      for (int q4 = 0; q4 < NS * WPL / 4; ++q4) {
+        const uint4_t r = *reinterpret_cast<const uint4_t*>(krow + 16 * q4);
+        kw[4 * q4 + 0] = r[0];
+        kw[4 * q4 + 1] = r[1];
+        kw[4 * q4 + 2] = r[2];
+        kw[4 * q4 + 3] = r[3];
+      }
+#pragma unroll
+      for (int sl = 0; sl < NS; ++sl) c = Ops::mfma(to_operand<KIND>(&kw[sl * WPL]), qop[sl], c);
+      const float4_t sc = *reinterpret_cast<const float4_t*>(ksc + 16 * tg + 4 * lk);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        // tokens past the end carry a -inf scale; keep them exactly -inf (0 * -inf would be NaN)
+        const float v = c[j] - qbias;
+        s[tg][j] = sc[j] == kNegInf ? kNegInf : v * sc[j];
+      }
+    }
+
+    // -- online softmax for head lr over the tile's 32 tokens ---------------------------------------------------
+    float mt = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                     fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+    mt = fmaxf(mt, wave_xor(mt, 16));
+    mt = fmaxf(mt, wave_xor(mt, 32));
+    const float m_new = fmaxf(m_run, mt);
+    const float m_safe = m_new == kNegInf ? 0.0f : m_new;
+    const float alpha = fast_exp2(m_run - m_safe);
+    m_run = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+      l_run *= alpha;
+      p_sum *= alpha;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[nb][j] *= alpha;
+      }
+    }
+    uint32_t pw[4];
+    {
+      const float4_t vs0 = *reinterpret_cast<const float4_t*>(vsc + 4 * lk);
+      const float4_t vs1 = *reinterpret_cast<const float4_t*>(vsc + 16 + 4 * lk);
+      float pe[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float e0 = fast_exp2(s[0][j] - m_safe);
+        const float e1 = fast_exp2(s[1][j] - m_safe);
+        l_run += e0 + e1;
+        pe[j] = e0 * vs0[j];
+        pe[4 + j] = e1 * vs1[j];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        pw[j] = pack_pair<KIND>(pe[2 * j], pe[2 * j + 1]);
+        if constexpr (KIND == KV_I8) {
+          const Pair pr = __builtin_bit_cast(Pair, pw[j]);
+          p_sum += static_cast<float>(pr.x) + static_cast<float>(pr.y);
+        }
+      }
+    }
+    const V8 pop = __builtin_bit_cast(V8, uint4_t{pw[0], pw[1], pw[2], pw[3]});
+
+    // -- O^T += V^T . P^T, one MFMA per 16-dim block -------------------------------------------------------------
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      uint32_t vw[4];
+      if constexpr (ES == 1) {
+        // lane i of a 16-lane group supplies row (i / 2), 8 bytes at column 16 nb + 8 (i % 2)
+        const int r8 = lr >> 1;
+        const int tok = r8 < 4 ? 4 * lk + r8 : 16 + 4 * lk + (r8 - 4);
+        char* a = v_tile + v_row_of(tok) * RSV + 16 * nb + 8 * (lr & 1);
+        const int2_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_int2*)a);
+        vw[0] = static_cast<uint32_t>(r[0]);
+        vw[1] = static_cast<uint32_t>(r[1]);
+      } else {
+        // lane i supplies row (i / 4), 4 elements at column 16 nb + 4 (i % 4); two reads of 4 tokens each
+        const int r4 = lr >> 2;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int tok = 16 * half + 4 * lk + r4;
+          char* a = v_tile + v_row_of(tok) * RSV + (16 * nb + 4 * (lr & 3)) * 2;
+          const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
+          const uint2_t u = __builtin_bit_cast(uint2_t, r);
+          vw[2 * half] = u[0];
+          vw[2 * half + 1] = u[1];
+        }
+      }
+      acc[nb] = Ops::mfma(to_operand<KIND>(vw), pop, acc[nb]);
+    }
+    // all LDS reads of this tile are done before the next iteration overwrites it
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // -- end of a sequence's share: emit its partial and switch to the next sequence ---------------------------
+    const bool last_of_piece = x + 1 == x1;
+    if (next_is_new_seq || last_of_piece) {
+      write_partial(cp_b);
+      if (!last_of_piece) {
+        cp_b = kv_cur.b;
+        adopt_q();
+        reset_state();
+      }
+    }
+    cp_tok = kv_cur.tok;
+    cp_end = kv_cur.end;
+  }
+}
+
+typedef void (*decode_mfma_fn)(MfmaDecodeParams);
+decode_mfma_fn decode_mfma_lookup_bf16(int head_dim, bool scale16);
+decode_mfma_fn decode_mfma_lookup_f16(int head_dim, bool scale16);
+decode_mfma_fn decode_mfma_lookup_i8(int head_dim, bool scale16);
+decode_mfma_fn decode_mfma_lookup_fp8(int head_dim, bool scale16);
+
+template <int KIND>
+decode_mfma_fn decode_mfma_lookup_impl(int head_dim, bool scale16) {
+  if constexpr (KVTraits<KIND>::kQuant) {
+    if (head_dim == 128) return scale16 ? decode_mfma_kernel<KIND, 128, true> : decode_mfma_kernel<KIND, 128, false>;
+    if (head_dim == 64) return scale16 ? decode_mfma_kernel<KIND, 64, true> : decode_mfma_kernel<KIND, 64, false>;
+  } else {
+    if (head_dim == 128) return decode_mfma_kernel<KIND, 128, false>;
+    if (head_dim == 64) return decode_mfma_kernel<KIND, 64, false>;
+  }
+  return nullptr;
+}
+
+}  // namespace areno

@@ -4,7 +4,10 @@
 //                                   reference), normalise, cast to the query dtype
 // The fast split kernels live in paged_decode_kernels.hpp.
 
-#include "paged_decode_kernels.hpp"
+#include <stdlib.h>
+#include <string.h>
+
+#include "decode_mfma_kernels.hpp"
 
 namespace areno {
 
@@ -125,6 +128,73 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_kernel(Decod
   }
 }
 
+// Merge of the MFMA path's partials: the pieces that own tiles of sequence b wrote slots (piece + b);
+// pieces that own no tile at all are skipped.  One wave per (sequence, q head).
+__global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel(MfmaDecodeParams mp) {
+  const DecodeParams& p = mp.d;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int row = blockIdx.x * kReduceRows + (threadIdx.x >> 6);
+  if (row >= p.batch * p.q_heads) return;
+  const int b = row / p.q_heads;
+  const int h = row - b * p.q_heads;
+  const int d = p.head_dim;
+  const int64_t nt = mp.plan[p.batch];
+  const int64_t np = mp.num_pieces;
+  const int64_t first_tile = mp.plan[b];
+  const int64_t last_tile = static_cast<int64_t>(mp.plan[b + 1]) - 1;
+  // owner(x): the largest piece whose first tile (piece * nt / np) is <= x
+  const int wp_lo = static_cast<int>(((first_tile + 1) * np + nt - 1) / nt - 1);
+  const int wp_hi = static_cast<int>(((last_tile + 1) * np + nt - 1) / nt - 1);
+
+  float acc[kGenericMaxPerLane];
+#pragma unroll
+  for (int e = 0; e < kGenericMaxPerLane; ++e) acc[e] = 0.0f;
+  float m = kNegInf, l = 0.0f;
+  for (int wp = wp_lo; wp <= wp_hi; ++wp) {
+    if (wp * nt / np == (wp + 1) * nt / np) continue;  // piece without tiles
+    const int64_t prow = static_cast<int64_t>(wp + b) * p.q_heads + h;
+    const float part_m = p.part_ml[prow * 2];
+    const float part_l = p.part_ml[prow * 2 + 1];
+    if (part_l == 0.0f) continue;
+    const float m_new = fmaxf(m, part_m);
+    const float alpha = fast_exp2(m - m_new);
+    const float beta = fast_exp2(part_m - m_new);
+    const float* part = p.part_acc + prow * d;
+#pragma unroll
+    for (int e = 0; e < kGenericMaxPerLane; ++e) {
+      const int idx = lane + e * kWave;
+      if (idx < d) acc[e] = acc[e] * alpha + part[idx] * beta;
+    }
+    l = l * alpha + part_l * beta;
+    m = m_new;
+  }
+#pragma unroll
+  for (int e = 0; e < kGenericMaxPerLane; ++e) {
+    const int idx = lane + e * kWave;
+    if (idx < d) store_from_float(p.out, static_cast<int64_t>(row) * d + idx, p.q_dtype, acc[e] / l);
+  }
+}
+
+// ---- geometry of the MFMA path ----------------------------------------------------------------------
+constexpr int kMfmaWorkgroups = 512;  // two resident workgroups on each of the 256 CUs
+constexpr int kMfmaMaxPieces = kMfmaWorkgroups * 4;
+
+size_t mfma_workspace_bytes(int batch, int q_heads, int head_dim) {
+  const size_t slots = static_cast<size_t>(kMfmaMaxPieces) + batch;
+  size_t bytes = slots * q_heads * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
+  bytes = (bytes + 255) / 256 * 256;
+  return bytes + (static_cast<size_t>(batch) + 1 + 63) / 64 * 64 * sizeof(int32_t);
+}
+
+// "valu" forces the vector-ALU split kernel, "mfma" (default) prefers the matrix-core kernel where it applies.
+bool prefer_mfma() {
+  static const int choice = [] {
+    const char* v = getenv("ARENO_DECODE_KERNEL");
+    return (v != nullptr && strcmp(v, "valu") == 0) ? 0 : 1;
+  }();
+  return choice == 1;
+}
+
 struct Chunking {
   int chunk;
   int max_parts;
@@ -163,8 +233,10 @@ extern "C" size_t areno_hip_paged_decode_workspace_bytes(int32_t batch, int32_t 
   if (batch <= 0 || q_heads <= 0 || head_dim <= 0 || num_splits < 1) return 0;
   if (!areno::pick_chunking(block_size, max_blocks, num_splits, &ch)) return 0;
   const size_t rows = static_cast<size_t>(batch) * q_heads * ch.max_parts;
-  const size_t bytes = rows * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
-  return (bytes + 255) / 256 * 256;
+  size_t bytes = rows * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
+  bytes = (bytes + 255) / 256 * 256;
+  const size_t mfma = areno::mfma_workspace_bytes(batch, q_heads, head_dim);
+  return bytes > mfma ? bytes : mfma;
 }
 
 extern "C" int areno_hip_paged_decode(const areno_paged_cache* cache, const void* q, const void* k_update,
@@ -260,6 +332,43 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
     }
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
+
+  // ---- matrix-core path: 16-bit or 8-bit caches, head_dim 64/128, up to 16 q heads per kv head ------------
+  decode_mfma_fn mfma = nullptr;
+  if (aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && num_splits != 1 && p.group <= 16 &&
+      batch <= kMfmaMaxBatch) {
+    switch (cache->cache_dtype) {
+      case ARENO_DT_BF16: mfma = decode_mfma_lookup_bf16(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
+      case ARENO_DT_F16: mfma = decode_mfma_lookup_f16(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
+      case ARENO_DT_I8: mfma = decode_mfma_lookup_i8(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
+      case ARENO_DT_FP8_E4M3: mfma = decode_mfma_lookup_fp8(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
+      default: break;
+    }
+  }
+  if (mfma != nullptr) {
+    MfmaDecodeParams mp;
+    mp.d = p;
+    const int head_groups = cache->kv_heads / p.heads_per_wg;
+    const int grid_x = kMfmaWorkgroups / head_groups > 0 ? kMfmaWorkgroups / head_groups : 1;
+    mp.tok_splits = 4 / p.heads_per_wg;
+    mp.num_pieces = grid_x * mp.tok_splits;
+    const size_t slots = static_cast<size_t>(mp.num_pieces) + batch;
+    const size_t part_bytes = (slots * q_heads * (static_cast<size_t>(p.head_dim) + 2) * sizeof(float) + 255) / 256 * 256;
+    mp.d.part_ml = static_cast<float*>(workspace);
+    mp.d.part_acc = mp.d.part_ml + slots * q_heads * 2;
+    mp.plan = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + part_bytes);
+    if (stages & ARENO_STAGE_SPLIT) {
+      hipLaunchKernelGGL(mfma, dim3(grid_x, head_groups), dim3(kDecodeThreads), 0, s, mp);
+      if (int rc = check_launch(op)) return rc;
+    }
+    if (stages & ARENO_STAGE_REDUCE) {
+      const int rblocks = (batch * q_heads + kReduceRows - 1) / kReduceRows;
+      hipLaunchKernelGGL(decode_reduce_slots_kernel, dim3(rblocks), dim3(kReduceRows * kWave), 0, s, mp);
+      if (int rc = check_launch(op)) return rc;
+    }
+    return ARENO_OK;
+  }
+
   if (!(stages & ARENO_STAGE_SPLIT)) {
     // skip
   } else if (fast != nullptr) {

@@ -46,12 +46,18 @@ def test_version_status_strings_and_workspace_size(lib):
     ws = lib.areno_hip_paged_decode_workspace_bytes
     ws.restype = ctypes.c_size_t
     ws.argtypes = [ctypes.c_int32] * 6
-    # B=64, Hq=28, D=128, bs=16, MB=257: 4112 tokens -> 17 chunks of 256 -> 64*28*17*(128+2)*4 bytes
-    assert ws(64, 28, 128, 16, 257, 8) == 64 * 28 * 17 * 130 * 4
-    assert ws(64, 28, 128, 16, 257, 1) == (64 * 28 * 1 * 130 * 4 + 255) // 256 * 256
+    # two layouts share the workspace: fixed chunks (B * Hq * chunks rows) and the balanced-piece layout
+    # ((2048 pieces + B) * Hq rows plus the B + 1 prefix sums); the size is the larger of the two
+    def pieces(b, hq, d):
+        rows = (2048 + b) * hq * (d + 2) * 4
+        return (rows + 255) // 256 * 256 + (b + 1 + 63) // 64 * 64 * 4
+
+    # B=64, Hq=28, D=128, bs=16, MB=257: 4112 tokens -> 17 chunks of 256
+    assert ws(64, 28, 128, 16, 257, 8) == max(64 * 28 * 17 * 130 * 4, pieces(64, 28, 128))
+    assert ws(4096, 28, 128, 16, 257, 8) == max(4096 * 28 * 17 * 130 * 4, pieces(4096, 28, 128))
     assert ws(0, 28, 128, 16, 257, 8) == 0 and ws(64, 28, 128, 16, 257, 0) == 0
-    # long tables fold into at most 64 partials per row
-    assert ws(1, 1, 128, 16, 4096, 8) == 1 * 1 * 64 * 130 * 4
+    # long tables fold into at most 64 chunks per row
+    assert ws(4096, 1, 128, 16, 4096, 8) == max(4096 * 64 * 130 * 4, pieces(4096, 1, 128))
 
 
 def test_argument_validation_runs_before_any_launch(lib):
