@@ -42,6 +42,9 @@
 namespace areno {
 
 constexpr int kMfmaMaxBatch = 1024;  // prefix-sum capacity of one workgroup
+#ifndef ARENO_MFMA_NW
+#define ARENO_MFMA_NW 4
+#endif
 constexpr int kTileTokens = 32;
 
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
@@ -51,9 +54,15 @@ typedef __attribute__((ext_vector_type(2))) int int2_t;
 
 struct MfmaDecodeParams {
   DecodeParams d;      // part_ml / part_acc are indexed [slot][q_head] here
-  int32_t* plan;        // [batch + 1] exclusive prefix sums of tiles per sequence, written by workgroup 0
-  int32_t tok_splits;   // waves of a workgroup that share a KV head (4 / heads_per_wg)
-  int32_t num_pieces;   // gridDim.x * tok_splits
+  int32_t* plan;         // [batch + 4]: exclusive prefix sums of tiles per sequence, then the unit geometry
+  int32_t* unit_counter;  // [head groups] dynamic-unit tickets, zero when the kernel starts
+  int32_t tok_splits;    // waves of a workgroup that share a KV head (waves per workgroup / heads_per_wg)
+  int32_t num_pieces;    // gridDim.x * tok_splits: statically assigned units
+  int32_t static_share;  // n/256 of all tiles are assigned statically, the rest is claimed in small units
+  int32_t min_unit_tiles;
+#ifdef ARENO_TRACE
+  unsigned long long* trace;  // [wave][16] timestamps, tuning builds only
+#endif
 };
 
 template <int KIND>
@@ -112,7 +121,45 @@ __device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
 // lane group reads through the transpose load ({4g..4g+3} and {16+4g..16+4g+3}) sit in rows distinct mod 16.
 __device__ __forceinline__ int v_row_of(int t) { return t < 16 ? t : 16 + ((t + 4) & 15); }
 
-// Position of a tile stream inside a wave piece: which sequence, which token of it comes next.
+// How the global tile range is cut into units (shared by the split and the reduce kernel).
+struct UnitGeometry {
+  int total_tiles;
+  int static_tiles;  // tiles covered by the static units
+  int static_units;  // one per wave piece
+  int unit_tiles;    // tiles per small unit
+  int small_units;
+
+  __host__ __device__ int unit_start(int u) const {
+    if (u <= static_units) return static_cast<int>(static_cast<long long>(u) * static_tiles / static_units);
+    const long long x = static_tiles + static_cast<long long>(u - static_units) * unit_tiles;
+    return x < total_tiles ? static_cast<int>(x) : total_tiles;
+  }
+  // unit that owns tile x (the largest unit whose first tile is <= x)
+  __host__ __device__ int unit_of(int x) const {
+    if (x < static_tiles)
+      return static_cast<int>((static_cast<long long>(x + 1) * static_units + static_tiles - 1) / static_tiles - 1);
+    return static_units + (x - static_tiles) / unit_tiles;
+  }
+};
+
+constexpr int kMaxSmallUnits = 1024;
+
+__host__ __device__ inline UnitGeometry make_unit_geometry(int total_tiles, int num_pieces, int static_share,
+                                                           int min_unit_tiles) {
+  UnitGeometry g;
+  g.total_tiles = total_tiles;
+  g.static_units = num_pieces;
+  g.static_tiles = static_cast<int>(static_cast<long long>(total_tiles) * static_share / 256);
+  // short batches are not worth a claimed tail: everything static
+  if (total_tiles < 4 * num_pieces || static_share >= 256) g.static_tiles = total_tiles;
+  const int rest = total_tiles - g.static_tiles;
+  g.unit_tiles = min_unit_tiles < 1 ? 1 : min_unit_tiles;
+  if (static_cast<long long>(g.unit_tiles) * kMaxSmallUnits < rest) g.unit_tiles = (rest + kMaxSmallUnits - 1) / kMaxSmallUnits;
+  g.small_units = (rest + g.unit_tiles - 1) / g.unit_tiles;
+  return g;
+}
+
+// Position of a tile stream inside a unit: which sequence, which token of it comes next.
 struct TileCursor {
   int b;         // sequence
   int tok;       // first token (position inside the sequence) of the tile
@@ -120,8 +167,8 @@ struct TileCursor {
   int next_end;  // same for sequence b + 1, fetched one sequence ahead
 };
 
-template <int KIND, int D, bool SCALE16>
-__global__ __launch_bounds__(kDecodeThreads, 2) void decode_mfma_kernel(MfmaDecodeParams mp) {
+template <int KIND, int D, bool SCALE16, int NW>
+__global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodeParams mp) {
   using T = KVTraits<KIND>;
   using Ops = MfmaOps<KIND>;
   using V8 = typename Ops::vec8;
@@ -142,13 +189,23 @@ __global__ __launch_bounds__(kDecodeThreads, 2) void decode_mfma_kernel(MfmaDeco
   constexpr int kWaveLds = TK * RSK + TK * RSV + 2 * TK * 4;
   static_assert(NLD >= 1 && LPT >= 4 && LPT <= 16, "unsupported head_dim");
 
-  __shared__ __attribute__((aligned(16))) char s_tiles[4][kWaveLds];
+  __shared__ __attribute__((aligned(16))) char s_tiles[NW][kWaveLds];
   __shared__ int s_cum[kMfmaMaxBatch + 1];
-  __shared__ int s_wave_tot[4];
+  __shared__ int s_wave_tot[NW];
+  constexpr int SPT = kMfmaMaxBatch / (NW * kWave);  // sequences per thread in the prefix sum
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
+#ifdef ARENO_TRACE
+  const int trace_wave = (blockIdx.y * gridDim.x + blockIdx.x) * NW + wave;
+  int trace_n = 2;
+  if (mp.trace && lane == 0) mp.trace[trace_wave * 16] = wall_clock64();
+#define ARENO_TRACE_POINT()                                                                   \
+  if (mp.trace && lane == 0 && trace_n < 16) mp.trace[trace_wave * 16 + trace_n++] = wall_clock64()
+#else
+#define ARENO_TRACE_POINT()
+#endif
   const int lr = lane & 15;  // MFMA row / column index
   const int lk = lane >> 4;  // MFMA k group
   const int grp = lane / LPT;
@@ -156,11 +213,11 @@ __global__ __launch_bounds__(kDecodeThreads, 2) void decode_mfma_kernel(MfmaDeco
 
   // ---- tiles per sequence, exclusive prefix sum over the batch ---------------------------------
   {
-    int nt[4];
+    int nt[SPT];
     int local = 0;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int b = 4 * tid + j;
+    for (int j = 0; j < SPT; ++j) {
+      const int b = SPT * tid + j;
       nt[j] = 0;
       if (b < p.batch) {
         const int length = p.cache_seqlens[b] + 1;
@@ -179,41 +236,29 @@ __global__ __launch_bounds__(kDecodeThreads, 2) void decode_mfma_kernel(MfmaDeco
     int excl = incl - local;
     for (int w2 = 0; w2 < wave; ++w2) excl += s_wave_tot[w2];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int b = 4 * tid + j;
+    for (int j = 0; j < SPT; ++j) {
+      const int b = SPT * tid + j;
       if (b <= p.batch) s_cum[b] = excl;
       excl += nt[j];
     }
     __syncthreads();
   }
+  // ---- unit geometry -----------------------------------------------------------------------------------
+  // Tiles [0, static_tiles) are cut into num_pieces equal static units (one per wave); the rest is cut into
+  // small units of unit_tiles tiles that waves claim from a ticket counter once their static unit is done:
+  // memory service is uneven across CUs, and without the claimed tail the slowest wave sets the run time.
   const int total_tiles = s_cum[p.batch];
+  const UnitGeometry geo = make_unit_geometry(total_tiles, mp.num_pieces, mp.static_share, mp.min_unit_tiles);
   if (blockIdx.x == 0 && blockIdx.y == 0) {
-    for (int b = tid; b <= p.batch; b += kDecodeThreads) mp.plan[b] = s_cum[b];
+    for (int b = tid; b <= p.batch; b += NW * kWave) mp.plan[b] = s_cum[b];
   }
 
   const int hw_count = p.heads_per_wg;
   const int hw = wave % hw_count;
   const int ts = wave / hw_count;
   const int kvh = blockIdx.y * hw_count + hw;
-  const int piece = blockIdx.x * mp.tok_splits + ts;
-  const int x0 = static_cast<int>(static_cast<int64_t>(piece) * total_tiles / mp.num_pieces);
-  const int x1 = static_cast<int>(static_cast<int64_t>(piece + 1) * total_tiles / mp.num_pieces);
-  if (x0 >= x1) return;
-
-  // sequence that owns tile x0: largest b with cum[b] <= x0
-  int b_first;
-  {
-    int lo = 0, hi = p.batch;
-    while (lo + 1 < hi) {
-      const int mid = (lo + hi) >> 1;
-      if (s_cum[mid] <= x0) {
-        lo = mid;
-      } else {
-        hi = mid;
-      }
-    }
-    b_first = lo;
-  }
+  // one ticket counter per KV head: every wave that works on this head draws from it
+  int* const ticket = mp.unit_counter + kvh;
 
   char* const k_tile = &s_tiles[wave][0];
   char* const v_tile = k_tile + TK * RSK;
@@ -239,14 +284,8 @@ __global__ __launch_bounds__(kDecodeThreads, 2) void decode_mfma_kernel(MfmaDeco
     return false;
   };
 
-  // ---- three cursors: block ids are fetched two tiles ahead, KV one tile ahead of the tile being computed ---
-  TileCursor kv_cur;
-  kv_cur.b = b_first;
-  kv_cur.end = seq_len(b_first);
-  kv_cur.next_end = seq_len(b_first + 1);
-  kv_cur.tok = first_allowed_key(kv_cur.end, p.window_left) + (x0 - s_cum[b_first]) * TK;
-  TileCursor id_cur = kv_cur;
-
+  TileCursor kv_cur, id_cur;
+  int unit = 0;
   int ids[NLD];
   auto issue_id_loads = [&]() {
     const int32_t* table_row = p.block_table + static_cast<int64_t>(id_cur.b) * p.max_blocks;
@@ -357,7 +396,7 @@ __global__ __launch_bounds__(kDecodeThreads, 2) void decode_mfma_kernel(MfmaDeco
       off = kI8Offset * ps;
     }
     if (lr < p.group) {
-      const int64_t prow = (static_cast<int64_t>(piece + b)) * p.q_heads + h0 + lr;
+      const int64_t prow = (static_cast<int64_t>(unit + b)) * p.q_heads + h0 + lr;
       float* dst = p.part_acc + prow * D + 4 * lk;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
@@ -373,171 +412,211 @@ __global__ __launch_bounds__(kDecodeThreads, 2) void decode_mfma_kernel(MfmaDeco
     }
   };
 
-  // ---- prologue -------------------------------------------------------------------------------------------
-  issue_id_loads();
-  issue_q_loads(kv_cur.b);
-  issue_kv_loads();  // tile x0 (waits for its ids)
-  if (x0 + 1 < x1) {
-    advance(id_cur, x0 + 1);
-    issue_id_loads();  // ids of tile x0 + 1
-  }
-  int cp_b = kv_cur.b, cp_tok = kv_cur.tok, cp_end = kv_cur.end;
-  adopt_q();
-  reset_state();
-
-  for (int x = x0; x < x1; ++x) {
-    // -- stage the fetched tile into LDS (waits for its loads) ---------------------------------------------
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const int t = i * TPL + grp;  // tile-local token
-      uint4_t kk = kreg[i], vv = vreg[i];
-      if constexpr (KIND == KV_I8) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          kk[j] ^= kI8Flip;
-          vv[j] ^= kI8Flip;
+  // ---- units: the wave's static unit first, then claimed ones ---------------------------------------------------
+  unit = blockIdx.x * mp.tok_splits + ts;
+  while (true) {
+    const int x0 = geo.unit_start(unit);
+    const int x1 = geo.unit_start(unit + 1);
+    if (x0 < x1) {
+      // sequence that owns tile x0: largest b with cum[b] <= x0
+      int b_first;
+      {
+        int lo = 0, hi = p.batch;
+        while (lo + 1 < hi) {
+          const int mid = (lo + hi) >> 1;
+          if (s_cum[mid] <= x0) {
+            lo = mid;
+          } else {
+            hi = mid;
+          }
         }
+        b_first = lo;
       }
-      *reinterpret_cast<uint4_t*>(k_tile + t * RSK + dc * 16) = kk;
-      *reinterpret_cast<uint4_t*>(v_tile + v_row_of(t) * RSV + dc * 16) = vv;
-      if (dc == 0) {
-        const bool ok = cp_tok + t < cp_end;
-        if constexpr (T::kQuant) {
-          ksc[t] = ok ? scale_value(ksreg[i]) * p.scale_log2e : kNegInf;
-          vsc[t] = ok ? scale_value(vsreg[i]) * kPScale : 0.0f;
-        } else {
-          ksc[t] = ok ? p.scale_log2e : kNegInf;
-          vsc[t] = ok ? kPScale : 0.0f;
+
+      // ---- three cursors: block ids are fetched two tiles ahead, KV one tile ahead of the tile being computed ---
+      kv_cur.b = b_first;
+      kv_cur.end = seq_len(b_first);
+      kv_cur.next_end = seq_len(b_first + 1);
+      kv_cur.tok = first_allowed_key(kv_cur.end, p.window_left) + (x0 - s_cum[b_first]) * TK;
+      id_cur = kv_cur;
+
+      // ---- prologue -------------------------------------------------------------------------------------------
+      issue_id_loads();
+      issue_q_loads(kv_cur.b);
+      issue_kv_loads();  // tile x0 (waits for its ids)
+      if (x0 + 1 < x1) {
+        advance(id_cur, x0 + 1);
+        issue_id_loads();  // ids of tile x0 + 1
+      }
+      int cp_b = kv_cur.b, cp_tok = kv_cur.tok, cp_end = kv_cur.end;
+      adopt_q();
+      reset_state();
+
+      for (int x = x0; x < x1; ++x) {
+        ARENO_TRACE_POINT();
+        // -- stage the fetched tile into LDS (waits for its loads) ---------------------------------------------
+    #pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+          const int t = i * TPL + grp;  // tile-local token
+          uint4_t kk = kreg[i], vv = vreg[i];
+          if constexpr (KIND == KV_I8) {
+    #pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              kk[j] ^= kI8Flip;
+              vv[j] ^= kI8Flip;
+            }
+          }
+          *reinterpret_cast<uint4_t*>(k_tile + t * RSK + dc * 16) = kk;
+          *reinterpret_cast<uint4_t*>(v_tile + v_row_of(t) * RSV + dc * 16) = vv;
+          if (dc == 0) {
+            const bool ok = cp_tok + t < cp_end;
+            if constexpr (T::kQuant) {
+              ksc[t] = ok ? scale_value(ksreg[i]) * p.scale_log2e : kNegInf;
+              vsc[t] = ok ? scale_value(vsreg[i]) * kPScale : 0.0f;
+            } else {
+              ksc[t] = ok ? p.scale_log2e : kNegInf;
+              vsc[t] = ok ? kPScale : 0.0f;
+            }
+          }
         }
-      }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-    // -- fetch tile x + 1 (its block ids arrived during the previous iteration) and the ids of tile x + 2 ------
-    bool next_is_new_seq = false;
-    if (x + 1 < x1) {
-      next_is_new_seq = advance(kv_cur, x + 1);
-      if (next_is_new_seq) issue_q_loads(kv_cur.b);
-      issue_kv_loads();
-      if (x + 2 < x1) {
-        advance(id_cur, x + 2);
-        issue_id_loads();
-      }
-    }
-
-    // -- S^T = K . Q^T for the two 16-token groups ------------------------------------------------------------
-    float s[2][4];
-#pragma unroll
-    for (int tg = 0; tg < 2; ++tg) {
-      float4_t c = {0.0f, 0.0f, 0.0f, 0.0f};
-      const char* krow = k_tile + (16 * tg + lr) * RSK + (D / 4) * ES * lk;
-      uint32_t kw[NS * WPL];
-#pragma unroll
-      for (int q4 = 0; q4 < NS * WPL / 4; ++q4) {
-        const uint4_t r = *reinterpret_cast<const uint4_t*>(krow + 16 * q4);
-        kw[4 * q4 + 0] = r[0];
-        kw[4 * q4 + 1] = r[1];
-        kw[4 * q4 + 2] = r[2];
-        kw[4 * q4 + 3] = r[3];
-      }
-#pragma unroll
-      for (int sl = 0; sl < NS; ++sl) c = Ops::mfma(to_operand<KIND>(&kw[sl * WPL]), qop[sl], c);
-      const float4_t sc = *reinterpret_cast<const float4_t*>(ksc + 16 * tg + 4 * lk);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // tokens past the end carry a -inf scale; keep them exactly -inf (0 * -inf would be NaN)
-        const float v = c[j] - qbias;
-        s[tg][j] = sc[j] == kNegInf ? kNegInf : v * sc[j];
-      }
-    }
-
-    // -- online softmax for head lr over the tile's 32 tokens ---------------------------------------------------
-    float mt = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
-                     fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
-    mt = fmaxf(mt, wave_xor(mt, 16));
-    mt = fmaxf(mt, wave_xor(mt, 32));
-    const float m_new = fmaxf(m_run, mt);
-    const float m_safe = m_new == kNegInf ? 0.0f : m_new;
-    const float alpha = fast_exp2(m_run - m_safe);
-    m_run = m_new;
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-      l_run *= alpha;
-      p_sum *= alpha;
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[nb][j] *= alpha;
-      }
-    }
-    uint32_t pw[4];
-    {
-      const float4_t vs0 = *reinterpret_cast<const float4_t*>(vsc + 4 * lk);
-      const float4_t vs1 = *reinterpret_cast<const float4_t*>(vsc + 16 + 4 * lk);
-      float pe[8];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float e0 = fast_exp2(s[0][j] - m_safe);
-        const float e1 = fast_exp2(s[1][j] - m_safe);
-        l_run += e0 + e1;
-        pe[j] = e0 * vs0[j];
-        pe[4 + j] = e1 * vs1[j];
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        pw[j] = pack_pair<KIND>(pe[2 * j], pe[2 * j + 1]);
-        if constexpr (KIND == KV_I8) {
-          const Pair pr = __builtin_bit_cast(Pair, pw[j]);
-          p_sum += static_cast<float>(pr.x) + static_cast<float>(pr.y);
+        // -- fetch tile x + 1 (its block ids arrived during the previous iteration) and the ids of tile x + 2 ------
+        bool next_is_new_seq = false;
+        if (x + 1 < x1) {
+          next_is_new_seq = advance(kv_cur, x + 1);
+          if (next_is_new_seq) issue_q_loads(kv_cur.b);
+          issue_kv_loads();
+          if (x + 2 < x1) {
+            advance(id_cur, x + 2);
+            issue_id_loads();
+          }
         }
-      }
-    }
-    const V8 pop = __builtin_bit_cast(V8, uint4_t{pw[0], pw[1], pw[2], pw[3]});
 
-    // -- O^T += V^T . P^T, one MFMA per 16-dim block -------------------------------------------------------------
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      uint32_t vw[4];
-      if constexpr (ES == 1) {
-        // lane i of a 16-lane group supplies row (i / 2), 8 bytes at column 16 nb + 8 (i % 2)
-        const int r8 = lr >> 1;
-        const int tok = r8 < 4 ? 4 * lk + r8 : 16 + 4 * lk + (r8 - 4);
-        char* a = v_tile + v_row_of(tok) * RSV + 16 * nb + 8 * (lr & 1);
-        const int2_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_int2*)a);
-        vw[0] = static_cast<uint32_t>(r[0]);
-        vw[1] = static_cast<uint32_t>(r[1]);
-      } else {
-        // lane i supplies row (i / 4), 4 elements at column 16 nb + 4 (i % 4); two reads of 4 tokens each
-        const int r4 = lr >> 2;
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const int tok = 16 * half + 4 * lk + r4;
-          char* a = v_tile + v_row_of(tok) * RSV + (16 * nb + 4 * (lr & 3)) * 2;
-          const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
-          const uint2_t u = __builtin_bit_cast(uint2_t, r);
-          vw[2 * half] = u[0];
-          vw[2 * half + 1] = u[1];
+        // -- S^T = K . Q^T for the two 16-token groups ------------------------------------------------------------
+        float s[2][4];
+    #pragma unroll
+        for (int tg = 0; tg < 2; ++tg) {
+          float4_t c = {0.0f, 0.0f, 0.0f, 0.0f};
+          const char* krow = k_tile + (16 * tg + lr) * RSK + (D / 4) * ES * lk;
+          uint32_t kw[NS * WPL];
+    #pragma unroll
+          for (int q4 = 0; q4 < NS * WPL / 4; ++q4) {
+            const uint4_t r = *reinterpret_cast<const uint4_t*>(krow + 16 * q4);
+            kw[4 * q4 + 0] = r[0];
+            kw[4 * q4 + 1] = r[1];
+            kw[4 * q4 + 2] = r[2];
+            kw[4 * q4 + 3] = r[3];
+          }
+    #pragma unroll
+          for (int sl = 0; sl < NS; ++sl) c = Ops::mfma(to_operand<KIND>(&kw[sl * WPL]), qop[sl], c);
+          const float4_t sc = *reinterpret_cast<const float4_t*>(ksc + 16 * tg + 4 * lk);
+    #pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            // tokens past the end carry a -inf scale; keep them exactly -inf (0 * -inf would be NaN)
+            const float v = c[j] - qbias;
+            s[tg][j] = sc[j] == kNegInf ? kNegInf : v * sc[j];
+          }
         }
-      }
-      acc[nb] = Ops::mfma(to_operand<KIND>(vw), pop, acc[nb]);
-    }
-    // all LDS reads of this tile are done before the next iteration overwrites it
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
 
-    // -- end of a sequence's share: emit its partial and switch to the next sequence ---------------------------
-    const bool last_of_piece = x + 1 == x1;
-    if (next_is_new_seq || last_of_piece) {
-      write_partial(cp_b);
-      if (!last_of_piece) {
-        cp_b = kv_cur.b;
-        adopt_q();
-        reset_state();
+        // -- online softmax for head lr over the tile's 32 tokens ---------------------------------------------------
+        float mt = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                         fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+        mt = fmaxf(mt, wave_xor(mt, 16));
+        mt = fmaxf(mt, wave_xor(mt, 32));
+        const float m_new = fmaxf(m_run, mt);
+        const float m_safe = m_new == kNegInf ? 0.0f : m_new;
+        const float alpha = fast_exp2(m_run - m_safe);
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+          l_run *= alpha;
+          p_sum *= alpha;
+    #pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+    #pragma unroll
+            for (int j = 0; j < 4; ++j) acc[nb][j] *= alpha;
+          }
+        }
+        uint32_t pw[4];
+        {
+          const float4_t vs0 = *reinterpret_cast<const float4_t*>(vsc + 4 * lk);
+          const float4_t vs1 = *reinterpret_cast<const float4_t*>(vsc + 16 + 4 * lk);
+          float pe[8];
+    #pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float e0 = fast_exp2(s[0][j] - m_safe);
+            const float e1 = fast_exp2(s[1][j] - m_safe);
+            l_run += e0 + e1;
+            pe[j] = e0 * vs0[j];
+            pe[4 + j] = e1 * vs1[j];
+          }
+    #pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            pw[j] = pack_pair<KIND>(pe[2 * j], pe[2 * j + 1]);
+            if constexpr (KIND == KV_I8) {
+              const Pair pr = __builtin_bit_cast(Pair, pw[j]);
+              p_sum += static_cast<float>(pr.x) + static_cast<float>(pr.y);
+            }
+          }
+        }
+        const V8 pop = __builtin_bit_cast(V8, uint4_t{pw[0], pw[1], pw[2], pw[3]});
+
+        // -- O^T += V^T . P^T, one MFMA per 16-dim block -------------------------------------------------------------
+    #pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          uint32_t vw[4];
+          if constexpr (ES == 1) {
+            // lane i of a 16-lane group supplies row (i / 2), 8 bytes at column 16 nb + 8 (i % 2)
+            const int r8 = lr >> 1;
+            const int tok = r8 < 4 ? 4 * lk + r8 : 16 + 4 * lk + (r8 - 4);
+            char* a = v_tile + v_row_of(tok) * RSV + 16 * nb + 8 * (lr & 1);
+            const int2_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_int2*)a);
+            vw[0] = static_cast<uint32_t>(r[0]);
+            vw[1] = static_cast<uint32_t>(r[1]);
+          } else {
+            // lane i supplies row (i / 4), 4 elements at column 16 nb + 4 (i % 4); two reads of 4 tokens each
+            const int r4 = lr >> 2;
+    #pragma unroll
+            for (int half = 0; half < 2; ++half) {
+              const int tok = 16 * half + 4 * lk + r4;
+              char* a = v_tile + v_row_of(tok) * RSV + (16 * nb + 4 * (lr & 3)) * 2;
+              const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
+              const uint2_t u = __builtin_bit_cast(uint2_t, r);
+              vw[2 * half] = u[0];
+              vw[2 * half + 1] = u[1];
+            }
+          }
+          acc[nb] = Ops::mfma(to_operand<KIND>(vw), pop, acc[nb]);
+        }
+        // all LDS reads of this tile are done before the next iteration overwrites it
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+
+        // -- end of a sequence's share: emit its partial and switch to the next sequence ---------------------------
+        const bool last_of_piece = x + 1 == x1;
+        if (next_is_new_seq || last_of_piece) {
+          write_partial(cp_b);
+          if (!last_of_piece) {
+            cp_b = kv_cur.b;
+            adopt_q();
+            reset_state();
+          }
+        }
+        cp_tok = kv_cur.tok;
+        cp_end = kv_cur.end;
       }
     }
-    cp_tok = kv_cur.tok;
-    cp_end = kv_cur.end;
+#ifdef ARENO_TRACE
+    if (mp.trace && lane == 0) mp.trace[trace_wave * 16 + 1] = wall_clock64();
+#endif
+    if (geo.small_units == 0) break;
+    int claimed = 0;
+    if (lane == 0) claimed = atomicAdd(ticket, 1);
+    claimed = __builtin_amdgcn_readfirstlane(claimed);
+    if (claimed >= geo.small_units) break;
+    unit = geo.static_units + claimed;
   }
 }
 
@@ -549,12 +628,13 @@ decode_mfma_fn decode_mfma_lookup_fp8(int head_dim, bool scale16);
 
 template <int KIND>
 decode_mfma_fn decode_mfma_lookup_impl(int head_dim, bool scale16) {
+  constexpr int NW = ARENO_MFMA_NW;
   if constexpr (KVTraits<KIND>::kQuant) {
-    if (head_dim == 128) return scale16 ? decode_mfma_kernel<KIND, 128, true> : decode_mfma_kernel<KIND, 128, false>;
-    if (head_dim == 64) return scale16 ? decode_mfma_kernel<KIND, 64, true> : decode_mfma_kernel<KIND, 64, false>;
+    if (head_dim == 128) return scale16 ? decode_mfma_kernel<KIND, 128, true, NW> : decode_mfma_kernel<KIND, 128, false, NW>;
+    if (head_dim == 64) return scale16 ? decode_mfma_kernel<KIND, 64, true, NW> : decode_mfma_kernel<KIND, 64, false, NW>;
   } else {
-    if (head_dim == 128) return decode_mfma_kernel<KIND, 128, false>;
-    if (head_dim == 64) return decode_mfma_kernel<KIND, 64, false>;
+    if (head_dim == 128) return decode_mfma_kernel<KIND, 128, false, NW>;
+    if (head_dim == 64) return decode_mfma_kernel<KIND, 64, false, NW>;
   }
   return nullptr;
 }

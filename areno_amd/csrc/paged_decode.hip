@@ -12,6 +12,9 @@
 namespace areno {
 
 int validate_paged_cache(const areno_paged_cache* c, const char* op);
+int launch_cache_write_decode(const areno_paged_cache* cache, const void* k_update, const void* v_update,
+                              int32_t in_dtype, int32_t batch, const int32_t* block_table, int32_t max_blocks,
+                              const int32_t* cache_seqlens, int32_t* zero_words, int32_t zero_count, void* stream);
 
 namespace {
 
@@ -128,8 +131,10 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_kernel(Decod
   }
 }
 
-// Merge of the MFMA path's partials: the pieces that own tiles of sequence b wrote slots (piece + b);
-// pieces that own no tile at all are skipped.  One wave per (sequence, q head).
+// Merge of the MFMA path's partials: the units that own tiles of sequence b wrote slots (unit + b); units that
+// own no tile at all are skipped.  One wave per (sequence, q head): lanes first fetch the (m, l) pairs of up to 64
+// slots in parallel and agree on the maximum, then every lane accumulates its share of the head dimension with
+// all partial loads of a group of four slots in flight together (the loop has no loop-carried memory dependence).
 __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel(MfmaDecodeParams mp) {
   const DecodeParams& p = mp.d;
   const int lane = threadIdx.x & (kWave - 1);
@@ -138,35 +143,54 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   const int b = row / p.q_heads;
   const int h = row - b * p.q_heads;
   const int d = p.head_dim;
-  const int64_t nt = mp.plan[p.batch];
-  const int64_t np = mp.num_pieces;
-  const int64_t first_tile = mp.plan[b];
-  const int64_t last_tile = static_cast<int64_t>(mp.plan[b + 1]) - 1;
-  // owner(x): the largest piece whose first tile (piece * nt / np) is <= x
-  const int wp_lo = static_cast<int>(((first_tile + 1) * np + nt - 1) / nt - 1);
-  const int wp_hi = static_cast<int>(((last_tile + 1) * np + nt - 1) / nt - 1);
+  const UnitGeometry geo = make_unit_geometry(mp.plan[p.batch], mp.num_pieces, mp.static_share, mp.min_unit_tiles);
+  const int u_lo = geo.unit_of(mp.plan[b]);
+  const int u_hi = geo.unit_of(mp.plan[b + 1] - 1);
 
   float acc[kGenericMaxPerLane];
 #pragma unroll
   for (int e = 0; e < kGenericMaxPerLane; ++e) acc[e] = 0.0f;
   float m = kNegInf, l = 0.0f;
-  for (int wp = wp_lo; wp <= wp_hi; ++wp) {
-    if (wp * nt / np == (wp + 1) * nt / np) continue;  // piece without tiles
-    const int64_t prow = static_cast<int64_t>(wp + b) * p.q_heads + h;
-    const float part_m = p.part_ml[prow * 2];
-    const float part_l = p.part_ml[prow * 2 + 1];
-    if (part_l == 0.0f) continue;
-    const float m_new = fmaxf(m, part_m);
-    const float alpha = fast_exp2(m - m_new);
-    const float beta = fast_exp2(part_m - m_new);
-    const float* part = p.part_acc + prow * d;
-#pragma unroll
-    for (int e = 0; e < kGenericMaxPerLane; ++e) {
-      const int idx = lane + e * kWave;
-      if (idx < d) acc[e] = acc[e] * alpha + part[idx] * beta;
+  for (int base = u_lo; base <= u_hi; base += kWave) {
+    // lane j looks at unit base + j
+    const int u = base + lane;
+    float part_m = kNegInf, part_l = 0.0f;
+    if (u <= u_hi && geo.unit_start(u) != geo.unit_start(u + 1)) {
+      const int64_t prow = static_cast<int64_t>(u + b) * p.q_heads + h;
+      part_m = p.part_ml[prow * 2];
+      part_l = p.part_ml[prow * 2 + 1];
+      if (part_l == 0.0f) part_m = kNegInf;  // a partial without keys contributes nothing
     }
-    l = l * alpha + part_l * beta;
+    const float m_new = fmaxf(m, wave_max(part_m));
+    const float m_safe = m_new == kNegInf ? 0.0f : m_new;
+    const float alpha = fast_exp2(m - m_safe);
+    const float w = fast_exp2(part_m - m_safe);  // 0 for absent slots
+    l = l * alpha + wave_sum(w * part_l);
     m = m_new;
+#pragma unroll
+    for (int e = 0; e < kGenericMaxPerLane; ++e) acc[e] *= alpha;
+    const int count = min(kWave, u_hi - base + 1);
+    for (int j0 = 0; j0 < count; j0 += 4) {
+      float wj[4];
+      float v[4][kGenericMaxPerLane];
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const int j = min(j0 + jj, count - 1);
+        wj[jj] = j0 + jj < count ? __shfl(w, j, kWave) : 0.0f;
+        const float* part = p.part_acc + (static_cast<int64_t>(base + j + b) * p.q_heads + h) * d;
+#pragma unroll
+        for (int e = 0; e < kGenericMaxPerLane; ++e) {
+          const int idx = lane + e * kWave;
+          // slots of units without tiles were never written: read them only with a non-zero weight
+          v[jj][e] = (idx < d && wj[jj] != 0.0f) ? part[idx] : 0.0f;
+        }
+      }
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+#pragma unroll
+        for (int e = 0; e < kGenericMaxPerLane; ++e) acc[e] += wj[jj] * v[jj][e];
+      }
+    }
   }
 #pragma unroll
   for (int e = 0; e < kGenericMaxPerLane; ++e) {
@@ -175,15 +199,30 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   }
 }
 
+__global__ void zero_words_kernel(int32_t* words, int count) {
+  if (static_cast<int>(threadIdx.x) < count) words[threadIdx.x] = 0;
+}
+
 // ---- geometry of the MFMA path ----------------------------------------------------------------------
-constexpr int kMfmaWorkgroups = 512;  // two resident workgroups on each of the 256 CUs
-constexpr int kMfmaMaxPieces = kMfmaWorkgroups * 4;
+constexpr int kMfmaWaves = ARENO_MFMA_NW;  // waves per workgroup
+constexpr int kMfmaWorkgroups = 512;       // two resident workgroups on each of the 256 CUs
+constexpr int kMfmaMaxPieces = kMfmaWorkgroups * kMfmaWaves;
+constexpr int kMaxKvHeadsCounters = 256;
+
+size_t mfma_partial_bytes(size_t slots, int q_heads, int head_dim) {
+  const size_t bytes = slots * q_heads * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
+  return (bytes + 255) / 256 * 256;
+}
 
 size_t mfma_workspace_bytes(int batch, int q_heads, int head_dim) {
-  const size_t slots = static_cast<size_t>(kMfmaMaxPieces) + batch;
-  size_t bytes = slots * q_heads * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
-  bytes = (bytes + 255) / 256 * 256;
-  return bytes + (static_cast<size_t>(batch) + 1 + 63) / 64 * 64 * sizeof(int32_t);
+  const size_t slots = static_cast<size_t>(kMfmaMaxPieces) + kMaxSmallUnits + batch;
+  const size_t plan_words = (static_cast<size_t>(batch) + 1 + 63) / 64 * 64 + kMaxKvHeadsCounters;
+  return mfma_partial_bytes(slots, q_heads, head_dim) + plan_words * sizeof(int32_t);
+}
+
+int env_int(const char* name, int fallback) {
+  const char* v = getenv(name);
+  return v != nullptr ? atoi(v) : fallback;
 }
 
 // "valu" forces the vector-ALU split kernel, "mfma" (default) prefers the matrix-core kernel where it applies.
@@ -283,12 +322,6 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
   if (workspace == nullptr || workspace_bytes < need)
     return fail(ARENO_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", op, need, workspace_bytes);
 
-  if (k_update != nullptr && (stages & ARENO_STAGE_APPEND)) {
-    if (int rc = areno_hip_cache_write_decode(cache, k_update, v_update, q_dtype, batch, block_table, max_blocks,
-                                              cache_seqlens, stream))
-      return rc;
-  }
-
   DecodeParams p;
   p.q = q;
   p.k_cache = cache->k;
@@ -336,7 +369,7 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
   // ---- matrix-core path: 16-bit or 8-bit caches, head_dim 64/128, up to 16 q heads per kv head ------------
   decode_mfma_fn mfma = nullptr;
   if (aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && num_splits != 1 && p.group <= 16 &&
-      batch <= kMfmaMaxBatch) {
+      batch <= kMfmaMaxBatch && cache->kv_heads <= kMaxKvHeadsCounters) {
     switch (cache->cache_dtype) {
       case ARENO_DT_BF16: mfma = decode_mfma_lookup_bf16(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
       case ARENO_DT_F16: mfma = decode_mfma_lookup_f16(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
@@ -345,20 +378,52 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
       default: break;
     }
   }
+  // ---- geometry of the MFMA launch (needed before the append: that kernel clears the ticket counters) ----------
+  MfmaDecodeParams mp;
+  int grid_x = 0, head_groups = 0;
   if (mfma != nullptr) {
-    MfmaDecodeParams mp;
     mp.d = p;
-    const int head_groups = cache->kv_heads / p.heads_per_wg;
-    const int grid_x = kMfmaWorkgroups / head_groups > 0 ? kMfmaWorkgroups / head_groups : 1;
-    mp.tok_splits = 4 / p.heads_per_wg;
+    head_groups = cache->kv_heads / p.heads_per_wg;
+    static const int wgs = [] {
+      const int v = env_int("ARENO_MFMA_WGS", kMfmaWorkgroups);
+      return v > 0 && v <= kMfmaWorkgroups ? v : kMfmaWorkgroups;
+    }();
+    static const int static_share = env_int("ARENO_MFMA_STATIC", 256);
+    static const int unit_tiles = env_int("ARENO_MFMA_UNIT", 4);
+    grid_x = wgs / head_groups > 0 ? wgs / head_groups : 1;
+    mp.tok_splits = kMfmaWaves / p.heads_per_wg;
     mp.num_pieces = grid_x * mp.tok_splits;
-    const size_t slots = static_cast<size_t>(mp.num_pieces) + batch;
-    const size_t part_bytes = (slots * q_heads * (static_cast<size_t>(p.head_dim) + 2) * sizeof(float) + 255) / 256 * 256;
+    mp.static_share = static_share;
+    mp.min_unit_tiles = unit_tiles;
+#ifdef ARENO_TRACE
+    mp.trace = getenv("ARENO_TRACE_BUF") ? reinterpret_cast<unsigned long long*>(strtoull(getenv("ARENO_TRACE_BUF"), nullptr, 0)) : nullptr;
+#endif
+    const size_t slots = static_cast<size_t>(mp.num_pieces) + kMaxSmallUnits + batch;
+    const size_t part_bytes = mfma_partial_bytes(slots, q_heads, p.head_dim);
     mp.d.part_ml = static_cast<float*>(workspace);
     mp.d.part_acc = mp.d.part_ml + slots * q_heads * 2;
     mp.plan = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + part_bytes);
+    mp.unit_counter = mp.plan + (static_cast<size_t>(batch) + 1 + 63) / 64 * 64;
+  }
+
+  // ---- append (first launch) ------------------------------------------------------------------------------------
+  bool counters_cleared = false;
+  if (k_update != nullptr && (stages & ARENO_STAGE_APPEND)) {
+    if (int rc = launch_cache_write_decode(cache, k_update, v_update, q_dtype, batch, block_table, max_blocks,
+                                           cache_seqlens, mfma != nullptr ? mp.unit_counter : nullptr,
+                                           mfma != nullptr ? cache->kv_heads : 0, stream))
+      return rc;
+    counters_cleared = mfma != nullptr;
+  }
+
+  if (mfma != nullptr) {
     if (stages & ARENO_STAGE_SPLIT) {
-      hipLaunchKernelGGL(mfma, dim3(grid_x, head_groups), dim3(kDecodeThreads), 0, s, mp);
+      // the ticket counters start at zero: the append kernel cleared them, otherwise a one-wave fill does
+      if (!counters_cleared) {
+        hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(kMaxKvHeadsCounters), 0, s, mp.unit_counter,
+                           static_cast<int>(cache->kv_heads));
+      }
+      hipLaunchKernelGGL(mfma, dim3(grid_x, head_groups), dim3(kMfmaWaves * kWave), 0, s, mp);
       if (int rc = check_launch(op)) return rc;
     }
     if (stages & ARENO_STAGE_REDUCE) {
