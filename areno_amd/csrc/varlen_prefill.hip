@@ -166,6 +166,21 @@ extern "C" int areno_hip_varlen_attention(const void* q, const void* k, const vo
     return fail(ARENO_ERR_UNSUPPORTED, "%s: dtype must be f32, f16 or bf16", op);
   if (head_dim > kMaxPerLane * kWave) return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim %d > 512", op, head_dim);
   if (tokens == 0) return ARENO_OK;
+  {
+    // packed K/V described as a one-block "cache" for the MFMA kernel (it addresses rows directly in this mode)
+    areno_paged_cache packed = {};
+    packed.k = const_cast<void*>(k);
+    packed.v = const_cast<void*>(v);
+    packed.num_blocks = 1;
+    packed.block_size = 1;
+    packed.kv_heads = kv_heads;
+    packed.head_dim = head_dim;
+    packed.cache_dtype = dtype;
+    packed.scale_dtype = ARENO_DT_F32;
+    const int rc = launch_prefill_mfma(&packed, q, out, dtype, tokens, q_heads, num_seqs, nullptr, 1, cu_seqlens,
+                                       nullptr, window_left, softmax_scale, stream);
+    if (rc != ARENO_ERR_UNSUPPORTED) return rc;
+  }
   VarlenParams p = {};
   p.q = q;
   p.k = k;

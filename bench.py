@@ -189,6 +189,57 @@ def measure_decode(w, steps, warmup, *, kernel_iters=60):
     }
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def measure_prefill(w, iters=20):
+    """Time the paged-prefill op (and the quantizing cache write that precedes it) on cfg 4; MFMA-bound."""
+    import torch
+
+    from areno_amd.accel import attention as ops
+
+    def write():
+        ops.areno_paged_cache_write(w.k_new, w.v_new, w.k_cache, w.v_cache, w.cache_block_ids, w.cache_block_offsets,
+                                    k_scale=w.k_scale, v_scale=w.v_scale)  # fmt: skip
+
+    def attend():
+        return ops.areno_paged_varlen_causal_attention(
+            w.q, w.k_cache, w.v_cache, w.block_table, w.cu_seqlens_q, w.context_lens,
+            softmax_scale=w.softmax_scale, k_scale=w.k_scale, v_scale=w.v_scale,
+        )  # fmt: skip
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        samples = []
+        for _ in range(iters):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            e1.synchronize()
+            samples.append(e0.elapsed_time(e1) * 1e3)
+        return statistics.median(samples)
+
+    us_write = timed(write)
+    us_attend = timed(attend)
+    flops = w.flops()
+    tflops = flops / (us_attend * 1e-6) / 1e12
+    return {
+        "workload": w.name,
+        "us_per_step": us_attend + us_write,
+        "kernel_us": {"cache_write": us_write, "prefill": us_attend},
+        "new_tokens": int(w.q.shape[0]),
+        "tokens_per_s": w.q.shape[0] / ((us_attend + us_write) * 1e-6),
+        "flops": flops,
+        "roofline": {
+            "bound": "mfma", "kernel": "prefill_mfma_kernel", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS,
+            "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+        },  # fmt: skip
+    }
+
+
 def cpu_baseline(w, rows=16, repeats=3):
     """The CPU oracle (PyTorch restatement of the reference's native path) on the first `rows` sequences."""
     import torch
@@ -227,7 +278,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3"], default=None, help="measure a single workload")
+    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4"], default=None, help="measure a single workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -252,20 +303,21 @@ def main() -> int:
         "cfg1": lambda: workloads.cfg1_qwen7b("bf16", device=dev),
         "cfg2": lambda: workloads.cfg2_qwen7b_int8(device=dev, quantize_fn=_gpu_quantize),
         "cfg3": lambda: workloads.cfg3_rollout("fp8", device=dev, quantize_fn=_gpu_quantize),
+        "cfg4": lambda: workloads.cfg4_prefill("fp8", device=dev, quantize_fn=_gpu_quantize),
     }
-    names = [args.only] if args.only else ["cfg1", "cfg2", "cfg3"]
+    names = [args.only] if args.only else ["cfg1", "cfg2", "cfg3", "cfg4"]
     results = {}
     baseline = None
     for name in names:
         w = builders[name]()
-        results[name] = measure_decode(w, args.steps, args.warmup)
-        if name == names[0] and not args.no_cpu:
+        results[name] = measure_prefill(w) if name == "cfg4" else measure_decode(w, args.steps, args.warmup)
+        if name == names[0] and not args.no_cpu and name != "cfg4":
             baseline = cpu_baseline(w)
         del w
         torch.cuda.empty_cache()
 
     head = results[names[0]]
-    dtype = {"cfg1": "bf16", "cfg2": "int8", "cfg3": "fp8"}[names[0]]
+    dtype = {"cfg1": "bf16", "cfg2": "int8", "cfg3": "fp8", "cfg4": "fp8"}[names[0]]
     line = {
         "metric": "paged_decode_attn_us_per_step",
         "value": head["us_per_step"],
@@ -285,7 +337,7 @@ def main() -> int:
             "launch": "HIP graph replay, KV pools rotated over >1.3 GB",
         },
         "tokens_per_s": head["tokens_per_s"],
-        "hbm_gbps_op": head["op_gbps"],
+        "hbm_gbps_op": head.get("op_gbps"),
         "roofline": head["roofline"],
         "cpu_baseline": baseline,
         "workloads": results,
