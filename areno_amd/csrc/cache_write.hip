@@ -37,8 +37,6 @@ struct WriteParams {
   int32_t in_dtype;
   int32_t cache_dtype;
   int32_t scale_dtype;
-  int32_t* zero_words;  // optional: block (0, 0) clears zero_count words (<= 256) for the decode op
-  int32_t zero_count;
 };
 
 constexpr int kRowsPerBlock = 4;  // one wave per row
@@ -46,8 +44,6 @@ constexpr int kMaxPerLane = 8;    // head_dim <= 512
 
 __global__ __launch_bounds__(kRowsPerBlock* kWave) void cache_write_kernel(WriteParams p) {
   const int lane = threadIdx.x & (kWave - 1);
-  if (p.zero_words != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && static_cast<int>(threadIdx.x) < p.zero_count)
-    p.zero_words[threadIdx.x] = 0;
   const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + (threadIdx.x >> 6);
   if (row >= p.tokens * p.kv_heads) return;
   const int which = blockIdx.y;  // 0 = K, 1 = V
@@ -156,8 +152,7 @@ int validate_cache(const areno_paged_cache* c, const char* op) {
 
 int launch_write(const areno_paged_cache* cache, const void* k, const void* v, int32_t in_dtype, int64_t tokens,
                  const int64_t* ids, const int64_t* offs, const int32_t* table, int32_t max_blocks,
-                 const int32_t* seqlens, void* stream, const char* op, int32_t* zero_words = nullptr,
-                 int32_t zero_count = 0) {
+                 const int32_t* seqlens, void* stream, const char* op) {
   if (int rc = validate_cache(cache, op)) return rc;
   if (tokens < 0) return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: negative token count", op);
   if (tokens > 0 && (k == nullptr || v == nullptr))
@@ -193,8 +188,6 @@ int launch_write(const areno_paged_cache* cache, const void* k, const void* v, i
   p.in_dtype = in_dtype;
   p.cache_dtype = cache->cache_dtype;
   p.scale_dtype = cache->scale_dtype;
-  p.zero_words = zero_words;
-  p.zero_count = zero_count;
   hipLaunchKernelGGL(cache_write_kernel, dim3(static_cast<unsigned>(blocks), 2), dim3(kRowsPerBlock * kWave), 0,
                      static_cast<hipStream_t>(stream), p);
   return check_launch(op);
@@ -203,17 +196,6 @@ int launch_write(const areno_paged_cache* cache, const void* k, const void* v, i
 }  // namespace
 
 int validate_paged_cache(const areno_paged_cache* c, const char* op) { return validate_cache(c, op); }
-
-// The decode op's first launch: the append, optionally clearing a few workspace words for the kernels after it.
-int launch_cache_write_decode(const areno_paged_cache* cache, const void* k_update, const void* v_update,
-                              int32_t in_dtype, int32_t batch, const int32_t* block_table, int32_t max_blocks,
-                              const int32_t* cache_seqlens, int32_t* zero_words, int32_t zero_count, void* stream) {
-  if (batch > 0 && (block_table == nullptr || cache_seqlens == nullptr || max_blocks <= 0))
-    return fail(ARENO_ERR_INVALID_ARGUMENT, "areno_hip_cache_write_decode: block_table/cache_seqlens missing");
-  if (zero_count > kRowsPerBlock * kWave) return fail(ARENO_ERR_INVALID_ARGUMENT, "too many words to clear");
-  return launch_write(cache, k_update, v_update, in_dtype, batch, nullptr, nullptr, block_table, max_blocks,
-                      cache_seqlens, stream, "areno_hip_cache_write_decode", zero_words, zero_count);
-}
 
 }  // namespace areno
 
@@ -229,6 +211,8 @@ extern "C" int areno_hip_cache_write(const areno_paged_cache* cache, const void*
 extern "C" int areno_hip_cache_write_decode(const areno_paged_cache* cache, const void* k_update, const void* v_update,
                                             int32_t in_dtype, int32_t batch, const int32_t* block_table,
                                             int32_t max_blocks, const int32_t* cache_seqlens, void* stream) {
-  return areno::launch_cache_write_decode(cache, k_update, v_update, in_dtype, batch, block_table, max_blocks,
-                                          cache_seqlens, nullptr, 0, stream);
+  if (batch > 0 && (block_table == nullptr || cache_seqlens == nullptr || max_blocks <= 0))
+    return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "areno_hip_cache_write_decode: block_table/cache_seqlens missing");
+  return areno::launch_write(cache, k_update, v_update, in_dtype, batch, nullptr, nullptr, block_table, max_blocks,
+                             cache_seqlens, stream, "areno_hip_cache_write_decode");
 }

@@ -54,11 +54,12 @@ typedef __attribute__((ext_vector_type(2))) int int2_t;
 
 struct MfmaDecodeParams {
   DecodeParams d;      // part_ml / part_acc are indexed [slot][q_head] here
-  int32_t* plan;         // [batch + 4]: exclusive prefix sums of tiles per sequence, then the unit geometry
-  int32_t* unit_counter;  // [head groups] dynamic-unit tickets, zero when the kernel starts
+  int32_t* plan;         // [batch + 1]: exclusive prefix sums of tiles per sequence (written by workgroup 0)
   int32_t tok_splits;    // waves of a workgroup that share a KV head (waves per workgroup / heads_per_wg)
-  int32_t num_pieces;    // gridDim.x * tok_splits: statically assigned units
-  int32_t static_share;  // n/256 of all tiles are assigned statically, the rest is claimed in small units
+  int32_t static_wgs;    // workgroups [0, static_wgs) own the big units, the rest of the grid the small ones
+  int32_t num_pieces;    // static_wgs * tok_splits: big units
+  int32_t max_small;     // (gridDim.x - static_wgs) * tok_splits: small units available
+  int32_t static_share;  // n/256 of all tiles go to the big units
   int32_t min_unit_tiles;
 #ifdef ARENO_TRACE
   unsigned long long* trace;  // [wave][16] timestamps, tuning builds only
@@ -142,19 +143,18 @@ struct UnitGeometry {
   }
 };
 
-constexpr int kMaxSmallUnits = 1024;
-
-__host__ __device__ inline UnitGeometry make_unit_geometry(int total_tiles, int num_pieces, int static_share,
-                                                           int min_unit_tiles) {
+__host__ __device__ inline UnitGeometry make_unit_geometry(int total_tiles, int num_pieces, int max_small,
+                                                           int static_share, int min_unit_tiles) {
   UnitGeometry g;
   g.total_tiles = total_tiles;
   g.static_units = num_pieces;
   g.static_tiles = static_cast<int>(static_cast<long long>(total_tiles) * static_share / 256);
-  // short batches are not worth a claimed tail: everything static
-  if (total_tiles < 4 * num_pieces || static_share >= 256) g.static_tiles = total_tiles;
+  // short batches are not worth a tail of small units: everything goes to the big ones
+  if (total_tiles < 4 * num_pieces || static_share >= 256 || max_small <= 0) g.static_tiles = total_tiles;
   const int rest = total_tiles - g.static_tiles;
   g.unit_tiles = min_unit_tiles < 1 ? 1 : min_unit_tiles;
-  if (static_cast<long long>(g.unit_tiles) * kMaxSmallUnits < rest) g.unit_tiles = (rest + kMaxSmallUnits - 1) / kMaxSmallUnits;
+  if (max_small > 0 && static_cast<long long>(g.unit_tiles) * max_small < rest)
+    g.unit_tiles = (rest + max_small - 1) / max_small;
   g.small_units = (rest + g.unit_tiles - 1) / g.unit_tiles;
   return g;
 }
@@ -244,11 +244,13 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
     __syncthreads();
   }
   // ---- unit geometry -----------------------------------------------------------------------------------
-  // Tiles [0, static_tiles) are cut into num_pieces equal static units (one per wave); the rest is cut into
-  // small units of unit_tiles tiles that waves claim from a ticket counter once their static unit is done:
-  // memory service is uneven across CUs, and without the claimed tail the slowest wave sets the run time.
+  // Tiles [0, static_tiles) are cut into num_pieces equal big units, one per wave of the first static_wgs
+  // workgroups; the rest is cut into small units for the workgroups behind them in the grid.  Those start as CUs
+  // become free, so the hardware dispatcher hands the tail to whichever CU got the better memory service:
+  // service is uneven across CUs, and with equal shares only the slowest wave would set the run time.
   const int total_tiles = s_cum[p.batch];
-  const UnitGeometry geo = make_unit_geometry(total_tiles, mp.num_pieces, mp.static_share, mp.min_unit_tiles);
+  const UnitGeometry geo =
+      make_unit_geometry(total_tiles, mp.num_pieces, mp.max_small, mp.static_share, mp.min_unit_tiles);
   if (blockIdx.x == 0 && blockIdx.y == 0) {
     for (int b = tid; b <= p.batch; b += NW * kWave) mp.plan[b] = s_cum[b];
   }
@@ -257,9 +259,6 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
   const int hw = wave % hw_count;
   const int ts = wave / hw_count;
   const int kvh = blockIdx.y * hw_count + hw;
-  // one ticket counter per KV head: every wave that works on this head draws from it
-  int* const ticket = mp.unit_counter + kvh;
-
   char* const k_tile = &s_tiles[wave][0];
   char* const v_tile = k_tile + TK * RSK;
   float* const ksc = reinterpret_cast<float*>(&s_tiles[wave][TK * RSK + TK * RSV]);
@@ -412,11 +411,12 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
     }
   };
 
-  // ---- units: the wave's static unit first, then claimed ones ---------------------------------------------------
-  unit = blockIdx.x * mp.tok_splits + ts;
-  while (true) {
+  // ---- this wave's unit ------------------------------------------------------------------------------------------
+  const int bx = blockIdx.x;
+  unit = bx < mp.static_wgs ? bx * mp.tok_splits + ts : geo.static_units + (bx - mp.static_wgs) * mp.tok_splits + ts;
+  {
     const int x0 = geo.unit_start(unit);
-    const int x1 = geo.unit_start(unit + 1);
+    const int x1 = unit < geo.static_units + geo.small_units ? geo.unit_start(unit + 1) : x0;
     if (x0 < x1) {
       // sequence that owns tile x0: largest b with cum[b] <= x0
       int b_first;
@@ -611,12 +611,6 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
 #ifdef ARENO_TRACE
     if (mp.trace && lane == 0) mp.trace[trace_wave * 16 + 1] = wall_clock64();
 #endif
-    if (geo.small_units == 0) break;
-    int claimed = 0;
-    if (lane == 0) claimed = atomicAdd(ticket, 1);
-    claimed = __builtin_amdgcn_readfirstlane(claimed);
-    if (claimed >= geo.small_units) break;
-    unit = geo.static_units + claimed;
   }
 }
 

@@ -12,9 +12,6 @@
 namespace areno {
 
 int validate_paged_cache(const areno_paged_cache* c, const char* op);
-int launch_cache_write_decode(const areno_paged_cache* cache, const void* k_update, const void* v_update,
-                              int32_t in_dtype, int32_t batch, const int32_t* block_table, int32_t max_blocks,
-                              const int32_t* cache_seqlens, int32_t* zero_words, int32_t zero_count, void* stream);
 
 namespace {
 
@@ -143,7 +140,8 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   const int b = row / p.q_heads;
   const int h = row - b * p.q_heads;
   const int d = p.head_dim;
-  const UnitGeometry geo = make_unit_geometry(mp.plan[p.batch], mp.num_pieces, mp.static_share, mp.min_unit_tiles);
+  const UnitGeometry geo =
+      make_unit_geometry(mp.plan[p.batch], mp.num_pieces, mp.max_small, mp.static_share, mp.min_unit_tiles);
   const int u_lo = geo.unit_of(mp.plan[b]);
   const int u_hi = geo.unit_of(mp.plan[b + 1] - 1);
 
@@ -199,15 +197,11 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   }
 }
 
-__global__ void zero_words_kernel(int32_t* words, int count) {
-  if (static_cast<int>(threadIdx.x) < count) words[threadIdx.x] = 0;
-}
-
 // ---- geometry of the MFMA path ----------------------------------------------------------------------
 constexpr int kMfmaWaves = ARENO_MFMA_NW;  // waves per workgroup
-constexpr int kMfmaWorkgroups = 512;       // two resident workgroups on each of the 256 CUs
-constexpr int kMfmaMaxPieces = kMfmaWorkgroups * kMfmaWaves;
-constexpr int kMaxKvHeadsCounters = 256;
+constexpr int kMfmaWorkgroups = 512;       // big units: two resident workgroups on each of the 256 CUs
+constexpr int kMfmaTailWorkgroups = 256;   // small units behind them in the grid
+constexpr int kMfmaMaxPieces = (kMfmaWorkgroups + kMfmaTailWorkgroups) * kMfmaWaves;
 
 size_t mfma_partial_bytes(size_t slots, int q_heads, int head_dim) {
   const size_t bytes = slots * q_heads * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
@@ -215,8 +209,8 @@ size_t mfma_partial_bytes(size_t slots, int q_heads, int head_dim) {
 }
 
 size_t mfma_workspace_bytes(int batch, int q_heads, int head_dim) {
-  const size_t slots = static_cast<size_t>(kMfmaMaxPieces) + kMaxSmallUnits + batch;
-  const size_t plan_words = (static_cast<size_t>(batch) + 1 + 63) / 64 * 64 + kMaxKvHeadsCounters;
+  const size_t slots = static_cast<size_t>(kMfmaMaxPieces) + batch;
+  const size_t plan_words = (static_cast<size_t>(batch) + 1 + 63) / 64 * 64;
   return mfma_partial_bytes(slots, q_heads, head_dim) + plan_words * sizeof(int32_t);
 }
 
@@ -369,7 +363,7 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
   // ---- matrix-core path: 16-bit or 8-bit caches, head_dim 64/128, up to 16 q heads per kv head ------------
   decode_mfma_fn mfma = nullptr;
   if (aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && num_splits != 1 && p.group <= 16 &&
-      batch <= kMfmaMaxBatch && cache->kv_heads <= kMaxKvHeadsCounters) {
+      batch <= kMfmaMaxBatch) {
     switch (cache->cache_dtype) {
       case ARENO_DT_BF16: mfma = decode_mfma_lookup_bf16(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
       case ARENO_DT_F16: mfma = decode_mfma_lookup_f16(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
@@ -378,52 +372,44 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
       default: break;
     }
   }
-  // ---- geometry of the MFMA launch (needed before the append: that kernel clears the ticket counters) ----------
-  MfmaDecodeParams mp;
-  int grid_x = 0, head_groups = 0;
+  // ---- append (first launch) ------------------------------------------------------------------------------------
+  if (k_update != nullptr && (stages & ARENO_STAGE_APPEND)) {
+    if (int rc = areno_hip_cache_write_decode(cache, k_update, v_update, q_dtype, batch, block_table, max_blocks,
+                                              cache_seqlens, stream))
+      return rc;
+  }
+
   if (mfma != nullptr) {
+    MfmaDecodeParams mp;
     mp.d = p;
-    head_groups = cache->kv_heads / p.heads_per_wg;
+    const int head_groups = cache->kv_heads / p.heads_per_wg;
     static const int wgs = [] {
       const int v = env_int("ARENO_MFMA_WGS", kMfmaWorkgroups);
       return v > 0 && v <= kMfmaWorkgroups ? v : kMfmaWorkgroups;
     }();
+    static const int tail_wgs = [] {
+      const int v = env_int("ARENO_MFMA_TAIL_WGS", 0);
+      return v >= 0 && v <= kMfmaTailWorkgroups ? v : kMfmaTailWorkgroups;
+    }();
     static const int static_share = env_int("ARENO_MFMA_STATIC", 256);
     static const int unit_tiles = env_int("ARENO_MFMA_UNIT", 4);
-    grid_x = wgs / head_groups > 0 ? wgs / head_groups : 1;
+    mp.static_wgs = wgs / head_groups > 0 ? wgs / head_groups : 1;
+    const int extra = tail_wgs / head_groups;
     mp.tok_splits = kMfmaWaves / p.heads_per_wg;
-    mp.num_pieces = grid_x * mp.tok_splits;
+    mp.num_pieces = mp.static_wgs * mp.tok_splits;
+    mp.max_small = extra * mp.tok_splits;
     mp.static_share = static_share;
     mp.min_unit_tiles = unit_tiles;
 #ifdef ARENO_TRACE
     mp.trace = getenv("ARENO_TRACE_BUF") ? reinterpret_cast<unsigned long long*>(strtoull(getenv("ARENO_TRACE_BUF"), nullptr, 0)) : nullptr;
 #endif
-    const size_t slots = static_cast<size_t>(mp.num_pieces) + kMaxSmallUnits + batch;
+    const size_t slots = static_cast<size_t>(mp.num_pieces) + mp.max_small + batch;
     const size_t part_bytes = mfma_partial_bytes(slots, q_heads, p.head_dim);
     mp.d.part_ml = static_cast<float*>(workspace);
     mp.d.part_acc = mp.d.part_ml + slots * q_heads * 2;
     mp.plan = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + part_bytes);
-    mp.unit_counter = mp.plan + (static_cast<size_t>(batch) + 1 + 63) / 64 * 64;
-  }
-
-  // ---- append (first launch) ------------------------------------------------------------------------------------
-  bool counters_cleared = false;
-  if (k_update != nullptr && (stages & ARENO_STAGE_APPEND)) {
-    if (int rc = launch_cache_write_decode(cache, k_update, v_update, q_dtype, batch, block_table, max_blocks,
-                                           cache_seqlens, mfma != nullptr ? mp.unit_counter : nullptr,
-                                           mfma != nullptr ? cache->kv_heads : 0, stream))
-      return rc;
-    counters_cleared = mfma != nullptr;
-  }
-
-  if (mfma != nullptr) {
     if (stages & ARENO_STAGE_SPLIT) {
-      // the ticket counters start at zero: the append kernel cleared them, otherwise a one-wave fill does
-      if (!counters_cleared) {
-        hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(kMaxKvHeadsCounters), 0, s, mp.unit_counter,
-                           static_cast<int>(cache->kv_heads));
-      }
-      hipLaunchKernelGGL(mfma, dim3(grid_x, head_groups), dim3(kMfmaWaves * kWave), 0, s, mp);
+      hipLaunchKernelGGL(mfma, dim3(mp.static_wgs + extra, head_groups), dim3(kMfmaWaves * kWave), 0, s, mp);
       if (int rc = check_launch(op)) return rc;
     }
     if (stages & ARENO_STAGE_REDUCE) {

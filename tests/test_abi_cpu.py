@@ -47,10 +47,10 @@ def test_version_status_strings_and_workspace_size(lib):
     ws.restype = ctypes.c_size_t
     ws.argtypes = [ctypes.c_int32] * 6
     # two layouts share the workspace: fixed chunks (B * Hq * chunks rows) and the balanced-piece layout
-    # ((2048 static + 1024 claimed units + B) * Hq rows plus the B + 1 prefix sums); the size is the larger of the two
+    # ((768 workgroups * 4 waves + B) * Hq rows plus the B + 1 prefix sums); the size is the larger of the two
     def pieces(b, hq, d):
-        rows = (2048 + 1024 + b) * hq * (d + 2) * 4
-        return (rows + 255) // 256 * 256 + ((b + 1 + 63) // 64 * 64 + 256) * 4
+        rows = (3072 + b) * hq * (d + 2) * 4
+        return (rows + 255) // 256 * 256 + (b + 1 + 63) // 64 * 64 * 4
 
     # B=64, Hq=28, D=128, bs=16, MB=257: 4112 tokens -> 17 chunks of 256
     assert ws(64, 28, 128, 16, 257, 8) == max(64 * 28 * 17 * 130 * 4, pieces(64, 28, 128))
