@@ -28,6 +28,9 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 POOL_TARGET_BYTES = 1.3e9  # rotate over at least this much distinct KV
+# HBM bytes per launch of the split kernel from two rocprofv3 counter runs of this script (FETCH_SIZE, scaled by the
+# factor 2.0 that a copy of known size gives for it, plus WRITE_SIZE); the counter summary is kept under profiles/.
+MEASURED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 315.65e6, "cfg2-qwen7b-int8": 158.30e6}
 
 
 def _clone_pools(w, copies):
@@ -170,6 +173,7 @@ def measure_decode(w, steps, warmup, *, kernel_iters=60):
     assert torch.equal(out2, out), "C-ABI staged run disagrees with the op"
 
     gbps = alg_bytes / (us_split * 1e-6) / 1e9
+    traffic = MEASURED_TRAFFIC_BYTES.get(w.name)
     return {
         "workload": w.name,
         "us_per_step": us_graph,
@@ -179,8 +183,8 @@ def measure_decode(w, steps, warmup, *, kernel_iters=60):
         "algorithmic_bytes": alg_bytes,
         "op_gbps": alg_bytes / (us_graph * 1e-6) / 1e9,
         "roofline": {
-            "bound": "hbm", "kernel": "decode_split_kernel", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": gbps / HBM_PEAK_GBPS, "traffic": None,
+            "bound": "hbm", "kernel": "decode_mfma_kernel", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic,
         },  # fmt: skip
         "pool_copies": copies,
         "parity_max_abs_4rows": parity,
