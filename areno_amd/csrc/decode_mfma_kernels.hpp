@@ -61,6 +61,11 @@ struct MfmaDecodeParams {
   int32_t max_small;     // (gridDim.x - static_wgs) * tok_splits: small units available
   int32_t static_share;  // n/256 of all tiles go to the big units
   int32_t min_unit_tiles;
+  // Fused append: when set, the wave that stages the last tile of a sequence takes the newest token's K / V row
+  // from here ([batch, kv_heads, head_dim], dtype q_dtype) instead of the cache, quantizes it like the cache
+  // writer and stores it (and its scales) into the page, so no separate append launch is needed.
+  const void* k_update;
+  const void* v_update;
 #ifdef ARENO_TRACE
   unsigned long long* trace;  // [wave][16] timestamps, tuning builds only
 #endif
@@ -116,6 +121,64 @@ template <int KIND>
 __device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
   using P = typename KVTraits<KIND>::pair_t;
   return __builtin_bit_cast(uint32_t, make_pair<P>(lo, hi));
+}
+
+// Quantize the 16 consecutive elements a lane holds of a new K or V row (32 raw bytes of 16-bit floats) exactly like
+// the cache writer does (cache_write.hip): the row's abs-max is combined over the LPT lanes that share the row.
+template <int KIND, bool SCALE16, int LPT>
+__device__ __forceinline__ void quantize_row_chunk(const uint4_t (&raw)[2], int in_dtype, uint4_t& codes,
+                                                   typename std::conditional<SCALE16, uint16_t, float>::type& scale_raw) {
+  float x[16];
+  float amax = 0.0f;
+#pragma unroll
+  for (int w = 0; w < 8; ++w) {
+    const uint32_t word = raw[w / 4][w % 4];
+    if (in_dtype == ARENO_DT_BF16) {
+      x[2 * w] = bf16_bits_to_float(word & 0xffffu);
+      x[2 * w + 1] = bf16_bits_to_float(word >> 16);
+    } else {
+      x[2 * w] = f16_bits_to_float(word & 0xffffu);
+      x[2 * w + 1] = f16_bits_to_float(word >> 16);
+    }
+    amax = fmaxf(amax, fmaxf(fabsf(x[2 * w]), fabsf(x[2 * w + 1])));
+  }
+#pragma unroll
+  for (int m = 1; m < LPT; m <<= 1) amax = fmaxf(amax, wave_xor(amax, m));
+  float s;
+  if constexpr (KIND == KV_I8) {
+    const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
+    const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
+    s = static_cast<float>(s16_fixed);
+    if constexpr (SCALE16) {
+      scale_raw = __builtin_bit_cast(uint16_t, s16_fixed);
+    } else {
+      scale_raw = s;
+    }
+  } else {
+    s = amax / 448.0f;
+    if (s == 0.0f) s = 1.0f;
+    if constexpr (SCALE16) {
+      scale_raw = static_cast<uint16_t>(float_to_f16_bits(s));
+    } else {
+      scale_raw = s;
+    }
+  }
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    uint32_t word = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint32_t byte;
+      if constexpr (KIND == KV_I8) {
+        const float code = fminf(fmaxf(rintf(x[4 * w + j] / s), -127.0f), 127.0f);
+        byte = static_cast<uint32_t>(static_cast<int>(code)) & 0xffu;
+      } else {
+        byte = float_to_fp8_byte(fminf(fmaxf(x[4 * w + j] / s, -448.0f), 448.0f));
+      }
+      word |= byte << (8 * j);
+    }
+    codes[w] = word;
+  }
 }
 
 // LDS row that holds tile token t of the V tile: the second half is rotated by 4 rows so that the 8 tokens a
@@ -299,17 +362,45 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
   uint4_t kreg[NLD], vreg[NLD];
   typedef typename std::conditional<SCALE16, uint16_t, float>::type scale_raw_t;
   scale_raw_t ksreg[NLD], vsreg[NLD];
+  // fused append state of the tile in flight
+  const bool fused_append = mp.k_update != nullptr;
+  bool tail_tile = false;  // wave-uniform: the tile in kreg / vreg ends its sequence (holds the newest token)
+  int64_t new_row = 0;     // cache row of the newest token, in the lanes that hold it
+  uint4_t upd_k[2], upd_v[2];
   auto issue_kv_loads = [&]() {
+    tail_tile = fused_append && kv_cur.tok + TK >= kv_cur.end;
+    const int64_t upd_row = static_cast<int64_t>(kv_cur.b) * p.kv_heads + kvh;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      const int t = min(kv_cur.tok + i * TPL + grp, kv_cur.end - 1);
+      const int tt = kv_cur.tok + i * TPL + grp;
+      const int t = min(tt, kv_cur.end - 1);
       const int slot = p.bs_shift >= 0 ? (t & (p.block_size - 1)) : (t % p.block_size);
       const int64_t row = (static_cast<int64_t>(ids[i]) * p.block_size + slot) * p.kv_heads + kvh;
-      kreg[i] = load16(p.k_cache, row * row_bytes + dc * 16);
-      vreg[i] = load16(p.v_cache, row * row_bytes + dc * 16);
+      const char* ka = static_cast<const char*>(p.k_cache) + row * row_bytes + dc * 16;
+      const char* va = static_cast<const char*>(p.v_cache) + row * row_bytes + dc * 16;
+      if (tail_tile && tt >= kv_cur.end - 1) {
+        // the page slot of the newest token (and the clamped rows behind it) is not written yet
+        if (tt == kv_cur.end - 1) new_row = row;
+        if constexpr (!T::kQuant) {
+          ka = static_cast<const char*>(mp.k_update) + upd_row * row_bytes + dc * 16;
+          va = static_cast<const char*>(mp.v_update) + upd_row * row_bytes + dc * 16;
+        }
+      }
+      kreg[i] = *reinterpret_cast<const uint4_t*>(ka);
+      vreg[i] = *reinterpret_cast<const uint4_t*>(va);
       if constexpr (T::kQuant) {
         ksreg[i] = static_cast<const scale_raw_t*>(p.k_scale)[row];
         vsreg[i] = static_cast<const scale_raw_t*>(p.v_scale)[row];
+      }
+    }
+    if constexpr (T::kQuant) {
+      if (tail_tile) {
+        // every lane group fetches the whole new row (16 elements per lane), so each can quantize it on its own
+        const int64_t off = (upd_row * D + dc * EPL) * 2;
+        upd_k[0] = load16(mp.k_update, off);
+        upd_k[1] = load16(mp.k_update, off + 16);
+        upd_v[0] = load16(mp.v_update, off);
+        upd_v[1] = load16(mp.v_update, off + 16);
       }
     }
   };
@@ -455,12 +546,45 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
       for (int x = x0; x < x1; ++x) {
         ARENO_TRACE_POINT();
         // -- stage the fetched tile into LDS (waits for its loads) ---------------------------------------------
-    #pragma unroll
+        if (tail_tile) {
+          // the newest token: quantize (8-bit caches), substitute it for the unwritten slot, store it into the page
+          if constexpr (T::kQuant) {
+            uint4_t qk, qv;
+            scale_raw_t qks, qvs;
+            quantize_row_chunk<KIND, SCALE16, LPT>(upd_k, p.q_dtype, qk, qks);
+            quantize_row_chunk<KIND, SCALE16, LPT>(upd_v, p.q_dtype, qv, qvs);
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+              if (cp_tok + i * TPL + grp >= cp_end - 1) {
+                kreg[i] = qk;
+                vreg[i] = qv;
+                ksreg[i] = qks;
+                vsreg[i] = qvs;
+              }
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < NLD; ++i) {
+            if (cp_tok + i * TPL + grp == cp_end - 1) {
+              char* kc = static_cast<char*>(const_cast<void*>(p.k_cache));
+              char* vc = static_cast<char*>(const_cast<void*>(p.v_cache));
+              *reinterpret_cast<uint4_t*>(kc + new_row * row_bytes + dc * 16) = kreg[i];
+              *reinterpret_cast<uint4_t*>(vc + new_row * row_bytes + dc * 16) = vreg[i];
+              if constexpr (T::kQuant) {
+                if (dc == 0) {
+                  static_cast<scale_raw_t*>(const_cast<void*>(p.k_scale))[new_row] = ksreg[i];
+                  static_cast<scale_raw_t*>(const_cast<void*>(p.v_scale))[new_row] = vsreg[i];
+                }
+              }
+            }
+          }
+        }
+#pragma unroll
         for (int i = 0; i < NLD; ++i) {
           const int t = i * TPL + grp;  // tile-local token
           uint4_t kk = kreg[i], vv = vreg[i];
           if constexpr (KIND == KV_I8) {
-    #pragma unroll
+#pragma unroll
             for (int j = 0; j < 4; ++j) {
               kk[j] ^= kI8Flip;
               vv[j] ^= kI8Flip;
@@ -497,12 +621,12 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
 
         // -- S^T = K . Q^T for the two 16-token groups ------------------------------------------------------------
         float s[2][4];
-    #pragma unroll
+#pragma unroll
         for (int tg = 0; tg < 2; ++tg) {
           float4_t c = {0.0f, 0.0f, 0.0f, 0.0f};
           const char* krow = k_tile + (16 * tg + lr) * RSK + (D / 4) * ES * lk;
           uint32_t kw[NS * WPL];
-    #pragma unroll
+#pragma unroll
           for (int q4 = 0; q4 < NS * WPL / 4; ++q4) {
             const uint4_t r = *reinterpret_cast<const uint4_t*>(krow + 16 * q4);
             kw[4 * q4 + 0] = r[0];
@@ -510,10 +634,10 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
             kw[4 * q4 + 2] = r[2];
             kw[4 * q4 + 3] = r[3];
           }
-    #pragma unroll
+#pragma unroll
           for (int sl = 0; sl < NS; ++sl) c = Ops::mfma(to_operand<KIND>(&kw[sl * WPL]), qop[sl], c);
           const float4_t sc = *reinterpret_cast<const float4_t*>(ksc + 16 * tg + 4 * lk);
-    #pragma unroll
+#pragma unroll
           for (int j = 0; j < 4; ++j) {
             // tokens past the end carry a -inf scale; keep them exactly -inf (0 * -inf would be NaN)
             const float v = c[j] - qbias;
@@ -533,9 +657,9 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
           l_run *= alpha;
           p_sum *= alpha;
-    #pragma unroll
+#pragma unroll
           for (int nb = 0; nb < NB; ++nb) {
-    #pragma unroll
+#pragma unroll
             for (int j = 0; j < 4; ++j) acc[nb][j] *= alpha;
           }
         }
@@ -544,7 +668,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
           const float4_t vs0 = *reinterpret_cast<const float4_t*>(vsc + 4 * lk);
           const float4_t vs1 = *reinterpret_cast<const float4_t*>(vsc + 16 + 4 * lk);
           float pe[8];
-    #pragma unroll
+#pragma unroll
           for (int j = 0; j < 4; ++j) {
             const float e0 = fast_exp2(s[0][j] - m_safe);
             const float e1 = fast_exp2(s[1][j] - m_safe);
@@ -552,7 +676,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
             pe[j] = e0 * vs0[j];
             pe[4 + j] = e1 * vs1[j];
           }
-    #pragma unroll
+#pragma unroll
           for (int j = 0; j < 4; ++j) {
             pw[j] = pack_pair<KIND>(pe[2 * j], pe[2 * j + 1]);
             if constexpr (KIND == KV_I8) {
@@ -564,7 +688,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
         const V8 pop = __builtin_bit_cast(V8, uint4_t{pw[0], pw[1], pw[2], pw[3]});
 
         // -- O^T += V^T . P^T, one MFMA per 16-dim block -------------------------------------------------------------
-    #pragma unroll
+#pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
           uint32_t vw[4];
           if constexpr (ES == 1) {
@@ -578,7 +702,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
           } else {
             // lane i supplies row (i / 4), 4 elements at column 16 nb + 4 (i % 4); two reads of 4 tokens each
             const int r4 = lr >> 2;
-    #pragma unroll
+#pragma unroll
             for (int half = 0; half < 2; ++half) {
               const int tok = 16 * half + 4 * lk + r4;
               char* a = v_tile + v_row_of(tok) * RSV + (16 * nb + 4 * (lr & 3)) * 2;

@@ -372,8 +372,15 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
       default: break;
     }
   }
-  // ---- append (first launch) ------------------------------------------------------------------------------------
-  if (k_update != nullptr && (stages & ARENO_STAGE_APPEND)) {
+  // ---- append: folded into the matrix-core split kernel when it can take the new rows as they are, else a launch of
+  // its own in front ------------------------------------------------------------------------------------------------
+  static const bool allow_fused_append = env_int("ARENO_FUSED_APPEND", 1) != 0;
+  const bool fuse_append =
+      mfma != nullptr && allow_fused_append && k_update != nullptr && v_update != nullptr &&
+      (stages & ARENO_STAGE_APPEND) && (stages & ARENO_STAGE_SPLIT) &&
+      (is_quantized(cache->cache_dtype) || q_dtype == cache->cache_dtype) &&
+      reinterpret_cast<uintptr_t>(k_update) % 16 == 0 && reinterpret_cast<uintptr_t>(v_update) % 16 == 0;
+  if (k_update != nullptr && (stages & ARENO_STAGE_APPEND) && !fuse_append) {
     if (int rc = areno_hip_cache_write_decode(cache, k_update, v_update, q_dtype, batch, block_table, max_blocks,
                                               cache_seqlens, stream))
       return rc;
@@ -400,6 +407,8 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
     mp.max_small = extra * mp.tok_splits;
     mp.static_share = static_share;
     mp.min_unit_tiles = unit_tiles;
+    mp.k_update = fuse_append ? k_update : nullptr;
+    mp.v_update = fuse_append ? v_update : nullptr;
 #ifdef ARENO_TRACE
     mp.trace = getenv("ARENO_TRACE_BUF") ? reinterpret_cast<unsigned long long*>(strtoull(getenv("ARENO_TRACE_BUF"), nullptr, 0)) : nullptr;
 #endif

@@ -293,7 +293,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(Prefil
 
     // a wave whose rows all sit before this tile's first key has nothing to do here (causal); it still takes
     // part in the barriers
-    const int wave_qmax = ctx + tok0 + min(tok_cnt, ((wave + 1) * kRowsPerWave - 1 >> p.group_shift) + 1) - 1;
+    const int wave_qmax = ctx + tok0 + min(tok_cnt, (((wave + 1) * kRowsPerWave - 1) >> p.group_shift) + 1) - 1;
     if (k0 <= wave_qmax && wave * kRowsPerWave < (tok_cnt << p.group_shift)) {
       // -- S^T = K . Q^T ------------------------------------------------------------------------------------------
       float s[kRowTiles][2][4];
