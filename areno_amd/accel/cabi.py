@@ -64,8 +64,10 @@ def lib() -> ctypes.CDLL:
         decode_args = [_P, _P, _P, _P, _P, _I32, _I32, _I32, _P, _I32, _P, _I32, _I32, _F, _P, _SZ]
         handle.areno_hip_paged_decode.argtypes = decode_args + [_P]
         handle.areno_hip_paged_decode_stages.argtypes = decode_args + [_I32, _P]
-        handle.areno_hip_varlen_attention.argtypes = [_P, _P, _P, _P, _I32, _I64, _I32, _I32, _I32, _P, _I32, _I32, _F, _P]
-        handle.areno_hip_paged_varlen_prefill.argtypes = [_P, _P, _P, _I32, _I64, _I32, _I32, _P, _I32, _P, _P, _I32, _F, _P]
+        handle.areno_hip_varlen_attention.argtypes = [_P, _P, _P, _P, _I32, _I64, _I32, _I32, _I32, _P, _I32, _I32, _F, _P, _SZ, _P]  # fmt: skip
+        handle.areno_hip_paged_varlen_prefill.argtypes = [_P, _P, _P, _I32, _I64, _I32, _I32, _P, _I32, _P, _P, _I32, _F, _P, _SZ, _P]  # fmt: skip
+        handle.areno_hip_prefill_workspace_bytes.restype = _SZ
+        handle.areno_hip_prefill_workspace_bytes.argtypes = [_I32, _I32]
         _LIB = handle
     return _LIB
 

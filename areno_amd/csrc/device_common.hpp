@@ -88,6 +88,54 @@ __device__ __forceinline__ float wave_max(float x) {
   return x;
 }
 
+// Reductions over the four 16-lane rows of a wave (lanes l, l + 16, l + 32, l + 48), result in all four: the MFMA
+// C layout keeps one matrix column in those lanes.  v_permlane16_swap / v_permlane32_swap exchange odd and even rows
+// (then upper and lower half) of two registers in the vector ALU, without the LDS round trip of ds_bpermute.  Inline
+// asm because the compiler's own lowering of the matching builtins merges the two results; the s_nop covers the
+// wait states the swap needs after a VALU write of its operands.
+__device__ __forceinline__ void swap_rows16(uint32_t& a, uint32_t& b) {
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap_rows32(uint32_t& a, uint32_t& b) {
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+
+// max without the canonicalising self-max the compiler puts in front of every fmaxf operand whose origin it cannot
+// see (IEEE mode); the hardware instruction already returns the other operand for a NaN input.
+__device__ __forceinline__ float max_f32(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float max3_f32(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+// x *= f in the register x lives in: as a plain multiply under a rarely taken branch the compiler copies whole
+// accumulator sets around the branch instead.
+__device__ __forceinline__ void scale_in_place(float& x, float f) { asm("v_mul_f32 %0, %1, %0" : "+v"(x) : "v"(f)); }
+
+__device__ __forceinline__ float rows_max(float x) {
+  uint32_t a = __builtin_bit_cast(uint32_t, x), b = a;
+  swap_rows16(a, b);
+  const float y = max_f32(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+  a = __builtin_bit_cast(uint32_t, y);
+  b = a;
+  swap_rows32(a, b);
+  return max_f32(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+}
+
+__device__ __forceinline__ float rows_sum(float x) {
+  uint32_t a = __builtin_bit_cast(uint32_t, x), b = a;
+  swap_rows16(a, b);
+  const float y = __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+  a = __builtin_bit_cast(uint32_t, y);
+  b = a;
+  swap_rows32(a, b);
+  return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 constexpr float kLog2e = 1.4426950408889634f;

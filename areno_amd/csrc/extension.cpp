@@ -171,11 +171,14 @@ at::Tensor varlen_forward(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor c
   TORCH_CHECK(cu_seqlens.size(0) >= 2, op, " cu_seqlens must contain at least one sequence");
   const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(q));
   auto out = at::empty_like(q);
+  const size_t ws_bytes =
+      areno_hip_prefill_workspace_bytes(static_cast<int32_t>(k.size(1)), static_cast<int32_t>(q.size(2)));
+  auto workspace = at::empty({static_cast<int64_t>(ws_bytes)}, q.options().dtype(at::kByte));
   const int status = areno_hip_varlen_attention(
       q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dtype_code(q, op, "q"), q.size(0),
       static_cast<int32_t>(q.size(1)), static_cast<int32_t>(k.size(1)), static_cast<int32_t>(q.size(2)),
       cu_seqlens.data_ptr<int32_t>(), static_cast<int32_t>(cu_seqlens.size(0) - 1), static_cast<int32_t>(window_left),
-      static_cast<float>(softmax_scale), current_stream(q));
+      static_cast<float>(softmax_scale), workspace.data_ptr(), ws_bytes, current_stream(q));
   check_status(status, op);
   return out;
 }
@@ -235,11 +238,14 @@ at::Tensor paged_varlen_forward(at::Tensor q, at::Tensor k_cache, at::Tensor v_c
   TORCH_CHECK(q.size(1) % k_cache.size(2) == 0, op, " q heads must be divisible by kv heads");
   const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(q));
   auto out = at::empty_like(q);
+  const size_t ws_bytes = areno_hip_prefill_workspace_bytes(cache.kv_heads, cache.head_dim);
+  auto workspace = at::empty({static_cast<int64_t>(ws_bytes)}, q.options().dtype(at::kByte));
   const int status = areno_hip_paged_varlen_prefill(
       &cache, q.data_ptr(), out.data_ptr(), dtype_code(q, op, "q"), q.size(0), static_cast<int32_t>(q.size(1)),
       static_cast<int32_t>(context_lens.size(0)), block_table.data_ptr<int32_t>(),
       static_cast<int32_t>(block_table.size(1)), cu_seqlens_q.data_ptr<int32_t>(), context_lens.data_ptr<int32_t>(),
-      static_cast<int32_t>(window_left), static_cast<float>(softmax_scale), current_stream(q));
+      static_cast<int32_t>(window_left), static_cast<float>(softmax_scale), workspace.data_ptr(), ws_bytes,
+      current_stream(q));
   check_status(status, op);
   return out;
 }

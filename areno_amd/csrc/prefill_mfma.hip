@@ -1,37 +1,55 @@
 // Causal varlen prefill over paged (optionally quantized) KV on the matrix cores (gfx950).
 //
-// Workgroup = 4 wave64 = one (sequence, kv head, block of query tokens).  The G query heads of the kv head
-// are folded into the query-row axis: row r of the block is (token r / GP, head r % GP) with GP = G rounded up
-// to a power of two, so one 16-row MFMA tile holds 16 / GP tokens of all heads and K/V are read once for the
-// whole group (GQA without expanding KV, as areno/accel/csrc/attention.cu:170-171 does per row).
-// Each wave owns 32 query rows (two 16-row tiles); the workgroup walks the visible keys in 32-token tiles:
-//   * all 256 threads fetch the next K/V tile with 16-byte coalesced loads (block ids resolved one tile ahead)
-//     while the current tile is computed, then store it into a shared LDS tile (padded rows, conflict free);
-//   * S^T[key][row] = K . Q^T   : A = K rows from LDS, B = Q^T in registers; C has row = lane % 16, 4 keys per lane;
-//   * causal / window / length mask, per-key K scale, online softmax in the log2 domain (per lane = per row);
+// Work item = (sequence, kv head, block of query tokens).  The G query heads of the kv head are folded into the
+// query-row axis: row r of the block is (token r / GP, head r % GP) with GP = G rounded up to a power of two, so one
+// 16-row MFMA tile holds 16 / GP tokens of all heads and K/V are read once for the whole group (GQA without
+// expanding KV, as areno/accel/csrc/attention.cu:170-171 does per row).  A block is 128 rows: each of the 4 waves
+// owns 32 (two 16-row tiles).
+//
+// Balance: an item costs one "tile step" per 32-key tile it may see, and items differ by orders of magnitude (a
+// query block on a 16k context next to one on an empty context).  Every workgroup computes the prefix sum of tile
+// steps over the sequences in LDS and takes an equal share of the global tile-step range of its kv head (a "unit"),
+// whatever the length distribution.  A unit is a run of segments, each a range of key tiles of one item:
+//   * an item that lies inside one unit is finished there and written to `out`;
+//   * an item cut by a unit border leaves un-normalised partials (running max, sum, accumulator) in the workspace
+//     -- slot 2u for the first item of unit u, slot 2u + 1 for its last -- and prefill_merge_kernel combines them.
+//
+// One segment, per 32-key tile t (all four waves share the K/V tiles in LDS):
+//   * the 256 threads fetch K three tiles and V two tiles ahead with 16-byte coalesced loads (block ids one more
+//     tile ahead) and publish them into double-buffered LDS tiles one iteration before their first use, so one
+//     barrier per tile is enough (padded rows, conflict free);
+//   * S^T[key][row] = K . Q^T of tile t + 1 is issued before the softmax of tile t, so the matrix cores have
+//     independent work while the vector ALU runs the softmax: A = K rows from LDS, B = Q^T in registers; C has
+//     row = lane % 16, 4 keys per lane;
+//   * per-key K scale, causal / window mask only on tiles that cross a mask edge, online softmax in the log2
+//     domain (per lane = per row);
 //   * O^T[dim][row] += V^T . P^T : A = V^T through the LDS transpose reads, B = P^T (= the C layout of S^T).
 // The dequantisation of int8 / fp8 codes and the layouts are the ones of the decode kernel
 // (decode_mfma_kernels.hpp).  Semantics: _reference_attention with query_start = context_lens[s]
 // (areno/accel/attention.py:25-41 in the reference); with context 0 it is the reference's varlen kernel
 // (areno/accel/csrc/attention.cu:145-242).
 
+#include <cstdlib>
+
 #include "decode_mfma_kernels.hpp"
 
 namespace areno {
 
+size_t prefill_mfma_workspace_bytes(int32_t kv_heads, int32_t head_dim);
 int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out, int32_t q_dtype, int64_t tokens,
                         int32_t q_heads, int32_t num_seqs, const int32_t* block_table, int32_t max_blocks,
                         const int32_t* cu_seqlens_q, const int32_t* context_lens, int32_t window_left,
-                        float softmax_scale, void* stream);
+                        float softmax_scale, void* workspace, size_t workspace_bytes, void* stream);
 
 namespace {
 
 constexpr int kPrefillThreads = 256;
 constexpr int kPrefillWaves = 4;
-constexpr int kRowTiles = 2;                          // 16-row MFMA tiles per wave
-constexpr int kRowsPerWave = 16 * kRowTiles;          // 32
-constexpr int kRowsPerWg = kRowsPerWave * kPrefillWaves;  // 128
+constexpr int kMaxRowTiles = 4;                                       // 16-row MFMA tiles per wave, at most
+constexpr int kMaxRowsPerWg = 16 * kMaxRowTiles * kPrefillWaves;      // 256
 constexpr int kMaxPrefillSeqs = 1024;
+constexpr int kPrefillTargetWgs = 512;  // two resident workgroups on each of the 256 CUs
+constexpr int kMaxPrefillUnits = 512;   // per kv head
 
 struct PrefillParams {
   const void* q;
@@ -43,209 +61,212 @@ struct PrefillParams {
   const int32_t* block_table;
   const int32_t* cu_seqlens_q;
   const int32_t* context_lens;
+  float* part_ml;   // [2 * units][kv_heads][128 rows][2]
+  float* part_acc;  // [2 * units][kv_heads][128 rows][head_dim]
   int32_t num_seqs;
   int32_t q_heads;
   int32_t kv_heads;
-  int32_t group;         // q heads per kv head
-  int32_t group_pad;     // rounded up to a power of two (<= 16)
-  int32_t group_shift;   // log2(group_pad)
+  int32_t head_dim;
+  int32_t group;        // q heads per kv head
+  int32_t group_pad;    // rounded up to a power of two (<= 16)
+  int32_t group_shift;  // log2(group_pad)
   int32_t block_size;
   int32_t bs_shift;
   int32_t max_blocks;
   int32_t window_left;
   int32_t q_dtype;
+  int32_t units;        // per kv head
+  int32_t rows_per_wg;  // query rows of one item: 64 per 16-row tile a wave owns
   float scale_log2e;
 };
 
-template <int KIND, int D, bool SCALE16>
-__global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(PrefillParams p) {
+// Key tiles query block j (tokens [j * tq, ...)) of a sequence may see: [tile_lo, tile_hi].
+struct BlockTiles {
+  int tok0, cnt, tile_lo, tile_hi;
+  __device__ int count() const { return tile_hi - tile_lo + 1; }
+};
+
+__device__ __forceinline__ BlockTiles block_tiles(int n_new, int ctx, int j, int tq, int window_left) {
+  BlockTiles b;
+  b.tok0 = j * tq;
+  b.cnt = min(tq, n_new - b.tok0);
+  const int key_hi = ctx + b.tok0 + b.cnt - 1;
+  const int key_lo = window_left >= 0 ? max(0, ctx + b.tok0 - window_left) : 0;
+  b.tile_lo = key_lo / kTileTokens;
+  b.tile_hi = key_hi / kTileTokens;
+  return b;
+}
+
+// Exclusive prefix sum of tile steps per sequence into s_cum[0 .. num_seqs] (all 256 threads take part).
+__device__ __forceinline__ void prefix_tile_steps(const PrefillParams& p, int tq, int* s_cum, int* s_wave_tot) {
+  constexpr int SPT = kMaxPrefillSeqs / kPrefillThreads;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  int steps[SPT];
+  int local = 0;
+#pragma unroll
+  for (int i = 0; i < SPT; ++i) {
+    const int s = SPT * tid + i;
+    steps[i] = 0;
+    if (s < p.num_seqs) {
+      const int n_new = p.cu_seqlens_q[s + 1] - p.cu_seqlens_q[s];
+      const int ctx = p.context_lens != nullptr ? p.context_lens[s] : 0;
+      for (int j = 0; j * tq < n_new; ++j) steps[i] += block_tiles(n_new, ctx, j, tq, p.window_left).count();
+    }
+    local += steps[i];
+  }
+  int incl = local;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int v = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += v;
+  }
+  if (lane == kWave - 1) s_wave_tot[wave] = incl;
+  __syncthreads();
+  int excl = incl - local;
+  for (int w2 = 0; w2 < wave; ++w2) excl += s_wave_tot[w2];
+#pragma unroll
+  for (int i = 0; i < SPT; ++i) {
+    const int s = SPT * tid + i;
+    if (s <= p.num_seqs) s_cum[s] = excl;
+    excl += steps[i];
+  }
+  __syncthreads();
+}
+
+// Where global tile step x lies: sequence, query block, key tile.
+struct StepPos {
+  int seq, j, tile;
+  int n_new, ctx;
+  int item_x0;  // global step of the item's first tile
+};
+
+__device__ __forceinline__ StepPos locate_step(const PrefillParams& p, const int* s_cum, int tq, int x) {
+  StepPos r;
+  int lo = 0, hi = p.num_seqs;
+  while (lo + 1 < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (s_cum[mid] <= x) {
+      lo = mid;
+    } else {
+      hi = mid;
+    }
+  }
+  r.seq = lo;
+  r.n_new = p.cu_seqlens_q[lo + 1] - p.cu_seqlens_q[lo];
+  r.ctx = p.context_lens != nullptr ? p.context_lens[lo] : 0;
+  int off = x - s_cum[lo];
+  r.item_x0 = s_cum[lo];
+  r.j = 0;
+  for (;;) {
+    const BlockTiles b = block_tiles(r.n_new, r.ctx, r.j, tq, p.window_left);
+    if (off < b.count()) {
+      r.tile = b.tile_lo + off;
+      break;
+    }
+    off -= b.count();
+    r.item_x0 += b.count();
+    ++r.j;
+    if (r.j * tq >= r.n_new) {  // x past the sequence's last step: callers never ask for it
+      r.j = 0;
+      r.tile = 0;
+      break;
+    }
+  }
+  return r;
+}
+
+__device__ __forceinline__ int unit_start_step(int total, int u, int units) {
+  return static_cast<int>(static_cast<long long>(total) * u / units);
+}
+
+// 16 codes of an 8-bit cache row (one 16-byte chunk) -> 16 fp16 values times the row's scale, as two 16-byte groups.
+// int8: (code ^ 0x80) under the exponent byte 0x64 is fp16 1152 + code, exactly; the packed subtract and multiply
+// that follow are exact resp. correctly rounded.  fp8: the hardware conversion is exact.
+template <int KIND>
+__device__ __forceinline__ void dequant_chunk(uint4_t codes, float scale, uint4_t& lo, uint4_t& hi) {
+  const _Float16 sh = static_cast<_Float16>(scale);
+  const half2_t s2 = {sh, sh};
+  uint32_t out[8];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const uint32_t word = codes[w];
+    half2_t a, c;
+    if constexpr (KIND == KV_I8) {
+      const uint32_t u = word ^ kI8Flip;
+      const half2_t offs = {static_cast<_Float16>(kI8Offset), static_cast<_Float16>(kI8Offset)};
+      a = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(kF16Filler, u, 0x04010400u)) - offs;
+      c = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(kF16Filler, u, 0x04030402u)) - offs;
+    } else {
+      a = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(word, 1.0f, false));
+      c = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(word, 1.0f, true));
+    }
+    out[2 * w] = __builtin_bit_cast(uint32_t, a * s2);
+    out[2 * w + 1] = __builtin_bit_cast(uint32_t, c * s2);
+  }
+  lo = uint4_t{out[0], out[1], out[2], out[3]};
+  hi = uint4_t{out[4], out[5], out[6], out[7]};
+}
+
+template <int KIND, int D, bool SCALE16, int RT>
+__global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma_kernel(PrefillParams p) {
+  constexpr int kRowTiles = RT;
+  constexpr int kRowsPerWave = 16 * RT;
+  constexpr int kRowsPerWg = kRowsPerWave * kPrefillWaves;
   using T = KVTraits<KIND>;
-  using Ops = MfmaOps<KIND>;
+  // The tiles in LDS are 16-bit whatever the cache holds: 8-bit codes are dequantized (times the per-token scale)
+  // once, by the thread that stages them, instead of by every wave that reads them.
+  constexpr int OPK = KIND == KV_BF16 ? KV_BF16 : KV_F16;
+  using Ops = MfmaOps<OPK>;
   using V8 = typename Ops::vec8;
-  using Pair = typename T::pair_t;
-  constexpr int ES = T::kBytes;
+  using Pair = typename KVTraits<OPK>::pair_t;
+  constexpr int ES = T::kBytes;  // bytes per element in the cache
   constexpr int EPL = 16 / ES;
-  constexpr int LPT = D / EPL;  // 16-byte chunks per token row
+  constexpr int LPT = D / EPL;  // 16-byte chunks per cached token row
   constexpr int TK = kTileTokens;
-  constexpr int CHUNKS = TK * LPT;                   // 16-byte chunks per K (or V) tile
+  constexpr int CHUNKS = TK * LPT;                                       // 16-byte chunks per cached K (or V) tile
   constexpr int NLD = (CHUNKS + kPrefillThreads - 1) / kPrefillThreads;  // loads per thread per tensor per tile
-  constexpr int RSK = D * ES + 16;
-  constexpr int RSV = ES == 1 ? D + 16 : 2 * D + 32;
+  constexpr int RSK = D * 2 + 16;
+  constexpr int RSV = 2 * D + 32;
   constexpr int NS = D / 32;
   constexpr int NB = D / 16;
-  constexpr int WPL = 8 * ES / 4;
-  constexpr float kPScale = T::kQuant ? 256.0f : 1.0f;
   typedef typename std::conditional<SCALE16, uint16_t, float>::type scale_raw_t;
 
-  __shared__ __attribute__((aligned(16))) char s_k[TK * RSK];
-  __shared__ __attribute__((aligned(16))) char s_v[TK * RSV];
-  __shared__ float s_ksc[TK];
-  __shared__ float s_vsc[TK];
+  __shared__ __attribute__((aligned(16))) char s_k[2][TK * RSK];
+  __shared__ __attribute__((aligned(16))) char s_v[2][TK * RSV];
   __shared__ int s_cum[kMaxPrefillSeqs + 1];
   __shared__ int s_wave_tot[kPrefillWaves];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lets the tile-level decisions stay scalar
   const int lr = lane & 15;
   const int lk = lane >> 4;
   const int kvh = blockIdx.y;
-  const int tokens_per_wg = kRowsPerWg >> p.group_shift;
+  const int unit = blockIdx.x;
+  const int tq = kRowsPerWg >> p.group_shift;  // query tokens per item
 
-  // ---- which (sequence, query block) is this workgroup?  prefix sum of blocks per sequence ---------------
-  {
-    constexpr int SPT = kMaxPrefillSeqs / kPrefillThreads;
-    int nb[SPT];
-    int local = 0;
-#pragma unroll
-    for (int j = 0; j < SPT; ++j) {
-      const int s = SPT * tid + j;
-      nb[j] = 0;
-      if (s < p.num_seqs) nb[j] = (p.cu_seqlens_q[s + 1] - p.cu_seqlens_q[s] + tokens_per_wg - 1) / tokens_per_wg;
-      local += nb[j];
-    }
-    int incl = local;
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-      const int v = __shfl_up(incl, off, kWave);
-      if (lane >= off) incl += v;
-    }
-    if (lane == kWave - 1) s_wave_tot[wave] = incl;
-    __syncthreads();
-    int excl = incl - local;
-    for (int w2 = 0; w2 < wave; ++w2) excl += s_wave_tot[w2];
-#pragma unroll
-    for (int j = 0; j < SPT; ++j) {
-      const int s = SPT * tid + j;
-      if (s <= p.num_seqs) s_cum[s] = excl;
-      excl += nb[j];
-    }
-    __syncthreads();
-  }
-  // heavy blocks (late query tokens see the most keys) are started first: walk the block list backwards
-  const int item = s_cum[p.num_seqs] - 1 - static_cast<int>(blockIdx.x);
-  if (item < 0) return;
-  int seq;
-  {
-    int lo = 0, hi = p.num_seqs;
-    while (lo + 1 < hi) {
-      const int mid = (lo + hi) >> 1;
-      if (s_cum[mid] <= item) {
-        lo = mid;
-      } else {
-        hi = mid;
-      }
-    }
-    seq = lo;
-  }
-  const int q_begin = p.cu_seqlens_q[seq];
-  const int n_new = p.cu_seqlens_q[seq + 1] - q_begin;
-  const int ctx = p.context_lens != nullptr ? p.context_lens[seq] : 0;
-  const int tok0 = (item - s_cum[seq]) * tokens_per_wg;       // first new token of this block
-  const int tok_cnt = min(tokens_per_wg, n_new - tok0);
+  prefix_tile_steps(p, tq, s_cum, s_wave_tot);
+  const int total = s_cum[p.num_seqs];
+  const int x_begin = unit_start_step(total, unit, p.units);
+  const int x_end = unit_start_step(total, unit + 1, p.units);
+  if (x_begin >= x_end) return;  // same for the whole workgroup
 
-  // keys this block may see: [key_lo, key_hi]
-  const int key_hi = ctx + tok0 + tok_cnt - 1;
-  int key_lo = 0;
-  if (p.window_left >= 0) key_lo = max(0, ctx + tok0 - p.window_left);
-  const int tile_lo = key_lo / TK;
-  const int tile_hi = key_hi / TK;
-
-  // ---- this lane's query rows ---------------------------------------------------------------------------------
-  // row R = wave * 32 + 16 * nq + lr  ->  token tok0 + (R >> group_shift), head R & (group_pad - 1)
-  int q_pos[kRowTiles];       // absolute position of the row's query, or -1 for a padding row
-  int64_t row_elem[kRowTiles];  // element offset of the row in q / out
-  V8 qop[kRowTiles][NS];
-  float qbias[kRowTiles];
-  const bool q_is_operand_type = (KIND == KV_BF16 && p.q_dtype == ARENO_DT_BF16) ||
-                                 (KIND != KV_BF16 && p.q_dtype == ARENO_DT_F16);
-#pragma unroll
-  for (int nq = 0; nq < kRowTiles; ++nq) {
-    const int r = wave * kRowsPerWave + 16 * nq + lr;
-    const int t = r >> p.group_shift;
-    const int hh = r & (p.group_pad - 1);
-    const bool live = t < tok_cnt && hh < p.group;
-    q_pos[nq] = live ? ctx + tok0 + t : -1;
-    row_elem[nq] = (static_cast<int64_t>(q_begin + tok0 + t) * p.q_heads + kvh * p.group + hh) * D;
-    float qsum = 0.0f;
-#pragma unroll
-    for (int sl = 0; sl < NS; ++sl) {
-      uint4_t w = {0u, 0u, 0u, 0u};
-      if (live) w = load16(p.q, (row_elem[nq] + (D / 4) * lk + 8 * sl) * 2);
-      if (!q_is_operand_type) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float a, c;
-          if constexpr (KIND == KV_BF16) {
-            a = f16_bits_to_float(w[j] & 0xffffu);
-            c = f16_bits_to_float(w[j] >> 16);
-          } else {
-            a = bf16_bits_to_float(w[j] & 0xffffu);
-            c = bf16_bits_to_float(w[j] >> 16);
-          }
-          w[j] = __builtin_bit_cast(uint32_t, make_pair<Pair>(a, c));
-        }
-      }
-      if constexpr (KIND == KV_I8) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const Pair pr = __builtin_bit_cast(Pair, static_cast<uint32_t>(w[j]));
-          qsum += static_cast<float>(pr.x) + static_cast<float>(pr.y);
-        }
-      }
-      qop[nq][sl] = __builtin_bit_cast(V8, w);
-    }
-    qbias[nq] = 0.0f;
-    if constexpr (KIND == KV_I8) {
-      qsum += wave_xor(qsum, 16);
-      qsum += wave_xor(qsum, 32);
-      qbias[nq] = kI8Offset * qsum;
-    }
-  }
-
-  float4_t acc[kRowTiles][NB];
-  float m_run[kRowTiles], l_run[kRowTiles], p_sum[kRowTiles];
-#pragma unroll
-  for (int nq = 0; nq < kRowTiles; ++nq) {
-    m_run[nq] = kNegInf;
-    l_run[nq] = 0.0f;
-    p_sum[nq] = 0.0f;
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) acc[nq][nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-  }
-
-  // ---- cooperative tile fetch: thread tid owns chunks tid + 256 * i --------------------------------------------
-  const int32_t* table_row = p.block_table + static_cast<int64_t>(seq) * p.max_blocks;
+  const bool q_is_operand_type = (OPK == KV_BF16 && p.q_dtype == ARENO_DT_BF16) ||
+                                 (OPK == KV_F16 && p.q_dtype == ARENO_DT_F16);
+  const bool packed = p.block_table == nullptr;  // K/V are (tokens, kv_heads, D): key t of a sequence is row q_begin + t
   constexpr int64_t row_bytes = static_cast<int64_t>(D) * ES;
-  int ids[NLD];
-  uint4_t kreg[NLD], vreg[NLD];
-  scale_raw_t ksreg[NLD], vsreg[NLD];
-  auto chunk_live = [&](int i) { return tid + kPrefillThreads * i < CHUNKS; };
-  auto chunk_token = [&](int i) { return min(tid + kPrefillThreads * i, CHUNKS - 1) / LPT; };
-  auto chunk_col = [&](int i) { return min(tid + kPrefillThreads * i, CHUNKS - 1) % LPT; };
-  const bool packed = p.block_table == nullptr;  // K/V are (tokens, kv_heads, D): key t of the sequence is row q_begin + t
-  auto issue_id_loads = [&](int tile) {
+  // this thread's chunks of a tile: token and 16-byte column, fixed for the whole kernel
+  int chunk_tok[NLD], chunk_col[NLD];
+  bool chunk_live[NLD];
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const int t = min(tile * TK + chunk_token(i), key_hi);
-      ids[i] = packed ? 0 : table_row[p.bs_shift >= 0 ? (t >> p.bs_shift) : (t / p.block_size)];
-    }
-  };
-  auto issue_kv_loads = [&](int tile) {
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const int t = min(tile * TK + chunk_token(i), key_hi);
-      const int slot = p.bs_shift >= 0 ? (t & (p.block_size - 1)) : (t % p.block_size);
-      const int64_t row = packed ? (static_cast<int64_t>(q_begin) + t) * p.kv_heads + kvh
-                                 : (static_cast<int64_t>(ids[i]) * p.block_size + slot) * p.kv_heads + kvh;
-      kreg[i] = load16(p.k_cache, row * row_bytes + chunk_col(i) * 16);
-      vreg[i] = load16(p.v_cache, row * row_bytes + chunk_col(i) * 16);
-      if constexpr (T::kQuant) {
-        ksreg[i] = static_cast<const scale_raw_t*>(p.k_scale)[row];
-        vsreg[i] = static_cast<const scale_raw_t*>(p.v_scale)[row];
-      }
-    }
-  };
+  for (int i = 0; i < NLD; ++i) {
+    const int c = tid + kPrefillThreads * i;
+    chunk_live[i] = c < CHUNKS;
+    chunk_tok[i] = min(c, CHUNKS - 1) / LPT;
+    chunk_col[i] = min(c, CHUNKS - 1) % LPT;
+  }
   auto scale_value = [](scale_raw_t raw) -> float {
     if constexpr (SCALE16) {
       return static_cast<float>(__builtin_bit_cast(_Float16, raw));
@@ -254,201 +275,408 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(Prefil
     }
   };
 
-  issue_id_loads(tile_lo);
-  issue_kv_loads(tile_lo);
-  if (tile_lo < tile_hi) issue_id_loads(tile_lo + 1);
+  StepPos pos = locate_step(p, s_cum, tq, x_begin);
+  int x = x_begin;
+  bool first_item = true;
+  while (x < x_end) {
+    // ---- one segment: key tiles [ta, tb] of item (pos.seq, pos.j) ------------------------------------------------
+    const BlockTiles item = block_tiles(pos.n_new, pos.ctx, pos.j, tq, p.window_left);
+    const int ta = pos.tile;
+    const int tb = min(item.tile_hi, ta + (x_end - x) - 1);
+    const bool whole = ta == item.tile_lo && tb == item.tile_hi;
+    const int q_begin = p.cu_seqlens_q[pos.seq];
+    const int ctx = pos.ctx;
+    const int tok0 = item.tok0;
+    const int tok_cnt = item.cnt;
+    const int key_hi = ctx + tok0 + tok_cnt - 1;
+    const int32_t* table_row = packed ? nullptr : p.block_table + static_cast<int64_t>(pos.seq) * p.max_blocks;
 
-  for (int tile = tile_lo; tile <= tile_hi; ++tile) {
-    const int k0 = tile * TK;
-    // -- publish the fetched tile ------------------------------------------------------------------------------
+    // ---- this lane's query rows: row R = wave * 16 RT + 16 * nq + lr -> token tok0 + (R >> group_shift), head
+    // R & (group_pad - 1) --------------------------------------------------------------------------------------------
+    int q_pos[kRowTiles];         // absolute position of the row's query, or -1 for a padding row
+    int64_t row_elem[kRowTiles];  // element offset of the row in q / out
+    V8 qop[kRowTiles][NS];
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const int t = chunk_token(i);
-      uint4_t kk = kreg[i], vv = vreg[i];
-      if constexpr (KIND == KV_I8) {
+    for (int nq = 0; nq < kRowTiles; ++nq) {
+      const int r = wave * kRowsPerWave + 16 * nq + lr;
+      const int t = r >> p.group_shift;
+      const int hh = r & (p.group_pad - 1);
+      const bool live = t < tok_cnt && hh < p.group;
+      q_pos[nq] = live ? ctx + tok0 + t : -1;
+      row_elem[nq] = (static_cast<int64_t>(q_begin + tok0 + t) * p.q_heads + kvh * p.group + hh) * D;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          kk[j] ^= kI8Flip;
-          vv[j] ^= kI8Flip;
-        }
-      }
-      if (!chunk_live(i)) continue;
-      *reinterpret_cast<uint4_t*>(s_k + t * RSK + chunk_col(i) * 16) = kk;
-      *reinterpret_cast<uint4_t*>(s_v + v_row_of(t) * RSV + chunk_col(i) * 16) = vv;
-      if (chunk_col(i) == 0) {
-        if constexpr (T::kQuant) {
-          s_ksc[t] = scale_value(ksreg[i]) * p.scale_log2e;
-          s_vsc[t] = scale_value(vsreg[i]) * kPScale;
-        } else {
-          s_ksc[t] = p.scale_log2e;
-          s_vsc[t] = kPScale;
-        }
-      }
-    }
-    __syncthreads();
-    if (tile < tile_hi) {
-      issue_kv_loads(tile + 1);
-      if (tile + 1 < tile_hi) issue_id_loads(tile + 2);
-    }
-
-    // a wave whose rows all sit before this tile's first key has nothing to do here (causal); it still takes
-    // part in the barriers
-    const int wave_qmax = ctx + tok0 + min(tok_cnt, (((wave + 1) * kRowsPerWave - 1) >> p.group_shift) + 1) - 1;
-    if (k0 <= wave_qmax && wave * kRowsPerWave < (tok_cnt << p.group_shift)) {
-      // -- S^T = K . Q^T ------------------------------------------------------------------------------------------
-      float s[kRowTiles][2][4];
-#pragma unroll
-      for (int tg = 0; tg < 2; ++tg) {
-        const char* krow = s_k + (16 * tg + lr) * RSK + (D / 4) * ES * lk;
-        uint32_t kw[NS * WPL];
-#pragma unroll
-        for (int q4 = 0; q4 < NS * WPL / 4; ++q4) {
-          const uint4_t r = *reinterpret_cast<const uint4_t*>(krow + 16 * q4);
-          kw[4 * q4 + 0] = r[0];
-          kw[4 * q4 + 1] = r[1];
-          kw[4 * q4 + 2] = r[2];
-          kw[4 * q4 + 3] = r[3];
-        }
-        V8 kop[NS];
-#pragma unroll
-        for (int sl = 0; sl < NS; ++sl) kop[sl] = to_operand<KIND>(&kw[sl * WPL]);
-        const float4_t sc = *reinterpret_cast<const float4_t*>(s_ksc + 16 * tg + 4 * lk);
-#pragma unroll
-        for (int nq = 0; nq < kRowTiles; ++nq) {
-          float4_t c = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-          for (int sl = 0; sl < NS; ++sl) c = Ops::mfma(kop[sl], qop[nq][sl], c);
+      for (int sl = 0; sl < NS; ++sl) {
+        uint4_t w = {0u, 0u, 0u, 0u};
+        if (live) w = load16(p.q, (row_elem[nq] + (D / 4) * lk + 8 * sl) * 2);
+        if (!q_is_operand_type) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const int kpos = k0 + 16 * tg + 4 * lk + j;
-            bool ok = kpos <= q_pos[nq];
-            if (p.window_left >= 0) ok = ok && kpos >= q_pos[nq] - p.window_left;
-            s[nq][tg][j] = ok ? (c[j] - qbias[nq]) * sc[j] : kNegInf;
+            const uint32_t word = w[j];
+            float a, c;
+            if constexpr (OPK == KV_BF16) {
+              a = f16_bits_to_float(word & 0xffffu);
+              c = f16_bits_to_float(word >> 16);
+            } else {
+              a = bf16_bits_to_float(word & 0xffffu);
+              c = bf16_bits_to_float(word >> 16);
+            }
+            w[j] = __builtin_bit_cast(uint32_t, make_pair<Pair>(a, c));
+          }
+        }
+        qop[nq][sl] = __builtin_bit_cast(V8, w);
+      }
+    }
+    // rows of this wave: which query positions they span (wave-uniform), for skipping the mask on interior tiles
+    const bool wave_live = wave * kRowsPerWave < (tok_cnt << p.group_shift);
+    const int wave_qmin = ctx + tok0 + ((wave * kRowsPerWave) >> p.group_shift);
+    const int wave_qmax = ctx + tok0 + min(tok_cnt - 1, ((wave + 1) * kRowsPerWave - 1) >> p.group_shift);
+
+    float4_t acc[kRowTiles][NB];
+    float m_run[kRowTiles], l_run[kRowTiles];
+#pragma unroll
+    for (int nq = 0; nq < kRowTiles; ++nq) {
+      m_run[nq] = kNegInf;
+      l_run[nq] = 0.0f;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) acc[nq][nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    // ---- the tile pipeline -----------------------------------------------------------------------------------------
+    int ids_n[NLD], ids_k[NLD];
+    uint4_t kreg[NLD], vreg[NLD];
+    scale_raw_t ksreg[NLD], vsreg[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      ids_n[i] = ids_k[i] = 0;
+      kreg[i] = vreg[i] = uint4_t{0u, 0u, 0u, 0u};
+      ksreg[i] = vsreg[i] = scale_raw_t(0);
+    }
+    auto key_of = [&](int tile, int i) { return max(0, min(tile * TK + chunk_tok[i], key_hi)); };
+    auto load_ids = [&](int tile) {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const int t = key_of(tile, i);
+        ids_n[i] = packed ? 0 : table_row[p.bs_shift >= 0 ? (t >> p.bs_shift) : (t / p.block_size)];
+      }
+    };
+    auto issue_kv = [&](int tile) {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const int t = key_of(tile, i);
+        const int slot = p.bs_shift >= 0 ? (t & (p.block_size - 1)) : (t % p.block_size);
+        const int64_t row = packed ? (static_cast<int64_t>(q_begin) + t) * p.kv_heads + kvh
+                                   : (static_cast<int64_t>(ids_k[i]) * p.block_size + slot) * p.kv_heads + kvh;
+        kreg[i] = load16(p.k_cache, row * row_bytes + chunk_col[i] * 16);
+        vreg[i] = load16(p.v_cache, row * row_bytes + chunk_col[i] * 16);
+        if constexpr (T::kQuant) {
+          ksreg[i] = static_cast<const scale_raw_t*>(p.k_scale)[row];
+          vsreg[i] = static_cast<const scale_raw_t*>(p.v_scale)[row];
+        }
+      }
+    };
+    auto publish = [&](int tile) {
+      char* kd = s_k[tile & 1];
+      char* vd = s_v[tile & 1];
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        if (!chunk_live[i]) continue;
+        const int t = chunk_tok[i];
+        if constexpr (T::kQuant) {
+          uint4_t lo, hi;
+          dequant_chunk<KIND>(kreg[i], scale_value(ksreg[i]), lo, hi);
+          char* kdst = kd + t * RSK + chunk_col[i] * 32;
+          *reinterpret_cast<uint4_t*>(kdst) = lo;
+          *reinterpret_cast<uint4_t*>(kdst + 16) = hi;
+          dequant_chunk<KIND>(vreg[i], scale_value(vsreg[i]), lo, hi);
+          char* vdst = vd + v_row_of(t) * RSV + chunk_col[i] * 32;
+          *reinterpret_cast<uint4_t*>(vdst) = lo;
+          *reinterpret_cast<uint4_t*>(vdst + 16) = hi;
+        } else {
+          *reinterpret_cast<uint4_t*>(kd + t * RSK + chunk_col[i] * 16) = kreg[i];
+          *reinterpret_cast<uint4_t*>(vd + v_row_of(t) * RSV + chunk_col[i] * 16) = vreg[i];
+        }
+      }
+    };
+
+    // One tile step of a wave: S^T = K . Q^T, softmax, O^T += V^T . P^T; the mask only on tiles that cross a mask edge.
+    auto tile_step = [&](bool need_mask, int t) {
+      float s[kRowTiles][2][4];
+      {
+        const char* kt = s_k[t & 1];
+#pragma unroll
+        for (int tg = 0; tg < 2; ++tg) {
+          const char* krow = kt + (16 * tg + lr) * RSK + (D / 4) * 2 * lk;
+          V8 kop[NS];
+#pragma unroll
+          for (int sl = 0; sl < NS; ++sl) kop[sl] = *reinterpret_cast<const V8*>(krow + 16 * sl);
+#pragma unroll
+          for (int nq = 0; nq < kRowTiles; ++nq) {
+            float4_t c = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int sl = 0; sl < NS; ++sl) c = Ops::mfma(kop[sl], qop[nq][sl], c);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s[nq][tg][j] = c[j];
           }
         }
       }
-
-      // -- online softmax per row ----------------------------------------------------------------------------------
-      V8 pop[kRowTiles];
-      const float4_t vs0 = *reinterpret_cast<const float4_t*>(s_vsc + 4 * lk);
-      const float4_t vs1 = *reinterpret_cast<const float4_t*>(s_vsc + 16 + 4 * lk);
+      if (need_mask) {
+        const int k0 = t * TK;
+#pragma unroll
+        for (int nq = 0; nq < kRowTiles; ++nq) {
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int kpos = k0 + 16 * tg + 4 * lk + j;
+              bool ok = kpos <= q_pos[nq];
+              if (p.window_left >= 0) ok = ok && kpos >= q_pos[nq] - p.window_left;
+              s[nq][tg][j] = ok ? s[nq][tg][j] : kNegInf;
+            }
+          }
+        }
+      }
+      // -- online softmax in the log2 domain; the (positive) softmax scale is applied to the row maximum and inside
+      // the exponent's multiply-add -----------------------------------------------------------------------------------
+      float m_safe[kRowTiles], alpha[kRowTiles];
+      bool changed = false;
 #pragma unroll
       for (int nq = 0; nq < kRowTiles; ++nq) {
-        float mt = fmaxf(fmaxf(fmaxf(s[nq][0][0], s[nq][0][1]), fmaxf(s[nq][0][2], s[nq][0][3])),
-                         fmaxf(fmaxf(s[nq][1][0], s[nq][1][1]), fmaxf(s[nq][1][2], s[nq][1][3])));
-        mt = fmaxf(mt, wave_xor(mt, 16));
-        mt = fmaxf(mt, wave_xor(mt, 32));
-        const float m_new = fmaxf(m_run[nq], mt);
-        const float m_safe = m_new == kNegInf ? 0.0f : m_new;
-        const float alpha = fast_exp2(m_run[nq] - m_safe);
+        float mt = max3_f32(max3_f32(s[nq][0][0], s[nq][0][1], s[nq][0][2]),
+                            max3_f32(s[nq][0][3], s[nq][1][0], s[nq][1][1]),
+                            max3_f32(s[nq][1][2], s[nq][1][3], s[nq][1][3]));
+        mt = rows_max(mt) * p.scale_log2e;
+        const float m_new = max_f32(m_run[nq], mt);
+        m_safe[nq] = m_new == kNegInf ? 0.0f : m_new;
+        alpha[nq] = fast_exp2(m_run[nq] - m_safe[nq]);
         m_run[nq] = m_new;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-          l_run[nq] *= alpha;
-          p_sum[nq] *= alpha;
+        changed = changed || alpha[nq] != 1.0f;
+      }
+      if (__builtin_amdgcn_ballot_w64(changed) != 0) {
+#pragma unroll
+        for (int nq = 0; nq < kRowTiles; ++nq) {
+          scale_in_place(l_run[nq], alpha[nq]);
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[nq][nb][j] *= alpha;
+            for (int j = 0; j < 4; ++j) {
+              float a = acc[nq][nb][j];
+              scale_in_place(a, alpha[nq]);
+              acc[nq][nb][j] = a;
+            }
           }
         }
+      }
+      V8 pop[kRowTiles];
+#pragma unroll
+      for (int nq = 0; nq < kRowTiles; ++nq) {
         float pe[8];
+        float lsum = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float e0 = fast_exp2(s[nq][0][j] - m_safe);
-          const float e1 = fast_exp2(s[nq][1][j] - m_safe);
-          l_run[nq] += e0 + e1;
-          pe[j] = e0 * vs0[j];
-          pe[4 + j] = e1 * vs1[j];
+          pe[j] = fast_exp2(__builtin_fmaf(s[nq][0][j], p.scale_log2e, -m_safe[nq]));
+          pe[4 + j] = fast_exp2(__builtin_fmaf(s[nq][1][j], p.scale_log2e, -m_safe[nq]));
+          lsum += pe[j] + pe[4 + j];
         }
+        l_run[nq] += lsum;
         uint32_t pw[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          pw[j] = pack_pair<KIND>(pe[2 * j], pe[2 * j + 1]);
-          if constexpr (KIND == KV_I8) {
-            const Pair pr = __builtin_bit_cast(Pair, pw[j]);
-            p_sum[nq] += static_cast<float>(pr.x) + static_cast<float>(pr.y);
-          }
-        }
+        for (int j = 0; j < 4; ++j) pw[j] = pack_pair<OPK>(pe[2 * j], pe[2 * j + 1]);
         pop[nq] = __builtin_bit_cast(V8, uint4_t{pw[0], pw[1], pw[2], pw[3]});
       }
 
-      // -- O^T += V^T . P^T -----------------------------------------------------------------------------------------
+      // -- O^T += V^T . P^T: lane i of a 16-lane group supplies row (i / 4), 4 elements at column 16 nb + 4 (i % 4);
+      // two transpose reads of 4 tokens each -----------------------------------------------------------------------------
+      char* vt = s_v[t & 1];
+      const int r4 = lr >> 2;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
         uint32_t vw[4];
-        if constexpr (ES == 1) {
-          const int r8 = lr >> 1;
-          const int tok = r8 < 4 ? 4 * lk + r8 : 16 + 4 * lk + (r8 - 4);
-          char* a = s_v + v_row_of(tok) * RSV + 16 * nb + 8 * (lr & 1);
-          const int2_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_int2*)a);
-          vw[0] = static_cast<uint32_t>(r[0]);
-          vw[1] = static_cast<uint32_t>(r[1]);
-        } else {
-          const int r4 = lr >> 2;
 #pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const int tok = 16 * half + 4 * lk + r4;
-            char* a = s_v + v_row_of(tok) * RSV + (16 * nb + 4 * (lr & 3)) * 2;
-            const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
-            const uint2_t u = __builtin_bit_cast(uint2_t, r);
-            vw[2 * half] = u[0];
-            vw[2 * half + 1] = u[1];
-          }
+        for (int half = 0; half < 2; ++half) {
+          const int tok = 16 * half + 4 * lk + r4;
+          char* a = vt + v_row_of(tok) * RSV + (16 * nb + 4 * (lr & 3)) * 2;
+          const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
+          const uint2_t u = __builtin_bit_cast(uint2_t, r);
+          vw[2 * half] = u[0];
+          vw[2 * half + 1] = u[1];
         }
-        const V8 vop = to_operand<KIND>(vw);
+        const V8 vop = __builtin_bit_cast(V8, uint4_t{vw[0], vw[1], vw[2], vw[3]});
 #pragma unroll
         for (int nq = 0; nq < kRowTiles; ++nq) acc[nq][nb] = Ops::mfma(vop, pop[nq], acc[nq][nb]);
       }
-    }
-    __syncthreads();  // every wave is done with the tile before the next one overwrites it
-  }
+    };
 
-  // ---- normalise and store ------------------------------------------------------------------------------------------
+    // Iteration t computes tile t from LDS buffer t & 1, publishes tile t + 1 from the registers into the other
+    // buffer (everybody left it at the barrier), fetches tile t + 2 into the registers and the block ids of tile
+    // t + 3; the first three iterations only fill the pipe.  Fetch and publish run for every t (key positions are
+    // clamped into the item's range): what they bring in for tiles outside [ta, tb] lands in buffers nobody reads.
+    for (int t = ta - 3; t <= tb; ++t) {
+      __syncthreads();
+      publish(t + 1);
 #pragma unroll
-  for (int nq = 0; nq < kRowTiles; ++nq) {
-    float l_tot = l_run[nq];
-    l_tot += wave_xor(l_tot, 16);
-    l_tot += wave_xor(l_tot, 32);
-    float off = 0.0f;
-    if constexpr (KIND == KV_I8) {
-      float ps = p_sum[nq];
-      ps += wave_xor(ps, 16);
-      ps += wave_xor(ps, 32);
-      off = kI8Offset * ps;
+      for (int i = 0; i < NLD; ++i) ids_k[i] = ids_n[i];
+      issue_kv(t + 2);
+      load_ids(t + 3);
+      if (!wave_live || t < ta) continue;
+      const int k0 = t * TK;
+      const bool need_mask = k0 + TK - 1 > wave_qmin || (p.window_left >= 0 && k0 < wave_qmax - p.window_left);
+      tile_step(need_mask, t);
     }
-    if (q_pos[nq] >= 0) {
-      const float inv = 1.0f / (l_tot * kPScale);
+
+    // ---- finish the segment: final rows go to `out`, a cut item leaves its partial in the workspace ---------------
+    const int slot = 2 * unit + (first_item ? 0 : 1);
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        const int64_t e0 = row_elem[nq] + 16 * nb + 4 * lk;
-        uint32_t lo, hi;
-        const float o0 = (acc[nq][nb][0] - off) * inv, o1 = (acc[nq][nb][1] - off) * inv;
-        const float o2 = (acc[nq][nb][2] - off) * inv, o3 = (acc[nq][nb][3] - off) * inv;
-        if (p.q_dtype == ARENO_DT_BF16) {
-          lo = float_to_bf16_bits(o0) | (float_to_bf16_bits(o1) << 16);
-          hi = float_to_bf16_bits(o2) | (float_to_bf16_bits(o3) << 16);
-        } else {
-          lo = float_to_f16_bits(o0) | (float_to_f16_bits(o1) << 16);
-          hi = float_to_f16_bits(o2) | (float_to_f16_bits(o3) << 16);
+    for (int nq = 0; nq < kRowTiles; ++nq) {
+      const float l_tot = rows_sum(l_run[nq]);
+      if (q_pos[nq] < 0) continue;
+      if (whole) {
+        const float inv = 1.0f / l_tot;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const int64_t e0 = row_elem[nq] + 16 * nb + 4 * lk;
+          uint32_t lo, hi;
+          const float o0 = acc[nq][nb][0] * inv, o1 = acc[nq][nb][1] * inv;
+          const float o2 = acc[nq][nb][2] * inv, o3 = acc[nq][nb][3] * inv;
+          if (p.q_dtype == ARENO_DT_BF16) {
+            lo = float_to_bf16_bits(o0) | (float_to_bf16_bits(o1) << 16);
+            hi = float_to_bf16_bits(o2) | (float_to_bf16_bits(o3) << 16);
+          } else {
+            lo = float_to_f16_bits(o0) | (float_to_f16_bits(o1) << 16);
+            hi = float_to_f16_bits(o2) | (float_to_f16_bits(o3) << 16);
+          }
+          *reinterpret_cast<uint2_t*>(static_cast<char*>(p.out) + e0 * 2) = uint2_t{lo, hi};
         }
-        *reinterpret_cast<uint2_t*>(static_cast<char*>(p.out) + e0 * 2) = uint2_t{lo, hi};
+      } else {
+        const int r = wave * kRowsPerWave + 16 * nq + lr;
+        const int64_t prow = (static_cast<int64_t>(slot) * p.kv_heads + kvh) * kRowsPerWg + r;
+        float* dst = p.part_acc + prow * D + 4 * lk;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) *reinterpret_cast<float4_t*>(dst + 16 * nb) = acc[nq][nb];
+        if (lk == 0) {
+          p.part_ml[prow * 2] = m_run[nq];
+          p.part_ml[prow * 2 + 1] = l_tot;
+        }
       }
+    }
+
+    // ---- next item ---------------------------------------------------------------------------------------------------
+    x += tb - ta + 1;
+    first_item = false;
+    if (x < x_end) {
+      ++pos.j;
+      if (pos.j * tq >= pos.n_new) {
+        pos.j = 0;
+        do {
+          ++pos.seq;
+          if (pos.seq >= p.num_seqs) break;
+          pos.n_new = p.cu_seqlens_q[pos.seq + 1] - p.cu_seqlens_q[pos.seq];
+        } while (pos.n_new == 0);
+        if (pos.seq >= p.num_seqs) break;  // cannot happen while the prefix sums and this walk agree
+        pos.ctx = p.context_lens != nullptr ? p.context_lens[pos.seq] : 0;
+      }
+      pos.tile = block_tiles(pos.n_new, pos.ctx, pos.j, tq, p.window_left).tile_lo;
+    }
+    __syncthreads();  // every wave has left the segment before its LDS tiles are reused
+  }
+}
+
+// Merge of the items cut by unit borders.  Workgroup (u, kv head) looks at the last item of unit u: if that item
+// starts in unit u and runs on into later units, it combines the partials of all units the item touches (slot
+// 2u' for a unit where the item comes first, 2u' + 1 where it comes last after other items), normalises and
+// writes the item's rows.
+__global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillParams p) {
+  __shared__ int s_cum[kMaxPrefillSeqs + 1];
+  __shared__ int s_wave_tot[kPrefillWaves];
+  const int tid = threadIdx.x;
+  const int unit = blockIdx.x;
+  const int kvh = blockIdx.y;
+  const int kRowsPerWg = p.rows_per_wg;
+  const int tq = kRowsPerWg >> p.group_shift;
+  const int d = p.head_dim;
+  prefix_tile_steps(p, tq, s_cum, s_wave_tot);
+  const int total = s_cum[p.num_seqs];
+  const int x_begin = unit_start_step(total, unit, p.units);
+  const int x_end = unit_start_step(total, unit + 1, p.units);
+  if (x_begin >= x_end) return;
+  const StepPos pos = locate_step(p, s_cum, tq, x_end - 1);
+  const BlockTiles item = block_tiles(pos.n_new, pos.ctx, pos.j, tq, p.window_left);
+  const int item_x1 = pos.item_x0 + item.count();
+  if (item_x1 <= x_end || pos.item_x0 < x_begin) return;  // not cut here, or merged by the unit where it starts
+  // last unit that owns a step of the item: the largest u with unit_start_step(u) <= item_x1 - 1
+  int u_hi = static_cast<int>((static_cast<long long>(item_x1) * p.units - 1) / total);
+  if (u_hi > p.units - 1) u_hi = p.units - 1;
+  while (unit_start_step(total, u_hi, p.units) > item_x1 - 1) --u_hi;
+  while (u_hi + 1 < p.units && unit_start_step(total, u_hi + 1, p.units) <= item_x1 - 1) ++u_hi;
+
+  const int q_begin = p.cu_seqlens_q[pos.seq];
+  // thread -> (row, half of the head dim), 128 rows per pass
+  const int half = tid & 1;
+  const int dh = d / 2;
+  for (int r = tid >> 1; r < kRowsPerWg; r += kPrefillThreads / 2) {
+    const int t = r >> p.group_shift;
+    const int hh = r & (p.group_pad - 1);
+    if (t >= item.cnt || hh >= p.group) continue;
+    float m = kNegInf;
+    for (int u = unit; u <= u_hi; ++u) {
+      if (unit_start_step(total, u, p.units) == unit_start_step(total, u + 1, p.units)) continue;  // empty unit
+      const int slot = 2 * u + ((u == unit && pos.item_x0 > x_begin) ? 1 : 0);
+      const int64_t prow = (static_cast<int64_t>(slot) * p.kv_heads + kvh) * kRowsPerWg + r;
+      const float pm = p.part_ml[prow * 2];
+      const float pl = p.part_ml[prow * 2 + 1];
+      if (pl != 0.0f) m = fmaxf(m, pm);
+    }
+    const float m_safe = m == kNegInf ? 0.0f : m;
+    const int64_t out_elem =
+        (static_cast<int64_t>(q_begin + item.tok0 + t) * p.q_heads + kvh * p.group + hh) * d + half * dh;
+    for (int e0 = 0; e0 < dh; e0 += 4) {
+      float4_t o = {0.0f, 0.0f, 0.0f, 0.0f};
+      float lsum = 0.0f;
+      for (int u = unit; u <= u_hi; ++u) {
+        if (unit_start_step(total, u, p.units) == unit_start_step(total, u + 1, p.units)) continue;
+        const int slot = 2 * u + ((u == unit && pos.item_x0 > x_begin) ? 1 : 0);
+        const int64_t prow = (static_cast<int64_t>(slot) * p.kv_heads + kvh) * kRowsPerWg + r;
+        const float pl = p.part_ml[prow * 2 + 1];
+        if (pl == 0.0f) continue;  // a partial without visible keys
+        const float w = fast_exp2(p.part_ml[prow * 2] - m_safe);
+        lsum += w * pl;
+        const float4_t a = *reinterpret_cast<const float4_t*>(p.part_acc + prow * d + half * dh + e0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] += w * a[j];
+      }
+      const float inv = 1.0f / lsum;
+      uint32_t lo, hi;
+      if (p.q_dtype == ARENO_DT_BF16) {
+        lo = float_to_bf16_bits(o[0] * inv) | (float_to_bf16_bits(o[1] * inv) << 16);
+        hi = float_to_bf16_bits(o[2] * inv) | (float_to_bf16_bits(o[3] * inv) << 16);
+      } else {
+        lo = float_to_f16_bits(o[0] * inv) | (float_to_f16_bits(o[1] * inv) << 16);
+        hi = float_to_f16_bits(o[2] * inv) | (float_to_f16_bits(o[3] * inv) << 16);
+      }
+      *reinterpret_cast<uint2_t*>(static_cast<char*>(p.out) + (out_elem + e0) * 2) = uint2_t{lo, hi};
     }
   }
 }
 
 typedef void (*prefill_fn)(PrefillParams);
 
-template <int KIND>
-prefill_fn prefill_lookup(int head_dim, bool scale16) {
+template <int KIND, int RT>
+prefill_fn prefill_lookup_rt(int head_dim, bool scale16) {
   if constexpr (KVTraits<KIND>::kQuant) {
-    if (head_dim == 128) return scale16 ? prefill_mfma_kernel<KIND, 128, true> : prefill_mfma_kernel<KIND, 128, false>;
-    if (head_dim == 64) return scale16 ? prefill_mfma_kernel<KIND, 64, true> : prefill_mfma_kernel<KIND, 64, false>;
+    if (head_dim == 128)
+      return scale16 ? prefill_mfma_kernel<KIND, 128, true, RT> : prefill_mfma_kernel<KIND, 128, false, RT>;
+    if (head_dim == 64)
+      return scale16 ? prefill_mfma_kernel<KIND, 64, true, RT> : prefill_mfma_kernel<KIND, 64, false, RT>;
   } else {
-    if (head_dim == 128) return prefill_mfma_kernel<KIND, 128, false>;
-    if (head_dim == 64) return prefill_mfma_kernel<KIND, 64, false>;
+    if (head_dim == 128) return prefill_mfma_kernel<KIND, 128, false, RT>;
+    if (head_dim == 64) return prefill_mfma_kernel<KIND, 64, false, RT>;
   }
   return nullptr;
+}
+
+template <int KIND>
+prefill_fn prefill_lookup(int head_dim, bool scale16, int row_tiles) {
+  (void)row_tiles;
+  return prefill_lookup_rt<KIND, 2>(head_dim, scale16);
 }
 
 int log2_exact_i(int x) {
@@ -458,32 +686,75 @@ int log2_exact_i(int x) {
   return s;
 }
 
+int prefill_units(int kv_heads) {
+  int u = kPrefillTargetWgs / kv_heads;
+  if (u < 1) u = 1;
+  if (u > kMaxPrefillUnits) u = kMaxPrefillUnits;
+  return u;
+}
+
+size_t prefill_ml_bytes(int units, int kv_heads) {
+  return static_cast<size_t>(2) * units * kv_heads * kMaxRowsPerWg * 2 * sizeof(float);
+}
+
+int prefill_row_tiles() {
+  static const int v = [] {
+    const char* e = getenv("ARENO_PREFILL_ROW_TILES");
+    (void)e;
+    return 2;
+  }();
+  return v;
+}
+
 }  // namespace
+
+size_t prefill_mfma_workspace_bytes(int32_t kv_heads, int32_t head_dim) {
+  if (kv_heads <= 0 || head_dim <= 0) return 0;
+  const int units = prefill_units(kv_heads);
+  return prefill_ml_bytes(units, kv_heads) +
+         static_cast<size_t>(2) * units * kv_heads * kMaxRowsPerWg * head_dim * sizeof(float);
+}
 
 // block_table == nullptr selects packed K/V: cache->k / cache->v then point at (tokens, kv_heads, D) tensors and
 // context_lens may be nullptr (no cached context).
 int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out, int32_t q_dtype, int64_t tokens,
                         int32_t q_heads, int32_t num_seqs, const int32_t* block_table, int32_t max_blocks,
                         const int32_t* cu_seqlens_q, const int32_t* context_lens, int32_t window_left,
-                        float softmax_scale, void* stream) {
+                        float softmax_scale, void* workspace, size_t workspace_bytes, void* stream) {
   const char* op = "areno_hip_paged_varlen_prefill";
   const int group = q_heads / cache->kv_heads;
   if (q_dtype != ARENO_DT_F16 && q_dtype != ARENO_DT_BF16) return ARENO_ERR_UNSUPPORTED;
+  if (!(softmax_scale > 0.0f)) return ARENO_ERR_UNSUPPORTED;  // the kernel takes row maxima before scaling
   if (group > 16 || num_seqs > kMaxPrefillSeqs || tokens > 0x3fffffff) return ARENO_ERR_UNSUPPORTED;
   if (cache->kv_heads > 65535) return ARENO_ERR_UNSUPPORTED;
   if (reinterpret_cast<uintptr_t>(cache->k) % 16 != 0 || reinterpret_cast<uintptr_t>(cache->v) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(q) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 8 != 0)
     return ARENO_ERR_UNSUPPORTED;
   const bool scale16 = cache->scale_dtype == ARENO_DT_F16;
+  const int row_tiles = prefill_row_tiles();
+  const int rows_per_wg = 16 * row_tiles * kPrefillWaves;
   prefill_fn fn = nullptr;
   switch (cache->cache_dtype) {
-    case ARENO_DT_BF16: fn = prefill_lookup<KV_BF16>(cache->head_dim, scale16); break;
-    case ARENO_DT_F16: fn = prefill_lookup<KV_F16>(cache->head_dim, scale16); break;
-    case ARENO_DT_I8: fn = prefill_lookup<KV_I8>(cache->head_dim, scale16); break;
-    case ARENO_DT_FP8_E4M3: fn = prefill_lookup<KV_FP8>(cache->head_dim, scale16); break;
+    case ARENO_DT_BF16: fn = prefill_lookup<KV_BF16>(cache->head_dim, scale16, row_tiles); break;
+    case ARENO_DT_F16: fn = prefill_lookup<KV_F16>(cache->head_dim, scale16, row_tiles); break;
+    case ARENO_DT_I8: fn = prefill_lookup<KV_I8>(cache->head_dim, scale16, row_tiles); break;
+    case ARENO_DT_FP8_E4M3: fn = prefill_lookup<KV_FP8>(cache->head_dim, scale16, row_tiles); break;
     default: break;
   }
   if (fn == nullptr) return ARENO_ERR_UNSUPPORTED;
+  // tile steps are counted in 32-bit: (tokens / query block + seqs) * (longest visible range / 32) must fit; the
+  // paged case is bounded by the table width
+  const int64_t max_keys = block_table != nullptr ? static_cast<int64_t>(max_blocks) * cache->block_size : tokens;
+  {
+    int gp = 1;
+    while (gp < group) gp <<= 1;
+    const int64_t items = tokens / (rows_per_wg / gp) + num_seqs;
+    if (items * (max_keys / kTileTokens + 1) > 0x7fffffffLL) return ARENO_ERR_UNSUPPORTED;
+  }
+  const size_t need = prefill_mfma_workspace_bytes(cache->kv_heads, cache->head_dim);
+  if (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+    return fail(ARENO_ERR_WORKSPACE, "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", op, need,
+                workspace_bytes);
 
   PrefillParams p;
   p.q = q;
@@ -498,6 +769,7 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   p.num_seqs = num_seqs;
   p.q_heads = q_heads;
   p.kv_heads = cache->kv_heads;
+  p.head_dim = cache->head_dim;
   p.group = group;
   p.group_pad = 1;
   while (p.group_pad < group) p.group_pad <<= 1;
@@ -507,13 +779,15 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   p.max_blocks = max_blocks;
   p.window_left = window_left;
   p.q_dtype = q_dtype;
+  p.units = prefill_units(cache->kv_heads);
+  p.rows_per_wg = rows_per_wg;
   p.scale_log2e = softmax_scale * kLog2e;
-  // upper bound of query blocks without knowing the sequence lengths on the host
-  const int tokens_per_wg = kRowsPerWg / p.group_pad;
-  const int64_t max_blocks_q = (tokens + tokens_per_wg - 1) / tokens_per_wg + num_seqs;
-  if (max_blocks_q > 0x7fffffff) return ARENO_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(fn, dim3(static_cast<unsigned>(max_blocks_q), cache->kv_heads), dim3(kPrefillThreads), 0,
-                     static_cast<hipStream_t>(stream), p);
+  p.part_ml = static_cast<float*>(workspace);
+  p.part_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + prefill_ml_bytes(p.units, cache->kv_heads));
+  const dim3 grid(p.units, cache->kv_heads);
+  hipLaunchKernelGGL(fn, grid, dim3(kPrefillThreads), 0, static_cast<hipStream_t>(stream), p);
+  if (int rc = check_launch(op)) return rc;
+  hipLaunchKernelGGL(prefill_merge_kernel, grid, dim3(kPrefillThreads), 0, static_cast<hipStream_t>(stream), p);
   return check_launch(op);
 }
 

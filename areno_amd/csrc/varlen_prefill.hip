@@ -147,14 +147,20 @@ int launch_generic(const VarlenParams& p, void* stream, const char* op) {
 int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out, int32_t q_dtype, int64_t tokens,
                         int32_t q_heads, int32_t num_seqs, const int32_t* block_table, int32_t max_blocks,
                         const int32_t* cu_seqlens_q, const int32_t* context_lens, int32_t window_left,
-                        float softmax_scale, void* stream);
+                        float softmax_scale, void* workspace, size_t workspace_bytes, void* stream);
+size_t prefill_mfma_workspace_bytes(int32_t kv_heads, int32_t head_dim);
 
 }  // namespace areno
+
+extern "C" size_t areno_hip_prefill_workspace_bytes(int32_t kv_heads, int32_t head_dim) {
+  return areno::prefill_mfma_workspace_bytes(kv_heads, head_dim);
+}
 
 extern "C" int areno_hip_varlen_attention(const void* q, const void* k, const void* v, void* out, int32_t dtype,
                                           int64_t tokens, int32_t q_heads, int32_t kv_heads, int32_t head_dim,
                                           const int32_t* cu_seqlens, int32_t num_seqs, int32_t window_left,
-                                          float softmax_scale, void* stream) {
+                                          float softmax_scale, void* workspace, size_t workspace_bytes,
+                                          void* stream) {
   using namespace areno;
   const char* op = "areno_hip_varlen_attention";
   if (q == nullptr || k == nullptr || v == nullptr || out == nullptr || cu_seqlens == nullptr)
@@ -178,7 +184,7 @@ extern "C" int areno_hip_varlen_attention(const void* q, const void* k, const vo
     packed.cache_dtype = dtype;
     packed.scale_dtype = ARENO_DT_F32;
     const int rc = launch_prefill_mfma(&packed, q, out, dtype, tokens, q_heads, num_seqs, nullptr, 1, cu_seqlens,
-                                       nullptr, window_left, softmax_scale, stream);
+                                       nullptr, window_left, softmax_scale, workspace, workspace_bytes, stream);
     if (rc != ARENO_ERR_UNSUPPORTED) return rc;
   }
   VarlenParams p = {};
@@ -204,7 +210,8 @@ extern "C" int areno_hip_paged_varlen_prefill(const areno_paged_cache* cache, co
                                               int32_t q_dtype, int64_t tokens, int32_t q_heads, int32_t num_seqs,
                                               const int32_t* block_table, int32_t max_blocks,
                                               const int32_t* cu_seqlens_q, const int32_t* context_lens,
-                                              int32_t window_left, float softmax_scale, void* stream) {
+                                              int32_t window_left, float softmax_scale, void* workspace,
+                                              size_t workspace_bytes, void* stream) {
   using namespace areno;
   const char* op = "areno_hip_paged_varlen_prefill";
   if (int rc = validate_paged_cache(cache, op)) return rc;
@@ -223,7 +230,8 @@ extern "C" int areno_hip_paged_varlen_prefill(const areno_paged_cache* cache, co
   if (tokens == 0) return ARENO_OK;
 
   const int rc = launch_prefill_mfma(cache, q, out, q_dtype, tokens, q_heads, num_seqs, block_table, max_blocks,
-                                     cu_seqlens_q, context_lens, window_left, softmax_scale, stream);
+                                     cu_seqlens_q, context_lens, window_left, softmax_scale, workspace, workspace_bytes,
+                                     stream);
   if (rc != ARENO_ERR_UNSUPPORTED) return rc;
 
   VarlenParams p = {};

@@ -131,10 +131,12 @@ int areno_hip_paged_decode_stages(const areno_paged_cache* cache, const void* q,
  * cu_seqlens[s] sees keys [max(cu_seqlens[s], t - window_left), t] (all of [cu_seqlens[s], t] when window_left < 0).
  *   q, out  device [tokens, q_heads, head_dim];  k, v  device [tokens, kv_heads, head_dim];  all `dtype`
  *   cu_seqlens  device [num_seqs + 1] int32
+ *   workspace   device, at least areno_hip_prefill_workspace_bytes(kv_heads, head_dim) bytes (may be NULL for F32)
  */
 int areno_hip_varlen_attention(const void* q, const void* k, const void* v, void* out, int32_t dtype, int64_t tokens,
                                int32_t q_heads, int32_t kv_heads, int32_t head_dim, const int32_t* cu_seqlens,
-                               int32_t num_seqs, int32_t window_left, float softmax_scale, void* stream);
+                               int32_t num_seqs, int32_t window_left, float softmax_scale, void* workspace,
+                               size_t workspace_bytes, void* stream);
 
 /*
  * Causal prefill of new queries over paged (optionally quantized) KV; the new tokens' K/V must already be in
@@ -145,11 +147,22 @@ int areno_hip_varlen_attention(const void* q, const void* k, const void* v, void
  *   q, out        device [tokens, q_heads, head_dim], q_dtype (F16/BF16)
  *   cu_seqlens_q  device [num_seqs + 1] int32;  context_lens device [num_seqs] int32
  *   block_table   device [num_seqs, max_blocks] int32
+ *   workspace     device, at least areno_hip_prefill_workspace_bytes(cache->kv_heads, cache->head_dim) bytes
  */
 int areno_hip_paged_varlen_prefill(const areno_paged_cache* cache, const void* q, void* out, int32_t q_dtype,
                                    int64_t tokens, int32_t q_heads, int32_t num_seqs, const int32_t* block_table,
                                    int32_t max_blocks, const int32_t* cu_seqlens_q, const int32_t* context_lens,
-                                   int32_t window_left, float softmax_scale, void* stream);
+                                   int32_t window_left, float softmax_scale, void* workspace, size_t workspace_bytes,
+                                   void* stream);
+
+/*
+ * Bytes of device workspace the two prefill entry points above need (the reference allocates nothing here: its
+ * varlen kernel keeps one query row per thread block, areno/accel/csrc/attention.cu:145-242).  The matrix-core
+ * kernels cut the work into equal shares of key tiles whatever the length distribution, and a query block cut by a
+ * share border leaves its un-normalised partial (running max, sum, accumulator) here for the merge kernel.  The
+ * size depends only on the head geometry, not on the batch.  16-byte aligned.
+ */
+size_t areno_hip_prefill_workspace_bytes(int32_t kv_heads, int32_t head_dim);
 
 #ifdef __cplusplus
 }
