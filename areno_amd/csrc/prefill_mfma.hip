@@ -263,7 +263,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
 #pragma unroll
   for (int i = 0; i < NLD; ++i) {
     const int c = tid + kPrefillThreads * i;
-    chunk_live[i] = c < CHUNKS;
+    chunk_live[i] = (i + 1) * kPrefillThreads <= CHUNKS || c < CHUNKS;
     chunk_tok[i] = min(c, CHUNKS - 1) / LPT;
     chunk_col[i] = min(c, CHUNKS - 1) % LPT;
   }
@@ -289,7 +289,9 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
     const int tok0 = item.tok0;
     const int tok_cnt = item.cnt;
     const int key_hi = ctx + tok0 + tok_cnt - 1;
-    const int32_t* table_row = packed ? nullptr : p.block_table + static_cast<int64_t>(pos.seq) * p.max_blocks;
+    // packed K/V have no table: the id load then reads a valid dummy word and its value is ignored
+    const int32_t* table_row =
+        packed ? p.cu_seqlens_q : p.block_table + static_cast<int64_t>(pos.seq) * p.max_blocks;
 
     // ---- this lane's query rows: row R = wave * 16 RT + 16 * nq + lr -> token tok0 + (R >> group_shift), head
     // R & (group_pad - 1) --------------------------------------------------------------------------------------------
@@ -356,29 +358,44 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
         const int t = key_of(tile, i);
-        ids_n[i] = packed ? 0 : table_row[p.bs_shift >= 0 ? (t >> p.bs_shift) : (t / p.block_size)];
+        ids_n[i] = table_row[packed ? 0 : (t >> p.bs_shift)];
       }
     };
-    auto issue_kv = [&](int tile) {
+    auto cache_row = [&](int tile, int i) -> int64_t {
+      const int t = key_of(tile, i);
+      // page size is a power of two here (the launcher sends other sizes to the generic kernel); packed K/V run as
+      // one page per token with the token's row as its id
+      const int slot = t & (p.block_size - 1);
+      const int64_t page_row = packed ? static_cast<int64_t>(q_begin) + t
+                                      : (static_cast<int64_t>(ids_k[i]) << p.bs_shift) + slot;
+      return page_row * p.kv_heads + kvh;
+    };
+    int64_t v_row[NLD];  // cache row of the K chunk in flight: its V chunk is fetched one iteration later
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) v_row[i] = 0;
+    auto issue_v = [&]() {
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
-        const int t = key_of(tile, i);
-        const int slot = p.bs_shift >= 0 ? (t & (p.block_size - 1)) : (t % p.block_size);
-        const int64_t row = packed ? (static_cast<int64_t>(q_begin) + t) * p.kv_heads + kvh
-                                   : (static_cast<int64_t>(ids_k[i]) * p.block_size + slot) * p.kv_heads + kvh;
+        vreg[i] = load16(p.v_cache, v_row[i] * row_bytes + chunk_col[i] * 16);
+        if constexpr (T::kQuant) vsreg[i] = static_cast<const scale_raw_t*>(p.v_scale)[v_row[i]];
+      }
+    };
+    auto issue_k = [&](int tile) {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const int64_t row = cache_row(tile, i);
+        v_row[i] = row;
         kreg[i] = load16(p.k_cache, row * row_bytes + chunk_col[i] * 16);
-        vreg[i] = load16(p.v_cache, row * row_bytes + chunk_col[i] * 16);
-        if constexpr (T::kQuant) {
-          ksreg[i] = static_cast<const scale_raw_t*>(p.k_scale)[row];
-          vsreg[i] = static_cast<const scale_raw_t*>(p.v_scale)[row];
-        }
+        if constexpr (T::kQuant) ksreg[i] = static_cast<const scale_raw_t*>(p.k_scale)[row];
       }
     };
-    auto publish = [&](int tile) {
+    // The empty asm pins the use of a fetched chunk to this point of the iteration: without it the compiler converts
+    // the codes right at the top of the loop and every tile waits there for the loads it has just issued.
+    auto publish_k = [&](int tile) {
       char* kd = s_k[tile & 1];
-      char* vd = s_v[tile & 1];
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
+        asm volatile("" : "+v"(kreg[i]));
         if (!chunk_live[i]) continue;
         const int t = chunk_tok[i];
         if constexpr (T::kQuant) {
@@ -387,40 +404,80 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
           char* kdst = kd + t * RSK + chunk_col[i] * 32;
           *reinterpret_cast<uint4_t*>(kdst) = lo;
           *reinterpret_cast<uint4_t*>(kdst + 16) = hi;
+        } else {
+          *reinterpret_cast<uint4_t*>(kd + t * RSK + chunk_col[i] * 16) = kreg[i];
+        }
+      }
+    };
+    auto publish_v = [&](int tile) {
+      char* vd = s_v[tile & 1];
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        asm volatile("" : "+v"(vreg[i]));
+        if (!chunk_live[i]) continue;
+        const int t = chunk_tok[i];
+        if constexpr (T::kQuant) {
+          uint4_t lo, hi;
           dequant_chunk<KIND>(vreg[i], scale_value(vsreg[i]), lo, hi);
           char* vdst = vd + v_row_of(t) * RSV + chunk_col[i] * 32;
           *reinterpret_cast<uint4_t*>(vdst) = lo;
           *reinterpret_cast<uint4_t*>(vdst + 16) = hi;
         } else {
-          *reinterpret_cast<uint4_t*>(kd + t * RSK + chunk_col[i] * 16) = kreg[i];
           *reinterpret_cast<uint4_t*>(vd + v_row_of(t) * RSV + chunk_col[i] * 16) = vreg[i];
         }
       }
     };
+    // Staging step of iteration t: K[t + 2] and V[t + 1] go from the registers into the LDS buffers the previous
+    // iteration was the last to read, then K[t + 3], V[t + 2] and the block ids of tile t + 4 are fetched.  It runs for
+    // every t (key positions are clamped into the item's range): tiles outside [ta, tb] land in buffers nobody reads.
+    auto stage = [&](int t) {
+      publish_k(t + 2);
+      publish_v(t + 1);
+      issue_v();  // rows of tile t + 2, remembered when its K chunk was fetched
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) ids_k[i] = ids_n[i];
+      issue_k(t + 3);
+      load_ids(t + 4);
+    };
 
-    // One tile step of a wave: S^T = K . Q^T, softmax, O^T += V^T . P^T; the mask only on tiles that cross a mask edge.
-    auto tile_step = [&](bool need_mask, int t) {
-      float s[kRowTiles][2][4];
-      {
-        const char* kt = s_k[t & 1];
+    // raw scores of one key tile: S^T = K . Q^T
+    float s_cur[kRowTiles][2][4];
+    auto scores = [&](int tile, float (&s)[kRowTiles][2][4]) {
+      const char* kt = s_k[tile & 1];
 #pragma unroll
-        for (int tg = 0; tg < 2; ++tg) {
-          const char* krow = kt + (16 * tg + lr) * RSK + (D / 4) * 2 * lk;
-          V8 kop[NS];
+      for (int tg = 0; tg < 2; ++tg) {
+        const char* krow = kt + (16 * tg + lr) * RSK + (D / 4) * 2 * lk;
+        V8 kop[NS];
 #pragma unroll
-          for (int sl = 0; sl < NS; ++sl) kop[sl] = *reinterpret_cast<const V8*>(krow + 16 * sl);
+        for (int sl = 0; sl < NS; ++sl) kop[sl] = *reinterpret_cast<const V8*>(krow + 16 * sl);
 #pragma unroll
-          for (int nq = 0; nq < kRowTiles; ++nq) {
-            float4_t c = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int nq = 0; nq < kRowTiles; ++nq) {
+          float4_t c = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int sl = 0; sl < NS; ++sl) c = Ops::mfma(kop[sl], qop[nq][sl], c);
+          for (int sl = 0; sl < NS; ++sl) c = Ops::mfma(kop[sl], qop[nq][sl], c);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) s[nq][tg][j] = c[j];
-          }
+          for (int j = 0; j < 4; ++j) s[nq][tg][j] = c[j];
         }
       }
+    };
+
+    // ---- fill the pipe: after these iterations K[ta], K[ta + 1] and V[ta] are in LDS ---------------------------------
+    for (int t = ta - 4; t < ta; ++t) {
+      __syncthreads();
+      stage(t);
+    }
+    __syncthreads();
+    if (wave_live) scores(ta, s_cur);
+
+    // ---- iteration t: staging first, then the scores of tile t + 1 go to the matrix cores in the same block as the row
+    // maxima of tile t ---------------------------------------------------------------------------------------------------
+    for (int t = ta; t <= tb; ++t) {
+      __syncthreads();
+      stage(t);  // first: the loads it issues then have the whole iteration to land
+      if (!wave_live) continue;
+      const int k0 = t * TK;
+      const bool need_mask = k0 + TK - 1 > wave_qmin || (p.window_left >= 0 && k0 < wave_qmax - p.window_left);
       if (need_mask) {
-        const int k0 = t * TK;
 #pragma unroll
         for (int nq = 0; nq < kRowTiles; ++nq) {
 #pragma unroll
@@ -430,20 +487,22 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
               const int kpos = k0 + 16 * tg + 4 * lk + j;
               bool ok = kpos <= q_pos[nq];
               if (p.window_left >= 0) ok = ok && kpos >= q_pos[nq] - p.window_left;
-              s[nq][tg][j] = ok ? s[nq][tg][j] : kNegInf;
+              s_cur[nq][tg][j] = ok ? s_cur[nq][tg][j] : kNegInf;
             }
           }
         }
       }
+      float s_next[kRowTiles][2][4];
+      scores(t + 1, s_next);  // past tb this reads a buffer of clamped or stale keys; the result is dropped
       // -- online softmax in the log2 domain; the (positive) softmax scale is applied to the row maximum and inside
       // the exponent's multiply-add -----------------------------------------------------------------------------------
       float m_safe[kRowTiles], alpha[kRowTiles];
       bool changed = false;
 #pragma unroll
       for (int nq = 0; nq < kRowTiles; ++nq) {
-        float mt = max3_f32(max3_f32(s[nq][0][0], s[nq][0][1], s[nq][0][2]),
-                            max3_f32(s[nq][0][3], s[nq][1][0], s[nq][1][1]),
-                            max3_f32(s[nq][1][2], s[nq][1][3], s[nq][1][3]));
+        float mt = max3_f32(max3_f32(s_cur[nq][0][0], s_cur[nq][0][1], s_cur[nq][0][2]),
+                            max3_f32(s_cur[nq][0][3], s_cur[nq][1][0], s_cur[nq][1][1]),
+                            max3_f32(s_cur[nq][1][2], s_cur[nq][1][3], s_cur[nq][1][3]));
         mt = rows_max(mt) * p.scale_log2e;
         const float m_new = max_f32(m_run[nq], mt);
         m_safe[nq] = m_new == kNegInf ? 0.0f : m_new;
@@ -473,8 +532,8 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
         float lsum = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          pe[j] = fast_exp2(__builtin_fmaf(s[nq][0][j], p.scale_log2e, -m_safe[nq]));
-          pe[4 + j] = fast_exp2(__builtin_fmaf(s[nq][1][j], p.scale_log2e, -m_safe[nq]));
+          pe[j] = fast_exp2(__builtin_fmaf(s_cur[nq][0][j], p.scale_log2e, -m_safe[nq]));
+          pe[4 + j] = fast_exp2(__builtin_fmaf(s_cur[nq][1][j], p.scale_log2e, -m_safe[nq]));
           lsum += pe[j] + pe[4 + j];
         }
         l_run[nq] += lsum;
@@ -504,23 +563,14 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
 #pragma unroll
         for (int nq = 0; nq < kRowTiles; ++nq) acc[nq][nb] = Ops::mfma(vop, pop[nq], acc[nq][nb]);
       }
-    };
-
-    // Iteration t computes tile t from LDS buffer t & 1, publishes tile t + 1 from the registers into the other
-    // buffer (everybody left it at the barrier), fetches tile t + 2 into the registers and the block ids of tile
-    // t + 3; the first three iterations only fill the pipe.  Fetch and publish run for every t (key positions are
-    // clamped into the item's range): what they bring in for tiles outside [ta, tb] lands in buffers nobody reads.
-    for (int t = ta - 3; t <= tb; ++t) {
-      __syncthreads();
-      publish(t + 1);
 #pragma unroll
-      for (int i = 0; i < NLD; ++i) ids_k[i] = ids_n[i];
-      issue_kv(t + 2);
-      load_ids(t + 3);
-      if (!wave_live || t < ta) continue;
-      const int k0 = t * TK;
-      const bool need_mask = k0 + TK - 1 > wave_qmin || (p.window_left >= 0 && k0 < wave_qmax - p.window_left);
-      tile_step(need_mask, t);
+      for (int nq = 0; nq < kRowTiles; ++nq) {
+#pragma unroll
+        for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) s_cur[nq][tg][j] = s_next[nq][tg][j];
+        }
+      }
     }
 
     // ---- finish the segment: final rows go to `out`, a cut item leaves its partial in the workspace ---------------
@@ -725,6 +775,7 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   const int group = q_heads / cache->kv_heads;
   if (q_dtype != ARENO_DT_F16 && q_dtype != ARENO_DT_BF16) return ARENO_ERR_UNSUPPORTED;
   if (!(softmax_scale > 0.0f)) return ARENO_ERR_UNSUPPORTED;  // the kernel takes row maxima before scaling
+  if (log2_exact_i(cache->block_size) < 0) return ARENO_ERR_UNSUPPORTED;  // page addressing by shift and mask
   if (group > 16 || num_seqs > kMaxPrefillSeqs || tokens > 0x3fffffff) return ARENO_ERR_UNSUPPORTED;
   if (cache->kv_heads > 65535) return ARENO_ERR_UNSUPPORTED;
   if (reinterpret_cast<uintptr_t>(cache->k) % 16 != 0 || reinterpret_cast<uintptr_t>(cache->v) % 16 != 0 ||
