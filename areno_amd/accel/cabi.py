@@ -15,6 +15,7 @@ from areno_amd.accel._extension import library_path
 
 DT_F32, DT_F16, DT_BF16, DT_I8, DT_FP8_E4M3 = 0, 1, 2, 3, 4
 STAGE_APPEND, STAGE_SPLIT, STAGE_REDUCE, STAGE_ALL = 1, 2, 4, 7
+OK, ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_LAUNCH = 0, -1, -2, -3, -4
 
 _DTYPE_CODES = {
     torch.float32: DT_F32,
@@ -114,3 +115,21 @@ def paged_decode(cache: PagedCache, q, k_update, v_update, out, block_table, cac
         current_stream_ptr() if stream is None else stream,
     )  # fmt: skip
     check(status, "areno_hip_paged_decode")
+
+
+def prefill_workspace_bytes(kv_heads: int, head_dim: int) -> int:
+    return int(lib().areno_hip_prefill_workspace_bytes(int(kv_heads), int(head_dim)))
+
+
+def paged_varlen_prefill(cache: PagedCache, q, out, block_table, cu_seqlens_q, context_lens, workspace, *,
+                         window_left=-1, softmax_scale=None, workspace_bytes=None, stream=None) -> int:  # fmt: skip
+    """``areno_hip_paged_varlen_prefill`` on raw pointers; returns the status code instead of raising, so a caller
+    can probe error paths (``check`` turns it into an exception)."""
+    scale = float(softmax_scale if softmax_scale is not None else q.shape[-1] ** -0.5)
+    return int(lib().areno_hip_paged_varlen_prefill(
+        ctypes.byref(cache), q.data_ptr(), out.data_ptr(), dtype_code(q), q.shape[0], q.shape[1],
+        context_lens.shape[0], block_table.data_ptr(), block_table.shape[1], cu_seqlens_q.data_ptr(),
+        context_lens.data_ptr(), int(window_left), scale, workspace.data_ptr(),
+        workspace.numel() if workspace_bytes is None else int(workspace_bytes),
+        current_stream_ptr() if stream is None else stream,
+    ))  # fmt: skip

@@ -17,19 +17,18 @@
 // One segment, per 32-key tile t (all four waves share the K/V tiles in LDS):
 //   * the 256 threads fetch K three tiles and V two tiles ahead with 16-byte coalesced loads (block ids one more
 //     tile ahead) and publish them into double-buffered LDS tiles one iteration before their first use, so one
-//     barrier per tile is enough (padded rows, conflict free);
-//   * S^T[key][row] = K . Q^T of tile t + 1 is issued before the softmax of tile t, so the matrix cores have
-//     independent work while the vector ALU runs the softmax: A = K rows from LDS, B = Q^T in registers; C has
-//     row = lane % 16, 4 keys per lane;
-//   * per-key K scale, causal / window mask only on tiles that cross a mask edge, online softmax in the log2
-//     domain (per lane = per row);
+//     barrier per tile is enough (padded rows, conflict free).  8-bit codes are dequantized (times the per-token
+//     scale) by the thread that stages them, once per workgroup: the tiles in LDS are always 16-bit;
+//   * S^T[key][row] = K . Q^T of tile t + 1 is issued in the same basic block as the row maxima of tile t, so the
+//     matrix cores have independent work while the vector ALU runs the softmax: A = K rows from LDS, B = Q^T in
+//     registers; C has row = lane % 16, 4 keys per lane;
+//   * causal / window mask only on tiles that cross a mask edge, online softmax in the log2 domain (per lane = per
+//     row; the four lanes of a row combine through v_permlane swaps), the softmax scale folded into the exponent's
+//     multiply-add;
 //   * O^T[dim][row] += V^T . P^T : A = V^T through the LDS transpose reads, B = P^T (= the C layout of S^T).
-// The dequantisation of int8 / fp8 codes and the layouts are the ones of the decode kernel
-// (decode_mfma_kernels.hpp).  Semantics: _reference_attention with query_start = context_lens[s]
-// (areno/accel/attention.py:25-41 in the reference); with context 0 it is the reference's varlen kernel
-// (areno/accel/csrc/attention.cu:145-242).
-
-#include <cstdlib>
+// The LDS layouts are the 16-bit ones of the decode kernel (decode_mfma_kernels.hpp).  Semantics:
+// _reference_attention with query_start = context_lens[s] (areno/accel/attention.py:25-41 in the reference); with
+// context 0 it is the reference's varlen kernel (areno/accel/csrc/attention.cu:145-242).
 
 #include "decode_mfma_kernels.hpp"
 
@@ -45,8 +44,8 @@ namespace {
 
 constexpr int kPrefillThreads = 256;
 constexpr int kPrefillWaves = 4;
-constexpr int kMaxRowTiles = 4;                                       // 16-row MFMA tiles per wave, at most
-constexpr int kMaxRowsPerWg = 16 * kMaxRowTiles * kPrefillWaves;      // 256
+constexpr int kMaxRowTiles = 2;                                   // 16-row MFMA tiles per wave
+constexpr int kMaxRowsPerWg = 16 * kMaxRowTiles * kPrefillWaves;  // 128
 constexpr int kMaxPrefillSeqs = 1024;
 constexpr int kPrefillTargetWgs = 512;  // two resident workgroups on each of the 256 CUs
 constexpr int kMaxPrefillUnits = 512;   // per kv head
@@ -725,7 +724,7 @@ prefill_fn prefill_lookup_rt(int head_dim, bool scale16) {
 
 template <int KIND>
 prefill_fn prefill_lookup(int head_dim, bool scale16, int row_tiles) {
-  (void)row_tiles;
+  (void)row_tiles;  // two 16-row tiles per wave is the only shape built: four need more registers than a wave has
   return prefill_lookup_rt<KIND, 2>(head_dim, scale16);
 }
 
@@ -747,14 +746,7 @@ size_t prefill_ml_bytes(int units, int kv_heads) {
   return static_cast<size_t>(2) * units * kv_heads * kMaxRowsPerWg * 2 * sizeof(float);
 }
 
-int prefill_row_tiles() {
-  static const int v = [] {
-    const char* e = getenv("ARENO_PREFILL_ROW_TILES");
-    (void)e;
-    return 2;
-  }();
-  return v;
-}
+int prefill_row_tiles() { return 2; }
 
 }  // namespace
 

@@ -85,6 +85,66 @@ def test_cfg4_reduced():
     assert_close(_run_prefill(w), _expected_prefill(w), *tolerances("fp8"), what="cfg4 reduced")
 
 
+@pytest.mark.parametrize("kv", ["bf16", "int8"])
+def test_prefill_one_query_block_cut_by_many_shares(kv):
+    """A single short chunk on a long context: every workgroup owns a slice of the same query block's keys, so the
+    result only exists after the merge of all their partials."""
+    w = workloads.make_prefill_workload("long-ctx", seed=21, new_lens=torch.tensor([9]), ctx_lens=torch.tensor([6000]),
+                                        hq=8, hkv=2, d=128, bs=16, kv=kv, device=DEV, quantize_fn=gpu_quantize)  # fmt: skip
+    assert_close(_run_prefill(w), _expected_prefill(w), *tolerances(kv), what="one block, many shares")
+
+
+def test_prefill_sequences_without_new_tokens_and_single_tokens():
+    """Empty chunks (cu_seqlens repeats) between chunks of 1, 33 and 200 tokens; contexts 0, tile-aligned and odd."""
+    new = torch.tensor([0, 1, 0, 33, 1, 0, 200, 0])
+    ctx = torch.tensor([50, 0, 0, 64, 1023, 7, 31, 0])
+    w = workloads.make_prefill_workload("ragged", seed=22, new_lens=new, ctx_lens=ctx, hq=12, hkv=4, d=64, bs=32,
+                                        kv="fp8", device=DEV, quantize_fn=gpu_quantize)  # fmt: skip
+    assert_close(_run_prefill(w), _expected_prefill(w), *tolerances("fp8"), what="ragged chunks")
+
+
+@pytest.mark.parametrize("window_left", [0, 31, 32, 100, 5000])
+def test_prefill_window_moves_the_first_tile(window_left):
+    """Sliding windows shorter than, equal to and longer than a key tile, and longer than every context."""
+    new = torch.tensor([70, 3, 130])
+    ctx = torch.tensor([900, 40, 0])
+    w = workloads.make_prefill_workload("window", seed=23, new_lens=new, ctx_lens=ctx, hq=8, hkv=2, d=128, bs=16,
+                                        kv="bf16", device=DEV)  # fmt: skip
+    assert_close(_run_prefill(w, window_left), _expected_prefill(w, window_left), *tolerances("bf16"),
+                 what=f"window {window_left}")  # fmt: skip
+
+
+def test_prefill_many_sequences():
+    """More sequences than workgroup shares per kv head: most shares hold several whole query blocks."""
+    g = torch.Generator().manual_seed(24)
+    new = torch.randint(1, 40, (300,), generator=g)
+    ctx = torch.randint(0, 90, (300,), generator=g)
+    w = workloads.make_prefill_workload("many", seed=24, new_lens=new, ctx_lens=ctx, hq=8, hkv=8, d=64, bs=16,
+                                        kv="int8", device=DEV, quantize_fn=gpu_quantize)  # fmt: skip
+    assert_close(_run_prefill(w), _expected_prefill(w), *tolerances("int8"), what="many sequences")
+
+
+def test_prefill_c_abi_rejects_a_short_workspace():
+    from areno_amd.accel import cabi
+
+    w = workloads.cfg4_prefill("fp8", device=DEV, seqs=2, new_hi=8, ctx_hi=40, quantize_fn=gpu_quantize, seed=5)
+    cache = cabi.describe_cache(w.k_cache, w.v_cache, w.k_scale, w.v_scale)
+    need = cabi.prefill_workspace_bytes(w.k_cache.shape[2], w.k_cache.shape[3])
+    assert need > 0
+    out = torch.empty_like(w.q)
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+
+    def call(nbytes):
+        return cabi.paged_varlen_prefill(cache, w.q, out, w.block_table, w.cu_seqlens_q, w.context_lens, ws,
+                                         softmax_scale=w.softmax_scale, workspace_bytes=nbytes)  # fmt: skip
+
+    assert call(need - 1) == cabi.ERR_WORKSPACE
+    assert b"workspace" in cabi.lib().areno_hip_last_error()
+    assert call(need) == 0
+    torch.cuda.synchronize()
+    assert_close(out, _expected_prefill(w), *tolerances("fp8"), what="c abi prefill")
+
+
 def test_dense_causal_attention_wrapper():
     g = torch.Generator().manual_seed(1)
     q = torch.randn(2, 4, 9, 64, generator=g).bfloat16()
