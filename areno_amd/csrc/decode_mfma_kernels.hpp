@@ -456,11 +456,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
       }
       qop[sl] = __builtin_bit_cast(V8, w);
     }
-    if constexpr (KIND == KV_I8) {
-      qsum += wave_xor(qsum, 16);
-      qsum += wave_xor(qsum, 32);
-      qbias = kI8Offset * qsum;
-    }
+    if constexpr (KIND == KV_I8) qbias = kI8Offset * rows_sum(qsum);
   };
 
   float4_t acc[NB];
@@ -475,16 +471,9 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
 
   auto write_partial = [&](int b) {
     // combine the four k-groups' row sums; every lane of a head ends with the head's totals
-    float l_tot = l_run;
-    l_tot += wave_xor(l_tot, 16);
-    l_tot += wave_xor(l_tot, 32);
+    const float l_tot = rows_sum(l_run);
     float off = 0.0f;
-    if constexpr (KIND == KV_I8) {
-      float ps = p_sum;
-      ps += wave_xor(ps, 16);
-      ps += wave_xor(ps, 32);
-      off = kI8Offset * ps;
-    }
+    if constexpr (KIND == KV_I8) off = kI8Offset * rows_sum(p_sum);
     if (lr < p.group) {
       const int64_t prow = (static_cast<int64_t>(unit + b)) * p.q_heads + h0 + lr;
       float* dst = p.part_acc + prow * D + 4 * lk;
@@ -646,11 +635,10 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
         }
 
         // -- online softmax for head lr over the tile's 32 tokens ---------------------------------------------------
-        float mt = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
-                         fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
-        mt = fmaxf(mt, wave_xor(mt, 16));
-        mt = fmaxf(mt, wave_xor(mt, 32));
-        const float m_new = fmaxf(m_run, mt);
+        float mt = max3_f32(max3_f32(s[0][0], s[0][1], s[0][2]), max3_f32(s[0][3], s[1][0], s[1][1]),
+                            max_f32(s[1][2], s[1][3]));
+        mt = rows_max(mt);
+        const float m_new = max_f32(m_run, mt);
         const float m_safe = m_new == kNegInf ? 0.0f : m_new;
         const float alpha = fast_exp2(m_run - m_safe);
         m_run = m_new;

@@ -166,7 +166,8 @@ def measure_decode(w, steps, warmup, *, kernel_iters=60):
             samples.append(e0.elapsed_time(e1) * 1e3 / kernel_iters)
         return statistics.median(samples)
 
-    us_split = time_stage(cabi.STAGE_SPLIT)
+    # the op folds the append into the split kernel; the stand-alone append launch is timed for reference only
+    us_split = time_stage(cabi.STAGE_APPEND | cabi.STAGE_SPLIT)
     us_reduce = time_stage(cabi.STAGE_REDUCE)
     us_append = time_stage(cabi.STAGE_APPEND)
     torch.cuda.synchronize()
@@ -178,7 +179,7 @@ def measure_decode(w, steps, warmup, *, kernel_iters=60):
         "workload": w.name,
         "us_per_step": us_graph,
         "us_per_step_eager": us_eager,
-        "kernel_us": {"append": us_append, "split": us_split, "reduce": us_reduce},
+        "kernel_us": {"split_with_append": us_split, "reduce": us_reduce, "append_alone_not_in_op": us_append},
         "tokens_per_s": w.q.shape[0] / (us_graph * 1e-6),
         "algorithmic_bytes": alg_bytes,
         "op_gbps": alg_bytes / (us_graph * 1e-6) / 1e9,

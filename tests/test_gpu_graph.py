@@ -1,0 +1,101 @@
+"""HIP-graph contract of the decode op, as the reference engine uses it
+(areno/engine/runtime/decode_graph.py:127-175): captured once against static buffers, replayed every step after the
+live values were copied into them, with the unused rows of the bucket parked on a scratch block at length 0.
+
+Every replay is checked against an eager run of the same step on a second copy of the cache and against the CPU
+oracle, with eager work and synchronisations between the replays."""
+
+import pytest
+import torch
+
+from areno_amd import workloads
+from areno_amd.accel import attention as ops
+from oracle import attention_ref as ar
+from tests.gpu_util import DEV, assert_close, dequant_cpu, gpu_quantize, tolerances
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = [17, 100, 33, 250, 5]  # every row has room for four more tokens in its last page
+BUCKET = 8
+STEPS = 4
+
+
+def _decode(q, ku, vu, kc, vc, table, lens, ks, vs, scale):
+    return ops.areno_paged_causal_attention_decode(q, ku, vu, kc, vc, table, lens, num_splits=8, softmax_scale=scale,
+                                                   k_scale=ks, v_scale=vs)  # fmt: skip
+
+
+@pytest.mark.parametrize("kv,hq,hkv,d", [("bf16", 8, 2, 64), ("int8", 28, 4, 128), ("fp8", 8, 8, 128)])
+def test_decode_graph_replays_match_eager_and_oracle(kv, hq, hkv, d):
+    actual = len(LENGTHS)
+    w = workloads.make_decode_workload(
+        f"graph-{kv}", seed=31, batch=actual, hq=hq, hkv=hkv, d=d, bs=16, kv=kv, lengths=torch.tensor(LENGTHS),
+        device=DEV, quantize_fn=gpu_quantize, pool_slack=0.5,
+    )  # fmt: skip
+    used = set(w.block_table.cpu().flatten().tolist())
+    scratch = max(i for i in range(w.k_cache.shape[0]) if i not in used)
+    cols = w.block_table.shape[1] + 3  # the graph's table is wider than any live row needs
+
+    def clone_cache():
+        return tuple(None if t is None else t.clone() for t in (w.k_cache, w.v_cache, w.k_scale, w.v_scale))
+
+    g_kc, g_vc, g_ks, g_vs = clone_cache()  # cache the graph appends to
+    e_kc, e_vc, e_ks, e_vs = clone_cache()  # cache the eager runs append to
+
+    # ---- static buffers of the graph, parked rows on the scratch block --------------------------------------------
+    s_q = torch.zeros((BUCKET, hq, d), dtype=w.q.dtype, device=DEV)
+    s_ku = torch.zeros((BUCKET, hkv, d), dtype=w.q.dtype, device=DEV)
+    s_vu = torch.zeros_like(s_ku)
+    s_table = torch.full((BUCKET, cols), scratch, dtype=torch.int32, device=DEV)
+    s_lens = torch.zeros(BUCKET, dtype=torch.int32, device=DEV)
+
+    def run_static():
+        return _decode(s_q, s_ku, s_vu, g_kc, g_vc, s_table, s_lens, g_ks, g_vs, w.softmax_scale)
+
+    # warm-up on a side stream with everything parked (touches only the scratch block), then capture
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run_static()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        s_out = run_static()
+
+    gen = torch.Generator(device=DEV).manual_seed(77)
+    live_blocks = sorted(used)
+    for step in range(STEPS):
+        q = (torch.randn((actual, hq, d), generator=gen, device=DEV) * d**-0.25).to(w.q.dtype)
+        ku = torch.randn((actual, hkv, d), generator=gen, device=DEV).to(w.q.dtype)
+        vu = torch.randn((actual, hkv, d), generator=gen, device=DEV).to(w.q.dtype)
+        lens = (w.cache_seqlens + step).to(torch.int32)
+
+        # the engine's replay_tensors: copy the live step in, pad columns and rows with the scratch block
+        s_q[:actual].copy_(q)
+        s_ku[:actual].copy_(ku)
+        s_vu[:actual].copy_(vu)
+        s_lens[:actual].copy_(lens)
+        s_lens[actual:].fill_(0)
+        s_table[:actual, : w.block_table.shape[1]].copy_(w.block_table)
+        s_table[:actual, w.block_table.shape[1] :].fill_(scratch)
+        s_table[actual:].fill_(scratch)
+        graph.replay()
+
+        # eager work of the program between replays, on its own cache copy and without the padding
+        eager = _decode(q, ku, vu, e_kc, e_vc, w.block_table, lens, e_ks, e_vs, w.softmax_scale)
+        torch.cuda.synchronize()
+
+        got = s_out[:actual].clone()
+        kc, vc = dequant_cpu(g_kc, g_ks), dequant_cpu(g_vc, g_vs)
+        want = ar.ref_paged_decode(q.cpu().float(), kc, vc, w.block_table.cpu(), lens.cpu(), -1, w.softmax_scale)
+        assert_close(got, want, *tolerances(kv), what=f"replay {step} vs oracle")
+        assert_close(got, eager.cpu().float(), 2e-3, what=f"replay {step} vs eager")
+        # both caches received the same appended rows, bit for bit (the scratch block is not compared)
+        idx = torch.tensor(live_blocks, device=DEV)
+        for a, b, name in ((g_kc, e_kc, "k"), (g_vc, e_vc, "v"), (g_ks, e_ks, "k_scale"), (g_vs, e_vs, "v_scale")):
+            if a is None:
+                continue
+            ra, rb = a[idx].view(torch.uint8), b[idx].view(torch.uint8)
+            assert torch.equal(ra, rb), f"replay {step}: {name} pages differ between graph and eager"
+        assert torch.isfinite(s_out[actual:].float()).all(), "parked rows must stay finite"
