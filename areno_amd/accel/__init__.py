@@ -1,7 +1,8 @@
 """Paged / quantized KV-cache attention ops (the hot path of ``areno.accel`` in the reference).
 
 Re-exports the op surface the reference's inference backend imports
-(``areno/accel/__init__.py:17-21`` there) plus this build's two additions.
+(``areno/accel/__init__.py:17-21`` there) plus this build's additions (cache write, paged prefill, and the fused
+QK-norm + rotary + cache-write step in front of the path).
 """
 
 from areno_amd.accel.attention import (
@@ -9,6 +10,7 @@ from areno_amd.accel.attention import (
     areno_paged_cache_write,
     areno_paged_causal_attention_decode,
     areno_paged_varlen_causal_attention,
+    areno_qk_norm_rope_cache_write,
     areno_varlen_causal_attention,
 )
 
@@ -17,5 +19,6 @@ __all__ = [
     "areno_paged_cache_write",
     "areno_paged_causal_attention_decode",
     "areno_paged_varlen_causal_attention",
+    "areno_qk_norm_rope_cache_write",
     "areno_varlen_causal_attention",
 ]

@@ -263,3 +263,56 @@ def areno_paged_varlen_causal_attention(
         cu_seqlens_q.contiguous(), context_lens.contiguous(), _window_left(window_left), _scale(q, softmax_scale),
         _contig(k_scale), _contig(v_scale),
     )  # fmt: skip
+
+
+@torch._dynamo.disable
+def areno_qk_norm_rope_cache_write(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    position_ids: torch.Tensor,
+    cos_cached: torch.Tensor,
+    sin_cached: torch.Tensor,
+    *,
+    q_norm_weight: torch.Tensor | None = None,
+    k_norm_weight: torch.Tensor | None = None,
+    eps: float = 1e-6,
+    k_cache: torch.Tensor | None = None,
+    v_cache: torch.Tensor | None = None,
+    cache_block_ids: torch.Tensor | None = None,
+    cache_block_offsets: torch.Tensor | None = None,
+    k_scale: torch.Tensor | None = None,
+    v_scale: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """The layer's steps in front of attention in one kernel: ``q_norm`` / ``k_norm`` (per-head RMSNorm, fp32
+    weights), rotary embedding from the ``(max_position, head_dim)`` float32 tables of ``RotaryEmbedding``, and,
+    when caches are given, the quantizing scatter of the new K/V rows to ``cache[ids[t], offsets[t]]``.
+
+    ``q (T, Hq, D)``, ``k`` / ``v (T, Hkv, D)`` fp16 or bf16; returns ``(q, k)`` after norm and rotary.  The pages
+    receive exactly what ``areno_paged_cache_write(k_out, v, ...)`` would store.
+    """
+    op = "areno_qk_norm_rope_cache_write"
+    tensors = (q, k, v, position_ids, cos_cached, sin_cached, q_norm_weight, k_norm_weight, k_cache, v_cache,
+               cache_block_ids, cache_block_offsets, k_scale, v_scale)  # fmt: skip
+    if not _all_on_gpu(*tensors):
+        raise RuntimeError(f"{op} requires CUDA tensors")
+    if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
+        raise ValueError(f"{op} expects q/k/v shaped (tokens, heads, head_dim)")
+    if q.dtype not in (torch.float16, torch.bfloat16) or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError(f"{op} expects fp16 or bf16 q/k/v of one dtype")
+    if (k_cache is None) != (v_cache is None):
+        raise ValueError(f"{op} expects k_cache and v_cache together")
+    if k_cache is not None:
+        if cache_block_ids is None or cache_block_offsets is None:
+            raise ValueError(f"{op} expects cache_block_ids and cache_block_offsets with the caches")
+        _check_scales(op, k_cache, k_scale, v_scale)
+        if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+            raise ValueError(f"{op} expects contiguous cache tensors (they are updated in place)")
+    q_out, k_out = _extension().areno_qk_norm_rope_cache_write(
+        q.contiguous(), k.contiguous(), v.contiguous(), position_ids.reshape(-1).to(torch.int64).contiguous(),
+        cos_cached.to(torch.float32).contiguous(), sin_cached.to(torch.float32).contiguous(),
+        None if q_norm_weight is None else q_norm_weight.to(torch.float32).contiguous(),
+        None if k_norm_weight is None else k_norm_weight.to(torch.float32).contiguous(),
+        float(eps), k_cache, v_cache, _contig(cache_block_ids), _contig(cache_block_offsets), k_scale, v_scale,
+    )  # fmt: skip
+    return q_out, k_out

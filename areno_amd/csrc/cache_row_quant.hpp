@@ -1,0 +1,68 @@
+// Per-row KV quantizer shared by the cache writers: one wave64 holds a (token, kv head) row as floats, element
+// idx = lane + 64 e in x[e]; the row's abs-max gives its scale, codes and scale go to the paged address.
+//
+// Closed forms (bit-exact contract; IEEE fp32 division, round half to even):
+//   int8: s = fp16(min(absmax / 127, 65504)); s == 0 -> 1; code = clamp(rint(x / float(s)), -127, 127)
+//   fp8 : s = absmax / 448 (fp32);            s == 0 -> 1; code = e4m3fn(clamp(x / s, -448, 448))
+#pragma once
+
+#include "device_common.hpp"
+
+namespace areno {
+
+constexpr int kMaxPerLane = 8;  // head_dim <= 512
+
+__host__ __device__ inline bool is_quantized_dtype(int dtype) {
+  return dtype == ARENO_DT_I8 || dtype == ARENO_DT_FP8_E4M3;
+}
+
+__device__ __forceinline__ void quantize_store_row(const float (&x)[kMaxPerLane], int lane, int d, int64_t dst_row,
+                                                   void* cache, void* scale, int cache_dtype, int scale_dtype) {
+  const int64_t dst_base = dst_row * d;
+  float amax = 0.0f;
+#pragma unroll
+  for (int e = 0; e < kMaxPerLane; ++e) amax = fmaxf(amax, fabsf(x[e]));
+  amax = wave_max(amax);
+  if (cache_dtype == ARENO_DT_I8) {
+    const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
+    const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
+    const float s = static_cast<float>(s16_fixed);
+    int8_t* out = static_cast<int8_t*>(cache);
+#pragma unroll
+    for (int e = 0; e < kMaxPerLane; ++e) {
+      const int idx = lane + e * kWave;
+      if (idx < d) {
+        const float code = fminf(fmaxf(rintf(x[e] / s), -127.0f), 127.0f);
+        out[dst_base + idx] = static_cast<int8_t>(static_cast<int>(code));
+      }
+    }
+    if (lane == 0) {
+      if (scale_dtype == ARENO_DT_F16) {
+        static_cast<uint16_t*>(scale)[dst_row] = __builtin_bit_cast(uint16_t, s16_fixed);
+      } else {
+        static_cast<float*>(scale)[dst_row] = s;
+      }
+    }
+  } else {
+    float s = amax / 448.0f;
+    if (s == 0.0f) s = 1.0f;
+    uint8_t* out = static_cast<uint8_t*>(cache);
+#pragma unroll
+    for (int e = 0; e < kMaxPerLane; ++e) {
+      const int idx = lane + e * kWave;
+      if (idx < d) {
+        const float y = fminf(fmaxf(x[e] / s, -448.0f), 448.0f);
+        out[dst_base + idx] = static_cast<uint8_t>(float_to_fp8_byte(y));
+      }
+    }
+    if (lane == 0) {
+      if (scale_dtype == ARENO_DT_F16) {
+        static_cast<uint16_t*>(scale)[dst_row] = static_cast<uint16_t>(float_to_f16_bits(s));
+      } else {
+        static_cast<float*>(scale)[dst_row] = s;
+      }
+    }
+  }
+}
+
+}  // namespace areno

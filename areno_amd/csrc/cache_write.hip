@@ -15,7 +15,7 @@
 // The work is launch-latency bound for decode (B * Hkv rows) and a plain streaming copy for
 // prefill; no LDS is needed.
 
-#include "device_common.hpp"
+#include "cache_row_quant.hpp"
 
 namespace areno {
 namespace {
@@ -40,7 +40,6 @@ struct WriteParams {
 };
 
 constexpr int kRowsPerBlock = 4;  // one wave per row
-constexpr int kMaxPerLane = 8;    // head_dim <= 512
 
 __global__ __launch_bounds__(kRowsPerBlock* kWave) void cache_write_kernel(WriteParams p) {
   const int lane = threadIdx.x & (kWave - 1);
@@ -71,55 +70,14 @@ __global__ __launch_bounds__(kRowsPerBlock* kWave) void cache_write_kernel(Write
   void* dst = p.cache[which];
 
   float x[kMaxPerLane];
-  float amax = 0.0f;
 #pragma unroll
   for (int e = 0; e < kMaxPerLane; ++e) {
     const int idx = lane + e * kWave;
     x[e] = idx < d ? load_as_float(src, src_base + idx, p.in_dtype) : 0.0f;
-    amax = fmaxf(amax, fabsf(x[e]));
   }
 
-  if (p.cache_dtype == ARENO_DT_I8) {
-    amax = wave_max(amax);
-    const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
-    const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
-    const float s = static_cast<float>(s16_fixed);
-    int8_t* out = static_cast<int8_t*>(dst);
-#pragma unroll
-    for (int e = 0; e < kMaxPerLane; ++e) {
-      const int idx = lane + e * kWave;
-      if (idx < d) {
-        const float code = fminf(fmaxf(rintf(x[e] / s), -127.0f), 127.0f);
-        out[dst_base + idx] = static_cast<int8_t>(static_cast<int>(code));
-      }
-    }
-    if (lane == 0) {
-      if (p.scale_dtype == ARENO_DT_F16) {
-        static_cast<uint16_t*>(p.scale[which])[dst_row] = __builtin_bit_cast(uint16_t, s16_fixed);
-      } else {
-        static_cast<float*>(p.scale[which])[dst_row] = s;
-      }
-    }
-  } else if (p.cache_dtype == ARENO_DT_FP8_E4M3) {
-    amax = wave_max(amax);
-    float s = amax / 448.0f;
-    if (s == 0.0f) s = 1.0f;
-    uint8_t* out = static_cast<uint8_t*>(dst);
-#pragma unroll
-    for (int e = 0; e < kMaxPerLane; ++e) {
-      const int idx = lane + e * kWave;
-      if (idx < d) {
-        const float y = fminf(fmaxf(x[e] / s, -448.0f), 448.0f);
-        out[dst_base + idx] = static_cast<uint8_t>(float_to_fp8_byte(y));
-      }
-    }
-    if (lane == 0) {
-      if (p.scale_dtype == ARENO_DT_F16) {
-        static_cast<uint16_t*>(p.scale[which])[dst_row] = static_cast<uint16_t>(float_to_f16_bits(s));
-      } else {
-        static_cast<float*>(p.scale[which])[dst_row] = s;
-      }
-    }
+  if (is_quantized_dtype(p.cache_dtype)) {
+    quantize_store_row(x, lane, d, dst_row, dst, p.scale[which], p.cache_dtype, p.scale_dtype);
   } else {
     // same-dtype copy: move raw bits so the stored row is bit-identical to the input row
     if (p.cache_dtype == ARENO_DT_F32) {

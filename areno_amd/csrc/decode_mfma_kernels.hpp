@@ -230,8 +230,12 @@ struct TileCursor {
   int next_end;  // same for sequence b + 1, fetched one sequence ahead
 };
 
+#ifndef ARENO_MFMA_QUANT_OCC
+#define ARENO_MFMA_QUANT_OCC 2
+#endif
 template <int KIND, int D, bool SCALE16, int NW>
-__global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodeParams mp) {
+__global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUANT_OCC : 2) void decode_mfma_kernel(
+    MfmaDecodeParams mp) {
   using T = KVTraits<KIND>;
   using Ops = MfmaOps<KIND>;
   using V8 = typename Ops::vec8;

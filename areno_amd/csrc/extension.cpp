@@ -250,6 +250,68 @@ at::Tensor paged_varlen_forward(at::Tensor q, at::Tensor k_cache, at::Tensor v_c
   return out;
 }
 
+std::vector<at::Tensor> qk_norm_rope_cache_write(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor positions,
+                                                 at::Tensor cos, at::Tensor sin, c10::optional<at::Tensor> q_weight,
+                                                 c10::optional<at::Tensor> k_weight, double eps,
+                                                 c10::optional<at::Tensor> k_cache, c10::optional<at::Tensor> v_cache,
+                                                 c10::optional<at::Tensor> block_ids,
+                                                 c10::optional<at::Tensor> block_offsets,
+                                                 c10::optional<at::Tensor> k_scale, c10::optional<at::Tensor> v_scale) {
+  const char* op = "areno_qk_norm_rope_cache_write";
+  TORCH_CHECK(q.is_cuda() && k.is_cuda() && v.is_cuda() && positions.is_cuda() && cos.is_cuda() && sin.is_cuda(), op,
+              " tensors must be CUDA");
+  TORCH_CHECK(q.is_contiguous() && k.is_contiguous() && v.is_contiguous() && positions.is_contiguous() &&
+                  cos.is_contiguous() && sin.is_contiguous(),
+              op, " tensors must be contiguous");
+  TORCH_CHECK(q.dim() == 3 && k.dim() == 3 && v.dim() == 3, op, " expects q/k/v shaped (tokens, heads, head_dim)");
+  TORCH_CHECK(q.scalar_type() == k.scalar_type() && q.scalar_type() == v.scalar_type(), op, " dtype mismatch");
+  TORCH_CHECK(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, op, " q/k/v must be fp16 or bf16");
+  TORCH_CHECK(k.sizes() == v.sizes(), op, " k/v shape mismatch");
+  TORCH_CHECK(q.size(0) == k.size(0) && q.size(2) == k.size(2), op, " q and k/v disagree on tokens or head_dim");
+  TORCH_CHECK(positions.dim() == 1 && positions.size(0) == q.size(0) && positions.scalar_type() == at::kLong, op,
+              " positions must be int64 (tokens,)");
+  TORCH_CHECK(cos.dim() == 2 && cos.sizes() == sin.sizes() && cos.size(1) == q.size(2) &&
+                  cos.scalar_type() == at::kFloat && sin.scalar_type() == at::kFloat,
+              op, " cos/sin must be float32 (max_position, head_dim)");
+  auto weight_ptr = [&](const c10::optional<at::Tensor>& w, const char* name) -> const float* {
+    if (!w.has_value()) return nullptr;
+    TORCH_CHECK(w->is_cuda() && w->is_contiguous() && w->scalar_type() == at::kFloat && w->dim() == 1 &&
+                    w->size(0) == q.size(2),
+                op, " ", name, " must be a CUDA float32 (head_dim,) tensor");
+    return w->data_ptr<float>();
+  };
+  const float* qw = weight_ptr(q_weight, "q_weight");
+  const float* kw = weight_ptr(k_weight, "k_weight");
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(q));
+  auto q_out = at::empty_like(q);
+  auto k_out = at::empty_like(k);
+  areno_paged_cache cache = {};
+  const areno_paged_cache* cache_ptr = nullptr;
+  const int64_t* ids = nullptr;
+  const int64_t* offs = nullptr;
+  if (k_cache.has_value()) {
+    TORCH_CHECK(v_cache.has_value() && block_ids.has_value() && block_offsets.has_value(), op,
+                " a cache write needs v_cache, cache_block_ids and cache_block_offsets");
+    cache = describe_cache(*k_cache, *v_cache, k_scale, v_scale, op);
+    TORCH_CHECK(block_ids->is_cuda() && block_offsets->is_cuda() && block_ids->is_contiguous() &&
+                    block_offsets->is_contiguous() && block_ids->scalar_type() == at::kLong &&
+                    block_offsets->scalar_type() == at::kLong && block_ids->dim() == 1 &&
+                    block_ids->size(0) == q.size(0) && block_offsets->sizes() == block_ids->sizes(),
+                op, " block ids/offsets must be int64 (tokens,)");
+    TORCH_CHECK(k.size(1) == k_cache->size(2) && k.size(2) == k_cache->size(3), op, " cache geometry mismatch");
+    cache_ptr = &cache;
+    ids = block_ids->data_ptr<int64_t>();
+    offs = block_offsets->data_ptr<int64_t>();
+  }
+  const int status = areno_hip_qk_norm_rope_cache_write(
+      cache_ptr, q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(), k_out.data_ptr(), dtype_code(q, op, "q"),
+      q.size(0), static_cast<int32_t>(q.size(1)), static_cast<int32_t>(k.size(1)), static_cast<int32_t>(q.size(2)),
+      positions.data_ptr<int64_t>(), cos.data_ptr<float>(), sin.data_ptr<float>(), static_cast<int32_t>(cos.size(0)), qw,
+      kw, static_cast<float>(eps), ids, offs, current_stream(q));
+  check_status(status, op);
+  return {q_out, k_out};
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -261,5 +323,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("areno_paged_cache_write", &cache_write, "quantize-and-scatter KV cache write");
   m.def("areno_paged_varlen_causal_attention_forward", &paged_varlen_forward,
         "causal varlen prefill over paged (optionally quantized) KV");
+  m.def("areno_qk_norm_rope_cache_write", &qk_norm_rope_cache_write,
+        "QK RMSNorm + rotary embedding + quantizing KV cache write in one pass");
   m.def("abi_version", &areno_hip_abi_version, "C ABI version of libareno_hip.so");
 }

@@ -392,7 +392,7 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
     const int head_groups = cache->kv_heads / p.heads_per_wg;
     static const int wgs = [] {
       const int v = env_int("ARENO_MFMA_WGS", kMfmaWorkgroups);
-      return v > 0 && v <= kMfmaWorkgroups ? v : kMfmaWorkgroups;
+      return v > 0 && v <= kMfmaWorkgroups + kMfmaTailWorkgroups ? v : kMfmaWorkgroups;
     }();
     static const int tail_wgs = [] {
       const int v = env_int("ARENO_MFMA_TAIL_WGS", 0);

@@ -1,0 +1,297 @@
+// The step in front of the attention path, fused: per-head QK RMSNorm, rotary embedding and the quantizing scatter of
+// the new K/V rows into the paged cache, in one pass over the projection output.
+//
+// Reference (one op each, every one a full read and write of its tensor):
+//   q = q_norm(q); k = k_norm(k)          areno/engine/layers/attention.py:90-93, kernel
+//                                          areno/accel/csrc/normalization.cu:34-56:
+//                                          y = dtype(x * rsqrt(mean(x^2) + eps) * w), fp32 arithmetic
+//   q, k = rope(q, k, position_ids)       areno/engine/layers/rotary.py:46-52 (rotate_half pairs i with i + D/2):
+//                                          dtype(dtype(y * cos) + dtype(rotate_half(y) * sin)) with the fp32 tables
+//                                          cast to the activation dtype first -- every product and the sum are
+//                                          rounded to the activation dtype, as the eager tensor ops do
+//   k_cache[ids, offs] = k; v_cache[...] = v   areno/engine/layers/attention_backend/infer.py:245-263
+//
+// A (token, head) row is a q head (norm + rope -> q_out), a k head (norm + rope -> k_out and the page) or a v head
+// (-> the page).  D / 8 adjacent lanes hold a row, 16 bytes each, so a wave64 carries 64 / (D / 8) rows and every
+// global access is 16 bytes wide; the rotary partner i +- D/2 is the same slot of the lane D/16 away.  The cache rows
+// use the closed forms of areno_hip_cache_write's quantizer, so the pages hold exactly quantize(k_out) and
+// quantize(v).  Bound: HBM streaming, T * (Hq + 2 Hkv) * D elements in, T * (Hq + Hkv) * D out plus the pages.
+
+#include "cache_row_quant.hpp"
+
+namespace areno {
+
+int validate_paged_cache(const areno_paged_cache* c, const char* op);
+
+namespace {
+
+struct RopeWriteParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* q_out;
+  void* k_out;  // may be null
+  const float* q_weight;  // [D] or null: no norm on q
+  const float* k_weight;  // [D] or null: no norm on k
+  const float* cos;       // [max_pos, D]
+  const float* sin;
+  const int64_t* positions;  // [tokens]
+  void* cache[2];            // k, v pools; null pools: no cache write
+  void* scale[2];
+  const int64_t* block_ids;
+  const int64_t* block_offsets;
+  int64_t tokens;
+  int64_t num_blocks;
+  int32_t block_size;
+  int32_t q_heads;
+  int32_t kv_heads;
+  int32_t head_dim;
+  int32_t max_pos;
+  int32_t dtype;  // activation dtype: F16 or BF16
+  int32_t cache_dtype;
+  int32_t scale_dtype;
+  float eps;
+};
+
+// x rounded to the activation dtype, as float
+__device__ __forceinline__ float round_to(float x, int dtype) {
+  return dtype == ARENO_DT_BF16 ? bf16_bits_to_float(float_to_bf16_bits(x)) : f16_bits_to_float(float_to_f16_bits(x));
+}
+
+__device__ __forceinline__ uint32_t pack_two(float lo, float hi, int dtype) {
+  return dtype == ARENO_DT_BF16 ? (float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16))
+                                : (float_to_f16_bits(lo) | (float_to_f16_bits(hi) << 16));
+}
+
+// Row layout: a row of D elements is held by LPR = D / 8 adjacent lanes, 8 consecutive elements (16 bytes of 16-bit
+// activations) per lane, so a wave64 carries 64 / LPR rows and every global access is a 16-byte one.  The rotary
+// partner of element i (i +- D/2) is the same element slot of lane ^ (LPR / 2).
+template <int LPR>
+__device__ __forceinline__ float group_sum(float x) {
+#pragma unroll
+  for (int m = 1; m < LPR; m <<= 1) x += wave_xor(x, m);
+  return x;
+}
+template <int LPR>
+__device__ __forceinline__ float group_max(float x) {
+#pragma unroll
+  for (int m = 1; m < LPR; m <<= 1) x = fmaxf(x, wave_xor(x, m));
+  return x;
+}
+
+template <int LPR>
+__global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
+  constexpr int D = LPR * 8;
+  constexpr int kRowsPerWave = kWave / LPR;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int sub = lane % LPR;  // which 8 elements of the row
+  const int heads = p.q_heads + 2 * p.kv_heads;
+  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + (threadIdx.x >> 6);
+  const int64_t total = p.tokens * heads;
+  const int64_t row_raw = wave_id * kRowsPerWave + lane / LPR;
+  const bool live = row_raw < total;
+  const int64_t row = live ? row_raw : total - 1;  // idle lane groups shadow the last row and store nothing
+  const int64_t token = row / heads;
+  const int slot = static_cast<int>(row - token * heads);
+  const int kind = slot < p.q_heads ? 0 : (slot < p.q_heads + p.kv_heads ? 1 : 2);  // q, k, v
+  const int head = kind == 0 ? slot : (kind == 1 ? slot - p.q_heads : slot - p.q_heads - p.kv_heads);
+  const void* src = kind == 0 ? p.q : (kind == 1 ? p.k : p.v);
+  const int src_heads = kind == 0 ? p.q_heads : p.kv_heads;
+  const int64_t src_base = (token * src_heads + head) * D + sub * 8;
+
+  float x[8];
+  {
+    const uint4_t raw = *reinterpret_cast<const uint4_t*>(static_cast<const char*>(src) + src_base * 2);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t word = raw[j];
+      if (p.dtype == ARENO_DT_BF16) {
+        x[2 * j] = bf16_bits_to_float(word & 0xffffu);
+        x[2 * j + 1] = bf16_bits_to_float(word >> 16);
+      } else {
+        x[2 * j] = f16_bits_to_float(word & 0xffffu);
+        x[2 * j + 1] = f16_bits_to_float(word >> 16);
+      }
+    }
+  }
+
+  // ---- q and k rows: norm and rotary (the selects keep every lane in the cross-lane steps) ------------------------
+  const float* weight = kind == 0 ? p.q_weight : (kind == 1 ? p.k_weight : nullptr);
+  {
+    float sum_sq = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sum_sq += x[j] * x[j];
+    sum_sq = group_sum<LPR>(sum_sq);
+    if (weight != nullptr) {
+      const float inv = rsqrtf(sum_sq / static_cast<float>(D) + p.eps);
+      const float4_t w0 = *reinterpret_cast<const float4_t*>(weight + sub * 8);
+      const float4_t w1 = *reinterpret_cast<const float4_t*>(weight + sub * 8 + 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[j] = round_to(x[j] * inv * w0[j], p.dtype);
+        x[4 + j] = round_to(x[4 + j] * inv * w1[j], p.dtype);
+      }
+    }
+  }
+  float partner[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) partner[j] = wave_xor(x[j], LPR / 2);
+  if (kind != 2) {
+    int64_t pos = p.positions[token];
+    pos = pos < 0 ? 0 : (pos >= p.max_pos ? p.max_pos - 1 : pos);
+    const float* cos_row = p.cos + pos * D + sub * 8;
+    const float* sin_row = p.sin + pos * D + sub * 8;
+    const float4_t c0 = *reinterpret_cast<const float4_t*>(cos_row);
+    const float4_t c1 = *reinterpret_cast<const float4_t*>(cos_row + 4);
+    const float4_t s0 = *reinterpret_cast<const float4_t*>(sin_row);
+    const float4_t s1 = *reinterpret_cast<const float4_t*>(sin_row + 4);
+    const bool low_half = sub < LPR / 2;  // rotate_half: -x[i + D/2] below D/2, x[i - D/2] above
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float c = round_to(j < 4 ? c0[j & 3] : c1[j & 3], p.dtype);
+      const float sn = round_to(j < 4 ? s0[j & 3] : s1[j & 3], p.dtype);
+      const float rot = low_half ? -partner[j] : partner[j];
+      x[j] = round_to(round_to(x[j] * c, p.dtype) + round_to(rot * sn, p.dtype), p.dtype);
+    }
+    void* out = kind == 0 ? p.q_out : p.k_out;
+    if (out != nullptr && live) {
+      const uint4_t packed = {pack_two(x[0], x[1], p.dtype), pack_two(x[2], x[3], p.dtype),
+                              pack_two(x[4], x[5], p.dtype), pack_two(x[6], x[7], p.dtype)};
+      *reinterpret_cast<uint4_t*>(static_cast<char*>(out) + src_base * 2) = packed;
+    }
+  }
+
+  // ---- k and v rows: into the page, through the cache writer's quantizer ------------------------------------------
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(x[j]));
+  amax = group_max<LPR>(amax);
+  if (kind == 0 || !live) return;
+  void* cache = p.cache[kind - 1];
+  if (cache == nullptr) return;
+  const int64_t blk = p.block_ids[token];
+  const int64_t off = p.block_offsets[token];
+  if (blk < 0 || blk >= p.num_blocks || off < 0 || off >= p.block_size) return;
+  const int64_t dst_row = (blk * p.block_size + off) * p.kv_heads + head;
+  const int64_t dst_elem = dst_row * D + sub * 8;
+  if (p.cache_dtype == ARENO_DT_I8) {
+    const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
+    const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
+    const float s = static_cast<float>(s16_fixed);
+    uint32_t words[2] = {0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float code = fminf(fmaxf(rintf(x[j] / s), -127.0f), 127.0f);
+      words[j / 4] |= (static_cast<uint32_t>(static_cast<int>(code)) & 0xffu) << (8 * (j & 3));
+    }
+    *reinterpret_cast<uint2_t*>(static_cast<char*>(cache) + dst_elem) = uint2_t{words[0], words[1]};
+    if (sub == 0) {
+      if (p.scale_dtype == ARENO_DT_F16) {
+        static_cast<uint16_t*>(p.scale[kind - 1])[dst_row] = __builtin_bit_cast(uint16_t, s16_fixed);
+      } else {
+        static_cast<float*>(p.scale[kind - 1])[dst_row] = s;
+      }
+    }
+  } else if (p.cache_dtype == ARENO_DT_FP8_E4M3) {
+    float s = amax / 448.0f;
+    if (s == 0.0f) s = 1.0f;
+    uint32_t words[2] = {0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float y = fminf(fmaxf(x[j] / s, -448.0f), 448.0f);
+      words[j / 4] |= float_to_fp8_byte(y) << (8 * (j & 3));
+    }
+    *reinterpret_cast<uint2_t*>(static_cast<char*>(cache) + dst_elem) = uint2_t{words[0], words[1]};
+    if (sub == 0) {
+      if (p.scale_dtype == ARENO_DT_F16) {
+        static_cast<uint16_t*>(p.scale[kind - 1])[dst_row] = static_cast<uint16_t>(float_to_f16_bits(s));
+      } else {
+        static_cast<float*>(p.scale[kind - 1])[dst_row] = s;
+      }
+    }
+  } else {
+    const uint4_t packed = {pack_two(x[0], x[1], p.cache_dtype), pack_two(x[2], x[3], p.cache_dtype),
+                            pack_two(x[4], x[5], p.cache_dtype), pack_two(x[6], x[7], p.cache_dtype)};
+    *reinterpret_cast<uint4_t*>(static_cast<char*>(cache) + dst_elem * 2) = packed;
+  }
+}
+
+typedef void (*rope_write_fn)(RopeWriteParams);
+rope_write_fn rope_write_lookup(int head_dim) {
+  switch (head_dim) {
+    case 64: return qk_rope_write_kernel<8>;
+    case 128: return qk_rope_write_kernel<16>;
+    case 256: return qk_rope_write_kernel<32>;
+    case 512: return qk_rope_write_kernel<64>;
+    default: return nullptr;
+  }
+}
+
+}  // namespace
+}  // namespace areno
+
+extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache, const void* q, const void* k,
+                                                  const void* v, void* q_out, void* k_out, int32_t dtype,
+                                                  int64_t tokens, int32_t q_heads, int32_t kv_heads, int32_t head_dim,
+                                                  const int64_t* positions, const float* cos, const float* sin,
+                                                  int32_t max_pos, const float* q_weight, const float* k_weight,
+                                                  float eps, const int64_t* block_ids, const int64_t* block_offsets,
+                                                  void* stream) {
+  using namespace areno;
+  const char* op = "areno_hip_qk_norm_rope_cache_write";
+  if (dtype != ARENO_DT_F16 && dtype != ARENO_DT_BF16)
+    return fail(ARENO_ERR_UNSUPPORTED, "%s: activations must be f16 or bf16", op);
+  if (tokens < 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || max_pos <= 0)
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: sizes out of range", op);
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256 && head_dim != 512)
+    return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim must be 64, 128, 256 or 512, got %d", op, head_dim);
+  if (tokens == 0) return ARENO_OK;
+  if (q == nullptr || k == nullptr || v == nullptr || q_out == nullptr || positions == nullptr || cos == nullptr ||
+      sin == nullptr)
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", op);
+  RopeWriteParams p = {};
+  if (cache != nullptr) {
+    if (int rc = validate_paged_cache(cache, op)) return rc;
+    if (cache->kv_heads != kv_heads || cache->head_dim != head_dim)
+      return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: cache geometry does not match k/v", op);
+    if (!is_quantized_dtype(cache->cache_dtype) && cache->cache_dtype != dtype)
+      return fail(ARENO_ERR_UNSUPPORTED, "%s: activation dtype must equal an unquantized cache's dtype", op);
+    if (block_ids == nullptr || block_offsets == nullptr)
+      return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: block_ids/block_offsets is NULL", op);
+    p.cache[0] = cache->k;
+    p.cache[1] = cache->v;
+    p.scale[0] = cache->k_scale;
+    p.scale[1] = cache->v_scale;
+    p.num_blocks = cache->num_blocks;
+    p.block_size = cache->block_size;
+    p.cache_dtype = cache->cache_dtype;
+    p.scale_dtype = cache->scale_dtype;
+  }
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.q_out = q_out;
+  p.k_out = k_out;
+  p.q_weight = q_weight;
+  p.k_weight = k_weight;
+  p.cos = cos;
+  p.sin = sin;
+  p.positions = positions;
+  p.block_ids = block_ids;
+  p.block_offsets = block_offsets;
+  p.tokens = tokens;
+  p.q_heads = q_heads;
+  p.kv_heads = kv_heads;
+  p.head_dim = head_dim;
+  p.max_pos = max_pos;
+  p.dtype = dtype;
+  p.eps = eps;
+  const rope_write_fn fn = rope_write_lookup(head_dim);
+  if (fn == nullptr) return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim must be 64, 128, 256 or 512, got %d", op, head_dim);
+  const int64_t rows = tokens * (q_heads + 2 * kv_heads);
+  const int rows_per_block = 4 * (kWave / (head_dim / 8));
+  const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+  if (blocks > 0x7fffffffLL) return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: too many rows", op);
+  hipLaunchKernelGGL(fn, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+  return check_launch(op);
+}

@@ -289,7 +289,7 @@ def cfg1_qwen7b(kv: str = "bf16", *, device="cpu", seed: int = 1001, batch: int 
     lengths = _randint(g, ctx_lo, ctx_hi, batch)
     outliers = 0.01 if kv in SCALE_DTYPES else 0.0
     return make_decode_workload(
-        f"cfg{2 if kv == 'int8' else 1}-qwen7b-{kv}", seed=seed, batch=batch, hq=28, hkv=4, d=128, bs=16, kv=kv,
+        f"cfg{2 if kv == 'int8' else 1}-qwen7b-{kv}" + ("" if batch == 64 else f"-b{batch}"), seed=seed, batch=batch, hq=28, hkv=4, d=128, bs=16, kv=kv,
         lengths=lengths, device=device, outlier_frac=outliers, table_cols=(ctx_hi + 1 + 15) // 16, **kw,
     )  # fmt: skip
 

@@ -213,7 +213,8 @@ def measure_prefill(w, iters=20):
             softmax_scale=w.softmax_scale, k_scale=w.k_scale, v_scale=w.v_scale,
         )  # fmt: skip
 
-    def timed(fn):
+    def timed(fn, inner=1):
+        """Median over `iters` samples of `inner` back-to-back calls (short ops: the queue stays ahead of the GPU)."""
         for _ in range(3):
             fn()
         torch.cuda.synchronize()
@@ -221,20 +222,48 @@ def measure_prefill(w, iters=20):
         for _ in range(iters):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            fn()
+            for _ in range(inner):
+                fn()
             e1.record()
             e1.synchronize()
-            samples.append(e0.elapsed_time(e1) * 1e3)
+            samples.append(e0.elapsed_time(e1) * 1e3 / inner)
         return statistics.median(samples)
 
-    us_write = timed(write)
+    us_write = timed(write, inner=20)
     us_attend = timed(attend)
+
+    # the fused step in front of the path at the same shape: QK RMSNorm + rotary + quantizing write of the new rows
+    t, hq, d = w.q.shape
+    hkv = w.k_new.shape[1]
+    gen = torch.Generator(device=w.q.device).manual_seed(5)
+    inv_freq = 1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    emb = torch.outer(torch.arange(32768, dtype=torch.float32), inv_freq)
+    cos, sin = (torch.cat((f, f), dim=-1).to(w.q.device) for f in (emb.cos(), emb.sin()))
+    positions = torch.randint(0, 32768, (t,), generator=gen, device=w.q.device)
+    ones = torch.ones(d, device=w.q.device)
+
+    def front():
+        return ops.areno_qk_norm_rope_cache_write(
+            w.q, w.k_new, w.v_new, positions, cos, sin, q_norm_weight=ones, k_norm_weight=ones, eps=1e-6,
+            k_cache=w.k_cache, v_cache=w.v_cache, cache_block_ids=w.cache_block_ids,
+            cache_block_offsets=w.cache_block_offsets, k_scale=w.k_scale, v_scale=w.v_scale,
+        )  # fmt: skip
+
+    us_front = timed(front, inner=20)
+    act = w.q.element_size()
+    scale_bytes = 0 if w.k_scale is None else 2 * w.k_scale.element_size()
+    front_bytes = t * ((hq + 2 * hkv) * d * act + (hq + hkv) * d * act + hkv * (2 * d * w.k_cache.element_size() + scale_bytes))
+    write()  # leave the pages as the attention measurement expects them
     flops = w.flops()
     tflops = flops / (us_attend * 1e-6) / 1e12
     return {
         "workload": w.name,
         "us_per_step": us_attend + us_write,
-        "kernel_us": {"cache_write": us_write, "prefill": us_attend},
+        "kernel_us": {"cache_write": us_write, "prefill": us_attend, "qk_norm_rope_cache_write": us_front},
+        "qk_norm_rope_cache_write": {
+            "us": us_front, "algorithmic_bytes": front_bytes, "gbps": front_bytes / (us_front * 1e-6) / 1e9,
+            "frac_of_hbm_peak": front_bytes / (us_front * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+        },  # fmt: skip
         "new_tokens": int(w.q.shape[0]),
         "tokens_per_s": w.q.shape[0] / ((us_attend + us_write) * 1e-6),
         "flops": flops,
@@ -283,7 +312,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4"], default=None, help="measure a single workload")
+    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg2_b256"], default=None,
+                    help="measure a single workload")  # fmt: skip
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -309,8 +339,11 @@ def main() -> int:
         "cfg2": lambda: workloads.cfg2_qwen7b_int8(device=dev, quantize_fn=_gpu_quantize),
         "cfg3": lambda: workloads.cfg3_rollout("fp8", device=dev, quantize_fn=_gpu_quantize),
         "cfg4": lambda: workloads.cfg4_prefill("fp8", device=dev, quantize_fn=_gpu_quantize),
+        # not a configuration of the benchmark: cfg 2 at four times the batch, to show how the per-launch fixed
+        # cost (launch, dependent first loads, uneven wave finish: ~13 us) weighs on the B = 64 figures
+        "cfg2_b256": lambda: workloads.cfg2_qwen7b_int8(device=dev, quantize_fn=_gpu_quantize, batch=256),
     }
-    names = [args.only] if args.only else ["cfg1", "cfg2", "cfg3", "cfg4"]
+    names = [args.only] if args.only else ["cfg1", "cfg2", "cfg3", "cfg4", "cfg2_b256"]
     results = {}
     baseline = None
     for name in names:
@@ -322,7 +355,7 @@ def main() -> int:
         torch.cuda.empty_cache()
 
     head = results[names[0]]
-    dtype = {"cfg1": "bf16", "cfg2": "int8", "cfg3": "fp8", "cfg4": "fp8"}[names[0]]
+    dtype = {"cfg1": "bf16", "cfg2": "int8", "cfg3": "fp8", "cfg4": "fp8", "cfg2_b256": "int8"}[names[0]]
     line = {
         "metric": "paged_decode_attn_us_per_step",
         "value": head["us_per_step"],

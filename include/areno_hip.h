@@ -156,6 +156,28 @@ int areno_hip_paged_varlen_prefill(const areno_paged_cache* cache, const void* q
                                    void* stream);
 
 /*
+ * The step in front of the path, fused into one pass over the projection output: per-head QK RMSNorm
+ * (areno/engine/layers/attention.py:90-93; y = dtype(x * rsqrt(mean(x^2) + eps) * w) in fp32,
+ * areno/accel/csrc/normalization.cu:34-56), rotary embedding with rotate_half pairing and every product and the sum
+ * rounded to the activation dtype (areno/engine/layers/rotary.py:17-52), and the scatter of the new K/V rows into the
+ * paged cache (areno/engine/layers/attention_backend/infer.py:245-263) through the quantizer of
+ * areno_hip_cache_write, so the pages hold exactly quantize(k_out) and quantize(v).
+ *   q, q_out      device [tokens, q_heads, head_dim];  k, v, k_out  device [tokens, kv_heads, head_dim];  all `dtype`
+ *                 (F16 / BF16); k_out may be NULL when only the pages are wanted
+ *   positions     device [tokens] int64, clamped into [0, max_pos)
+ *   cos, sin      device [max_pos, head_dim] float32 (the doubled-frequency tables of RotaryEmbedding)
+ *   q_weight, k_weight  device [head_dim] float32, NULL = no norm on that tensor
+ *   cache         NULL = no cache write (then block_ids / block_offsets are ignored)
+ * head_dim 64, 128, 256 or 512; every tensor 16-byte aligned.
+ */
+int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache, const void* q, const void* k, const void* v,
+                                       void* q_out, void* k_out, int32_t dtype, int64_t tokens, int32_t q_heads,
+                                       int32_t kv_heads, int32_t head_dim, const int64_t* positions, const float* cos,
+                                       const float* sin, int32_t max_pos, const float* q_weight,
+                                       const float* k_weight, float eps, const int64_t* block_ids,
+                                       const int64_t* block_offsets, void* stream);
+
+/*
  * Bytes of device workspace the two prefill entry points above need (the reference allocates nothing here: its
  * varlen kernel keeps one query row per thread block, areno/accel/csrc/attention.cu:145-242).  The matrix-core
  * kernels cut the work into equal shares of key tiles whatever the length distribution, and a query block cut by a

@@ -4,8 +4,11 @@ TEST INFRASTRUCTURE ONLY.  Nothing under ``areno_amd/`` may import this package;
 it is the checker that the HIP kernels are compared against (tests, the smoke
 entry point and the CPU-baseline leg of the benchmark), never a fallback.
 
-Two independent restatements live here:
+Three restatements live here:
 
+* ``rope_ref`` -- the layer's steps in front of the path: per-head RMSNorm
+  (``areno/accel/csrc/normalization.cu:34-56``) and rotary embedding
+  (``areno/engine/layers/rotary.py:17-52``) with the eager ops' roundings.
 * ``attention_ref`` / ``quant_ref`` -- PyTorch (CPU) restatement of the
   reference's pure-PyTorch attention (``areno/accel/attention.py:25-76``), of
   its cache stores (``areno/engine/layers/attention_backend/infer.py:245-288``)
@@ -32,6 +35,11 @@ quantize_int8              numpy float64 brute force of the closed form; error
                            bound |x - x^| <= s/2; absmax -> +-127; zero rows
 quantize_fp8               exhaustive 256-entry decode table built from the
                            OCP e4m3fn bit layout; torch's own CPU cast
+ref_rmsnorm                float64 restatement; unit-RMS output for w = 1,
+                           scale invariance rmsnorm(c x) == rmsnorm(x)
+ref_rope                   position 0 is the identity; pair norms preserved;
+                           rope(p1) then rope(p2) == rope(p1 + p2) in float64;
+                           complex-multiplication form x * exp(i p w)
 =========================  ====================================================
 
 The reference repository holds no golden vectors, known-answer tests or
