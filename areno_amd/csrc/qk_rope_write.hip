@@ -79,32 +79,58 @@ __device__ __forceinline__ float group_max(float x) {
   return x;
 }
 
+constexpr int kRowsPerGroup = 1;  // rows a lane group works through (more than one measured slower: 53 vs 36 us at 4)
+
 template <int LPR>
 __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
   constexpr int D = LPR * 8;
   constexpr int kRowsPerWave = kWave / LPR;
+  constexpr int R = kRowsPerGroup;
   const int lane = threadIdx.x & (kWave - 1);
   const int sub = lane % LPR;  // which 8 elements of the row
   const int heads = p.q_heads + 2 * p.kv_heads;
   const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + (threadIdx.x >> 6);
   const int64_t total = p.tokens * heads;
-  const int64_t row_raw = wave_id * kRowsPerWave + lane / LPR;
-  const bool live = row_raw < total;
-  const int64_t row = live ? row_raw : total - 1;  // idle lane groups shadow the last row and store nothing
-  const int64_t token = row / heads;
-  const int slot = static_cast<int>(row - token * heads);
-  const int kind = slot < p.q_heads ? 0 : (slot < p.q_heads + p.kv_heads ? 1 : 2);  // q, k, v
-  const int head = kind == 0 ? slot : (kind == 1 ? slot - p.q_heads : slot - p.q_heads - p.kv_heads);
-  const void* src = kind == 0 ? p.q : (kind == 1 ? p.k : p.v);
-  const int src_heads = kind == 0 ? p.q_heads : p.kv_heads;
-  const int64_t src_base = (token * src_heads + head) * D + sub * 8;
 
-  float x[8];
-  {
-    const uint4_t raw = *reinterpret_cast<const uint4_t*>(static_cast<const char*>(src) + src_base * 2);
+  // ---- fetch: row r of this lane group is wave_base + r * rows_per_wave + group, so each load instruction of the
+  // wave covers 1 KB of consecutive rows --------------------------------------------------------------------------
+  bool live[R];
+  int kind[R], head[R];
+  int64_t token[R], src_base[R], pos[R];
+  uint4_t raw[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t row_raw = (wave_id * R + r) * kRowsPerWave + lane / LPR;
+    live[r] = row_raw < total;
+    const int64_t row = live[r] ? row_raw : total - 1;  // idle lane groups shadow the last row and store nothing
+    token[r] = row / heads;
+    const int slot = static_cast<int>(row - token[r] * heads);
+    kind[r] = slot < p.q_heads ? 0 : (slot < p.q_heads + p.kv_heads ? 1 : 2);  // q, k, v
+    head[r] = kind[r] == 0 ? slot : (kind[r] == 1 ? slot - p.q_heads : slot - p.q_heads - p.kv_heads);
+    const void* src = kind[r] == 0 ? p.q : (kind[r] == 1 ? p.k : p.v);
+    const int src_heads = kind[r] == 0 ? p.q_heads : p.kv_heads;
+    src_base[r] = (token[r] * src_heads + head[r]) * D + sub * 8;
+    raw[r] = *reinterpret_cast<const uint4_t*>(static_cast<const char*>(src) + src_base[r] * 2);
+    pos[r] = p.positions[token[r]];
+  }
+  float4_t c0[R], c1[R], s0[R], s1[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t pc = pos[r] < 0 ? 0 : (pos[r] >= p.max_pos ? p.max_pos - 1 : pos[r]);
+    const float* cos_row = p.cos + pc * D + sub * 8;
+    const float* sin_row = p.sin + pc * D + sub * 8;
+    c0[r] = *reinterpret_cast<const float4_t*>(cos_row);
+    c1[r] = *reinterpret_cast<const float4_t*>(cos_row + 4);
+    s0[r] = *reinterpret_cast<const float4_t*>(sin_row);
+    s1[r] = *reinterpret_cast<const float4_t*>(sin_row + 4);
+  }
+
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float x[8];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t word = raw[j];
+      const uint32_t word = raw[r][j];
       if (p.dtype == ARENO_DT_BF16) {
         x[2 * j] = bf16_bits_to_float(word & 0xffffu);
         x[2 * j + 1] = bf16_bits_to_float(word >> 16);
@@ -113,106 +139,98 @@ __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
         x[2 * j + 1] = f16_bits_to_float(word >> 16);
       }
     }
-  }
 
-  // ---- q and k rows: norm and rotary (the selects keep every lane in the cross-lane steps) ------------------------
-  const float* weight = kind == 0 ? p.q_weight : (kind == 1 ? p.k_weight : nullptr);
-  {
-    float sum_sq = 0.0f;
+    // ---- q and k rows: norm and rotary (selects, not branches, keep every lane in the cross-lane steps) ----------
+    const float* weight = kind[r] == 0 ? p.q_weight : (kind[r] == 1 ? p.k_weight : nullptr);
+    {
+      float sum_sq = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) sum_sq += x[j] * x[j];
-    sum_sq = group_sum<LPR>(sum_sq);
-    if (weight != nullptr) {
-      const float inv = rsqrtf(sum_sq / static_cast<float>(D) + p.eps);
-      const float4_t w0 = *reinterpret_cast<const float4_t*>(weight + sub * 8);
-      const float4_t w1 = *reinterpret_cast<const float4_t*>(weight + sub * 8 + 4);
+      for (int j = 0; j < 8; ++j) sum_sq += x[j] * x[j];
+      sum_sq = group_sum<LPR>(sum_sq);
+      if (weight != nullptr) {
+        const float inv = rsqrtf(sum_sq / static_cast<float>(D) + p.eps);
+        const float4_t w0 = *reinterpret_cast<const float4_t*>(weight + sub * 8);
+        const float4_t w1 = *reinterpret_cast<const float4_t*>(weight + sub * 8 + 4);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        x[j] = round_to(x[j] * inv * w0[j], p.dtype);
-        x[4 + j] = round_to(x[4 + j] * inv * w1[j], p.dtype);
+        for (int j = 0; j < 4; ++j) {
+          x[j] = round_to(x[j] * inv * w0[j], p.dtype);
+          x[4 + j] = round_to(x[4 + j] * inv * w1[j], p.dtype);
+        }
       }
     }
-  }
-  float partner[8];
+    float partner[8];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) partner[j] = wave_xor(x[j], LPR / 2);
-  if (kind != 2) {
-    int64_t pos = p.positions[token];
-    pos = pos < 0 ? 0 : (pos >= p.max_pos ? p.max_pos - 1 : pos);
-    const float* cos_row = p.cos + pos * D + sub * 8;
-    const float* sin_row = p.sin + pos * D + sub * 8;
-    const float4_t c0 = *reinterpret_cast<const float4_t*>(cos_row);
-    const float4_t c1 = *reinterpret_cast<const float4_t*>(cos_row + 4);
-    const float4_t s0 = *reinterpret_cast<const float4_t*>(sin_row);
-    const float4_t s1 = *reinterpret_cast<const float4_t*>(sin_row + 4);
-    const bool low_half = sub < LPR / 2;  // rotate_half: -x[i + D/2] below D/2, x[i - D/2] above
+    for (int j = 0; j < 8; ++j) partner[j] = wave_xor(x[j], LPR / 2);
+    if (kind[r] != 2) {
+      const bool low_half = sub < LPR / 2;  // rotate_half: -x[i + D/2] below D/2, x[i - D/2] above
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float c = round_to(j < 4 ? c0[j & 3] : c1[j & 3], p.dtype);
-      const float sn = round_to(j < 4 ? s0[j & 3] : s1[j & 3], p.dtype);
-      const float rot = low_half ? -partner[j] : partner[j];
-      x[j] = round_to(round_to(x[j] * c, p.dtype) + round_to(rot * sn, p.dtype), p.dtype);
+      for (int j = 0; j < 8; ++j) {
+        const float c = round_to(j < 4 ? c0[r][j & 3] : c1[r][j & 3], p.dtype);
+        const float sn = round_to(j < 4 ? s0[r][j & 3] : s1[r][j & 3], p.dtype);
+        const float rot = low_half ? -partner[j] : partner[j];
+        x[j] = round_to(round_to(x[j] * c, p.dtype) + round_to(rot * sn, p.dtype), p.dtype);
+      }
+      void* out = kind[r] == 0 ? p.q_out : p.k_out;
+      if (out != nullptr && live[r]) {
+        const uint4_t packed = {pack_two(x[0], x[1], p.dtype), pack_two(x[2], x[3], p.dtype),
+                                pack_two(x[4], x[5], p.dtype), pack_two(x[6], x[7], p.dtype)};
+        *reinterpret_cast<uint4_t*>(static_cast<char*>(out) + src_base[r] * 2) = packed;
+      }
     }
-    void* out = kind == 0 ? p.q_out : p.k_out;
-    if (out != nullptr && live) {
-      const uint4_t packed = {pack_two(x[0], x[1], p.dtype), pack_two(x[2], x[3], p.dtype),
-                              pack_two(x[4], x[5], p.dtype), pack_two(x[6], x[7], p.dtype)};
-      *reinterpret_cast<uint4_t*>(static_cast<char*>(out) + src_base * 2) = packed;
-    }
-  }
 
-  // ---- k and v rows: into the page, through the cache writer's quantizer ------------------------------------------
-  float amax = 0.0f;
+    // ---- k and v rows: into the page, through the cache writer's closed forms --------------------------------------
+    float amax = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(x[j]));
-  amax = group_max<LPR>(amax);
-  if (kind == 0 || !live) return;
-  void* cache = p.cache[kind - 1];
-  if (cache == nullptr) return;
-  const int64_t blk = p.block_ids[token];
-  const int64_t off = p.block_offsets[token];
-  if (blk < 0 || blk >= p.num_blocks || off < 0 || off >= p.block_size) return;
-  const int64_t dst_row = (blk * p.block_size + off) * p.kv_heads + head;
-  const int64_t dst_elem = dst_row * D + sub * 8;
-  if (p.cache_dtype == ARENO_DT_I8) {
-    const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
-    const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
-    const float s = static_cast<float>(s16_fixed);
-    uint32_t words[2] = {0u, 0u};
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(x[j]));
+    amax = group_max<LPR>(amax);
+    if (kind[r] == 0 || !live[r]) continue;
+    void* cache = p.cache[kind[r] - 1];
+    if (cache == nullptr) continue;
+    const int64_t blk = p.block_ids[token[r]];
+    const int64_t off = p.block_offsets[token[r]];
+    if (blk < 0 || blk >= p.num_blocks || off < 0 || off >= p.block_size) continue;
+    const int64_t dst_row = (blk * p.block_size + off) * p.kv_heads + head[r];
+    const int64_t dst_elem = dst_row * D + sub * 8;
+    if (p.cache_dtype == ARENO_DT_I8) {
+      const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
+      const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
+      const float s = static_cast<float>(s16_fixed);
+      uint32_t words[2] = {0u, 0u};
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float code = fminf(fmaxf(rintf(x[j] / s), -127.0f), 127.0f);
-      words[j / 4] |= (static_cast<uint32_t>(static_cast<int>(code)) & 0xffu) << (8 * (j & 3));
-    }
-    *reinterpret_cast<uint2_t*>(static_cast<char*>(cache) + dst_elem) = uint2_t{words[0], words[1]};
-    if (sub == 0) {
-      if (p.scale_dtype == ARENO_DT_F16) {
-        static_cast<uint16_t*>(p.scale[kind - 1])[dst_row] = __builtin_bit_cast(uint16_t, s16_fixed);
-      } else {
-        static_cast<float*>(p.scale[kind - 1])[dst_row] = s;
+      for (int j = 0; j < 8; ++j) {
+        const float code = fminf(fmaxf(rintf(x[j] / s), -127.0f), 127.0f);
+        words[j / 4] |= (static_cast<uint32_t>(static_cast<int>(code)) & 0xffu) << (8 * (j & 3));
       }
-    }
-  } else if (p.cache_dtype == ARENO_DT_FP8_E4M3) {
-    float s = amax / 448.0f;
-    if (s == 0.0f) s = 1.0f;
-    uint32_t words[2] = {0u, 0u};
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float y = fminf(fmaxf(x[j] / s, -448.0f), 448.0f);
-      words[j / 4] |= float_to_fp8_byte(y) << (8 * (j & 3));
-    }
-    *reinterpret_cast<uint2_t*>(static_cast<char*>(cache) + dst_elem) = uint2_t{words[0], words[1]};
-    if (sub == 0) {
-      if (p.scale_dtype == ARENO_DT_F16) {
-        static_cast<uint16_t*>(p.scale[kind - 1])[dst_row] = static_cast<uint16_t>(float_to_f16_bits(s));
-      } else {
-        static_cast<float*>(p.scale[kind - 1])[dst_row] = s;
+      *reinterpret_cast<uint2_t*>(static_cast<char*>(cache) + dst_elem) = uint2_t{words[0], words[1]};
+      if (sub == 0) {
+        if (p.scale_dtype == ARENO_DT_F16) {
+          static_cast<uint16_t*>(p.scale[kind[r] - 1])[dst_row] = __builtin_bit_cast(uint16_t, s16_fixed);
+        } else {
+          static_cast<float*>(p.scale[kind[r] - 1])[dst_row] = s;
+        }
       }
+    } else if (p.cache_dtype == ARENO_DT_FP8_E4M3) {
+      float s = amax / 448.0f;
+      if (s == 0.0f) s = 1.0f;
+      uint32_t words[2] = {0u, 0u};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float y = fminf(fmaxf(x[j] / s, -448.0f), 448.0f);
+        words[j / 4] |= float_to_fp8_byte(y) << (8 * (j & 3));
+      }
+      *reinterpret_cast<uint2_t*>(static_cast<char*>(cache) + dst_elem) = uint2_t{words[0], words[1]};
+      if (sub == 0) {
+        if (p.scale_dtype == ARENO_DT_F16) {
+          static_cast<uint16_t*>(p.scale[kind[r] - 1])[dst_row] = static_cast<uint16_t>(float_to_f16_bits(s));
+        } else {
+          static_cast<float*>(p.scale[kind[r] - 1])[dst_row] = s;
+        }
+      }
+    } else {
+      const uint4_t packed = {pack_two(x[0], x[1], p.cache_dtype), pack_two(x[2], x[3], p.cache_dtype),
+                              pack_two(x[4], x[5], p.cache_dtype), pack_two(x[6], x[7], p.cache_dtype)};
+      *reinterpret_cast<uint4_t*>(static_cast<char*>(cache) + dst_elem * 2) = packed;
     }
-  } else {
-    const uint4_t packed = {pack_two(x[0], x[1], p.cache_dtype), pack_two(x[2], x[3], p.cache_dtype),
-                            pack_two(x[4], x[5], p.cache_dtype), pack_two(x[6], x[7], p.cache_dtype)};
-    *reinterpret_cast<uint4_t*>(static_cast<char*>(cache) + dst_elem * 2) = packed;
   }
 }
 
@@ -289,7 +307,7 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
   const rope_write_fn fn = rope_write_lookup(head_dim);
   if (fn == nullptr) return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim must be 64, 128, 256 or 512, got %d", op, head_dim);
   const int64_t rows = tokens * (q_heads + 2 * kv_heads);
-  const int rows_per_block = 4 * (kWave / (head_dim / 8));
+  const int rows_per_block = 4 * kRowsPerGroup * (kWave / (head_dim / 8));
   const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
   if (blocks > 0x7fffffffLL) return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: too many rows", op);
   hipLaunchKernelGGL(fn, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), p);

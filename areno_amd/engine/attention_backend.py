@@ -84,8 +84,8 @@ class HipInferBackend(nn.Module):
                     meta.cache_block_ids, meta.cache_block_offsets, k_scale=k_scale, v_scale=v_scale,
                 )  # fmt: skip
             if meta.context_lens is not None:
-                if not update_cache:
-                    raise ValueError("prefill over cached context reads the new tokens from the cache: update_cache=True")
+                # reads the new tokens from the pages: with update_cache=False the caller has already stored them
+                # (the fused norm + rotary + cache-write op does)
                 out = areno_paged_varlen_causal_attention(
                     q_flat.contiguous(), k_cache, v_cache, meta.block_table.contiguous(), meta.cu_seqlens.contiguous(),
                     meta.context_lens.contiguous(), window_left=window_left, softmax_scale=softmax_scale,
