@@ -75,6 +75,8 @@ def areno_paged_causal_attention_decode(
     softmax_scale: float | None = None,
     k_scale: torch.Tensor | None = None,
     v_scale: torch.Tensor | None = None,
+    prefix_group_rows: int | None = None,
+    shared_prefix_lens: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Apply single-token paged-cache causal attention to ``(batch, heads, dim)`` Q.
 
@@ -82,6 +84,11 @@ def areno_paged_causal_attention_decode(
     (mutating the caches, and the scale pools for quantized caches, in place), then attends
     over positions ``[0, cache_seqlens[b]]``.  ``num_splits`` is a hint: ``1`` keeps one
     partial per row, any other value lets the kernel pick fixed-size KV chunks.
+
+    ``prefix_group_rows`` / ``shared_prefix_lens`` (optional, together): rows
+    ``[i * prefix_group_rows, (i + 1) * prefix_group_rows)`` list the same block ids for their first
+    ``shared_prefix_lens[i]`` tokens (the samples of one prompt in a rollout); those pages are then read once for
+    several rows instead of once per row.  The result is the same.
     """
     op = "areno_paged_causal_attention_decode"
     if not _all_on_gpu(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, k_scale, v_scale):
@@ -108,9 +115,21 @@ def areno_paged_causal_attention_decode(
         block_table.contiguous(), cache_seqlens.contiguous(),
         _window_left(window_left), int(num_splits), _scale(q, softmax_scale),
     )  # fmt: skip
+    if (prefix_group_rows is None) != (shared_prefix_lens is None):
+        raise ValueError(f"{op} expects prefix_group_rows and shared_prefix_lens together")
+    if shared_prefix_lens is not None:
+        if not shared_prefix_lens.is_cuda:
+            raise RuntimeError(f"{op} requires CUDA tensors")
+        if int(prefix_group_rows) < 1 or q.shape[0] % int(prefix_group_rows) != 0:
+            raise ValueError(f"{op} expects the batch to be a multiple of prefix_group_rows")
+        if shared_prefix_lens.dtype != torch.int32 or shared_prefix_lens.shape != (q.shape[0] // int(prefix_group_rows),):
+            raise ValueError(f"{op} expects int32 shared_prefix_lens shaped (batch / prefix_group_rows,)")
+        return ext.areno_paged_causal_attention_decode_forward_scaled(
+            *args, k_scale, v_scale, int(prefix_group_rows), shared_prefix_lens.contiguous()
+        )
     if k_scale is None:
         return ext.areno_paged_causal_attention_decode_forward(*args)
-    return ext.areno_paged_causal_attention_decode_forward_scaled(*args, k_scale, v_scale)
+    return ext.areno_paged_causal_attention_decode_forward_scaled(*args, k_scale, v_scale, 0, None)
 
 
 @torch._dynamo.disable

@@ -65,6 +65,9 @@ def lib() -> ctypes.CDLL:
         decode_args = [_P, _P, _P, _P, _P, _I32, _I32, _I32, _P, _I32, _P, _I32, _I32, _F, _P, _SZ]
         handle.areno_hip_paged_decode.argtypes = decode_args + [_P]
         handle.areno_hip_paged_decode_stages.argtypes = decode_args + [_I32, _P]
+        handle.areno_hip_paged_decode_grouped.argtypes = decode_args[:-2] + [_I32, _P, _P, _SZ, _I32, _P]
+        handle.areno_hip_paged_decode_grouped_workspace_bytes.restype = _SZ
+        handle.areno_hip_paged_decode_grouped_workspace_bytes.argtypes = [_I32] * 8
         handle.areno_hip_varlen_attention.argtypes = [_P, _P, _P, _P, _I32, _I64, _I32, _I32, _I32, _P, _I32, _I32, _F, _P, _SZ, _P]  # fmt: skip
         handle.areno_hip_paged_varlen_prefill.argtypes = [_P, _P, _P, _I32, _I64, _I32, _I32, _P, _I32, _P, _P, _I32, _F, _P, _SZ, _P]  # fmt: skip
         handle.areno_hip_prefill_workspace_bytes.restype = _SZ
@@ -103,10 +106,28 @@ def decode_workspace_bytes(batch, q_heads, head_dim, block_size, max_blocks, num
     return int(lib().areno_hip_paged_decode_workspace_bytes(batch, q_heads, head_dim, block_size, max_blocks, num_splits))
 
 
+def decode_grouped_workspace_bytes(batch, q_heads, kv_heads, head_dim, block_size, max_blocks, group_rows,
+                                   num_splits=8) -> int:  # fmt: skip
+    return int(lib().areno_hip_paged_decode_grouped_workspace_bytes(batch, q_heads, kv_heads, head_dim, block_size,
+                                                                    max_blocks, num_splits, group_rows))  # fmt: skip
+
+
 def paged_decode(cache: PagedCache, q, k_update, v_update, out, block_table, cache_seqlens, workspace, *,
-                 window_left=-1, num_splits=8, softmax_scale=None, stages=STAGE_ALL, stream=None) -> None:  # fmt: skip
-    """``areno_hip_paged_decode_stages`` on raw pointers; ``workspace`` is a uint8 device tensor."""
+                 window_left=-1, num_splits=8, softmax_scale=None, stages=STAGE_ALL, stream=None,
+                 group_rows=None, shared_lens=None) -> None:  # fmt: skip
+    """``areno_hip_paged_decode_stages`` (or ``_grouped`` when ``shared_lens`` is given) on raw pointers;
+    ``workspace`` is a uint8 device tensor."""
     scale = float(softmax_scale if softmax_scale is not None else q.shape[-1] ** -0.5)
+    if shared_lens is not None:
+        status = lib().areno_hip_paged_decode_grouped(
+            ctypes.byref(cache), q.data_ptr(), None if k_update is None else k_update.data_ptr(),
+            None if v_update is None else v_update.data_ptr(), out.data_ptr(), dtype_code(q), q.shape[0], q.shape[1],
+            block_table.data_ptr(), block_table.shape[1], cache_seqlens.data_ptr(), int(window_left), int(num_splits),
+            scale, int(group_rows), shared_lens.data_ptr(), workspace.data_ptr(), workspace.numel(), int(stages),
+            current_stream_ptr() if stream is None else stream,
+        )  # fmt: skip
+        check(status, "areno_hip_paged_decode_grouped")
+        return
     status = lib().areno_hip_paged_decode_stages(
         ctypes.byref(cache), q.data_ptr(), None if k_update is None else k_update.data_ptr(),
         None if v_update is None else v_update.data_ptr(), out.data_ptr(), dtype_code(q), q.shape[0], q.shape[1],

@@ -66,6 +66,18 @@ struct MfmaDecodeParams {
   // writer and stores it (and its scales) into the page, so no separate append launch is needed.
   const void* k_update;
   const void* v_update;
+  // Prefix groups (GROUPED kernels only): rows [i * group_rows, (i + 1) * group_rows) share the pages of their first
+  // shared_lens[i] tokens (an RL rollout's samples of one prompt).  Those tokens become "shared items" that are read
+  // once for up to cols_seqs = 16 / q-heads-per-kv-head sequences side by side in the 16 MFMA columns; the rest of
+  // each sequence is an item of its own.  Shared items leave their partials in a second region (16 columns per kv
+  // head and slot).
+  const int32_t* shared_lens;  // [batch / group_rows]
+  int32_t group_rows;          // rows per prefix group
+  int32_t cols_seqs;           // sequences that fit side by side: 16 / group
+  int32_t subs_per_group;      // ceil(group_rows / cols_seqs)
+  int32_t num_shared;          // shared items: (batch / group_rows) * subs_per_group, listed before the per-row items
+  float* shared_ml;            // [slot][kv_head][16][2]
+  float* shared_acc;           // [slot][kv_head][16][head_dim]
 #ifdef ARENO_TRACE
   unsigned long long* trace;  // [wave][16] timestamps, tuning builds only
 #endif
@@ -223,17 +235,25 @@ __host__ __device__ inline UnitGeometry make_unit_geometry(int total_tiles, int 
 }
 
 // Position of a tile stream inside a unit: which sequence, which token of it comes next.
+// An item is a run of tokens [lo, hi) read through the block table of row `row`: a whole sequence's visible keys
+// in the plain kernel; in a GROUPED kernel either the shared prefix of `nseq` adjacent rows or the rest of one row.
+struct ItemInfo {
+  int lo, hi, row, nseq;
+};
+
 struct TileCursor {
-  int b;         // sequence
-  int tok;       // first token (position inside the sequence) of the tile
-  int end;       // visible length of the sequence (cache_seqlens[b] + 1)
-  int next_end;  // same for sequence b + 1, fetched one sequence ahead
+  int b;    // item (= sequence in the plain kernel)
+  int tok;  // first token (position inside the sequence) of the tile
+  int end;  // end of the item's token range (cache_seqlens[b] + 1 for a sequence)
+  int row;  // block-table / query row of the item
+  int nseq;
+  ItemInfo next;  // item b + 1, fetched one item ahead
 };
 
 #ifndef ARENO_MFMA_QUANT_OCC
 #define ARENO_MFMA_QUANT_OCC 2
 #endif
-template <int KIND, int D, bool SCALE16, int NW>
+template <int KIND, int D, bool SCALE16, int NW, bool GROUPED = false>
 __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUANT_OCC : 2) void decode_mfma_kernel(
     MfmaDecodeParams mp) {
   using T = KVTraits<KIND>;
@@ -257,9 +277,10 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   static_assert(NLD >= 1 && LPT >= 4 && LPT <= 16, "unsupported head_dim");
 
   __shared__ __attribute__((aligned(16))) char s_tiles[NW][kWaveLds];
-  __shared__ int s_cum[kMfmaMaxBatch + 1];
+  constexpr int kMaxItems = (GROUPED ? 2 : 1) * kMfmaMaxBatch;  // at most one shared item per row on top of the rows
+  __shared__ int s_cum[kMaxItems + 1];
   __shared__ int s_wave_tot[NW];
-  constexpr int SPT = kMfmaMaxBatch / (NW * kWave);  // sequences per thread in the prefix sum
+  constexpr int SPT = kMaxItems / (NW * kWave);  // items per thread in the prefix sum
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -278,17 +299,52 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   const int grp = lane / LPT;
   const int dc = lane % LPT;
 
-  // ---- tiles per sequence, exclusive prefix sum over the batch ---------------------------------
+  // ---- the item list ----------------------------------------------------------------------------------------------
+  const int num_items = GROUPED ? mp.num_shared + p.batch : p.batch;
+  // tokens of a sub-group's shared prefix: the caller's figure, clipped to what every member has cached and cut to a
+  // whole number of tiles
+  auto shared_tokens = [&](int sub, int& row0, int& count) {
+    const int gi = sub / mp.subs_per_group;
+    const int j = sub - gi * mp.subs_per_group;
+    row0 = gi * mp.group_rows + j * mp.cols_seqs;
+    count = min(mp.cols_seqs, mp.group_rows - j * mp.cols_seqs);
+    int len = mp.shared_lens[gi];
+    for (int m = 0; m < count; ++m) len = min(len, p.cache_seqlens[row0 + m]);
+    return max(len, 0) & ~(TK - 1);
+  };
+  auto item_info = [&](int v) {
+    ItemInfo it = {0, 0, 0, 1};
+    if (v >= num_items) return it;
+    if constexpr (GROUPED) {
+      if (v < mp.num_shared) {
+        it.hi = shared_tokens(v, it.row, it.nseq);
+        return it;
+      }
+      const int b = v - mp.num_shared;
+      const int gi = b / mp.group_rows;
+      int row0, count;
+      it.lo = shared_tokens(gi * mp.subs_per_group + (b - gi * mp.group_rows) / mp.cols_seqs, row0, count);
+      it.hi = p.cache_seqlens[b] + 1;
+      it.row = b;
+      return it;
+    } else {
+      it.hi = p.cache_seqlens[v] + 1;
+      it.lo = first_allowed_key(it.hi, p.window_left);
+      it.row = v;
+      return it;
+    }
+  };
+  // ---- tiles per item, exclusive prefix sum over the items --------------------------------------------------------
   {
     int nt[SPT];
     int local = 0;
 #pragma unroll
     for (int j = 0; j < SPT; ++j) {
-      const int b = SPT * tid + j;
+      const int v = SPT * tid + j;
       nt[j] = 0;
-      if (b < p.batch) {
-        const int length = p.cache_seqlens[b] + 1;
-        nt[j] = (length - first_allowed_key(length, p.window_left) + TK - 1) / TK;
+      if (v < num_items) {
+        const ItemInfo it = item_info(v);
+        nt[j] = (it.hi - it.lo + TK - 1) / TK;
       }
       local += nt[j];
     }
@@ -304,8 +360,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     for (int w2 = 0; w2 < wave; ++w2) excl += s_wave_tot[w2];
 #pragma unroll
     for (int j = 0; j < SPT; ++j) {
-      const int b = SPT * tid + j;
-      if (b <= p.batch) s_cum[b] = excl;
+      const int v = SPT * tid + j;
+      if (v <= num_items) s_cum[v] = excl;
       excl += nt[j];
     }
     __syncthreads();
@@ -315,11 +371,11 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   // workgroups; the rest is cut into small units for the workgroups behind them in the grid.  Those start as CUs
   // become free, so the hardware dispatcher hands the tail to whichever CU got the better memory service:
   // service is uneven across CUs, and with equal shares only the slowest wave would set the run time.
-  const int total_tiles = s_cum[p.batch];
+  const int total_tiles = s_cum[num_items];
   const UnitGeometry geo =
       make_unit_geometry(total_tiles, mp.num_pieces, mp.max_small, mp.static_share, mp.min_unit_tiles);
   if (blockIdx.x == 0 && blockIdx.y == 0) {
-    for (int b = tid; b <= p.batch; b += NW * kWave) mp.plan[b] = s_cum[b];
+    for (int v = tid; v <= num_items; v += NW * kWave) mp.plan[v] = s_cum[v];
   }
 
   const int hw_count = p.heads_per_wg;
@@ -336,25 +392,41 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   const bool q_is_operand_type = (KIND == KV_BF16 && p.q_dtype == ARENO_DT_BF16) ||
                                  (KIND != KV_BF16 && p.q_dtype == ARENO_DT_F16);
 
-  auto seq_len = [&](int b) { return b < p.batch ? p.cache_seqlens[b] + 1 : 0; };
-  // move a cursor from tile x to tile x + 1; returns true when that tile starts a new sequence
+  auto enter_item = [&](TileCursor& c, const ItemInfo& it) {
+    c.tok = it.lo;
+    c.end = it.hi;
+    c.row = it.row;
+    c.nseq = it.nseq;
+  };
+  // move a cursor from tile x to tile x + 1; returns true when that tile starts a new item
   auto advance = [&](TileCursor& c, int x_next) {
     if (x_next == s_cum[c.b + 1]) {
       ++c.b;
-      c.end = c.next_end;
-      c.next_end = seq_len(c.b + 1);
-      c.tok = first_allowed_key(c.end, p.window_left);
+      if constexpr (GROUPED) {
+        if (s_cum[c.b + 1] == x_next) {
+          // items without tiles (a group with no shared prefix): skip them; the prefetched item is not the right one
+          do {
+            ++c.b;
+          } while (s_cum[c.b + 1] == x_next);
+          enter_item(c, item_info(c.b));
+          c.next = item_info(c.b + 1);
+          return true;
+        }
+      }
+      enter_item(c, c.next);
+      c.next = item_info(c.b + 1);
       return true;
     }
     c.tok += TK;
     return false;
   };
+  auto is_shared = [&](int v) { return GROUPED && v < mp.num_shared; };
 
   TileCursor kv_cur, id_cur;
   int unit = 0;
   int ids[NLD];
   auto issue_id_loads = [&]() {
-    const int32_t* table_row = p.block_table + static_cast<int64_t>(id_cur.b) * p.max_blocks;
+    const int32_t* table_row = p.block_table + static_cast<int64_t>(id_cur.row) * p.max_blocks;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int t = min(id_cur.tok + i * TPL + grp, id_cur.end - 1);
@@ -372,8 +444,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   int64_t new_row = 0;     // cache row of the newest token, in the lanes that hold it
   uint4_t upd_k[2], upd_v[2];
   auto issue_kv_loads = [&]() {
-    tail_tile = fused_append && kv_cur.tok + TK >= kv_cur.end;
-    const int64_t upd_row = static_cast<int64_t>(kv_cur.b) * p.kv_heads + kvh;
+    tail_tile = fused_append && !is_shared(kv_cur.b) && kv_cur.tok + TK >= kv_cur.end;
+    const int64_t upd_row = static_cast<int64_t>(kv_cur.row) * p.kv_heads + kvh;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int tt = kv_cur.tok + i * TPL + grp;
@@ -419,12 +491,19 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   // Q of a sequence: lane (lr = head, lk) needs dims (D/4)*lk + 8*s + [0, 8) of head h0 + lr, 16 raw bytes per
   // slice for 16-bit queries; fetched when the KV cursor enters the sequence, converted when compute gets there.
   uint4_t qraw[NS];
-  auto issue_q_loads = [&](int b) {
+  // column lr of the MFMA tiles: head lr of the row in a per-row item, (row lr / G, head lr % G) in a shared item
+  const int col_seq = GROUPED ? lr / p.group : 0;
+  const int col_head = GROUPED ? lr - col_seq * p.group : lr;
+  auto issue_q_loads = [&](const TileCursor& c) {
+    const bool shared = is_shared(c.b);
+    const int m = shared ? col_seq : 0;
+    const int g = shared ? col_head : lr;
+    const bool live = shared ? m < c.nseq : lr < p.group;
 #pragma unroll
     for (int sl = 0; sl < NS; ++sl) {
       qraw[sl] = uint4_t{0u, 0u, 0u, 0u};
-      if (lr < p.group) {
-        const int64_t idx = (static_cast<int64_t>(b) * p.q_heads + h0 + lr) * D + (D / 4) * lk + 8 * sl;
+      if (live) {
+        const int64_t idx = (static_cast<int64_t>(c.row + m) * p.q_heads + h0 + g) * D + (D / 4) * lk + 8 * sl;
         qraw[sl] = load16(p.q, idx * 2);
       }
     }
@@ -473,14 +552,19 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     p_sum = 0.0f;
   };
 
-  auto write_partial = [&](int b) {
+  auto write_partial = [&](int v, int row, int nseq) {
     // combine the four k-groups' row sums; every lane of a head ends with the head's totals
     const float l_tot = rows_sum(l_run);
     float off = 0.0f;
     if constexpr (KIND == KV_I8) off = kI8Offset * rows_sum(p_sum);
-    if (lr < p.group) {
-      const int64_t prow = (static_cast<int64_t>(unit + b)) * p.q_heads + h0 + lr;
-      float* dst = p.part_acc + prow * D + 4 * lk;
+    const bool shared = is_shared(v);
+    const bool live = shared ? col_seq < nseq : lr < p.group;
+    if (live) {
+      // per-row items: slot unit + row, one row per q head; shared items: slot unit + item, 16 columns per kv head
+      const int64_t prow = shared ? (static_cast<int64_t>(unit + v) * p.kv_heads + kvh) * 16 + lr
+                                  : static_cast<int64_t>(unit + row) * p.q_heads + h0 + lr;
+      float* ml = shared ? mp.shared_ml : p.part_ml;
+      float* dst = (shared ? mp.shared_acc : p.part_acc) + prow * D + 4 * lk;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
         float4_t o = acc[nb];
@@ -489,8 +573,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
         *reinterpret_cast<float4_t*>(dst + 16 * nb) = o;
       }
       if (lk == 0) {
-        p.part_ml[prow * 2] = m_run;
-        p.part_ml[prow * 2 + 1] = l_tot;
+        ml[prow * 2] = m_run;
+        ml[prow * 2 + 1] = l_tot;
       }
     }
   };
@@ -502,10 +586,10 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     const int x0 = geo.unit_start(unit);
     const int x1 = unit < geo.static_units + geo.small_units ? geo.unit_start(unit + 1) : x0;
     if (x0 < x1) {
-      // sequence that owns tile x0: largest b with cum[b] <= x0
-      int b_first;
+      // item that owns tile x0: the largest v with cum[v] <= x0
+      int v_first;
       {
-        int lo = 0, hi = p.batch;
+        int lo = 0, hi = num_items;
         while (lo + 1 < hi) {
           const int mid = (lo + hi) >> 1;
           if (s_cum[mid] <= x0) {
@@ -514,25 +598,25 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
             hi = mid;
           }
         }
-        b_first = lo;
+        v_first = lo;
       }
 
       // ---- three cursors: block ids are fetched two tiles ahead, KV one tile ahead of the tile being computed ---
-      kv_cur.b = b_first;
-      kv_cur.end = seq_len(b_first);
-      kv_cur.next_end = seq_len(b_first + 1);
-      kv_cur.tok = first_allowed_key(kv_cur.end, p.window_left) + (x0 - s_cum[b_first]) * TK;
+      kv_cur.b = v_first;
+      enter_item(kv_cur, item_info(v_first));
+      kv_cur.next = item_info(v_first + 1);
+      kv_cur.tok += (x0 - s_cum[v_first]) * TK;
       id_cur = kv_cur;
 
       // ---- prologue -------------------------------------------------------------------------------------------
       issue_id_loads();
-      issue_q_loads(kv_cur.b);
+      issue_q_loads(kv_cur);
       issue_kv_loads();  // tile x0 (waits for its ids)
       if (x0 + 1 < x1) {
         advance(id_cur, x0 + 1);
         issue_id_loads();  // ids of tile x0 + 1
       }
-      int cp_b = kv_cur.b, cp_tok = kv_cur.tok, cp_end = kv_cur.end;
+      int cp_b = kv_cur.b, cp_row = kv_cur.row, cp_nseq = kv_cur.nseq, cp_tok = kv_cur.tok, cp_end = kv_cur.end;
       adopt_q();
       reset_state();
 
@@ -604,7 +688,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
         bool next_is_new_seq = false;
         if (x + 1 < x1) {
           next_is_new_seq = advance(kv_cur, x + 1);
-          if (next_is_new_seq) issue_q_loads(kv_cur.b);
+          if (next_is_new_seq) issue_q_loads(kv_cur);
           issue_kv_loads();
           if (x + 2 < x1) {
             advance(id_cur, x + 2);
@@ -713,9 +797,11 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
         // -- end of a sequence's share: emit its partial and switch to the next sequence ---------------------------
         const bool last_of_piece = x + 1 == x1;
         if (next_is_new_seq || last_of_piece) {
-          write_partial(cp_b);
+          write_partial(cp_b, cp_row, cp_nseq);
           if (!last_of_piece) {
             cp_b = kv_cur.b;
+            cp_row = kv_cur.row;
+            cp_nseq = kv_cur.nseq;
             adopt_q();
             reset_state();
           }
@@ -731,20 +817,22 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
 }
 
 typedef void (*decode_mfma_fn)(MfmaDecodeParams);
-decode_mfma_fn decode_mfma_lookup_bf16(int head_dim, bool scale16);
-decode_mfma_fn decode_mfma_lookup_f16(int head_dim, bool scale16);
-decode_mfma_fn decode_mfma_lookup_i8(int head_dim, bool scale16);
-decode_mfma_fn decode_mfma_lookup_fp8(int head_dim, bool scale16);
+decode_mfma_fn decode_mfma_lookup_bf16(int head_dim, bool scale16, bool grouped);
+decode_mfma_fn decode_mfma_lookup_f16(int head_dim, bool scale16, bool grouped);
+decode_mfma_fn decode_mfma_lookup_i8(int head_dim, bool scale16, bool grouped);
+decode_mfma_fn decode_mfma_lookup_fp8(int head_dim, bool scale16, bool grouped);
 
-template <int KIND>
+template <int KIND, bool GROUPED>
 decode_mfma_fn decode_mfma_lookup_impl(int head_dim, bool scale16) {
   constexpr int NW = ARENO_MFMA_NW;
   if constexpr (KVTraits<KIND>::kQuant) {
-    if (head_dim == 128) return scale16 ? decode_mfma_kernel<KIND, 128, true, NW> : decode_mfma_kernel<KIND, 128, false, NW>;
-    if (head_dim == 64) return scale16 ? decode_mfma_kernel<KIND, 64, true, NW> : decode_mfma_kernel<KIND, 64, false, NW>;
+    if (head_dim == 128)
+      return scale16 ? decode_mfma_kernel<KIND, 128, true, NW, GROUPED> : decode_mfma_kernel<KIND, 128, false, NW, GROUPED>;
+    if (head_dim == 64)
+      return scale16 ? decode_mfma_kernel<KIND, 64, true, NW, GROUPED> : decode_mfma_kernel<KIND, 64, false, NW, GROUPED>;
   } else {
-    if (head_dim == 128) return decode_mfma_kernel<KIND, 128, false, NW>;
-    if (head_dim == 64) return decode_mfma_kernel<KIND, 64, false, NW>;
+    if (head_dim == 128) return decode_mfma_kernel<KIND, 128, false, NW, GROUPED>;
+    if (head_dim == 64) return decode_mfma_kernel<KIND, 64, false, NW, GROUPED>;
   }
   return nullptr;
 }

@@ -86,7 +86,8 @@ areno_paged_cache describe_cache(const at::Tensor& k_cache, const at::Tensor& v_
 at::Tensor paged_decode_forward_impl(at::Tensor q, at::Tensor k_update, at::Tensor v_update, at::Tensor k_cache,
                                      at::Tensor v_cache, at::Tensor block_table, at::Tensor cache_seqlens,
                                      int64_t window_left, int64_t num_splits, double softmax_scale,
-                                     c10::optional<at::Tensor> k_scale, c10::optional<at::Tensor> v_scale) {
+                                     c10::optional<at::Tensor> k_scale, c10::optional<at::Tensor> v_scale,
+                                     int64_t prefix_group_rows, c10::optional<at::Tensor> shared_prefix_lens) {
   const char* op = "areno_paged_causal_attention_decode";
   TORCH_CHECK(q.is_cuda(), op, " q must be CUDA");
   TORCH_CHECK(k_update.is_cuda(), op, " k_update must be CUDA");
@@ -126,17 +127,29 @@ at::Tensor paged_decode_forward_impl(at::Tensor q, at::Tensor k_update, at::Tens
   const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(q));
   auto out = at::empty_like(q);
   if (q.size(0) == 0) return out;
-  const size_t ws_bytes = areno_hip_paged_decode_workspace_bytes(
-      static_cast<int32_t>(q.size(0)), static_cast<int32_t>(q.size(1)), cache.head_dim, cache.block_size,
-      static_cast<int32_t>(block_table.size(1)), static_cast<int32_t>(num_splits));
+  const int32_t* shared_ptr = nullptr;
+  int32_t group_rows = 0;
+  if (shared_prefix_lens.has_value()) {
+    const at::Tensor& sl = *shared_prefix_lens;
+    TORCH_CHECK(prefix_group_rows >= 1 && q.size(0) % prefix_group_rows == 0, op,
+                " batch must be a multiple of prefix_group_rows");
+    TORCH_CHECK(sl.is_cuda() && sl.is_contiguous() && sl.scalar_type() == at::kInt && sl.dim() == 1 &&
+                    sl.size(0) == q.size(0) / prefix_group_rows,
+                op, " shared_prefix_lens must be a CUDA int32 (batch / prefix_group_rows,) tensor");
+    shared_ptr = sl.data_ptr<int32_t>();
+    group_rows = static_cast<int32_t>(prefix_group_rows);
+  }
+  const size_t ws_bytes = areno_hip_paged_decode_grouped_workspace_bytes(
+      static_cast<int32_t>(q.size(0)), static_cast<int32_t>(q.size(1)), cache.kv_heads, cache.head_dim,
+      cache.block_size, static_cast<int32_t>(block_table.size(1)), static_cast<int32_t>(num_splits), group_rows);
   TORCH_CHECK(ws_bytes > 0, op, " invalid shapes for the split-KV workspace");
   auto workspace = at::empty({static_cast<int64_t>(ws_bytes)}, q.options().dtype(at::kByte));
-  const int status = areno_hip_paged_decode(
+  const int status = areno_hip_paged_decode_grouped(
       &cache, q.data_ptr(), k_update.data_ptr(), v_update.data_ptr(), out.data_ptr(), dtype_code(q, op, "q"),
       static_cast<int32_t>(q.size(0)), static_cast<int32_t>(q.size(1)), block_table.data_ptr<int32_t>(),
       static_cast<int32_t>(block_table.size(1)), cache_seqlens.data_ptr<int32_t>(), static_cast<int32_t>(window_left),
-      static_cast<int32_t>(num_splits), static_cast<float>(softmax_scale), workspace.data_ptr(), ws_bytes,
-      current_stream(q));
+      static_cast<int32_t>(num_splits), static_cast<float>(softmax_scale), group_rows, shared_ptr,
+      workspace.data_ptr(), ws_bytes, ARENO_STAGE_ALL, current_stream(q));
   check_status(status, op);
   return out;
 }
@@ -146,7 +159,7 @@ at::Tensor paged_decode_forward(at::Tensor q, at::Tensor k_update, at::Tensor v_
                                 at::Tensor v_cache, at::Tensor block_table, at::Tensor cache_seqlens,
                                 int64_t window_left, int64_t num_splits, double softmax_scale) {
   return paged_decode_forward_impl(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, window_left,
-                                   num_splits, softmax_scale, c10::nullopt, c10::nullopt);
+                                   num_splits, softmax_scale, c10::nullopt, c10::nullopt, 0, c10::nullopt);
 }
 
 at::Tensor varlen_forward(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor cu_seqlens, int64_t window_left,

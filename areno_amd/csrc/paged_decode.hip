@@ -128,10 +128,12 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_kernel(Decod
   }
 }
 
-// Merge of the MFMA path's partials: the units that own tiles of sequence b wrote slots (unit + b); units that
-// own no tile at all are skipped.  One wave per (sequence, q head): lanes first fetch the (m, l) pairs of up to 64
-// slots in parallel and agree on the maximum, then every lane accumulates its share of the head dimension with
-// all partial loads of a group of four slots in flight together (the loop has no loop-carried memory dependence).
+// Merge of the MFMA path's partials.  The units that own tiles of an item wrote one partial each: a per-row item
+// into slot (unit + row) of the per-row region, a shared-prefix item (grouped mode) into slot (unit + item) of the
+// shared region, where the row's head sits in column (row - first row) * G + head of its kv head.  One wave per
+// (row, q head) gathers the candidates of both kinds: lanes first fetch up to 64 (m, l) pairs in parallel and agree
+// on the maximum, then every lane accumulates its share of the head dimension with the partial loads of a group of
+// four candidates in flight together (the loop has no loop-carried memory dependence).
 __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel(MfmaDecodeParams mp) {
   const DecodeParams& p = mp.d;
   const int lane = threadIdx.x & (kWave - 1);
@@ -140,34 +142,71 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   const int b = row / p.q_heads;
   const int h = row - b * p.q_heads;
   const int d = p.head_dim;
+  const int num_items = mp.num_shared + p.batch;
   const UnitGeometry geo =
-      make_unit_geometry(mp.plan[p.batch], mp.num_pieces, mp.max_small, mp.static_share, mp.min_unit_tiles);
-  const int u_lo = geo.unit_of(mp.plan[b]);
-  const int u_hi = geo.unit_of(mp.plan[b + 1] - 1);
+      make_unit_geometry(mp.plan[num_items], mp.num_pieces, mp.max_small, mp.static_share, mp.min_unit_tiles);
+  // the row's own item (always at least one tile) ...
+  const int v_own = mp.num_shared + b;
+  const int own_lo = geo.unit_of(mp.plan[v_own]);
+  const int own_n = geo.unit_of(mp.plan[v_own + 1] - 1) - own_lo + 1;
+  // ... and the shared item of its sub-group, if it has tiles
+  int sh_lo = 0, sh_n = 0, sh_item = 0, sh_col = 0;
+  if (mp.num_shared > 0) {
+    const int gi = b / mp.group_rows;
+    const int j = (b - gi * mp.group_rows) / mp.cols_seqs;
+    sh_item = gi * mp.subs_per_group + j;
+    const int first_row = gi * mp.group_rows + j * mp.cols_seqs;
+    const int kvh = h / p.group;
+    sh_col = kvh * 16 + (b - first_row) * p.group + (h - kvh * p.group);
+    if (mp.plan[sh_item + 1] > mp.plan[sh_item]) {
+      sh_lo = geo.unit_of(mp.plan[sh_item]);
+      sh_n = geo.unit_of(mp.plan[sh_item + 1] - 1) - sh_lo + 1;
+    }
+  }
+  const int total = own_n + sh_n;
+  // candidate c: the unit it belongs to, and where its (m, l) pair and its accumulator row are
+  auto unit_of_candidate = [&](int c) { return c < own_n ? own_lo + c : sh_lo + (c - own_n); };
+  auto locate = [&](int c, const float*& ml, const float*& acc_row) {
+    const int u = unit_of_candidate(c);
+    if (c < own_n) {
+      const int64_t prow = static_cast<int64_t>(u + b) * p.q_heads + h;
+      ml = p.part_ml + prow * 2;
+      acc_row = p.part_acc + prow * d;
+    } else {
+      const int64_t prow = static_cast<int64_t>(u + sh_item) * p.kv_heads * 16 + sh_col;
+      ml = mp.shared_ml + prow * 2;
+      acc_row = mp.shared_acc + prow * d;
+    }
+  };
 
   float acc[kGenericMaxPerLane];
 #pragma unroll
   for (int e = 0; e < kGenericMaxPerLane; ++e) acc[e] = 0.0f;
   float m = kNegInf, l = 0.0f;
-  for (int base = u_lo; base <= u_hi; base += kWave) {
-    // lane j looks at unit base + j
-    const int u = base + lane;
+  for (int base = 0; base < total; base += kWave) {
+    // lane j looks at candidate base + j
     float part_m = kNegInf, part_l = 0.0f;
-    if (u <= u_hi && geo.unit_start(u) != geo.unit_start(u + 1)) {
-      const int64_t prow = static_cast<int64_t>(u + b) * p.q_heads + h;
-      part_m = p.part_ml[prow * 2];
-      part_l = p.part_ml[prow * 2 + 1];
-      if (part_l == 0.0f) part_m = kNegInf;  // a partial without keys contributes nothing
+    if (base + lane < total) {
+      // a unit without tiles wrote nothing: its candidate is absent (weight 0 below)
+      const int u = unit_of_candidate(base + lane);
+      if (geo.unit_start(u) != geo.unit_start(u + 1)) {
+        const float* ml = nullptr;
+        const float* unused = nullptr;
+        locate(base + lane, ml, unused);
+        part_m = ml[0];
+        part_l = ml[1];
+        if (part_l == 0.0f) part_m = kNegInf;  // a partial without keys contributes nothing
+      }
     }
     const float m_new = fmaxf(m, wave_max(part_m));
     const float m_safe = m_new == kNegInf ? 0.0f : m_new;
     const float alpha = fast_exp2(m - m_safe);
-    const float w = fast_exp2(part_m - m_safe);  // 0 for absent slots
+    const float w = fast_exp2(part_m - m_safe);  // 0 for absent candidates
     l = l * alpha + wave_sum(w * part_l);
     m = m_new;
 #pragma unroll
     for (int e = 0; e < kGenericMaxPerLane; ++e) acc[e] *= alpha;
-    const int count = min(kWave, u_hi - base + 1);
+    const int count = min(kWave, total - base);
     for (int j0 = 0; j0 < count; j0 += 4) {
       float wj[4];
       float v[4][kGenericMaxPerLane];
@@ -175,12 +214,15 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
       for (int jj = 0; jj < 4; ++jj) {
         const int j = min(j0 + jj, count - 1);
         wj[jj] = j0 + jj < count ? __shfl(w, j, kWave) : 0.0f;
-        const float* part = p.part_acc + (static_cast<int64_t>(base + j + b) * p.q_heads + h) * d;
+        const float* ml = nullptr;
+        const float* part = nullptr;
+        locate(base + j, ml, part);
+        const bool present = wj[jj] != 0.0f;
 #pragma unroll
         for (int e = 0; e < kGenericMaxPerLane; ++e) {
           const int idx = lane + e * kWave;
-          // slots of units without tiles were never written: read them only with a non-zero weight
-          v[jj][e] = (idx < d && wj[jj] != 0.0f) ? part[idx] : 0.0f;
+          // partials of units without tiles were never written: read only what carries a non-zero weight
+          v[jj][e] = (idx < d && present) ? part[idx] : 0.0f;
         }
       }
 #pragma unroll
@@ -282,13 +324,40 @@ extern "C" int areno_hip_paged_decode(const areno_paged_cache* cache, const void
                                        workspace_bytes, ARENO_STAGE_ALL, stream);
 }
 
-extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, const void* q, const void* k_update,
-                                             const void* v_update, void* out, int32_t q_dtype, int32_t batch,
-                                             int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
-                                             const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
-                                             float softmax_scale, void* workspace, size_t workspace_bytes,
-                                             int32_t stages, void* stream) {
-  using namespace areno;
+namespace areno {
+namespace {
+
+// Sub-groups of a prefix group that can sit side by side in the 16 MFMA columns, or 0 when grouping does not apply.
+int shared_items_for(int batch, int group, int group_rows, int* cols_seqs, int* subs_per_group) {
+  const int cs = group > 0 ? 16 / group : 0;
+  if (group_rows < 2 || cs < 2 || batch % group_rows != 0) return 0;
+  *cols_seqs = cs;
+  *subs_per_group = (group_rows + cs - 1) / cs;
+  return batch / group_rows * *subs_per_group;
+}
+
+// Units (wave pieces) the split kernel can use at most for a kv-head count: what the partial regions are sized for.
+int max_units_for(int kv_heads) {
+  const int heads_per_wg = kv_heads % 4 == 0 ? 4 : (kv_heads % 2 == 0 ? 2 : 1);
+  const int head_groups = kv_heads / heads_per_wg;
+  const int tok_splits = kMfmaWaves / heads_per_wg;
+  const int wgs = (kMfmaWorkgroups + kMfmaTailWorkgroups) / head_groups;
+  return (wgs > 0 ? wgs : 1) * tok_splits + (kMfmaTailWorkgroups / head_groups) * tok_splits;
+}
+
+// plan of the grouped item list (up to one shared item per row on top of the rows), kept 256-byte granular
+size_t grouped_plan_bytes(int batch) { return ((2 * static_cast<size_t>(batch) + 64) * sizeof(int32_t) + 255) / 256 * 256; }
+
+size_t shared_region_bytes(int kv_heads, int head_dim, int num_shared) {
+  const size_t slots = static_cast<size_t>(max_units_for(kv_heads)) + num_shared;
+  return slots * kv_heads * 16 * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
+}
+
+int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_update, const void* v_update, void* out,
+                int32_t q_dtype, int32_t batch, int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
+                const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits, float softmax_scale,
+                int32_t group_rows, const int32_t* shared_lens, void* workspace, size_t workspace_bytes,
+                int32_t stages, void* stream) {
   const char* op = "areno_hip_paged_decode";
   if (int rc = validate_paged_cache(cache, op)) return rc;
   if (q == nullptr || out == nullptr || block_table == nullptr || cache_seqlens == nullptr)
@@ -311,8 +380,16 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
   Chunking ch;
   if (!pick_chunking(cache->block_size, max_blocks, num_splits, &ch))
     return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: block_size * max_blocks out of range", op);
-  const size_t need = areno_hip_paged_decode_workspace_bytes(batch, q_heads, cache->head_dim, cache->block_size,
-                                                             max_blocks, num_splits);
+  const size_t base_need = areno_hip_paged_decode_workspace_bytes(batch, q_heads, cache->head_dim, cache->block_size,
+                                                                  max_blocks, num_splits);
+  // prefix groups: only without a window, on the matrix-core path, when at least two rows fit side by side
+  int cols_seqs = 0, subs_per_group = 0;
+  int num_shared = 0;
+  if (shared_lens != nullptr && window_left < 0)
+    num_shared = shared_items_for(batch, q_heads / cache->kv_heads, group_rows, &cols_seqs, &subs_per_group);
+  const size_t plan_extra = num_shared > 0 ? grouped_plan_bytes(batch) : 0;
+  const size_t need =
+      base_need + plan_extra + (num_shared > 0 ? shared_region_bytes(cache->kv_heads, cache->head_dim, num_shared) : 0);
   if (workspace == nullptr || workspace_bytes < need)
     return fail(ARENO_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", op, need, workspace_bytes);
 
@@ -364,14 +441,17 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
   decode_mfma_fn mfma = nullptr;
   if (aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && num_splits != 1 && p.group <= 16 &&
       batch <= kMfmaMaxBatch) {
+    const bool s16 = cache->scale_dtype == ARENO_DT_F16;
+    const bool grouped = num_shared > 0;
     switch (cache->cache_dtype) {
-      case ARENO_DT_BF16: mfma = decode_mfma_lookup_bf16(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
-      case ARENO_DT_F16: mfma = decode_mfma_lookup_f16(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
-      case ARENO_DT_I8: mfma = decode_mfma_lookup_i8(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
-      case ARENO_DT_FP8_E4M3: mfma = decode_mfma_lookup_fp8(p.head_dim, cache->scale_dtype == ARENO_DT_F16); break;
+      case ARENO_DT_BF16: mfma = decode_mfma_lookup_bf16(p.head_dim, s16, grouped); break;
+      case ARENO_DT_F16: mfma = decode_mfma_lookup_f16(p.head_dim, s16, grouped); break;
+      case ARENO_DT_I8: mfma = decode_mfma_lookup_i8(p.head_dim, s16, grouped); break;
+      case ARENO_DT_FP8_E4M3: mfma = decode_mfma_lookup_fp8(p.head_dim, s16, grouped); break;
       default: break;
     }
   }
+  if (mfma == nullptr) num_shared = 0;  // the other kernels read every row's pages on their own
   // ---- append: folded into the matrix-core split kernel when it can take the new rows as they are, else a launch of
   // its own in front ------------------------------------------------------------------------------------------------
   static const bool allow_fused_append = env_int("ARENO_FUSED_APPEND", 1) != 0;
@@ -417,6 +497,21 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
     mp.d.part_ml = static_cast<float*>(workspace);
     mp.d.part_acc = mp.d.part_ml + slots * q_heads * 2;
     mp.plan = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + part_bytes);
+    mp.shared_lens = shared_lens;
+    mp.group_rows = num_shared > 0 ? group_rows : 1;
+    mp.cols_seqs = num_shared > 0 ? cols_seqs : 1;
+    mp.subs_per_group = num_shared > 0 ? subs_per_group : 1;
+    mp.num_shared = num_shared;
+    mp.shared_ml = nullptr;
+    mp.shared_acc = nullptr;
+    if (num_shared > 0) {
+      // behind the ungrouped layout: the (longer) plan of the item list, then the shared partial region
+      mp.plan = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + base_need);
+      char* region = static_cast<char*>(workspace) + base_need + plan_extra;
+      const size_t shared_slots = static_cast<size_t>(mp.num_pieces) + mp.max_small + num_shared;
+      mp.shared_ml = reinterpret_cast<float*>(region);
+      mp.shared_acc = mp.shared_ml + shared_slots * cache->kv_heads * 16 * 2;
+    }
     if (stages & ARENO_STAGE_SPLIT) {
       hipLaunchKernelGGL(mfma, dim3(mp.static_wgs + extra, head_groups), dim3(kMfmaWaves * kWave), 0, s, mp);
       if (int rc = check_launch(op)) return rc;
@@ -443,4 +538,44 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
   const int rblocks = (batch * q_heads + kReduceRows - 1) / kReduceRows;
   hipLaunchKernelGGL(decode_reduce_kernel, dim3(rblocks), dim3(kReduceRows * kWave), 0, s, p);
   return check_launch(op);
+}
+
+}  // namespace
+}  // namespace areno
+
+extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, const void* q, const void* k_update,
+                                             const void* v_update, void* out, int32_t q_dtype, int32_t batch,
+                                             int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
+                                             const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
+                                             float softmax_scale, void* workspace, size_t workspace_bytes,
+                                             int32_t stages, void* stream) {
+  return areno::decode_impl(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
+                            cache_seqlens, window_left, num_splits, softmax_scale, 0, nullptr, workspace,
+                            workspace_bytes, stages, stream);
+}
+
+extern "C" size_t areno_hip_paged_decode_grouped_workspace_bytes(int32_t batch, int32_t q_heads, int32_t kv_heads,
+                                                                 int32_t head_dim, int32_t block_size,
+                                                                 int32_t max_blocks, int32_t num_splits,
+                                                                 int32_t group_rows) {
+  const size_t base = areno_hip_paged_decode_workspace_bytes(batch, q_heads, head_dim, block_size, max_blocks, num_splits);
+  if (base == 0 || kv_heads <= 0 || q_heads % kv_heads != 0) return 0;
+  int cols_seqs = 0, subs_per_group = 0;
+  const int num_shared = areno::shared_items_for(batch, q_heads / kv_heads, group_rows, &cols_seqs, &subs_per_group);
+  if (num_shared == 0) return base;
+  return base + areno::grouped_plan_bytes(batch) + areno::shared_region_bytes(kv_heads, head_dim, num_shared);
+}
+
+extern "C" int areno_hip_paged_decode_grouped(const areno_paged_cache* cache, const void* q, const void* k_update,
+                                              const void* v_update, void* out, int32_t q_dtype, int32_t batch,
+                                              int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
+                                              const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
+                                              float softmax_scale, int32_t group_rows, const int32_t* shared_lens,
+                                              void* workspace, size_t workspace_bytes, int32_t stages, void* stream) {
+  if (shared_lens != nullptr && (group_rows < 1 || (batch > 0 && batch % group_rows != 0)))
+    return areno::fail(ARENO_ERR_INVALID_ARGUMENT,
+                       "areno_hip_paged_decode_grouped: batch %d is not a multiple of group_rows %d", batch, group_rows);
+  return areno::decode_impl(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
+                            cache_seqlens, window_left, num_splits, softmax_scale, group_rows, shared_lens, workspace,
+                            workspace_bytes, stages, stream);
 }

@@ -268,6 +268,11 @@ def make_decode_workload(
         logical_tokens=int((lengths + 1).sum()),
         meta={"seed": seed, "pool_blocks": nb, "used_blocks": next_block},
     )
+    if shared_prefix_blocks is not None:
+        # what the scheduler knows about the batch: rows per prompt and tokens of each prompt's shared pages
+        w.meta["prefix_group_rows"] = int(group_size)
+        w.meta["shared_prefix_lens"] = torch.tensor([int(n) * bs for n in shared_prefix_blocks], dtype=torch.int32,
+                                                    device=device)  # fmt: skip
     if poison:
         poison_unused_slots(w)
     return w
@@ -299,7 +304,8 @@ def cfg2_qwen7b_int8(**kw) -> DecodeWorkload:
 
 
 def cfg3_rollout(kv: str = "fp8", *, device="cpu", seed: int = 1003, prompts: int = 32, samples: int = 8,
-                 prefix_lo=256, prefix_hi=2048, median=1000.0, sigma=1.0, cap=32768, **kw) -> DecodeWorkload:  # fmt: skip
+                 prefix_lo=256, prefix_hi=2048, median=1000.0, sigma=1.0, cap=32768, hq: int = 32, hkv: int = 8,
+                 **kw) -> DecodeWorkload:  # fmt: skip
     """RL-rollout decode: ``prompts x samples`` rows, samples of a prompt share the prompt's full pages."""
     g = _gen(seed + 1)
     bs = 16
@@ -309,7 +315,7 @@ def cfg3_rollout(kv: str = "fp8", *, device="cpu", seed: int = 1003, prompts: in
     lengths = prefix.repeat_interleave(samples) + cont
     shared = [int(p) // bs for p in prefix]
     return make_decode_workload(
-        f"cfg3-rollout-{kv}", seed=seed, batch=prompts * samples, hq=32, hkv=8, d=128, bs=bs, kv=kv, lengths=lengths,
+        f"cfg3-rollout-{kv}", seed=seed, batch=prompts * samples, hq=hq, hkv=hkv, d=128, bs=bs, kv=kv, lengths=lengths,
         device=device, shared_prefix_blocks=shared, group_size=samples, **kw,
     )  # fmt: skip
 

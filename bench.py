@@ -60,9 +60,12 @@ def _step(w, pool):
     from areno_amd.accel import attention as ops
 
     kc, vc, ks, vs = pool
+    groups = {}
+    if "shared_prefix_lens" in w.meta:  # what the rollout scheduler knows: rows per prompt, shared tokens per prompt
+        groups = dict(prefix_group_rows=w.meta["prefix_group_rows"], shared_prefix_lens=w.meta["shared_prefix_lens"])
     return ops.areno_paged_causal_attention_decode(
         w.q, w.k_update, w.v_update, kc, vc, w.block_table, w.cache_seqlens,
-        softmax_scale=w.softmax_scale, k_scale=ks, v_scale=vs,
+        softmax_scale=w.softmax_scale, k_scale=ks, v_scale=vs, **groups,
     )  # fmt: skip
 
 
@@ -142,7 +145,12 @@ def measure_decode(w, steps, warmup, *, kernel_iters=60):
 
     # ---- per-kernel durations: events on the launch stream around back-to-back launches through the C ABI ---
     b, hq, hkv, d, bs = w.shape
-    ws_bytes = cabi.decode_workspace_bytes(b, hq, d, bs, w.block_table.shape[1])
+    group_rows = w.meta.get("prefix_group_rows")
+    shared_lens = w.meta.get("shared_prefix_lens")
+    if shared_lens is None:
+        ws_bytes = cabi.decode_workspace_bytes(b, hq, d, bs, w.block_table.shape[1])
+    else:
+        ws_bytes = cabi.decode_grouped_workspace_bytes(b, hq, hkv, d, bs, w.block_table.shape[1], group_rows)
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=w.q.device)
     caches = [cabi.describe_cache(*pool) for pool in pools]
     out2 = torch.empty_like(w.q)
@@ -150,7 +158,8 @@ def measure_decode(w, steps, warmup, *, kernel_iters=60):
     def time_stage(stage):
         def launch(i):
             cabi.paged_decode(caches[i % copies], w.q, w.k_update, w.v_update, out2, w.block_table, w.cache_seqlens,
-                              workspace, softmax_scale=w.softmax_scale, stages=stage)  # fmt: skip
+                              workspace, softmax_scale=w.softmax_scale, stages=stage, group_rows=group_rows,
+                              shared_lens=shared_lens)  # fmt: skip
 
         for i in range(copies):
             launch(i)

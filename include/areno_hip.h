@@ -125,6 +125,29 @@ int areno_hip_paged_decode_stages(const areno_paged_cache* cache, const void* q,
                                   size_t workspace_bytes, int32_t stages, void* stream);
 
 /*
+ * The decode op for batches whose rows come in prefix groups (the samples of one prompt in an RL rollout share the
+ * prompt's pages: identical block ids for the prefix).  Rows [i * group_rows, (i + 1) * group_rows) share the pages
+ * of their first shared_lens[i] tokens; the kernel reads those pages once for as many rows as fit side by side in
+ * the 16 matrix-core columns (16 / (q_heads / kv_heads)) instead of once per row.  Same results as
+ * areno_hip_paged_decode up to the order of the fp32 merges.  No counterpart in the reference, which reads every
+ * row's history on its own (areno/accel/csrc/attention.cu:555-654).
+ *   shared_lens   device [batch / group_rows] int32; each value is clipped to what every row of the group has cached
+ *                 and cut to a multiple of 32 tokens; NULL (or a window, or fewer than two rows side by side) makes
+ *                 this areno_hip_paged_decode
+ *   workspace     at least areno_hip_paged_decode_grouped_workspace_bytes(...) bytes
+ *   stages        ARENO_STAGE_* mask as in areno_hip_paged_decode_stages (ARENO_STAGE_ALL for the op)
+ */
+size_t areno_hip_paged_decode_grouped_workspace_bytes(int32_t batch, int32_t q_heads, int32_t kv_heads,
+                                                      int32_t head_dim, int32_t block_size, int32_t max_blocks,
+                                                      int32_t num_splits, int32_t group_rows);
+int areno_hip_paged_decode_grouped(const areno_paged_cache* cache, const void* q, const void* k_update,
+                                   const void* v_update, void* out, int32_t q_dtype, int32_t batch, int32_t q_heads,
+                                   const int32_t* block_table, int32_t max_blocks, const int32_t* cache_seqlens,
+                                   int32_t window_left, int32_t num_splits, float softmax_scale, int32_t group_rows,
+                                   const int32_t* shared_lens, void* workspace, size_t workspace_bytes,
+                                   int32_t stages, void* stream);
+
+/*
  * Packed causal self-attention over new tokens only, GQA without expanding KV:
  * areno_varlen_causal_attention_forward_cuda (areno/accel/csrc/attention.cu:813-861; pybind name
  * areno_varlen_causal_attention_forward, extension.cpp:182).  Token t of the sequence starting at

@@ -28,7 +28,9 @@ def lib():
 def test_header_declares_the_expected_entry_points():
     names = _declared_functions()
     for required in ("areno_hip_cache_write", "areno_hip_cache_write_decode", "areno_hip_paged_decode",
-                     "areno_hip_paged_decode_workspace_bytes", "areno_hip_varlen_attention",
+                     "areno_hip_paged_decode_workspace_bytes", "areno_hip_paged_decode_grouped",
+                     "areno_hip_paged_decode_grouped_workspace_bytes", "areno_hip_qk_norm_rope_cache_write",
+                     "areno_hip_varlen_attention",
                      "areno_hip_paged_varlen_prefill", "areno_hip_prefill_workspace_bytes", "areno_hip_abi_version"):  # fmt: skip
         assert required in names
 

@@ -158,3 +158,61 @@ def test_error_behaviour_matches_the_reference_shim():
     empty = ops.areno_paged_causal_attention_decode(w.q[:0], w.k_update[:0], w.v_update[:0], w.k_cache, w.v_cache,
                                                     w.block_table[:0], w.cache_seqlens[:0])  # fmt: skip
     assert empty.shape == (0, 8, 64)
+
+
+# ---- prefix groups: shared pages read once for several rows --------------------------------------------------------
+def _grouped_decode(w, **kw):
+    return ops.areno_paged_causal_attention_decode(
+        w.q, w.k_update, w.v_update, w.k_cache, w.v_cache, w.block_table, w.cache_seqlens,
+        softmax_scale=w.softmax_scale, k_scale=w.k_scale, v_scale=w.v_scale,
+        prefix_group_rows=w.meta["prefix_group_rows"], shared_prefix_lens=w.meta["shared_prefix_lens"], **kw,
+    )  # fmt: skip
+
+
+@pytest.mark.parametrize("kv,hq,hkv,samples", [("fp8", 32, 8, 8), ("int8", 28, 4, 4), ("bf16", 8, 2, 3), ("fp8", 8, 8, 5)])
+def test_prefix_groups_match_the_plain_op_and_the_oracle(kv, hq, hkv, samples):
+    """Rollout batches at reduced size: 4 / 2 / 4 / 16 rows side by side, groups that do not fill the columns, prompts
+    shorter than a tile (nothing to share) next to long ones."""
+    w = workloads.cfg3_rollout(kv, device=DEV, prompts=6, samples=samples, prefix_lo=8, prefix_hi=700, median=120.0,
+                               cap=900, quantize_fn=gpu_quantize, seed=77, hq=hq, hkv=hkv, poison=True)  # fmt: skip
+    snapshot = tuple(None if t is None else t.clone() for t in (w.k_cache, w.v_cache, w.k_scale, w.v_scale))
+    plain = run_decode(w)
+    after_plain = tuple(None if t is None else t.clone() for t in (w.k_cache, w.v_cache, w.k_scale, w.v_scale))
+    for dst, src in zip((w.k_cache, w.v_cache, w.k_scale, w.v_scale), snapshot):
+        if dst is not None:
+            dst.copy_(src)
+    grouped = _grouped_decode(w)
+    assert_close(grouped, expected_decode(w), *tolerances(kv), what=f"grouped {kv} vs oracle")
+    assert_close(grouped, plain.cpu().float(), 2e-3, what=f"grouped {kv} vs plain op")
+    for a, b, name in zip((w.k_cache, w.v_cache, w.k_scale, w.v_scale), after_plain, ("k", "v", "k_scale", "v_scale")):
+        if a is not None:
+            same = a.view(torch.uint8) == b.view(torch.uint8)
+            assert bool(same.all()), f"{name}: the append differs between the grouped and the plain op"
+
+
+def test_prefix_groups_clip_an_overstated_shared_length():
+    """shared_prefix_lens larger than what a row has cached is clipped to the shortest row of the group."""
+    w = workloads.cfg3_rollout("fp8", device=DEV, prompts=3, samples=4, prefix_lo=64, prefix_hi=200, median=50.0,
+                               cap=300, quantize_fn=gpu_quantize, seed=78, hq=8, hkv=2)  # fmt: skip
+    # claim far more than the prompts hold: only identical pages may be merged, so this must still be exact whenever
+    # the claim is cut back to the rows' cached lengths (rows of a group differ only behind the prompt here)
+    w.meta["shared_prefix_lens"] = w.meta["shared_prefix_lens"].clone()
+    w.meta["shared_prefix_lens"][1] = 0  # and one group that shares nothing
+    out = _grouped_decode(w)
+    assert_close(out, expected_decode(w), *tolerances("fp8"), what="clipped shared length")
+
+
+def test_prefix_groups_argument_checks():
+    w = workloads.cfg3_rollout("fp8", device=DEV, prompts=2, samples=4, prefix_lo=64, prefix_hi=100, median=30.0, cap=100,
+                               quantize_fn=gpu_quantize, seed=79, hq=8, hkv=2)  # fmt: skip
+    with pytest.raises(ValueError, match="together"):
+        ops.areno_paged_causal_attention_decode(w.q, w.k_update, w.v_update, w.k_cache, w.v_cache, w.block_table,
+                                                w.cache_seqlens, k_scale=w.k_scale, v_scale=w.v_scale,
+                                                prefix_group_rows=4)  # fmt: skip
+    with pytest.raises(ValueError, match="multiple of prefix_group_rows"):
+        ops.areno_paged_causal_attention_decode(w.q, w.k_update, w.v_update, w.k_cache, w.v_cache, w.block_table,
+                                                w.cache_seqlens, k_scale=w.k_scale, v_scale=w.v_scale,
+                                                prefix_group_rows=3, shared_prefix_lens=w.meta["shared_prefix_lens"])  # fmt: skip
+    # a window switches the grouping off, the result is the plain op's
+    out = _grouped_decode(w, window_left=40)
+    assert_close(out, expected_decode(w, window_left=40), *tolerances("fp8"), what="window with groups")
