@@ -658,9 +658,12 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
   while (u_hi + 1 < p.units && unit_start_step(total, u_hi + 1, p.units) <= item_x1 - 1) ++u_hi;
 
   const int q_begin = p.cu_seqlens_q[pos.seq];
-  // thread -> (row, half of the head dim), 128 rows per pass
+  // thread -> (row, half of the head dim), 128 rows per pass.  Per unit all of a thread's accumulator loads are issued
+  // together (no store in between), the normalised row is written once at the end.
+  constexpr int kMaxChunks = 128 / 2 / 4;  // float4 chunks of half a row at the largest head dim (128)
   const int half = tid & 1;
   const int dh = d / 2;
+  const int chunks = dh / 4;
   for (int r = tid >> 1; r < kRowsPerWg; r += kPrefillThreads / 2) {
     const int t = r >> p.group_shift;
     const int hh = r & (p.group_pad - 1);
@@ -675,33 +678,43 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
       if (pl != 0.0f) m = fmaxf(m, pm);
     }
     const float m_safe = m == kNegInf ? 0.0f : m;
+    float4_t o[kMaxChunks];
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) o[c] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    float lsum = 0.0f;
+    for (int u = unit; u <= u_hi; ++u) {
+      if (unit_start_step(total, u, p.units) == unit_start_step(total, u + 1, p.units)) continue;
+      const int slot = 2 * u + ((u == unit && pos.item_x0 > x_begin) ? 1 : 0);
+      const int64_t prow = (static_cast<int64_t>(slot) * p.kv_heads + kvh) * kRowsPerWg + r;
+      const float pl = p.part_ml[prow * 2 + 1];
+      if (pl == 0.0f) continue;  // a partial without visible keys
+      const float w = fast_exp2(p.part_ml[prow * 2] - m_safe);
+      lsum += w * pl;
+      const float4_t* src = reinterpret_cast<const float4_t*>(p.part_acc + prow * d + half * dh);
+      float4_t a[kMaxChunks];
+#pragma unroll
+      for (int c = 0; c < kMaxChunks; ++c) a[c] = c < chunks ? src[c] : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int c = 0; c < kMaxChunks; ++c) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[c][j] += w * a[c][j];
+      }
+    }
+    const float inv = 1.0f / lsum;
     const int64_t out_elem =
         (static_cast<int64_t>(q_begin + item.tok0 + t) * p.q_heads + kvh * p.group + hh) * d + half * dh;
-    for (int e0 = 0; e0 < dh; e0 += 4) {
-      float4_t o = {0.0f, 0.0f, 0.0f, 0.0f};
-      float lsum = 0.0f;
-      for (int u = unit; u <= u_hi; ++u) {
-        if (unit_start_step(total, u, p.units) == unit_start_step(total, u + 1, p.units)) continue;
-        const int slot = 2 * u + ((u == unit && pos.item_x0 > x_begin) ? 1 : 0);
-        const int64_t prow = (static_cast<int64_t>(slot) * p.kv_heads + kvh) * kRowsPerWg + r;
-        const float pl = p.part_ml[prow * 2 + 1];
-        if (pl == 0.0f) continue;  // a partial without visible keys
-        const float w = fast_exp2(p.part_ml[prow * 2] - m_safe);
-        lsum += w * pl;
-        const float4_t a = *reinterpret_cast<const float4_t*>(p.part_acc + prow * d + half * dh + e0);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) o[j] += w * a[j];
-      }
-      const float inv = 1.0f / lsum;
+    for (int c = 0; c < kMaxChunks; ++c) {
+      if (c >= chunks) continue;
       uint32_t lo, hi;
       if (p.q_dtype == ARENO_DT_BF16) {
-        lo = float_to_bf16_bits(o[0] * inv) | (float_to_bf16_bits(o[1] * inv) << 16);
-        hi = float_to_bf16_bits(o[2] * inv) | (float_to_bf16_bits(o[3] * inv) << 16);
+        lo = float_to_bf16_bits(o[c][0] * inv) | (float_to_bf16_bits(o[c][1] * inv) << 16);
+        hi = float_to_bf16_bits(o[c][2] * inv) | (float_to_bf16_bits(o[c][3] * inv) << 16);
       } else {
-        lo = float_to_f16_bits(o[0] * inv) | (float_to_f16_bits(o[1] * inv) << 16);
-        hi = float_to_f16_bits(o[2] * inv) | (float_to_f16_bits(o[3] * inv) << 16);
+        lo = float_to_f16_bits(o[c][0] * inv) | (float_to_f16_bits(o[c][1] * inv) << 16);
+        hi = float_to_f16_bits(o[c][2] * inv) | (float_to_f16_bits(o[c][3] * inv) << 16);
       }
-      *reinterpret_cast<uint2_t*>(static_cast<char*>(p.out) + (out_elem + e0) * 2) = uint2_t{lo, hi};
+      *reinterpret_cast<uint2_t*>(static_cast<char*>(p.out) + (out_elem + 4 * c) * 2) = uint2_t{lo, hi};
     }
   }
 }
