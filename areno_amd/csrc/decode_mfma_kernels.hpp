@@ -31,6 +31,15 @@
 // the offsets are removed algebraically (1152 * sum(q) per head, 1152 * sum(p) per head).  fp8 uses
 // v_cvt_scalef32_pk_f16_fp8 with scale 1 (exact).  bf16 / fp16 caches feed the MFMA directly.
 //
+// The single-token append (areno/accel/csrc/attention.cu:526-553) rides along: the wave that stages the last tile of a
+// sequence takes the newest token's row from k_update / v_update instead of the not yet written page slot, quantizes
+// it with the cache writer's closed form and stores it into the page.
+//
+// GROUPED instantiation (batches whose rows come in prefix groups, e.g. the samples of one prompt): the item list is
+// [shared prefix of every sub-group of rows that fits side by side in the 16 MFMA columns] + [the rest of every
+// row]; a shared item is streamed once with column = (row in sub-group, head) and leaves its partials in a second
+// region, the merge kernel adds them to the row's own.
+//
 // Semantics: the reference's split kernel (areno/accel/csrc/attention.cu:555-654) -- keys [first_allowed, L_b],
 // q head h <-> kv head h / G, fp32 accumulation.
 #pragma once
