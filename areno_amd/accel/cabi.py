@@ -43,6 +43,23 @@ class PagedCache(ctypes.Structure):
     ]
 
 
+class BlockTables(ctypes.Structure):
+    """``struct areno_block_tables``."""
+
+    _fields_ = [
+        ("table", ctypes.c_void_p),
+        ("row_blocks", ctypes.c_void_p),
+        ("free_ring", ctypes.c_void_p),
+        ("state", ctypes.c_void_p),
+        ("max_rows", ctypes.c_int32),
+        ("max_blocks", ctypes.c_int32),
+        ("num_blocks", ctypes.c_int32),
+        ("block_size", ctypes.c_int32),
+    ]
+
+
+PAD_LAST_BLOCK, PAD_SCRATCH_BLOCK = 0, 1
+
 _LIB: ctypes.CDLL | None = None
 _P, _I32, _I64, _F, _SZ = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_size_t
 
@@ -72,6 +89,13 @@ def lib() -> ctypes.CDLL:
         handle.areno_hip_paged_varlen_prefill.argtypes = [_P, _P, _P, _I32, _I64, _I32, _I32, _P, _I32, _P, _P, _I32, _F, _P, _SZ, _P]  # fmt: skip
         handle.areno_hip_prefill_workspace_bytes.restype = _SZ
         handle.areno_hip_prefill_workspace_bytes.argtypes = [_I32, _I32]
+        handle.areno_hip_block_tables_init.argtypes = [_P, _P]
+        handle.areno_hip_block_tables_reserve.argtypes = [_P, _P, _P, _I32, _P]
+        handle.areno_hip_block_tables_ensure_decode.argtypes = [_P, _P, _P, _I32, _P]
+        handle.areno_hip_block_tables_release.argtypes = [_P, _P, _I32, _P]
+        handle.areno_hip_block_tables_gather.argtypes = [_P, _P, _I32, _I32, _P, _P]
+        handle.areno_hip_block_tables_decode_step.argtypes = [_P, _P, _P, _I32, _I32, _P, _P]
+        handle.areno_hip_block_tables_prefill_slots.argtypes = [_P, _P, _P, _P, _I32, _I64, _P, _P, _P, _P]
         _LIB = handle
     return _LIB
 
@@ -154,3 +178,48 @@ def paged_varlen_prefill(cache: PagedCache, q, out, block_table, cu_seqlens_q, c
         workspace.numel() if workspace_bytes is None else int(workspace_bytes),
         current_stream_ptr() if stream is None else stream,
     ))  # fmt: skip
+
+
+def describe_block_tables(table, row_blocks, free_ring, state, block_size: int) -> BlockTables:
+    """Descriptor over four int32 device tensors: table [rows, max_blocks], row_blocks [rows], free_ring [pages],
+    state [4]."""
+    return BlockTables(table.data_ptr(), row_blocks.data_ptr(), free_ring.data_ptr(), state.data_ptr(),
+                       table.shape[0], table.shape[1], free_ring.shape[0], block_size)  # fmt: skip
+
+
+def block_tables_init(bt: BlockTables) -> int:
+    return lib().areno_hip_block_tables_init(ctypes.byref(bt), current_stream_ptr())
+
+
+def block_tables_reserve(bt: BlockTables, rows, token_counts) -> int:
+    return lib().areno_hip_block_tables_reserve(ctypes.byref(bt), rows.data_ptr(), token_counts.data_ptr(),
+                                                rows.numel(), current_stream_ptr())  # fmt: skip
+
+
+def block_tables_ensure_decode(bt: BlockTables, rows, next_positions) -> int:
+    return lib().areno_hip_block_tables_ensure_decode(ctypes.byref(bt), rows.data_ptr(), next_positions.data_ptr(),
+                                                      rows.numel(), current_stream_ptr())  # fmt: skip
+
+
+def block_tables_release(bt: BlockTables, rows) -> int:
+    return lib().areno_hip_block_tables_release(ctypes.byref(bt), rows.data_ptr(), rows.numel(), current_stream_ptr())
+
+
+def block_tables_gather(bt: BlockTables, rows, pad_mode: int, out_table) -> int:
+    return lib().areno_hip_block_tables_gather(ctypes.byref(bt), rows.data_ptr(), rows.numel(), pad_mode,
+                                               out_table.data_ptr(), current_stream_ptr())  # fmt: skip
+
+
+def block_tables_decode_step(bt: BlockTables, rows, next_positions, pad_mode: int, out_table) -> int:
+    return lib().areno_hip_block_tables_decode_step(ctypes.byref(bt), rows.data_ptr(), next_positions.data_ptr(),
+                                                    rows.numel(), pad_mode, out_table.data_ptr(),
+                                                    current_stream_ptr())  # fmt: skip
+
+
+def block_tables_prefill_slots(bt: BlockTables, rows, cursors, cu_seqlens, tokens: int, out_ids, out_offsets,
+                               out_positions=None) -> int:  # fmt: skip
+    return lib().areno_hip_block_tables_prefill_slots(
+        ctypes.byref(bt), rows.data_ptr(), cursors.data_ptr(), cu_seqlens.data_ptr(), rows.numel(), tokens,
+        out_ids.data_ptr(), out_offsets.data_ptr(), None if out_positions is None else out_positions.data_ptr(),
+        current_stream_ptr(),
+    )

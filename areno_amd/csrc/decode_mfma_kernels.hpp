@@ -297,9 +297,14 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
 #ifdef ARENO_TRACE
   const int trace_wave = (blockIdx.y * gridDim.x + blockIdx.x) * NW + wave;
   int trace_n = 2;
-  if (mp.trace && lane == 0) mp.trace[trace_wave * 16] = wall_clock64();
+  if (mp.trace && lane == 0) {
+    // start time, and in word 15 where the wave runs: XCC id (hardware register 20) above the HW_ID word (register 4)
+    mp.trace[trace_wave * 16] = wall_clock64();
+    mp.trace[trace_wave * 16 + 15] = (static_cast<unsigned long long>(__builtin_amdgcn_s_getreg((31 << 11) | 20)) << 32) |
+                                     static_cast<unsigned int>(__builtin_amdgcn_s_getreg((31 << 11) | 4));
+  }
 #define ARENO_TRACE_POINT()                                                                   \
-  if (mp.trace && lane == 0 && trace_n < 16) mp.trace[trace_wave * 16 + trace_n++] = wall_clock64()
+  if (mp.trace && lane == 0 && trace_n < 15) mp.trace[trace_wave * 16 + trace_n++] = wall_clock64()
 #else
 #define ARENO_TRACE_POINT()
 #endif

@@ -325,6 +325,139 @@ std::vector<at::Tensor> qk_norm_rope_cache_write(at::Tensor q, at::Tensor k, at:
   return {q_out, k_out};
 }
 
+// ---- device-resident block tables ------------------------------------------------------------------------------------
+// state tensors of one pool: table [max_rows, max_blocks], row_blocks [max_rows], free_ring [num_blocks], state [4],
+// all int32 on one device
+areno_block_tables describe_tables(const at::Tensor& table, const at::Tensor& row_blocks, const at::Tensor& free_ring,
+                                   const at::Tensor& state, int64_t block_size, const char* op) {
+  for (const at::Tensor* t : {&table, &row_blocks, &free_ring, &state}) {
+    TORCH_CHECK(t->is_cuda() && t->is_contiguous() && t->scalar_type() == at::kInt, op,
+                " block-table state must be contiguous CUDA int32 tensors");
+    TORCH_CHECK(t->device() == table.device(), op, " block-table state must live on one device");
+  }
+  TORCH_CHECK(table.dim() == 2 && row_blocks.dim() == 1 && row_blocks.size(0) == table.size(0) && free_ring.dim() == 1 &&
+                  state.dim() == 1 && state.size(0) == 4,
+              op, " block-table state has the wrong shape");
+  TORCH_CHECK(block_size > 0 && table.size(0) > 0 && table.size(1) > 0 && free_ring.size(0) > 0, op,
+              " block-table sizes must be positive");
+  areno_block_tables bt;
+  bt.table = table.data_ptr<int32_t>();
+  bt.row_blocks = row_blocks.data_ptr<int32_t>();
+  bt.free_ring = free_ring.data_ptr<int32_t>();
+  bt.state = state.data_ptr<int32_t>();
+  bt.max_rows = static_cast<int32_t>(table.size(0));
+  bt.max_blocks = static_cast<int32_t>(table.size(1));
+  bt.num_blocks = static_cast<int32_t>(free_ring.size(0));
+  bt.block_size = static_cast<int32_t>(block_size);
+  return bt;
+}
+
+void check_rows(const at::Tensor& rows, const at::Tensor& like, const char* op) {
+  TORCH_CHECK(rows.is_cuda() && rows.device() == like.device() && rows.is_contiguous() &&
+                  rows.scalar_type() == at::kLong && rows.dim() == 1,
+              op, " rows must be a contiguous CUDA int64 vector on the tables' device");
+}
+
+void check_counts(const at::Tensor& v, int64_t n, const at::Tensor& like, const char* op, const char* name) {
+  TORCH_CHECK(v.is_cuda() && v.device() == like.device() && v.is_contiguous() && v.scalar_type() == at::kInt &&
+                  v.dim() == 1 && v.size(0) == n,
+              op, " ", name, " must be a contiguous CUDA int32 vector of ", n, " entries");
+}
+
+void block_tables_init(at::Tensor table, at::Tensor row_blocks, at::Tensor free_ring, at::Tensor state,
+                       int64_t block_size) {
+  const char* op = "areno_block_tables_init";
+  const areno_block_tables bt = describe_tables(table, row_blocks, free_ring, state, block_size, op);
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(table));
+  check_status(areno_hip_block_tables_init(&bt, current_stream(table)), op);
+}
+
+// decode = false: amounts are token counts the rows must hold; decode = true: the positions the rows write next
+void block_tables_reserve(at::Tensor table, at::Tensor row_blocks, at::Tensor free_ring, at::Tensor state,
+                          int64_t block_size, at::Tensor rows, at::Tensor amounts, bool decode) {
+  const char* op = decode ? "areno_block_tables_ensure_decode" : "areno_block_tables_reserve";
+  const areno_block_tables bt = describe_tables(table, row_blocks, free_ring, state, block_size, op);
+  check_rows(rows, table, op);
+  check_counts(amounts, rows.size(0), table, op, decode ? "next_positions" : "token_counts");
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(table));
+  const int32_t n = static_cast<int32_t>(rows.size(0));
+  const int status =
+      decode ? areno_hip_block_tables_ensure_decode(&bt, rows.data_ptr<int64_t>(), amounts.data_ptr<int32_t>(), n,
+                                                    current_stream(table))
+             : areno_hip_block_tables_reserve(&bt, rows.data_ptr<int64_t>(), amounts.data_ptr<int32_t>(), n,
+                                              current_stream(table));
+  check_status(status, op);
+}
+
+void block_tables_release(at::Tensor table, at::Tensor row_blocks, at::Tensor free_ring, at::Tensor state,
+                          int64_t block_size, at::Tensor rows) {
+  const char* op = "areno_block_tables_release";
+  const areno_block_tables bt = describe_tables(table, row_blocks, free_ring, state, block_size, op);
+  check_rows(rows, table, op);
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(table));
+  check_status(areno_hip_block_tables_release(&bt, rows.data_ptr<int64_t>(), static_cast<int32_t>(rows.size(0)),
+                                              current_stream(table)),
+               op);
+}
+
+at::Tensor block_tables_gather(at::Tensor table, at::Tensor row_blocks, at::Tensor free_ring, at::Tensor state,
+                               int64_t block_size, at::Tensor rows, bool pad_scratch,
+                               c10::optional<at::Tensor> out_opt) {
+  const char* op = "areno_block_tables_gather";
+  const areno_block_tables bt = describe_tables(table, row_blocks, free_ring, state, block_size, op);
+  check_rows(rows, table, op);
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(table));
+  at::Tensor out = out_opt.has_value() ? *out_opt : at::empty({rows.size(0), table.size(1)}, table.options());
+  TORCH_CHECK(out.is_cuda() && out.device() == table.device() && out.is_contiguous() && out.scalar_type() == at::kInt &&
+                  out.dim() == 2 && out.size(0) == rows.size(0) && out.size(1) == table.size(1),
+              op, " out must be a contiguous CUDA int32 (rows, max_blocks) tensor");
+  check_status(areno_hip_block_tables_gather(&bt, rows.data_ptr<int64_t>(), static_cast<int32_t>(rows.size(0)),
+                                             pad_scratch ? ARENO_PAD_SCRATCH_BLOCK : ARENO_PAD_LAST_BLOCK,
+                                             out.data_ptr<int32_t>(), current_stream(table)),
+               op);
+  return out;
+}
+
+at::Tensor block_tables_decode_step(at::Tensor table, at::Tensor row_blocks, at::Tensor free_ring, at::Tensor state,
+                                    int64_t block_size, at::Tensor rows, at::Tensor next_positions, bool pad_scratch,
+                                    c10::optional<at::Tensor> out_opt) {
+  const char* op = "areno_block_tables_decode_step";
+  const areno_block_tables bt = describe_tables(table, row_blocks, free_ring, state, block_size, op);
+  check_rows(rows, table, op);
+  check_counts(next_positions, rows.size(0), table, op, "next_positions");
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(table));
+  at::Tensor out = out_opt.has_value() ? *out_opt : at::empty({rows.size(0), table.size(1)}, table.options());
+  TORCH_CHECK(out.is_cuda() && out.device() == table.device() && out.is_contiguous() && out.scalar_type() == at::kInt &&
+                  out.dim() == 2 && out.size(0) == rows.size(0) && out.size(1) == table.size(1),
+              op, " out must be a contiguous CUDA int32 (rows, max_blocks) tensor");
+  check_status(areno_hip_block_tables_decode_step(
+                   &bt, rows.data_ptr<int64_t>(), next_positions.data_ptr<int32_t>(), static_cast<int32_t>(rows.size(0)),
+                   pad_scratch ? ARENO_PAD_SCRATCH_BLOCK : ARENO_PAD_LAST_BLOCK, out.data_ptr<int32_t>(),
+                   current_stream(table)),
+               op);
+  return out;
+}
+
+std::vector<at::Tensor> block_tables_prefill_slots(at::Tensor table, at::Tensor row_blocks, at::Tensor free_ring,
+                                                   at::Tensor state, int64_t block_size, at::Tensor rows,
+                                                   at::Tensor cursors, at::Tensor cu_seqlens, int64_t tokens) {
+  const char* op = "areno_block_tables_prefill_slots";
+  const areno_block_tables bt = describe_tables(table, row_blocks, free_ring, state, block_size, op);
+  check_rows(rows, table, op);
+  check_counts(cursors, rows.size(0), table, op, "cursors");
+  check_counts(cu_seqlens, rows.size(0) + 1, table, op, "cu_seqlens");
+  TORCH_CHECK(tokens >= 0, op, " negative token count");
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(table));
+  const auto opts = table.options().dtype(at::kLong);
+  at::Tensor ids = at::empty({tokens}, opts), offs = at::empty({tokens}, opts), pos = at::empty({tokens}, opts);
+  check_status(areno_hip_block_tables_prefill_slots(
+                   &bt, rows.data_ptr<int64_t>(), cursors.data_ptr<int32_t>(), cu_seqlens.data_ptr<int32_t>(),
+                   static_cast<int32_t>(rows.size(0)), tokens, ids.data_ptr<int64_t>(), offs.data_ptr<int64_t>(),
+                   pos.data_ptr<int64_t>(), current_stream(table)),
+               op);
+  return {ids, offs, pos};
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -338,5 +471,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "causal varlen prefill over paged (optionally quantized) KV");
   m.def("areno_qk_norm_rope_cache_write", &qk_norm_rope_cache_write,
         "QK RMSNorm + rotary embedding + quantizing KV cache write in one pass");
+  m.def("areno_block_tables_init", &block_tables_init, "device-resident block tables: all pages free");
+  m.def("areno_block_tables_reserve", &block_tables_reserve, "device-resident block tables: pages for prefill / decode");
+  m.def("areno_block_tables_release", &block_tables_release, "device-resident block tables: give rows' pages back");
+  m.def("areno_block_tables_gather", &block_tables_gather, "device-resident block tables: padded table of rows");
+  m.def("areno_block_tables_decode_step", &block_tables_decode_step,
+        "device-resident block tables: pages for the next decode position, then the padded table");
+  m.def("areno_block_tables_prefill_slots", &block_tables_prefill_slots,
+        "device-resident block tables: page id, slot and position of packed prefill tokens");
   m.def("abi_version", &areno_hip_abi_version, "C ABI version of libareno_hip.so");
 }

@@ -200,7 +200,70 @@ def measure_decode(w, steps, warmup, *, kernel_iters=60):
         "parity_max_abs_4rows": parity,
         "graph_replay_matches_eager": graph_ok,
         "kv_tokens": {"logical": w.logical_tokens, "unique": w.unique_tokens},
+        "block_tables": measure_block_tables(w),
     }
+
+
+def measure_block_tables(w, inner=20, repeats=5):
+    """The page bookkeeping of one decode step for the workload's rows: on the device (pages for the next position, then the
+    padded table; replayed from a HIP graph) and the way the reference does it (positions to the host, a walk over Python lists,
+    a new table uploaded; areno/engine/inference.py:561-580), here with the oracle's list code as the port."""
+    import torch
+
+    from areno_amd.engine import DeviceBlockTables
+    from oracle.block_table_ref import RefBlockTables
+
+    dev = w.q.device
+    b, _, _, _, bs = w.shape
+    max_blocks = w.block_table.shape[1]
+    lens = w.cache_seqlens.cpu().tolist()
+    pages_needed = sum(-(-(n + 1) // bs) for n in lens)
+    rows = list(range(b))
+    tables = DeviceBlockTables(pages_needed + b, b, max_blocks, bs, dev)
+    lists = RefBlockTables(pages_needed + b, b, max_blocks, bs)
+    tables.reserve(rows, lens)
+    lists.reserve(rows, lens)
+    rows_dev = torch.arange(b, device=dev)
+    out = torch.empty(b, max_blocks, dtype=torch.int32, device=dev)
+
+    def device_step():
+        tables.decode_step(rows_dev, w.cache_seqlens, out=out)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        device_step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(inner):
+            device_step()
+    samples = []
+    for _ in range(repeats):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        samples.append((time.perf_counter() - t0) / inner * 1e6)
+    us_device = statistics.median(samples)
+
+    def host_step():
+        active = rows_dev.cpu().tolist()
+        positions = w.cache_seqlens.cpu().tolist()
+        lists.ensure_decode(active, positions)
+        table = torch.tensor(lists.gather(active, False), dtype=torch.int32, device=dev)
+        torch.cuda.synchronize()
+        return table
+
+    same = bool(torch.equal(host_step(), out))
+    samples = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        host_step()
+        samples.append((time.perf_counter() - t0) * 1e6)
+    return {"rows": b, "max_blocks": max_blocks, "device_us_per_step": us_device,
+            "host_lists_us_per_step": statistics.median(samples), "tables_equal": same}  # fmt: skip
 
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0

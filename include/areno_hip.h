@@ -209,6 +209,90 @@ int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache, const voi
  */
 size_t areno_hip_prefill_workspace_bytes(int32_t kv_heads, int32_t head_dim);
 
+/*
+ * Device-resident page allocator and block tables.  The reference keeps the free list and the page list of every
+ * running sequence as Python lists (areno/engine/data/rollout_state.py:55-56), walks them on the host each step
+ * and uploads a freshly built rectangular table (areno/engine/inference.py:561-580).  These entry points keep the
+ * same state in device memory and make the same transitions there, in the same order, so a row receives the page
+ * ids the reference would hand out for the same sequence of requests.
+ *   table       device [max_rows, max_blocks] int32: page ids of a row, valid for its first row_blocks[r] columns
+ *   row_blocks  device [max_rows] int32: pages a row owns, 0 = the row is not running
+ *   free_ring   device [num_blocks] int32: FIFO of free page ids
+ *   state       device [4] int32: ring head, free count, status (enum areno_blocks_status, the worst since init),
+ *               index of the first request that was refused or cut short in the call that set the status (-1: none)
+ * Requests of one call are served in index order.  The host never needs `state` to issue the next call; it reads it
+ * when it wants to know that the pool ran dry (the reference raises "paged KV cache exhausted" at that point).
+ */
+typedef struct areno_block_tables {
+  int32_t* table;
+  int32_t* row_blocks;
+  int32_t* free_ring;
+  int32_t* state;
+  int32_t max_rows;
+  int32_t max_blocks;
+  int32_t num_blocks;
+  int32_t block_size;
+} areno_block_tables;
+
+enum areno_blocks_status {
+  ARENO_BLOCKS_OK = 0,
+  ARENO_BLOCKS_EXHAUSTED = 1, /* the free list ran out; the request took what was left, later ones nothing */
+  ARENO_BLOCKS_ROW_FULL = 2,  /* a row asked for more than max_blocks pages; it was cut to max_blocks */
+  ARENO_BLOCKS_BAD_ROW = 3    /* row index out of range, a row named twice in a reserve call, or a row without pages */
+};
+
+enum areno_table_padding {
+  ARENO_PAD_LAST_BLOCK = 0,   /* eager tables: rollout_state.py:282-285 */
+  ARENO_PAD_SCRATCH_BLOCK = 1 /* captured-graph tables: the scratch page id num_blocks, runtime/decode_graph.py:95 */
+};
+
+/* All pages free in id order (rollout_state.py:55), no row running, status OK. */
+int areno_hip_block_tables_init(const areno_block_tables* tables, void* stream);
+
+/*
+ * Prefill admission (rollout_state.py:128-151): row rows[i] must be able to hold token_counts[i] tokens
+ * (cursor + chunk length); missing pages are taken from the head of the free list.  rows device [n] int64, distinct.
+ */
+int areno_hip_block_tables_reserve(const areno_block_tables* tables, const int64_t* rows, const int32_t* token_counts,
+                                   int32_t n, void* stream);
+
+/*
+ * ensure_decode_blocks (rollout_state.py:212-225): a running row whose next position next_positions[i] (device
+ * [n] int32, the decode op's cache_seqlens) starts a page gets that page; other rows, and negative row indices (the
+ * padded rows of a bucketed batch), are left alone.
+ */
+int areno_hip_block_tables_ensure_decode(const areno_block_tables* tables, const int64_t* rows,
+                                         const int32_t* next_positions, int32_t n, void* stream);
+
+/* _free_rollout_rows (inference.py:651-658): the pages of the rows go to the tail of the free list, in row order. */
+int areno_hip_block_tables_release(const areno_block_tables* tables, const int64_t* rows, int32_t n, void* stream);
+
+/*
+ * _block_table_for_active_rows (inference.py:573-580): out_table device [n, max_blocks] int32, row i = pages of
+ * rows[i] right-padded as pad_mode says; a negative rows[i] gives a row of scratch ids (the padded rows of a
+ * captured decode batch, runtime/decode_graph.py:163-174).  n <= 65535.
+ */
+int areno_hip_block_tables_gather(const areno_block_tables* tables, const int64_t* rows, int32_t n, int32_t pad_mode,
+                                  int32_t* out_table, void* stream);
+
+/*
+ * One decode step's bookkeeping in one call: areno_hip_block_tables_ensure_decode followed by
+ * areno_hip_block_tables_gather for the same rows (inference.py:561-580 does the two on the host every step).
+ */
+int areno_hip_block_tables_decode_step(const areno_block_tables* tables, const int64_t* rows,
+                                       const int32_t* next_positions, int32_t n, int32_t pad_mode, int32_t* out_table,
+                                       void* stream);
+
+/*
+ * Per packed prefill token t of sequence i (cu_seqlens[i] <= t < cu_seqlens[i + 1], device [n + 1] int32): position
+ * cursors[i] + t - cu_seqlens[i], its page id and slot (rollout_state.py:141-149).  out_* device [tokens] int64,
+ * the dtype of cache_block_ids / cache_block_offsets / position_ids there; out_positions may be NULL.
+ */
+int areno_hip_block_tables_prefill_slots(const areno_block_tables* tables, const int64_t* rows,
+                                         const int32_t* cursors, const int32_t* cu_seqlens, int32_t n, int64_t tokens,
+                                         int64_t* out_block_ids, int64_t* out_block_offsets, int64_t* out_positions,
+                                         void* stream);
+
 #ifdef __cplusplus
 }
 #endif

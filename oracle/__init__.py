@@ -4,8 +4,11 @@ TEST INFRASTRUCTURE ONLY.  Nothing under ``areno_amd/`` may import this package;
 it is the checker that the HIP kernels are compared against (tests, the smoke
 entry point and the CPU-baseline leg of the benchmark), never a fallback.
 
-Three restatements live here:
+Four restatements live here:
 
+* ``block_table_ref`` -- the page lists of the scheduler state (free list, per-sequence pages,
+  padded tables, prefill slots; ``areno/engine/data/rollout_state.py:55-56,128-151,212-225,282-285``,
+  ``areno/engine/inference.py:573-580,651-658``).
 * ``rope_ref`` -- the layer's steps in front of the path: per-head RMSNorm
   (``areno/accel/csrc/normalization.cu:34-56``) and rotary embedding
   (``areno/engine/layers/rotary.py:17-52``) with the eager ops' roundings.
@@ -40,11 +43,16 @@ ref_rmsnorm                float64 restatement; unit-RMS output for w = 1,
 ref_rope                   position 0 is the identity; pair norms preserved;
                            rope(p1) then rope(p2) == rope(p1 + p2) in float64;
                            complex-multiplication form x * exp(i p w)
+RefBlockTables             the values the reference's scheduler test holds
+                           (tests/test_inference_scheduler_cpu.py:110-156
+                           there); every page free or owned exactly once;
+                           FIFO hand-out and give-back order
+                           (tests/test_block_table_oracle_cpu.py)
 =========================  ====================================================
 
 The reference repository holds no golden vectors, known-answer tests or
-fixtures for this path (its 27 test files are CPU-only and never execute the
-kernels), so there is nothing of the reference's to replay; the reference's
+fixtures for the attention kernels (its 27 test files are CPU-only and never
+execute them), so there is nothing of the reference's to replay there; the reference's
 Python was read, not imported.  The CUDA sources cannot be compiled here (no
 nvcc), so there is no ``oracle/_ref`` build.
 """

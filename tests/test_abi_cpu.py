@@ -31,7 +31,11 @@ def test_header_declares_the_expected_entry_points():
                      "areno_hip_paged_decode_workspace_bytes", "areno_hip_paged_decode_grouped",
                      "areno_hip_paged_decode_grouped_workspace_bytes", "areno_hip_qk_norm_rope_cache_write",
                      "areno_hip_varlen_attention",
-                     "areno_hip_paged_varlen_prefill", "areno_hip_prefill_workspace_bytes", "areno_hip_abi_version"):  # fmt: skip
+                     "areno_hip_paged_varlen_prefill", "areno_hip_prefill_workspace_bytes", "areno_hip_abi_version",
+                     "areno_hip_block_tables_init", "areno_hip_block_tables_reserve",
+                     "areno_hip_block_tables_ensure_decode", "areno_hip_block_tables_release",
+                     "areno_hip_block_tables_gather", "areno_hip_block_tables_decode_step",
+                     "areno_hip_block_tables_prefill_slots"):  # fmt: skip
         assert required in names
 
 

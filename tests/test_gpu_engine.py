@@ -92,3 +92,77 @@ def test_prefill_chunk_decode_loop(kv, hq, hkv, d, dv):
         kc, vc = cache_cpu()
         want = ar.ref_paged_decode(q[0].float(), kc, vc, table, lens + step, -1, scale)[..., :dv]
         assert_close(out[0], want, *tolerances(name), what=f"decode step {step}")
+
+
+def test_loop_driven_by_device_block_tables():
+    """Same loop with the page bookkeeping on the device: tables, write slots and positions come from
+    DeviceBlockTables (no host-built table is uploaded), decode crosses page borders, one sequence finishes and a
+    new one is admitted into the freed pages; outputs against the oracle reading through the device's own table."""
+    from areno_amd.engine import DeviceBlockTables
+    from oracle.block_table_ref import RefBlockTables
+
+    gen = torch.Generator().manual_seed(43)
+    dtype, hq, hkv, d = torch.bfloat16, 8, 2, 64
+    scale = d**-0.5
+    num_blocks, max_rows, max_blocks = 12, 4, 6
+    layer = allocate_kv_caches(1, num_blocks + 1, BS, hkv, d, DEV, dtype, "int8")[0]
+    pages = DeviceBlockTables(num_blocks, max_rows, max_blocks, BS, DEV)
+    lists = RefBlockTables(num_blocks, max_rows, max_blocks, BS)  # the reference's host lists, kept in step
+    backend = build_infer_attention_backend()
+
+    def same_pages():
+        for row in range(max_rows):
+            assert pages.row_pages(row) == lists.row_pages(row), f"row {row}"
+        assert pages.free_list() == lists.free_list() and pages.status() == (0, -1)
+
+    def rand(t, h):
+        return torch.randn(1, t, h, d, generator=gen).to(dtype)
+
+    def call(q, k, v, meta):
+        return backend(q.to(DEV), k.to(DEV), v.to(DEV), layer.k_cache, layer.v_cache, meta, softmax_scale=scale,
+                       k_scale=layer.k_scale, v_scale=layer.v_scale)  # fmt: skip
+
+    def prefill(rows, lens):
+        pages.reserve(rows, lens)
+        lists.reserve(rows, lens)
+        cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+        t = int(cu[-1])
+        ids, offs, pos = pages.prefill_slots(rows, [0] * len(rows), cu, t)
+        assert pos.cpu().tolist() == [p for n in lens for p in range(n)]
+        table = pages.block_table(rows)
+        q, k, v = rand(t, hq), rand(t, hkv), rand(t, hkv)
+        meta = InferMeta(mode="prefill", cu_seqlens=cu.to(DEV), max_seqlen=max(lens), block_table=table,
+                         cache_block_ids=ids, cache_block_offsets=offs)  # fmt: skip
+        out = call(q, k, v, meta)
+        want = ar.ref_varlen(q[0].float(), k[0].float(), v[0].float(), cu, -1, scale)
+        assert_close(out[0], want, *tolerances("bf16"), what="prefill")
+
+    def decode(rows, lens_dev, steps):
+        rows_dev = torch.tensor(rows, device=DEV)
+        for step in range(steps):
+            pages.ensure_decode(rows_dev, lens_dev)
+            lists.ensure_decode(rows, lens_dev.cpu().tolist())
+            table = pages.block_table(rows_dev)
+            assert table.cpu().tolist() == lists.gather(rows, False)
+            q, k, v = rand(len(rows), hq), rand(len(rows), hkv), rand(len(rows), hkv)
+            meta = InferMeta(mode="decode", cache_seqlens=lens_dev, block_table=table)
+            out = call(q, k, v, meta)
+            kc, vc = dequant_cpu(layer.k_cache, layer.k_scale), dequant_cpu(layer.v_cache, layer.v_scale)
+            want = ar.ref_paged_decode(q[0].float(), kc, vc, table.cpu(), lens_dev.cpu(), -1, scale)
+            assert_close(out[0], want, *tolerances("int8"), what=f"decode step {step}")
+            lens_dev += 1
+        pages.check()
+
+    prefill([2, 0, 3], [30, 16, 5])
+    lens_dev = torch.tensor([30, 16, 5], dtype=torch.int32, device=DEV)
+    decode([2, 0, 3], lens_dev, 4)  # row 0 opens its second page at position 16, row 2 its third at 32
+    assert pages.row_pages(2) == [0, 1, 5] and pages.row_pages(0) == [2, 4] and pages.row_pages(3) == [3]
+    same_pages()
+    pages.release([0])
+    lists.release([0])
+    prefill([1], [40])  # takes pages 6 .. 8 from the head of the free list; row 0's pages wait at the tail
+    assert pages.row_pages(1) == [6, 7, 8] and pages.free_list() == [9, 10, 11, 2, 4]
+    lens_dev = torch.tensor([34, 40, 9], dtype=torch.int32, device=DEV)
+    decode([2, 1, 3], lens_dev, 9)  # row 3 reaches position 16 one step before row 1 reaches 48
+    assert pages.row_pages(1) == [6, 7, 8, 10] and pages.row_pages(3) == [3, 9]
+    same_pages()
