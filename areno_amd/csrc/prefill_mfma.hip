@@ -3,8 +3,9 @@
 // Work item = (sequence, kv head, block of query tokens).  The G query heads of the kv head are folded into the
 // query-row axis: row r of the block is (token r / GP, head r % GP) with GP = G rounded up to a power of two, so one
 // 16-row MFMA tile holds 16 / GP tokens of all heads and K/V are read once for the whole group (GQA without
-// expanding KV, as areno/accel/csrc/attention.cu:170-171 does per row).  A block is 128 rows: each of the 4 waves
-// owns 32 (two 16-row tiles).
+// expanding KV, as areno/accel/csrc/attention.cu:170-171 does per row).  A block is 256 rows: each of the 8 waves
+// owns 32 (two 16-row tiles).  One such workgroup per CU (the registers allow two waves per SIMD either way; eight
+// waves behind one set of K/V tiles halve the staging work per wave against two workgroups of four).
 //
 // Balance: an item costs one "tile step" per 32-key tile it may see, and items differ by orders of magnitude (a
 // query block on a 16k context next to one on an empty context).  Every workgroup computes the prefix sum of tile
@@ -14,8 +15,8 @@
 //   * an item cut by a unit border leaves un-normalised partials (running max, sum, accumulator) in the workspace
 //     -- slot 2u for the first item of unit u, slot 2u + 1 for its last -- and prefill_merge_kernel combines them.
 //
-// One segment, per 32-key tile t (all four waves share the K/V tiles in LDS):
-//   * the 256 threads fetch K three tiles and V two tiles ahead with 16-byte coalesced loads (block ids one more
+// One segment, per 32-key tile t (all waves share the K/V tiles in LDS):
+//   * the threads fetch K three tiles and V two tiles ahead with 16-byte coalesced loads (block ids one more
 //     tile ahead) and publish them into double-buffered LDS tiles one iteration before their first use, so one
 //     barrier per tile is enough (padded rows, conflict free).  8-bit codes are dequantized (times the per-token
 //     scale) by the thread that stages them, once per workgroup: the tiles in LDS are always 16-bit;
@@ -25,7 +26,10 @@
 //   * causal / window mask only on tiles that cross a mask edge, online softmax in the log2 domain (per lane = per
 //     row; the four lanes of a row combine through v_permlane swaps), the softmax scale folded into the exponent's
 //     multiply-add;
-//   * O^T[dim][row] += V^T . P^T : A = V^T through the LDS transpose reads, B = P^T (= the C layout of S^T).
+//   * O^T[dim][row] += V^T . P^T : A = V^T through the LDS transpose reads, B = P^T (= the C layout of S^T); one
+//     more product with an all-ones A operand accumulates the row sums of P.
+// The loop is bound by vector-ALU issue: with two waves per SIMD a plain VALU instruction issues every ~5.7 cycles
+// (4 with more waves), v_exp_f32 every ~9, while the 34 MFMAs of a wave's tile step need 18 cycles each and overlap.
 // The LDS layouts are the 16-bit ones of the decode kernel (decode_mfma_kernels.hpp).  Semantics:
 // _reference_attention with query_start = context_lens[s] (areno/accel/attention.py:25-41 in the reference); with
 // context 0 it is the reference's varlen kernel (areno/accel/csrc/attention.cu:145-242).
@@ -42,12 +46,15 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
 
 namespace {
 
-constexpr int kPrefillThreads = 256;
-constexpr int kPrefillWaves = 4;
+#ifndef ARENO_PREFILL_WAVES
+#define ARENO_PREFILL_WAVES 8
+#endif
+constexpr int kPrefillWaves = ARENO_PREFILL_WAVES;
+constexpr int kPrefillThreads = 64 * kPrefillWaves;
 constexpr int kMaxRowTiles = 2;                                   // 16-row MFMA tiles per wave
-constexpr int kMaxRowsPerWg = 16 * kMaxRowTiles * kPrefillWaves;  // 128
+constexpr int kMaxRowsPerWg = 16 * kMaxRowTiles * kPrefillWaves;
 constexpr int kMaxPrefillSeqs = 1024;
-constexpr int kPrefillTargetWgs = 512;  // two resident workgroups on each of the 256 CUs
+constexpr int kPrefillTargetWgs = 2048 / kPrefillWaves;  // eight resident waves on each of the 256 CUs
 constexpr int kMaxPrefillUnits = 512;   // per kv head
 
 struct PrefillParams {
@@ -60,8 +67,8 @@ struct PrefillParams {
   const int32_t* block_table;
   const int32_t* cu_seqlens_q;
   const int32_t* context_lens;
-  float* part_ml;   // [2 * units][kv_heads][128 rows][2]
-  float* part_acc;  // [2 * units][kv_heads][128 rows][head_dim]
+  float* part_ml;   // [2 * units][kv_heads][rows_per_wg][2]
+  float* part_acc;  // [2 * units][kv_heads][rows_per_wg][head_dim]
   int32_t num_seqs;
   int32_t q_heads;
   int32_t kv_heads;
@@ -209,7 +216,7 @@ __device__ __forceinline__ void dequant_chunk(uint4_t codes, float scale, uint4_
 }
 
 template <int KIND, int D, bool SCALE16, int RT>
-__global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma_kernel(PrefillParams p) {
+__global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) void prefill_mfma_kernel(PrefillParams p) {
   constexpr int kRowTiles = RT;
   constexpr int kRowsPerWave = 16 * RT;
   constexpr int kRowsPerWg = kRowsPerWave * kPrefillWaves;
@@ -333,11 +340,17 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
     const int wave_qmax = ctx + tok0 + min(tok_cnt - 1, ((wave + 1) * kRowsPerWave - 1) >> p.group_shift);
 
     float4_t acc[kRowTiles][NB];
-    float m_run[kRowTiles], l_run[kRowTiles];
+    // Row sums of the probabilities come from the matrix cores as well: one more product per key tile with an
+    // all-ones A operand puts the sum over the tile's 32 keys of column (= query row) lr into every element of the
+    // lane's accumulator, already complete over the four k groups.  Element 0 is the one kept (and rescaled).
+    float4_t l_acc[kRowTiles];
+    float m_run[kRowTiles];
+    constexpr uint32_t kOnePair = OPK == KV_BF16 ? 0x3f803f80u : 0x3c003c00u;  // two 1.0 in the operand type
+    const V8 ones_op = __builtin_bit_cast(V8, uint4_t{kOnePair, kOnePair, kOnePair, kOnePair});
 #pragma unroll
     for (int nq = 0; nq < kRowTiles; ++nq) {
       m_run[nq] = kNegInf;
-      l_run[nq] = 0.0f;
+      l_acc[nq] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) acc[nq][nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     }
@@ -472,7 +485,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
     // maxima of tile t ---------------------------------------------------------------------------------------------------
     for (int t = ta; t <= tb; ++t) {
       __syncthreads();
-      stage(t);  // first: the loads it issues then have the whole iteration to land
+      stage(t);
       if (!wave_live) continue;
       const int k0 = t * TK;
       const bool need_mask = k0 + TK - 1 > wave_qmin || (p.window_left >= 0 && k0 < wave_qmax - p.window_left);
@@ -512,7 +525,11 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
       if (__builtin_amdgcn_ballot_w64(changed) != 0) {
 #pragma unroll
         for (int nq = 0; nq < kRowTiles; ++nq) {
-          scale_in_place(l_run[nq], alpha[nq]);
+          {
+            float l0 = l_acc[nq][0];
+            scale_in_place(l0, alpha[nq]);
+            l_acc[nq][0] = l0;
+          }
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
@@ -528,18 +545,16 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
 #pragma unroll
       for (int nq = 0; nq < kRowTiles; ++nq) {
         float pe[8];
-        float lsum = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           pe[j] = fast_exp2(__builtin_fmaf(s_cur[nq][0][j], p.scale_log2e, -m_safe[nq]));
           pe[4 + j] = fast_exp2(__builtin_fmaf(s_cur[nq][1][j], p.scale_log2e, -m_safe[nq]));
-          lsum += pe[j] + pe[4 + j];
         }
-        l_run[nq] += lsum;
         uint32_t pw[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) pw[j] = pack_pair<OPK>(pe[2 * j], pe[2 * j + 1]);
         pop[nq] = __builtin_bit_cast(V8, uint4_t{pw[0], pw[1], pw[2], pw[3]});
+        l_acc[nq] = Ops::mfma(ones_op, pop[nq], l_acc[nq]);  // sums the probabilities as rounded for the product
       }
 
       // -- O^T += V^T . P^T: lane i of a 16-lane group supplies row (i / 4), 4 elements at column 16 nb + 4 (i % 4);
@@ -576,7 +591,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 2 : 1) void prefill_mfma
     const int slot = 2 * unit + (first_item ? 0 : 1);
 #pragma unroll
     for (int nq = 0; nq < kRowTiles; ++nq) {
-      const float l_tot = rows_sum(l_run[nq]);
+      const float l_tot = l_acc[nq][0];
       if (q_pos[nq] < 0) continue;
       if (whole) {
         const float inv = 1.0f / l_tot;
@@ -658,7 +673,7 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
   while (u_hi + 1 < p.units && unit_start_step(total, u_hi + 1, p.units) <= item_x1 - 1) ++u_hi;
 
   const int q_begin = p.cu_seqlens_q[pos.seq];
-  // thread -> (row, half of the head dim), 128 rows per pass.  Per unit all of a thread's accumulator loads are issued
+  // thread -> (row, half of the head dim), kPrefillThreads / 2 rows per pass.  Per unit all of a thread's accumulator loads are issued
   // together (no store in between), the normalised row is written once at the end.
   constexpr int kMaxChunks = 128 / 2 / 4;  // float4 chunks of half a row at the largest head dim (128)
   const int half = tid & 1;
