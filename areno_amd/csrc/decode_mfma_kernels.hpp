@@ -262,7 +262,13 @@ struct TileCursor {
 #ifndef ARENO_MFMA_QUANT_OCC
 #define ARENO_MFMA_QUANT_OCC 2
 #endif
-template <int KIND, int D, bool SCALE16, int NW, bool GROUPED = false>
+// DSPLIT = 2 serves heads of 2 * D elements: two adjacent waves of the workgroup take one half of the head dimension
+// each.  Every wave computes the part of S = K . Q^T over its half, the pair exchanges the parts through LDS (each
+// wave's K tile is dead once its products are issued, so the part is parked there) and both go on with identical
+// scores: the same softmax in both, P . V over the wave's own half of V, the wave's half of the partial row.  The
+// pair synchronises through two counters in LDS (part ready / part consumed); no workgroup barrier is involved, so
+// pairs of one workgroup may run different units.
+template <int KIND, int D, bool SCALE16, int NW, bool GROUPED = false, int DSPLIT = 1>
 __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUANT_OCC : 2) void decode_mfma_kernel(
     MfmaDecodeParams mp) {
   using T = KVTraits<KIND>;
@@ -284,11 +290,14 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   constexpr float kPScale = T::kQuant ? 256.0f : 1.0f;
   constexpr int kWaveLds = TK * RSK + TK * RSV + 2 * TK * 4;
   static_assert(NLD >= 1 && LPT >= 4 && LPT <= 16, "unsupported head_dim");
+  static_assert(DSPLIT == 1 || (DSPLIT == 2 && !GROUPED && NW % 2 == 0), "unsupported head split");
+  constexpr int DFULL = D * DSPLIT;  // elements of a whole head (row of Q, of a cache page, of a partial)
 
   __shared__ __attribute__((aligned(16))) char s_tiles[NW][kWaveLds];
   constexpr int kMaxItems = (GROUPED ? 2 : 1) * kMfmaMaxBatch;  // at most one shared item per row on top of the rows
   __shared__ int s_cum[kMaxItems + 1];
   __shared__ int s_wave_tot[NW];
+  __shared__ int s_pair_flags[2][NW];  // [0]: score parts this wave has published, [1]: partner parts it has consumed
   constexpr int SPT = kMaxItems / (NW * kWave);  // items per thread in the prefix sum
 
   const int tid = threadIdx.x;
@@ -369,6 +378,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       if (lane >= off) incl += v;
     }
     if (lane == kWave - 1) s_wave_tot[wave] = incl;
+    if (lane == 0) s_pair_flags[0][wave] = s_pair_flags[1][wave] = 0;
     __syncthreads();
     int excl = incl - local;
     for (int w2 = 0; w2 < wave; ++w2) excl += s_wave_tot[w2];
@@ -393,15 +403,17 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   }
 
   const int hw_count = p.heads_per_wg;
-  const int hw = wave % hw_count;
-  const int ts = wave / hw_count;
+  const int half = wave % DSPLIT;  // which part of the head dimension this wave owns
+  const int hw = (wave / DSPLIT) % hw_count;
+  const int ts = (wave / DSPLIT) / hw_count;
   const int kvh = blockIdx.y * hw_count + hw;
   char* const k_tile = &s_tiles[wave][0];
   char* const v_tile = k_tile + TK * RSK;
   float* const ksc = reinterpret_cast<float*>(&s_tiles[wave][TK * RSK + TK * RSV]);
   float* const vsc = ksc + TK;
 
-  constexpr int64_t row_bytes = static_cast<int64_t>(D) * ES;
+  constexpr int64_t row_bytes = static_cast<int64_t>(DFULL) * ES;
+  const int64_t half_bytes = static_cast<int64_t>(half) * D * ES;  // of this wave's part inside a cache / update row
   const int h0 = kvh * p.group;
   const bool q_is_operand_type = (KIND == KV_BF16 && p.q_dtype == ARENO_DT_BF16) ||
                                  (KIND != KV_BF16 && p.q_dtype == ARENO_DT_F16);
@@ -466,14 +478,14 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       const int t = min(tt, kv_cur.end - 1);
       const int slot = p.bs_shift >= 0 ? (t & (p.block_size - 1)) : (t % p.block_size);
       const int64_t row = (static_cast<int64_t>(ids[i]) * p.block_size + slot) * p.kv_heads + kvh;
-      const char* ka = static_cast<const char*>(p.k_cache) + row * row_bytes + dc * 16;
-      const char* va = static_cast<const char*>(p.v_cache) + row * row_bytes + dc * 16;
+      const char* ka = static_cast<const char*>(p.k_cache) + row * row_bytes + half_bytes + dc * 16;
+      const char* va = static_cast<const char*>(p.v_cache) + row * row_bytes + half_bytes + dc * 16;
       if (tail_tile && tt >= kv_cur.end - 1) {
         // the page slot of the newest token (and the clamped rows behind it) is not written yet
         if (tt == kv_cur.end - 1) new_row = row;
         if constexpr (!T::kQuant) {
-          ka = static_cast<const char*>(mp.k_update) + upd_row * row_bytes + dc * 16;
-          va = static_cast<const char*>(mp.v_update) + upd_row * row_bytes + dc * 16;
+          ka = static_cast<const char*>(mp.k_update) + upd_row * row_bytes + half_bytes + dc * 16;
+          va = static_cast<const char*>(mp.v_update) + upd_row * row_bytes + half_bytes + dc * 16;
         }
       }
       kreg[i] = *reinterpret_cast<const uint4_t*>(ka);
@@ -517,7 +529,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     for (int sl = 0; sl < NS; ++sl) {
       qraw[sl] = uint4_t{0u, 0u, 0u, 0u};
       if (live) {
-        const int64_t idx = (static_cast<int64_t>(c.row + m) * p.q_heads + h0 + g) * D + (D / 4) * lk + 8 * sl;
+        const int64_t idx =
+            (static_cast<int64_t>(c.row + m) * p.q_heads + h0 + g) * DFULL + half * D + (D / 4) * lk + 8 * sl;
         qraw[sl] = load16(p.q, idx * 2);
       }
     }
@@ -578,7 +591,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       const int64_t prow = shared ? (static_cast<int64_t>(unit + v) * p.kv_heads + kvh) * 16 + lr
                                   : static_cast<int64_t>(unit + row) * p.q_heads + h0 + lr;
       float* ml = shared ? mp.shared_ml : p.part_ml;
-      float* dst = (shared ? mp.shared_acc : p.part_acc) + prow * D + 4 * lk;
+      float* dst = (shared ? mp.shared_acc : p.part_acc) + prow * DFULL + half * D + 4 * lk;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
         float4_t o = acc[nb];
@@ -590,6 +603,16 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
         ml[prow * 2] = m_run;
         ml[prow * 2 + 1] = l_tot;
       }
+    }
+  };
+
+  // ---- pair synchronisation of the split-head variant ----------------------------------------------------------------
+  int pair_step = 0;  // tiles this wave has gone through; the pair's waves go through the same tiles
+  auto pair_wait = [&](const int* flag, int target) {
+    // bounded: a partner that never arrives (it cannot, both run the same tile sequence) must not hang the wave
+    for (int spin = 0; spin < (1 << 18); ++spin) {
+      if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= target) break;
+      __builtin_amdgcn_s_sleep(1);
     }
   };
 
@@ -636,6 +659,10 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
 
       for (int x = x0; x < x1; ++x) {
         ARENO_TRACE_POINT();
+        if constexpr (DSPLIT == 2) {
+          // the partner must have picked up the score part parked in this wave's K tile before the tile is rewritten
+          pair_wait(&s_pair_flags[1][wave ^ 1], pair_step);
+        }
         // -- stage the fetched tile into LDS (waits for its loads) ---------------------------------------------
         if (tail_tile) {
           // the newest token: quantize (8-bit caches), substitute it for the unwritten slot, store it into the page
@@ -659,8 +686,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
             if (cp_tok + i * TPL + grp == cp_end - 1) {
               char* kc = static_cast<char*>(const_cast<void*>(p.k_cache));
               char* vc = static_cast<char*>(const_cast<void*>(p.v_cache));
-              *reinterpret_cast<uint4_t*>(kc + new_row * row_bytes + dc * 16) = kreg[i];
-              *reinterpret_cast<uint4_t*>(vc + new_row * row_bytes + dc * 16) = vreg[i];
+              *reinterpret_cast<uint4_t*>(kc + new_row * row_bytes + half_bytes + dc * 16) = kreg[i];
+              *reinterpret_cast<uint4_t*>(vc + new_row * row_bytes + half_bytes + dc * 16) = vreg[i];
               if constexpr (T::kQuant) {
                 if (dc == 0) {
                   static_cast<scale_raw_t*>(const_cast<void*>(p.k_scale))[new_row] = ksreg[i];
@@ -727,12 +754,54 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
           }
 #pragma unroll
           for (int sl = 0; sl < NS; ++sl) c = Ops::mfma(to_operand<KIND>(&kw[sl * WPL]), qop[sl], c);
-          const float4_t sc = *reinterpret_cast<const float4_t*>(ksc + 16 * tg + 4 * lk);
+          if constexpr (DSPLIT == 1) {
+            const float4_t sc = *reinterpret_cast<const float4_t*>(ksc + 16 * tg + 4 * lk);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            // tokens past the end carry a -inf scale; keep them exactly -inf (0 * -inf would be NaN)
-            const float v = c[j] - qbias;
-            s[tg][j] = sc[j] == kNegInf ? kNegInf : v * sc[j];
+            for (int j = 0; j < 4; ++j) {
+              // tokens past the end carry a -inf scale; keep them exactly -inf (0 * -inf would be NaN)
+              const float v = c[j] - qbias;
+              s[tg][j] = sc[j] == kNegInf ? kNegInf : v * sc[j];
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s[tg][j] = c[j] - qbias;  // this wave's part of the dot products
+          }
+        }
+        if constexpr (DSPLIT == 2) {
+          // Park the part where the K tile was (its rows have been read by the products above), tell the partner,
+          // wait for the partner's part, add it.  Both waves of the pair end up with the same eight sums.
+          float* mine = reinterpret_cast<float*>(k_tile);
+          const float* theirs = reinterpret_cast<const float*>(&s_tiles[wave ^ 1][0]);
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) mine[(4 * tg + j) * kWave + lane] = s[tg][j];
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+          ++pair_step;
+          if (lane == 0)
+            __hip_atomic_store(&s_pair_flags[0][wave], pair_step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          pair_wait(&s_pair_flags[0][wave ^ 1], pair_step);
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+          float other[2][4];
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) other[tg][j] = theirs[(4 * tg + j) * kWave + lane];
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the reads above are done before the partner hears
+          if (lane == 0)
+            __hip_atomic_store(&s_pair_flags[1][wave], pair_step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+            const float4_t sc = *reinterpret_cast<const float4_t*>(ksc + 16 * tg + 4 * lk);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              // halves are added in a fixed order so that both waves round alike
+              const float lo = half == 0 ? s[tg][j] : other[tg][j];
+              const float hi = half == 0 ? other[tg][j] : s[tg][j];
+              s[tg][j] = sc[j] == kNegInf ? kNegInf : (lo + hi) * sc[j];
+            }
           }
         }
 
@@ -848,7 +917,19 @@ decode_mfma_fn decode_mfma_lookup_impl(int head_dim, bool scale16) {
     if (head_dim == 128) return decode_mfma_kernel<KIND, 128, false, NW, GROUPED>;
     if (head_dim == 64) return decode_mfma_kernel<KIND, 64, false, NW, GROUPED>;
   }
+  if constexpr (!GROUPED && NW % 2 == 0) {
+    // head dim 256: two waves per head, 128 elements each
+    if (head_dim == 256) {
+      if constexpr (KVTraits<KIND>::kQuant) {
+        if (scale16) return decode_mfma_kernel<KIND, 128, true, NW, false, 2>;
+      }
+      return decode_mfma_kernel<KIND, 128, false, NW, false, 2>;
+    }
+  }
   return nullptr;
 }
+
+// Waves of a workgroup that share one head (the head-dimension split of decode_mfma_kernel).
+inline int decode_mfma_head_split(int head_dim) { return head_dim == 256 ? 2 : 1; }
 
 }  // namespace areno

@@ -437,7 +437,7 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
 
-  // ---- matrix-core path: 16-bit or 8-bit caches, head_dim 64/128, up to 16 q heads per kv head ------------
+  // ---- matrix-core path: 16-bit or 8-bit caches, head_dim 64/128/256, up to 16 q heads per kv head --------
   decode_mfma_fn mfma = nullptr;
   if (aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && num_splits != 1 && p.group <= 16 &&
       batch <= kMfmaMaxBatch) {
@@ -451,14 +451,31 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
       default: break;
     }
   }
+  if (mfma == nullptr && num_shared > 0) {
+    // no grouped kernel for this shape: the plain matrix-core kernel, every row reading its own pages
+    num_shared = 0;
+    const bool s16 = cache->scale_dtype == ARENO_DT_F16;
+    if (aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && num_splits != 1 && p.group <= 16 &&
+        batch <= kMfmaMaxBatch) {
+      switch (cache->cache_dtype) {
+        case ARENO_DT_BF16: mfma = decode_mfma_lookup_bf16(p.head_dim, s16, false); break;
+        case ARENO_DT_F16: mfma = decode_mfma_lookup_f16(p.head_dim, s16, false); break;
+        case ARENO_DT_I8: mfma = decode_mfma_lookup_i8(p.head_dim, s16, false); break;
+        case ARENO_DT_FP8_E4M3: mfma = decode_mfma_lookup_fp8(p.head_dim, s16, false); break;
+        default: break;
+      }
+    }
+  }
   if (mfma == nullptr) num_shared = 0;  // the other kernels read every row's pages on their own
+  // waves per head in the matrix-core kernel: a 256-wide head is shared by two
+  const int head_split = mfma != nullptr ? decode_mfma_head_split(p.head_dim) : 1;
   // ---- append: folded into the matrix-core split kernel when it can take the new rows as they are, else a launch of
   // its own in front ------------------------------------------------------------------------------------------------
   static const bool allow_fused_append = env_int("ARENO_FUSED_APPEND", 1) != 0;
   const bool fuse_append =
       mfma != nullptr && allow_fused_append && k_update != nullptr && v_update != nullptr &&
       (stages & ARENO_STAGE_APPEND) && (stages & ARENO_STAGE_SPLIT) &&
-      (is_quantized(cache->cache_dtype) || q_dtype == cache->cache_dtype) &&
+      (is_quantized(cache->cache_dtype) ? head_split == 1 : q_dtype == cache->cache_dtype) &&
       reinterpret_cast<uintptr_t>(k_update) % 16 == 0 && reinterpret_cast<uintptr_t>(v_update) % 16 == 0;
   if (k_update != nullptr && (stages & ARENO_STAGE_APPEND) && !fuse_append) {
     if (int rc = areno_hip_cache_write_decode(cache, k_update, v_update, q_dtype, batch, block_table, max_blocks,
@@ -469,7 +486,12 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
   if (mfma != nullptr) {
     MfmaDecodeParams mp;
     mp.d = p;
-    const int head_groups = cache->kv_heads / p.heads_per_wg;
+    if (head_split > 1) {
+      // a workgroup's waves pair up: half as many kv heads per workgroup
+      const int pairs = kMfmaWaves / head_split;
+      mp.d.heads_per_wg = cache->kv_heads % pairs == 0 ? pairs : (pairs >= 2 && cache->kv_heads % 2 == 0 ? 2 : 1);
+    }
+    const int head_groups = cache->kv_heads / mp.d.heads_per_wg;
     static const int wgs = [] {
       const int v = env_int("ARENO_MFMA_WGS", kMfmaWorkgroups);
       return v > 0 && v <= kMfmaWorkgroups + kMfmaTailWorkgroups ? v : kMfmaWorkgroups;
@@ -482,7 +504,7 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     static const int unit_tiles = env_int("ARENO_MFMA_UNIT", 4);
     mp.static_wgs = wgs / head_groups > 0 ? wgs / head_groups : 1;
     const int extra = tail_wgs / head_groups;
-    mp.tok_splits = kMfmaWaves / p.heads_per_wg;
+    mp.tok_splits = kMfmaWaves / (mp.d.heads_per_wg * head_split);
     mp.num_pieces = mp.static_wgs * mp.tok_splits;
     mp.max_small = extra * mp.tok_splits;
     mp.static_share = static_share;

@@ -673,13 +673,14 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
   while (u_hi + 1 < p.units && unit_start_step(total, u_hi + 1, p.units) <= item_x1 - 1) ++u_hi;
 
   const int q_begin = p.cu_seqlens_q[pos.seq];
-  // thread -> (row, half of the head dim), kPrefillThreads / 2 rows per pass.  Per unit all of a thread's accumulator loads are issued
+  // thread -> (row, 64-element part of the head dim).  Per unit all of a thread's accumulator loads are issued
   // together (no store in between), the normalised row is written once at the end.
-  constexpr int kMaxChunks = 128 / 2 / 4;  // float4 chunks of half a row at the largest head dim (128)
-  const int half = tid & 1;
-  const int dh = d / 2;
+  constexpr int kMaxChunks = 16;  // float4 chunks per thread: 64 elements of a row
+  const int parts = d > 64 ? d / 64 : 1;  // threads per row (head dim 64, 128 or 256)
+  const int half = tid % parts;
+  const int dh = d / parts;
   const int chunks = dh / 4;
-  for (int r = tid >> 1; r < kRowsPerWg; r += kPrefillThreads / 2) {
+  for (int r = tid / parts; r < kRowsPerWg; r += kPrefillThreads / parts) {
     const int t = r >> p.group_shift;
     const int hh = r & (p.group_pad - 1);
     if (t >= item.cnt || hh >= p.group) continue;
@@ -738,22 +739,38 @@ typedef void (*prefill_fn)(PrefillParams);
 
 template <int KIND, int RT>
 prefill_fn prefill_lookup_rt(int head_dim, bool scale16) {
-  if constexpr (KVTraits<KIND>::kQuant) {
-    if (head_dim == 128)
-      return scale16 ? prefill_mfma_kernel<KIND, 128, true, RT> : prefill_mfma_kernel<KIND, 128, false, RT>;
-    if (head_dim == 64)
-      return scale16 ? prefill_mfma_kernel<KIND, 64, true, RT> : prefill_mfma_kernel<KIND, 64, false, RT>;
+  constexpr bool kQuant = KVTraits<KIND>::kQuant;
+  if constexpr (RT == 2) {
+    if (head_dim == 128) {
+      if constexpr (kQuant) {
+        if (scale16) return prefill_mfma_kernel<KIND, 128, true, 2>;
+      }
+      return prefill_mfma_kernel<KIND, 128, false, 2>;
+    }
+    if (head_dim == 64) {
+      if constexpr (kQuant) {
+        if (scale16) return prefill_mfma_kernel<KIND, 64, true, 2>;
+      }
+      return prefill_mfma_kernel<KIND, 64, false, 2>;
+    }
   } else {
-    if (head_dim == 128) return prefill_mfma_kernel<KIND, 128, false, RT>;
-    if (head_dim == 64) return prefill_mfma_kernel<KIND, 64, false, RT>;
+    if (head_dim == 256) {
+      if constexpr (kQuant) {
+        if (scale16) return prefill_mfma_kernel<KIND, 256, true, 1>;
+      }
+      return prefill_mfma_kernel<KIND, 256, false, 1>;
+    }
   }
   return nullptr;
 }
 
+// 16-row tiles per wave: two up to head dim 128 (four need more registers than a wave has), one at head dim 256,
+// where the accumulators and the Q operands of one tile take the registers two take at 128.
+int prefill_row_tiles(int head_dim) { return head_dim > 128 ? 1 : 2; }
+
 template <int KIND>
 prefill_fn prefill_lookup(int head_dim, bool scale16, int row_tiles) {
-  (void)row_tiles;  // two 16-row tiles per wave is the only shape built: four need more registers than a wave has
-  return prefill_lookup_rt<KIND, 2>(head_dim, scale16);
+  return row_tiles == 1 ? prefill_lookup_rt<KIND, 1>(head_dim, scale16) : prefill_lookup_rt<KIND, 2>(head_dim, scale16);
 }
 
 int log2_exact_i(int x) {
@@ -773,8 +790,6 @@ int prefill_units(int kv_heads) {
 size_t prefill_ml_bytes(int units, int kv_heads) {
   return static_cast<size_t>(2) * units * kv_heads * kMaxRowsPerWg * 2 * sizeof(float);
 }
-
-int prefill_row_tiles() { return 2; }
 
 }  // namespace
 
@@ -802,7 +817,7 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
       reinterpret_cast<uintptr_t>(q) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 8 != 0)
     return ARENO_ERR_UNSUPPORTED;
   const bool scale16 = cache->scale_dtype == ARENO_DT_F16;
-  const int row_tiles = prefill_row_tiles();
+  const int row_tiles = prefill_row_tiles(cache->head_dim);
   const int rows_per_wg = 16 * row_tiles * kPrefillWaves;
   prefill_fn fn = nullptr;
   switch (cache->cache_dtype) {

@@ -93,6 +93,24 @@ def test_shapes_head_ratios_and_block_sizes(kv, hq, hkv, d, bs):
     assert_close(out, expected_decode(w), *tolerances(kv), what=f"{kv} {hq}/{hkv} d={d} bs={bs}")
 
 
+@pytest.mark.parametrize("kv", ["bf16", "fp16", "int8", "fp8"])
+@pytest.mark.parametrize("hq,hkv,window_left", [(16, 8, None), (8, 2, None), (4, 1, 300), (24, 4, None)])
+def test_head_dim_256_on_the_matrix_core_kernel(kv, hq, hkv, window_left):
+    """Head dim 256 (Gemma-family sliding layers, Qwen3.5): two waves share a head, each with half of the head
+    dimension, and exchange their parts of the scores.  Long and short rows so that units cross sequence borders, one
+    kv head per workgroup pair so that the pairs of a workgroup run different units, the append checked bit for bit."""
+    g = torch.Generator().manual_seed(hq * 7 + hkv)
+    batch = 9
+    lengths = torch.randint(0, 2500, (batch,), generator=g)
+    lengths[0], lengths[1], lengths[2] = 0, 15, 16
+    w = workloads.make_decode_workload("d256", seed=79, batch=batch, hq=hq, hkv=hkv, d=256, bs=16, kv=kv,
+                                       lengths=lengths, device=DEV, quantize_fn=gpu_quantize, poison=True)  # fmt: skip
+    before = _snapshot(w)
+    out = run_decode(w, window_left=window_left)
+    assert_close(out, expected_decode(w, window_left=window_left), *tolerances(kv), what=f"D=256 {kv} {hq}/{hkv}")
+    _check_append(w, before)
+
+
 def test_graph_padded_rows_on_a_scratch_block_are_harmless():
     """Rows with cache_seqlens = 0 and an all-scratch block table (how the decode graph pads a bucket)."""
     w = workloads.cfg0_tiny("bf16", device=DEV)
