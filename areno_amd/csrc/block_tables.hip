@@ -70,14 +70,24 @@ __device__ int workgroup_exclusive_scan(int value, int* s_wave, int* total) {
 // True when an earlier request of the call names the same row.  The reference walks the requests one by one and
 // would see the row's updated state at the later one; a parallel pass cannot, so the later one is set aside.
 // s_rows holds the rows of the current pass of kAllocThreads requests (requests before `base` are read from memory).
-__device__ bool named_earlier(const int64_t* rows, int base, int64_t r, int64_t* s_rows) {
+// The scan over the earlier entries of the pass has no early exit, so its LDS reads pipeline.
+__device__ bool named_earlier(const int64_t* rows, int base, int live, int64_t r, int* s_rows) {
   __syncthreads();  // the previous pass is done with s_rows
-  s_rows[threadIdx.x] = r;
+  s_rows[threadIdx.x] = static_cast<int>(r);  // rows are < max_rows <= 2^31 - 1, or -1
   __syncthreads();
-  if (r < 0) return false;
-  for (int j = 0; j < static_cast<int>(threadIdx.x); ++j) {
-    if (s_rows[j] == r) return true;
+  const int tid = threadIdx.x;
+  const int mine = static_cast<int>(r);
+  // uniform over the wave; nothing to scan for waves behind the pass's last request
+  const int wave_end = min((tid | (kWave - 1)) + 1, (live + 3) & ~3);
+  bool found = false;
+#pragma unroll 4
+  for (int j = 0; j < wave_end; j += 4) {
+    const int4 v = *reinterpret_cast<const int4*>(&s_rows[j]);
+    found |= (j + 0 < tid && v.x == mine) | (j + 1 < tid && v.y == mine) | (j + 2 < tid && v.z == mine) |
+             (j + 3 < tid && v.w == mine);
   }
+  if (r < 0) return false;
+  if (found) return true;
   for (int j = 0; j < base; ++j) {
     if (rows[j] == r) return true;
   }
@@ -93,7 +103,7 @@ __device__ void report(const areno_block_tables& bt, int status, int index) {
 // Serves the requests of one call in index order; runs in one workgroup of kAllocThreads threads.
 // mode 0: amounts[i] = tokens the row must be able to hold; mode 1: amounts[i] = position the row writes next.
 __device__ void serve_requests(const areno_block_tables& bt, const int64_t* rows, const int32_t* amounts, int n,
-                               int mode, int* s_wave, int64_t* s_rows) {
+                               int mode, int* s_wave, int* s_rows) {
   const int head = bt.state[kStateHead];
   const int count = bt.state[kStateCount];
   int taken = 0;  // pages asked for by the requests of earlier passes
@@ -106,7 +116,7 @@ __device__ void serve_requests(const areno_block_tables& bt, const int64_t* rows
       r = -1;
     }
     // (a negative row in a decode request is a padded row of a bucketed batch: nothing to do)
-    const bool repeated = named_earlier(rows, base, r, s_rows);
+    const bool repeated = named_earlier(rows, base, min(n - base, kAllocThreads), r, s_rows);
     if (r >= 0) {
       const int64_t amount = amounts[i];
       if (repeated) {
@@ -151,14 +161,14 @@ __device__ void serve_requests(const areno_block_tables& bt, const int64_t* rows
 __global__ __launch_bounds__(kAllocThreads) void block_tables_reserve_kernel(areno_block_tables bt, const int64_t* rows,
                                                                             const int32_t* amounts, int n, int mode) {
   __shared__ int s_wave[kAllocThreads / kWave];
-  __shared__ int64_t s_rows[kAllocThreads];
+  __shared__ __attribute__((aligned(16))) int s_rows[kAllocThreads];
   serve_requests(bt, rows, amounts, n, mode, s_wave, s_rows);
 }
 
 __global__ __launch_bounds__(kAllocThreads) void block_tables_release_kernel(areno_block_tables bt, const int64_t* rows,
                                                                             int n) {
   __shared__ int s_wave[kAllocThreads / kWave];
-  __shared__ int64_t s_rows[kAllocThreads];
+  __shared__ __attribute__((aligned(16))) int s_rows[kAllocThreads];
   const int head = bt.state[kStateHead];
   const int count = bt.state[kStateCount];
   int returned = 0;
@@ -171,7 +181,7 @@ __global__ __launch_bounds__(kAllocThreads) void block_tables_release_kernel(are
       r = -1;
     }
     // a row named twice gives its pages back once, like dict.pop(row, None)
-    const bool repeated = named_earlier(rows, base, r, s_rows);
+    const bool repeated = named_earlier(rows, base, min(n - base, kAllocThreads), r, s_rows);
     if (r >= 0 && !repeated) have = bt.row_blocks[r];
     int total;
     const int off = returned + workgroup_exclusive_scan(have, s_wave, &total);

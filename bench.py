@@ -84,7 +84,7 @@ def _parity_sample(w, out, rows=4):
     return float((out[:rows].cpu().float() - want).abs().max())
 
 
-def measure_decode(w, steps, warmup, *, kernel_iters=60):
+def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
     """Time the whole op (graph replay and eager) and each kernel of it; returns a dict of numbers."""
     import torch
 
@@ -161,11 +161,11 @@ def measure_decode(w, steps, warmup, *, kernel_iters=60):
                               workspace, softmax_scale=w.softmax_scale, stages=stage, group_rows=group_rows,
                               shared_lens=shared_lens)  # fmt: skip
 
-        for i in range(copies):
+        for i in range(max(copies, 20)):
             launch(i)
         torch.cuda.synchronize()
         samples = []
-        for _ in range(5):
+        for _ in range(kernel_samples):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             for i in range(kernel_iters):
@@ -173,7 +173,11 @@ def measure_decode(w, steps, warmup, *, kernel_iters=60):
             e1.record()
             e1.synchronize()
             samples.append(e0.elapsed_time(e1) * 1e3 / kernel_iters)
+        samples.sort()
+        spread[stage] = (samples[len(samples) // 10], samples[(len(samples) * 9) // 10])
         return statistics.median(samples)
+
+    spread = {}
 
     # the op folds the append into the split kernel; the stand-alone append launch is timed for reference only
     us_split = time_stage(cabi.STAGE_APPEND | cabi.STAGE_SPLIT)
@@ -189,6 +193,8 @@ def measure_decode(w, steps, warmup, *, kernel_iters=60):
         "us_per_step": us_graph,
         "us_per_step_eager": us_eager,
         "kernel_us": {"split_with_append": us_split, "reduce": us_reduce, "append_alone_not_in_op": us_append},
+        # 10th / 90th percentile of the split kernel's samples (each the mean of back-to-back launches)
+        "split_us_p10_p90": list(spread[cabi.STAGE_APPEND | cabi.STAGE_SPLIT]),
         "tokens_per_s": w.q.shape[0] / (us_graph * 1e-6),
         "algorithmic_bytes": alg_bytes,
         "op_gbps": alg_bytes / (us_graph * 1e-6) / 1e9,
