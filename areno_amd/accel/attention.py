@@ -21,7 +21,9 @@ defaulting to the reference behaviour:
   context (chunked prefill that re-reads earlier chunks).
 
 Everything runs as HIP kernels through ``areno_amd.accel._areno_accel``; there is no Python
-fallback and no autograd (the ops are used under ``torch.inference_mode``).
+fallback and no autograd: the ops are used under ``torch.inference_mode`` / ``torch.no_grad``, and a call
+whose inputs require gradients while gradients are being recorded is refused instead of returning an
+output without a graph.
 """
 
 from __future__ import annotations
@@ -47,6 +49,17 @@ def _all_on_gpu(*tensors: torch.Tensor | None) -> bool:
 
 def _contig(t: torch.Tensor | None) -> torch.Tensor | None:
     return None if t is None else t.contiguous()
+
+
+def _no_autograd(op: str, *tensors: torch.Tensor | None) -> None:
+    """The reference's shims are autograd functions with native backward kernels (``accel/attention.py:78-118,
+    145-183`` there) for its training backend.  This build serves inference only: rather than hand back an output
+    that silently carries no gradient, a call that autograd would have to record is refused."""
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        raise RuntimeError(
+            f"{op}: backward is not implemented in this build (inference path only); call it under "
+            "torch.no_grad() / torch.inference_mode() or detach the inputs"
+        )
 
 
 def _check_scales(op: str, cache: torch.Tensor, k_scale, v_scale) -> None:
@@ -91,6 +104,7 @@ def areno_paged_causal_attention_decode(
     several rows instead of once per row.  The result is the same.
     """
     op = "areno_paged_causal_attention_decode"
+    _no_autograd(op, q, k_update, v_update)
     if not _all_on_gpu(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, k_scale, v_scale):
         raise RuntimeError(f"{op} requires CUDA tensors")
     if q.dim() != 3:
@@ -144,6 +158,7 @@ def areno_varlen_causal_attention(
 ) -> torch.Tensor:
     """Apply packed causal attention to flat ``(tokens, heads, head_dim)`` tensors."""
     op = "areno_varlen_causal_attention"
+    _no_autograd(op, q, k, v)
     if not _all_on_gpu(q, k, v, cu_seqlens):
         raise RuntimeError(f"{op} requires CUDA q, k, v, and cu_seqlens tensors")
     if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
@@ -180,6 +195,7 @@ def areno_causal_attention(
     query may see exists as a key).
     """
     op = "areno_causal_attention"
+    _no_autograd(op, q, k, v)
     if not _all_on_gpu(q, k, v):
         raise RuntimeError(f"{op} requires CUDA q, k, and v tensors")
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
@@ -266,6 +282,7 @@ def areno_paged_varlen_causal_attention(
     absolute position ``context_lens[s] + i`` and sees keys ``[0, context_lens[s] + i]``.
     """
     op = "areno_paged_varlen_causal_attention"
+    _no_autograd(op, q)
     if not _all_on_gpu(q, k_cache, v_cache, block_table, cu_seqlens_q, context_lens, k_scale, v_scale):
         raise RuntimeError(f"{op} requires CUDA tensors")
     if q.dim() != 3:

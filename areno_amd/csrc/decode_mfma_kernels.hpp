@@ -262,12 +262,13 @@ struct TileCursor {
 #ifndef ARENO_MFMA_QUANT_OCC
 #define ARENO_MFMA_QUANT_OCC 2
 #endif
-// DSPLIT = 2 serves heads of 2 * D elements: two adjacent waves of the workgroup take one half of the head dimension
-// each.  Every wave computes the part of S = K . Q^T over its half, the pair exchanges the parts through LDS (each
-// wave's K tile is dead once its products are issued, so the part is parked there) and both go on with identical
-// scores: the same softmax in both, P . V over the wave's own half of V, the wave's half of the partial row.  The
-// pair synchronises through two counters in LDS (part ready / part consumed); no workgroup barrier is involved, so
-// pairs of one workgroup may run different units.
+// DSPLIT > 1 serves heads of DSPLIT * D elements (256 = 2 x 128, 192 = 3 x 64): DSPLIT adjacent waves of the
+// workgroup take one part of the head dimension each.  Every wave computes the part of S = K . Q^T over its
+// elements, the waves exchange the parts through LDS (a wave's K tile is dead once its products are issued, so the
+// part is parked there), add them in the same order and go on with identical scores: the same softmax in all,
+// P . V over the wave's own part of V, the wave's part of the partial row.  The waves of a head synchronise through
+// two counters each in LDS (part ready / parts consumed); no workgroup barrier is involved, so the heads of one
+// workgroup may run different units.
 template <int KIND, int D, bool SCALE16, int NW, bool GROUPED = false, int DSPLIT = 1>
 __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUANT_OCC : 2) void decode_mfma_kernel(
     MfmaDecodeParams mp) {
@@ -290,15 +291,15 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   constexpr float kPScale = T::kQuant ? 256.0f : 1.0f;
   constexpr int kWaveLds = TK * RSK + TK * RSV + 2 * TK * 4;
   static_assert(NLD >= 1 && LPT >= 4 && LPT <= 16, "unsupported head_dim");
-  static_assert(DSPLIT == 1 || (DSPLIT == 2 && !GROUPED && NW % 2 == 0), "unsupported head split");
+  static_assert(DSPLIT == 1 || ((DSPLIT == 2 || DSPLIT == 3) && !GROUPED && NW % DSPLIT == 0), "unsupported head split");
   constexpr int DFULL = D * DSPLIT;  // elements of a whole head (row of Q, of a cache page, of a partial)
 
   __shared__ __attribute__((aligned(16))) char s_tiles[NW][kWaveLds];
   constexpr int kMaxItems = (GROUPED ? 2 : 1) * kMfmaMaxBatch;  // at most one shared item per row on top of the rows
   __shared__ int s_cum[kMaxItems + 1];
   __shared__ int s_wave_tot[NW];
-  __shared__ int s_pair_flags[2][NW];  // [0]: score parts this wave has published, [1]: partner parts it has consumed
-  constexpr int SPT = kMaxItems / (NW * kWave);  // items per thread in the prefix sum
+  __shared__ int s_pair_flags[2][NW];  // [0]: score parts this wave has published, [1]: steps whose parts it has read
+  constexpr int SPT = (kMaxItems + NW * kWave - 1) / (NW * kWave);  // items per thread in the prefix sum
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -659,9 +660,13 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
 
       for (int x = x0; x < x1; ++x) {
         ARENO_TRACE_POINT();
-        if constexpr (DSPLIT == 2) {
-          // the partner must have picked up the score part parked in this wave's K tile before the tile is rewritten
-          pair_wait(&s_pair_flags[1][wave ^ 1], pair_step);
+        if constexpr (DSPLIT > 1) {
+          // the other waves of the head must have read the score part parked in this wave's K tile before the tile
+          // is rewritten
+#pragma unroll
+          for (int part = 0; part < DSPLIT; ++part) {
+            if (part != half) pair_wait(&s_pair_flags[1][wave - half + part], pair_step);
+          }
         }
         // -- stage the fetched tile into LDS (waits for its loads) ---------------------------------------------
         if (tail_tile) {
@@ -767,11 +772,11 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
             for (int j = 0; j < 4; ++j) s[tg][j] = c[j] - qbias;  // this wave's part of the dot products
           }
         }
-        if constexpr (DSPLIT == 2) {
-          // Park the part where the K tile was (its rows have been read by the products above), tell the partner,
-          // wait for the partner's part, add it.  Both waves of the pair end up with the same eight sums.
+        if constexpr (DSPLIT > 1) {
+          // Park the part where the K tile was (its rows have been read by the products above), tell the other waves of
+          // the head, wait for their parts, add all parts in the order of the head dimension.  Every wave of the head
+          // ends up with the same eight sums.
           float* mine = reinterpret_cast<float*>(k_tile);
-          const float* theirs = reinterpret_cast<const float*>(&s_tiles[wave ^ 1][0]);
 #pragma unroll
           for (int tg = 0; tg < 2; ++tg) {
 #pragma unroll
@@ -781,27 +786,40 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
           ++pair_step;
           if (lane == 0)
             __hip_atomic_store(&s_pair_flags[0][wave], pair_step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          pair_wait(&s_pair_flags[0][wave ^ 1], pair_step);
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-          float other[2][4];
+          const int first_wave = wave - half;
+          float total[2][4];
 #pragma unroll
           for (int tg = 0; tg < 2; ++tg) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) other[tg][j] = theirs[(4 * tg + j) * kWave + lane];
+            for (int j = 0; j < 4; ++j) total[tg][j] = 0.0f;
           }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the reads above are done before the partner hears
+#pragma unroll
+          for (int part = 0; part < DSPLIT; ++part) {
+            if (part == half) {
+#pragma unroll
+              for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) total[tg][j] += s[tg][j];
+              }
+            } else {
+              pair_wait(&s_pair_flags[0][first_wave + part], pair_step);
+              __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+              const float* theirs = reinterpret_cast<const float*>(&s_tiles[first_wave + part][0]);
+#pragma unroll
+              for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) total[tg][j] += theirs[(4 * tg + j) * kWave + lane];
+              }
+            }
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the reads above are done before the others hear
           if (lane == 0)
             __hip_atomic_store(&s_pair_flags[1][wave], pair_step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 #pragma unroll
           for (int tg = 0; tg < 2; ++tg) {
             const float4_t sc = *reinterpret_cast<const float4_t*>(ksc + 16 * tg + 4 * lk);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              // halves are added in a fixed order so that both waves round alike
-              const float lo = half == 0 ? s[tg][j] : other[tg][j];
-              const float hi = half == 0 ? other[tg][j] : s[tg][j];
-              s[tg][j] = sc[j] == kNegInf ? kNegInf : (lo + hi) * sc[j];
-            }
+            for (int j = 0; j < 4; ++j) s[tg][j] = sc[j] == kNegInf ? kNegInf : total[tg][j] * sc[j];
           }
         }
 
@@ -926,10 +944,21 @@ decode_mfma_fn decode_mfma_lookup_impl(int head_dim, bool scale16) {
       return decode_mfma_kernel<KIND, 128, false, NW, false, 2>;
     }
   }
+  if constexpr (!GROUPED) {
+    // head dim 192: three waves per head, 64 elements each, in workgroups of six waves
+    if (head_dim == 192) {
+      if constexpr (KVTraits<KIND>::kQuant) {
+        if (scale16) return decode_mfma_kernel<KIND, 64, true, 6, false, 3>;
+      }
+      return decode_mfma_kernel<KIND, 64, false, 6, false, 3>;
+    }
+  }
   return nullptr;
 }
 
-// Waves of a workgroup that share one head (the head-dimension split of decode_mfma_kernel).
-inline int decode_mfma_head_split(int head_dim) { return head_dim == 256 ? 2 : 1; }
+// Waves of a workgroup that share one head (the head-dimension split of decode_mfma_kernel), and the waves per
+// workgroup of the kernel the lookup returns for a head dim.
+inline int decode_mfma_head_split(int head_dim) { return head_dim == 256 ? 2 : (head_dim == 192 ? 3 : 1); }
+inline int decode_mfma_waves(int head_dim) { return head_dim == 192 ? 6 : ARENO_MFMA_NW; }
 
 }  // namespace areno

@@ -486,9 +486,10 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
   if (mfma != nullptr) {
     MfmaDecodeParams mp;
     mp.d = p;
+    const int waves = decode_mfma_waves(p.head_dim);
     if (head_split > 1) {
-      // a workgroup's waves pair up: half as many kv heads per workgroup
-      const int pairs = kMfmaWaves / head_split;
+      // several waves share a head: fewer kv heads per workgroup
+      const int pairs = waves / head_split;
       mp.d.heads_per_wg = cache->kv_heads % pairs == 0 ? pairs : (pairs >= 2 && cache->kv_heads % 2 == 0 ? 2 : 1);
     }
     const int head_groups = cache->kv_heads / mp.d.heads_per_wg;
@@ -504,7 +505,7 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     static const int unit_tiles = env_int("ARENO_MFMA_UNIT", 4);
     mp.static_wgs = wgs / head_groups > 0 ? wgs / head_groups : 1;
     const int extra = tail_wgs / head_groups;
-    mp.tok_splits = kMfmaWaves / (mp.d.heads_per_wg * head_split);
+    mp.tok_splits = waves / (mp.d.heads_per_wg * head_split);
     mp.num_pieces = mp.static_wgs * mp.tok_splits;
     mp.max_small = extra * mp.tok_splits;
     mp.static_share = static_share;
@@ -535,7 +536,7 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
       mp.shared_acc = mp.shared_ml + shared_slots * cache->kv_heads * 16 * 2;
     }
     if (stages & ARENO_STAGE_SPLIT) {
-      hipLaunchKernelGGL(mfma, dim3(mp.static_wgs + extra, head_groups), dim3(kMfmaWaves * kWave), 0, s, mp);
+      hipLaunchKernelGGL(mfma, dim3(mp.static_wgs + extra, head_groups), dim3(waves * kWave), 0, s, mp);
       if (int rc = check_launch(op)) return rc;
     }
     if (stages & ARENO_STAGE_REDUCE) {

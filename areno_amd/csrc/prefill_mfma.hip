@@ -676,11 +676,12 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
   // thread -> (row, 64-element part of the head dim).  Per unit all of a thread's accumulator loads are issued
   // together (no store in between), the normalised row is written once at the end.
   constexpr int kMaxChunks = 16;  // float4 chunks per thread: 64 elements of a row
-  const int parts = d > 64 ? d / 64 : 1;  // threads per row (head dim 64, 128 or 256)
+  const int parts = d > 64 ? d / 64 : 1;  // threads per row (head dim 64, 128, 192 or 256)
   const int half = tid % parts;
   const int dh = d / parts;
   const int chunks = dh / 4;
-  for (int r = tid / parts; r < kRowsPerWg; r += kPrefillThreads / parts) {
+  const int rows_per_pass = kPrefillThreads / parts;  // threads beyond rows_per_pass * parts sit out (parts = 3)
+  for (int r = tid / parts; r < kRowsPerWg && tid < rows_per_pass * parts; r += rows_per_pass) {
     const int t = r >> p.group_shift;
     const int hh = r & (p.group_pad - 1);
     if (t >= item.cnt || hh >= p.group) continue;
@@ -760,12 +761,18 @@ prefill_fn prefill_lookup_rt(int head_dim, bool scale16) {
       }
       return prefill_mfma_kernel<KIND, 256, false, 1>;
     }
+    if (head_dim == 192) {
+      if constexpr (kQuant) {
+        if (scale16) return prefill_mfma_kernel<KIND, 192, true, 1>;
+      }
+      return prefill_mfma_kernel<KIND, 192, false, 1>;
+    }
   }
   return nullptr;
 }
 
-// 16-row tiles per wave: two up to head dim 128 (four need more registers than a wave has), one at head dim 256,
-// where the accumulators and the Q operands of one tile take the registers two take at 128.
+// 16-row tiles per wave: two up to head dim 128 (four need more registers than a wave has), one at head dims 192 and
+// 256, where the accumulators and the Q operands of one tile take the registers two take at 128.
 int prefill_row_tiles(int head_dim) { return head_dim > 128 ? 1 : 2; }
 
 template <int KIND>

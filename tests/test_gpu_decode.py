@@ -94,20 +94,22 @@ def test_shapes_head_ratios_and_block_sizes(kv, hq, hkv, d, bs):
 
 
 @pytest.mark.parametrize("kv", ["bf16", "fp16", "int8", "fp8"])
+@pytest.mark.parametrize("d", [256, 192])
 @pytest.mark.parametrize("hq,hkv,window_left", [(16, 8, None), (8, 2, None), (4, 1, 300), (24, 4, None)])
-def test_head_dim_256_on_the_matrix_core_kernel(kv, hq, hkv, window_left):
-    """Head dim 256 (Gemma-family sliding layers, Qwen3.5): two waves share a head, each with half of the head
-    dimension, and exchange their parts of the scores.  Long and short rows so that units cross sequence borders, one
-    kv head per workgroup pair so that the pairs of a workgroup run different units, the append checked bit for bit."""
+def test_head_dims_192_256_on_the_matrix_core_kernel(kv, d, hq, hkv, window_left):
+    """Head dims 256 (Gemma-family sliding layers, Qwen3.5) and 192 (128 + 64 rotary channels of MLA-style layers):
+    two resp. three waves share a head, each with a part of the head dimension, and exchange their parts of the
+    scores.  Long and short rows so that units cross sequence borders, one kv head per workgroup so that the heads of
+    a workgroup run different units, the append checked bit for bit."""
     g = torch.Generator().manual_seed(hq * 7 + hkv)
     batch = 9
     lengths = torch.randint(0, 2500, (batch,), generator=g)
     lengths[0], lengths[1], lengths[2] = 0, 15, 16
-    w = workloads.make_decode_workload("d256", seed=79, batch=batch, hq=hq, hkv=hkv, d=256, bs=16, kv=kv,
+    w = workloads.make_decode_workload("wide", seed=79, batch=batch, hq=hq, hkv=hkv, d=d, bs=16, kv=kv,
                                        lengths=lengths, device=DEV, quantize_fn=gpu_quantize, poison=True)  # fmt: skip
     before = _snapshot(w)
     out = run_decode(w, window_left=window_left)
-    assert_close(out, expected_decode(w, window_left=window_left), *tolerances(kv), what=f"D=256 {kv} {hq}/{hkv}")
+    assert_close(out, expected_decode(w, window_left=window_left), *tolerances(kv), what=f"D={d} {kv} {hq}/{hkv}")
     _check_append(w, before)
 
 
@@ -176,6 +178,12 @@ def test_error_behaviour_matches_the_reference_shim():
     empty = ops.areno_paged_causal_attention_decode(w.q[:0], w.k_update[:0], w.v_update[:0], w.k_cache, w.v_cache,
                                                     w.block_table[:0], w.cache_seqlens[:0])  # fmt: skip
     assert empty.shape == (0, 8, 64)
+    # the reference's shims record a backward; this build refuses such a call rather than drop the gradient
+    q_grad = w.q.clone().requires_grad_(True)
+    with pytest.raises(RuntimeError, match="backward is not implemented"):
+        ops.areno_paged_causal_attention_decode(q_grad, *args[1:])
+    with torch.no_grad():
+        ops.areno_paged_causal_attention_decode(q_grad, *args[1:])
 
 
 # ---- prefix groups: shared pages read once for several rows --------------------------------------------------------

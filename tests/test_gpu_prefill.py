@@ -22,7 +22,7 @@ def _packed(lens, hq, hkv, d, dtype, seed=0):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("window_left", [None, 0, 7])
-@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (28, 4, 128), (4, 4, 80), (8, 2, 256)])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (28, 4, 128), (4, 4, 80), (8, 2, 256), (6, 6, 192)])
 def test_varlen_new_tokens_only(dtype, window_left, hq, hkv, d):
     q, k, v, cu = _packed([5, 1, 130, 0, 67], hq, hkv, d, dtype)
     out = ops.areno_varlen_causal_attention(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), window_left=window_left)
@@ -63,16 +63,18 @@ def test_paged_prefill_shapes(hq, hkv, d, bs):
 
 
 @pytest.mark.parametrize("kv", ["bf16", "fp16", "int8", "fp8"])
+@pytest.mark.parametrize("d", [256, 192])
 @pytest.mark.parametrize("hq,hkv,window_left", [(16, 8, None), (8, 1, 40), (12, 4, None)])
-def test_paged_prefill_head_dim_256(kv, hq, hkv, window_left):
-    """Head dim 256 (the sliding-attention layers of the Gemma family, Qwen3.5) on the matrix-core kernel: one 16-row
-    tile per wave; a query block cut by many shares goes through the merge of 256-wide partials."""
+def test_paged_prefill_head_dims_192_256(kv, d, hq, hkv, window_left):
+    """Head dims 256 (the sliding-attention layers of the Gemma family, Qwen3.5) and 192 (128 + 64 rotary channels of
+    the MLA-style layers) on the matrix-core kernel: one 16-row tile per wave; a query block cut by many shares goes
+    through the merge of the wide partials."""
     new = torch.tensor([3, 150, 64, 1, 33])
     ctx = torch.tensor([900, 0, 77, 2500, 310])
-    w = workloads.make_prefill_workload("d256", seed=11 + hq, new_lens=new, ctx_lens=ctx, hq=hq, hkv=hkv, d=256, bs=16,
+    w = workloads.make_prefill_workload("wide", seed=11 + hq, new_lens=new, ctx_lens=ctx, hq=hq, hkv=hkv, d=d, bs=16,
                                         kv=kv, device=DEV, quantize_fn=gpu_quantize)  # fmt: skip
     assert_close(_run_prefill(w, window_left), _expected_prefill(w, window_left), *tolerances(kv),
-                 what=f"prefill D=256 {kv}")  # fmt: skip
+                 what=f"prefill D={d} {kv}")  # fmt: skip
 
 
 def test_write_then_prefill_then_decode_are_consistent():
