@@ -262,7 +262,7 @@ struct TileCursor {
 #ifndef ARENO_MFMA_QUANT_OCC
 #define ARENO_MFMA_QUANT_OCC 2
 #endif
-// DSPLIT > 1 serves heads of DSPLIT * D elements (256 = 2 x 128, 192 = 3 x 64): DSPLIT adjacent waves of the
+// DSPLIT > 1 serves heads of DSPLIT * D elements (256 = 2 x 128, 192 = 3 x 64, 512 = 4 x 128): DSPLIT adjacent waves of the
 // workgroup take one part of the head dimension each.  Every wave computes the part of S = K . Q^T over its
 // elements, the waves exchange the parts through LDS (a wave's K tile is dead once its products are issued, so the
 // part is parked there), add them in the same order and go on with identical scores: the same softmax in all,
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   constexpr float kPScale = T::kQuant ? 256.0f : 1.0f;
   constexpr int kWaveLds = TK * RSK + TK * RSV + 2 * TK * 4;
   static_assert(NLD >= 1 && LPT >= 4 && LPT <= 16, "unsupported head_dim");
-  static_assert(DSPLIT == 1 || ((DSPLIT == 2 || DSPLIT == 3) && !GROUPED && NW % DSPLIT == 0), "unsupported head split");
+  static_assert(DSPLIT == 1 || (DSPLIT >= 2 && DSPLIT <= 4 && !GROUPED && NW % DSPLIT == 0), "unsupported head split");
   constexpr int DFULL = D * DSPLIT;  // elements of a whole head (row of Q, of a cache page, of a partial)
 
   __shared__ __attribute__((aligned(16))) char s_tiles[NW][kWaveLds];
@@ -944,6 +944,15 @@ decode_mfma_fn decode_mfma_lookup_impl(int head_dim, bool scale16) {
       return decode_mfma_kernel<KIND, 128, false, NW, false, 2>;
     }
   }
+  if constexpr (!GROUPED && NW % 4 == 0) {
+    // head dim 512: four waves per head, 128 elements each
+    if (head_dim == 512) {
+      if constexpr (KVTraits<KIND>::kQuant) {
+        if (scale16) return decode_mfma_kernel<KIND, 128, true, NW, false, 4>;
+      }
+      return decode_mfma_kernel<KIND, 128, false, NW, false, 4>;
+    }
+  }
   if constexpr (!GROUPED) {
     // head dim 192: three waves per head, 64 elements each, in workgroups of six waves
     if (head_dim == 192) {
@@ -958,7 +967,9 @@ decode_mfma_fn decode_mfma_lookup_impl(int head_dim, bool scale16) {
 
 // Waves of a workgroup that share one head (the head-dimension split of decode_mfma_kernel), and the waves per
 // workgroup of the kernel the lookup returns for a head dim.
-inline int decode_mfma_head_split(int head_dim) { return head_dim == 256 ? 2 : (head_dim == 192 ? 3 : 1); }
+inline int decode_mfma_head_split(int head_dim) {
+  return head_dim == 256 ? 2 : (head_dim == 192 ? 3 : (head_dim == 512 ? 4 : 1));
+}
 inline int decode_mfma_waves(int head_dim) { return head_dim == 192 ? 6 : ARENO_MFMA_NW; }
 
 }  // namespace areno
