@@ -389,6 +389,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       if (v <= num_items) s_cum[v] = excl;
       excl += nt[j];
     }
+    // the entry behind the last thread's items has no owner of its own: it is the total when the list is full
+    if (tid == NW * kWave - 1 && SPT * (tid + 1) <= num_items) s_cum[SPT * (tid + 1)] = excl;
     __syncthreads();
   }
   // ---- unit geometry -----------------------------------------------------------------------------------

@@ -566,13 +566,52 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
 }  // namespace
 }  // namespace areno
 
+namespace areno {
+namespace {
+
+// Batches beyond what one launch of the matrix-core kernel indexes (kMfmaMaxBatch rows: its prefix sum over the rows
+// lives in LDS) run as consecutive launches over row ranges, on the same stream and through the same workspace.
+int decode_in_row_ranges(const areno_paged_cache* cache, const void* q, const void* k_update, const void* v_update,
+                         void* out, int32_t q_dtype, int32_t batch, int32_t q_heads, const int32_t* block_table,
+                         int32_t max_blocks, const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
+                         float softmax_scale, int32_t group_rows, const int32_t* shared_lens, void* workspace,
+                         size_t workspace_bytes, int32_t stages, void* stream) {
+  if (batch <= kMfmaMaxBatch || cache == nullptr || q == nullptr || out == nullptr || block_table == nullptr ||
+      cache_seqlens == nullptr || q_heads <= 0 || max_blocks <= 0 || cache->kv_heads <= 0 || cache->head_dim <= 0)
+    return decode_impl(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
+                       cache_seqlens, window_left, num_splits, softmax_scale, group_rows, shared_lens, workspace,
+                       workspace_bytes, stages, stream);
+  int rows_per_launch = kMfmaMaxBatch;
+  if (shared_lens != nullptr && group_rows > 1) rows_per_launch = kMfmaMaxBatch / group_rows * group_rows;
+  if (rows_per_launch <= 0) rows_per_launch = kMfmaMaxBatch;  // groups wider than a launch: decode_impl drops the hint
+  const size_t es = dtype_size(q_dtype);
+  const size_t q_row = static_cast<size_t>(q_heads) * cache->head_dim * es;
+  const size_t kv_row = static_cast<size_t>(cache->kv_heads) * cache->head_dim * es;
+  for (int32_t r0 = 0; r0 < batch; r0 += rows_per_launch) {
+    const int32_t rows = batch - r0 < rows_per_launch ? batch - r0 : rows_per_launch;
+    const bool grouped = shared_lens != nullptr && group_rows > 1 && rows_per_launch % group_rows == 0;
+    const int rc = decode_impl(
+        cache, static_cast<const char*>(q) + r0 * q_row,
+        k_update != nullptr ? static_cast<const char*>(k_update) + r0 * kv_row : nullptr,
+        v_update != nullptr ? static_cast<const char*>(v_update) + r0 * kv_row : nullptr,
+        static_cast<char*>(out) + r0 * q_row, q_dtype, rows, q_heads, block_table + static_cast<size_t>(r0) * max_blocks,
+        max_blocks, cache_seqlens + r0, window_left, num_splits, softmax_scale, grouped ? group_rows : 1,
+        grouped ? shared_lens + r0 / group_rows : nullptr, workspace, workspace_bytes, stages, stream);
+    if (rc != ARENO_OK) return rc;
+  }
+  return ARENO_OK;
+}
+
+}  // namespace
+}  // namespace areno
+
 extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, const void* q, const void* k_update,
                                              const void* v_update, void* out, int32_t q_dtype, int32_t batch,
                                              int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
                                              const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
                                              float softmax_scale, void* workspace, size_t workspace_bytes,
                                              int32_t stages, void* stream) {
-  return areno::decode_impl(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
+  return areno::decode_in_row_ranges(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
                             cache_seqlens, window_left, num_splits, softmax_scale, 0, nullptr, workspace,
                             workspace_bytes, stages, stream);
 }
@@ -598,7 +637,7 @@ extern "C" int areno_hip_paged_decode_grouped(const areno_paged_cache* cache, co
   if (shared_lens != nullptr && (group_rows < 1 || (batch > 0 && batch % group_rows != 0)))
     return areno::fail(ARENO_ERR_INVALID_ARGUMENT,
                        "areno_hip_paged_decode_grouped: batch %d is not a multiple of group_rows %d", batch, group_rows);
-  return areno::decode_impl(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
+  return areno::decode_in_row_ranges(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
                             cache_seqlens, window_left, num_splits, softmax_scale, group_rows, shared_lens, workspace,
                             workspace_bytes, stages, stream);
 }

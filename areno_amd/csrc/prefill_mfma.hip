@@ -103,7 +103,7 @@ __device__ __forceinline__ BlockTiles block_tiles(int n_new, int ctx, int j, int
   return b;
 }
 
-// Exclusive prefix sum of tile steps per sequence into s_cum[0 .. num_seqs] (all 256 threads take part).
+// Exclusive prefix sum of tile steps per sequence into s_cum[0 .. num_seqs] (all threads take part).
 __device__ __forceinline__ void prefix_tile_steps(const PrefillParams& p, int tq, int* s_cum, int* s_wave_tot) {
   constexpr int SPT = kMaxPrefillSeqs / kPrefillThreads;
   const int tid = threadIdx.x;
@@ -138,6 +138,8 @@ __device__ __forceinline__ void prefix_tile_steps(const PrefillParams& p, int tq
     if (s <= p.num_seqs) s_cum[s] = excl;
     excl += steps[i];
   }
+  // the entry behind the last thread's sequences has no owner of its own: it is the total when the list is full
+  if (tid == kPrefillThreads - 1 && SPT * (tid + 1) <= p.num_seqs) s_cum[SPT * (tid + 1)] = excl;
   __syncthreads();
 }
 

@@ -216,6 +216,23 @@ def test_prefix_groups_match_the_plain_op_and_the_oracle(kv, hq, hkv, samples):
             assert bool(same.all()), f"{name}: the append differs between the grouped and the plain op"
 
 
+def test_batches_beyond_one_launch_run_in_row_ranges():
+    """More rows than the matrix-core kernel indexes in one launch (1024): the library runs row ranges one after the
+    other; plain rows (1500) and rollout groups of 3 (1200 rows: ranges end on group borders)."""
+    g = torch.Generator().manual_seed(5)
+    lengths = torch.randint(0, 90, (1500,), generator=g)
+    w = workloads.make_decode_workload("wide-batch", seed=81, batch=1500, hq=8, hkv=2, d=128, bs=16, kv="int8",
+                                       lengths=lengths, device=DEV, quantize_fn=gpu_quantize, poison=True)  # fmt: skip
+    before = _snapshot(w)
+    out = run_decode(w)
+    assert_close(out, expected_decode(w), *tolerances("int8"), what="1500 rows")
+    _check_append(w, before)
+    r = workloads.cfg3_rollout("fp8", device=DEV, prompts=400, samples=3, prefix_lo=40, prefix_hi=120, median=30.0,
+                               cap=100, quantize_fn=gpu_quantize, seed=83, hq=8, hkv=2)  # fmt: skip
+    grouped = _grouped_decode(r)
+    assert_close(grouped, expected_decode(r), *tolerances("fp8"), what="1200 grouped rows")
+
+
 def test_prefix_groups_clip_an_overstated_shared_length():
     """shared_prefix_lens larger than what a row has cached is clipped to the shortest row of the group."""
     w = workloads.cfg3_rollout("fp8", device=DEV, prompts=3, samples=4, prefix_lo=64, prefix_hi=200, median=50.0,

@@ -77,6 +77,17 @@ def test_paged_prefill_head_dims_192_256(kv, d, hq, hkv, window_left):
                  what=f"prefill D={d} {kv}")  # fmt: skip
 
 
+def test_prefill_with_a_full_sequence_list():
+    """1024 sequences, the most one launch of the matrix-core kernel indexes: the prefix sum over the sequences must
+    also produce its last entry, the total."""
+    g = torch.Generator().manual_seed(3)
+    new = torch.randint(1, 4, (1024,), generator=g)
+    ctx = torch.randint(0, 40, (1024,), generator=g)
+    w = workloads.make_prefill_workload("full-list", seed=31, new_lens=new, ctx_lens=ctx, hq=4, hkv=2, d=64, bs=16,
+                                        kv="bf16", device=DEV)  # fmt: skip
+    assert_close(_run_prefill(w), _expected_prefill(w), *tolerances("bf16"), what="1024 sequences")
+
+
 def test_write_then_prefill_then_decode_are_consistent():
     """The three ops agree with each other: cache write of the new tokens, prefill with ctx,
     and n = 1 prefill == decode without append."""
