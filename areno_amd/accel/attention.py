@@ -21,9 +21,9 @@ defaulting to the reference behaviour:
   context (chunked prefill that re-reads earlier chunks).
 
 Everything runs as HIP kernels through ``areno_amd.accel._areno_accel``; there is no Python
-fallback and no autograd: the ops are used under ``torch.inference_mode`` / ``torch.no_grad``, and a call
-whose inputs require gradients while gradients are being recorded is refused instead of returning an
-output without a graph.
+fallback.  The varlen and dense ops are autograd functions with HIP backward kernels like the
+reference's; the paged ops (decode, paged prefill) are inference-only and refuse inputs that require
+gradients while gradients are being recorded, instead of returning an output without a graph.
 """
 
 from __future__ import annotations
@@ -52,13 +52,13 @@ def _contig(t: torch.Tensor | None) -> torch.Tensor | None:
 
 
 def _no_autograd(op: str, *tensors: torch.Tensor | None) -> None:
-    """The reference's shims are autograd functions with native backward kernels (``accel/attention.py:78-118,
-    145-183`` there) for its training backend.  This build serves inference only: rather than hand back an output
+    """The paged ops have no backward here (the reference's decode backward recomputes with its PyTorch reference,
+    ``accel/attention.py:245-264`` there; the paged prefill op is this build's own).  Rather than hand back an output
     that silently carries no gradient, a call that autograd would have to record is refused."""
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
         raise RuntimeError(
-            f"{op}: backward is not implemented in this build (inference path only); call it under "
-            "torch.no_grad() / torch.inference_mode() or detach the inputs"
+            f"{op}: backward is not implemented for the paged ops; call it under torch.no_grad() / "
+            "torch.inference_mode() or detach the inputs"
         )
 
 
@@ -71,6 +71,80 @@ def _check_scales(op: str, cache: torch.Tensor, k_scale, v_scale) -> None:
         raise ValueError(f"{op} got scales for an unquantized cache")
     if k_scale is not None and (k_scale.dim() != 3 or v_scale.dim() != 3):
         raise ValueError(f"{op} expects scales shaped (num_blocks, block_size, kv_heads)")
+
+
+class _VarlenCausalAttention(torch.autograd.Function):
+    """Forward and backward of the packed varlen op, as ``_ArenoVarlenCausalAttention`` in the reference
+    (``areno/accel/attention.py:145-183``): the forward saves q, k, v, the output and cu_seqlens; the backward kernels
+    return fp32 gradients that are cast to the inputs' dtypes."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seqlens, window_left: int, softmax_scale: float):
+        out = _extension().areno_varlen_causal_attention_forward(
+            q.contiguous(), k.contiguous(), v.contiguous(), cu_seqlens.contiguous(), window_left, softmax_scale
+        )
+        ctx.save_for_backward(q, k, v, out, cu_seqlens)
+        ctx.window_left = window_left
+        ctx.softmax_scale = softmax_scale
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        q, k, v, out, cu_seqlens = ctx.saved_tensors
+        dq, dk, dv = _extension().areno_attention_backward(
+            grad_output.contiguous(), q.contiguous(), k.contiguous(), v.contiguous(), out.contiguous(),
+            cu_seqlens.contiguous(), None, None, ctx.window_left, ctx.softmax_scale,
+        )  # fmt: skip
+        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None
+
+
+def _rows_of(x: torch.Tensor) -> torch.Tensor:
+    """``(batch, heads, seq, d)`` -> contiguous ``(batch * seq, heads, d)``."""
+    b, h, n, d = x.shape
+    return x.transpose(1, 2).reshape(b * n, h, d).contiguous()
+
+
+class _CausalAttention(torch.autograd.Function):
+    """Forward and backward of the dense op (``_ArenoCausalAttention``, ``areno/accel/attention.py:78-118`` there).
+    The forward is served by the paged prefill kernel: ``k`` / ``v`` are viewed as one page per batch row
+    (``block_size = Sk``) and ``query_start`` becomes the cached-context length."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, query_start: int, window_left: int, softmax_scale: float):
+        batch, heads, sq, d = q.shape
+        dev = q.device
+        k_pool = k.transpose(1, 2).contiguous()  # (batch, Sk, heads, D): one page per row
+        v_pool = v.transpose(1, 2).contiguous()
+        table = torch.arange(batch, device=dev, dtype=torch.int32).view(batch, 1)
+        cu = torch.arange(batch + 1, device=dev, dtype=torch.int32) * sq
+        start = torch.full((batch,), query_start, device=dev, dtype=torch.int32)
+        out = _extension().areno_paged_varlen_causal_attention_forward(
+            _rows_of(q), k_pool, v_pool, table, cu, start, window_left, softmax_scale, None, None
+        )
+        out = out.view(batch, sq, heads, d).transpose(1, 2)
+        ctx.save_for_backward(q, k, v, out)
+        ctx.query_start = query_start
+        ctx.window_left = window_left
+        ctx.softmax_scale = softmax_scale
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        q, k, v, out = ctx.saved_tensors
+        batch, heads, sq, d = q.shape
+        sk = k.shape[2]
+        dev = q.device
+        cu_q = torch.arange(batch + 1, device=dev, dtype=torch.int32) * sq
+        cu_k = torch.arange(batch + 1, device=dev, dtype=torch.int32) * sk
+        start = torch.full((batch,), ctx.query_start, device=dev, dtype=torch.int32)
+        dq, dk, dv = _extension().areno_attention_backward(
+            _rows_of(grad_output), _rows_of(q), _rows_of(k), _rows_of(v), _rows_of(out), cu_q, cu_k, start,
+            ctx.window_left, ctx.softmax_scale,
+        )  # fmt: skip
+        dq = dq.view(batch, sq, heads, d).transpose(1, 2)
+        dk = dk.view(batch, sk, heads, d).transpose(1, 2)
+        dv = dv.view(batch, sk, heads, d).transpose(1, 2)
+        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None
 
 
 @torch._dynamo.disable
@@ -158,7 +232,6 @@ def areno_varlen_causal_attention(
 ) -> torch.Tensor:
     """Apply packed causal attention to flat ``(tokens, heads, head_dim)`` tensors."""
     op = "areno_varlen_causal_attention"
-    _no_autograd(op, q, k, v)
     if not _all_on_gpu(q, k, v, cu_seqlens):
         raise RuntimeError(f"{op} requires CUDA q, k, v, and cu_seqlens tensors")
     if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
@@ -171,10 +244,7 @@ def areno_varlen_causal_attention(
         raise ValueError(f"{op} expects q heads to be divisible by kv heads")
     if q.shape[2] != k.shape[2] or q.shape[2] != v.shape[2]:
         raise ValueError(f"{op} head dim mismatch")
-    return _extension().areno_varlen_causal_attention_forward(
-        q.contiguous(), k.contiguous(), v.contiguous(), cu_seqlens.contiguous(),
-        _window_left(window_left), _scale(q, softmax_scale),
-    )  # fmt: skip
+    return _VarlenCausalAttention.apply(q, k, v, cu_seqlens, _window_left(window_left), _scale(q, softmax_scale))
 
 
 @torch._dynamo.disable
@@ -195,7 +265,6 @@ def areno_causal_attention(
     query may see exists as a key).
     """
     op = "areno_causal_attention"
-    _no_autograd(op, q, k, v)
     if not _all_on_gpu(q, k, v):
         raise RuntimeError(f"{op} requires CUDA q, k, and v tensors")
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
@@ -206,21 +275,10 @@ def areno_causal_attention(
         raise ValueError(f"{op} head count mismatch")
     if q.shape[-1] != k.shape[-1] or q.shape[-1] != v.shape[-1]:
         raise ValueError(f"{op} head dim mismatch")
-    batch, heads, sq, _ = q.shape
     sk = k.shape[2]
-    if sk < int(query_start) + sq:
-        raise ValueError(f"{op} needs at least query_start + q_len = {int(query_start) + sq} keys, got {sk}")
-    q_flat = q.transpose(1, 2).reshape(batch * sq, heads, q.shape[-1]).contiguous()
-    k_pool = k.transpose(1, 2).contiguous()  # (batch, Sk, heads, D): one page per row
-    v_pool = v.transpose(1, 2).contiguous()
-    dev = q.device
-    table = torch.arange(batch, device=dev, dtype=torch.int32).view(batch, 1)
-    cu = torch.arange(batch + 1, device=dev, dtype=torch.int32) * sq
-    ctx = torch.full((batch,), int(query_start), device=dev, dtype=torch.int32)
-    out = _extension().areno_paged_varlen_causal_attention_forward(
-        q_flat, k_pool, v_pool, table, cu, ctx, _window_left(window_left), _scale(q, softmax_scale), None, None
-    )
-    return out.view(batch, sq, heads, q.shape[-1]).transpose(1, 2)
+    if sk < int(query_start) + q.shape[2]:
+        raise ValueError(f"{op} needs at least query_start + q_len = {int(query_start) + q.shape[2]} keys, got {sk}")
+    return _CausalAttention.apply(q, k, v, int(query_start), _window_left(window_left), _scale(q, softmax_scale))
 
 
 @torch._dynamo.disable

@@ -458,6 +458,49 @@ std::vector<at::Tensor> block_tables_prefill_slots(at::Tensor table, at::Tensor 
   return {ids, offs, pos};
 }
 
+// Backward of the varlen / dense ops.  q / grad_out / out: (Tq, Hq, D); k / v: (Tk, Hkv, D); returns fp32 gradients
+// like the reference's launchers (attention.cu:786-811, 898-925 there).
+std::vector<at::Tensor> attention_backward(at::Tensor grad_out, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor out,
+                                           at::Tensor cu_q, c10::optional<at::Tensor> cu_k,
+                                           c10::optional<at::Tensor> context_lens, int64_t window_left,
+                                           double softmax_scale) {
+  const char* op = "areno_attention_backward";
+  for (const at::Tensor* t : {&grad_out, &q, &k, &v, &out}) {
+    TORCH_CHECK(t->is_cuda(), op, " tensors must be CUDA");
+    TORCH_CHECK(t->is_contiguous(), op, " tensors must be contiguous");
+    TORCH_CHECK(t->dim() == 3, op, " expects 3D tensors (tokens, heads, head_dim)");
+    TORCH_CHECK(t->scalar_type() == q.scalar_type(), op, " dtype mismatch");
+  }
+  TORCH_CHECK(grad_out.sizes() == q.sizes() && out.sizes() == q.sizes(), op, " grad/out shape mismatch");
+  TORCH_CHECK(k.sizes() == v.sizes(), op, " key/value shape mismatch");
+  TORCH_CHECK(q.size(1) % k.size(1) == 0, op, " q heads must be divisible by kv heads");
+  TORCH_CHECK(q.size(2) == k.size(2), op, " head dim mismatch");
+  auto check_i32 = [&](const at::Tensor& t, int64_t n, const char* name) {
+    TORCH_CHECK(t.is_cuda() && t.is_contiguous() && t.scalar_type() == at::kInt && t.dim() == 1 && t.size(0) == n, op,
+                " ", name, " must be a contiguous CUDA int32 vector of ", n, " entries");
+  };
+  TORCH_CHECK(cu_q.dim() == 1 && cu_q.size(0) >= 2, op, " cu_seqlens must contain at least one sequence");
+  const int64_t num_seqs = cu_q.size(0) - 1;
+  check_i32(cu_q, num_seqs + 1, "cu_seqlens_q");
+  if (cu_k.has_value()) check_i32(*cu_k, num_seqs + 1, "cu_seqlens_k");
+  if (context_lens.has_value()) check_i32(*context_lens, num_seqs, "context_lens");
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(q));
+  const auto fopts = q.options().dtype(at::kFloat);
+  at::Tensor dq = at::empty(q.sizes(), fopts), dk = at::empty(k.sizes(), fopts), dv = at::empty(v.sizes(), fopts);
+  const size_t ws_bytes = areno_hip_attention_backward_workspace_bytes(q.size(0), static_cast<int32_t>(q.size(1)));
+  at::Tensor workspace = at::empty({static_cast<int64_t>(ws_bytes)}, q.options().dtype(at::kByte));
+  const int status = areno_hip_attention_backward(
+      grad_out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dq.data_ptr<float>(),
+      dk.data_ptr<float>(), dv.data_ptr<float>(), dtype_code(q, op, "q"), q.size(0), k.size(0),
+      static_cast<int32_t>(q.size(1)), static_cast<int32_t>(k.size(1)), static_cast<int32_t>(q.size(2)),
+      cu_q.data_ptr<int32_t>(), cu_k.has_value() ? cu_k->data_ptr<int32_t>() : nullptr,
+      context_lens.has_value() ? context_lens->data_ptr<int32_t>() : nullptr, static_cast<int32_t>(num_seqs),
+      static_cast<int32_t>(window_left), static_cast<float>(softmax_scale), workspace.data_ptr(), ws_bytes,
+      current_stream(q));
+  check_status(status, op);
+  return {dq, dk, dv};
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -479,5 +522,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "device-resident block tables: pages for the next decode position, then the padded table");
   m.def("areno_block_tables_prefill_slots", &block_tables_prefill_slots,
         "device-resident block tables: page id, slot and position of packed prefill tokens");
+  m.def("areno_attention_backward", &attention_backward, "gradients of the varlen / dense causal attention ops");
   m.def("abi_version", &areno_hip_abi_version, "C ABI version of libareno_hip.so");
 }

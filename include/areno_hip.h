@@ -293,6 +293,27 @@ int areno_hip_block_tables_prefill_slots(const areno_block_tables* tables, const
                                          int64_t* out_block_ids, int64_t* out_block_offsets, int64_t* out_positions,
                                          void* stream);
 
+/*
+ * Backward of the causal varlen / dense attention ops: areno_varlen_causal_attention_backward_cuda and
+ * areno_causal_attention_backward_cuda (areno/accel/csrc/attention.cu:753-811,862-925), which the reference's
+ * autograd functions call (areno/accel/attention.py:104-118,170-183).  Gradients are fp32 and every element is
+ * written (no zero-fill needed), as there.
+ *   grad_out, q, out  device [q_tokens, q_heads, head_dim];  k, v  device [k_tokens, kv_heads, head_dim];  all `dtype`
+ *                     (F32 / F16 / BF16), 16-byte aligned
+ *   grad_q            device [q_tokens, q_heads, head_dim] float;  grad_k, grad_v  device [k_tokens, kv_heads, head_dim] float
+ *   cu_seqlens_q      device [num_seqs + 1] int32;  cu_seqlens_k  the same for the keys, NULL = cu_seqlens_q (varlen op)
+ *   context_lens      device [num_seqs] int32 position of each sequence's first query, NULL = 0 (dense op: query_start)
+ *   workspace         areno_hip_attention_backward_workspace_bytes(q_tokens, q_heads) bytes: per-row log-sum-exp and dO . O
+ * head_dim 64, 128, 192 or 256.  Two launches; deterministic (no atomics).
+ */
+size_t areno_hip_attention_backward_workspace_bytes(int64_t q_tokens, int32_t q_heads);
+int areno_hip_attention_backward(const void* grad_out, const void* q, const void* k, const void* v, const void* out,
+                                 float* grad_q, float* grad_k, float* grad_v, int32_t dtype, int64_t q_tokens,
+                                 int64_t k_tokens, int32_t q_heads, int32_t kv_heads, int32_t head_dim,
+                                 const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* context_lens,
+                                 int32_t num_seqs, int32_t window_left, float softmax_scale, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

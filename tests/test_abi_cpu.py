@@ -35,7 +35,8 @@ def test_header_declares_the_expected_entry_points():
                      "areno_hip_block_tables_init", "areno_hip_block_tables_reserve",
                      "areno_hip_block_tables_ensure_decode", "areno_hip_block_tables_release",
                      "areno_hip_block_tables_gather", "areno_hip_block_tables_decode_step",
-                     "areno_hip_block_tables_prefill_slots"):  # fmt: skip
+                     "areno_hip_block_tables_prefill_slots", "areno_hip_attention_backward",
+                     "areno_hip_attention_backward_workspace_bytes"):  # fmt: skip
         assert required in names
 
 
