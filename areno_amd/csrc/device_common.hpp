@@ -100,21 +100,24 @@ __device__ __forceinline__ void swap_rows32(uint32_t& a, uint32_t& b) {
   asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
 }
 
-// max without the canonicalising self-max the compiler puts in front of every fmaxf operand whose origin it cannot
-// see (IEEE mode); the hardware instruction already returns the other operand for a NaN input.
-__device__ __forceinline__ float max_f32(float a, float b) {
-  float r;
-  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
+// Maxima as plain compiler-visible operations, so that the compiler's hazard handling around matrix-core
+// instructions covers them (a VALU write into a register that an MFMA issued a few cycles earlier still reads as its
+// C operand needs wait states that only the compiler can place; an inline-asm v_max3_f32 that the register allocator
+// put there corrupted scores).  The build passes -fno-honor-nans, which is what lets fmaxf become a bare v_max_f32 /
+// v_max3_f32 without a canonicalising self-max in front of every operand; no kernel here produces or tests for NaN.
+__device__ __forceinline__ float max_f32(float a, float b) { return __builtin_fmaxf(a, b); }
 __device__ __forceinline__ float max3_f32(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
+  return __builtin_fmaxf(__builtin_fmaxf(a, b), c);
 }
 // x *= f in the register x lives in: as a plain multiply under a rarely taken branch the compiler copies whole
-// accumulator sets around the branch instead.
+// accumulator sets around the branch instead.  The compiler places hazard wait states only for its own instructions,
+// not for inline asm: a factor that comes straight out of a transcendental op (v_exp_f32) must pass through
+// settled() first, or the first multiply issued behind it reads the register before the result has landed.
 __device__ __forceinline__ void scale_in_place(float& x, float f) { asm("v_mul_f32 %0, %1, %0" : "+v"(x) : "v"(f)); }
+__device__ __forceinline__ float settled(float x) {
+  asm("s_nop 1" : "+v"(x));
+  return x;
+}
 
 __device__ __forceinline__ float rows_max(float x) {
   uint32_t a = __builtin_bit_cast(uint32_t, x), b = a;

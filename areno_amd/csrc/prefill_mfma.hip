@@ -510,26 +510,33 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
       scores(t + 1, s_next);  // past tb this reads a buffer of clamped or stale keys; the result is dropped
       // -- online softmax in the log2 domain; the (positive) softmax scale is applied to the row maximum and inside
       // the exponent's multiply-add -----------------------------------------------------------------------------------
-      float m_safe[kRowTiles], alpha[kRowTiles];
-      bool changed = false;
+      // The reference value m of a row only has to be the same for all its keys and to bound the scores well enough
+      // for the exponentials to fit the operand type; it need not be the exact maximum.  So it is raised (and the
+      // accumulators rescaled) only when a tile's scores exceed it by more than kLazy in the log2 domain (a factor
+      // 2^kLazy in the probabilities, far inside fp16's range); each lane checks its own eight scores and one ballot
+      // decides for the wave, which skips the cross-lane maximum and the rescale on most tiles.
+      constexpr float kLazy = 8.0f;
+      float mt_lane[kRowTiles];
+      bool raise = false;
 #pragma unroll
       for (int nq = 0; nq < kRowTiles; ++nq) {
-        float mt = max3_f32(max3_f32(s_cur[nq][0][0], s_cur[nq][0][1], s_cur[nq][0][2]),
-                            max3_f32(s_cur[nq][0][3], s_cur[nq][1][0], s_cur[nq][1][1]),
-                            max3_f32(s_cur[nq][1][2], s_cur[nq][1][3], s_cur[nq][1][3]));
-        mt = rows_max(mt) * p.scale_log2e;
-        const float m_new = max_f32(m_run[nq], mt);
-        m_safe[nq] = m_new == kNegInf ? 0.0f : m_new;
-        alpha[nq] = fast_exp2(m_run[nq] - m_safe[nq]);
-        m_run[nq] = m_new;
-        changed = changed || alpha[nq] != 1.0f;
+        mt_lane[nq] = max3_f32(max3_f32(s_cur[nq][0][0], s_cur[nq][0][1], s_cur[nq][0][2]),
+                               max3_f32(s_cur[nq][0][3], s_cur[nq][1][0], s_cur[nq][1][1]),
+                               max3_f32(s_cur[nq][1][2], s_cur[nq][1][3], s_cur[nq][1][3]));
+        // (-inf > -inf + kLazy is false: a fully masked row stays at -inf; anything finite beats -inf)
+        raise = raise | (mt_lane[nq] * p.scale_log2e > m_run[nq] + kLazy);  // no short circuit: straight-line code
       }
-      if (__builtin_amdgcn_ballot_w64(changed) != 0) {
+      if (__builtin_amdgcn_ballot_w64(raise) != 0) {
 #pragma unroll
         for (int nq = 0; nq < kRowTiles; ++nq) {
+          const float mt = rows_max(mt_lane[nq]) * p.scale_log2e;
+          const float m_new = max_f32(m_run[nq], mt);
+          const float m_ref = m_new == kNegInf ? 0.0f : m_new;
+          const float alpha = settled(fast_exp2(m_run[nq] - m_ref));
+          m_run[nq] = m_new;
           {
             float l0 = l_acc[nq][0];
-            scale_in_place(l0, alpha[nq]);
+            scale_in_place(l0, alpha);
             l_acc[nq][0] = l0;
           }
 #pragma unroll
@@ -537,12 +544,15 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               float a = acc[nq][nb][j];
-              scale_in_place(a, alpha[nq]);
+              scale_in_place(a, alpha);
               acc[nq][nb][j] = a;
             }
           }
         }
       }
+      float m_safe[kRowTiles];
+#pragma unroll
+      for (int nq = 0; nq < kRowTiles; ++nq) m_safe[nq] = m_run[nq] == kNegInf ? 0.0f : m_run[nq];
       V8 pop[kRowTiles];
 #pragma unroll
       for (int nq = 0; nq < kRowTiles; ++nq) {
