@@ -31,6 +31,35 @@ def test_varlen_new_tokens_only(dtype, window_left, hq, hkv, d):
     assert_close(out, want, *tolerances("bf16"), what="varlen")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d", [64, 128, 192, 256])
+@pytest.mark.parametrize("profile", ["climb", "jump", "fall", "wide"])
+def test_varlen_score_ranges_that_move_along_the_keys(dtype, d, profile):
+    """The matrix-core kernel keeps a softmax reference value per row that it raises only when a key tile exceeds it
+    by a margin, so rows whose scores climb slowly (the reference lags), jump far (a late raise rescales everything
+    before it), fall (the first tile dominates) or spread over a wide range all have to come out like the oracle's
+    exact-maximum softmax."""
+    lens = [300, 33, 1, 150]
+    q, k, v, cu = _packed(lens, 4, 2, d, torch.float32, seed=d)
+    pos = torch.cat([torch.arange(n, dtype=torch.float32) for n in lens])
+    if profile == "climb":  # a shared direction whose weight grows by a little per key
+        gain = 0.02 * pos
+    elif profile == "jump":  # every 97th key scores far above its neighbours
+        gain = torch.where(pos % 97 == 96, 9.0, 0.0)
+    elif profile == "fall":
+        gain = 6.0 - 0.03 * pos
+    else:
+        gain = torch.zeros_like(pos)
+        q, k = 5.0 * q, 5.0 * k
+    direction = torch.ones(d) * (d**-0.5)
+    q = q + 2.0 * (d**0.25) * direction  # every query has a component along the shared direction
+    k = k + gain[:, None, None] * (d**0.25) * direction
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    out = ops.areno_varlen_causal_attention(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV))
+    want = ar.ref_varlen(q, k, v, cu, ar.window_left_arg(None), d**-0.5)
+    assert_close(out, want, *tolerances("bf16"), what=f"varlen {profile}")
+
+
 def _expected_prefill(w, window_left=None):
     kc, vc = dequant_cpu(w.k_cache, w.k_scale), dequant_cpu(w.v_cache, w.v_scale)
     return ar.ref_paged_varlen_prefill(w.q.cpu().float(), kc, vc, w.block_table.cpu(), w.cu_seqlens_q.cpu(),
