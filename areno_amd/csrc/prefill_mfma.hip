@@ -485,28 +485,41 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
 
     // ---- iteration t: staging first, then the scores of tile t + 1 go to the matrix cores in the same block as the row
     // maxima of tile t ---------------------------------------------------------------------------------------------------
-    for (int t = ta; t <= tb; ++t) {
+    // One tile step is a lambda over (scores of tile t, room for the scores of tile t + 1) and the loop calls it twice
+    // with the two arrays swapped: the scores of the next tile are then computed where the following step reads them
+    // and no per-tile register copy of the 8 * kRowTiles scores is left.
+    float s_alt[kRowTiles][2][4];
+    auto tile_step = [&](int t, float (&s_cur)[kRowTiles][2][4], float (&s_next)[kRowTiles][2][4]) {
       __syncthreads();
       stage(t);
-      if (!wave_live) continue;
+      if (!wave_live) return;
       const int k0 = t * TK;
       const bool need_mask = k0 + TK - 1 > wave_qmin || (p.window_left >= 0 && k0 < wave_qmax - p.window_left);
       if (need_mask) {
 #pragma unroll
         for (int nq = 0; nq < kRowTiles; ++nq) {
+          // key 16 tg + j of this lane's 4-key groups is visible iff its index is <= hi (causal) and >= hi - window
+          const int hi = q_pos[nq] - k0 - 4 * lk;
+          if (p.window_left < 0) {
 #pragma unroll
-          for (int tg = 0; tg < 2; ++tg) {
+            for (int tg = 0; tg < 2; ++tg) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const int kpos = k0 + 16 * tg + 4 * lk + j;
-              bool ok = kpos <= q_pos[nq];
-              if (p.window_left >= 0) ok = ok && kpos >= q_pos[nq] - p.window_left;
-              s_cur[nq][tg][j] = ok ? s_cur[nq][tg][j] : kNegInf;
+              for (int j = 0; j < 4; ++j) s_cur[nq][tg][j] = 16 * tg + j <= hi ? s_cur[nq][tg][j] : kNegInf;
+            }
+          } else {
+            const int lo = hi - p.window_left;
+            const uint32_t span = static_cast<uint32_t>(p.window_left);
+#pragma unroll
+            for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const bool ok = static_cast<uint32_t>(16 * tg + j - lo) <= span;  // 0 <= index - lo <= window
+                s_cur[nq][tg][j] = ok ? s_cur[nq][tg][j] : kNegInf;
+              }
             }
           }
         }
       }
-      float s_next[kRowTiles][2][4];
       scores(t + 1, s_next);  // past tb this reads a buffer of clamped or stale keys; the result is dropped
       // -- online softmax in the log2 domain; the (positive) softmax scale is applied to the row maximum and inside
       // the exponent's multiply-add -----------------------------------------------------------------------------------
@@ -589,14 +602,11 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
 #pragma unroll
         for (int nq = 0; nq < kRowTiles; ++nq) acc[nq][nb] = Ops::mfma(vop, pop[nq], acc[nq][nb]);
       }
-#pragma unroll
-      for (int nq = 0; nq < kRowTiles; ++nq) {
-#pragma unroll
-        for (int tg = 0; tg < 2; ++tg) {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) s_cur[nq][tg][j] = s_next[nq][tg][j];
-        }
-      }
+    };
+    for (int t = ta; t <= tb; t += 2) {
+      tile_step(t, s_cur, s_alt);
+      if (t + 1 > tb) break;
+      tile_step(t + 1, s_alt, s_cur);
     }
 
     // ---- finish the segment: final rows go to `out`, a cut item leaves its partial in the workspace ---------------
