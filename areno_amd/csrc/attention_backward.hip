@@ -15,7 +15,9 @@
 // Geometry: sequence s has queries [cu_q[s], cu_q[s+1]) at positions ctx[s] + i and keys [cu_k[s], cu_k[s+1]) at
 // positions 0 ..; query at position t sees keys max(0, t - window) .. t.  The varlen op has cu_k = cu_q, ctx = 0; the
 // dense op one sequence per batch row with ctx = query_start.
-// Head dims 64, 128, 192, 256 (a quarter of the head per lane in registers); 16-bit or fp32 inputs.
+// Head dims that are multiples of 8 up to 256: a lane owns a quarter of the head in registers, 16 / 32 / 48 / 64
+// elements wide (the smallest that covers the head; slices past the head's end read as zeros and are not stored);
+// 16-bit or fp32 inputs.
 
 #include "device_common.hpp"
 
@@ -41,6 +43,7 @@ struct BwdParams {
   int32_t q_heads;
   int32_t kv_heads;
   int32_t window_left;
+  int32_t head_dim;
   int32_t dtype;
   float scale;
   float scale_log2e;
@@ -64,14 +67,15 @@ __device__ __forceinline__ int find_seq(const int32_t* cu, int num_seqs, int64_t
   return lo;
 }
 
-// EPL consecutive elements starting at element index idx (a multiple of 8) as floats
+// The first `valid` (a multiple of 8) of EPL consecutive elements starting at element index idx (a multiple of 8) as
+// floats, zeros behind them
 template <int EPL>
-__device__ __forceinline__ void load_slice(const void* base, int64_t idx, int dtype, float (&x)[EPL]) {
+__device__ __forceinline__ void load_slice(const void* base, int64_t idx, int dtype, int valid, float (&x)[EPL]) {
   if (dtype == ARENO_DT_F32) {
     const float4_t* src = reinterpret_cast<const float4_t*>(static_cast<const float*>(base) + idx);
 #pragma unroll
     for (int c = 0; c < EPL / 4; ++c) {
-      const float4_t w = src[c];
+      const float4_t w = 4 * c < valid ? src[c] : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int j = 0; j < 4; ++j) x[4 * c + j] = w[j];
     }
@@ -79,7 +83,7 @@ __device__ __forceinline__ void load_slice(const void* base, int64_t idx, int dt
     const uint4_t* src = reinterpret_cast<const uint4_t*>(static_cast<const uint16_t*>(base) + idx);
 #pragma unroll
     for (int c = 0; c < EPL / 8; ++c) {
-      const uint4_t w = src[c];
+      const uint4_t w = 8 * c < valid ? src[c] : uint4_t{0u, 0u, 0u, 0u};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (dtype == ARENO_DT_BF16) {
@@ -110,7 +114,7 @@ __device__ __forceinline__ float groups_sum(float x) {
 
 template <int EPL>
 __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_rows_kernel(BwdParams p) {
-  constexpr int D = EPL * kLanesPerKey;
+  const int D = p.head_dim;
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t row = static_cast<int64_t>(blockIdx.x) * kBwdWaves + (threadIdx.x >> 6);
   if (row >= p.q_tokens * p.q_heads) return;
@@ -119,12 +123,13 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_rows_kern
   const int kvh = h / (p.q_heads / p.kv_heads);
   const int grp = lane / kLanesPerKey;
   const int sub = lane % kLanesPerKey;
+  const int valid_e = min(max(D - sub * EPL, 0), EPL);  // elements of this lane's slice that lie inside the head
   const int64_t q_base = row * D + sub * EPL;
 
   if (token >= p.cu_q[p.num_seqs]) {  // rows past the last sequence take part in nothing
 #pragma unroll
     for (int e = 0; e < EPL; ++e) {
-      if (grp == 0) p.grad_q[q_base + e] = 0.0f;
+      if (grp == 0 && e < valid_e) p.grad_q[q_base + e] = 0.0f;
     }
     return;
   }
@@ -136,12 +141,12 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_rows_kern
   const int first = (p.window_left >= 0 && q_pos > p.window_left) ? q_pos - p.window_left : 0;
 
   float qv[EPL], go[EPL];
-  load_slice<EPL>(p.q, q_base, p.dtype, qv);
-  load_slice<EPL>(p.grad_out, q_base, p.dtype, go);
+  load_slice<EPL>(p.q, q_base, p.dtype, valid_e, qv);
+  load_slice<EPL>(p.grad_out, q_base, p.dtype, valid_e, go);
   float d_part = 0.0f;
   {
     float ov[EPL];
-    load_slice<EPL>(p.out, q_base, p.dtype, ov);
+    load_slice<EPL>(p.out, q_base, p.dtype, valid_e, ov);
 #pragma unroll
     for (int e = 0; e < EPL; ++e) d_part += go[e] * ov[e];
   }
@@ -155,7 +160,7 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_rows_kern
     const int pos = base + grp;
     const bool valid = pos <= last;
     float kx[EPL];
-    load_slice<EPL>(p.k, key_base(valid ? pos : last), p.dtype, kx);
+    load_slice<EPL>(p.k, key_base(valid ? pos : last), p.dtype, valid_e, kx);
     float dot = 0.0f;
 #pragma unroll
     for (int e = 0; e < EPL; ++e) dot += qv[e] * kx[e];
@@ -183,8 +188,8 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_rows_kern
     const bool valid = pos <= last;
     const int64_t kb = key_base(valid ? pos : last);
     float kx[EPL], vx[EPL];
-    load_slice<EPL>(p.k, kb, p.dtype, kx);
-    load_slice<EPL>(p.v, kb, p.dtype, vx);
+    load_slice<EPL>(p.k, kb, p.dtype, valid_e, kx);
+    load_slice<EPL>(p.v, kb, p.dtype, valid_e, vx);
     float dot = 0.0f, dpv = 0.0f;
 #pragma unroll
     for (int e = 0; e < EPL; ++e) {
@@ -200,13 +205,13 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_rows_kern
 #pragma unroll
   for (int e = 0; e < EPL; ++e) {
     const float total = groups_sum(acc[e]);
-    if (grp == 0) p.grad_q[q_base + e] = total * p.scale;
+    if (grp == 0 && e < valid_e) p.grad_q[q_base + e] = total * p.scale;
   }
 }
 
 template <int EPL>
 __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_keys_kernel(BwdParams p) {
-  constexpr int D = EPL * kLanesPerKey;
+  const int D = p.head_dim;
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t krow = static_cast<int64_t>(blockIdx.x) * kBwdWaves + (threadIdx.x >> 6);
   if (krow >= p.k_tokens * p.kv_heads) return;
@@ -215,6 +220,7 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_keys_kern
   const int group = p.q_heads / p.kv_heads;
   const int grp = lane / kLanesPerKey;
   const int sub = lane % kLanesPerKey;
+  const int valid_e = min(max(D - sub * EPL, 0), EPL);
   const int64_t k_base = krow * D + sub * EPL;
 
   float dk[EPL], dv[EPL];
@@ -231,8 +237,8 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_keys_kern
     const int i_hi = p.window_left >= 0 ? min(n_q - 1, pos + p.window_left - ctx) : n_q - 1;
     if (i_lo <= i_hi) {
       float kx[EPL], vx[EPL];
-      load_slice<EPL>(p.k, k_base, p.dtype, kx);
-      load_slice<EPL>(p.v, k_base, p.dtype, vx);
+      load_slice<EPL>(p.k, k_base, p.dtype, valid_e, kx);
+      load_slice<EPL>(p.v, k_base, p.dtype, valid_e, vx);
       const int64_t pairs = static_cast<int64_t>(i_hi - i_lo + 1) * group;
       for (int64_t t0 = 0; t0 < pairs; t0 += kKeysPerPass) {
         const int64_t t = t0 + grp;
@@ -242,8 +248,8 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_keys_kern
         const int hh = static_cast<int>(tc % group);
         const int64_t row = (q_begin + i) * p.q_heads + kvh * group + hh;
         float qv[EPL], go[EPL];
-        load_slice<EPL>(p.q, row * D + sub * EPL, p.dtype, qv);
-        load_slice<EPL>(p.grad_out, row * D + sub * EPL, p.dtype, go);
+        load_slice<EPL>(p.q, row * D + sub * EPL, p.dtype, valid_e, qv);
+        load_slice<EPL>(p.grad_out, row * D + sub * EPL, p.dtype, valid_e, go);
         const float lse = p.row_stats[row * 2];
         const float d_row = p.row_stats[row * 2 + 1];
         float dot = 0.0f, dpv = 0.0f;
@@ -267,7 +273,7 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_keys_kern
   for (int e = 0; e < EPL; ++e) {
     const float tk = groups_sum(dk[e]);
     const float tv = groups_sum(dv[e]);
-    if (grp == 0) {
+    if (grp == 0 && e < valid_e) {
       p.grad_k[k_base + e] = tk * p.scale;
       p.grad_v[k_base + e] = tv;
     }
@@ -276,24 +282,21 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_keys_kern
 
 typedef void (*bwd_fn)(BwdParams);
 
+// the narrowest per-lane slice whose four lanes cover the head
 bwd_fn rows_kernel_for(int head_dim) {
-  switch (head_dim) {
-    case 64: return attention_backward_rows_kernel<16>;
-    case 128: return attention_backward_rows_kernel<32>;
-    case 192: return attention_backward_rows_kernel<48>;
-    case 256: return attention_backward_rows_kernel<64>;
-    default: return nullptr;
-  }
+  if (head_dim <= 0 || head_dim > 256 || head_dim % 8 != 0) return nullptr;
+  if (head_dim <= 64) return attention_backward_rows_kernel<16>;
+  if (head_dim <= 128) return attention_backward_rows_kernel<32>;
+  if (head_dim <= 192) return attention_backward_rows_kernel<48>;
+  return attention_backward_rows_kernel<64>;
 }
 
 bwd_fn keys_kernel_for(int head_dim) {
-  switch (head_dim) {
-    case 64: return attention_backward_keys_kernel<16>;
-    case 128: return attention_backward_keys_kernel<32>;
-    case 192: return attention_backward_keys_kernel<48>;
-    case 256: return attention_backward_keys_kernel<64>;
-    default: return nullptr;
-  }
+  if (head_dim <= 0 || head_dim > 256 || head_dim % 8 != 0) return nullptr;
+  if (head_dim <= 64) return attention_backward_keys_kernel<16>;
+  if (head_dim <= 128) return attention_backward_keys_kernel<32>;
+  if (head_dim <= 192) return attention_backward_keys_kernel<48>;
+  return attention_backward_keys_kernel<64>;
 }
 
 }  // namespace
@@ -320,7 +323,7 @@ extern "C" int areno_hip_attention_backward(const void* grad_out, const void* q,
   bwd_fn rows = rows_kernel_for(head_dim);
   bwd_fn keys = keys_kernel_for(head_dim);
   if (rows == nullptr || keys == nullptr)
-    return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim %d (64, 128, 192 and 256 are built)", op, head_dim);
+    return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim %d (multiples of 8 up to 256 are built)", op, head_dim);
   if (q_tokens == 0 && k_tokens == 0) return ARENO_OK;
   if (grad_out == nullptr || q == nullptr || k == nullptr || v == nullptr || out == nullptr || grad_q == nullptr ||
       grad_k == nullptr || grad_v == nullptr || cu_seqlens_q == nullptr)
@@ -355,6 +358,7 @@ extern "C" int areno_hip_attention_backward(const void* grad_out, const void* q,
   p.q_heads = q_heads;
   p.kv_heads = kv_heads;
   p.window_left = window_left;
+  p.head_dim = head_dim;
   p.dtype = dtype;
   p.scale = softmax_scale;
   p.scale_log2e = softmax_scale * kLog2e;

@@ -29,7 +29,7 @@ def _close(got, want, rel, what):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("window_left", [None, 0, 9])
-@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (6, 3, 128), (4, 4, 192), (4, 1, 256)])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (6, 3, 128), (4, 4, 192), (4, 1, 256), (4, 4, 80), (4, 1, 96), (2, 1, 8), (6, 2, 200)])
 def test_varlen_backward(dtype, window_left, hq, hkv, d):
     g = torch.Generator().manual_seed(hq * 17 + d)
     lens = [5, 1, 70, 0, 33]
@@ -83,8 +83,10 @@ def test_backward_is_deterministic_and_refuses_other_head_dims():
         grads.append((qd.grad, kd.grad, vd.grad))
     for a, b_ in zip(*grads):
         assert torch.equal(a, b_), "no atomics: two runs must agree bit for bit"
-    q80 = torch.randn(10, 2, 80, device=DEV, dtype=torch.bfloat16, requires_grad=True)
-    cu80 = torch.tensor([0, 10], dtype=torch.int32, device=DEV)
-    out = ops.areno_varlen_causal_attention(q80, q80.detach(), q80.detach(), cu80)
-    with pytest.raises(RuntimeError, match="head_dim 80"):
-        out.sum().backward()
+    # head dims the backward kernels do not cover (not a multiple of 8, or above 256) are refused by name
+    for d in (20, 264):
+        qx = torch.randn(10, 2, d, device=DEV, dtype=torch.float32, requires_grad=True)
+        cux = torch.tensor([0, 10], dtype=torch.int32, device=DEV)
+        out = ops.areno_varlen_causal_attention(qx, qx.detach(), qx.detach(), cux)
+        with pytest.raises(RuntimeError, match=f"head_dim {d}"):
+            out.sum().backward()
