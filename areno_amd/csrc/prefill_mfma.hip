@@ -265,12 +265,18 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
                                  (OPK == KV_F16 && p.q_dtype == ARENO_DT_F16);
   const bool packed = p.block_table == nullptr;  // K/V are (tokens, kv_heads, D): key t of a sequence is row q_begin + t
   constexpr int64_t row_bytes = static_cast<int64_t>(D) * ES;
+  // A tile whose K and V chunks together are at most one per thread (8-bit tiles up to head dim 128, 16-bit ones at
+  // 64) is staged with the workgroup split in two: the first half of the waves fetch, convert and publish K, the
+  // second half V, one chunk per thread.  Otherwise every thread handles chunk i of K and of V for i < NLD, and for
+  // such a tile the upper half of the workgroup would fetch clamped duplicates and publish nothing.
+  constexpr bool kRoleSplit = 2 * CHUNKS <= kPrefillThreads;
+  const bool role_v = kRoleSplit && wave >= kPrefillWaves / 2;  // wave-uniform
   // this thread's chunks of a tile: token and 16-byte column, fixed for the whole kernel
   int chunk_tok[NLD], chunk_col[NLD];
   bool chunk_live[NLD];
 #pragma unroll
   for (int i = 0; i < NLD; ++i) {
-    const int c = tid + kPrefillThreads * i;
+    const int c = (kRoleSplit && role_v ? tid - kPrefillThreads / 2 : tid) + kPrefillThreads * i;
     chunk_live[i] = (i + 1) * kPrefillThreads <= CHUNKS || c < CHUNKS;
     chunk_tok[i] = min(c, CHUNKS - 1) / LPT;
     chunk_col[i] = min(c, CHUNKS - 1) % LPT;
@@ -445,13 +451,39 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
     // iteration was the last to read, then K[t + 3], V[t + 2] and the block ids of tile t + 4 are fetched.  It runs for
     // every t (key positions are clamped into the item's range): tiles outside [ta, tb] land in buffers nobody reads.
     auto stage = [&](int t) {
-      publish_k(t + 2);
-      publish_v(t + 1);
-      issue_v();  // rows of tile t + 2, remembered when its K chunk was fetched
+      if constexpr (kRoleSplit) {
+        // one chunk per thread: kreg / ksreg / ids hold the K chunk in a K wave and the V chunk in a V wave.  V runs
+        // one tile behind K, as in the unsplit scheme: published V[t + 1] / K[t + 2], fetched V[t + 2] / K[t + 3],
+        // ids of V[t + 3] / K[t + 4].
+        const int behind = role_v ? 1 : 0;
+        asm volatile("" : "+v"(kreg[0]));
+        if (chunk_live[0]) {
+          const int tk = chunk_tok[0];
+          const int pub = t + 2 - behind;
+          char* dst = role_v ? s_v[pub & 1] + v_row_of(tk) * RSV : s_k[pub & 1] + tk * RSK;
+          if constexpr (T::kQuant) {
+            uint4_t lo, hi;
+            dequant_chunk<KIND>(kreg[0], scale_value(ksreg[0]), lo, hi);
+            *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 32) = lo;
+            *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 32 + 16) = hi;
+          } else {
+            *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 16) = kreg[0];
+          }
+        }
+        ids_k[0] = ids_n[0];
+        const int64_t row = cache_row(t + 3 - behind, 0);
+        kreg[0] = load16(role_v ? p.v_cache : p.k_cache, row * row_bytes + chunk_col[0] * 16);
+        if constexpr (T::kQuant) ksreg[0] = static_cast<const scale_raw_t*>(role_v ? p.v_scale : p.k_scale)[row];
+        load_ids(t + 4 - behind);
+      } else {
+        publish_k(t + 2);
+        publish_v(t + 1);
+        issue_v();  // rows of tile t + 2, remembered when its K chunk was fetched
 #pragma unroll
-      for (int i = 0; i < NLD; ++i) ids_k[i] = ids_n[i];
-      issue_k(t + 3);
-      load_ids(t + 4);
+        for (int i = 0; i < NLD; ++i) ids_k[i] = ids_n[i];
+        issue_k(t + 3);
+        load_ids(t + 4);
+      }
     };
 
     // raw scores of one key tile: S^T = K . Q^T
