@@ -291,9 +291,12 @@ def measure_prefill(w, iters=20):
             softmax_scale=w.softmax_scale, k_scale=w.k_scale, v_scale=w.v_scale,
         )  # fmt: skip
 
-    def timed(fn, inner=1):
-        """Median over `iters` samples of `inner` back-to-back calls (short ops: the queue stays ahead of the GPU)."""
-        for _ in range(3):
+    spread = {}
+
+    def timed(fn, inner=1, warm=3, name=None):
+        """Median over `iters` samples of `inner` back-to-back calls (short ops: the queue stays ahead of the GPU);
+        with a name, the 10th and 90th percentile of the samples are kept in `spread`."""
+        for _ in range(warm):
             fn()
         torch.cuda.synchronize()
         samples = []
@@ -305,6 +308,9 @@ def measure_prefill(w, iters=20):
             e1.record()
             e1.synchronize()
             samples.append(e0.elapsed_time(e1) * 1e3 / inner)
+        if name is not None:
+            ordered = sorted(samples)
+            spread[name] = [ordered[len(ordered) // 10], ordered[(len(ordered) * 9) // 10]]
         return statistics.median(samples)
 
     def timed_graph(fn, inner=20):
@@ -323,7 +329,7 @@ def measure_prefill(w, iters=20):
         return timed(g.replay) / inner
 
     us_write = timed_graph(write)
-    us_attend = timed(attend)
+    us_attend = timed(attend, warm=40, name="prefill")  # ~1 ms launches: an idle part's clocks settle over tens of ms
 
     # the fused step in front of the path at the same shape: QK RMSNorm + rotary + quantizing write of the new rows
     t, hq, d = w.q.shape
@@ -353,6 +359,7 @@ def measure_prefill(w, iters=20):
         "workload": w.name,
         "us_per_step": us_attend + us_write,
         "kernel_us": {"cache_write": us_write, "prefill": us_attend, "qk_norm_rope_cache_write": us_front},
+        "prefill_us_p10_p90": spread["prefill"],
         "qk_norm_rope_cache_write": {
             "us": us_front, "algorithmic_bytes": front_bytes, "gbps": front_bytes / (us_front * 1e-6) / 1e9,
             "frac_of_hbm_peak": front_bytes / (us_front * 1e-6) / 1e9 / HBM_PEAK_GBPS,
