@@ -19,17 +19,23 @@
 //   * the threads fetch K three tiles and V two tiles ahead with 16-byte coalesced loads (block ids one more
 //     tile ahead) and publish them into double-buffered LDS tiles one iteration before their first use, so one
 //     barrier per tile is enough (padded rows, conflict free).  8-bit codes are dequantized (times the per-token
-//     scale) by the thread that stages them, once per workgroup: the tiles in LDS are always 16-bit;
+//     scale) by the thread that stages them, once per workgroup: the tiles in LDS are always 16-bit.  When a tile
+//     has at most one chunk per thread (8-bit tiles, 16-bit tiles at head dim 64) the first four waves stage K and
+//     the last four V, one chunk each;
 //   * S^T[key][row] = K . Q^T of tile t + 1 is issued in the same basic block as the row maxima of tile t, so the
 //     matrix cores have independent work while the vector ALU runs the softmax: A = K rows from LDS, B = Q^T in
 //     registers; C has row = lane % 16, 4 keys per lane;
-//   * causal / window mask only on tiles that cross a mask edge, online softmax in the log2 domain (per lane = per
-//     row; the four lanes of a row combine through v_permlane swaps), the softmax scale folded into the exponent's
-//     multiply-add;
+//   * causal / window mask only on tiles that cross a mask edge, online softmax in the log2 domain with the softmax
+//     scale folded into the exponent's multiply-add.  The value the exponentials are taken against is raised (and
+//     the accumulators rescaled) only when a tile exceeds it by more than 2^8: each lane checks its own scores and a
+//     ballot decides for the wave, so most tiles skip the cross-lane maxima (v_permlane swaps over the four lanes
+//     of a row) and the rescale;
 //   * O^T[dim][row] += V^T . P^T : A = V^T through the LDS transpose reads, B = P^T (= the C layout of S^T); one
 //     more product with an all-ones A operand accumulates the row sums of P.
-// The loop is bound by vector-ALU issue: with two waves per SIMD a plain VALU instruction issues every ~5.7 cycles
-// (4 with more waves), v_exp_f32 every ~9, while the 34 MFMAs of a wave's tile step need 18 cycles each and overlap.
+// The tile loop is unrolled by two with the roles of the two score arrays swapped, so the scores of tile t + 1 are
+// computed where the next step reads them.  Vector-ALU and matrix-core time add up more than they overlap here: with
+// two waves per SIMD a plain VALU instruction issues every ~5.7 cycles (4 with more waves), v_exp_f32 every ~9, the
+// 34 MFMAs of a wave's tile step need 18 cycles each, and a wave's tile step has ~110 VALU instructions.
 // The LDS layouts are the 16-bit ones of the decode kernel (decode_mfma_kernels.hpp).  Semantics:
 // _reference_attention with query_start = context_lens[s] (areno/accel/attention.py:25-41 in the reference); with
 // context 0 it is the reference's varlen kernel (areno/accel/csrc/attention.cu:145-242).
