@@ -134,6 +134,7 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_kernel(Decod
 // (row, q head) gathers the candidates of both kinds: lanes first fetch up to 64 (m, l) pairs in parallel and agree
 // on the maximum, then every lane accumulates its share of the head dimension with the partial loads of a group of
 // four candidates in flight together (the loop has no loop-carried memory dependence).
+template <int EPW>  // head-dimension elements per lane: head_dim <= 64 EPW
 __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel(MfmaDecodeParams mp) {
   const DecodeParams& p = mp.d;
   const int lane = threadIdx.x & (kWave - 1);
@@ -179,9 +180,9 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
     }
   };
 
-  float acc[kGenericMaxPerLane];
+  float acc[EPW];
 #pragma unroll
-  for (int e = 0; e < kGenericMaxPerLane; ++e) acc[e] = 0.0f;
+  for (int e = 0; e < EPW; ++e) acc[e] = 0.0f;
   float m = kNegInf, l = 0.0f;
   for (int base = 0; base < total; base += kWave) {
     // lane j looks at candidate base + j
@@ -205,11 +206,11 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
     l = l * alpha + wave_sum(w * part_l);
     m = m_new;
 #pragma unroll
-    for (int e = 0; e < kGenericMaxPerLane; ++e) acc[e] *= alpha;
+    for (int e = 0; e < EPW; ++e) acc[e] *= alpha;
     const int count = min(kWave, total - base);
     for (int j0 = 0; j0 < count; j0 += 4) {
       float wj[4];
-      float v[4][kGenericMaxPerLane];
+      float v[4][EPW];
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
         const int j = min(j0 + jj, count - 1);
@@ -219,7 +220,7 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
         locate(base + j, ml, part);
         const bool present = wj[jj] != 0.0f;
 #pragma unroll
-        for (int e = 0; e < kGenericMaxPerLane; ++e) {
+        for (int e = 0; e < EPW; ++e) {
           const int idx = lane + e * kWave;
           // partials of units without tiles were never written: read only what carries a non-zero weight
           v[jj][e] = (idx < d && present) ? part[idx] : 0.0f;
@@ -228,15 +229,25 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
 #pragma unroll
-        for (int e = 0; e < kGenericMaxPerLane; ++e) acc[e] += wj[jj] * v[jj][e];
+        for (int e = 0; e < EPW; ++e) acc[e] += wj[jj] * v[jj][e];
       }
     }
   }
 #pragma unroll
-  for (int e = 0; e < kGenericMaxPerLane; ++e) {
+  for (int e = 0; e < EPW; ++e) {
     const int idx = lane + e * kWave;
     if (idx < d) store_from_float(p.out, static_cast<int64_t>(row) * d + idx, p.q_dtype, acc[e] / l);
   }
+}
+
+typedef void (*reduce_slots_fn)(MfmaDecodeParams);
+// the narrowest instantiation that covers the head: the kernel is a few hundred instructions per wave and mostly
+// launch latency, so slots that would only be predicated off are worth leaving out
+reduce_slots_fn reduce_slots_kernel_for(int head_dim) {
+  if (head_dim <= 64) return decode_reduce_slots_kernel<1>;
+  if (head_dim <= 128) return decode_reduce_slots_kernel<2>;
+  if (head_dim <= 256) return decode_reduce_slots_kernel<4>;
+  return decode_reduce_slots_kernel<kGenericMaxPerLane>;
 }
 
 // ---- geometry of the MFMA path ----------------------------------------------------------------------
@@ -541,7 +552,7 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     }
     if (stages & ARENO_STAGE_REDUCE) {
       const int rblocks = (batch * q_heads + kReduceRows - 1) / kReduceRows;
-      hipLaunchKernelGGL(decode_reduce_slots_kernel, dim3(rblocks), dim3(kReduceRows * kWave), 0, s, mp);
+      hipLaunchKernelGGL(reduce_slots_kernel_for(mp.d.head_dim), dim3(rblocks), dim3(kReduceRows * kWave), 0, s, mp);
       if (int rc = check_launch(op)) return rc;
     }
     return ARENO_OK;
