@@ -106,6 +106,20 @@ def test_paged_prefill_head_dims_192_256(kv, d, hq, hkv, window_left):
                  what=f"prefill D={d} {kv}")  # fmt: skip
 
 
+@pytest.mark.parametrize("kv", ["bf16", "fp16", "int8", "fp8"])
+@pytest.mark.parametrize("d,bs", [(64, 16), (64, 64), (128, 8), (128, 128)])
+def test_paged_prefill_staging_schemes(kv, d, bs):
+    """The staging of a key tile has two schemes: one K and one V chunk per thread and round, or, when a tile has at
+    most one chunk per thread (8-bit tiles up to head dim 128, 16-bit tiles at 64), K staged by the first half of
+    the workgroup and V by the second.  8-bit tiles at head dim 64 leave half of each half without a live chunk.
+    Page sizes below, at and above the 32-key tile."""
+    new = torch.tensor([70, 1, 200, 33])
+    ctx = torch.tensor([0, 1300, 95, 640])
+    w = workloads.make_prefill_workload("staging", seed=d + bs, new_lens=new, ctx_lens=ctx, hq=8, hkv=2, d=d, bs=bs,
+                                        kv=kv, device=DEV, quantize_fn=gpu_quantize)  # fmt: skip
+    assert_close(_run_prefill(w), _expected_prefill(w), *tolerances(kv), what=f"prefill staging D={d} {kv} page {bs}")
+
+
 def test_prefill_with_a_full_sequence_list():
     """1024 sequences, the most one launch of the matrix-core kernel indexes: the prefix sum over the sequences must
     also produce its last entry, the total."""
