@@ -298,6 +298,9 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   constexpr int kMaxItems = (GROUPED ? 2 : 1) * kMfmaMaxBatch;  // at most one shared item per row on top of the rows
   __shared__ int s_cum[kMaxItems + 1];
   __shared__ int s_wave_tot[NW];
+  // the sequence lengths, kept from the prefix sum: what a wave needs to know about an item afterwards comes from
+  // here instead of from another memory round trip (without prefix groups; with them item_info stays on global memory)
+  __shared__ int s_len[GROUPED ? 1 : kMaxItems];
   __shared__ int s_pair_flags[2][NW];  // [0]: score parts this wave has published, [1]: steps whose parts it has read
   constexpr int SPT = (kMaxItems + NW * kWave - 1) / (NW * kWave);  // items per thread in the prefix sum
 
@@ -352,7 +355,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       it.row = b;
       return it;
     } else {
-      it.hi = p.cache_seqlens[v] + 1;
+      it.hi = s_len[v] + 1;
       it.lo = first_allowed_key(it.hi, p.window_left);
       it.row = v;
       return it;
@@ -362,15 +365,31 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   {
     int nt[SPT];
     int local = 0;
+    if constexpr (GROUPED) {
 #pragma unroll
-    for (int j = 0; j < SPT; ++j) {
-      const int v = SPT * tid + j;
-      nt[j] = 0;
-      if (v < num_items) {
-        const ItemInfo it = item_info(v);
-        nt[j] = (it.hi - it.lo + TK - 1) / TK;
+      for (int j = 0; j < SPT; ++j) {
+        const int v = SPT * tid + j;
+        nt[j] = 0;
+        if (v < num_items) {
+          const ItemInfo it = item_info(v);
+          nt[j] = (it.hi - it.lo + TK - 1) / TK;
+        }
+        local += nt[j];
       }
-      local += nt[j];
+    } else {
+      // the thread's sequence lengths are fetched together (clamped index, no branch around the load): as loads
+      // under `if (v < num_items)` they went out one at a time, SPT memory round trips at the start of every launch
+      int len[SPT];
+#pragma unroll
+      for (int j = 0; j < SPT; ++j) len[j] = p.cache_seqlens[min(SPT * tid + j, num_items - 1)];
+#pragma unroll
+      for (int j = 0; j < SPT; ++j) {
+        const int v = SPT * tid + j;
+        const int hi = len[j] + 1;
+        nt[j] = v < num_items ? (hi - first_allowed_key(hi, p.window_left) + TK - 1) / TK : 0;
+        if (v < num_items) s_len[v] = len[j];
+        local += nt[j];
+      }
     }
     int incl = local;
 #pragma unroll
