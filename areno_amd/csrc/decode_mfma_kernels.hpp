@@ -298,9 +298,16 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   constexpr int kMaxItems = (GROUPED ? 2 : 1) * kMfmaMaxBatch;  // at most one shared item per row on top of the rows
   __shared__ int s_cum[kMaxItems + 1];
   __shared__ int s_wave_tot[NW];
-  // the sequence lengths, kept from the prefix sum: what a wave needs to know about an item afterwards comes from
-  // here instead of from another memory round trip (without prefix groups; with them item_info stays on global memory)
-  __shared__ int s_len[GROUPED ? 1 : kMaxItems];
+  // The length arrays in LDS: what a wave needs to know about an item comes from here instead of from a memory round
+  // trip per lookup.  Without prefix groups the prefix sum's own loads fill s_len.  With them an item's extent takes up
+  // to six dependent reads (the group's shared length, the members' lengths, the row's own) and the prefix sum asks for
+  // 2 * 1024 / threads items per thread -- from global memory some forty round trips one after the other in the first
+  // wave of every workgroup -- so the workgroup first copies both arrays with independent loads.  Where the copies
+  // would cost the second resident workgroup (prefix groups over 16-bit caches) the lookups stay on global memory.
+  constexpr bool kLocalLens = !GROUPED || ES == 1;
+  constexpr int kMaxGroups = kMfmaMaxBatch / 2;  // groups have at least two rows
+  __shared__ int s_len[kLocalLens ? kMfmaMaxBatch : 1];            // sequence lengths of the rows
+  __shared__ int s_group_len[GROUPED && kLocalLens ? kMaxGroups : 1];  // shared prefix length of each group
   __shared__ int s_pair_flags[2][NW];  // [0]: score parts this wave has published, [1]: steps whose parts it has read
   constexpr int SPT = (kMaxItems + NW * kWave - 1) / (NW * kWave);  // items per thread in the prefix sum
 
@@ -330,13 +337,35 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   const int num_items = GROUPED ? mp.num_shared + p.batch : p.batch;
   // tokens of a sub-group's shared prefix: the caller's figure, clipped to what every member has cached and cut to a
   // whole number of tiles
+  if constexpr (GROUPED && kLocalLens) {
+    // the launcher sends whole groups of at least two rows, at most kMfmaMaxBatch rows
+    const int groups = min(p.batch / max(mp.group_rows, 2), kMaxGroups);
+    for (int i = tid; i < min(p.batch, kMfmaMaxBatch); i += NW * kWave) s_len[i] = p.cache_seqlens[i];
+    for (int i = tid; i < groups; i += NW * kWave) s_group_len[i] = mp.shared_lens[i];
+    __syncthreads();
+  }
+  // length of row b / shared prefix length of group gi (indices clamped into the LDS copies)
+  auto row_len = [&](int b) {
+    if constexpr (GROUPED && kLocalLens) {
+      return s_len[min(max(b, 0), kMfmaMaxBatch - 1)];
+    } else {
+      return p.cache_seqlens[b];
+    }
+  };
+  auto group_len = [&](int gi) {
+    if constexpr (GROUPED && kLocalLens) {
+      return s_group_len[min(max(gi, 0), kMaxGroups - 1)];
+    } else {
+      return mp.shared_lens[gi];
+    }
+  };
   auto shared_tokens = [&](int sub, int& row0, int& count) {
     const int gi = sub / mp.subs_per_group;
     const int j = sub - gi * mp.subs_per_group;
     row0 = gi * mp.group_rows + j * mp.cols_seqs;
     count = min(mp.cols_seqs, mp.group_rows - j * mp.cols_seqs);
-    int len = mp.shared_lens[gi];
-    for (int m = 0; m < count; ++m) len = min(len, p.cache_seqlens[row0 + m]);
+    int len = group_len(gi);
+    for (int m = 0; m < count; ++m) len = min(len, row_len(row0 + m));
     return max(len, 0) & ~(TK - 1);
   };
   auto item_info = [&](int v) {
@@ -351,7 +380,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       const int gi = b / mp.group_rows;
       int row0, count;
       it.lo = shared_tokens(gi * mp.subs_per_group + (b - gi * mp.group_rows) / mp.cols_seqs, row0, count);
-      it.hi = p.cache_seqlens[b] + 1;
+      it.hi = row_len(b) + 1;
       it.row = b;
       return it;
     } else {
