@@ -144,12 +144,13 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   const int h = row - b * p.q_heads;
   const int d = p.head_dim;
   const int num_items = mp.num_shared + p.batch;
-  const UnitGeometry geo =
-      make_unit_geometry(mp.plan[num_items], mp.num_pieces, mp.max_small, mp.static_share, mp.min_unit_tiles);
-  // the row's own item (always at least one tile) ...
+  // the plan entries this row needs, fetched together (their indices follow from the row alone)
   const int v_own = mp.num_shared + b;
-  const int own_lo = geo.unit_of(mp.plan[v_own]);
-  const int own_n = geo.unit_of(mp.plan[v_own + 1] - 1) - own_lo + 1;
+  const int plan_total = mp.plan[num_items], plan_own = mp.plan[v_own], plan_own_end = mp.plan[v_own + 1];
+  const UnitGeometry geo = make_unit_geometry(plan_total, mp.num_pieces, mp.max_small, mp.static_share, mp.min_unit_tiles);
+  // the row's own item (always at least one tile) ...
+  const int own_lo = geo.unit_of(plan_own);
+  const int own_n = geo.unit_of(plan_own_end - 1) - own_lo + 1;
   // ... and the shared item of its sub-group, if it has tiles
   int sh_lo = 0, sh_n = 0, sh_item = 0, sh_col = 0;
   if (mp.num_shared > 0) {
