@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0
 POOL_TARGET_BYTES = 1.3e9  # rotate over at least this much distinct KV
 # HBM bytes per launch of the split kernel from two rocprofv3 counter runs of this script (FETCH_SIZE, scaled by the
 # factor 2.0 that a copy of known size gives for it, plus WRITE_SIZE); the counter summary is kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 315.82e6, "cfg2-qwen7b-int8": 158.68e6, "cfg3-rollout-fp8": 1070.41e6,
+MEASURED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 315.82e6, "cfg2-qwen7b-int8": 158.68e6, "cfg3-rollout-fp8": 1071.17e6,
                           "cfg4-prefill-fp8": 1623.08e6}
 
 
