@@ -65,4 +65,65 @@ __device__ __forceinline__ void quantize_store_row(const float (&x)[kMaxPerLane]
   }
 }
 
+// The same closed forms for a row held by a group of LPR adjacent lanes, 8 consecutive elements per lane (lane `sub`
+// of the group holds elements 8 sub .. 8 sub + 7; head_dim = 8 LPR): 16-byte accesses instead of one element per
+// lane.  `amax` is the row's abs-max, already combined over the group.  16-bit caches get the values rounded to the
+// cache dtype.
+__device__ __forceinline__ uint32_t pack_two_16(float lo, float hi, int dtype) {
+  return dtype == ARENO_DT_BF16 ? (float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16))
+                                : (float_to_f16_bits(lo) | (float_to_f16_bits(hi) << 16));
+}
+
+template <int LPR>
+__device__ __forceinline__ float lane_group_max(float x) {
+#pragma unroll
+  for (int m = 1; m < LPR; m <<= 1) x = fmaxf(x, wave_xor(x, m));
+  return x;
+}
+
+__device__ __forceinline__ void store_row_slice(const float (&x)[8], float amax, int sub, int64_t dst_row, int d,
+                                                void* cache, void* scale, int cache_dtype, int scale_dtype) {
+  const int64_t dst_elem = dst_row * d + sub * 8;
+  if (cache_dtype == ARENO_DT_I8) {
+    const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
+    const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
+    const float s = static_cast<float>(s16_fixed);
+    uint32_t words[2] = {0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float code = fminf(fmaxf(rintf(x[j] / s), -127.0f), 127.0f);
+      words[j / 4] |= (static_cast<uint32_t>(static_cast<int>(code)) & 0xffu) << (8 * (j & 3));
+    }
+    *reinterpret_cast<uint2_t*>(static_cast<char*>(cache) + dst_elem) = uint2_t{words[0], words[1]};
+    if (sub == 0) {
+      if (scale_dtype == ARENO_DT_F16) {
+        static_cast<uint16_t*>(scale)[dst_row] = __builtin_bit_cast(uint16_t, s16_fixed);
+      } else {
+        static_cast<float*>(scale)[dst_row] = s;
+      }
+    }
+  } else if (cache_dtype == ARENO_DT_FP8_E4M3) {
+    float s = amax / 448.0f;
+    if (s == 0.0f) s = 1.0f;
+    uint32_t words[2] = {0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float y = fminf(fmaxf(x[j] / s, -448.0f), 448.0f);
+      words[j / 4] |= float_to_fp8_byte(y) << (8 * (j & 3));
+    }
+    *reinterpret_cast<uint2_t*>(static_cast<char*>(cache) + dst_elem) = uint2_t{words[0], words[1]};
+    if (sub == 0) {
+      if (scale_dtype == ARENO_DT_F16) {
+        static_cast<uint16_t*>(scale)[dst_row] = static_cast<uint16_t>(float_to_f16_bits(s));
+      } else {
+        static_cast<float*>(scale)[dst_row] = s;
+      }
+    }
+  } else {
+    const uint4_t packed = {pack_two_16(x[0], x[1], cache_dtype), pack_two_16(x[2], x[3], cache_dtype),
+                            pack_two_16(x[4], x[5], cache_dtype), pack_two_16(x[6], x[7], cache_dtype)};
+    *reinterpret_cast<uint4_t*>(static_cast<char*>(cache) + dst_elem * 2) = packed;
+  }
+}
+
 }  // namespace areno

@@ -92,6 +92,77 @@ __global__ __launch_bounds__(kRowsPerBlock* kWave) void cache_write_kernel(Write
   }
 }
 
+// The common shapes (16-bit rows, head_dim = 8 LPR with LPR a power of two up to 64): a row is held by LPR adjacent
+// lanes with 8 consecutive elements each, so a wave moves 64 / LPR rows with 16-byte loads and 8- or 16-byte stores
+// instead of one row with one element per lane.  Same closed forms, same bits (store_row_slice).
+template <int LPR>
+__global__ __launch_bounds__(kRowsPerBlock* kWave) void cache_write_rows_kernel(WriteParams p) {
+  constexpr int D = LPR * 8;
+  constexpr int kRowsPerWave = kWave / LPR;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int sub = lane % LPR;
+  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + (threadIdx.x >> 6);
+  const int64_t total = p.tokens * p.kv_heads;
+  const int64_t row_raw = wave_id * kRowsPerWave + lane / LPR;
+  const bool live = row_raw < total;
+  const int64_t row = live ? row_raw : total - 1;  // idle lane groups shadow the last row and store nothing
+  const int which = blockIdx.y;                    // 0 = K, 1 = V
+  const int64_t token = row / p.kv_heads;
+  const int head = static_cast<int>(row - token * p.kv_heads);
+
+  const uint4_t raw = *reinterpret_cast<const uint4_t*>(static_cast<const char*>(p.src[which]) + (row * D + sub * 8) * 2);
+  int64_t blk, slot;
+  bool ok = live;
+  if (p.block_ids != nullptr) {
+    blk = p.block_ids[token];
+    slot = p.block_offsets[token];
+  } else {
+    const int64_t pos = p.cache_seqlens[token];
+    const int64_t col = pos / p.block_size;
+    ok = ok && pos >= 0 && col < p.max_blocks;
+    slot = pos - col * p.block_size;
+    blk = ok ? p.block_table[token * p.max_blocks + col] : 0;
+  }
+  ok = ok && blk >= 0 && blk < p.num_blocks && slot >= 0 && slot < p.block_size;
+
+  float x[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t word = raw[j];
+    if (p.in_dtype == ARENO_DT_BF16) {
+      x[2 * j] = bf16_bits_to_float(word & 0xffffu);
+      x[2 * j + 1] = bf16_bits_to_float(word >> 16);
+    } else {
+      x[2 * j] = f16_bits_to_float(word & 0xffffu);
+      x[2 * j + 1] = f16_bits_to_float(word >> 16);
+    }
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(x[j]));
+  amax = lane_group_max<LPR>(amax);  // every lane of the wave takes part
+  if (!ok) return;
+  const int64_t dst_row = (blk * p.block_size + slot) * p.kv_heads + head;
+  if (is_quantized_dtype(p.cache_dtype)) {
+    store_row_slice(x, amax, sub, dst_row, D, p.cache[which], p.scale[which], p.cache_dtype, p.scale_dtype);
+  } else {
+    // same-dtype copy: the raw bits, so the stored row is bit-identical to the input row
+    *reinterpret_cast<uint4_t*>(static_cast<char*>(p.cache[which]) + (dst_row * D + sub * 8) * 2) = raw;
+  }
+}
+
+typedef void (*write_rows_fn)(WriteParams);
+write_rows_fn write_rows_kernel_for(int head_dim, int in_dtype) {
+  if (in_dtype != ARENO_DT_F16 && in_dtype != ARENO_DT_BF16) return nullptr;
+  switch (head_dim) {
+    case 64: return cache_write_rows_kernel<8>;
+    case 128: return cache_write_rows_kernel<16>;
+    case 256: return cache_write_rows_kernel<32>;
+    case 512: return cache_write_rows_kernel<64>;
+    default: return nullptr;
+  }
+}
+
 int validate_cache(const areno_paged_cache* c, const char* op) {
   if (c == nullptr) return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: cache descriptor is NULL", op);
   if (c->k == nullptr || c->v == nullptr) return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: cache pool pointer is NULL", op);
@@ -146,6 +217,18 @@ int launch_write(const areno_paged_cache* cache, const void* k, const void* v, i
   p.in_dtype = in_dtype;
   p.cache_dtype = cache->cache_dtype;
   p.scale_dtype = cache->scale_dtype;
+  // 16-byte row slices need 16-byte aligned tensors (rows are multiples of 128 bytes there)
+  const bool aligned = (reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                        reinterpret_cast<uintptr_t>(cache->k) | reinterpret_cast<uintptr_t>(cache->v)) % 16 == 0;
+  const write_rows_fn rows_kernel = aligned ? write_rows_kernel_for(cache->head_dim, in_dtype) : nullptr;
+  if (rows_kernel != nullptr) {
+    const int rows_per_wave = kWave / (cache->head_dim / 8);
+    const int64_t waves = (rows + rows_per_wave - 1) / rows_per_wave;
+    const int64_t wgs = (waves + kRowsPerBlock - 1) / kRowsPerBlock;
+    hipLaunchKernelGGL(rows_kernel, dim3(static_cast<unsigned>(wgs), 2), dim3(kRowsPerBlock * kWave), 0,
+                       static_cast<hipStream_t>(stream), p);
+    return check_launch(op);
+  }
   hipLaunchKernelGGL(cache_write_kernel, dim3(static_cast<unsigned>(blocks), 2), dim3(kRowsPerBlock * kWave), 0,
                      static_cast<hipStream_t>(stream), p);
   return check_launch(op);

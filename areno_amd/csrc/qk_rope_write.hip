@@ -190,47 +190,7 @@ __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
     const int64_t off = p.block_offsets[token[r]];
     if (blk < 0 || blk >= p.num_blocks || off < 0 || off >= p.block_size) continue;
     const int64_t dst_row = (blk * p.block_size + off) * p.kv_heads + head[r];
-    const int64_t dst_elem = dst_row * D + sub * 8;
-    if (p.cache_dtype == ARENO_DT_I8) {
-      const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
-      const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
-      const float s = static_cast<float>(s16_fixed);
-      uint32_t words[2] = {0u, 0u};
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float code = fminf(fmaxf(rintf(x[j] / s), -127.0f), 127.0f);
-        words[j / 4] |= (static_cast<uint32_t>(static_cast<int>(code)) & 0xffu) << (8 * (j & 3));
-      }
-      *reinterpret_cast<uint2_t*>(static_cast<char*>(cache) + dst_elem) = uint2_t{words[0], words[1]};
-      if (sub == 0) {
-        if (p.scale_dtype == ARENO_DT_F16) {
-          static_cast<uint16_t*>(p.scale[kind[r] - 1])[dst_row] = __builtin_bit_cast(uint16_t, s16_fixed);
-        } else {
-          static_cast<float*>(p.scale[kind[r] - 1])[dst_row] = s;
-        }
-      }
-    } else if (p.cache_dtype == ARENO_DT_FP8_E4M3) {
-      float s = amax / 448.0f;
-      if (s == 0.0f) s = 1.0f;
-      uint32_t words[2] = {0u, 0u};
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float y = fminf(fmaxf(x[j] / s, -448.0f), 448.0f);
-        words[j / 4] |= float_to_fp8_byte(y) << (8 * (j & 3));
-      }
-      *reinterpret_cast<uint2_t*>(static_cast<char*>(cache) + dst_elem) = uint2_t{words[0], words[1]};
-      if (sub == 0) {
-        if (p.scale_dtype == ARENO_DT_F16) {
-          static_cast<uint16_t*>(p.scale[kind[r] - 1])[dst_row] = static_cast<uint16_t>(float_to_f16_bits(s));
-        } else {
-          static_cast<float*>(p.scale[kind[r] - 1])[dst_row] = s;
-        }
-      }
-    } else {
-      const uint4_t packed = {pack_two(x[0], x[1], p.cache_dtype), pack_two(x[2], x[3], p.cache_dtype),
-                              pack_two(x[4], x[5], p.cache_dtype), pack_two(x[6], x[7], p.cache_dtype)};
-      *reinterpret_cast<uint4_t*>(static_cast<char*>(cache) + dst_elem * 2) = packed;
-    }
+    store_row_slice(x, amax, sub, dst_row, D, cache, p.scale[kind[r] - 1], p.cache_dtype, p.scale_dtype);
   }
 }
 

@@ -30,7 +30,7 @@ def _addresses(t, nb, bs, seed=1):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("d", [64, 128, 80])
+@pytest.mark.parametrize("d", [64, 128, 80, 256, 512, 192])
 def test_unquantized_scatter_is_a_bit_exact_copy(dtype, d):
     t, hkv, nb, bs = 37, 4, 9, 16
     k, v = _inputs(t, hkv, d, dtype)
@@ -47,8 +47,10 @@ def test_unquantized_scatter_is_a_bit_exact_copy(dtype, d):
 
 @pytest.mark.parametrize("cache_dtype,scale_dtype", [(torch.int8, torch.float16), (torch.float8_e4m3fn, torch.float32)])
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("d", [128, 64, 256, 512, 96])
 def test_quantize_and_scatter_bit_exact(cache_dtype, scale_dtype, in_dtype, d):
+    # 16-bit rows of 64 / 128 / 256 / 512 elements take the writer's lane-group kernel (several rows per wave, 300 x 4
+    # rows do not fill the last wave), everything else the one-row-per-wave kernel; both must give the same bits
     t, hkv, nb, bs = 300, 4, 40, 16
     k, v = _inputs(t, hkv, d, in_dtype, seed=3)
     ids, offs = _addresses(t, nb, bs, seed=4)
