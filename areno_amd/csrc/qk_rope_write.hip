@@ -58,11 +58,6 @@ __device__ __forceinline__ float round_to(float x, int dtype) {
   return dtype == ARENO_DT_BF16 ? bf16_bits_to_float(float_to_bf16_bits(x)) : f16_bits_to_float(float_to_f16_bits(x));
 }
 
-__device__ __forceinline__ uint32_t pack_two(float lo, float hi, int dtype) {
-  return dtype == ARENO_DT_BF16 ? (float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16))
-                                : (float_to_f16_bits(lo) | (float_to_f16_bits(hi) << 16));
-}
-
 // Row layout: a row of D elements is held by LPR = D / 8 adjacent lanes, 8 consecutive elements (16 bytes of 16-bit
 // activations) per lane, so a wave64 carries 64 / LPR rows and every global access is a 16-byte one.  The rotary
 // partner of element i (i +- D/2) is the same element slot of lane ^ (LPR / 2).
@@ -70,12 +65,6 @@ template <int LPR>
 __device__ __forceinline__ float group_sum(float x) {
 #pragma unroll
   for (int m = 1; m < LPR; m <<= 1) x += wave_xor(x, m);
-  return x;
-}
-template <int LPR>
-__device__ __forceinline__ float group_max(float x) {
-#pragma unroll
-  for (int m = 1; m < LPR; m <<= 1) x = fmaxf(x, wave_xor(x, m));
   return x;
 }
 
@@ -172,8 +161,8 @@ __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
       }
       void* out = kind[r] == 0 ? p.q_out : p.k_out;
       if (out != nullptr && live[r]) {
-        const uint4_t packed = {pack_two(x[0], x[1], p.dtype), pack_two(x[2], x[3], p.dtype),
-                                pack_two(x[4], x[5], p.dtype), pack_two(x[6], x[7], p.dtype)};
+        const uint4_t packed = {pack_two_16(x[0], x[1], p.dtype), pack_two_16(x[2], x[3], p.dtype),
+                                pack_two_16(x[4], x[5], p.dtype), pack_two_16(x[6], x[7], p.dtype)};
         *reinterpret_cast<uint4_t*>(static_cast<char*>(out) + src_base[r] * 2) = packed;
       }
     }
@@ -182,7 +171,7 @@ __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
     float amax = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(x[j]));
-    amax = group_max<LPR>(amax);
+    amax = lane_group_max<LPR>(amax);
     if (kind[r] == 0 || !live[r]) continue;
     void* cache = p.cache[kind[r] - 1];
     if (cache == nullptr) continue;
