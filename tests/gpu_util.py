@@ -66,3 +66,28 @@ def assert_close(got: torch.Tensor, want: torch.Tensor, max_abs: float, mean_abs
 
 def tolerances(kv: str):
     return (QUANT_MAX_ABS, None) if kv in ("int8", "fp8") else (BF16_MAX_ABS, BF16_MEAN_ABS)
+
+
+def compact_pages(cache, scale, table_rows: torch.Tensor):
+    """The pages that ``table_rows`` (CPU int tensor, any shape) names, dequantized on the CPU, and the same table with the ids
+    renumbered into that compact pool: the oracle then works on a pool of a few hundred MB instead of the whole cache."""
+    ids, inverse = torch.unique(table_rows.long().flatten(), return_inverse=True)
+    pages = cache[ids.to(cache.device)].cpu()
+    sc = None if scale is None else scale[ids.to(scale.device)].cpu()
+    dense = pages.float() if sc is None else qr.dequantize(pages, sc)
+    return dense, inverse.view(table_rows.shape).to(torch.int32)
+
+
+def expected_decode_rows(w: workloads.DecodeWorkload, rows, *, window_left=None):
+    """Oracle on the post-step cache for the rows in ``rows`` (a list of row indices), touching only the pages those rows read."""
+    rows = torch.as_tensor(rows, dtype=torch.long)
+    bs = w.k_cache.shape[1]
+    lens = w.cache_seqlens.cpu()[rows]
+    table = w.block_table.cpu()[rows]
+    # columns past a row's last page repeat a valid id (padding): the compact pool keeps them, the oracle never reads them
+    cols = int((int(lens.max()) + bs) // bs)
+    table = table[:, :cols]
+    kc, compact = compact_pages(w.k_cache, w.k_scale, table)
+    vc, _ = compact_pages(w.v_cache, w.v_scale, table)
+    return ar.ref_paged_decode(w.q[rows.to(w.q.device)].cpu().float(), kc, vc, compact, lens,
+                               ar.window_left_arg(window_left), w.softmax_scale)  # fmt: skip

@@ -11,7 +11,8 @@ import torch
 from areno_amd import workloads
 from areno_amd.accel import attention as ops
 from oracle import quant_ref as qr
-from tests.gpu_util import DEV, assert_close, expected_decode, gpu_quantize, run_decode, tolerances
+from tests.gpu_util import (DEV, assert_close, expected_decode, expected_decode_rows, gpu_quantize, run_decode,
+                            tolerances)
 
 pytestmark = pytest.mark.gpu
 
@@ -214,6 +215,38 @@ def test_prefix_groups_match_the_plain_op_and_the_oracle(kv, hq, hkv, samples):
         if a is not None:
             same = a.view(torch.uint8) == b.view(torch.uint8)
             assert bool(same.all()), f"{name}: the append differs between the grouped and the plain op"
+
+
+def test_cfg3_full_size_grouped():
+    """The rollout configuration at its stated size, through the prefix-group kernel the benchmark times: 32 prompts x 8
+    samples, 32 / 8 heads, fp8 pages with fp32 scales, prefixes U[256, 2048], continuations lognormal capped at 32 768
+    (block tables ~2 100 columns wide).  The append is checked bit for bit over the whole pool; the output against the
+    oracle on one whole group, the eight longest rows, the shortest row and the last row, and against the plain op
+    (every row reading its own pages) on all 256 rows."""
+    w = workloads.cfg3_rollout("fp8", device=DEV, quantize_fn=gpu_quantize)
+    assert w.q.shape == (256, 32, 128) and w.meta["prefix_group_rows"] == 8
+    pools = (w.k_cache, w.v_cache, w.k_scale, w.v_scale)
+    on_device = tuple(t.clone() for t in pools)
+    before = _snapshot(w)
+    grouped = _grouped_decode(w)
+    torch.cuda.synchronize()
+    _check_append(w, before)
+    del before
+    lens = w.cache_seqlens.cpu()
+    order = torch.argsort(lens, descending=True)
+    longest_group = int(order[0]) // 8
+    rows = sorted(set(range(8 * longest_group, 8 * longest_group + 8)) | set(order[:8].tolist()) | {int(order[-1]), 255})
+    print(f"cfg3 full: longest row {int(lens.max())} tokens, table {tuple(w.block_table.shape)}, oracle rows {rows}")
+    want = expected_decode_rows(w, rows)
+    mx, mean = assert_close(grouped[rows], want, *tolerances("fp8"), what="cfg3 full size, grouped kernel vs oracle")
+    print(f"cfg3 full grouped: max-abs {mx:.3e} mean-abs {mean:.3e} on {len(rows)} rows")
+    after_grouped = tuple(t.clone() for t in pools)
+    for dst, src in zip(pools, on_device):
+        dst.copy_(src)
+    plain = run_decode(w)
+    assert_close(grouped, plain.cpu().float(), 2e-3, what="cfg3 full size, grouped vs plain op, all rows")
+    for a, b, name in zip(pools, after_grouped, ("k", "v", "k_scale", "v_scale")):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"{name}: grouped and plain appends differ"
 
 
 def test_batches_beyond_one_launch_run_in_row_ranges():

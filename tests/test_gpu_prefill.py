@@ -7,7 +7,7 @@ import torch
 from areno_amd import workloads
 from areno_amd.accel import attention as ops
 from oracle import attention_ref as ar
-from tests.gpu_util import DEV, assert_close, dequant_cpu, gpu_quantize, tolerances
+from tests.gpu_util import DEV, assert_close, compact_pages, dequant_cpu, gpu_quantize, tolerances
 
 pytestmark = pytest.mark.gpu
 
@@ -152,6 +152,45 @@ def test_cfg4_reduced():
     """cfg 4 shape (32/8 heads, D=128, fp8) with the full range of new lengths and a reduced context range."""
     w = workloads.cfg4_prefill("fp8", device=DEV, seqs=6, new_hi=512, ctx_hi=3000, quantize_fn=gpu_quantize)
     assert_close(_run_prefill(w), _expected_prefill(w), *tolerances("fp8"), what="cfg4 reduced")
+
+
+def test_cfg4_full_size():
+    """cfg 4 at its stated size: 16 sequences, 1..512 new tokens on 0..16 384 cached ones, 32 / 8 heads, fp8 pages.  The new
+    tokens go through the quantizing cache write first, as in the op sequence the benchmark times.  Every sequence is checked
+    against the oracle on its first and last query row and 16 random ones in between (a row sees all of its sequence's keys
+    up to its own position, so the long contexts are covered by every sampled row)."""
+    w = workloads.cfg4_prefill("fp8", device=DEV, quantize_fn=gpu_quantize)
+    assert w.context_lens.shape == (16,)
+    ops.areno_paged_cache_write(w.k_new, w.v_new, w.k_cache, w.v_cache, w.cache_block_ids, w.cache_block_offsets,
+                                k_scale=w.k_scale, v_scale=w.v_scale)  # fmt: skip
+    out = _run_prefill(w)
+    torch.cuda.synchronize()
+    got = out.cpu().float()
+    assert torch.isfinite(got).all()
+    cu = w.cu_seqlens_q.cpu().tolist()
+    ctx = w.context_lens.cpu().tolist()
+    print(f"cfg4 full: new {[cu[i + 1] - cu[i] for i in range(16)]} ctx {ctx}")
+    g = torch.Generator().manual_seed(4)
+    hq, hkv = w.q.shape[1], w.k_cache.shape[2]
+    worst = 0.0
+    for s in range(16):
+        n = cu[s + 1] - cu[s]
+        picks = sorted({0, n - 1} | set(torch.randint(0, n, (16,), generator=g).tolist()))
+        bs = w.k_cache.shape[1]
+        cols = (ctx[s] + n + bs - 1) // bs
+        table = w.block_table[s : s + 1, :cols].cpu()
+        kc, compact = compact_pages(w.k_cache, w.k_scale, table)
+        vc, _ = compact_pages(w.v_cache, w.v_scale, table)
+        k = ar.gather_paged(kc, compact[0], ctx[s] + n).repeat_interleave(hq // hkv, dim=1).transpose(0, 1).unsqueeze(0)
+        v = ar.gather_paged(vc, compact[0], ctx[s] + n).repeat_interleave(hq // hkv, dim=1).transpose(0, 1).unsqueeze(0)
+        for i in picks:
+            upto = ctx[s] + i + 1
+            q1 = w.q[cu[s] + i].cpu().float().view(1, hq, 1, -1)
+            want = ar.ref_attention(q1, k[:, :, :upto], v[:, :, :upto], ctx[s] + i, -1, w.softmax_scale).view(hq, -1)
+            err = (got[cu[s] + i] - want).abs().max().item()
+            worst = max(worst, err)
+            assert err <= tolerances("fp8")[0], f"cfg4 full: sequence {s} (ctx {ctx[s]}, new {n}) row {i}: max-abs {err:.4g}"
+    print(f"cfg4 full: max-abs {worst:.3e} over the sampled rows")
 
 
 @pytest.mark.parametrize("kv", ["bf16", "int8"])
