@@ -7,33 +7,43 @@
 // form the (zero padded) 16-wide N side of v_mfma_f32_16x16x32 tiles; the vector ALU only dequantizes
 // (<= 0.75 op per element) and runs the softmax.
 //
-// Work decomposition (exactly balanced, no host knowledge of the lengths):
+// Work decomposition (decode_items.hpp; exactly balanced, no host knowledge of the lengths):
 //   * a sequence contributes ceil(visible_keys / 32) tiles of 32 tokens; every workgroup computes the
 //     prefix sum of tile counts over the batch in LDS and takes an equal share of the global tile range
-//     ("wave piece"), so all waves stream the same number of bytes whatever the length distribution;
-//   * a piece that crosses a sequence boundary emits one partial per sequence it touches, into slot
-//     (piece index + sequence index), which is unique and contiguous per sequence; the reduce kernel merges
-//     the slots of each sequence.
+//     (a "unit" per wave), so all waves stream the same number of bytes whatever the length distribution;
+//   * a unit that crosses a sequence boundary emits one partial per sequence it touches, into slot
+//     (unit index + sequence index), which is unique and contiguous per sequence; the reduce kernel merges
+//     the slots of each sequence;
 //   * block = 4 wave64; wave w owns KV head z*HW + w % HW, so with kv_heads >= 4 the four waves of a
 //     workgroup read whole pages ([slot][kv_head][D] is contiguous).  Waves never synchronise after the
-//     prefix sum: each has private LDS tiles.
-// Data path per 32-token tile and wave:
-//   global --16 B/lane coalesced loads--> registers (in flight while the previous tile is computed)
-//          --ds_write_b128--> LDS K tile [32][D*es + 16] and V tile (row padding makes every access below
-//          bank-conflict free)
-//   S^T[token][head] = K . Q^T : A = K rows read straight from LDS (8 consecutive dims per lane), B = Q^T held in
-//          registers for the whole sequence; C puts head = lane % 16, 4 tokens per lane.
-//   online softmax in the log2 domain on C; the per-token K scale multiplies S, the V scale multiplies P.
-//   O^T[dim][head] += V^T . P^T : A = V^T through ds_read_b64_tr_b8 / _tr_b16 (the LDS transpose read gives each
-//          lane 8 tokens of one dim), B = P^T which *is* the C layout of S^T (token order chosen to match), so
-//          no cross-lane movement of P is needed.
+//     prefix sum.
+// Data path per 32-token tile and wave (lane = (lr, lk) = (lane % 16, lane / 16); token group tg = 0, 1):
+//   K  global --16 B/lane--> registers --> MFMA A operand, no LDS: lane (lr, lk) fetches from token 16 tg + lr the
+//      16-byte chunks lk, lk + 4, ... of the head's row, i.e. 64 contiguous bytes per token and load instruction.
+//      The k index of the products is whatever dims those chunks hold; Q^T (B operand, in registers for the whole
+//      sequence) is loaded in the same order, so S^T[token][head] = K . Q^T needs no shuffle.
+//   V  global --same lane / chunk assignment--> registers --ds_write_b128--> LDS, chunk-major
+//      ([token group][chunk][16 tokens][16 B]; 256 contiguous bytes per 16 lanes) --ds_read_b64_tr_b8 / _tr_b16-->
+//      A operand V^T (the LDS transpose read gives each lane 8 tokens of one dim).  So that the 32 lanes of one pass of
+//      the transpose read cover all 64 banks once, the second token group starts 128 bytes off a multiple of 256 and,
+//      for 16-bit elements (one read touches an even and an odd chunk), an odd chunk keeps its token rows 8..15 in
+//      front of rows 0..7.
+//   online softmax in the log2 domain on the C layout of S^T (head = lane % 16, 4 tokens per lane and group); the
+//      per-token K scale multiplies S, the V scale multiplies P (scales travel through 64 floats of LDS per tile).
+//   O^T[dim][head] += V^T . P^T, where P^T *is* the C layout of S^T, so no cross-lane movement of P is needed.
+// 8-bit caches keep two tiles in flight per wave (two register sets, the loop is unrolled over them): a tile is half
+// the bytes of a 16-bit one and it is the bytes in flight that cover the memory latency.  Within a step the V
+// registers are free once the tile is staged and the K registers once the scores are issued, so the loads of the
+// tile two steps ahead go out early in the step.
 // int8 codes become fp16 by placing (code ^ 0x80) under the exponent byte 0x64 (v_perm): 1152 + code exactly;
 // the offsets are removed algebraically (1152 * sum(q) per head, 1152 * sum(p) per head).  fp8 uses
 // v_cvt_scalef32_pk_f16_fp8 with scale 1 (exact).  bf16 / fp16 caches feed the MFMA directly.
 //
-// The single-token append (areno/accel/csrc/attention.cu:526-553) rides along: the wave that stages the last tile of a
-// sequence takes the newest token's row from k_update / v_update instead of the not yet written page slot, quantizes
-// it with the cache writer's closed form and stores it into the page.
+// The single-token append (areno/accel/csrc/attention.cu:526-553) rides along as a tile of its own at the end of
+// each row's item: the wave that owns it reads the row of k_update / v_update (8 bytes per lane), quantizes it with
+// the cache writer's closed form, stores codes and scales into the page and folds the token into its running
+// softmax on the vector ALU (one token is not worth a matrix product).  The cached tokens in front of it never touch
+// the unwritten slot.
 //
 // GROUPED instantiation (batches whose rows come in prefix groups, e.g. the samples of one prompt): the item list is
 // [shared prefix of every sub-group of rows that fits side by side in the 16 MFMA columns] + [the rest of every
@@ -46,15 +56,14 @@
 
 #include <type_traits>
 
+#include "decode_items.hpp"
 #include "paged_decode_kernels.hpp"
 
 namespace areno {
 
-constexpr int kMfmaMaxBatch = 1024;  // prefix-sum capacity of one workgroup
 #ifndef ARENO_MFMA_NW
 #define ARENO_MFMA_NW 4
 #endif
-constexpr int kTileTokens = 32;
 
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -63,33 +72,20 @@ typedef __attribute__((ext_vector_type(2))) int int2_t;
 
 struct MfmaDecodeParams {
   DecodeParams d;      // part_ml / part_acc are indexed [slot][q_head] here
-  int32_t* plan;         // [batch + 1]: exclusive prefix sums of tiles per sequence (written by workgroup 0)
-  int32_t tok_splits;    // waves of a workgroup that share a KV head (waves per workgroup / heads_per_wg)
-  int32_t static_wgs;    // workgroups [0, static_wgs) own the big units, the rest of the grid the small ones
-  int32_t num_pieces;    // static_wgs * tok_splits: big units
-  int32_t max_small;     // (gridDim.x - static_wgs) * tok_splits: small units available
-  int32_t static_share;  // n/256 of all tiles go to the big units
-  int32_t min_unit_tiles;
-  // Fused append: when set, the wave that stages the last tile of a sequence takes the newest token's K / V row
-  // from here ([batch, kv_heads, head_dim], dtype q_dtype) instead of the cache, quantizes it like the cache
-  // writer and stores it (and its scales) into the page, so no separate append launch is needed.
+  int32_t* plan;       // [items + 1]: exclusive prefix sums of tiles per item (written by workgroup 0)
+  int32_t tok_splits;  // waves of a workgroup that share a KV head (waves per workgroup / heads_per_wg / head split)
+  int32_t num_units;   // gridDim.x * tok_splits
+  ItemShape items;     // rows -> items (prefix groups, window, whether the append rides along)
+  // Fused append: per-row items end in a tile for the newest token, whose K / V row comes from here
+  // ([batch, kv_heads, head_dim], dtype q_dtype), is quantized like the cache writer does and stored into the page.
   const void* k_update;
   const void* v_update;
   // Prefix groups (GROUPED kernels only): rows [i * group_rows, (i + 1) * group_rows) share the pages of their first
-  // shared_lens[i] tokens (an RL rollout's samples of one prompt).  Those tokens become "shared items" that are read
-  // once for up to cols_seqs = 16 / q-heads-per-kv-head sequences side by side in the 16 MFMA columns; the rest of
-  // each sequence is an item of its own.  Shared items leave their partials in a second region (16 columns per kv
-  // head and slot).
+  // shared_lens[i] tokens.  Shared items leave their partials in a second region (16 columns per kv head and slot).
   const int32_t* shared_lens;  // [batch / group_rows]
-  int32_t group_rows;          // rows per prefix group
-  int32_t cols_seqs;           // sequences that fit side by side: 16 / group
-  int32_t subs_per_group;      // ceil(group_rows / cols_seqs)
-  int32_t num_shared;          // shared items: (batch / group_rows) * subs_per_group, listed before the per-row items
   float* shared_ml;            // [slot][kv_head][16][2]
   float* shared_acc;           // [slot][kv_head][16][head_dim]
-#ifdef ARENO_TRACE
-  unsigned long long* trace;  // [wave][16] timestamps, tuning builds only
-#endif
+  unsigned long long* trace;   // [wave][8] timestamps; NULL outside tuning runs (ARENO_TRACE builds only read it)
 };
 
 template <int KIND>
@@ -124,7 +120,7 @@ __device__ __forceinline__ typename MfmaOps<KIND>::vec8 to_operand(const uint32_
   uint4_t r;
   if constexpr (KIND == KV_BF16 || KIND == KV_F16) {
     r = uint4_t{w[0], w[1], w[2], w[3]};
-  } else if constexpr (KIND == KV_I8) {  // bytes already flipped to offset binary when staged
+  } else if constexpr (KIND == KV_I8) {  // bytes already flipped to offset binary
     r[0] = __builtin_amdgcn_perm(kF16Filler, w[0], 0x04010400u);
     r[1] = __builtin_amdgcn_perm(kF16Filler, w[0], 0x04030402u);
     r[2] = __builtin_amdgcn_perm(kF16Filler, w[1], 0x04010400u);
@@ -144,169 +140,64 @@ __device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, make_pair<P>(lo, hi));
 }
 
-// Quantize the 16 consecutive elements a lane holds of a new K or V row (32 raw bytes of 16-bit floats) exactly like
-// the cache writer does (cache_write.hip): the row's abs-max is combined over the LPT lanes that share the row.
-template <int KIND, bool SCALE16, int LPT>
-__device__ __forceinline__ void quantize_row_chunk(const uint4_t (&raw)[2], int in_dtype, uint4_t& codes,
-                                                   typename std::conditional<SCALE16, uint16_t, float>::type& scale_raw) {
-  float x[16];
-  float amax = 0.0f;
-#pragma unroll
-  for (int w = 0; w < 8; ++w) {
-    const uint32_t word = raw[w / 4][w % 4];
-    if (in_dtype == ARENO_DT_BF16) {
-      x[2 * w] = bf16_bits_to_float(word & 0xffffu);
-      x[2 * w + 1] = bf16_bits_to_float(word >> 16);
-    } else {
-      x[2 * w] = f16_bits_to_float(word & 0xffffu);
-      x[2 * w + 1] = f16_bits_to_float(word >> 16);
-    }
-    amax = fmaxf(amax, fmaxf(fabsf(x[2 * w]), fabsf(x[2 * w + 1])));
-  }
-#pragma unroll
-  for (int m = 1; m < LPT; m <<= 1) amax = fmaxf(amax, wave_xor(amax, m));
-  float s;
-  if constexpr (KIND == KV_I8) {
-    const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
-    const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
-    s = static_cast<float>(s16_fixed);
-    if constexpr (SCALE16) {
-      scale_raw = __builtin_bit_cast(uint16_t, s16_fixed);
-    } else {
-      scale_raw = s;
-    }
-  } else {
-    s = amax / 448.0f;
-    if (s == 0.0f) s = 1.0f;
-    if constexpr (SCALE16) {
-      scale_raw = static_cast<uint16_t>(float_to_f16_bits(s));
-    } else {
-      scale_raw = s;
-    }
-  }
-#pragma unroll
-  for (int w = 0; w < 4; ++w) {
-    uint32_t word = 0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      uint32_t byte;
-      if constexpr (KIND == KV_I8) {
-        const float code = fminf(fmaxf(rintf(x[4 * w + j] / s), -127.0f), 127.0f);
-        byte = static_cast<uint32_t>(static_cast<int>(code)) & 0xffu;
-      } else {
-        byte = float_to_fp8_byte(fminf(fmaxf(x[4 * w + j] / s, -448.0f), 448.0f));
-      }
-      word |= byte << (8 * j);
-    }
-    codes[w] = word;
-  }
-}
+// a wave-uniform value that the compiler cannot prove uniform (it came out of LDS): move it to a scalar register
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
-// LDS row that holds tile token t of the V tile: the second half is rotated by 4 rows so that the 8 tokens a
-// lane group reads through the transpose load ({4g..4g+3} and {16+4g..16+4g+3}) sit in rows distinct mod 16.
-__device__ __forceinline__ int v_row_of(int t) { return t < 16 ? t : 16 + ((t + 4) & 15); }
-
-// How the global tile range is cut into units (shared by the split and the reduce kernel).
-struct UnitGeometry {
-  int total_tiles;
-  int static_tiles;  // tiles covered by the static units
-  int static_units;  // one per wave piece
-  int unit_tiles;    // tiles per small unit
-  int small_units;
-  // the products below fit 32 bits (every workload but the very largest): 32-bit divisions, which are a fifth of the
-  // instructions of 64-bit ones and show in the launch-latency-sized reduce kernel
-  bool narrow;
-
-  __host__ __device__ int unit_start(int u) const {
-    if (u <= static_units) {
-      if (narrow)
-        return static_cast<int>(static_cast<uint32_t>(u) * static_cast<uint32_t>(static_tiles) /
-                                static_cast<uint32_t>(static_units));
-      return static_cast<int>(static_cast<long long>(u) * static_tiles / static_units);
-    }
-    const long long x = static_tiles + static_cast<long long>(u - static_units) * unit_tiles;
-    return x < total_tiles ? static_cast<int>(x) : total_tiles;
-  }
-  // unit that owns tile x (the largest unit whose first tile is <= x)
-  __host__ __device__ int unit_of(int x) const {
-    if (x < static_tiles) {
-      if (narrow)
-        return static_cast<int>((static_cast<uint32_t>(x + 1) * static_cast<uint32_t>(static_units) +
-                                 static_cast<uint32_t>(static_tiles) - 1u) /
-                                static_cast<uint32_t>(static_tiles)) -
-               1;
-      return static_cast<int>((static_cast<long long>(x + 1) * static_units + static_tiles - 1) / static_tiles - 1);
-    }
-    return static_units + (x - static_tiles) / unit_tiles;
-  }
+// The length arrays and the tile prefix sums in LDS, as the item functions of decode_items.hpp want them.  The
+// "uniform" flavour is for lookups whose index is the same in all lanes of a wave (the tile cursors): the values
+// then live in scalar registers.
+template <bool UNIFORM>
+struct LdsLens {
+  const int* len;
+  const int* glen;
+  __device__ __forceinline__ int row_len(int b) const { return UNIFORM ? uniform(len[b]) : len[b]; }
+  __device__ __forceinline__ int group_len(int g) const { return UNIFORM ? uniform(glen[g]) : glen[g]; }
+};
+struct LdsCum {
+  const int* cum;
+  __device__ __forceinline__ int at(int i) const { return uniform(cum[i]); }
 };
 
-__host__ __device__ inline UnitGeometry make_unit_geometry(int total_tiles, int num_pieces, int max_small,
-                                                           int static_share, int min_unit_tiles) {
-  UnitGeometry g;
-  g.total_tiles = total_tiles;
-  g.static_units = num_pieces;
-  g.static_tiles = static_cast<int>(static_cast<long long>(total_tiles) * static_share / 256);
-  // short batches are not worth a tail of small units: everything goes to the big ones
-  if (total_tiles < 4 * num_pieces || static_share >= 256 || max_small <= 0) g.static_tiles = total_tiles;
-  const int rest = total_tiles - g.static_tiles;
-  g.unit_tiles = min_unit_tiles < 1 ? 1 : min_unit_tiles;
-  if (max_small > 0 && static_cast<long long>(g.unit_tiles) * max_small < rest)
-    g.unit_tiles = (rest + max_small - 1) / max_small;
-  g.small_units = (rest + g.unit_tiles - 1) / g.unit_tiles;
-  // largest product in unit_start / unit_of: (static_tiles + 1) * static_units + static_tiles
-  g.narrow = (static_cast<long long>(g.static_tiles) + 2) * (static_cast<long long>(num_pieces) + 1) < (1LL << 31);
-  return g;
-}
-
-// Position of a tile stream inside a unit: which sequence, which token of it comes next.
-// An item is a run of tokens [lo, hi) read through the block table of row `row`: a whole sequence's visible keys
-// in the plain kernel; in a GROUPED kernel either the shared prefix of `nseq` adjacent rows or the rest of one row.
-struct ItemInfo {
-  int lo, hi, row, nseq;
+// What the pipeline remembers of a tile between the moment its block ids are requested and the moment it is computed
+// (all wave-uniform).
+struct TileDesc {
+  int tok;   // first token of the tile inside its sequence
+  int end;   // end of the item's cached tokens
+  int row;   // block-table / query row
+  int nseq;  // rows side by side (shared items), else 1
+  int b;     // item index
+  int kind;  // bit 0: the tile opens its item; bit 1: it holds only the token being appended
 };
+constexpr int kTileOpens = 1, kTileNewToken = 2;
 
-struct TileCursor {
-  int b;    // item (= sequence in the plain kernel)
-  int tok;  // first token (position inside the sequence) of the tile
-  int end;  // end of the item's token range (cache_seqlens[b] + 1 for a sequence)
-  int row;  // block-table / query row of the item
-  int nseq;
-  ItemInfo next;  // item b + 1, fetched one item ahead
-};
-
-#ifndef ARENO_MFMA_QUANT_OCC
-#define ARENO_MFMA_QUANT_OCC 2
-#endif
-// DSPLIT > 1 serves heads of DSPLIT * D elements (256 = 2 x 128, 192 = 3 x 64, 512 = 4 x 128): DSPLIT adjacent waves of the
-// workgroup take one part of the head dimension each.  Every wave computes the part of S = K . Q^T over its
-// elements, the waves exchange the parts through LDS (a wave's K tile is dead once its products are issued, so the
-// part is parked there), add them in the same order and go on with identical scores: the same softmax in all,
-// P . V over the wave's own part of V, the wave's part of the partial row.  The waves of a head synchronise through
-// two counters each in LDS (part ready / parts consumed); no workgroup barrier is involved, so the heads of one
-// workgroup may run different units.
+// DSPLIT > 1 serves heads of DSPLIT * D elements (256 = 2 x 128, 192 = 3 x 64, 512 = 4 x 128): DSPLIT adjacent waves
+// of the workgroup take one part of the head dimension each.  Every wave computes the part of S = K . Q^T over its
+// elements, the waves exchange the parts through LDS, add them in the same order and go on with identical scores:
+// the same softmax in all, P . V over the wave's own part of V, the wave's part of the partial row.  The waves of a
+// head synchronise through two counters each in LDS (part ready / parts consumed); no workgroup barrier is involved,
+// so the heads of one workgroup may run different units.
 template <int KIND, int D, bool SCALE16, int NW, bool GROUPED = false, int DSPLIT = 1>
-__global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUANT_OCC : 2) void decode_mfma_kernel(
-    MfmaDecodeParams mp) {
+__global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodeParams mp) {
   using T = KVTraits<KIND>;
   using Ops = MfmaOps<KIND>;
   using V8 = typename Ops::vec8;
   using Pair = typename T::pair_t;
   const DecodeParams& p = mp.d;
   constexpr int ES = T::kBytes;
-  constexpr int EPL = 16 / ES;
-  constexpr int LPT = D / EPL;
-  constexpr int TPL = kWave / LPT;
   constexpr int TK = kTileTokens;
-  constexpr int NLD = TK / TPL;  // 16-byte loads per lane, per tensor, per tile
-  constexpr int RSK = D * ES + 16;
-  constexpr int RSV = ES == 1 ? D + 16 : 2 * D + 32;
-  constexpr int NS = D / 32;       // QK^T k-slices
-  constexpr int NB = D / 16;       // P.V dim blocks
-  constexpr int WPL = 8 * ES / 4;  // dwords per lane per k-slice of 8 elements
+  constexpr int CPT = D * ES / 16;     // 16-byte chunks per token row
+  constexpr int CPL = CPT / 4;         // chunks per lane and token: lk, lk + 4, ...
+  constexpr int NS = D / 32;           // QK^T k-slices
+  constexpr int NB = D / 16;           // P.V dim blocks
+  constexpr int WPS = 8 * ES / 4;      // dwords per k-slice of 8 elements
+  constexpr int DEPTH = ES == 1 ? 2 : 1;  // tiles in flight per wave
+  constexpr int TGS = CPT * 256 + 128;    // bytes of one token group of the V tile in LDS (128 of padding behind it)
   constexpr float kPScale = T::kQuant ? 256.0f : 1.0f;
-  constexpr int kWaveLds = TK * RSK + TK * RSV + 2 * TK * 4;
-  static_assert(NLD >= 1 && LPT >= 4 && LPT <= 16, "unsupported head_dim");
+  constexpr int kParkFloats = DSPLIT > 1 ? 8 * kWave : 0;
+  constexpr int kWaveLds = 2 * TGS + 2 * TK * 4 + kParkFloats * 4;
+  constexpr int UPW = D / 64;          // dwords per lane of an update row pair (K row in lanes 0..31, V row in 32..63)
+  static_assert(CPL >= 1 && CPL <= 4 && (D == 64 || D == 128), "unsupported head_dim");
+  static_assert(2 * TGS >= 2 * D * 4, "the new token's rows borrow the V tile");
   static_assert(DSPLIT == 1 || (DSPLIT >= 2 && DSPLIT <= 4 && !GROUPED && NW % DSPLIT == 0), "unsupported head split");
   constexpr int DFULL = D * DSPLIT;  // elements of a whole head (row of Q, of a cache page, of a partial)
 
@@ -314,16 +205,9 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   constexpr int kMaxItems = (GROUPED ? 2 : 1) * kMfmaMaxBatch;  // at most one shared item per row on top of the rows
   __shared__ int s_cum[kMaxItems + 1];
   __shared__ int s_wave_tot[NW];
-  // The length arrays in LDS: what a wave needs to know about an item comes from here instead of from a memory round
-  // trip per lookup.  Without prefix groups the prefix sum's own loads fill s_len.  With them an item's extent takes up
-  // to six dependent reads (the group's shared length, the members' lengths, the row's own) and the prefix sum asks for
-  // 2 * 1024 / threads items per thread -- from global memory some forty round trips one after the other in the first
-  // wave of every workgroup -- so the workgroup first copies both arrays with independent loads.  Where the copies
-  // would cost the second resident workgroup (prefix groups over 16-bit caches) the lookups stay on global memory.
-  constexpr bool kLocalLens = !GROUPED || ES == 1;
-  constexpr int kMaxGroups = kMfmaMaxBatch / 2;  // groups have at least two rows
-  __shared__ int s_len[kLocalLens ? kMfmaMaxBatch : 1];            // sequence lengths of the rows
-  __shared__ int s_group_len[GROUPED && kLocalLens ? kMaxGroups : 1];  // shared prefix length of each group
+  __shared__ int s_len[kMfmaMaxBatch];                          // sequence lengths of the rows
+  constexpr int kMaxGroups = kMfmaMaxBatch / 2;                 // groups have at least two rows
+  __shared__ int s_group_len[GROUPED ? kMaxGroups : 1];         // shared prefix length of each group
   __shared__ int s_pair_flags[2][NW];  // [0]: score parts this wave has published, [1]: steps whose parts it has read
   constexpr int SPT = (kMaxItems + NW * kWave - 1) / (NW * kWave);  // items per thread in the prefix sum
 
@@ -332,107 +216,59 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   const int wave = tid >> 6;
 #ifdef ARENO_TRACE
   const int trace_wave = (blockIdx.y * gridDim.x + blockIdx.x) * NW + wave;
-  int trace_n = 2;
+  int trace_n = 1;
   if (mp.trace && lane == 0) {
-    // start time, and in word 15 where the wave runs: XCC id (hardware register 20) above the HW_ID word (register 4)
-    mp.trace[trace_wave * 16] = wall_clock64();
-    mp.trace[trace_wave * 16 + 15] = (static_cast<unsigned long long>(__builtin_amdgcn_s_getreg((31 << 11) | 20)) << 32) |
-                                     static_cast<unsigned int>(__builtin_amdgcn_s_getreg((31 << 11) | 4));
+    // start time, and in word 7 where the wave runs: XCC id (hardware register 20) above the HW_ID word (register 4)
+    mp.trace[trace_wave * 8] = wall_clock64();
+    mp.trace[trace_wave * 8 + 7] = (static_cast<unsigned long long>(__builtin_amdgcn_s_getreg((31 << 11) | 20)) << 32) |
+                                    static_cast<unsigned int>(__builtin_amdgcn_s_getreg((31 << 11) | 4));
   }
-#define ARENO_TRACE_POINT()                                                                   \
-  if (mp.trace && lane == 0 && trace_n < 15) mp.trace[trace_wave * 16 + trace_n++] = wall_clock64()
+#define ARENO_TRACE_POINT() \
+  if (mp.trace && lane == 0 && trace_n < 6) mp.trace[trace_wave * 8 + trace_n++] = wall_clock64()
 #else
 #define ARENO_TRACE_POINT()
 #endif
   const int lr = lane & 15;  // MFMA row / column index
   const int lk = lane >> 4;  // MFMA k group
-  const int grp = lane / LPT;
-  const int dc = lane % LPT;
 
-  // ---- the item list ----------------------------------------------------------------------------------------------
-  const int num_items = GROUPED ? mp.num_shared + p.batch : p.batch;
-  // tokens of a sub-group's shared prefix: the caller's figure, clipped to what every member has cached and cut to a
-  // whole number of tiles
-  if constexpr (GROUPED && kLocalLens) {
-    // the launcher sends whole groups of at least two rows, at most kMfmaMaxBatch rows
-    const int groups = min(p.batch / max(mp.group_rows, 2), kMaxGroups);
-    for (int i = tid; i < min(p.batch, kMfmaMaxBatch); i += NW * kWave) s_len[i] = p.cache_seqlens[i];
-    for (int i = tid; i < groups; i += NW * kWave) s_group_len[i] = mp.shared_lens[i];
-    __syncthreads();
-  }
-  // length of row b / shared prefix length of group gi (indices clamped into the LDS copies)
-  auto row_len = [&](int b) {
-    if constexpr (GROUPED && kLocalLens) {
-      return s_len[min(max(b, 0), kMfmaMaxBatch - 1)];
-    } else {
-      return p.cache_seqlens[b];
-    }
-  };
-  auto group_len = [&](int gi) {
-    if constexpr (GROUPED && kLocalLens) {
-      return s_group_len[min(max(gi, 0), kMaxGroups - 1)];
-    } else {
-      return mp.shared_lens[gi];
-    }
-  };
-  auto shared_tokens = [&](int sub, int& row0, int& count) {
-    const int gi = sub / mp.subs_per_group;
-    const int j = sub - gi * mp.subs_per_group;
-    row0 = gi * mp.group_rows + j * mp.cols_seqs;
-    count = min(mp.cols_seqs, mp.group_rows - j * mp.cols_seqs);
-    int len = group_len(gi);
-    for (int m = 0; m < count; ++m) len = min(len, row_len(row0 + m));
-    return max(len, 0) & ~(TK - 1);
-  };
-  auto item_info = [&](int v) {
-    ItemInfo it = {0, 0, 0, 1};
-    if (v >= num_items) return it;
-    if constexpr (GROUPED) {
-      if (v < mp.num_shared) {
-        it.hi = shared_tokens(v, it.row, it.nseq);
-        return it;
-      }
-      const int b = v - mp.num_shared;
-      const int gi = b / mp.group_rows;
-      int row0, count;
-      it.lo = shared_tokens(gi * mp.subs_per_group + (b - gi * mp.group_rows) / mp.cols_seqs, row0, count);
-      it.hi = row_len(b) + 1;
-      it.row = b;
-      return it;
-    } else {
-      it.hi = s_len[v] + 1;
-      it.lo = first_allowed_key(it.hi, p.window_left);
-      it.row = v;
-      return it;
-    }
-  };
-  // ---- tiles per item, exclusive prefix sum over the items --------------------------------------------------------
+  // ---- the item list: lengths into LDS, tiles per item, exclusive prefix sum over the items ------------------------
+  const ItemShape& shape = mp.items;
+  const int num_items = shape.num_items();
+  const LdsLens<false> lens_any = {s_len, s_group_len};
+  const LdsLens<true> lens = {s_len, s_group_len};
+  const LdsCum cum = {s_cum};
   {
     int nt[SPT];
     int local = 0;
     if constexpr (GROUPED) {
+      // an item's extent takes the group's length, its members' lengths and the row's own: the workgroup copies both
+      // arrays with independent loads first (the launcher sends at most kMfmaMaxBatch rows in groups of >= 2)
+      for (int i = tid; i < shape.batch; i += NW * kWave) s_len[i] = p.cache_seqlens[i];
+      for (int i = tid; i < shape.num_groups(); i += NW * kWave) s_group_len[i] = mp.shared_lens[i];
+      __syncthreads();
 #pragma unroll
       for (int j = 0; j < SPT; ++j) {
         const int v = SPT * tid + j;
-        nt[j] = 0;
-        if (v < num_items) {
-          const ItemInfo it = item_info(v);
-          nt[j] = (it.hi - it.lo + TK - 1) / TK;
-        }
+        nt[j] = v < num_items ? item_info<true>(shape, lens_any, v).tiles() : 0;
         local += nt[j];
       }
     } else {
-      // the thread's sequence lengths are fetched together (clamped index, no branch around the load): as loads
-      // under `if (v < num_items)` they went out one at a time, SPT memory round trips at the start of every launch
+      // the thread's sequence lengths are fetched together (clamped index, no branch around the load)
       int len[SPT];
 #pragma unroll
       for (int j = 0; j < SPT; ++j) len[j] = p.cache_seqlens[min(SPT * tid + j, num_items - 1)];
 #pragma unroll
       for (int j = 0; j < SPT; ++j) {
         const int v = SPT * tid + j;
-        const int hi = len[j] + 1;
-        nt[j] = v < num_items ? (hi - first_allowed_key(hi, p.window_left) + TK - 1) / TK : 0;
-        if (v < num_items) s_len[v] = len[j];
+        nt[j] = 0;
+        if (v < num_items) {
+          s_len[v] = len[j];
+          ItemInfo it;
+          it.lo = first_visible_key(len[j] + 1, shape.window_left);
+          it.end = len[j] + 1 - shape.new_token_tile;
+          it.has_new = shape.new_token_tile;
+          nt[j] = it.tiles();
+        }
         local += nt[j];
       }
     }
@@ -457,120 +293,107 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     if (tid == NW * kWave - 1 && SPT * (tid + 1) <= num_items) s_cum[SPT * (tid + 1)] = excl;
     __syncthreads();
   }
-  // ---- unit geometry -----------------------------------------------------------------------------------
-  // Tiles [0, static_tiles) are cut into num_pieces equal big units, one per wave of the first static_wgs
-  // workgroups; the rest is cut into small units for the workgroups behind them in the grid.  Those start as CUs
-  // become free, so the hardware dispatcher hands the tail to whichever CU got the better memory service:
-  // service is uneven across CUs, and with equal shares only the slowest wave would set the run time.
-  const int total_tiles = s_cum[num_items];
-  const UnitGeometry geo =
-      make_unit_geometry(total_tiles, mp.num_pieces, mp.max_small, mp.static_share, mp.min_unit_tiles);
+  const int total_tiles = cum.at(num_items);
+  const UnitGeometry geo = make_unit_geometry(total_tiles, mp.num_units);
   if (blockIdx.x == 0 && blockIdx.y == 0) {
     for (int v = tid; v <= num_items; v += NW * kWave) mp.plan[v] = s_cum[v];
   }
+  ARENO_TRACE_POINT();
 
   const int hw_count = p.heads_per_wg;
   const int half = wave % DSPLIT;  // which part of the head dimension this wave owns
   const int hw = (wave / DSPLIT) % hw_count;
   const int ts = (wave / DSPLIT) / hw_count;
   const int kvh = blockIdx.y * hw_count + hw;
-  char* const k_tile = &s_tiles[wave][0];
-  char* const v_tile = k_tile + TK * RSK;
-  float* const ksc = reinterpret_cast<float*>(&s_tiles[wave][TK * RSK + TK * RSV]);
-  float* const vsc = ksc + TK;
+  char* const v_tile = &s_tiles[wave][0];
+  float* const sc_lds = reinterpret_cast<float*>(&s_tiles[wave][2 * TGS]);  // [0, 32): K scales, [32, 64): V scales
+  float* const park = reinterpret_cast<float*>(&s_tiles[wave][2 * TGS + 2 * TK * 4]);
 
   constexpr int64_t row_bytes = static_cast<int64_t>(DFULL) * ES;
   const int64_t half_bytes = static_cast<int64_t>(half) * D * ES;  // of this wave's part inside a cache / update row
   const int h0 = kvh * p.group;
   const bool q_is_operand_type = (KIND == KV_BF16 && p.q_dtype == ARENO_DT_BF16) ||
                                  (KIND != KV_BF16 && p.q_dtype == ARENO_DT_F16);
+  auto is_shared = [&](int v) { return GROUPED && v < shape.num_shared; };
+  // first element of the 8 that k-slice sl holds in this lane (the chunk order of the K loads)
+  auto slice_base = [&](int sl) { return ES == 1 ? 16 * (lk + 4 * (sl >> 1)) + 8 * (sl & 1) : 8 * (lk + 4 * sl); };
+  // byte offset of token row r (0..15) of chunk c inside a token group of the V tile: 16-bit tiles keep the two
+  // halves of an odd chunk's rows swapped (see the layout note above)
+  auto chunk_row_pos = [](int c, int r) { return c * 256 + ((ES == 2 && (c & 1)) ? (r ^ 8) : r) * 16; };
 
-  auto enter_item = [&](TileCursor& c, const ItemInfo& it) {
-    c.tok = it.lo;
-    c.end = it.hi;
-    c.row = it.row;
-    c.nseq = it.nseq;
-  };
-  // move a cursor from tile x to tile x + 1; returns true when that tile starts a new item
-  auto advance = [&](TileCursor& c, int x_next) {
-    if (x_next == s_cum[c.b + 1]) {
-      ++c.b;
-      if constexpr (GROUPED) {
-        if (s_cum[c.b + 1] == x_next) {
-          // items without tiles (a group with no shared prefix): skip them; the prefetched item is not the right one
-          do {
-            ++c.b;
-          } while (s_cum[c.b + 1] == x_next);
-          enter_item(c, item_info(c.b));
-          c.next = item_info(c.b + 1);
-          return true;
-        }
-      }
-      enter_item(c, c.next);
-      c.next = item_info(c.b + 1);
-      return true;
-    }
-    c.tok += TK;
-    return false;
-  };
-  auto is_shared = [&](int v) { return GROUPED && v < mp.num_shared; };
-
-  TileCursor kv_cur, id_cur;
-  int unit = 0;
-  int ids[NLD];
-  auto issue_id_loads = [&]() {
-    const int32_t* table_row = p.block_table + static_cast<int64_t>(id_cur.row) * p.max_blocks;
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const int t = min(id_cur.tok + i * TPL + grp, id_cur.end - 1);
-      const int col = p.bs_shift >= 0 ? (t >> p.bs_shift) : (t / p.block_size);
-      ids[i] = table_row[col];
-    }
-  };
-
-  uint4_t kreg[NLD], vreg[NLD];
+  // ---- the pipeline's registers ------------------------------------------------------------------------------------
   typedef typename std::conditional<SCALE16, uint16_t, float>::type scale_raw_t;
-  scale_raw_t ksreg[NLD], vsreg[NLD];
-  // fused append state of the tile in flight
-  const bool fused_append = mp.k_update != nullptr;
-  bool tail_tile = false;  // wave-uniform: the tile in kreg / vreg ends its sequence (holds the newest token)
-  int64_t new_row = 0;     // cache row of the newest token, in the lanes that hold it
-  uint4_t upd_k[2], upd_v[2];
-  auto issue_kv_loads = [&]() {
-    tail_tile = fused_append && !is_shared(kv_cur.b) && kv_cur.tok + TK >= kv_cur.end;
-    const int64_t upd_row = static_cast<int64_t>(kv_cur.row) * p.kv_heads + kvh;
+  uint4_t kreg[DEPTH][2 * CPL], vreg[DEPTH][2 * CPL];
+  scale_raw_t sreg[DEPTH];   // lane l < 32: K scale of tile token l; else V scale of token l - 32
+  uint32_t upd[DEPTH][UPW];  // a new-token tile: the update rows, K in lanes 0..31, V in 32..63
+  uint32_t new_row[DEPTH];   // a new-token tile: cache row (block, slot, head) the token goes to
+  TileDesc desc[DEPTH];
+  TileCursor cur;      // the furthest tile requested so far (its block ids are on their way)
+  TileDesc desc_ids;   // = that tile
+  int ids[2];          // its block ids, for this lane's token of each group (new-token tile: of the token's page)
+
+  auto describe = [&](const TileCursor& c, bool opens) {
+    TileDesc t;
+    t.tok = c.tok;
+    t.end = c.it.end;
+    t.row = c.it.row;
+    t.nseq = c.it.nseq;
+    t.b = c.b;
+    t.kind = (opens ? kTileOpens : 0) | (c.on_new_token() ? kTileNewToken : 0);
+    return t;
+  };
+  auto column_of = [&](int t) { return p.bs_shift >= 0 ? (t >> p.bs_shift) : (t / p.block_size); };
+  auto slot_of = [&](int t) { return p.bs_shift >= 0 ? (t & (p.block_size - 1)) : (t % p.block_size); };
+  auto issue_id_loads = [&](const TileDesc& t) {
+    const int32_t* table_row = p.block_table + static_cast<int64_t>(t.row) * p.max_blocks;
+    if (t.kind & kTileNewToken) {
+      ids[0] = ids[1] = table_row[column_of(t.end)];  // position L_b = end of the cached tokens
+    } else {
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const int tt = kv_cur.tok + i * TPL + grp;
-      const int t = min(tt, kv_cur.end - 1);
-      const int slot = p.bs_shift >= 0 ? (t & (p.block_size - 1)) : (t % p.block_size);
-      const int64_t row = (static_cast<int64_t>(ids[i]) * p.block_size + slot) * p.kv_heads + kvh;
-      const char* ka = static_cast<const char*>(p.k_cache) + row * row_bytes + half_bytes + dc * 16;
-      const char* va = static_cast<const char*>(p.v_cache) + row * row_bytes + half_bytes + dc * 16;
-      if (tail_tile && tt >= kv_cur.end - 1) {
-        // the page slot of the newest token (and the clamped rows behind it) is not written yet
-        if (tt == kv_cur.end - 1) new_row = row;
-        if constexpr (!T::kQuant) {
-          ka = static_cast<const char*>(mp.k_update) + upd_row * row_bytes + half_bytes + dc * 16;
-          va = static_cast<const char*>(mp.v_update) + upd_row * row_bytes + half_bytes + dc * 16;
-        }
+      for (int tg = 0; tg < 2; ++tg) ids[tg] = table_row[column_of(min(t.tok + 16 * tg + lr, t.end - 1))];
+    }
+  };
+  // cache row (block, slot, head) of this lane's token of group tg, from the block ids that have arrived
+  uint32_t rows[2];
+  auto rows_from_ids = [&](const TileDesc& t) {
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+      const int tok = (t.kind & kTileNewToken) ? t.end : min(t.tok + 16 * tg + lr, t.end - 1);
+      rows[tg] = (static_cast<uint32_t>(ids[tg]) * p.block_size + slot_of(tok)) * p.kv_heads + kvh;
+    }
+  };
+  auto issue_v_loads = [&](auto set_c, const TileDesc& t) {
+    constexpr int SET = decltype(set_c)::value;
+    if (t.kind & kTileNewToken) {
+      if constexpr (DSPLIT == 1) {
+        const void* src = lane < 32 ? mp.k_update : mp.v_update;
+        const int64_t off = (static_cast<int64_t>(t.row) * p.kv_heads + kvh) * D * 2 + (lane & 31) * (UPW * 4);
+#pragma unroll
+        for (int w = 0; w < UPW; ++w) upd[SET][w] = *reinterpret_cast<const uint32_t*>(static_cast<const char*>(src) + off + 4 * w);
+        new_row[SET] = rows[0];
       }
-      kreg[i] = *reinterpret_cast<const uint4_t*>(ka);
-      vreg[i] = *reinterpret_cast<const uint4_t*>(va);
-      if constexpr (T::kQuant) {
-        ksreg[i] = static_cast<const scale_raw_t*>(p.k_scale)[row];
-        vsreg[i] = static_cast<const scale_raw_t*>(p.v_scale)[row];
-      }
+      return;
+    }
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+      const char* va = static_cast<const char*>(p.v_cache) + rows[tg] * row_bytes + half_bytes + lk * 16;
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) vreg[SET][tg * CPL + j] = *reinterpret_cast<const uint4_t*>(va + 64 * j);
     }
     if constexpr (T::kQuant) {
-      if (tail_tile) {
-        // every lane group fetches the whole new row (16 elements per lane), so each can quantize it on its own
-        const int64_t off = (upd_row * D + dc * EPL) * 2;
-        upd_k[0] = load16(mp.k_update, off);
-        upd_k[1] = load16(mp.k_update, off + 16);
-        upd_v[0] = load16(mp.v_update, off);
-        upd_v[1] = load16(mp.v_update, off + 16);
-      }
+      const uint32_t r = (lk & 1) ? rows[1] : rows[0];
+      const void* sp = lk < 2 ? p.k_scale : p.v_scale;
+      sreg[SET] = static_cast<const scale_raw_t*>(sp)[r];
+    }
+  };
+  auto issue_k_loads = [&](auto set_c, const TileDesc& t) {
+    constexpr int SET = decltype(set_c)::value;
+    if (t.kind & kTileNewToken) return;
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+      const char* ka = static_cast<const char*>(p.k_cache) + rows[tg] * row_bytes + half_bytes + lk * 16;
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) kreg[SET][tg * CPL + j] = *reinterpret_cast<const uint4_t*>(ka + 64 * j);
     }
   };
   auto scale_value = [](scale_raw_t raw) -> float {
@@ -581,23 +404,23 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     }
   };
 
-  // Q of a sequence: lane (lr = head, lk) needs dims (D/4)*lk + 8*s + [0, 8) of head h0 + lr, 16 raw bytes per
-  // slice for 16-bit queries; fetched when the KV cursor enters the sequence, converted when compute gets there.
+  // Q of an item: lane (lr = column, lk) needs, per k-slice, the 8 elements the K loads put there; 16 raw bytes per
+  // slice for 16-bit queries.  Requested one step before the item's first tile is computed, converted when compute
+  // gets there.  Column lr of the MFMA tiles: head lr of the row in a per-row item, (row lr / G, head lr % G) in a
+  // shared item.
   uint4_t qraw[NS];
-  // column lr of the MFMA tiles: head lr of the row in a per-row item, (row lr / G, head lr % G) in a shared item
   const int col_seq = GROUPED ? lr / p.group : 0;
   const int col_head = GROUPED ? lr - col_seq * p.group : lr;
-  auto issue_q_loads = [&](const TileCursor& c) {
-    const bool shared = is_shared(c.b);
+  auto issue_q_loads = [&](const TileDesc& t) {
+    const bool shared = is_shared(t.b);
     const int m = shared ? col_seq : 0;
     const int g = shared ? col_head : lr;
-    const bool live = shared ? m < c.nseq : lr < p.group;
+    const bool live = shared ? m < t.nseq : lr < p.group;
 #pragma unroll
     for (int sl = 0; sl < NS; ++sl) {
       qraw[sl] = uint4_t{0u, 0u, 0u, 0u};
       if (live) {
-        const int64_t idx =
-            (static_cast<int64_t>(c.row + m) * p.q_heads + h0 + g) * DFULL + half * D + (D / 4) * lk + 8 * sl;
+        const int64_t idx = (static_cast<int64_t>(t.row + m) * p.q_heads + h0 + g) * DFULL + half * D + slice_base(sl);
         qraw[sl] = load16(p.q, idx * 2);
       }
     }
@@ -646,6 +469,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     p_sum = 0.0f;
   };
 
+  int unit = 0;
   auto write_partial = [&](int v, int row, int nseq) {
     // combine the four k-groups' row sums; every lane of a head ends with the head's totals
     const float l_tot = rows_sum(l_run);
@@ -682,305 +506,420 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       __builtin_amdgcn_s_sleep(1);
     }
   };
+  auto lds_fence = [&]() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
 
-  // ---- this wave's unit ------------------------------------------------------------------------------------------
-  const int bx = blockIdx.x;
-  unit = bx < mp.static_wgs ? bx * mp.tok_splits + ts : geo.static_units + (bx - mp.static_wgs) * mp.tok_splits + ts;
-  {
-    const int x0 = geo.unit_start(unit);
-    const int x1 = unit < geo.static_units + geo.small_units ? geo.unit_start(unit + 1) : x0;
-    if (x0 < x1) {
-      // item that owns tile x0: the largest v with cum[v] <= x0
-      int v_first;
-      {
-        int lo = 0, hi = num_items;
-        while (lo + 1 < hi) {
-          const int mid = (lo + hi) >> 1;
-          if (s_cum[mid] <= x0) {
-            lo = mid;
+  // ---- the token being appended: quantize, store into the page, fold into the running softmax (vector ALU) ---------
+  auto new_token_step = [&](auto set_c, const TileDesc& t) {
+    constexpr int SET = decltype(set_c)::value;
+    if constexpr (DSPLIT == 1) {
+      constexpr int EPU = 2 * UPW;  // elements of the row this lane holds: (lane % 32) * EPU ...
+      const int sub = lane & 31;
+      const bool is_v = lane >= 32;
+      float x[EPU];
+#pragma unroll
+      for (int w = 0; w < UPW; ++w) {
+        const uint32_t word = upd[SET][w];
+        if (p.q_dtype == ARENO_DT_BF16) {
+          x[2 * w] = bf16_bits_to_float(word & 0xffffu);
+          x[2 * w + 1] = bf16_bits_to_float(word >> 16);
+        } else {
+          x[2 * w] = f16_bits_to_float(word & 0xffffu);
+          x[2 * w + 1] = f16_bits_to_float(word >> 16);
+        }
+      }
+      const int64_t dst_row = new_row[SET];
+      char* cache = static_cast<char*>(const_cast<void*>(is_v ? p.v_cache : p.k_cache));
+      float xhat[EPU];  // what a reader of the page sees
+      if constexpr (T::kQuant) {
+        float amax = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPU; ++e) amax = fmaxf(amax, fabsf(x[e]));
+#pragma unroll
+        for (int m = 1; m < 32; m <<= 1) amax = fmaxf(amax, wave_xor(amax, m));
+        float s, s_stored;
+        scale_raw_t raw;
+        if constexpr (KIND == KV_I8) {
+          const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
+          const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
+          s = static_cast<float>(s16_fixed);
+          s_stored = s;
+          if constexpr (SCALE16) {
+            raw = __builtin_bit_cast(uint16_t, s16_fixed);
           } else {
-            hi = mid;
+            raw = s;
+          }
+        } else {
+          s = amax / 448.0f;
+          if (s == 0.0f) s = 1.0f;
+          if constexpr (SCALE16) {
+            raw = static_cast<uint16_t>(float_to_f16_bits(s));
+            s_stored = f16_bits_to_float(raw);
+          } else {
+            raw = s;
+            s_stored = s;
           }
         }
-        v_first = lo;
-      }
-
-      // ---- three cursors: block ids are fetched two tiles ahead, KV one tile ahead of the tile being computed ---
-      kv_cur.b = v_first;
-      enter_item(kv_cur, item_info(v_first));
-      kv_cur.next = item_info(v_first + 1);
-      kv_cur.tok += (x0 - s_cum[v_first]) * TK;
-      id_cur = kv_cur;
-
-      // ---- prologue -------------------------------------------------------------------------------------------
-      issue_id_loads();
-      issue_q_loads(kv_cur);
-      issue_kv_loads();  // tile x0 (waits for its ids)
-      if (x0 + 1 < x1) {
-        advance(id_cur, x0 + 1);
-        issue_id_loads();  // ids of tile x0 + 1
-      }
-      int cp_b = kv_cur.b, cp_row = kv_cur.row, cp_nseq = kv_cur.nseq, cp_tok = kv_cur.tok, cp_end = kv_cur.end;
-      adopt_q();
-      reset_state();
-
-      for (int x = x0; x < x1; ++x) {
-        ARENO_TRACE_POINT();
-        if constexpr (DSPLIT > 1) {
-          // the other waves of the head must have read the score part parked in this wave's K tile before the tile
-          // is rewritten
+        uint32_t word = 0;
 #pragma unroll
-          for (int part = 0; part < DSPLIT; ++part) {
-            if (part != half) pair_wait(&s_pair_flags[1][wave - half + part], pair_step);
-          }
-        }
-        // -- stage the fetched tile into LDS (waits for its loads) ---------------------------------------------
-        if (tail_tile) {
-          // the newest token: quantize (8-bit caches), substitute it for the unwritten slot, store it into the page
-          if constexpr (T::kQuant) {
-            uint4_t qk, qv;
-            scale_raw_t qks, qvs;
-            quantize_row_chunk<KIND, SCALE16, LPT>(upd_k, p.q_dtype, qk, qks);
-            quantize_row_chunk<KIND, SCALE16, LPT>(upd_v, p.q_dtype, qv, qvs);
-#pragma unroll
-            for (int i = 0; i < NLD; ++i) {
-              if (cp_tok + i * TPL + grp >= cp_end - 1) {
-                kreg[i] = qk;
-                vreg[i] = qv;
-                ksreg[i] = qks;
-                vsreg[i] = qvs;
-              }
-            }
-          }
-#pragma unroll
-          for (int i = 0; i < NLD; ++i) {
-            if (cp_tok + i * TPL + grp == cp_end - 1) {
-              char* kc = static_cast<char*>(const_cast<void*>(p.k_cache));
-              char* vc = static_cast<char*>(const_cast<void*>(p.v_cache));
-              *reinterpret_cast<uint4_t*>(kc + new_row * row_bytes + half_bytes + dc * 16) = kreg[i];
-              *reinterpret_cast<uint4_t*>(vc + new_row * row_bytes + half_bytes + dc * 16) = vreg[i];
-              if constexpr (T::kQuant) {
-                if (dc == 0) {
-                  static_cast<scale_raw_t*>(const_cast<void*>(p.k_scale))[new_row] = ksreg[i];
-                  static_cast<scale_raw_t*>(const_cast<void*>(p.v_scale))[new_row] = vsreg[i];
-                }
-              }
-            }
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-          const int t = i * TPL + grp;  // tile-local token
-          uint4_t kk = kreg[i], vv = vreg[i];
+        for (int e = 0; e < EPU; ++e) {
+          uint32_t byte;
+          float code_value;
           if constexpr (KIND == KV_I8) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              kk[j] ^= kI8Flip;
-              vv[j] ^= kI8Flip;
-            }
-          }
-          *reinterpret_cast<uint4_t*>(k_tile + t * RSK + dc * 16) = kk;
-          *reinterpret_cast<uint4_t*>(v_tile + v_row_of(t) * RSV + dc * 16) = vv;
-          if (dc == 0) {
-            const bool ok = cp_tok + t < cp_end;
-            if constexpr (T::kQuant) {
-              ksc[t] = ok ? scale_value(ksreg[i]) * p.scale_log2e : kNegInf;
-              vsc[t] = ok ? scale_value(vsreg[i]) * kPScale : 0.0f;
-            } else {
-              ksc[t] = ok ? p.scale_log2e : kNegInf;
-              vsc[t] = ok ? kPScale : 0.0f;
-            }
-          }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-        // -- fetch tile x + 1 (its block ids arrived during the previous iteration) and the ids of tile x + 2 ------
-        bool next_is_new_seq = false;
-        if (x + 1 < x1) {
-          next_is_new_seq = advance(kv_cur, x + 1);
-          if (next_is_new_seq) issue_q_loads(kv_cur);
-          issue_kv_loads();
-          if (x + 2 < x1) {
-            advance(id_cur, x + 2);
-            issue_id_loads();
-          }
-        }
-
-        // -- S^T = K . Q^T for the two 16-token groups ------------------------------------------------------------
-        float s[2][4];
-#pragma unroll
-        for (int tg = 0; tg < 2; ++tg) {
-          float4_t c = {0.0f, 0.0f, 0.0f, 0.0f};
-          const char* krow = k_tile + (16 * tg + lr) * RSK + (D / 4) * ES * lk;
-          uint32_t kw[NS * WPL];
-#pragma unroll
-          for (int q4 = 0; q4 < NS * WPL / 4; ++q4) {
-            const uint4_t r = *reinterpret_cast<const uint4_t*>(krow + 16 * q4);
-            kw[4 * q4 + 0] = r[0];
-            kw[4 * q4 + 1] = r[1];
-            kw[4 * q4 + 2] = r[2];
-            kw[4 * q4 + 3] = r[3];
-          }
-#pragma unroll
-          for (int sl = 0; sl < NS; ++sl) c = Ops::mfma(to_operand<KIND>(&kw[sl * WPL]), qop[sl], c);
-          if constexpr (DSPLIT == 1) {
-            const float4_t sc = *reinterpret_cast<const float4_t*>(ksc + 16 * tg + 4 * lk);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              // tokens past the end carry a -inf scale; keep them exactly -inf (0 * -inf would be NaN)
-              const float v = c[j] - qbias;
-              s[tg][j] = sc[j] == kNegInf ? kNegInf : v * sc[j];
-            }
+            const float code = fminf(fmaxf(rintf(x[e] / s), -127.0f), 127.0f);
+            byte = static_cast<uint32_t>(static_cast<int>(code)) & 0xffu;
+            code_value = code;
           } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) s[tg][j] = c[j] - qbias;  // this wave's part of the dot products
+            byte = float_to_fp8_byte(fminf(fmaxf(x[e] / s, -448.0f), 448.0f));
+            code_value = fp8_byte_to_float(byte);
           }
+          word |= byte << (8 * e);
+          xhat[e] = code_value * s_stored;
         }
-        if constexpr (DSPLIT > 1) {
-          // Park the part where the K tile was (its rows have been read by the products above), tell the other waves of
-          // the head, wait for their parts, add all parts in the order of the head dimension.  Every wave of the head
-          // ends up with the same eight sums.
-          float* mine = reinterpret_cast<float*>(k_tile);
-#pragma unroll
-          for (int tg = 0; tg < 2; ++tg) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) mine[(4 * tg + j) * kWave + lane] = s[tg][j];
-          }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-          ++pair_step;
-          if (lane == 0)
-            __hip_atomic_store(&s_pair_flags[0][wave], pair_step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          const int first_wave = wave - half;
-          float total[2][4];
-#pragma unroll
-          for (int tg = 0; tg < 2; ++tg) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) total[tg][j] = 0.0f;
-          }
-#pragma unroll
-          for (int part = 0; part < DSPLIT; ++part) {
-            if (part == half) {
-#pragma unroll
-              for (int tg = 0; tg < 2; ++tg) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) total[tg][j] += s[tg][j];
-              }
-            } else {
-              pair_wait(&s_pair_flags[0][first_wave + part], pair_step);
-              __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-              const float* theirs = reinterpret_cast<const float*>(&s_tiles[first_wave + part][0]);
-#pragma unroll
-              for (int tg = 0; tg < 2; ++tg) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) total[tg][j] += theirs[(4 * tg + j) * kWave + lane];
-              }
-            }
-          }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the reads above are done before the others hear
-          if (lane == 0)
-            __hip_atomic_store(&s_pair_flags[1][wave], pair_step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-#pragma unroll
-          for (int tg = 0; tg < 2; ++tg) {
-            const float4_t sc = *reinterpret_cast<const float4_t*>(ksc + 16 * tg + 4 * lk);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) s[tg][j] = sc[j] == kNegInf ? kNegInf : total[tg][j] * sc[j];
-          }
+        char* dst = cache + dst_row * row_bytes + sub * EPU;
+        if constexpr (EPU == 4) {
+          *reinterpret_cast<uint32_t*>(dst) = word;
+        } else {
+          *reinterpret_cast<uint16_t*>(dst) = static_cast<uint16_t>(word);
         }
+        if (sub == 0) static_cast<scale_raw_t*>(const_cast<void*>(is_v ? p.v_scale : p.k_scale))[dst_row] = raw;
+      } else {
+        // 16-bit pages hold the update row as it is (the launcher only fuses when the dtypes agree)
+        char* dst = cache + dst_row * row_bytes + sub * (EPU * 2);
+#pragma unroll
+        for (int w = 0; w < UPW; ++w) *reinterpret_cast<uint32_t*>(dst + 4 * w) = upd[SET][w];
+#pragma unroll
+        for (int e = 0; e < EPU; ++e) xhat[e] = x[e];
+      }
+      // both rows as floats where the V tile is (no tile is staged at this point): K row, then V row
+      float* rowbuf = reinterpret_cast<float*>(v_tile);
+#pragma unroll
+      for (int e = 0; e < EPU; ++e) rowbuf[(is_v ? D : 0) + sub * EPU + e] = xhat[e];
+      lds_fence();
+      // score of the token for column lr: this lane's 8 elements of every k-slice, then the four lanes of the column
+      float dot = 0.0f;
+#pragma unroll
+      for (int sl = 0; sl < NS; ++sl) {
+        const float* kk = rowbuf + slice_base(sl);
+        const uint4_t qw = __builtin_bit_cast(uint4_t, qop[sl]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const Pair pr = __builtin_bit_cast(Pair, static_cast<uint32_t>(qw[j]));
+          dot += static_cast<float>(pr.x) * kk[2 * j] + static_cast<float>(pr.y) * kk[2 * j + 1];
+        }
+      }
+      const float s_new = rows_sum(dot) * p.scale_log2e;
+      const float m_new = max_f32(m_run, s_new);
+      const float alpha = fast_exp2(m_run - m_new);  // m_run = -inf for a row without cached tokens -> 0
+      const float pn = fast_exp2(s_new - m_new);
+      m_run = m_new;
+      l_run = l_run * alpha + (lk == 0 ? pn : 0.0f);
+      p_sum *= alpha;
+      const float pv = pn * kPScale;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        const float4_t vv = *reinterpret_cast<const float4_t*>(rowbuf + D + 16 * nb + 4 * lk);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[nb][j] = acc[nb][j] * alpha + pv * vv[j];
+      }
+      lds_fence();
+    }
+  };
 
-        // -- online softmax for head lr over the tile's 32 tokens ---------------------------------------------------
-        float mt = max3_f32(max3_f32(s[0][0], s[0][1], s[0][2]), max3_f32(s[0][3], s[1][0], s[1][1]),
-                            max_f32(s[1][2], s[1][3]));
-        mt = rows_max(mt);
-        const float m_new = max_f32(m_run, mt);
-        const float m_safe = m_new == kNegInf ? 0.0f : m_new;
-        const float alpha = fast_exp2(m_run - m_safe);
-        m_run = m_new;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-          l_run *= alpha;
-          p_sum *= alpha;
+  // ---- one regular tile: stage V and the scales, scores, softmax, P.V ----------------------------------------------
+  // `between_v` runs once the V registers of the set are free, `between_k` once the K registers are.
+  auto tile_step = [&](auto set_c, const TileDesc& t, auto&& between_v, auto&& between_k) {
+    constexpr int SET = decltype(set_c)::value;
+    if constexpr (DSPLIT > 1) {
+      // the other waves of the head must have read the score part this wave parked in the previous step
 #pragma unroll
-          for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[nb][j] *= alpha;
-          }
-        }
-        uint32_t pw[4];
-        {
-          const float4_t vs0 = *reinterpret_cast<const float4_t*>(vsc + 4 * lk);
-          const float4_t vs1 = *reinterpret_cast<const float4_t*>(vsc + 16 + 4 * lk);
-          float pe[8];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float e0 = fast_exp2(s[0][j] - m_safe);
-            const float e1 = fast_exp2(s[1][j] - m_safe);
-            l_run += e0 + e1;
-            pe[j] = e0 * vs0[j];
-            pe[4 + j] = e1 * vs1[j];
-          }
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            pw[j] = pack_pair<KIND>(pe[2 * j], pe[2 * j + 1]);
-            if constexpr (KIND == KV_I8) {
-              const Pair pr = __builtin_bit_cast(Pair, pw[j]);
-              p_sum += static_cast<float>(pr.x) + static_cast<float>(pr.y);
-            }
-          }
-        }
-        const V8 pop = __builtin_bit_cast(V8, uint4_t{pw[0], pw[1], pw[2], pw[3]});
-
-        // -- O^T += V^T . P^T, one MFMA per 16-dim block -------------------------------------------------------------
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          uint32_t vw[4];
-          if constexpr (ES == 1) {
-            // lane i of a 16-lane group supplies row (i / 2), 8 bytes at column 16 nb + 8 (i % 2)
-            const int r8 = lr >> 1;
-            const int tok = r8 < 4 ? 4 * lk + r8 : 16 + 4 * lk + (r8 - 4);
-            char* a = v_tile + v_row_of(tok) * RSV + 16 * nb + 8 * (lr & 1);
-            const int2_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_int2*)a);
-            vw[0] = static_cast<uint32_t>(r[0]);
-            vw[1] = static_cast<uint32_t>(r[1]);
-          } else {
-            // lane i supplies row (i / 4), 4 elements at column 16 nb + 4 (i % 4); two reads of 4 tokens each
-            const int r4 = lr >> 2;
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-              const int tok = 16 * half + 4 * lk + r4;
-              char* a = v_tile + v_row_of(tok) * RSV + (16 * nb + 4 * (lr & 3)) * 2;
-              const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
-              const uint2_t u = __builtin_bit_cast(uint2_t, r);
-              vw[2 * half] = u[0];
-              vw[2 * half + 1] = u[1];
-            }
-          }
-          acc[nb] = Ops::mfma(to_operand<KIND>(vw), pop, acc[nb]);
-        }
-        // all LDS reads of this tile are done before the next iteration overwrites it
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-
-        // -- end of a sequence's share: emit its partial and switch to the next sequence ---------------------------
-        const bool last_of_piece = x + 1 == x1;
-        if (next_is_new_seq || last_of_piece) {
-          write_partial(cp_b, cp_row, cp_nseq);
-          if (!last_of_piece) {
-            cp_b = kv_cur.b;
-            cp_row = kv_cur.row;
-            cp_nseq = kv_cur.nseq;
-            adopt_q();
-            reset_state();
-          }
-        }
-        cp_tok = kv_cur.tok;
-        cp_end = kv_cur.end;
+      for (int part = 0; part < DSPLIT; ++part) {
+        if (part != half) pair_wait(&s_pair_flags[1][wave - half + part], pair_step);
       }
     }
-#ifdef ARENO_TRACE
-    if (mp.trace && lane == 0) mp.trace[trace_wave * 16 + 1] = wall_clock64();
-#endif
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        uint4_t vv = vreg[SET][tg * CPL + j];
+        if constexpr (KIND == KV_I8) {
+#pragma unroll
+          for (int w = 0; w < 4; ++w) vv[w] ^= kI8Flip;
+        }
+        *reinterpret_cast<uint4_t*>(v_tile + tg * TGS + chunk_row_pos(lk + 4 * j, lr)) = vv;
+      }
+    }
+    if constexpr (T::kQuant) {
+      const bool ok = t.tok + (lane & 31) < t.end;
+      const float s = scale_value(sreg[SET]);
+      sc_lds[lane] = lane < 32 ? (ok ? s * p.scale_log2e : kNegInf) : (ok ? s * kPScale : 0.0f);
+    }
+    lds_fence();
+    between_v();
+
+    // -- S^T = K . Q^T for the two 16-token groups ------------------------------------------------------------------
+    float s[2][4];
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+      float4_t c = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int sl = 0; sl < NS; ++sl) {
+        uint32_t w[WPS];
+#pragma unroll
+        for (int i = 0; i < WPS; ++i) {
+          const int word = sl * WPS + i;  // dword of this lane's row part, in load order
+          w[i] = kreg[SET][tg * CPL + word / 4][word % 4];
+          if constexpr (KIND == KV_I8) w[i] ^= kI8Flip;
+        }
+        c = Ops::mfma(to_operand<KIND>(w), qop[sl], c);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[tg][j] = c[j] - qbias;  // (this wave's part of) the dot products
+    }
+    between_k();
+    if constexpr (DSPLIT > 1) {
+      // Park the part, tell the other waves of the head, wait for their parts, add all parts in the order of the head
+      // dimension.  Every wave of the head ends up with the same eight sums.
+#pragma unroll
+      for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) park[(4 * tg + j) * kWave + lane] = s[tg][j];
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      ++pair_step;
+      if (lane == 0)
+        __hip_atomic_store(&s_pair_flags[0][wave], pair_step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      const int first_wave = wave - half;
+      float total[2][4];
+#pragma unroll
+      for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) total[tg][j] = 0.0f;
+      }
+#pragma unroll
+      for (int part = 0; part < DSPLIT; ++part) {
+        if (part == half) {
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) total[tg][j] += s[tg][j];
+          }
+        } else {
+          pair_wait(&s_pair_flags[0][first_wave + part], pair_step);
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+          const float* theirs = reinterpret_cast<const float*>(&s_tiles[first_wave + part][2 * TGS + 2 * TK * 4]);
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) total[tg][j] += theirs[(4 * tg + j) * kWave + lane];
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the reads above are done before the others hear
+      if (lane == 0)
+        __hip_atomic_store(&s_pair_flags[1][wave], pair_step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+#pragma unroll
+      for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[tg][j] = total[tg][j];
+      }
+    }
+    // the per-token K scale (softmax scale and log2 e folded in); tokens past the end stay exactly -inf
+    float vs[2][4];
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+      if constexpr (T::kQuant) {
+        const float4_t ks = *reinterpret_cast<const float4_t*>(sc_lds + 16 * tg + 4 * lk);
+        const float4_t vv = *reinterpret_cast<const float4_t*>(sc_lds + 32 + 16 * tg + 4 * lk);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          s[tg][j] = ks[j] == kNegInf ? kNegInf : s[tg][j] * ks[j];
+          vs[tg][j] = vv[j];
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bool ok = t.tok + 16 * tg + 4 * lk + j < t.end;
+          s[tg][j] = ok ? s[tg][j] * p.scale_log2e : kNegInf;
+          vs[tg][j] = 1.0f;
+        }
+      }
+    }
+
+    // -- online softmax for column lr over the tile's 32 tokens ------------------------------------------------------
+    float mt = max3_f32(max3_f32(s[0][0], s[0][1], s[0][2]), max3_f32(s[0][3], s[1][0], s[1][1]),
+                        max_f32(s[1][2], s[1][3]));
+    mt = rows_max(mt);
+    const float m_new = max_f32(m_run, mt);
+    const float m_safe = m_new == kNegInf ? 0.0f : m_new;
+    const float alpha = fast_exp2(m_run - m_safe);
+    m_run = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+      l_run *= alpha;
+      p_sum *= alpha;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[nb][j] *= alpha;
+      }
+    }
+    uint32_t pw[4];
+    {
+      float pe[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float e0 = fast_exp2(s[0][j] - m_safe);
+        const float e1 = fast_exp2(s[1][j] - m_safe);
+        l_run += e0 + e1;
+        pe[j] = T::kQuant ? e0 * vs[0][j] : e0;
+        pe[4 + j] = T::kQuant ? e1 * vs[1][j] : e1;
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        pw[j] = pack_pair<KIND>(pe[2 * j], pe[2 * j + 1]);
+        if constexpr (KIND == KV_I8) {
+          const Pair pr = __builtin_bit_cast(Pair, pw[j]);
+          p_sum += static_cast<float>(pr.x) + static_cast<float>(pr.y);
+        }
+      }
+    }
+    const V8 pop = __builtin_bit_cast(V8, uint4_t{pw[0], pw[1], pw[2], pw[3]});
+
+    // -- O^T += V^T . P^T, one MFMA per 16-dim block -----------------------------------------------------------------
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      uint32_t vw[4];
+      if constexpr (ES == 1) {
+        // lane i of a 16-lane group supplies token row (i / 2), 8 bytes at column 8 (i % 2) of chunk nb: rows 0..3 are
+        // tokens 4 lk .. 4 lk + 3 of group 0, rows 4..7 the same tokens of group 1
+        const int r8 = lr >> 1;
+        const int tg = r8 >> 2;
+        const int tok = 4 * lk + (r8 & 3);
+        char* a = v_tile + tg * TGS + chunk_row_pos(nb, tok) + 8 * (lr & 1);
+        const int2_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_int2*)a);
+        vw[0] = static_cast<uint32_t>(r[0]);
+        vw[1] = static_cast<uint32_t>(r[1]);
+      } else {
+        // lane i supplies token row (i / 4), 4 elements at column 4 (i % 4) of the 16-dim block: chunk 2 nb + (i % 4) / 2,
+        // byte 8 ((i % 4) % 2); two reads of 4 tokens, one per token group
+        const int r4 = lr >> 2;
+        const int c4 = lr & 3;
+#pragma unroll
+        for (int tg = 0; tg < 2; ++tg) {
+          char* a = v_tile + tg * TGS + chunk_row_pos(2 * nb + (c4 >> 1), 4 * lk + r4) + 8 * (c4 & 1);
+          const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
+          const uint2_t u = __builtin_bit_cast(uint2_t, r);
+          vw[2 * tg] = u[0];
+          vw[2 * tg + 1] = u[1];
+        }
+      }
+      acc[nb] = Ops::mfma(to_operand<KIND>(vw), pop, acc[nb]);
+    }
+    // all LDS reads of this tile are done before the next step overwrites it
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
+
+  // ---- this wave's unit --------------------------------------------------------------------------------------------
+  unit = blockIdx.x * mp.tok_splits + ts;
+  const int x0 = geo.unit_start(unit);
+  const int x1 = geo.unit_start(unit + 1);
+  if (x0 < x1) {
+    // ---- prologue: block ids of the first DEPTH + 1 tiles one after the other, Q of the first item, the first
+    // DEPTH tiles' loads ----------------------------------------------------------------------------------------------
+    cursor_seek<GROUPED>(cur, shape, lens, cum, x0);
+    desc_ids = describe(cur, true);
+    issue_id_loads(desc_ids);
+    issue_q_loads(desc_ids);
+    auto request_next = [&](int x_next) {
+      // move the request cursor to tile x_next and ask for its block ids
+      const bool opens = cursor_advance<GROUPED>(cur, shape, lens, cum, x_next);
+      desc_ids = describe(cur, opens);
+      issue_id_loads(desc_ids);
+    };
+    auto issue_tile = [&](auto set_c, int x_after) {
+      // the tile whose ids have arrived goes out into register set SET; then the ids of tile x_after are requested
+      constexpr int SET = decltype(set_c)::value;
+      rows_from_ids(desc_ids);
+      desc[SET] = desc_ids;
+      if (x_after < x1) request_next(x_after);
+      issue_v_loads(set_c, desc[SET]);
+      issue_k_loads(set_c, desc[SET]);
+    };
+    issue_tile(std::integral_constant<int, 0>{}, x0 + 1);
+    if constexpr (DEPTH == 2) {
+      if (x0 + 1 < x1) issue_tile(std::integral_constant<int, 1>{}, x0 + 2);
+    }
+    adopt_q();
+    reset_state();
+    bool q_pending = false;  // qraw holds the Q of the item that the next tile opens
+
+    auto step = [&](auto set_c, int x) {
+      constexpr int SET = decltype(set_c)::value;
+      ARENO_TRACE_POINT();
+      const TileDesc t = desc[SET];
+      // tile x + DEPTH: its ids were requested a step ago; its loads go out as this tile's registers become free
+      const bool more = x + DEPTH < x1;
+      TileDesc nt = t;
+      if (more) {
+        rows_from_ids(desc_ids);
+        nt = desc_ids;
+        if (x + DEPTH + 1 < x1) request_next(x + DEPTH + 1);
+      }
+      if (t.kind & kTileNewToken) {
+        new_token_step(set_c, t);
+        if (more) {
+          issue_v_loads(set_c, nt);
+          issue_k_loads(set_c, nt);
+        }
+      } else {
+        tile_step(
+            set_c, t, [&]() { if (more) issue_v_loads(set_c, nt); }, [&]() { if (more) issue_k_loads(set_c, nt); });
+      }
+      if (more) desc[SET] = nt;
+      // -- end of an item's share: emit its partial and switch to the next item -------------------------------------
+      const bool last_of_unit = x + 1 == x1;
+      const TileDesc& next = DEPTH == 1 ? nt : desc[DEPTH == 1 ? 0 : 1 - SET];  // tile x + 1
+      const bool next_opens = !last_of_unit && (next.kind & kTileOpens);
+      if (next_opens || last_of_unit) {
+        write_partial(t.b, t.row, t.nseq);
+        if (!last_of_unit) {
+          if (!q_pending) issue_q_loads(next);  // an item of one tile right behind another: its Q was not asked for yet
+          adopt_q();
+          reset_state();
+          q_pending = false;
+        }
+      }
+      // Q of the item that tile x + 2 opens: a step of lead
+      if (x + 2 < x1) {
+        const TileDesc& ahead = DEPTH == 1 ? desc_ids : nt;  // tile x + 2
+        if (ahead.kind & kTileOpens) {
+          issue_q_loads(ahead);
+          q_pending = true;
+        }
+      }
+    };
+    // Q of the item tile x0 + 1 opens (tile x0 + 2's is asked for by the first step)
+    if (x0 + 1 < x1) {
+      const TileDesc& second = DEPTH == 1 ? desc_ids : desc[DEPTH - 1];
+      if (second.kind & kTileOpens) {
+        issue_q_loads(second);
+        q_pending = true;
+      }
+    }
+    for (int x = x0; x < x1; x += DEPTH) {
+      step(std::integral_constant<int, 0>{}, x);
+      if constexpr (DEPTH == 2) {
+        if (x + 1 < x1) step(std::integral_constant<int, 1>{}, x + 1);
+      }
+    }
   }
+#ifdef ARENO_TRACE
+  if (mp.trace && lane == 0) mp.trace[trace_wave * 8 + 6] = wall_clock64();
+#endif
 }
 
 typedef void (*decode_mfma_fn)(MfmaDecodeParams);

@@ -7,6 +7,14 @@
 
 #include "../../include/areno_hip.h"
 
+// The kernels are written against two code-generation flags that only the build script passes, together with this
+// define: -fno-honor-nans (maxima as bare v_max_f32 / v_max3_f32; inputs may hold NaN in slots no query may see, the
+// kernels neither produce nor test for NaN) and packed-FP32 VALU forms off.  A build without them would compile and
+// give different code for every maximum, so it is refused here.
+#if !defined(ARENO_DEVICE_FLAGS_OK)
+#error "build areno_amd/csrc through setup.py: it needs -fno-honor-nans and -Xclang -target-feature -Xclang -packed-fp32-ops (HIP_DEVICE_FLAGS)"
+#endif
+
 namespace areno {
 
 constexpr int kWave = 64;

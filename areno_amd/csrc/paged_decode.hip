@@ -143,21 +143,22 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   const int b = row / p.q_heads;
   const int h = row - b * p.q_heads;
   const int d = p.head_dim;
-  const int num_items = mp.num_shared + p.batch;
+  const ItemShape& shape = mp.items;
+  const int num_items = shape.num_items();
   // the plan entries this row needs, fetched together (their indices follow from the row alone)
-  const int v_own = mp.num_shared + b;
+  const int v_own = shape.num_shared + b;
   const int plan_total = mp.plan[num_items], plan_own = mp.plan[v_own], plan_own_end = mp.plan[v_own + 1];
-  const UnitGeometry geo = make_unit_geometry(plan_total, mp.num_pieces, mp.max_small, mp.static_share, mp.min_unit_tiles);
+  const UnitGeometry geo = make_unit_geometry(plan_total, mp.num_units);
   // the row's own item (always at least one tile) ...
   const int own_lo = geo.unit_of(plan_own);
   const int own_n = geo.unit_of(plan_own_end - 1) - own_lo + 1;
   // ... and the shared item of its sub-group, if it has tiles
   int sh_lo = 0, sh_n = 0, sh_item = 0, sh_col = 0;
-  if (mp.num_shared > 0) {
-    const int gi = b / mp.group_rows;
-    const int j = (b - gi * mp.group_rows) / mp.cols_seqs;
-    sh_item = gi * mp.subs_per_group + j;
-    const int first_row = gi * mp.group_rows + j * mp.cols_seqs;
+  if (shape.num_shared > 0) {
+    const int gi = b / shape.group_rows;
+    const int j = (b - gi * shape.group_rows) / shape.cols_seqs;
+    sh_item = gi * shape.subs_per_group + j;
+    const int first_row = gi * shape.group_rows + j * shape.cols_seqs;
     const int kvh = h / p.group;
     sh_col = kvh * 16 + (b - first_row) * p.group + (h - kvh * p.group);
     if (mp.plan[sh_item + 1] > mp.plan[sh_item]) {
@@ -253,9 +254,8 @@ reduce_slots_fn reduce_slots_kernel_for(int head_dim) {
 
 // ---- geometry of the MFMA path ----------------------------------------------------------------------
 constexpr int kMfmaWaves = ARENO_MFMA_NW;  // waves per workgroup
-constexpr int kMfmaWorkgroups = 512;       // big units: two resident workgroups on each of the 256 CUs
-constexpr int kMfmaTailWorkgroups = 256;   // small units behind them in the grid
-constexpr int kMfmaMaxPieces = (kMfmaWorkgroups + kMfmaTailWorkgroups) * kMfmaWaves;
+constexpr int kMfmaWorkgroups = 512;       // two resident workgroups on each of the 256 CUs
+constexpr int kMfmaMaxUnits = kMfmaWorkgroups * kMfmaWaves;  // one kv head, every wave a unit of its own
 
 size_t mfma_partial_bytes(size_t slots, int q_heads, int head_dim) {
   const size_t bytes = slots * q_heads * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
@@ -263,17 +263,15 @@ size_t mfma_partial_bytes(size_t slots, int q_heads, int head_dim) {
 }
 
 size_t mfma_workspace_bytes(int batch, int q_heads, int head_dim) {
-  const size_t slots = static_cast<size_t>(kMfmaMaxPieces) + batch;
+  const size_t slots = static_cast<size_t>(kMfmaMaxUnits) + batch;
   const size_t plan_words = (static_cast<size_t>(batch) + 1 + 63) / 64 * 64;
   return mfma_partial_bytes(slots, q_heads, head_dim) + plan_words * sizeof(int32_t);
 }
 
-int env_int(const char* name, int fallback) {
-  const char* v = getenv(name);
-  return v != nullptr ? atoi(v) : fallback;
-}
+// "valu" forces the vector-ALU split kernel (a diagnosis switch), anything else prefers the matrix-core kernel.
+// Per-wave timestamps of the split kernel; set through areno_hip_debug_set_trace in ARENO_TRACE builds only.
+unsigned long long* g_trace_buffer = nullptr;
 
-// "valu" forces the vector-ALU split kernel, "mfma" (default) prefers the matrix-core kernel where it applies.
 bool prefer_mfma() {
   static const int choice = [] {
     const char* v = getenv("ARENO_DECODE_KERNEL");
@@ -339,29 +337,28 @@ extern "C" int areno_hip_paged_decode(const areno_paged_cache* cache, const void
 namespace areno {
 namespace {
 
-// Sub-groups of a prefix group that can sit side by side in the 16 MFMA columns, or 0 when grouping does not apply.
-int shared_items_for(int batch, int group, int group_rows, int* cols_seqs, int* subs_per_group) {
-  const int cs = group > 0 ? 16 / group : 0;
-  if (group_rows < 2 || cs < 2 || batch % group_rows != 0) return 0;
-  *cols_seqs = cs;
-  *subs_per_group = (group_rows + cs - 1) / cs;
-  return batch / group_rows * *subs_per_group;
-}
-
-// Units (wave pieces) the split kernel can use at most for a kv-head count: what the partial regions are sized for.
-int max_units_for(int kv_heads) {
-  const int heads_per_wg = kv_heads % 4 == 0 ? 4 : (kv_heads % 2 == 0 ? 2 : 1);
-  const int head_groups = kv_heads / heads_per_wg;
-  const int tok_splits = kMfmaWaves / heads_per_wg;
-  const int wgs = (kMfmaWorkgroups + kMfmaTailWorkgroups) / head_groups;
-  return (wgs > 0 ? wgs : 1) * tok_splits + (kMfmaTailWorkgroups / head_groups) * tok_splits;
+// Units (one per wave) the split kernel uses for a kv-head count and head dim: what the partial regions are indexed by.
+struct MfmaGrid {
+  int waves, head_split, heads_per_wg, head_groups, tok_splits, workgroups, units;
+};
+MfmaGrid mfma_grid_for(int kv_heads, int head_dim) {
+  MfmaGrid g;
+  g.waves = decode_mfma_waves(head_dim);
+  g.head_split = decode_mfma_head_split(head_dim);
+  const int heads = g.waves / g.head_split;  // kv heads a workgroup can serve at once
+  g.heads_per_wg = (heads >= 4 && kv_heads % 4 == 0) ? 4 : ((heads >= 2 && kv_heads % 2 == 0) ? 2 : 1);
+  g.head_groups = kv_heads / g.heads_per_wg;
+  g.tok_splits = heads / g.heads_per_wg;
+  g.workgroups = kMfmaWorkgroups / g.head_groups > 0 ? kMfmaWorkgroups / g.head_groups : 1;
+  g.units = g.workgroups * g.tok_splits;
+  return g;
 }
 
 // plan of the grouped item list (up to one shared item per row on top of the rows), kept 256-byte granular
 size_t grouped_plan_bytes(int batch) { return ((2 * static_cast<size_t>(batch) + 64) * sizeof(int32_t) + 255) / 256 * 256; }
 
 size_t shared_region_bytes(int kv_heads, int head_dim, int num_shared) {
-  const size_t slots = static_cast<size_t>(max_units_for(kv_heads)) + num_shared;
+  const size_t slots = static_cast<size_t>(mfma_grid_for(kv_heads, head_dim).units) + num_shared;
   return slots * kv_heads * 16 * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
 }
 
@@ -451,8 +448,11 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
 
   // ---- matrix-core path: 16-bit or 8-bit caches, head_dim 64/128/256, up to 16 q heads per kv head --------
   decode_mfma_fn mfma = nullptr;
-  if (aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && num_splits != 1 && p.group <= 16 &&
-      batch <= kMfmaMaxBatch) {
+  // the kernel indexes cache rows (block, slot, head) with 32 bits
+  const bool rows_fit = static_cast<double>(cache->num_blocks) * cache->block_size * cache->kv_heads < 4294967296.0;
+  const bool mfma_ok = aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && num_splits != 1 && p.group <= 16 &&
+                       batch <= kMfmaMaxBatch && rows_fit;
+  if (mfma_ok) {
     const bool s16 = cache->scale_dtype == ARENO_DT_F16;
     const bool grouped = num_shared > 0;
     switch (cache->cache_dtype) {
@@ -467,8 +467,7 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     // no grouped kernel for this shape: the plain matrix-core kernel, every row reading its own pages
     num_shared = 0;
     const bool s16 = cache->scale_dtype == ARENO_DT_F16;
-    if (aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && num_splits != 1 && p.group <= 16 &&
-        batch <= kMfmaMaxBatch) {
+    if (mfma_ok) {
       switch (cache->cache_dtype) {
         case ARENO_DT_BF16: mfma = decode_mfma_lookup_bf16(p.head_dim, s16, false); break;
         case ARENO_DT_F16: mfma = decode_mfma_lookup_f16(p.head_dim, s16, false); break;
@@ -479,16 +478,15 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     }
   }
   if (mfma == nullptr) num_shared = 0;  // the other kernels read every row's pages on their own
-  // waves per head in the matrix-core kernel: a 256-wide head is shared by two
-  const int head_split = mfma != nullptr ? decode_mfma_head_split(p.head_dim) : 1;
-  // ---- append: folded into the matrix-core split kernel when it can take the new rows as they are, else a launch of
-  // its own in front ------------------------------------------------------------------------------------------------
-  static const bool allow_fused_append = env_int("ARENO_FUSED_APPEND", 1) != 0;
+  const MfmaGrid grid = mfma_grid_for(cache->kv_heads, p.head_dim);
+  // ---- append: rides along in the matrix-core split kernel as a tile of its own per row when the kernel can take the
+  // new rows as they are (one wave per head, 16-bit pages of the query's dtype or 8-bit pages), else a launch of its
+  // own in front ------------------------------------------------------------------------------------------------------
   const bool fuse_append =
-      mfma != nullptr && allow_fused_append && k_update != nullptr && v_update != nullptr &&
-      (stages & ARENO_STAGE_APPEND) && (stages & ARENO_STAGE_SPLIT) &&
-      (is_quantized(cache->cache_dtype) ? head_split == 1 : q_dtype == cache->cache_dtype) &&
-      reinterpret_cast<uintptr_t>(k_update) % 16 == 0 && reinterpret_cast<uintptr_t>(v_update) % 16 == 0;
+      mfma != nullptr && k_update != nullptr && v_update != nullptr && (stages & ARENO_STAGE_APPEND) &&
+      (stages & ARENO_STAGE_SPLIT) && grid.head_split == 1 &&
+      (is_quantized(cache->cache_dtype) || q_dtype == cache->cache_dtype) &&
+      reinterpret_cast<uintptr_t>(k_update) % 8 == 0 && reinterpret_cast<uintptr_t>(v_update) % 8 == 0;
   if (k_update != nullptr && (stages & ARENO_STAGE_APPEND) && !fuse_append) {
     if (int rc = areno_hip_cache_write_decode(cache, k_update, v_update, q_dtype, batch, block_table, max_blocks,
                                               cache_seqlens, stream))
@@ -498,57 +496,37 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
   if (mfma != nullptr) {
     MfmaDecodeParams mp;
     mp.d = p;
-    const int waves = decode_mfma_waves(p.head_dim);
-    if (head_split > 1) {
-      // several waves share a head: fewer kv heads per workgroup
-      const int pairs = waves / head_split;
-      mp.d.heads_per_wg = cache->kv_heads % pairs == 0 ? pairs : (pairs >= 2 && cache->kv_heads % 2 == 0 ? 2 : 1);
-    }
-    const int head_groups = cache->kv_heads / mp.d.heads_per_wg;
-    static const int wgs = [] {
-      const int v = env_int("ARENO_MFMA_WGS", kMfmaWorkgroups);
-      return v > 0 && v <= kMfmaWorkgroups + kMfmaTailWorkgroups ? v : kMfmaWorkgroups;
-    }();
-    static const int tail_wgs = [] {
-      const int v = env_int("ARENO_MFMA_TAIL_WGS", 0);
-      return v >= 0 && v <= kMfmaTailWorkgroups ? v : kMfmaTailWorkgroups;
-    }();
-    static const int static_share = env_int("ARENO_MFMA_STATIC", 256);
-    static const int unit_tiles = env_int("ARENO_MFMA_UNIT", 4);
-    mp.static_wgs = wgs / head_groups > 0 ? wgs / head_groups : 1;
-    const int extra = tail_wgs / head_groups;
-    mp.tok_splits = waves / (mp.d.heads_per_wg * head_split);
-    mp.num_pieces = mp.static_wgs * mp.tok_splits;
-    mp.max_small = extra * mp.tok_splits;
-    mp.static_share = static_share;
-    mp.min_unit_tiles = unit_tiles;
+    mp.d.heads_per_wg = grid.heads_per_wg;
+    mp.tok_splits = grid.tok_splits;
+    mp.num_units = grid.units;
+    mp.items.batch = batch;
+    mp.items.window_left = window_left;
+    mp.items.new_token_tile = fuse_append ? 1 : 0;
+    mp.items.num_shared = num_shared;
+    mp.items.group_rows = num_shared > 0 ? group_rows : 1;
+    mp.items.cols_seqs = num_shared > 0 ? cols_seqs : 1;
+    mp.items.subs_per_group = num_shared > 0 ? subs_per_group : 1;
     mp.k_update = fuse_append ? k_update : nullptr;
     mp.v_update = fuse_append ? v_update : nullptr;
-#ifdef ARENO_TRACE
-    mp.trace = getenv("ARENO_TRACE_BUF") ? reinterpret_cast<unsigned long long*>(strtoull(getenv("ARENO_TRACE_BUF"), nullptr, 0)) : nullptr;
-#endif
-    const size_t slots = static_cast<size_t>(mp.num_pieces) + mp.max_small + batch;
+    mp.trace = g_trace_buffer;
+    const size_t slots = static_cast<size_t>(grid.units) + batch;
     const size_t part_bytes = mfma_partial_bytes(slots, q_heads, p.head_dim);
     mp.d.part_ml = static_cast<float*>(workspace);
     mp.d.part_acc = mp.d.part_ml + slots * q_heads * 2;
     mp.plan = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + part_bytes);
     mp.shared_lens = shared_lens;
-    mp.group_rows = num_shared > 0 ? group_rows : 1;
-    mp.cols_seqs = num_shared > 0 ? cols_seqs : 1;
-    mp.subs_per_group = num_shared > 0 ? subs_per_group : 1;
-    mp.num_shared = num_shared;
     mp.shared_ml = nullptr;
     mp.shared_acc = nullptr;
     if (num_shared > 0) {
       // behind the ungrouped layout: the (longer) plan of the item list, then the shared partial region
       mp.plan = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + base_need);
       char* region = static_cast<char*>(workspace) + base_need + plan_extra;
-      const size_t shared_slots = static_cast<size_t>(mp.num_pieces) + mp.max_small + num_shared;
+      const size_t shared_slots = static_cast<size_t>(grid.units) + num_shared;
       mp.shared_ml = reinterpret_cast<float*>(region);
       mp.shared_acc = mp.shared_ml + shared_slots * cache->kv_heads * 16 * 2;
     }
     if (stages & ARENO_STAGE_SPLIT) {
-      hipLaunchKernelGGL(mfma, dim3(mp.static_wgs + extra, head_groups), dim3(waves * kWave), 0, s, mp);
+      hipLaunchKernelGGL(mfma, dim3(grid.workgroups, grid.head_groups), dim3(grid.waves * kWave), 0, s, mp);
       if (int rc = check_launch(op)) return rc;
     }
     if (stages & ARENO_STAGE_REDUCE) {
@@ -653,3 +631,10 @@ extern "C" int areno_hip_paged_decode_grouped(const areno_paged_cache* cache, co
                             cache_seqlens, window_left, num_splits, softmax_scale, group_rows, shared_lens, workspace,
                             workspace_bytes, stages, stream);
 }
+
+#ifdef ARENO_TRACE
+// Tuning builds only: a device buffer of [waves][8] 64-bit words that the split kernel fills with its wave timestamps.
+extern "C" void areno_hip_debug_set_trace(void* device_buffer) {
+  areno::g_trace_buffer = static_cast<unsigned long long*>(device_buffer);
+}
+#endif

@@ -44,6 +44,10 @@
 
 namespace areno {
 
+// LDS row that holds tile token t of the V tile: the second half is rotated by 4 rows so that the 8 tokens a
+// lane group reads through the transpose load ({4g..4g+3} and {16+4g..16+4g+3}) sit in rows distinct mod 16.
+__device__ __forceinline__ int v_row_of(int t) { return t < 16 ? t : 16 + ((t + 4) & 15); }
+
 size_t prefill_mfma_workspace_bytes(int32_t kv_heads, int32_t head_dim);
 int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out, int32_t q_dtype, int64_t tokens,
                         int32_t q_heads, int32_t num_seqs, const int32_t* block_table, int32_t max_blocks,

@@ -303,16 +303,22 @@ def cfg2_qwen7b_int8(**kw) -> DecodeWorkload:
     return cfg1_qwen7b("int8", seed=kw.pop("seed", 1002), **kw)
 
 
+def cfg3_lengths(seed: int = 1003, prompts: int = 32, samples: int = 8, prefix_lo=256, prefix_hi=2048, median=1000.0,
+                 sigma=1.0, cap=32768):
+    """The integer draws of the rollout configuration: ``(prefix (prompts,), lengths (prompts * samples,))``."""
+    g = _gen(seed + 1)
+    prefix = _randint(g, prefix_lo, prefix_hi, prompts)
+    cont = torch.exp(torch.randn(prompts * samples, generator=g) * sigma + math.log(median))
+    cont = torch.clamp(cont, max=float(cap)).to(torch.int64)
+    return prefix, prefix.repeat_interleave(samples) + cont
+
+
 def cfg3_rollout(kv: str = "fp8", *, device="cpu", seed: int = 1003, prompts: int = 32, samples: int = 8,
                  prefix_lo=256, prefix_hi=2048, median=1000.0, sigma=1.0, cap=32768, hq: int = 32, hkv: int = 8,
                  **kw) -> DecodeWorkload:  # fmt: skip
     """RL-rollout decode: ``prompts x samples`` rows, samples of a prompt share the prompt's full pages."""
-    g = _gen(seed + 1)
     bs = 16
-    prefix = _randint(g, prefix_lo, prefix_hi, prompts)
-    cont = torch.exp(torch.randn(prompts * samples, generator=g) * sigma + math.log(median))
-    cont = torch.clamp(cont, max=float(cap)).to(torch.int64)
-    lengths = prefix.repeat_interleave(samples) + cont
+    prefix, lengths = cfg3_lengths(seed, prompts, samples, prefix_lo, prefix_hi, median, sigma, cap)
     shared = [int(p) // bs for p in prefix]
     return make_decode_workload(
         f"cfg3-rollout-{kv}", seed=seed, batch=prompts * samples, hq=hq, hkv=hkv, d=128, bs=bs, kv=kv, lengths=lengths,

@@ -210,7 +210,8 @@ def test_prefix_groups_match_the_plain_op_and_the_oracle(kv, hq, hkv, samples):
             dst.copy_(src)
     grouped = _grouped_decode(w)
     assert_close(grouped, expected_decode(w), *tolerances(kv), what=f"grouped {kv} vs oracle")
-    assert_close(grouped, plain.cpu().float(), 2e-3, what=f"grouped {kv} vs plain op")
+    # same math in another summation order: the outputs may differ by one unit of the 16-bit output format
+    assert_close(grouped, plain.cpu().float(), 8e-3, what=f"grouped {kv} vs plain op")
     for a, b, name in zip((w.k_cache, w.v_cache, w.k_scale, w.v_scale), after_plain, ("k", "v", "k_scale", "v_scale")):
         if a is not None:
             same = a.view(torch.uint8) == b.view(torch.uint8)
@@ -244,7 +245,7 @@ def test_cfg3_full_size_grouped():
     for dst, src in zip(pools, on_device):
         dst.copy_(src)
     plain = run_decode(w)
-    assert_close(grouped, plain.cpu().float(), 2e-3, what="cfg3 full size, grouped vs plain op, all rows")
+    assert_close(grouped, plain.cpu().float(), 8e-3, what="cfg3 full size, grouped vs plain op, all rows")
     for a, b, name in zip(pools, after_grouped, ("k", "v", "k_scale", "v_scale")):
         assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"{name}: grouped and plain appends differ"
 
