@@ -82,6 +82,9 @@ def lib() -> ctypes.CDLL:
         decode_args = [_P, _P, _P, _P, _P, _I32, _I32, _I32, _P, _I32, _P, _I32, _I32, _F, _P, _SZ]
         handle.areno_hip_paged_decode.argtypes = decode_args + [_P]
         handle.areno_hip_paged_decode_stages.argtypes = decode_args + [_I32, _P]
+        handle.areno_hip_paged_decode_static.argtypes = decode_args[:-2] + [_P]
+        handle.areno_hip_paged_decode_static_capacity.restype = _SZ
+        handle.areno_hip_paged_decode_static_capacity.argtypes = []
         handle.areno_hip_paged_decode_grouped.argtypes = decode_args[:-2] + [_I32, _P, _P, _SZ, _I32, _P]
         handle.areno_hip_paged_decode_grouped_workspace_bytes.restype = _SZ
         handle.areno_hip_paged_decode_grouped_workspace_bytes.argtypes = [_I32] * 8
@@ -160,6 +163,19 @@ def paged_decode(cache: PagedCache, q, k_update, v_update, out, block_table, cac
         current_stream_ptr() if stream is None else stream,
     )  # fmt: skip
     check(status, "areno_hip_paged_decode")
+
+
+def paged_decode_static(cache: PagedCache, q, k_update, v_update, out, block_table, cache_seqlens, *, window_left=-1,
+                        num_splits=8, softmax_scale=None, stream=None) -> int:  # fmt: skip
+    """``areno_hip_paged_decode_static`` (the decode op on the library's built-in scratch buffer) on raw pointers;
+    returns the status code."""
+    scale = float(softmax_scale if softmax_scale is not None else q.shape[-1] ** -0.5)
+    return int(lib().areno_hip_paged_decode_static(
+        ctypes.byref(cache), q.data_ptr(), None if k_update is None else k_update.data_ptr(),
+        None if v_update is None else v_update.data_ptr(), out.data_ptr(), dtype_code(q), q.shape[0], q.shape[1],
+        block_table.data_ptr(), block_table.shape[1], cache_seqlens.data_ptr(), int(window_left), int(num_splits),
+        scale, current_stream_ptr() if stream is None else stream,
+    ))  # fmt: skip
 
 
 def prefill_workspace_bytes(kv_heads: int, head_dim: int) -> int:

@@ -7,6 +7,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "decode_mfma_kernels.hpp"
 
 namespace areno {
@@ -630,6 +632,74 @@ extern "C" int areno_hip_paged_decode_grouped(const areno_paged_cache* cache, co
   return areno::decode_in_row_ranges(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
                             cache_seqlens, window_left, num_splits, softmax_scale, group_rows, shared_lens, workspace,
                             workspace_bytes, stages, stream);
+}
+
+// ---- the decode op for callers that cannot allocate -----------------------------------------------------------------
+// The split-KV partials of areno_hip_paged_decode_static live in this array instead of a caller workspace.  Every
+// GPU the library runs on holds its own copy, at its own address, until the process ends.  In host code the array's
+// name is only a handle for hipGetSymbolAddress: the device address is looked up once per device and kept, and that
+// pointer is what the kernels receive.
+#define ARENO_STATIC_SCRATCH_BYTES (64u << 20)
+static __device__ __align__(256) unsigned char scratch[ARENO_STATIC_SCRATCH_BYTES];
+
+namespace areno {
+namespace {
+
+constexpr int kMaxScratchDevices = 64;
+
+// Device address of `scratch` on the current device (looked up at the first call on that device), or NULL with the
+// error recorded.
+void* static_scratch(const char* op) {
+  static std::mutex lock;
+  static void* address[kMaxScratchDevices] = {};
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess || device < 0 || device >= kMaxScratchDevices) {
+    fail(ARENO_ERR_LAUNCH, "%s: no current device (%s)", op, hipGetErrorString(err));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> guard(lock);
+  if (address[device] == nullptr) {
+    void* ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr) {
+      fail(ARENO_ERR_LAUNCH, "%s: the built-in scratch buffer has no address on device %d (%s)", op, device,
+           hipGetErrorString(err));
+      return nullptr;
+    }
+    address[device] = ptr;
+  }
+  return address[device];
+}
+
+}  // namespace
+}  // namespace areno
+
+extern "C" size_t areno_hip_paged_decode_static_capacity(void) { return ARENO_STATIC_SCRATCH_BYTES; }
+
+extern "C" int areno_hip_paged_decode_static(const areno_paged_cache* cache, const void* q, const void* k_update,
+                                             const void* v_update, void* out, int32_t q_dtype, int32_t batch,
+                                             int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
+                                             const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
+                                             float softmax_scale, void* stream) {
+  const char* op = "areno_hip_paged_decode_static";
+  if (cache == nullptr) return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: cache is NULL", op);
+  if (batch == 0) return ARENO_OK;
+  const size_t need = areno_hip_paged_decode_workspace_bytes(batch, q_heads, cache->head_dim, cache->block_size,
+                                                             max_blocks, num_splits);
+  if (need == 0) return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: batch/q_heads/head_dim/max_blocks out of range", op);
+  if (need > ARENO_STATIC_SCRATCH_BYTES)
+    return areno::fail(ARENO_ERR_WORKSPACE,
+                       "%s: these shapes need %zu bytes for the split-KV partials, the built-in buffer holds %zu; call "
+                       "areno_hip_paged_decode with a workspace of the caller's",
+                       op, need, static_cast<size_t>(ARENO_STATIC_SCRATCH_BYTES));
+  void* ptr = areno::static_scratch(op);
+  if (ptr == nullptr) return ARENO_ERR_LAUNCH;
+  // every partial, prefix sum and plan entry a launch reads was written earlier in the same launch sequence, so
+  // nothing left by the previous call has to be cleared
+  return areno_hip_paged_decode_stages(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table,
+                                       max_blocks, cache_seqlens, window_left, num_splits, softmax_scale, ptr,
+                                       ARENO_STATIC_SCRATCH_BYTES, ARENO_STAGE_ALL, stream);
 }
 
 #ifdef ARENO_TRACE

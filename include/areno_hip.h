@@ -125,6 +125,24 @@ int areno_hip_paged_decode_stages(const areno_paged_cache* cache, const void* q,
                                   size_t workspace_bytes, int32_t stages, void* stream);
 
 /*
+ * areno_hip_paged_decode without a workspace argument, for callers that cannot allocate device memory (code under
+ * HIP stream capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference, whose
+ * launcher allocates its partials with torch (areno/accel/csrc/attention.cu:974-977).  The split-KV partials live in
+ * a buffer built into the library: areno_hip_paged_decode_static_capacity() bytes (64 MiB) of device memory that every
+ * GPU the library is used on holds until the process ends.  Shapes whose
+ * areno_hip_paged_decode_workspace_bytes(...) exceeds the capacity are refused with ARENO_ERR_WORKSPACE.  The call
+ * itself allocates and frees nothing; the first call on a device looks the buffer's address up
+ * (hipGetSymbolAddress) and should be made outside stream capture.  All calls on one GPU share the buffer: calls that
+ * overlap on one GPU (two streams, two threads) race; calls on one stream do not.  Same arguments, results and error
+ * behaviour as areno_hip_paged_decode otherwise.
+ */
+size_t areno_hip_paged_decode_static_capacity(void);
+int areno_hip_paged_decode_static(const areno_paged_cache* cache, const void* q, const void* k_update,
+                                  const void* v_update, void* out, int32_t q_dtype, int32_t batch, int32_t q_heads,
+                                  const int32_t* block_table, int32_t max_blocks, const int32_t* cache_seqlens,
+                                  int32_t window_left, int32_t num_splits, float softmax_scale, void* stream);
+
+/*
  * The decode op for batches whose rows come in prefix groups (the samples of one prompt in an RL rollout share the
  * prompt's pages: identical block ids for the prefix).  Rows [i * group_rows, (i + 1) * group_rows) share the pages
  * of their first shared_lens[i] tokens; the kernel reads those pages once for as many rows as fit side by side in
