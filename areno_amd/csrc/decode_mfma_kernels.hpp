@@ -31,10 +31,13 @@
 //   online softmax in the log2 domain on the C layout of S^T (head = lane % 16, 4 tokens per lane and group); the
 //      per-token K scale multiplies S, the V scale multiplies P (scales travel through 64 floats of LDS per tile).
 //   O^T[dim][head] += V^T . P^T, where P^T *is* the C layout of S^T, so no cross-lane movement of P is needed.
-// 8-bit caches keep two tiles in flight per wave (two register sets, the loop is unrolled over them): a tile is half
-// the bytes of a 16-bit one and it is the bytes in flight that cover the memory latency.  Within a step the V
-// registers are free once the tile is staged and the K registers once the scores are issued, so the loads of the
-// tile two steps ahead go out early in the step.
+// One tile is in flight per wave: the loads of tile x + 1 go out while tile x is computed (V registers are free once
+// the tile is staged, K registers once the scores are issued), the block ids of tile x + 2 in front of them.  The
+// loop over the regular tiles of an item has no branches around loads, so every wait the compiler places counts
+// exactly the loads younger than the one needed.  Measured on the part: with every wave holding a tile in flight the
+// memory system is saturated (a tile takes ~2.6 us to arrive at 6.4 TB/s aggregate), more tiles or waves in flight
+// only lengthen the queues; what a launch loses is its start (work list, block ids, first tile: ~4.5 us) and the
+// spread of the waves' finish times.
 // int8 codes become fp16 by placing (code ^ 0x80) under the exponent byte 0x64 (v_perm): 1152 + code exactly;
 // the offsets are removed algebraically (1152 * sum(q) per head, 1152 * sum(p) per head).  fp8 uses
 // v_cvt_scalef32_pk_f16_fp8 with scale 1 (exact).  bf16 / fp16 caches feed the MFMA directly.
@@ -63,6 +66,13 @@ namespace areno {
 
 #ifndef ARENO_MFMA_NW
 #define ARENO_MFMA_NW 4
+#endif
+// waves per SIMD the register budget of the 8-bit / 16-bit kernels is set for
+#ifndef ARENO_MFMA_QUANT_OCC
+#define ARENO_MFMA_QUANT_OCC 2
+#endif
+#ifndef ARENO_MFMA_WIDE_OCC
+#define ARENO_MFMA_WIDE_OCC 2
 #endif
 
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
@@ -166,9 +176,10 @@ struct TileDesc {
   int row;   // block-table / query row
   int nseq;  // rows side by side (shared items), else 1
   int b;     // item index
-  int kind;  // bit 0: the tile opens its item; bit 1: it holds only the token being appended
+  int x_end; // global index of the item's last tile + 1
+  int kind;  // bit 0: the tile opens its item; bit 1: it holds only the token being appended; bit 2: past the unit
 };
-constexpr int kTileOpens = 1, kTileNewToken = 2;
+constexpr int kTileOpens = 1, kTileNewToken = 2, kTilePhantom = 4;
 
 // DSPLIT > 1 serves heads of DSPLIT * D elements (256 = 2 x 128, 192 = 3 x 64, 512 = 4 x 128): DSPLIT adjacent waves
 // of the workgroup take one part of the head dimension each.  Every wave computes the part of S = K . Q^T over its
@@ -177,7 +188,8 @@ constexpr int kTileOpens = 1, kTileNewToken = 2;
 // head synchronise through two counters each in LDS (part ready / parts consumed); no workgroup barrier is involved,
 // so the heads of one workgroup may run different units.
 template <int KIND, int D, bool SCALE16, int NW, bool GROUPED = false, int DSPLIT = 1>
-__global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodeParams mp) {
+__global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUANT_OCC : ARENO_MFMA_WIDE_OCC) void decode_mfma_kernel(
+    MfmaDecodeParams mp) {
   using T = KVTraits<KIND>;
   using Ops = MfmaOps<KIND>;
   using V8 = typename Ops::vec8;
@@ -190,7 +202,6 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
   constexpr int NS = D / 32;           // QK^T k-slices
   constexpr int NB = D / 16;           // P.V dim blocks
   constexpr int WPS = 8 * ES / 4;      // dwords per k-slice of 8 elements
-  constexpr int DEPTH = ES == 1 ? 2 : 1;  // tiles in flight per wave
   constexpr int TGS = CPT * 256 + 128;    // bytes of one token group of the V tile in LDS (128 of padding behind it)
   constexpr float kPScale = T::kQuant ? 256.0f : 1.0f;
   constexpr int kParkFloats = DSPLIT > 1 ? 8 * kWave : 0;
@@ -213,7 +224,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: the unit's bounds and the loop follow
 #ifdef ARENO_TRACE
   const int trace_wave = (blockIdx.y * gridDim.x + blockIdx.x) * NW + wave;
   int trace_n = 1;
@@ -322,15 +333,18 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
   auto chunk_row_pos = [](int c, int r) { return c * 256 + ((ES == 2 && (c & 1)) ? (r ^ 8) : r) * 16; };
 
   // ---- the pipeline's registers ------------------------------------------------------------------------------------
+  // Every step issues the same loads in the same order whatever the kinds of the tiles involved (only their addresses
+  // differ), so that the waits the compiler places count exactly the loads that are younger than the one needed and
+  // the tiles behind it stay in flight.  Loads that depend on a tile's kind (the update rows of an appended token, the
+  // Q of the next item) are extra loads on rare paths.
   typedef typename std::conditional<SCALE16, uint16_t, float>::type scale_raw_t;
-  uint4_t kreg[DEPTH][2 * CPL], vreg[DEPTH][2 * CPL];
-  scale_raw_t sreg[DEPTH];   // lane l < 32: K scale of tile token l; else V scale of token l - 32
-  uint32_t upd[DEPTH][UPW];  // a new-token tile: the update rows, K in lanes 0..31, V in 32..63
-  uint32_t new_row[DEPTH];   // a new-token tile: cache row (block, slot, head) the token goes to
-  TileDesc desc[DEPTH];
+  uint4_t kreg[2 * CPL], vreg[2 * CPL];
+  scale_raw_t sreg;   // lane l < 32: K scale of tile token l; else V scale of token l - 32
+  uint32_t upd[UPW];  // a new-token tile: the update rows, K in lanes 0..31, V in 32..63
+  uint32_t new_row = 0;   // a new-token tile: cache row (block, slot, head) the token goes to
+  TileDesc desc0;      // the tile whose loads are in the registers
   TileCursor cur;      // the furthest tile requested so far (its block ids are on their way)
   TileDesc desc_ids;   // = that tile
-  int ids[2];          // its block ids, for this lane's token of each group (new-token tile: of the token's page)
 
   auto describe = [&](const TileCursor& c, bool opens) {
     TileDesc t;
@@ -339,61 +353,67 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
     t.row = c.it.row;
     t.nseq = c.it.nseq;
     t.b = c.b;
+    t.x_end = c.x_end;
     t.kind = (opens ? kTileOpens : 0) | (c.on_new_token() ? kTileNewToken : 0);
     return t;
   };
-  auto column_of = [&](int t) { return p.bs_shift >= 0 ? (t >> p.bs_shift) : (t / p.block_size); };
-  auto slot_of = [&](int t) { return p.bs_shift >= 0 ? (t & (p.block_size - 1)) : (t % p.block_size); };
+  // (the launcher sends only page sizes that are powers of two here)
+  auto column_of = [&](int t) { return t >> p.bs_shift; };
+  auto slot_of = [&](int t) { return t & (p.block_size - 1); };
+  // The token whose cache row this lane fetches for group tg: its own token of a regular tile (clamped to the last
+  // cached one); the position being appended for a new-token tile (the row is not used, it only has to exist); one
+  // token for all lanes of a phantom tile (a tile past the unit's end: its loads keep the pipeline's shape and hit
+  // one cache line each).
+  auto lane_token = [&](const TileDesc& t, int tg) {
+    const int own = (t.kind & kTilePhantom) ? 0 : 16 * tg + lr;
+    return (t.kind & kTileNewToken) ? t.end : min(t.tok + own, t.end - 1);
+  };
+  // (block ids and cache rows are pairs of scalars, one per token group, not arrays: an array indexed by a lane-dependent
+  // value would live in scratch memory, and scratch loads count with the global loads and drain the pipeline)
+  struct IdPair {
+    int g0, g1;
+  };
   auto issue_id_loads = [&](const TileDesc& t) {
     const int32_t* table_row = p.block_table + static_cast<int64_t>(t.row) * p.max_blocks;
-    if (t.kind & kTileNewToken) {
-      ids[0] = ids[1] = table_row[column_of(t.end)];  // position L_b = end of the cached tokens
-    } else {
-#pragma unroll
-      for (int tg = 0; tg < 2; ++tg) ids[tg] = table_row[column_of(min(t.tok + 16 * tg + lr, t.end - 1))];
-    }
+    IdPair r;
+    r.g0 = table_row[column_of(lane_token(t, 0))];
+    r.g1 = table_row[column_of(lane_token(t, 1))];
+    return r;
   };
-  // cache row (block, slot, head) of this lane's token of group tg, from the block ids that have arrived
-  uint32_t rows[2];
-  auto rows_from_ids = [&](const TileDesc& t) {
-#pragma unroll
-    for (int tg = 0; tg < 2; ++tg) {
-      const int tok = (t.kind & kTileNewToken) ? t.end : min(t.tok + 16 * tg + lr, t.end - 1);
-      rows[tg] = (static_cast<uint32_t>(ids[tg]) * p.block_size + slot_of(tok)) * p.kv_heads + kvh;
-    }
+  // cache row (block, slot, head) of this lane's token of each group, from the block ids that have arrived
+  uint32_t row_g0 = 0, row_g1 = 0;
+  auto rows_from_ids = [&](const TileDesc& t, const IdPair& src) {
+    row_g0 = (static_cast<uint32_t>(src.g0) * p.block_size + slot_of(lane_token(t, 0))) * p.kv_heads + kvh;
+    row_g1 = (static_cast<uint32_t>(src.g1) * p.block_size + slot_of(lane_token(t, 1))) * p.kv_heads + kvh;
   };
-  auto issue_v_loads = [&](auto set_c, const TileDesc& t) {
-    constexpr int SET = decltype(set_c)::value;
-    if (t.kind & kTileNewToken) {
-      if constexpr (DSPLIT == 1) {
+  auto issue_v_loads = [&](const TileDesc& t) {
+    if constexpr (DSPLIT == 1) {
+      if ((t.kind & (kTileNewToken | kTilePhantom)) == kTileNewToken) {
         const void* src = lane < 32 ? mp.k_update : mp.v_update;
         const int64_t off = (static_cast<int64_t>(t.row) * p.kv_heads + kvh) * D * 2 + (lane & 31) * (UPW * 4);
 #pragma unroll
-        for (int w = 0; w < UPW; ++w) upd[SET][w] = *reinterpret_cast<const uint32_t*>(static_cast<const char*>(src) + off + 4 * w);
-        new_row[SET] = rows[0];
+        for (int w = 0; w < UPW; ++w) upd[w] = *reinterpret_cast<const uint32_t*>(static_cast<const char*>(src) + off + 4 * w);
       }
-      return;
+      new_row = row_g0;
     }
 #pragma unroll
     for (int tg = 0; tg < 2; ++tg) {
-      const char* va = static_cast<const char*>(p.v_cache) + rows[tg] * row_bytes + half_bytes + lk * 16;
+      const char* va = static_cast<const char*>(p.v_cache) + (tg ? row_g1 : row_g0) * row_bytes + half_bytes + lk * 16;
 #pragma unroll
-      for (int j = 0; j < CPL; ++j) vreg[SET][tg * CPL + j] = *reinterpret_cast<const uint4_t*>(va + 64 * j);
+      for (int j = 0; j < CPL; ++j) vreg[tg * CPL + j] = *reinterpret_cast<const uint4_t*>(va + 64 * j);
     }
     if constexpr (T::kQuant) {
-      const uint32_t r = (lk & 1) ? rows[1] : rows[0];
+      const uint32_t r = (lk & 1) ? row_g1 : row_g0;
       const void* sp = lk < 2 ? p.k_scale : p.v_scale;
-      sreg[SET] = static_cast<const scale_raw_t*>(sp)[r];
+      sreg = static_cast<const scale_raw_t*>(sp)[r];
     }
   };
-  auto issue_k_loads = [&](auto set_c, const TileDesc& t) {
-    constexpr int SET = decltype(set_c)::value;
-    if (t.kind & kTileNewToken) return;
+  auto issue_k_loads = [&](const TileDesc& t) {
 #pragma unroll
     for (int tg = 0; tg < 2; ++tg) {
-      const char* ka = static_cast<const char*>(p.k_cache) + rows[tg] * row_bytes + half_bytes + lk * 16;
+      const char* ka = static_cast<const char*>(p.k_cache) + (tg ? row_g1 : row_g0) * row_bytes + half_bytes + lk * 16;
 #pragma unroll
-      for (int j = 0; j < CPL; ++j) kreg[SET][tg * CPL + j] = *reinterpret_cast<const uint4_t*>(ka + 64 * j);
+      for (int j = 0; j < CPL; ++j) kreg[tg * CPL + j] = *reinterpret_cast<const uint4_t*>(ka + 64 * j);
     }
   };
   auto scale_value = [](scale_raw_t raw) -> float {
@@ -411,16 +431,16 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
   uint4_t qraw[NS];
   const int col_seq = GROUPED ? lr / p.group : 0;
   const int col_head = GROUPED ? lr - col_seq * p.group : lr;
-  auto issue_q_loads = [&](const TileDesc& t) {
-    const bool shared = is_shared(t.b);
+  auto issue_q_loads = [&](int item, int row, int nseq) {
+    const bool shared = is_shared(item);
     const int m = shared ? col_seq : 0;
     const int g = shared ? col_head : lr;
-    const bool live = shared ? m < t.nseq : lr < p.group;
+    const bool live = shared ? m < nseq : lr < p.group;
 #pragma unroll
     for (int sl = 0; sl < NS; ++sl) {
       qraw[sl] = uint4_t{0u, 0u, 0u, 0u};
       if (live) {
-        const int64_t idx = (static_cast<int64_t>(t.row + m) * p.q_heads + h0 + g) * DFULL + half * D + slice_base(sl);
+        const int64_t idx = (static_cast<int64_t>(row + m) * p.q_heads + h0 + g) * DFULL + half * D + slice_base(sl);
         qraw[sl] = load16(p.q, idx * 2);
       }
     }
@@ -513,8 +533,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
   };
 
   // ---- the token being appended: quantize, store into the page, fold into the running softmax (vector ALU) ---------
-  auto new_token_step = [&](auto set_c, const TileDesc& t) {
-    constexpr int SET = decltype(set_c)::value;
+  auto new_token_step = [&](const TileDesc& t) {
     if constexpr (DSPLIT == 1) {
       constexpr int EPU = 2 * UPW;  // elements of the row this lane holds: (lane % 32) * EPU ...
       const int sub = lane & 31;
@@ -522,7 +541,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
       float x[EPU];
 #pragma unroll
       for (int w = 0; w < UPW; ++w) {
-        const uint32_t word = upd[SET][w];
+        const uint32_t word = upd[w];
         if (p.q_dtype == ARENO_DT_BF16) {
           x[2 * w] = bf16_bits_to_float(word & 0xffffu);
           x[2 * w + 1] = bf16_bits_to_float(word >> 16);
@@ -531,7 +550,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
           x[2 * w + 1] = f16_bits_to_float(word >> 16);
         }
       }
-      const int64_t dst_row = new_row[SET];
+      const int64_t dst_row = new_row;
       char* cache = static_cast<char*>(const_cast<void*>(is_v ? p.v_cache : p.k_cache));
       float xhat[EPU];  // what a reader of the page sees
       if constexpr (T::kQuant) {
@@ -590,7 +609,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
         // 16-bit pages hold the update row as it is (the launcher only fuses when the dtypes agree)
         char* dst = cache + dst_row * row_bytes + sub * (EPU * 2);
 #pragma unroll
-        for (int w = 0; w < UPW; ++w) *reinterpret_cast<uint32_t*>(dst + 4 * w) = upd[SET][w];
+        for (int w = 0; w < UPW; ++w) *reinterpret_cast<uint32_t*>(dst + 4 * w) = upd[w];
 #pragma unroll
         for (int e = 0; e < EPU; ++e) xhat[e] = x[e];
       }
@@ -631,8 +650,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
 
   // ---- one regular tile: stage V and the scales, scores, softmax, P.V ----------------------------------------------
   // `between_v` runs once the V registers of the set are free, `between_k` once the K registers are.
-  auto tile_step = [&](auto set_c, const TileDesc& t, auto&& between_v, auto&& between_k) {
-    constexpr int SET = decltype(set_c)::value;
+  auto tile_step = [&](const TileDesc& t, auto&& between_v, auto&& between_k) {
     if constexpr (DSPLIT > 1) {
       // the other waves of the head must have read the score part this wave parked in the previous step
 #pragma unroll
@@ -644,7 +662,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
     for (int tg = 0; tg < 2; ++tg) {
 #pragma unroll
       for (int j = 0; j < CPL; ++j) {
-        uint4_t vv = vreg[SET][tg * CPL + j];
+        uint4_t vv = vreg[tg * CPL + j];
         if constexpr (KIND == KV_I8) {
 #pragma unroll
           for (int w = 0; w < 4; ++w) vv[w] ^= kI8Flip;
@@ -654,11 +672,11 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
     }
     if constexpr (T::kQuant) {
       const bool ok = t.tok + (lane & 31) < t.end;
-      const float s = scale_value(sreg[SET]);
+      const float s = scale_value(sreg);
       sc_lds[lane] = lane < 32 ? (ok ? s * p.scale_log2e : kNegInf) : (ok ? s * kPScale : 0.0f);
     }
     lds_fence();
-    between_v();
+    between_v();  // the V registers of the set are free
 
     // -- S^T = K . Q^T for the two 16-token groups ------------------------------------------------------------------
     float s[2][4];
@@ -671,7 +689,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
 #pragma unroll
         for (int i = 0; i < WPS; ++i) {
           const int word = sl * WPS + i;  // dword of this lane's row part, in load order
-          w[i] = kreg[SET][tg * CPL + word / 4][word % 4];
+          w[i] = kreg[tg * CPL + word / 4][word % 4];
           if constexpr (KIND == KV_I8) w[i] ^= kI8Flip;
         }
         c = Ops::mfma(to_operand<KIND>(w), qop[sl], c);
@@ -828,93 +846,89 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_mfma_kernel(MfmaDecodePa
   const int x0 = geo.unit_start(unit);
   const int x1 = geo.unit_start(unit + 1);
   if (x0 < x1) {
-    // ---- prologue: block ids of the first DEPTH + 1 tiles one after the other, Q of the first item, the first
-    // DEPTH tiles' loads ----------------------------------------------------------------------------------------------
+    // move the request cursor to tile x (a phantom past the unit's end) and ask for its block ids
+    IdPair ids;  // block ids of the tile the request cursor is on
+    auto request = [&](int x) {
+      if (x < x1) {
+        const bool opens = cursor_advance<GROUPED>(cur, shape, lens, cum, x);
+        desc_ids = describe(cur, opens);
+      } else {
+        desc_ids.kind = (desc_ids.kind & kTileNewToken) | kTilePhantom;
+      }
+      ids = issue_id_loads(desc_ids);
+    };
+    // ---- prologue: block ids of the first two tiles one behind the other, Q of the first item, the first tile's
+    // loads ------------------------------------------------------------------------------------------------------------
     cursor_seek<GROUPED>(cur, shape, lens, cum, x0);
     desc_ids = describe(cur, true);
-    issue_id_loads(desc_ids);
-    issue_q_loads(desc_ids);
-    auto request_next = [&](int x_next) {
-      // move the request cursor to tile x_next and ask for its block ids
-      const bool opens = cursor_advance<GROUPED>(cur, shape, lens, cum, x_next);
-      desc_ids = describe(cur, opens);
-      issue_id_loads(desc_ids);
-    };
-    auto issue_tile = [&](auto set_c, int x_after) {
-      // the tile whose ids have arrived goes out into register set SET; then the ids of tile x_after are requested
-      constexpr int SET = decltype(set_c)::value;
-      rows_from_ids(desc_ids);
-      desc[SET] = desc_ids;
-      if (x_after < x1) request_next(x_after);
-      issue_v_loads(set_c, desc[SET]);
-      issue_k_loads(set_c, desc[SET]);
-    };
-    issue_tile(std::integral_constant<int, 0>{}, x0 + 1);
-    if constexpr (DEPTH == 2) {
-      if (x0 + 1 < x1) issue_tile(std::integral_constant<int, 1>{}, x0 + 2);
-    }
+    const IdPair ids_first = issue_id_loads(desc_ids);
+    issue_q_loads(desc_ids.b, desc_ids.row, desc_ids.nseq);
+    desc0 = desc_ids;
+    request(x0 + 1);
+    rows_from_ids(desc0, ids_first);
+    issue_v_loads(desc0);
+    issue_k_loads(desc0);
     adopt_q();
     reset_state();
-    bool q_pending = false;  // qraw holds the Q of the item that the next tile opens
 
-    auto step = [&](auto set_c, int x) {
-      constexpr int SET = decltype(set_c)::value;
+    // One step of the pipeline on the tile in the registers (tile x): the ids of tile x + 1 have arrived (requested a
+    // step ago), those of tile x + 2 are requested, and tile x + 1's loads go out as `work` frees the V registers
+    // (`between_v`) and the K registers (`between_k`).
+    auto step = [&](int x, auto&& work) {
       ARENO_TRACE_POINT();
-      const TileDesc t = desc[SET];
-      // tile x + DEPTH: its ids were requested a step ago; its loads go out as this tile's registers become free
-      const bool more = x + DEPTH < x1;
-      TileDesc nt = t;
-      if (more) {
-        rows_from_ids(desc_ids);
-        nt = desc_ids;
-        if (x + DEPTH + 1 < x1) request_next(x + DEPTH + 1);
-      }
-      if (t.kind & kTileNewToken) {
-        new_token_step(set_c, t);
-        if (more) {
-          issue_v_loads(set_c, nt);
-          issue_k_loads(set_c, nt);
-        }
-      } else {
-        tile_step(
-            set_c, t, [&]() { if (more) issue_v_loads(set_c, nt); }, [&]() { if (more) issue_k_loads(set_c, nt); });
-      }
-      if (more) desc[SET] = nt;
-      // -- end of an item's share: emit its partial and switch to the next item -------------------------------------
-      const bool last_of_unit = x + 1 == x1;
-      const TileDesc& next = DEPTH == 1 ? nt : desc[DEPTH == 1 ? 0 : 1 - SET];  // tile x + 1
-      const bool next_opens = !last_of_unit && (next.kind & kTileOpens);
-      if (next_opens || last_of_unit) {
-        write_partial(t.b, t.row, t.nseq);
-        if (!last_of_unit) {
-          if (!q_pending) issue_q_loads(next);  // an item of one tile right behind another: its Q was not asked for yet
-          adopt_q();
-          reset_state();
-          q_pending = false;
-        }
-      }
-      // Q of the item that tile x + 2 opens: a step of lead
-      if (x + 2 < x1) {
-        const TileDesc& ahead = DEPTH == 1 ? desc_ids : nt;  // tile x + 2
-        if (ahead.kind & kTileOpens) {
-          issue_q_loads(ahead);
-          q_pending = true;
-        }
-      }
+      const TileDesc t = desc0;
+      const TileDesc nt = desc_ids;
+      rows_from_ids(nt, ids);
+      // the ids are consumed before the next ones are requested into the same registers
+      __builtin_amdgcn_sched_barrier(0);
+      request(x + 2);
+      // (scheduling barriers: a load of the next tile must not move in front of the last use of the registers it
+      // fills, or the two values would need different registers and a copy of a value still in flight)
+      work(
+          t,
+          [&]() {
+            __builtin_amdgcn_sched_barrier(0);
+            issue_v_loads(nt);
+            __builtin_amdgcn_sched_barrier(0);
+          },
+          [&]() {
+            __builtin_amdgcn_sched_barrier(0);
+            issue_k_loads(nt);
+            __builtin_amdgcn_sched_barrier(0);
+          });
+      desc0 = nt;
     };
-    // Q of the item tile x0 + 1 opens (tile x0 + 2's is asked for by the first step)
-    if (x0 + 1 < x1) {
-      const TileDesc& second = DEPTH == 1 ? desc_ids : desc[DEPTH - 1];
-      if (second.kind & kTileOpens) {
-        issue_q_loads(second);
-        q_pending = true;
+
+    // The unit as a sequence of item segments: the tiles of one item that fall into the unit.  The loop over a
+    // segment's regular tiles has no item logic in it (so nothing but the tile stream is carried around it); the
+    // appended token's tile, the partial and the switch to the next item's Q come behind it.
+    int x = x0;
+    for (;;) {
+      const TileDesc first = desc0;
+      const int seg_end = min(x1, first.x_end);
+      const bool appended = shape.new_token_tile && !is_shared(first.b) && seg_end == first.x_end;
+      const int regular_end = seg_end - (appended ? 1 : 0);
+      if (first.x_end < x1) {
+        // Q of the next item with tiles: requested now (qraw is free), adopted when this segment is done
+        int b2 = first.b + 1;
+        while (cum.at(b2 + 1) == first.x_end) ++b2;
+        const ItemInfo it2 = item_info<GROUPED>(shape, lens, b2);
+        issue_q_loads(b2, it2.row, it2.nseq);
       }
-    }
-    for (int x = x0; x < x1; x += DEPTH) {
-      step(std::integral_constant<int, 0>{}, x);
-      if constexpr (DEPTH == 2) {
-        if (x + 1 < x1) step(std::integral_constant<int, 1>{}, x + 1);
+      for (; x < regular_end; ++x)
+        step(x, [&](const TileDesc& t, auto&& between_v, auto&& between_k) { tile_step(t, between_v, between_k); });
+      if (appended) {
+        step(x, [&](const TileDesc& t, auto&& between_v, auto&& between_k) {
+          new_token_step(t);
+          between_v();
+          between_k();
+        });
+        ++x;
       }
+      write_partial(first.b, first.row, first.nseq);
+      if (x >= x1) break;
+      adopt_q();
+      reset_state();
     }
   }
 #ifdef ARENO_TRACE

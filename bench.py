@@ -375,6 +375,54 @@ def measure_prefill(w, iters=20):
     }
 
 
+def wave_trace(w, launches=12):
+    """Per-wave timeline of the split kernel (tuning builds only: ``ARENO_TRACE=1 python setup.py build_ext --inplace``
+    makes the kernel stamp its waves with the 100 MHz wall clock): when waves start, have the work list, start their
+    first four tiles and finish, relative to the first wave's start, over the last launches of a warm sequence."""
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    from areno_amd.accel import cabi
+
+    lib = cabi.lib()
+    if not hasattr(lib, "areno_hip_debug_set_trace"):
+        raise SystemExit("--wave-trace needs a library built with ARENO_TRACE=1")
+    lib.areno_hip_debug_set_trace.argtypes = [ctypes.c_void_p]
+    b, hq, hkv, d, bs = w.shape
+    pools = _clone_pools(w, 6)
+    workspace = torch.empty(cabi.decode_workspace_bytes(b, hq, d, bs, w.block_table.shape[1]), dtype=torch.uint8, device=w.q.device)
+    out = torch.empty_like(w.q)
+    buf = torch.zeros(8192 * 8, dtype=torch.int64, device=w.q.device)
+    lib.areno_hip_debug_set_trace(buf.data_ptr())
+    runs = []
+    for it in range(launches):
+        buf.zero_()
+        cabi.paged_decode(cabi.describe_cache(*pools[it % len(pools)]), w.q, w.k_update, w.v_update, out, w.block_table,
+                          w.cache_seqlens, workspace, softmax_scale=w.softmax_scale, stages=cabi.STAGE_APPEND | cabi.STAGE_SPLIT)  # fmt: skip
+        torch.cuda.synchronize()
+        runs.append(buf.cpu().view(-1, 8).numpy().copy())
+    lib.areno_hip_debug_set_trace(None)
+
+    def pct(a, q):
+        return float(np.percentile(a, q))
+
+    summary = []
+    for t in runs[launches // 2:]:
+        t = t[t[:, 6] != 0].astype(np.float64)
+        t0 = t[:, 0].min()
+        us = lambda col: (t[:, col] - t0) / 100.0  # noqa: E731
+        rec = {"waves": int(len(t))}
+        for name, col in (("start", 0), ("work_list_ready", 1), ("tile0", 2), ("tile1", 3), ("tile2", 4), ("tile3", 5), ("finish", 6)):
+            v = us(col)[t[:, col] != 0]
+            rec[name] = {"mean": float(v.mean()), "p10": pct(v, 10), "p50": pct(v, 50), "p90": pct(v, 90), "max": float(v.max())}
+        summary.append(rec)
+    keys = ("start", "work_list_ready", "tile0", "tile1", "tile2", "tile3", "finish")
+    mean = {k: {s: float(np.mean([r[k][s] for r in summary])) for s in ("mean", "p10", "p50", "p90", "max")} for k in keys}
+    return {"workload": w.name, "launches_averaged": len(summary), "waves": summary[-1]["waves"], "us_since_first_wave_start": mean}
+
+
 def cpu_baseline(w, rows=16, repeats=3):
     """The CPU oracle (PyTorch restatement of the reference's native path) on the first `rows` sequences."""
     import torch
@@ -416,6 +464,8 @@ def main() -> int:
     ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg2_b256"], default=None,
                     help="measure a single workload")  # fmt: skip
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--wave-trace", choices=["cfg1", "cfg2", "cfg3"], default=None,
+                    help="print the split kernel's per-wave timeline for a workload (needs an ARENO_TRACE=1 build) and exit")  # fmt: skip
     args = ap.parse_args()
     if args.gpus != 1:
         print(
@@ -444,6 +494,11 @@ def main() -> int:
         # cost (launch, dependent first loads, uneven wave finish: ~13 us) weighs on the B = 64 figures
         "cfg2_b256": lambda: workloads.cfg2_qwen7b_int8(device=dev, quantize_fn=_gpu_quantize, batch=256),
     }
+    if args.wave_trace:
+        w = builders[args.wave_trace]()
+        w.meta.pop("shared_prefix_lens", None)  # the plain kernel's timeline
+        print(json.dumps(wave_trace(w)))
+        return 0
     names = [args.only] if args.only else ["cfg1", "cfg2", "cfg3", "cfg4", "cfg2_b256"]
     results = {}
     baseline = None

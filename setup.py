@@ -38,7 +38,7 @@ HIP_DEVICE_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-fno-honor-nans",  # fmaxf as a bare v_max_f32 / v_max3_f32 (no canonicalising self-max); nothing here relies on NaN
     "-DARENO_DEVICE_FLAGS_OK=1",  # device_common.hpp refuses to compile without the two flags above
-] + [f"-D{name}={os.environ[name]}" for name in ("ARENO_MFMA_NW", "ARENO_TRACE", "ARENO_MFMA_QUANT_OCC", "ARENO_PREFILL_WAVES") if os.environ.get(name)]  # fmt: skip
+] + [f"-D{name}={os.environ[name]}" for name in ("ARENO_MFMA_NW", "ARENO_TRACE", "ARENO_MFMA_QUANT_OCC", "ARENO_MFMA_WIDE_OCC", "ARENO_PREFILL_WAVES") if os.environ.get(name)]  # fmt: skip
 
 
 def _hipcc() -> str:
