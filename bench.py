@@ -2,15 +2,15 @@
 
 A step is one call of the decode op (fused cache append + split-KV GQA attention + merge) for one layer over
 one batch of synthetic sequences.  The headline workload is the Qwen2.5-7B-like shape (B=64, 28 q heads /
-4 kv heads, D=128, page 16, contexts uniform in [512, 4096]) with a bf16 KV cache; the same shape with an
-int8 cache (quantizing append included) and the fp8 rollout shape are measured too and reported under
-"workloads".  Inputs are resident in HBM before timing starts.  Steps rotate over several copies of the KV
+4 kv heads, D=128, page 16, contexts uniform in [512, 4096]) with an int8 KV cache (quantizing append included), the
+configuration the bandwidth target is stated on; the same shape with a bf16 cache, the fp8 rollout shape and the fp8
+prefill shape are measured too and reported under "workloads".  Inputs are resident in HBM before timing starts.  Steps rotate over several copies of the KV
 pools so that the working set exceeds the 256 MB Infinity Cache and the reads really come from HBM.
 
 Prints ONE JSON line.  `value` is microseconds per step measured over exactly `--steps` steps replayed from
 HIP graphs (how the engine runs decode); `roofline` is for the split-KV kernel alone: algorithmic bytes of one
-launch divided by its mean duration measured with events on the launch stream; `cpu_baseline` is the CPU
-oracle timed on the host cores on a stated sample.
+launch divided by its mean duration measured with events on the launch stream, next to what a plain reader of the
+same pools reaches (`stream_ceiling_gbps`); `cpu_baseline` is the CPU oracle timed on the host cores.
 """
 
 from __future__ import annotations
@@ -28,10 +28,15 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 POOL_TARGET_BYTES = 1.3e9  # rotate over at least this much distinct KV
-# HBM bytes per launch of the split kernel from two rocprofv3 counter runs of this script (FETCH_SIZE, scaled by the
-# factor 2.0 that a copy of known size gives for it, plus WRITE_SIZE); the counter summary is kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 315.82e6, "cfg2-qwen7b-int8": 158.68e6, "cfg3-rollout-fp8": 1071.17e6,
+# HBM bytes per launch of the dominant kernel as two rocprofv3 counter runs of this script recorded them (FETCH_SIZE,
+# scaled by the factor 2.0 that a copy of known size gives for it, plus WRITE_SIZE).  Recorded constants, not
+# measurements of the present run: the summaries they come from are under profiles/.
+PROFILED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 315.82e6, "cfg2-qwen7b-int8": 158.68e6, "cfg3-rollout-fp8": 1071.17e6,
                           "cfg4-prefill-fp8": 1623.08e6}
+PROFILED_TRAFFIC_SOURCE = {
+    "decode": "recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script: profiles/decode_mfma_kernel_hbm_traffic_cfg1_cfg2_cfg3.md",
+    "prefill": "recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script: profiles/prefill_mfma_kernel_hbm_traffic_cfg4.md",
+}
 
 
 def _clone_pools(w, copies):
@@ -188,7 +193,8 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
     assert torch.equal(out2, out), "C-ABI staged run disagrees with the op"
 
     gbps = alg_bytes / (us_split * 1e-6) / 1e9
-    traffic = MEASURED_TRAFFIC_BYTES.get(w.name)
+    traffic = PROFILED_TRAFFIC_BYTES.get(w.name)
+    ceiling = measure_stream_ceiling(w, pools)
     return {
         "workload": w.name,
         "us_per_step": us_graph,
@@ -201,7 +207,12 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
         "op_gbps": alg_bytes / (us_graph * 1e-6) / 1e9,
         "roofline": {
             "bound": "hbm", "kernel": "decode_mfma_kernel", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic,
+            "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic, "traffic_profiled": traffic,
+            "traffic_source": PROFILED_TRAFFIC_SOURCE["decode"],
+            # what a reader that computes nothing reaches over the same pools (all pages in address order / the distinct
+            # pages of the block table in random order), and the split kernel against the latter
+            "stream_ceiling_gbps": ceiling["linear_gbps"], "stream_ceiling_paged_gbps": ceiling["paged_gbps"],
+            "frac_of_stream_ceiling": gbps / ceiling["paged_gbps"],
         },  # fmt: skip
         "pool_copies": copies,
         "parity_max_abs_4rows": parity,
@@ -209,6 +220,45 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
         "kv_tokens": {"logical": w.logical_tokens, "unique": w.unique_tokens},
         "block_tables": measure_block_tables(w),
     }
+
+
+def measure_stream_ceiling(w, pools, iters=10, samples=9):
+    """GB/s of `areno_hip_probe_stream_read` (16-byte loads, a page per wave at a time, nothing computed) over the K and
+    V pools of all pool copies: every page in address order, and the distinct pages the block table names in a random order."""
+    import torch
+
+    from areno_amd.accel import cabi
+
+    page_bytes = w.k_cache[0].numel() * w.k_cache.element_size()
+    sink = torch.zeros(16, dtype=torch.int32, device=w.q.device)
+    bs = w.k_cache.shape[1]
+    lens = w.cache_seqlens.cpu()
+    table = w.block_table.cpu()
+    used = torch.unique(torch.cat([table[b, : (int(lens[b]) + bs) // bs] for b in range(table.shape[0])]))
+    # every page once (rows of a rollout share pages), in a fixed random order as the shuffled pools give it to the kernel
+    used = used[torch.randperm(used.numel(), generator=torch.Generator().manual_seed(7))].to(torch.int32).to(w.q.device)
+
+    def timed(ids):
+        def once():
+            for pool in pools:
+                cabi.probe_stream_read(pool[0], page_bytes, sink, ids)
+                cabi.probe_stream_read(pool[1], page_bytes, sink, ids)
+
+        once()
+        torch.cuda.synchronize()
+        out = []
+        for _ in range(samples):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                once()
+            e1.record()
+            e1.synchronize()
+            out.append(e0.elapsed_time(e1) * 1e-3 / iters)
+        pages = (pools[0][0].numel() * pools[0][0].element_size()) // page_bytes if ids is None else ids.numel()
+        return 2 * len(pools) * pages * page_bytes / statistics.median(out) / 1e9
+
+    return {"linear_gbps": timed(None), "paged_gbps": timed(used), "page_bytes": page_bytes}
 
 
 def measure_block_tables(w, inner=20, repeats=5):
@@ -370,7 +420,8 @@ def measure_prefill(w, iters=20):
         "flops": flops,
         "roofline": {
             "bound": "mfma", "kernel": "prefill_mfma_kernel", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS,
-            "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
+            "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": PROFILED_TRAFFIC_BYTES.get(w.name),
+            "traffic_profiled": PROFILED_TRAFFIC_BYTES.get(w.name), "traffic_source": PROFILED_TRAFFIC_SOURCE["prefill"],
         },  # fmt: skip
     }
 
@@ -423,8 +474,10 @@ def wave_trace(w, launches=12):
     return {"workload": w.name, "launches_averaged": len(summary), "waves": summary[-1]["waves"], "us_since_first_wave_start": mean}
 
 
-def cpu_baseline(w, rows=16, repeats=3):
-    """The CPU oracle (PyTorch restatement of the reference's native path) on the first `rows` sequences."""
+def cpu_baseline(w, warmups=3, repeats=7):
+    """The CPU oracle (PyTorch restatement of the reference's native path: cache append, per-sequence block-table gather,
+    fp32 softmax attention with GQA) on all sequences of the workload, on the host cores: three warm-ups, median of
+    seven runs."""
     import torch
 
     from oracle import attention_ref as ar
@@ -435,24 +488,24 @@ def cpu_baseline(w, rows=16, repeats=3):
         kc, vc = w.k_cache.cpu().float(), w.v_cache.cpu().float()
     else:
         kc, vc = qr.dequantize(w.k_cache.cpu(), w.k_scale.cpu()), qr.dequantize(w.v_cache.cpu(), w.v_scale.cpu())
-    q, ku, vu = w.q[:rows].cpu().float(), w.k_update[:rows].cpu().float(), w.v_update[:rows].cpu().float()
-    table, lens = w.block_table[:rows].cpu(), w.cache_seqlens[:rows].cpu()
+    q, ku, vu = w.q.cpu().float(), w.k_update.cpu().float(), w.v_update.cpu().float()
+    table, lens = w.block_table.cpu(), w.cache_seqlens.cpu()
 
     def once():
         ar.ref_decode_update(ku, vu, kc, vc, table, lens)
         return ar.ref_paged_decode(q, kc, vc, table, lens, -1, w.softmax_scale)
 
-    once()
+    for _ in range(warmups):
+        once()
     times = []
     for _ in range(repeats):
         t0 = time.perf_counter()
         once()
         times.append(time.perf_counter() - t0)
-    per_step_us = statistics.median(times) * 1e6 * (w.q.shape[0] / rows)
     return {
-        "value": per_step_us, "unit": "us/step", "cores": threads, "kind": "port",
-        "sample": f"{rows} of {w.q.shape[0]} sequences of {w.name} (fp32 caches, append + gather + attention), "
-                  f"median of {repeats}, scaled by {w.q.shape[0] / rows:g}",
+        "value": statistics.median(times) * 1e6, "unit": "us/step", "cores": threads, "kind": "port",
+        "sample": f"all {w.q.shape[0]} sequences of {w.name} (dequantized fp32 caches; append + gather + attention), "
+                  f"{warmups} warm-ups, median of {repeats} runs, fastest-slowest {min(times) * 1e6:.0f}-{max(times) * 1e6:.0f} us",
     }  # fmt: skip
 
 
@@ -499,7 +552,7 @@ def main() -> int:
         w.meta.pop("shared_prefix_lens", None)  # the plain kernel's timeline
         print(json.dumps(wave_trace(w)))
         return 0
-    names = [args.only] if args.only else ["cfg1", "cfg2", "cfg3", "cfg4", "cfg2_b256"]
+    names = [args.only] if args.only else ["cfg2", "cfg1", "cfg3", "cfg4", "cfg2_b256"]
     results = {}
     baseline = None
     for name in names:
