@@ -196,14 +196,20 @@ __global__ __launch_bounds__(kAllocThreads) void block_tables_release_kernel(are
   if (threadIdx.x == 0) bt.state[kStateCount] = count + returned;
 }
 
-// Entry (i, c) of the rectangular table of `rows`.
-__device__ void gather_entry(const areno_block_tables& bt, const int64_t* rows, int i, int c, int pad_mode,
-                             int32_t* out) {
+// Entry (i, c) of the rectangular table of `rows`.  With next_positions (the table of a decode step), a row that
+// has no page for the position it writes next -- the pool ran dry when it asked -- becomes a row of scratch ids: the
+// decode op then appends its token to the scratch page instead of overwriting slot 0 of the row's last page.
+__device__ void gather_entry(const areno_block_tables& bt, const int64_t* rows, const int32_t* next_positions, int i,
+                             int c, int pad_mode, int32_t* out) {
   const int64_t r = rows[i];
   int32_t id = bt.num_blocks;  // the scratch page
   if (r >= 0 && r < bt.max_rows) {
     const int have = bt.row_blocks[r];
-    if (c < have) {
+    const bool unserved = next_positions != nullptr && have > 0 &&
+                          static_cast<int64_t>(next_positions[i]) >= static_cast<int64_t>(have) * bt.block_size;
+    if (unserved) {
+      // parked; the status word already says why (exhausted pool or full row)
+    } else if (c < have) {
       id = bt.table[r * bt.max_blocks + c];
     } else if (have > 0 && pad_mode == ARENO_PAD_LAST_BLOCK) {
       id = bt.table[r * bt.max_blocks + have - 1];
@@ -216,10 +222,10 @@ __device__ void gather_entry(const areno_block_tables& bt, const int64_t* rows, 
   out[static_cast<int64_t>(i) * bt.max_blocks + c] = id;
 }
 
-__global__ void block_tables_gather_kernel(areno_block_tables bt, const int64_t* rows, int n, int pad_mode,
-                                           int32_t* out) {
+__global__ void block_tables_gather_kernel(areno_block_tables bt, const int64_t* rows, const int32_t* next_positions,
+                                           int n, int pad_mode, int32_t* out) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c < bt.max_blocks) gather_entry(bt, rows, blockIdx.y, c, pad_mode, out);
+  if (c < bt.max_blocks) gather_entry(bt, rows, next_positions, blockIdx.y, c, pad_mode, out);
 }
 
 __global__ void block_tables_prefill_slots_kernel(areno_block_tables bt, const int64_t* rows, const int32_t* cursors,
@@ -271,6 +277,21 @@ int launch_reserve(const areno_block_tables* bt, const int64_t* rows, const int3
   return check_launch(op);
 }
 
+
+int launch_gather(const areno_block_tables* bt, const int64_t* rows, const int32_t* next_positions, int32_t n,
+                  int32_t pad_mode, int32_t* out_table, void* stream, const char* op) {
+  if (int rc = areno::validate_tables(bt, op)) return rc;
+  if (n < 0 || n > 65535) return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: row count %d out of range", op, n);
+  if (pad_mode != ARENO_PAD_LAST_BLOCK && pad_mode != ARENO_PAD_SCRATCH_BLOCK)
+    return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: unknown pad mode %d", op, pad_mode);
+  if (n == 0) return ARENO_OK;
+  if (rows == nullptr || out_table == nullptr)
+    return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: rows / out_table is NULL", op);
+  const unsigned col_blocks = static_cast<unsigned>((bt->max_blocks + 255) / 256);
+  hipLaunchKernelGGL(areno::block_tables_gather_kernel, dim3(col_blocks, static_cast<unsigned>(n)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), *bt, rows, next_positions, n, pad_mode, out_table);
+  return areno::check_launch(op);
+}
 }  // namespace
 }  // namespace areno
 
@@ -307,19 +328,9 @@ extern "C" int areno_hip_block_tables_release(const areno_block_tables* bt, cons
 
 extern "C" int areno_hip_block_tables_gather(const areno_block_tables* bt, const int64_t* rows, int32_t n,
                                              int32_t pad_mode, int32_t* out_table, void* stream) {
-  const char* op = "areno_hip_block_tables_gather";
-  if (int rc = areno::validate_tables(bt, op)) return rc;
-  if (n < 0 || n > 65535) return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: row count %d out of range", op, n);
-  if (pad_mode != ARENO_PAD_LAST_BLOCK && pad_mode != ARENO_PAD_SCRATCH_BLOCK)
-    return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: unknown pad mode %d", op, pad_mode);
-  if (n == 0) return ARENO_OK;
-  if (rows == nullptr || out_table == nullptr)
-    return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: rows / out_table is NULL", op);
-  const unsigned col_blocks = static_cast<unsigned>((bt->max_blocks + 255) / 256);
-  hipLaunchKernelGGL(areno::block_tables_gather_kernel, dim3(col_blocks, static_cast<unsigned>(n)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), *bt, rows, n, pad_mode, out_table);
-  return areno::check_launch(op);
+  return areno::launch_gather(bt, rows, nullptr, n, pad_mode, out_table, stream, "areno_hip_block_tables_gather");
 }
+
 
 extern "C" int areno_hip_block_tables_decode_step(const areno_block_tables* bt, const int64_t* rows,
                                                   const int32_t* next_positions, int32_t n, int32_t pad_mode,
@@ -335,7 +346,8 @@ extern "C" int areno_hip_block_tables_decode_step(const areno_block_tables* bt, 
   // (one workgroup doing both was measured slower than the two launches: its table pass is a chain of dependent
   // loads that the many workgroups of the gather kernel overlap)
   if (int rc = areno_hip_block_tables_ensure_decode(bt, rows, next_positions, n, stream)) return rc;
-  return areno_hip_block_tables_gather(bt, rows, n, pad_mode, out_table, stream);
+  // rows the pool could not serve come out as rows of scratch ids (see gather_entry)
+  return areno::launch_gather(bt, rows, next_positions, n, pad_mode, out_table, stream, op);
 }
 
 extern "C" int areno_hip_block_tables_prefill_slots(const areno_block_tables* bt, const int64_t* rows,

@@ -296,6 +296,10 @@ int areno_hip_block_tables_gather(const areno_block_tables* tables, const int64_
 /*
  * One decode step's bookkeeping in one call: areno_hip_block_tables_ensure_decode followed by
  * areno_hip_block_tables_gather for the same rows (inference.py:561-580 does the two on the host every step).
+ * A row that did not get the page its next position needs (the pool ran dry, or the row is at max_blocks; the status
+ * word says which) comes out as a row of scratch ids, so that the decode op's append cannot land in a page that holds
+ * live tokens; the caller reads `state` before it trusts that step's outputs (the reference raises before it decodes,
+ * rollout_state.py:222-224).
  */
 int areno_hip_block_tables_decode_step(const areno_block_tables* tables, const int64_t* rows,
                                        const int32_t* next_positions, int32_t n, int32_t pad_mode, int32_t* out_table,

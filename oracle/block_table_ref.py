@@ -107,12 +107,17 @@ class RefBlockTables:
             if blocks:
                 self.free.extend(blocks)
 
-    def gather(self, rows: list[int], pad_scratch: bool) -> list[list[int]]:
+    def gather(self, rows: list[int], pad_scratch: bool, next_positions: list[int] | None = None) -> list[list[int]]:
+        """``next_positions`` (the table of a decode step): a row without a page for the position it writes next -- the
+        reference has raised by then (rollout_state.py:222-224); a device-side step cannot -- is parked on the scratch
+        page, so that its token cannot land in a page that holds live tokens."""
         out = []
         for i, row in enumerate(rows):
             blocks = self.rows.get(row) if 0 <= row < self.max_rows else None
             if row >= self.max_rows or (row >= 0 and not blocks):
                 self._report(BAD_ROW, i)
+            if blocks and next_positions is not None and next_positions[i] >= len(blocks) * self.block_size:
+                blocks = None
             if not blocks:
                 out.append([self.num_blocks] * self.max_blocks)
                 continue

@@ -70,7 +70,7 @@ def test_random_traffic_matches_the_host_lists(seed, num_blocks, max_rows, max_b
                 scratch = bool(step % 4)
                 got = dev.decode_step(rows_t, pos_t, pad="scratch" if scratch else "last")
                 ref.ensure_decode(rows, pos)
-                assert got.cpu().tolist() == ref.gather(rows, scratch)
+                assert got.cpu().tolist() == ref.gather(rows, scratch, pos)
             for r in rows:
                 if len(ref.row_pages(r)) * bs > lengths[r]:
                     lengths[r] += 1
@@ -110,6 +110,42 @@ def test_exhaustion_is_recorded_and_raised_like_the_reference():
     bad = DeviceBlockTables(9, 2, 4, 2, DEV)
     bad.reserve([0, 5, 0], [2, 2, 4])
     assert bad.row_pages(0) == [0] and bad.status() == (BAD_ROW, 1)
+
+
+def test_a_decode_step_on_a_dry_pool_touches_no_live_page():
+    """Rows whose next token opens a page while the pool is empty: the step's table parks them on the scratch page, so
+    the decode op's append lands there and every page that holds live tokens keeps its bytes (the reference raises
+    before it decodes, rollout_state.py:222-224; a device-side step reports through the status word instead)."""
+    from areno_amd.accel import attention as ops
+
+    bs, hkv, d, rows = 4, 2, 64, 3
+    num_pages = 6
+    dev = DeviceBlockTables(num_pages, rows, 8, bs, DEV)
+    dev.reserve([0, 1, 2], [8, 8, 6])  # 2 + 2 + 2 pages: the pool is empty; rows 0 and 1 are at a page border
+    assert dev.free_count() == 0 and dev.status() == (OK, -1)
+    g = torch.Generator(device=DEV).manual_seed(3)
+    k_cache = torch.randn(num_pages + 1, bs, hkv, d, device=DEV, dtype=torch.bfloat16, generator=g)  # + the scratch page
+    v_cache = torch.randn_like(k_cache)
+    before_k, before_v = k_cache.clone(), v_cache.clone()
+    lens = torch.tensor([8, 8, 6], dtype=torch.int32, device=DEV)
+    table = dev.decode_step(torch.arange(rows, device=DEV), lens)
+    assert dev.status() == (EXHAUSTED, 0)
+    tab = table.cpu().tolist()
+    assert tab[0] == [num_pages] * 8 and tab[1] == [num_pages] * 8, "unserved rows are parked on the scratch page"
+    assert tab[2][:2] == dev.row_pages(2) and dev.row_pages(0) == [0, 1]
+    q = torch.randn(rows, 4, d, device=DEV, dtype=torch.bfloat16, generator=g)
+    ku = torch.randn(rows, hkv, d, device=DEV, dtype=torch.bfloat16, generator=g)
+    vu = torch.randn_like(ku)
+    ops.areno_paged_causal_attention_decode(q, ku, vu, k_cache, v_cache, table, lens)
+    torch.cuda.synchronize()
+    changed = (k_cache != before_k).flatten(1).any(1) | (v_cache != before_v).flatten(1).any(1)
+    pages = set(torch.nonzero(changed).flatten().tolist())
+    # row 2 appends at position 6 = slot 2 of its second page; the parked rows write into the scratch page only
+    assert pages == {dev.row_pages(2)[1], num_pages}
+    served = dev.row_pages(2)[1]
+    assert torch.equal(k_cache[served, 2], ku[2]) and torch.equal(k_cache[served, :2], before_k[served, :2])
+    with pytest.raises(RuntimeError, match="paged KV cache exhausted"):
+        dev.check()
 
 
 def test_prefill_slots_follow_the_payload_layout():
