@@ -21,12 +21,8 @@ def extension() -> ModuleType:
         try:
             _EXT = importlib.import_module("areno_amd.accel._areno_accel")
         except ImportError as exc:
-            build_ext = os.environ.get("ARENO_BUILD_EXT")
-            build_hint = (
-                " The current environment has ARENO_BUILD_EXT=0, which intentionally skips compiling the extension."
-                if build_ext is not None and build_ext.lower() in {"0", "false", "no", "off"}
-                else ""
-            )
+            skipped = os.environ.get("ARENO_BUILD_EXT", "").strip().lower() in {"0", "false", "no", "off"}
+            build_hint = " ARENO_BUILD_EXT is set to skip the native build in this environment." if skipped else ""
             raise RuntimeError(
                 "AReno runtime setup failed: the compiled `areno_accel` extension is not installed."
                 f"{build_hint}\n"

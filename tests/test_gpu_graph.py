@@ -99,3 +99,80 @@ def test_decode_graph_replays_match_eager_and_oracle(kv, hq, hkv, d):
             ra, rb = a[idx].view(torch.uint8), b[idx].view(torch.uint8)
             assert torch.equal(ra, rb), f"replay {step}: {name} pages differ between graph and eager"
         assert torch.isfinite(s_out[actual:].float()).all(), "parked rows must stay finite"
+
+
+def test_bucketed_decode_graphs_share_one_cache():
+    """One graph per bucket size, as the reference captures them (areno/engine/runtime/decode_graph.py:64-178 with the
+    bucket list of areno/engine/config.py:51-53), all against the same cache, replayed interleaved as the number of
+    active rows changes from step to step; each graph keeps the workspace its capture allocated.  Every replay must
+    equal an eager step on a second copy of the cache (outputs and appended rows), whatever ran before it."""
+    hq, hkv, d, bs = 8, 2, 128, 16
+    rows = 40
+    g = torch.Generator().manual_seed(91)
+    lengths = torch.randint(3, 400, (rows,), generator=g)
+    w = workloads.make_decode_workload("graph-buckets", seed=33, batch=rows, hq=hq, hkv=hkv, d=d, bs=bs, kv="int8",
+                                       lengths=lengths, device=DEV, quantize_fn=gpu_quantize, pool_slack=0.5)  # fmt: skip
+    used = set(w.block_table.cpu().flatten().tolist())
+    scratch = max(i for i in range(w.k_cache.shape[0]) if i not in used)
+    cols = w.block_table.shape[1] + 2
+    pools = (w.k_cache, w.v_cache, w.k_scale, w.v_scale)
+    e_kc, e_vc, e_ks, e_vs = (t.clone() for t in pools)
+
+    class Bucket:
+        def __init__(self, size):
+            self.size = size
+            self.q = torch.zeros((size, hq, d), dtype=w.q.dtype, device=DEV)
+            self.ku = torch.zeros((size, hkv, d), dtype=w.q.dtype, device=DEV)
+            self.vu = torch.zeros_like(self.ku)
+            self.table = torch.full((size, cols), scratch, dtype=torch.int32, device=DEV)
+            self.lens = torch.zeros(size, dtype=torch.int32, device=DEV)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                self.run()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self.out = self.run()
+
+        def run(self):
+            return _decode(self.q, self.ku, self.vu, *pools[:2], self.table, self.lens, *pools[2:], w.softmax_scale)
+
+        def replay(self, q, ku, vu, table, lens):
+            n = q.shape[0]
+            self.q[:n].copy_(q)
+            self.ku[:n].copy_(ku)
+            self.vu[:n].copy_(vu)
+            self.lens[:n].copy_(lens)
+            self.lens[n:].fill_(0)
+            self.table[:n, : table.shape[1]].copy_(table)
+            self.table[:n, table.shape[1] :].fill_(scratch)
+            self.table[n:].fill_(scratch)
+            self.graph.replay()
+            return self.out[:n]
+
+    buckets = [Bucket(size) for size in (8, 16, 64)]
+    lens = w.cache_seqlens.clone()
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    live = torch.tensor(sorted(used), device=DEV)
+    # rows that have room for the steps below in their last page keep decoding; the active count picks the bucket
+    room = ((lens.cpu() % bs) + 6 < bs).nonzero().flatten().tolist()
+    for step, actual in enumerate((5, 12, len(room), 7, 16, 3)):
+        active = torch.tensor(room[:actual], device=DEV)
+        q = (torch.randn((actual, hq, d), generator=gen, device=DEV) * d**-0.25).to(w.q.dtype)
+        ku = torch.randn((actual, hkv, d), generator=gen, device=DEV).to(w.q.dtype)
+        vu = torch.randn((actual, hkv, d), generator=gen, device=DEV).to(w.q.dtype)
+        table, now = w.block_table[active].contiguous(), lens[active].contiguous()
+        bucket = next(b for b in buckets if b.size >= actual)
+        got = bucket.replay(q, ku, vu, table, now).clone()
+        eager = _decode(q, ku, vu, e_kc, e_vc, table, now, e_ks, e_vs, w.softmax_scale)
+        torch.cuda.synchronize()
+        # (the bucket's launch cuts the work differently from the eager one: same math, another summation order)
+        assert_close(got, eager.cpu().float(), 8e-3, what=f"step {step}: bucket {bucket.size} with {actual} rows vs the eager step")
+        for a, b, name in zip(pools, (e_kc, e_vc, e_ks, e_vs), ("k", "v", "k_scale", "v_scale")):
+            assert torch.equal(a[live].view(torch.uint8), b[live].view(torch.uint8)), f"step {step}: {name} pages differ"
+        kc, vc = dequant_cpu(pools[0], pools[2]), dequant_cpu(pools[1], pools[3])
+        want = ar.ref_paged_decode(q.cpu().float(), kc, vc, table.cpu(), now.cpu(), -1, w.softmax_scale)
+        assert_close(got, want, *tolerances("int8"), what=f"step {step} vs oracle")
+        lens[active] += 1
