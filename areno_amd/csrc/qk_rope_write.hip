@@ -70,7 +70,7 @@ __device__ __forceinline__ float group_sum(float x) {
 
 constexpr int kRowsPerGroup = 1;  // rows a lane group works through (more than one measured slower: 53 vs 36 us at 4)
 
-template <int LPR>
+template <int LPR, int ACT>  // ACT: the activation dtype (ARENO_DT_F16 / ARENO_DT_BF16): no rounding step branches on it
 __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
   constexpr int D = LPR * 8;
   constexpr int kRowsPerWave = kWave / LPR;
@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t word = raw[r][j];
-      if (p.dtype == ARENO_DT_BF16) {
+      if (ACT == ARENO_DT_BF16) {
         x[2 * j] = bf16_bits_to_float(word & 0xffffu);
         x[2 * j + 1] = bf16_bits_to_float(word >> 16);
       } else {
@@ -142,8 +142,8 @@ __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
         const float4_t w1 = *reinterpret_cast<const float4_t*>(weight + sub * 8 + 4);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          x[j] = round_to(x[j] * inv * w0[j], p.dtype);
-          x[4 + j] = round_to(x[4 + j] * inv * w1[j], p.dtype);
+          x[j] = round_to(x[j] * inv * w0[j], ACT);
+          x[4 + j] = round_to(x[4 + j] * inv * w1[j], ACT);
         }
       }
     }
@@ -154,15 +154,15 @@ __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
       const bool low_half = sub < LPR / 2;  // rotate_half: -x[i + D/2] below D/2, x[i - D/2] above
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float c = round_to(j < 4 ? c0[r][j & 3] : c1[r][j & 3], p.dtype);
-        const float sn = round_to(j < 4 ? s0[r][j & 3] : s1[r][j & 3], p.dtype);
+        const float c = round_to(j < 4 ? c0[r][j & 3] : c1[r][j & 3], ACT);
+        const float sn = round_to(j < 4 ? s0[r][j & 3] : s1[r][j & 3], ACT);
         const float rot = low_half ? -partner[j] : partner[j];
-        x[j] = round_to(round_to(x[j] * c, p.dtype) + round_to(rot * sn, p.dtype), p.dtype);
+        x[j] = round_to(round_to(x[j] * c, ACT) + round_to(rot * sn, ACT), ACT);
       }
       void* out = kind[r] == 0 ? p.q_out : p.k_out;
       if (out != nullptr && live[r]) {
-        const uint4_t packed = {pack_two_16(x[0], x[1], p.dtype), pack_two_16(x[2], x[3], p.dtype),
-                                pack_two_16(x[4], x[5], p.dtype), pack_two_16(x[6], x[7], p.dtype)};
+        const uint4_t packed = {pack_two_16(x[0], x[1], ACT), pack_two_16(x[2], x[3], ACT),
+                                pack_two_16(x[4], x[5], ACT), pack_two_16(x[6], x[7], ACT)};
         *reinterpret_cast<uint4_t*>(static_cast<char*>(out) + src_base[r] * 2) = packed;
       }
     }
@@ -184,12 +184,13 @@ __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
 }
 
 typedef void (*rope_write_fn)(RopeWriteParams);
-rope_write_fn rope_write_lookup(int head_dim) {
+rope_write_fn rope_write_lookup(int head_dim, int dtype) {
+  const bool bf16 = dtype == ARENO_DT_BF16;
   switch (head_dim) {
-    case 64: return qk_rope_write_kernel<8>;
-    case 128: return qk_rope_write_kernel<16>;
-    case 256: return qk_rope_write_kernel<32>;
-    case 512: return qk_rope_write_kernel<64>;
+    case 64: return bf16 ? qk_rope_write_kernel<8, ARENO_DT_BF16> : qk_rope_write_kernel<8, ARENO_DT_F16>;
+    case 128: return bf16 ? qk_rope_write_kernel<16, ARENO_DT_BF16> : qk_rope_write_kernel<16, ARENO_DT_F16>;
+    case 256: return bf16 ? qk_rope_write_kernel<32, ARENO_DT_BF16> : qk_rope_write_kernel<32, ARENO_DT_F16>;
+    case 512: return bf16 ? qk_rope_write_kernel<64, ARENO_DT_BF16> : qk_rope_write_kernel<64, ARENO_DT_F16>;
     default: return nullptr;
   }
 }
@@ -253,7 +254,7 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
   p.max_pos = max_pos;
   p.dtype = dtype;
   p.eps = eps;
-  const rope_write_fn fn = rope_write_lookup(head_dim);
+  const rope_write_fn fn = rope_write_lookup(head_dim, dtype);
   if (fn == nullptr) return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim must be 64, 128, 256 or 512, got %d", op, head_dim);
   const int64_t rows = tokens * (q_heads + 2 * kv_heads);
   const int rows_per_block = 4 * kRowsPerGroup * (kWave / (head_dim / 8));
