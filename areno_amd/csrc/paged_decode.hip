@@ -257,16 +257,13 @@ reduce_slots_fn reduce_slots_kernel_for(int head_dim) {
 // ---- geometry of the MFMA path ----------------------------------------------------------------------
 constexpr int kMfmaWaves = ARENO_MFMA_NW;  // waves per workgroup
 constexpr int kComputeUnits = 256;
-constexpr int kMfmaMaxWorkgroups = 2 * kComputeUnits;          // the kernels' register budget lets two be resident per CU
-constexpr int kMfmaMaxUnits = kMfmaMaxWorkgroups * kMfmaWaves;  // one kv head, every wave a unit of its own
-// Workgroups of a launch.  Every wave keeps one 32-token tile (K and V) in flight; ~17 MB in flight over the chip
-// saturate the memory system, twice that only lengthens its queues and spreads the waves' finish times (bf16 pages at
-// head dim 128, 16 KB tiles: 61.7 us with 512 workgroups, 59.1 us with 256).  So: two workgroups per CU while a
-// wave's tile is at most 8 KB, one beyond.
-inline int mfma_workgroups(int head_dim_per_wave, int element_bytes) {
-  const int tile_bytes = 2 * kTileTokens * head_dim_per_wave * element_bytes;
-  return tile_bytes <= 8192 ? kMfmaMaxWorkgroups : kComputeUnits;
-}
+// One workgroup per CU: a wave keeps one 32-token tile (K and V) in flight, and 1024 waves with a tile each already
+// saturate the memory system; a second resident workgroup per CU only lengthens its queues and spreads the waves'
+// finish times (measured, split kernel / whole step: bf16 pages, 16 KB tiles, 61.7 / 69.7 us with 512 workgroups
+// against 59.1 / 65.8 us with 256; fp8 rollout 212.3 / 228.9 against 206.8 / 223.6; int8, 8 KB tiles, 32.9 / 41.6
+// against 33.2 / 40.5: the split kernel's loss is made up by the merge, which has half the partials to read).
+constexpr int kMfmaWorkgroups = kComputeUnits;
+constexpr int kMfmaMaxUnits = kMfmaWorkgroups * kMfmaWaves;  // one kv head, every wave a unit of its own
 
 size_t mfma_partial_bytes(size_t slots, int q_heads, int head_dim) {
   const size_t bytes = slots * q_heads * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
@@ -352,7 +349,7 @@ namespace {
 struct MfmaGrid {
   int waves, head_split, heads_per_wg, head_groups, tok_splits, workgroups, units;
 };
-MfmaGrid mfma_grid_for(int kv_heads, int head_dim, int element_bytes) {
+MfmaGrid mfma_grid_for(int kv_heads, int head_dim) {
   MfmaGrid g;
   g.waves = decode_mfma_waves(head_dim);
   g.head_split = decode_mfma_head_split(head_dim);
@@ -360,8 +357,7 @@ MfmaGrid mfma_grid_for(int kv_heads, int head_dim, int element_bytes) {
   g.heads_per_wg = (heads >= 4 && kv_heads % 4 == 0) ? 4 : ((heads >= 2 && kv_heads % 2 == 0) ? 2 : 1);
   g.head_groups = kv_heads / g.heads_per_wg;
   g.tok_splits = heads / g.heads_per_wg;
-  const int wgs = mfma_workgroups(head_dim / g.head_split, element_bytes);
-  g.workgroups = wgs / g.head_groups > 0 ? wgs / g.head_groups : 1;
+  g.workgroups = kMfmaWorkgroups / g.head_groups > 0 ? kMfmaWorkgroups / g.head_groups : 1;
   g.units = g.workgroups * g.tok_splits;
   return g;
 }
@@ -370,9 +366,7 @@ MfmaGrid mfma_grid_for(int kv_heads, int head_dim, int element_bytes) {
 size_t grouped_plan_bytes(int batch) { return ((2 * static_cast<size_t>(batch) + 64) * sizeof(int32_t) + 255) / 256 * 256; }
 
 size_t shared_region_bytes(int kv_heads, int head_dim, int num_shared) {
-  // sized for the larger of the two grids (the size query does not know the cache's dtype)
-  const int units_q = mfma_grid_for(kv_heads, head_dim, 1).units, units_w = mfma_grid_for(kv_heads, head_dim, 2).units;
-  const size_t slots = static_cast<size_t>(units_q > units_w ? units_q : units_w) + num_shared;
+  const size_t slots = static_cast<size_t>(mfma_grid_for(kv_heads, head_dim).units) + num_shared;
   return slots * kv_heads * 16 * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
 }
 
@@ -492,7 +486,7 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     }
   }
   if (mfma == nullptr) num_shared = 0;  // the other kernels read every row's pages on their own
-  const MfmaGrid grid = mfma_grid_for(cache->kv_heads, p.head_dim, static_cast<int>(dtype_size(cache->cache_dtype)));
+  const MfmaGrid grid = mfma_grid_for(cache->kv_heads, p.head_dim);
   // ---- append: rides along in the matrix-core split kernel as a tile of its own per row when the kernel can take the
   // new rows as they are (one wave per head, 16-bit pages of the query's dtype or 8-bit pages), else a launch of its
   // own in front ------------------------------------------------------------------------------------------------------

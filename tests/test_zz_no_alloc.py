@@ -41,7 +41,7 @@ def _both_ways(w, **kw):
 
 
 def test_static_scratch_decode_matches_the_workspace_entry_point_twice_in_a_row():
-    big = workloads.cfg2_qwen7b_int8(device=DEV, quantize_fn=gpu_quantize)  # 64 rows, contexts to 4096, 31 MB of partials
+    big = workloads.cfg2_qwen7b_int8(device=DEV, quantize_fn=gpu_quantize)  # 64 rows, contexts to 4096, 16 MB of partials
     got, want = _both_ways(big)
     assert torch.equal(got, want), "first call (64 rows, int8 pages)"
     assert_close(got, expected_decode(big), *tolerances("int8"), what="static entry point, cfg 2, vs oracle")
@@ -61,7 +61,7 @@ def test_static_scratch_decode_refuses_shapes_beyond_its_buffer():
     assert capacity == 64 << 20
     w = workloads.cfg0_tiny("bf16", device=DEV)
     cache = cabi.describe_cache(w.k_cache, w.v_cache)
-    # 1024 rows x 64 q heads x 64 dims: (2048 + 1024) slots x 64 heads x 66 floats = 52 MB fits ...
+    # 1024 rows x 64 q heads x 64 dims: (1024 + 1024) slots x 64 heads x 66 floats = 35 MB fits ...
     assert cabi.decode_workspace_bytes(1024, 64, 64, 16, 32) <= capacity
     # ... the same with 128 q heads does not; the check comes before any launch, so the pointers are never used
     assert cabi.decode_workspace_bytes(1024, 128, 64, 16, 32) > capacity
