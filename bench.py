@@ -31,7 +31,7 @@ POOL_TARGET_BYTES = 1.3e9  # rotate over at least this much distinct KV
 # HBM bytes per launch of the dominant kernel as two rocprofv3 counter runs of this script recorded them (FETCH_SIZE,
 # scaled by the factor 2.0 that a copy of known size gives for it, plus WRITE_SIZE).  Recorded constants, not
 # measurements of the present run: the summaries they come from are under profiles/.
-PROFILED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 315.82e6, "cfg2-qwen7b-int8": 158.68e6, "cfg3-rollout-fp8": 1071.17e6,
+PROFILED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 310.95e6, "cfg2-qwen7b-int8": 153.72e6, "cfg3-rollout-fp8": 1064.65e6,
                           "cfg4-prefill-fp8": 1623.08e6}
 PROFILED_TRAFFIC_SOURCE = {
     "decode": "recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script: profiles/decode_mfma_kernel_hbm_traffic_cfg1_cfg2_cfg3.md",
