@@ -338,7 +338,7 @@ int areno_hip_attention_backward(const void* grad_out, const void* q, const void
 
 /*
  * Measurement aid, no counterpart in the reference: reads `pages` runs of page_bytes bytes (page i starts at
- * base + page_ids[i] * page_bytes, or at base + i * page_bytes when page_ids is NULL) with 16-byte loads, 512 workgroups
+ * base + page_ids[i] * page_bytes, or at base + i * page_bytes when page_ids is NULL) with 16-byte loads, workgroups
  * of four waves, one page per wave at a time, and computes nothing.  What this reaches over a set of KV pools is the
  * streaming ceiling the decode kernels' bandwidth is compared with (bench.py).
  *   base      device, 16-byte aligned;  page_bytes a multiple of 1024;  sink  device, >= 4 bytes (written practically never)
