@@ -1,8 +1,8 @@
 // Measurement aid: how fast this part streams KV pages when nothing is computed on them.  The decode kernels are
 // bound by HBM bandwidth; the figure they are held against is what a plain reader reaches over the same pools, with
-// the same 16-byte accesses and page-sized pieces.  One wave reads whole pages (a contiguous run of page_bytes, or the
-// page a table of ids names), two pages in flight, and folds what it read into one word so that the loads cannot be
-// dropped.
+// the same 16-byte accesses and page-sized pieces, and the same bytes per launch: one launch reads the pages of two
+// pools (K and V).  One wave reads whole pages (a contiguous run of page_bytes, or the page a table of ids names), eight
+// loads in flight, and folds what it read into one word so that the loads cannot be dropped.
 
 #include "device_common.hpp"
 
@@ -10,24 +10,29 @@ namespace areno {
 namespace {
 
 constexpr int kProbeWaves = 4;        // per workgroup
-constexpr int kProbeWorkgroups = 512;  // two per CU, as the decode kernels
+constexpr int kProbeWorkgroups = 512;  // two per CU
+constexpr int kProbeLoads = 8;         // 16-byte loads per lane in flight
 
-__global__ __launch_bounds__(kProbeWaves* kWave, 2) void stream_read_kernel(const char* base, const int32_t* page_ids, int64_t pages,
+__global__ __launch_bounds__(kProbeWaves* kWave, 2) void stream_read_kernel(const char* base_a, const char* base_b,
+                                                                            const int32_t* page_ids, int64_t pages,
                                                                             int32_t page_bytes, uint32_t* sink) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t wave = static_cast<int64_t>(blockIdx.x) * kProbeWaves + (threadIdx.x >> 6);
   const int64_t waves = static_cast<int64_t>(gridDim.x) * kProbeWaves;
   const int pieces = page_bytes / (kWave * 16);  // 1 KB per wave and load instruction
   uint32_t fold = 0;
-  for (int64_t i = wave; i < pages; i += waves) {
-    const int64_t page = page_ids != nullptr ? page_ids[i] : i;
-    const char* src = base + page * page_bytes + lane * 16;
-    for (int j = 0; j < pieces; j += 4) {
-      uint4_t v[4];
+  const int64_t runs = base_b != nullptr ? 2 * pages : pages;  // the two pools' copies of a page one after the other
+  for (int64_t i = wave; i < runs; i += waves) {
+    const int64_t index = base_b != nullptr ? i >> 1 : i;
+    const int64_t page = page_ids != nullptr ? page_ids[index] : index;
+    const char* src = ((base_b != nullptr && (i & 1)) ? base_b : base_a) + page * page_bytes + lane * 16;
+    for (int j = 0; j < pieces; j += kProbeLoads) {
+      uint4_t v[kProbeLoads];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const uint4_t*>(src + static_cast<int64_t>(min(j + u, pieces - 1)) * kWave * 16);
+      for (int u = 0; u < kProbeLoads; ++u)
+        v[u] = *reinterpret_cast<const uint4_t*>(src + static_cast<int64_t>(min(j + u, pieces - 1)) * kWave * 16);
 #pragma unroll
-      for (int u = 0; u < 4; ++u) fold ^= v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3];
+      for (int u = 0; u < kProbeLoads; ++u) fold ^= v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3];
     }
   }
   if (fold == 0x9e3779b9u) sink[0] = fold;  // practically never: the store only keeps the loads alive
@@ -36,15 +41,17 @@ __global__ __launch_bounds__(kProbeWaves* kWave, 2) void stream_read_kernel(cons
 }  // namespace
 }  // namespace areno
 
-extern "C" int areno_hip_probe_stream_read(const void* base, const int32_t* page_ids, int64_t pages, int32_t page_bytes,
-                                           void* sink, void* stream) {
+extern "C" int areno_hip_probe_stream_read(const void* base_a, const void* base_b, const int32_t* page_ids, int64_t pages,
+                                           int32_t page_bytes, void* sink, void* stream) {
   const char* op = "areno_hip_probe_stream_read";
-  if (base == nullptr || sink == nullptr || pages < 0 || page_bytes < 1024 || page_bytes % 1024 != 0)
+  if (base_a == nullptr || sink == nullptr || pages < 0 || page_bytes < 1024 || page_bytes % 1024 != 0)
     return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: NULL pointer, or page_bytes not a positive multiple of 1024", op);
-  if (reinterpret_cast<uintptr_t>(base) % 16 != 0) return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: base must be 16-byte aligned", op);
+  if (reinterpret_cast<uintptr_t>(base_a) % 16 != 0 || reinterpret_cast<uintptr_t>(base_b) % 16 != 0)
+    return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: the pools must be 16-byte aligned", op);
   if (pages == 0) return ARENO_OK;
   hipLaunchKernelGGL(areno::stream_read_kernel, dim3(areno::kProbeWorkgroups), dim3(areno::kProbeWaves * areno::kWave), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const char*>(base), page_ids, pages, page_bytes,
+                     static_cast<hipStream_t>(stream), static_cast<const char*>(base_a), static_cast<const char*>(base_b), page_ids, pages,
+                     page_bytes,
                      static_cast<uint32_t*>(sink));
   return areno::check_launch(op);
 }

@@ -223,8 +223,8 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
 
 
 def measure_stream_ceiling(w, pools, iters=10, samples=9):
-    """GB/s of `areno_hip_probe_stream_read` (16-byte loads, a page per wave at a time, nothing computed) over the K and
-    V pools of all pool copies: every page in address order, and the distinct pages the block table names in a random order."""
+    """GB/s of `areno_hip_probe_stream_read` (16-byte loads, a page per wave at a time, nothing computed; one launch
+    reads a page set from the K and the V pool, as a decode launch does) over the K and V pools of all pool copies: every page in address order, and the distinct pages the block table names in a random order."""
     import torch
 
     from areno_amd.accel import cabi
@@ -240,11 +240,9 @@ def measure_stream_ceiling(w, pools, iters=10, samples=9):
 
     def timed(ids):
         def once():
-            for pool in pools:
-                cabi.probe_stream_read(pool[0], page_bytes, sink, ids)
-                cabi.probe_stream_read(pool[1], page_bytes, sink, ids)
+            return sum(cabi.probe_stream_read(pool[0], pool[1], page_bytes, sink, ids) for pool in pools)
 
-        once()
+        nbytes = once()
         torch.cuda.synchronize()
         out = []
         for _ in range(samples):
@@ -255,8 +253,7 @@ def measure_stream_ceiling(w, pools, iters=10, samples=9):
             e1.record()
             e1.synchronize()
             out.append(e0.elapsed_time(e1) * 1e-3 / iters)
-        pages = (pools[0][0].numel() * pools[0][0].element_size()) // page_bytes if ids is None else ids.numel()
-        return 2 * len(pools) * pages * page_bytes / statistics.median(out) / 1e9
+        return nbytes / statistics.median(out) / 1e9
 
     return {"linear_gbps": timed(None), "paged_gbps": timed(used), "page_bytes": page_bytes}
 

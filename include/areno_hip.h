@@ -337,14 +337,16 @@ int areno_hip_attention_backward(const void* grad_out, const void* q, const void
                                  size_t workspace_bytes, void* stream);
 
 /*
- * Measurement aid, no counterpart in the reference: reads `pages` runs of page_bytes bytes (page i starts at
- * base + page_ids[i] * page_bytes, or at base + i * page_bytes when page_ids is NULL) with 16-byte loads, workgroups
- * of four waves, one page per wave at a time, and computes nothing.  What this reaches over a set of KV pools is the
- * streaming ceiling the decode kernels' bandwidth is compared with (bench.py).
- *   base      device, 16-byte aligned;  page_bytes a multiple of 1024;  sink  device, >= 4 bytes (written practically never)
+ * Measurement aid, no counterpart in the reference: reads `pages` runs of page_bytes bytes from one pool or from two
+ * (page i starts at base + page_ids[i] * page_bytes, or at base + i * page_bytes when page_ids is NULL; base_b NULL =
+ * one pool) with 16-byte loads, one workgroup of four waves per CU, one page per wave at a time, and computes nothing.
+ * What this reaches over the K and V pools of a workload is the streaming ceiling the decode kernels' bandwidth is
+ * compared with (bench.py): same pages, same bytes per launch.
+ *   base_a, base_b  device, 16-byte aligned;  page_bytes a multiple of 1024;  sink  device, >= 4 bytes (written
+ *                   practically never)
  */
-int areno_hip_probe_stream_read(const void* base, const int32_t* page_ids, int64_t pages, int32_t page_bytes, void* sink,
-                                void* stream);
+int areno_hip_probe_stream_read(const void* base_a, const void* base_b, const int32_t* page_ids, int64_t pages,
+                                int32_t page_bytes, void* sink, void* stream);
 
 #ifdef __cplusplus
 }
