@@ -293,3 +293,37 @@ def test_prefix_groups_argument_checks():
     # a window switches the grouping off, the result is the plain op's
     out = _grouped_decode(w, window_left=40)
     assert_close(out, expected_decode(w, window_left=40), *tolerances("fp8"), what="window with groups")
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_draws_of_shape_length_window_and_cache_type(seed):
+    """Seeded random configurations through the whole op: cache type, head counts, head dim, page size, batch, window and
+    length distribution (empty rows, rows of a few tokens next to long ones, many short rows so that a wave's share of
+    the tiles crosses several rows).  Output against the oracle, append bit for bit over the whole pool."""
+    import random
+
+    rng = random.Random(1000 + seed)
+    kv = rng.choice(["bf16", "fp16", "int8", "fp8"])
+    hkv = rng.choice([1, 2, 4, 8])
+    group = rng.choice([1, 2, 4, 7, 8, 16])
+    d = rng.choice([64, 128])
+    bs = rng.choice([8, 16, 32, 64])
+    batch = rng.choice([1, 3, 17, 64, 130])
+    profile = rng.choice(["short", "mixed", "long"])
+    g = torch.Generator().manual_seed(seed)
+    if profile == "short":
+        lengths = torch.randint(0, 40, (batch,), generator=g)
+    elif profile == "mixed":
+        lengths = torch.where(torch.rand(batch, generator=g) < 0.7, torch.randint(0, 60, (batch,), generator=g),
+                              torch.randint(200, 3000, (batch,), generator=g))  # fmt: skip
+    else:
+        lengths = torch.randint(500, 2500, (batch,), generator=g)
+    window = rng.choice([None, None, 0, 33, 700])
+    w = workloads.make_decode_workload(f"draw-{seed}", seed=500 + seed, batch=batch, hq=hkv * group, hkv=hkv, d=d, bs=bs,
+                                       kv=kv, lengths=lengths, device=DEV, quantize_fn=gpu_quantize, poison=True,
+                                       act_dtype=torch.float16 if kv == "fp16" else torch.bfloat16)  # fmt: skip
+    before = _snapshot(w)
+    out = run_decode(w, window_left=window)
+    what = f"draw {seed}: {kv} {hkv * group}/{hkv} d={d} bs={bs} batch={batch} {profile} window={window}"
+    assert_close(out, expected_decode(w, window_left=window), *tolerances(kv), what=what)
+    _check_append(w, before)
