@@ -458,7 +458,7 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
   decode_mfma_fn mfma = nullptr;
   // the kernel indexes cache rows (block, slot, head) with 32 bits
   const bool rows_fit = static_cast<double>(cache->num_blocks) * cache->block_size * cache->kv_heads < 4294967296.0;
-  const bool mfma_ok = aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && num_splits != 1 && p.group <= 16 &&
+  const bool mfma_ok = aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && p.group <= 16 &&
                        batch <= kMfmaMaxBatch && rows_fit && p.bs_shift >= 0;
   if (mfma_ok) {
     const bool s16 = cache->scale_dtype == ARENO_DT_F16;

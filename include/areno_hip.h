@@ -84,8 +84,9 @@ int areno_hip_cache_write_decode(const areno_paged_cache* cache, const void* k_u
 
 /*
  * Bytes of device workspace areno_hip_paged_decode needs for these shapes (split-KV partials).
- * num_splits is the caller's hint (the reference passes 8, attention_backend/infer.py:240);
- * 1 forces a single partial per row, anything else lets the library pick the chunking.
+ * num_splits is the caller's hint (the reference passes 8, attention_backend/infer.py:240): the matrix-core kernel
+ * cuts the work by itself whatever the hint; on the vector-ALU kernels 1 forces a single partial per row and anything
+ * else lets the library pick the chunking.
  * Returns 0 for invalid shapes.
  */
 size_t areno_hip_paged_decode_workspace_bytes(int32_t batch, int32_t q_heads, int32_t head_dim, int32_t block_size,

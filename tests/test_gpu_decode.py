@@ -80,6 +80,7 @@ def test_fp16_query_with_quantized_cache():
     ("bf16", 28, 4, 128, 16), ("int8", 28, 4, 128, 16), ("fp8", 32, 8, 128, 16), ("bf16", 16, 2, 128, 256),
     ("int8", 4, 4, 64, 16), ("bf16", 6, 2, 128, 16), ("fp16", 12, 1, 64, 32), ("int8", 5, 1, 128, 8),
     ("bf16", 8, 2, 96, 16), ("bf16", 24, 2, 128, 16), ("fp8", 8, 8, 128, 48), ("fp32", 8, 2, 128, 16),
+    ("int8", 32, 1, 128, 16), ("bf16", 40, 2, 64, 16),  # more than 16 q heads per kv head: the vector-ALU kernels
 ])  # fmt: skip
 def test_shapes_head_ratios_and_block_sizes(kv, hq, hkv, d, bs):
     g = torch.Generator().manual_seed(hq * 131 + d)
