@@ -386,7 +386,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     row_g0 = (static_cast<uint32_t>(src.g0) * p.block_size + slot_of(lane_token(t, 0))) * p.kv_heads + kvh;
     row_g1 = (static_cast<uint32_t>(src.g1) * p.block_size + slot_of(lane_token(t, 1))) * p.kv_heads + kvh;
   };
-  auto issue_v_loads = [&](const TileDesc& t) {
+  // what an appended token's tile needs: the update rows (first 32 lanes K, the others V) and the cache row they go to
+  auto issue_update_loads = [&](const TileDesc& t) {
     if constexpr (DSPLIT == 1) {
       if ((t.kind & (kTileNewToken | kTilePhantom)) == kTileNewToken) {
         const void* src = lane < 32 ? mp.k_update : mp.v_update;
@@ -396,6 +397,9 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       }
       new_row = row_g0;
     }
+  };
+  auto issue_v_loads = [&](const TileDesc& t) {
+    issue_update_loads(t);
 #pragma unroll
     for (int tg = 0; tg < 2; ++tg) {
       const char* va = static_cast<const char*>(p.v_cache) + (tg ? row_g1 : row_g0) * row_bytes + half_bytes + lk * 16;
@@ -533,15 +537,23 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   };
 
   // ---- the token being appended: quantize, store into the page, fold into the running softmax (vector ALU) ---------
-  auto new_token_step = [&](const TileDesc& t) {
+  // `after_read` runs once the update rows are out of their load registers: the next tile's loads go out there, ahead
+  // of the arithmetic, which is long for a step that streams nothing (the next tile may be an appended token's as well
+  // and load into the same registers).
+  auto new_token_step = [&](const TileDesc& t, auto&& after_read) {
     if constexpr (DSPLIT == 1) {
       constexpr int EPU = 2 * UPW;  // elements of the row this lane holds: (lane % 32) * EPU ...
       const int sub = lane & 31;
       const bool is_v = lane >= 32;
       float x[EPU];
+      uint32_t raw_row[UPW];
+#pragma unroll
+      for (int w = 0; w < UPW; ++w) raw_row[w] = upd[w];
+      const int64_t dst_row = new_row;  // (the loads of the next tile replace it with theirs)
+      after_read();
 #pragma unroll
       for (int w = 0; w < UPW; ++w) {
-        const uint32_t word = upd[w];
+        const uint32_t word = raw_row[w];
         if (p.q_dtype == ARENO_DT_BF16) {
           x[2 * w] = bf16_bits_to_float(word & 0xffffu);
           x[2 * w + 1] = bf16_bits_to_float(word >> 16);
@@ -550,7 +562,6 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
           x[2 * w + 1] = f16_bits_to_float(word >> 16);
         }
       }
-      const int64_t dst_row = new_row;
       char* cache = static_cast<char*>(const_cast<void*>(is_v ? p.v_cache : p.k_cache));
       float xhat[EPU];  // what a reader of the page sees
       if constexpr (T::kQuant) {
@@ -609,7 +620,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
         // 16-bit pages hold the update row as it is (the launcher only fuses when the dtypes agree)
         char* dst = cache + dst_row * row_bytes + sub * (EPU * 2);
 #pragma unroll
-        for (int w = 0; w < UPW; ++w) *reinterpret_cast<uint32_t*>(dst + 4 * w) = upd[w];
+        for (int w = 0; w < UPW; ++w) *reinterpret_cast<uint32_t*>(dst + 4 * w) = raw_row[w];
 #pragma unroll
         for (int e = 0; e < EPU; ++e) xhat[e] = x[e];
       }
@@ -645,6 +656,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
         for (int j = 0; j < 4; ++j) acc[nb][j] = acc[nb][j] * alpha + pv * vv[j];
       }
       lds_fence();
+    } else {
+      after_read();  // (the split-head variant appends in a launch of its own and never gets here)
     }
   };
 
@@ -874,7 +887,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     // One step of the pipeline on the tile in the registers (tile x): the ids of tile x + 1 have arrived (requested a
     // step ago), those of tile x + 2 are requested, and tile x + 1's loads go out as `work` frees the V registers
     // (`between_v`) and the K registers (`between_k`).
-    auto step = [&](int x, auto&& work) {
+    auto step = [&](int x, auto&& work, auto stream_next) {
       ARENO_TRACE_POINT();
       const TileDesc t = desc0;
       const TileDesc nt = desc_ids;
@@ -888,16 +901,22 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
           t,
           [&]() {
             __builtin_amdgcn_sched_barrier(0);
-            issue_v_loads(nt);
+            if constexpr (decltype(stream_next)::value) {
+              issue_v_loads(nt);
+            } else {
+              issue_update_loads(nt);  // the next tile is an appended token's: it streams nothing
+            }
             __builtin_amdgcn_sched_barrier(0);
           },
           [&]() {
             __builtin_amdgcn_sched_barrier(0);
-            issue_k_loads(nt);
+            if constexpr (decltype(stream_next)::value) issue_k_loads(nt);
             __builtin_amdgcn_sched_barrier(0);
           });
       desc0 = nt;
     };
+    using std::false_type;
+    using std::true_type;
 
     // The unit as a sequence of item segments: the tiles of one item that fall into the unit.  The loop over a
     // segment's regular tiles has no item logic in it (so nothing but the tile stream is carried around it); the
@@ -915,14 +934,25 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
         const ItemInfo it2 = item_info<GROUPED>(shape, lens, b2);
         issue_q_loads(b2, it2.row, it2.nseq);
       }
-      for (; x < regular_end; ++x)
-        step(x, [&](const TileDesc& t, auto&& between_v, auto&& between_k) { tile_step(t, between_v, between_k); });
+      // An appended token's tile streams nothing, so the regular tile in front of it fetches only the update rows,
+      // and the tile behind it is requested at the start of the appended token's own step.
+      auto regular = [&](const TileDesc& t, auto&& between_v, auto&& between_k) { tile_step(t, between_v, between_k); };
+      const int streaming_end = regular_end - (appended ? 1 : 0);
+      for (; x < streaming_end; ++x) step(x, regular, true_type{});
       if (appended) {
-        step(x, [&](const TileDesc& t, auto&& between_v, auto&& between_k) {
-          new_token_step(t);
-          between_v();
-          between_k();
-        });
+        if (x < regular_end) {
+          step(x, regular, false_type{});
+          ++x;
+        }
+        step(
+            x,
+            [&](const TileDesc& t, auto&& between_v, auto&& between_k) {
+              new_token_step(t, [&]() {
+                between_v();
+                between_k();
+              });
+            },
+            true_type{});
         ++x;
       }
       write_partial(first.b, first.row, first.nseq);
