@@ -374,125 +374,145 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
     }
 
     // ---- the tile pipeline -----------------------------------------------------------------------------------------
-    int ids_n[NLD], ids_k[NLD];
-    uint4_t kreg[NLD], vreg[NLD];
-    scale_raw_t ksreg[NLD], vsreg[NLD];
+    // What one staging step fetches is published two steps later, so a fetch has two tile steps to arrive; block ids
+    // are fetched two steps ahead of the chunk they locate.  Two sets of fetch registers alternate from step to step
+    // (the tile loop is unrolled by two, so which set a step uses is fixed at compile time).
+    struct FetchSet {
+      int ids[NLD], keys[NLD];  // block id and key position of the tile to fetch next into this set
+      uint4_t kreg[NLD], vreg[NLD];
+      scale_raw_t ksreg[NLD], vsreg[NLD];
+      uint32_t k_row[NLD];  // page row of the K chunk in this set: the V chunk of the same tile is fetched a step later
+    };
+    FetchSet set_a, set_b;
+    {
+      FetchSet zero;
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      ids_n[i] = ids_k[i] = 0;
-      kreg[i] = vreg[i] = uint4_t{0u, 0u, 0u, 0u};
-      ksreg[i] = vsreg[i] = scale_raw_t(0);
+      for (int i = 0; i < NLD; ++i) {
+        zero.ids[i] = zero.keys[i] = 0;
+        zero.kreg[i] = zero.vreg[i] = uint4_t{0u, 0u, 0u, 0u};
+        zero.ksreg[i] = zero.vsreg[i] = scale_raw_t(0);
+        zero.k_row[i] = 0;
+      }
+      set_a = zero;
+      set_b = zero;
     }
-    auto key_of = [&](int tile, int i) { return max(0, min(tile * TK + chunk_tok[i], key_hi)); };
-    auto load_ids = [&](int tile) {
+    // Addresses.  The cache row of key t is page_row * kv_heads + kvh with page_row = (block id << bs_shift) + t's slot
+    // (packed K/V: q_begin + t), so a chunk's byte address is one 32 x 32 -> 64-bit multiply-add on a base that already
+    // holds the pool, the head and the chunk's column (the launcher checks that page rows fit 32 bits).  The key a
+    // block id was fetched for travels with the id.
+    const uint32_t row_stride = static_cast<uint32_t>(p.kv_heads) * static_cast<uint32_t>(row_bytes);
+    const uint32_t scale_stride = static_cast<uint32_t>(p.kv_heads) * static_cast<uint32_t>(sizeof(scale_raw_t));
+    const uint32_t slot_mask = static_cast<uint32_t>(p.block_size - 1);
+    auto chunk_base = [&](const void* pool, int i) {
+      return static_cast<const char*>(pool) + static_cast<int64_t>(kvh) * row_bytes + chunk_col[i] * 16;
+    };
+    auto scale_base = [&](const void* pool) {
+      return static_cast<const char*>(pool) + static_cast<int64_t>(kvh) * static_cast<int64_t>(sizeof(scale_raw_t));
+    };
+    auto chunk_at = [&](const char* base, uint32_t page_row) {
+      return *reinterpret_cast<const uint4_t*>(base + static_cast<uint64_t>(page_row) * row_stride);
+    };
+    auto scale_at = [&](const char* base, uint32_t page_row) {
+      return *reinterpret_cast<const scale_raw_t*>(base + static_cast<uint64_t>(page_row) * scale_stride);
+    };
+    auto load_ids = [&](FetchSet& f, int tile) {
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
-        const int t = key_of(tile, i);
-        ids_n[i] = table_row[packed ? 0 : (t >> p.bs_shift)];
+        f.keys[i] = max(0, min(tile * TK + chunk_tok[i], key_hi));
+        f.ids[i] = table_row[packed ? 0 : (f.keys[i] >> p.bs_shift)];
       }
     };
-    auto cache_row = [&](int tile, int i) -> int64_t {
-      const int t = key_of(tile, i);
-      // page size is a power of two here (the launcher sends other sizes to the generic kernel); packed K/V run as
-      // one page per token with the token's row as its id
-      const int slot = t & (p.block_size - 1);
-      const int64_t page_row = packed ? static_cast<int64_t>(q_begin) + t
-                                      : (static_cast<int64_t>(ids_k[i]) << p.bs_shift) + slot;
-      return page_row * p.kv_heads + kvh;
-    };
-    int64_t v_row[NLD];  // cache row of the K chunk in flight: its V chunk is fetched one iteration later
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) v_row[i] = 0;
-    auto issue_v = [&]() {
-#pragma unroll
-      for (int i = 0; i < NLD; ++i) {
-        vreg[i] = load16(p.v_cache, v_row[i] * row_bytes + chunk_col[i] * 16);
-        if constexpr (T::kQuant) vsreg[i] = static_cast<const scale_raw_t*>(p.v_scale)[v_row[i]];
-      }
-    };
-    auto issue_k = [&](int tile) {
-#pragma unroll
-      for (int i = 0; i < NLD; ++i) {
-        const int64_t row = cache_row(tile, i);
-        v_row[i] = row;
-        kreg[i] = load16(p.k_cache, row * row_bytes + chunk_col[i] * 16);
-        if constexpr (T::kQuant) ksreg[i] = static_cast<const scale_raw_t*>(p.k_scale)[row];
-      }
+    // page size is a power of two here (the launcher sends other sizes to the generic kernel); packed K/V run as one
+    // page per token with the token's row as its id
+    auto page_row_of = [&](const FetchSet& f, int i) -> uint32_t {
+      const uint32_t paged = (static_cast<uint32_t>(f.ids[i]) << p.bs_shift) + (static_cast<uint32_t>(f.keys[i]) & slot_mask);
+      return packed ? static_cast<uint32_t>(q_begin + f.keys[i]) : paged;
     };
     // The empty asm pins the use of a fetched chunk to this point of the iteration: without it the compiler converts
     // the codes right at the top of the loop and every tile waits there for the loads it has just issued.
-    auto publish_k = [&](int tile) {
+    auto publish_k = [&](FetchSet& f, int tile) {
       char* kd = s_k[tile & 1];
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
-        asm volatile("" : "+v"(kreg[i]));
+        asm volatile("" : "+v"(f.kreg[i]));
         if (!chunk_live[i]) continue;
         const int t = chunk_tok[i];
         if constexpr (T::kQuant) {
           uint4_t lo, hi;
-          dequant_chunk<KIND>(kreg[i], scale_value(ksreg[i]), lo, hi);
+          dequant_chunk<KIND>(f.kreg[i], scale_value(f.ksreg[i]), lo, hi);
           char* kdst = kd + t * RSK + chunk_col[i] * 32;
           *reinterpret_cast<uint4_t*>(kdst) = lo;
           *reinterpret_cast<uint4_t*>(kdst + 16) = hi;
         } else {
-          *reinterpret_cast<uint4_t*>(kd + t * RSK + chunk_col[i] * 16) = kreg[i];
+          *reinterpret_cast<uint4_t*>(kd + t * RSK + chunk_col[i] * 16) = f.kreg[i];
         }
       }
     };
-    auto publish_v = [&](int tile) {
+    auto publish_v = [&](FetchSet& f, int tile) {
       char* vd = s_v[tile & 1];
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
-        asm volatile("" : "+v"(vreg[i]));
+        asm volatile("" : "+v"(f.vreg[i]));
         if (!chunk_live[i]) continue;
         const int t = chunk_tok[i];
         if constexpr (T::kQuant) {
           uint4_t lo, hi;
-          dequant_chunk<KIND>(vreg[i], scale_value(vsreg[i]), lo, hi);
+          dequant_chunk<KIND>(f.vreg[i], scale_value(f.vsreg[i]), lo, hi);
           char* vdst = vd + v_row_of(t) * RSV + chunk_col[i] * 32;
           *reinterpret_cast<uint4_t*>(vdst) = lo;
           *reinterpret_cast<uint4_t*>(vdst + 16) = hi;
         } else {
-          *reinterpret_cast<uint4_t*>(vd + v_row_of(t) * RSV + chunk_col[i] * 16) = vreg[i];
+          *reinterpret_cast<uint4_t*>(vd + v_row_of(t) * RSV + chunk_col[i] * 16) = f.vreg[i];
         }
       }
     };
-    // Staging step of iteration t: K[t + 2] and V[t + 1] go from the registers into the LDS buffers the previous
-    // iteration was the last to read, then K[t + 3], V[t + 2] and the block ids of tile t + 4 are fetched.  It runs for
-    // every t (key positions are clamped into the item's range): tiles outside [ta, tb] land in buffers nobody reads.
-    auto stage = [&](int t) {
+    const char* const role_base = chunk_base(role_v ? p.v_cache : p.k_cache, 0);
+    const char* const role_scale_base = scale_base(role_v ? p.v_scale : p.k_scale);
+    // Staging step of iteration t with the fetch set `mine` of its parity (`other` is the previous and the next
+    // step's): K[t + 2] and V[t + 1], fetched two steps ago, go from the registers into the LDS buffers the previous
+    // iteration was the last to read; then K[t + 4] and V[t + 3] are fetched into the same registers, and the block
+    // ids of K[t + 6] / V[t + 5].  It runs for every t (key positions are clamped into the item's range): tiles
+    // outside [ta, tb] land in buffers nobody reads.
+    auto stage = [&](int t, FetchSet& mine, FetchSet& other) {
       if constexpr (kRoleSplit) {
         // one chunk per thread: kreg / ksreg / ids hold the K chunk in a K wave and the V chunk in a V wave.  V runs
-        // one tile behind K, as in the unsplit scheme: published V[t + 1] / K[t + 2], fetched V[t + 2] / K[t + 3],
-        // ids of V[t + 3] / K[t + 4].
+        // one tile behind K, as in the unsplit scheme.
         const int behind = role_v ? 1 : 0;
-        asm volatile("" : "+v"(kreg[0]));
+        asm volatile("" : "+v"(mine.kreg[0]));
         if (chunk_live[0]) {
           const int tk = chunk_tok[0];
           const int pub = t + 2 - behind;
           char* dst = role_v ? s_v[pub & 1] + v_row_of(tk) * RSV : s_k[pub & 1] + tk * RSK;
           if constexpr (T::kQuant) {
             uint4_t lo, hi;
-            dequant_chunk<KIND>(kreg[0], scale_value(ksreg[0]), lo, hi);
+            dequant_chunk<KIND>(mine.kreg[0], scale_value(mine.ksreg[0]), lo, hi);
             *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 32) = lo;
             *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 32 + 16) = hi;
           } else {
-            *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 16) = kreg[0];
+            *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 16) = mine.kreg[0];
           }
         }
-        ids_k[0] = ids_n[0];
-        const int64_t row = cache_row(t + 3 - behind, 0);
-        kreg[0] = load16(role_v ? p.v_cache : p.k_cache, row * row_bytes + chunk_col[0] * 16);
-        if constexpr (T::kQuant) ksreg[0] = static_cast<const scale_raw_t*>(role_v ? p.v_scale : p.k_scale)[row];
-        load_ids(t + 4 - behind);
+        const uint32_t row = page_row_of(mine, 0);  // the ids of tile t + 4 - behind, fetched two steps ago
+        mine.kreg[0] = chunk_at(role_base, row);
+        if constexpr (T::kQuant) mine.ksreg[0] = scale_at(role_scale_base, row);
+        load_ids(mine, t + 6 - behind);
       } else {
-        publish_k(t + 2);
-        publish_v(t + 1);
-        issue_v();  // rows of tile t + 2, remembered when its K chunk was fetched
+        publish_k(mine, t + 2);
+        publish_v(mine, t + 1);
 #pragma unroll
-        for (int i = 0; i < NLD; ++i) ids_k[i] = ids_n[i];
-        issue_k(t + 3);
-        load_ids(t + 4);
+        for (int i = 0; i < NLD; ++i) {
+          // V[t + 3]: the rows of K[t + 3], which the previous step fetched
+          mine.vreg[i] = chunk_at(chunk_base(p.v_cache, i), other.k_row[i]);
+          if constexpr (T::kQuant) mine.vsreg[i] = scale_at(scale_base(p.v_scale), other.k_row[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+          const uint32_t row = page_row_of(mine, i);  // the ids of tile t + 4, fetched two steps ago
+          mine.k_row[i] = row;
+          mine.kreg[i] = chunk_at(chunk_base(p.k_cache, i), row);
+          if constexpr (T::kQuant) mine.ksreg[i] = scale_at(scale_base(p.k_scale), row);
+        }
+        load_ids(mine, t + 6);
       }
     };
 
@@ -517,10 +537,12 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
       }
     };
 
-    // ---- fill the pipe: after these iterations K[ta], K[ta + 1] and V[ta] are in LDS ---------------------------------
-    for (int t = ta - 4; t < ta; ++t) {
+    // ---- fill the pipe: after these iterations K[ta], K[ta + 1] and V[ta] are in LDS (the first ones only fetch) ------
+    for (int t = ta - 6; t < ta; t += 2) {
       __syncthreads();
-      stage(t);
+      stage(t, set_a, set_b);
+      __syncthreads();
+      stage(t + 1, set_b, set_a);
     }
     __syncthreads();
     if (wave_live) scores(ta, s_cur);
@@ -531,9 +553,10 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
     // with the two arrays swapped: the scores of the next tile are then computed where the following step reads them
     // and no per-tile register copy of the 8 * kRowTiles scores is left.
     float s_alt[kRowTiles][2][4];
-    auto tile_step = [&](int t, float (&s_cur)[kRowTiles][2][4], float (&s_next)[kRowTiles][2][4]) {
+    auto tile_step = [&](int t, float (&s_cur)[kRowTiles][2][4], float (&s_next)[kRowTiles][2][4], FetchSet& mine,
+                         FetchSet& other) {
       __syncthreads();
-      stage(t);
+      stage(t, mine, other);
       if (!wave_live) return;
       const int k0 = t * TK;
       const bool need_mask = k0 + TK - 1 > wave_qmin || (p.window_left >= 0 && k0 < wave_qmax - p.window_left);
@@ -646,9 +669,9 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
       }
     };
     for (int t = ta; t <= tb; t += 2) {
-      tile_step(t, s_cur, s_alt);
+      tile_step(t, s_cur, s_alt, set_a, set_b);
       if (t + 1 > tb) break;
-      tile_step(t + 1, s_alt, s_cur);
+      tile_step(t + 1, s_alt, s_cur, set_b, set_a);
     }
 
     // ---- finish the segment: final rows go to `out`, a cut item leaves its partial in the workspace ---------------
@@ -884,6 +907,8 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   if (log2_exact_i(cache->block_size) < 0) return ARENO_ERR_UNSUPPORTED;  // page addressing by shift and mask
   if (group > 16 || num_seqs > kMaxPrefillSeqs || tokens > 0x3fffffff) return ARENO_ERR_UNSUPPORTED;
   if (cache->kv_heads > 65535) return ARENO_ERR_UNSUPPORTED;
+  // page rows (block id * page size + slot, or token rows of packed K/V) are 32-bit in the kernel's address arithmetic
+  if (block_table != nullptr && cache->num_blocks * cache->block_size > 0xffffffffLL) return ARENO_ERR_UNSUPPORTED;
   if (reinterpret_cast<uintptr_t>(cache->k) % 16 != 0 || reinterpret_cast<uintptr_t>(cache->v) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(q) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 8 != 0)
     return ARENO_ERR_UNSUPPORTED;
