@@ -58,129 +58,183 @@ __device__ __forceinline__ float round_to(float x, int dtype) {
   return dtype == ARENO_DT_BF16 ? bf16_bits_to_float(float_to_bf16_bits(x)) : f16_bits_to_float(float_to_f16_bits(x));
 }
 
+// Two values rounded to the activation dtype, as floats: one packed conversion and two unpacking steps for bf16
+template <int ACT>
+__device__ __forceinline__ void round_pair(float& a, float& b) {
+  if constexpr (ACT == ARENO_DT_BF16) {
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{a, b}, bf16x2_t));
+    a = __builtin_bit_cast(float, w << 16);
+    b = __builtin_bit_cast(float, w & 0xffff0000u);
+  } else {
+    a = round_to(a, ACT);
+    b = round_to(b, ACT);
+  }
+}
+
 // Row layout: a row of D elements is held by LPR = D / 8 adjacent lanes, 8 consecutive elements (16 bytes of 16-bit
 // activations) per lane, so a wave64 carries 64 / LPR rows and every global access is a 16-byte one.  The rotary
 // partner of element i (i +- D/2) is the same element slot of lane ^ (LPR / 2).
-template <int LPR>
-__device__ __forceinline__ float group_sum(float x) {
+//
+// Exchanges inside a 16-lane row go through the vector ALU's lane-permute modifiers instead of the LDS crossbar:
+// lane ^ 1 and lane ^ 2 are quad permutes; after those the four lanes of a quad agree, so mirroring the row's halves
+// (lane -> 7 - lane in each 8) and then the row (lane -> 15 - lane) fetch what lane ^ 4 and lane ^ 8 hold; a rotation
+// by 8 is lane ^ 8 exactly.
+template <int CTRL>
+__device__ __forceinline__ float row_permute(float x) {
+  const int v = __builtin_bit_cast(int, x);
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(v, v, CTRL, 0xf, 0xf, false));
+}
+constexpr int kDppQuadXor1 = 0xB1;     // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;     // quad_perm:[2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // row_half_mirror
+constexpr int kDppMirror = 0x140;      // row_mirror
+constexpr int kDppRotate8 = 0x128;     // row_ror:8
+
+// all-reduce over the LPR lanes of a row with `op`, every lane ends with the result (the combination order is that of
+// an xor butterfly over masks 1, 2, 4, ...)
+template <int LPR, typename Op>
+__device__ __forceinline__ float group_reduce(float x, Op op) {
+  if constexpr (LPR >= 2) x = op(x, row_permute<kDppQuadXor1>(x));
+  if constexpr (LPR >= 4) x = op(x, row_permute<kDppQuadXor2>(x));
+  if constexpr (LPR >= 8) x = op(x, row_permute<kDppHalfMirror>(x));
+  if constexpr (LPR >= 16) x = op(x, row_permute<kDppMirror>(x));
 #pragma unroll
-  for (int m = 1; m < LPR; m <<= 1) x += wave_xor(x, m);
+  for (int m = 16; m < LPR; m <<= 1) x = op(x, wave_xor(x, m));
   return x;
 }
 
-constexpr int kRowsPerGroup = 1;  // rows a lane group works through (more than one measured slower: 53 vs 36 us at 4)
+template <int LPR>
+__device__ __forceinline__ float rotary_partner(float x) {
+  if constexpr (LPR == 16) {
+    return row_permute<kDppRotate8>(x);
+  } else {
+    return wave_xor(x, LPR / 2);
+  }
+}
 
-template <int LPR, int ACT>  // ACT: the activation dtype (ARENO_DT_F16 / ARENO_DT_BF16): no rounding step branches on it
+// ACT: the activation dtype (ARENO_DT_F16 / ARENO_DT_BF16): no rounding step branches on it.  The launcher checks that
+// rows, element offsets of q / k / v and page rows fit 32 bits, so the index arithmetic is 32-bit: one division per
+// wave (rows of a wave are consecutive) and multiply-adds of 24-bit factors.
+template <int LPR, int ACT>
 __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
   constexpr int D = LPR * 8;
   constexpr int kRowsPerWave = kWave / LPR;
-  constexpr int R = kRowsPerGroup;
   const int lane = threadIdx.x & (kWave - 1);
   const int sub = lane % LPR;  // which 8 elements of the row
-  const int heads = p.q_heads + 2 * p.kv_heads;
-  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + (threadIdx.x >> 6);
-  const int64_t total = p.tokens * heads;
+  const uint32_t heads = static_cast<uint32_t>(p.q_heads + 2 * p.kv_heads);
+  const uint32_t total = static_cast<uint32_t>(p.tokens) * heads;
+  const uint32_t wave_row =
+      (blockIdx.x * (blockDim.x / kWave) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) * kRowsPerWave;
 
-  // ---- fetch: row r of this lane group is wave_base + r * rows_per_wave + group, so each load instruction of the
-  // wave covers 1 KB of consecutive rows --------------------------------------------------------------------------
-  bool live[R];
-  int kind[R], head[R];
-  int64_t token[R], src_base[R], pos[R];
-  uint4_t raw[R];
+  // ---- which row: (token, head slot) of the wave's first row by one scalar division, the lane group's from there ---
+  const uint32_t row_raw = wave_row + lane / LPR;
+  const bool live = row_raw < total;
+  const uint32_t first = min(wave_row, total - 1);  // idle lane groups shadow the last row and store nothing
+  uint32_t token = first / heads;
+  uint32_t slot = first - token * heads + min(static_cast<uint32_t>(lane / LPR), total - 1 - first);
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int64_t row_raw = (wave_id * R + r) * kRowsPerWave + lane / LPR;
-    live[r] = row_raw < total;
-    const int64_t row = live[r] ? row_raw : total - 1;  // idle lane groups shadow the last row and store nothing
-    token[r] = row / heads;
-    const int slot = static_cast<int>(row - token[r] * heads);
-    kind[r] = slot < p.q_heads ? 0 : (slot < p.q_heads + p.kv_heads ? 1 : 2);  // q, k, v
-    head[r] = kind[r] == 0 ? slot : (kind[r] == 1 ? slot - p.q_heads : slot - p.q_heads - p.kv_heads);
-    const void* src = kind[r] == 0 ? p.q : (kind[r] == 1 ? p.k : p.v);
-    const int src_heads = kind[r] == 0 ? p.q_heads : p.kv_heads;
-    src_base[r] = (token[r] * src_heads + head[r]) * D + sub * 8;
-    raw[r] = *reinterpret_cast<const uint4_t*>(static_cast<const char*>(src) + src_base[r] * 2);
-    pos[r] = p.positions[token[r]];
+  for (int i = 0; i < 3; ++i) {  // heads >= 3 and at most 7 rows further on: at most three tokens further
+    const bool wrap = slot >= heads;
+    slot -= wrap ? heads : 0u;
+    token += wrap ? 1u : 0u;
   }
-  float4_t c0[R], c1[R], s0[R], s1[R];
+  const int kind = slot < static_cast<uint32_t>(p.q_heads) ? 0 : (slot < static_cast<uint32_t>(p.q_heads + p.kv_heads) ? 1 : 2);
+  const uint32_t head = kind == 0 ? slot : (kind == 1 ? slot - p.q_heads : slot - p.q_heads - p.kv_heads);
+  const void* src = kind == 0 ? p.q : (kind == 1 ? p.k : p.v);
+  const uint32_t src_heads = kind == 0 ? p.q_heads : p.kv_heads;
+  const uint32_t src_elem = (__umul24(token, src_heads) + head) * D + sub * 8;
+  const uint4_t raw = *reinterpret_cast<const uint4_t*>(static_cast<const char*>(src) + static_cast<uint64_t>(src_elem) * 2);
+  const int64_t pos = p.positions[token];
+  const uint32_t pc = pos < 0 ? 0u : (pos >= p.max_pos ? static_cast<uint32_t>(p.max_pos - 1) : static_cast<uint32_t>(pos));
+  const float* cos_row = p.cos + static_cast<uint64_t>(pc * D + sub * 8);
+  const float* sin_row = p.sin + static_cast<uint64_t>(pc * D + sub * 8);
+  const float4_t c0 = *reinterpret_cast<const float4_t*>(cos_row);
+  const float4_t c1 = *reinterpret_cast<const float4_t*>(cos_row + 4);
+  const float4_t s0 = *reinterpret_cast<const float4_t*>(sin_row);
+  const float4_t s1 = *reinterpret_cast<const float4_t*>(sin_row + 4);
+
+  float x[8];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int64_t pc = pos[r] < 0 ? 0 : (pos[r] >= p.max_pos ? p.max_pos - 1 : pos[r]);
-    const float* cos_row = p.cos + pc * D + sub * 8;
-    const float* sin_row = p.sin + pc * D + sub * 8;
-    c0[r] = *reinterpret_cast<const float4_t*>(cos_row);
-    c1[r] = *reinterpret_cast<const float4_t*>(cos_row + 4);
-    s0[r] = *reinterpret_cast<const float4_t*>(sin_row);
-    s1[r] = *reinterpret_cast<const float4_t*>(sin_row + 4);
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t word = raw[j];
+    if (ACT == ARENO_DT_BF16) {
+      x[2 * j] = bf16_bits_to_float(word & 0xffffu);
+      x[2 * j + 1] = __builtin_bit_cast(float, word & 0xffff0000u);
+    } else {
+      x[2 * j] = f16_bits_to_float(word & 0xffffu);
+      x[2 * j + 1] = f16_bits_to_float(word >> 16);
+    }
   }
 
+  // ---- q and k rows: norm and rotary (selects, not branches, keep every lane in the cross-lane steps) --------------
+  const float* weight = kind == 0 ? p.q_weight : (kind == 1 ? p.k_weight : nullptr);
+  {
+    float sum_sq = 0.0f;
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    float x[8];
+    for (int j = 0; j < 8; ++j) sum_sq += x[j] * x[j];
+    sum_sq = group_reduce<LPR>(sum_sq, [](float a, float b) { return a + b; });
+    if (weight != nullptr) {
+      const float inv = rsqrtf(sum_sq / static_cast<float>(D) + p.eps);
+      const float4_t w0 = *reinterpret_cast<const float4_t*>(weight + sub * 8);
+      const float4_t w1 = *reinterpret_cast<const float4_t*>(weight + sub * 8 + 4);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t word = raw[r][j];
-      if (ACT == ARENO_DT_BF16) {
-        x[2 * j] = bf16_bits_to_float(word & 0xffffu);
-        x[2 * j + 1] = bf16_bits_to_float(word >> 16);
-      } else {
-        x[2 * j] = f16_bits_to_float(word & 0xffffu);
-        x[2 * j + 1] = f16_bits_to_float(word >> 16);
+      for (int j = 0; j < 8; j += 2) {
+        float a = x[j] * inv * (j < 4 ? w0[j & 3] : w1[j & 3]);
+        float b = x[j + 1] * inv * (j < 4 ? w0[(j + 1) & 3] : w1[(j + 1) & 3]);
+        round_pair<ACT>(a, b);
+        x[j] = a;
+        x[j + 1] = b;
       }
     }
-
-    // ---- q and k rows: norm and rotary (selects, not branches, keep every lane in the cross-lane steps) ----------
-    const float* weight = kind[r] == 0 ? p.q_weight : (kind[r] == 1 ? p.k_weight : nullptr);
-    {
-      float sum_sq = 0.0f;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) sum_sq += x[j] * x[j];
-      sum_sq = group_sum<LPR>(sum_sq);
-      if (weight != nullptr) {
-        const float inv = rsqrtf(sum_sq / static_cast<float>(D) + p.eps);
-        const float4_t w0 = *reinterpret_cast<const float4_t*>(weight + sub * 8);
-        const float4_t w1 = *reinterpret_cast<const float4_t*>(weight + sub * 8 + 4);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          x[j] = round_to(x[j] * inv * w0[j], ACT);
-          x[4 + j] = round_to(x[4 + j] * inv * w1[j], ACT);
-        }
-      }
-    }
-    float partner[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) partner[j] = wave_xor(x[j], LPR / 2);
-    if (kind[r] != 2) {
-      const bool low_half = sub < LPR / 2;  // rotate_half: -x[i + D/2] below D/2, x[i - D/2] above
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float c = round_to(j < 4 ? c0[r][j & 3] : c1[r][j & 3], ACT);
-        const float sn = round_to(j < 4 ? s0[r][j & 3] : s1[r][j & 3], ACT);
-        const float rot = low_half ? -partner[j] : partner[j];
-        x[j] = round_to(round_to(x[j] * c, ACT) + round_to(rot * sn, ACT), ACT);
-      }
-      void* out = kind[r] == 0 ? p.q_out : p.k_out;
-      if (out != nullptr && live[r]) {
-        const uint4_t packed = {pack_two_16(x[0], x[1], ACT), pack_two_16(x[2], x[3], ACT),
-                                pack_two_16(x[4], x[5], ACT), pack_two_16(x[6], x[7], ACT)};
-        *reinterpret_cast<uint4_t*>(static_cast<char*>(out) + src_base[r] * 2) = packed;
-      }
-    }
-
-    // ---- k and v rows: into the page, through the cache writer's closed forms --------------------------------------
-    float amax = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(x[j]));
-    amax = lane_group_max<LPR>(amax);
-    if (kind[r] == 0 || !live[r]) continue;
-    void* cache = p.cache[kind[r] - 1];
-    if (cache == nullptr) continue;
-    const int64_t blk = p.block_ids[token[r]];
-    const int64_t off = p.block_offsets[token[r]];
-    if (blk < 0 || blk >= p.num_blocks || off < 0 || off >= p.block_size) continue;
-    const int64_t dst_row = (blk * p.block_size + off) * p.kv_heads + head[r];
-    store_row_slice(x, amax, sub, dst_row, D, cache, p.scale[kind[r] - 1], p.cache_dtype, p.scale_dtype);
   }
+  float partner[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) partner[j] = rotary_partner<LPR>(x[j]);
+  if (kind != 2) {
+    // rotate_half: -x[i + D/2] below D/2, x[i - D/2] above; the sign goes onto the (rounded) sine, which leaves every
+    // rounded product what it was
+    const uint32_t sign = sub < LPR / 2 ? 0x80000000u : 0u;
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+      float ca = j < 4 ? c0[j & 3] : c1[j & 3], cb = j < 4 ? c0[(j + 1) & 3] : c1[(j + 1) & 3];
+      float sa = j < 4 ? s0[j & 3] : s1[j & 3], sb = j < 4 ? s0[(j + 1) & 3] : s1[(j + 1) & 3];
+      round_pair<ACT>(ca, cb);
+      round_pair<ACT>(sa, sb);
+      sa = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, sa) ^ sign);
+      sb = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, sb) ^ sign);
+      float xa = x[j] * ca, xb = x[j + 1] * cb;
+      round_pair<ACT>(xa, xb);
+      float ra = partner[j] * sa, rb = partner[j + 1] * sb;
+      round_pair<ACT>(ra, rb);
+      float ya = xa + ra, yb = xb + rb;
+      round_pair<ACT>(ya, yb);
+      x[j] = ya;
+      x[j + 1] = yb;
+    }
+    void* out = kind == 0 ? p.q_out : p.k_out;
+    if (out != nullptr && live) {
+      const uint4_t packed = {pack_two_16(x[0], x[1], ACT), pack_two_16(x[2], x[3], ACT),
+                              pack_two_16(x[4], x[5], ACT), pack_two_16(x[6], x[7], ACT)};
+      *reinterpret_cast<uint4_t*>(static_cast<char*>(out) + static_cast<uint64_t>(src_elem) * 2) = packed;
+    }
+  }
+
+  // ---- k and v rows: into the page, through the cache writer's closed forms ------------------------------------------
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(x[j]));
+  amax = group_reduce<LPR>(amax, [](float a, float b) { return fmaxf(a, b); });
+  if (kind == 0 || !live) return;
+  void* cache = p.cache[kind - 1];
+  if (cache == nullptr) return;
+  const int64_t blk = p.block_ids[token];
+  const int64_t off = p.block_offsets[token];
+  if (blk < 0 || blk >= p.num_blocks || off < 0 || off >= p.block_size) return;
+  const uint32_t page_row = static_cast<uint32_t>(blk) * static_cast<uint32_t>(p.block_size) + static_cast<uint32_t>(off);
+  const int64_t dst_row = static_cast<int64_t>(static_cast<uint64_t>(page_row) * static_cast<uint32_t>(p.kv_heads) + head);
+  store_row_slice(x, amax, sub, dst_row, D, cache, p.scale[kind - 1], p.cache_dtype, p.scale_dtype);
 }
 
 typedef void (*rope_write_fn)(RopeWriteParams);
@@ -257,7 +311,14 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
   const rope_write_fn fn = rope_write_lookup(head_dim, dtype);
   if (fn == nullptr) return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim must be 64, 128, 256 or 512, got %d", op, head_dim);
   const int64_t rows = tokens * (q_heads + 2 * kv_heads);
-  const int rows_per_block = 4 * kRowsPerGroup * (kWave / (head_dim / 8));
+  // the kernel's index arithmetic: 32-bit rows and element offsets, 24-bit factors in the multiply-adds
+  if (tokens >= (1 << 24) || q_heads >= (1 << 24) || rows * head_dim >= 0x7fffffffLL ||
+      static_cast<int64_t>(max_pos) * head_dim >= 0x3fffffffLL)
+    return fail(ARENO_ERR_UNSUPPORTED, "%s: %lld tokens x %d heads x %d is past the kernel's 32-bit indexing", op,
+                static_cast<long long>(tokens), q_heads + 2 * kv_heads, head_dim);
+  if (cache != nullptr && cache->num_blocks * cache->block_size > 0xffffffffLL)
+    return fail(ARENO_ERR_UNSUPPORTED, "%s: the pool's page rows do not fit 32 bits", op);
+  const int rows_per_block = 4 * (kWave / (head_dim / 8));
   const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
   if (blocks > 0x7fffffffLL) return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: too many rows", op);
   hipLaunchKernelGGL(fn, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
