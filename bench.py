@@ -31,8 +31,8 @@ POOL_TARGET_BYTES = 1.3e9  # rotate over at least this much distinct KV
 # HBM bytes per launch of the dominant kernel as two rocprofv3 counter runs of this script recorded them (FETCH_SIZE,
 # scaled by the factor 2.0 that a copy of known size gives for it, plus WRITE_SIZE).  Recorded constants, not
 # measurements of the present run: the summaries they come from are under profiles/.
-PROFILED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 310.95e6, "cfg2-qwen7b-int8": 153.72e6, "cfg3-rollout-fp8": 1064.65e6,
-                          "cfg4-prefill-fp8": 1623.08e6}
+PROFILED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 310.91e6, "cfg2-qwen7b-int8": 153.71e6, "cfg3-rollout-fp8": 1065.34e6,
+                          "cfg4-prefill-fp8": 1624.88e6}
 PROFILED_TRAFFIC_SOURCE = {
     "decode": "recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script: profiles/decode_mfma_kernel_hbm_traffic_cfg1_cfg2_cfg3.md",
     "prefill": "recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script: profiles/prefill_mfma_kernel_hbm_traffic_cfg4.md",
@@ -468,7 +468,32 @@ def wave_trace(w, launches=12):
         summary.append(rec)
     keys = ("start", "work_list_ready", "tile0", "tile1", "tile2", "tile3", "finish")
     mean = {k: {s: float(np.mean([r[k][s] for r in summary])) for s in ("mean", "p10", "p50", "p90", "max")} for k in keys}
-    return {"workload": w.name, "launches_averaged": len(summary), "waves": summary[-1]["waves"], "us_since_first_wave_start": mean}
+    out = {"workload": w.name, "launches_averaged": len(summary), "waves": summary[-1]["waves"], "us_since_first_wave_start": mean}
+
+    # Who finishes last: waves by whether a row ends in their unit (plain launches of one workgroup row, where wave i
+    # belongs to unit i // 4: the tile range [u T / U, (u + 1) T / U) of the list "cached tiles + 1 per row").
+    waves = summary[-1]["waves"]
+    if hkv <= 4 and waves % 4 == 0:
+        lens = w.cache_seqlens.cpu().numpy().astype(np.int64)
+        cum = np.concatenate([[0], np.cumsum((lens + 31) // 32 + 1)])
+        units = waves // 4
+        starts = np.arange(units + 1) * cum[-1] // units
+        ends_in_unit = np.array([((cum[1:] > a) & (cum[1:] <= e)).sum() for a, e in zip(starts[:-1], starts[1:])])
+        has_end = ends_in_unit[np.arange(waves) // 4] > 0
+        groups = {"no_row_ends_in_unit": [], "a_row_ends_in_unit": []}
+        for t in runs[launches // 2:]:
+            t = t[:waves].astype(np.float64)
+            finish = (t[:, 6] - t[:, 0].min()) / 100.0
+            for name, sel in (("no_row_ends_in_unit", ~has_end), ("a_row_ends_in_unit", has_end)):
+                if sel.any():
+                    groups[name].append((int(sel.sum()), float(finish[sel].mean()), pct(finish[sel], 90), float(finish[sel].max())))
+        out["finish_by_row_end"] = {
+            name: {"waves": v[0][0], "mean": [min(x[1] for x in v), max(x[1] for x in v)],
+                   "p90": [min(x[2] for x in v), max(x[2] for x in v)], "max": [min(x[3] for x in v), max(x[3] for x in v)]}
+            for name, v in groups.items() if v
+        }  # fmt: skip
+        out["tiles_per_unit"] = [int((starts[1:] - starts[:-1]).min()), int((starts[1:] - starts[:-1]).max())]
+    return out
 
 
 def cpu_baseline(w, warmups=3, repeats=7):
