@@ -210,7 +210,9 @@ int areno_hip_paged_varlen_prefill(const areno_paged_cache* cache, const void* q
  *   cos, sin      device [max_pos, head_dim] float32 (the doubled-frequency tables of RotaryEmbedding)
  *   q_weight, k_weight  device [head_dim] float32, NULL = no norm on that tensor
  *   cache         NULL = no cache write (then block_ids / block_offsets are ignored)
- * head_dim 64, 128, 256 or 512; every tensor 16-byte aligned.
+ * head_dim 64, 128, 256 or 512; every tensor 16-byte aligned.  The kernel indexes with 32 bits: tokens < 2^24,
+ * tokens * (q_heads + 2 kv_heads) * head_dim < 2^31, max_pos * head_dim < 2^30, num_blocks * block_size < 2^32;
+ * anything larger returns ARENO_ERR_UNSUPPORTED before a launch (run it in token ranges).
  */
 int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache, const void* q, const void* k, const void* v,
                                        void* q_out, void* k_out, int32_t dtype, int64_t tokens, int32_t q_heads,

@@ -89,3 +89,34 @@ def test_argument_validation_runs_before_any_launch(lib):
     cache = Cache(0x1000, 0x1000, None, None, 4, 16, 2, 64, 2, 0)
     assert fn(ctypes.byref(cache), 0x1000, 0x1000, 1, 0, None, None, None) == -2  # f16 rows into a bf16 cache
     assert fn(ctypes.byref(cache), 0x1000, 0x1000, 2, 0, None, None, None) == 0  # zero tokens: nothing to do
+
+
+def test_the_fused_front_step_refuses_sizes_past_its_32_bit_indexing(lib):
+    """areno_hip_qk_norm_rope_cache_write indexes rows, elements and page rows with 32 bits; the launcher turns larger
+    problems down by name before anything is launched (fake pointers: nothing dereferences them)."""
+    class Cache(ctypes.Structure):
+        _fields_ = [("k", ctypes.c_void_p), ("v", ctypes.c_void_p), ("k_scale", ctypes.c_void_p),
+                    ("v_scale", ctypes.c_void_p), ("num_blocks", ctypes.c_int64), ("block_size", ctypes.c_int32),
+                    ("kv_heads", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("cache_dtype", ctypes.c_int32),
+                    ("scale_dtype", ctypes.c_int32)]  # fmt: skip
+
+    lib.areno_hip_last_error.restype = ctypes.c_char_p
+    fn = lib.areno_hip_qk_norm_rope_cache_write
+    fn.restype = ctypes.c_int
+    p, i32, i64, f32 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_float
+    fn.argtypes = [p, p, p, p, p, p, i32, i64, i32, i32, i32, p, p, p, i32, p, p, f32, p, p, p]
+    fake = 0x1000
+    bf16, unsupported = 2, -2
+
+    def call(cache, tokens, q_heads, kv_heads, d, max_pos=4096):
+        return fn(cache, fake, fake, fake, fake, fake, bf16, tokens, q_heads, kv_heads, d, fake, fake, fake, max_pos,
+                  None, None, 1e-6, fake, fake, None)  # fmt: skip
+
+    assert call(None, 1 << 24, 8, 2, 128) == unsupported  # 24-bit factors in the row arithmetic
+    assert b"32-bit" in lib.areno_hip_last_error()
+    assert call(None, 1 << 20, 32, 8, 128) == unsupported  # 2^20 x 48 rows x 128 elements
+    assert call(None, 16, 8, 2, 128, max_pos=1 << 24) == unsupported  # rotary table offsets
+    pool = Cache(fake, fake, None, None, 1 << 29, 16, 2, 128, bf16, 0)  # 2^33 page rows
+    assert call(ctypes.byref(pool), 16, 8, 2, 128) == unsupported
+    assert b"page rows" in lib.areno_hip_last_error()
+    assert call(None, 0, 8, 2, 128) == 0  # nothing to do
