@@ -250,6 +250,8 @@ rope_write_fn rope_write_lookup(int head_dim, int dtype) {
 }
 
 }  // namespace
+
+int64_t g_rope_tokens_per_launch = 0;  // test hook, see areno_hip_debug_set_rope_tokens_per_launch
 }  // namespace areno
 
 extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache, const void* q, const void* k,
@@ -310,17 +312,46 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
   p.eps = eps;
   const rope_write_fn fn = rope_write_lookup(head_dim, dtype);
   if (fn == nullptr) return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim must be 64, 128, 256 or 512, got %d", op, head_dim);
-  const int64_t rows = tokens * (q_heads + 2 * kv_heads);
-  // the kernel's index arithmetic: 32-bit rows and element offsets, 24-bit factors in the multiply-adds
-  if (tokens >= (1 << 24) || q_heads >= (1 << 24) || rows * head_dim >= 0x7fffffffLL ||
-      static_cast<int64_t>(max_pos) * head_dim >= 0x3fffffffLL)
-    return fail(ARENO_ERR_UNSUPPORTED, "%s: %lld tokens x %d heads x %d is past the kernel's 32-bit indexing", op,
-                static_cast<long long>(tokens), q_heads + 2 * kv_heads, head_dim);
+  // The kernel's index arithmetic is 32-bit (rows, element offsets of q / k / v, rotary table offsets, page rows), with
+  // 24-bit factors in its multiply-adds.  The table and the pool must fit as they are; a token count past the limits
+  // runs as consecutive launches over token ranges.
+  const int heads = q_heads + 2 * kv_heads;
+  if (heads >= (1 << 16) || static_cast<int64_t>(max_pos) * head_dim >= 0x3fffffffLL)
+    return fail(ARENO_ERR_UNSUPPORTED, "%s: %d heads, %d positions x %d are past the kernel's 32-bit indexing", op, heads,
+                max_pos, head_dim);
   if (cache != nullptr && cache->num_blocks * cache->block_size > 0xffffffffLL)
     return fail(ARENO_ERR_UNSUPPORTED, "%s: the pool's page rows do not fit 32 bits", op);
+  int64_t tokens_per_launch = 0x7fffffffLL / (static_cast<int64_t>(heads) * head_dim) - 1;
+  if (tokens_per_launch > (1 << 24) - 1) tokens_per_launch = (1 << 24) - 1;
+  if (g_rope_tokens_per_launch > 0 && g_rope_tokens_per_launch < tokens_per_launch)
+    tokens_per_launch = g_rope_tokens_per_launch;
+  if (tokens_per_launch < 1) return fail(ARENO_ERR_UNSUPPORTED, "%s: one token's rows are past 32-bit indexing", op);
   const int rows_per_block = 4 * (kWave / (head_dim / 8));
-  const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-  if (blocks > 0x7fffffffLL) return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: too many rows", op);
-  hipLaunchKernelGGL(fn, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
-  return check_launch(op);
+  const int64_t act_bytes = 2;
+  for (int64_t t0 = 0; t0 < tokens; t0 += tokens_per_launch) {
+    RopeWriteParams r = p;
+    r.tokens = tokens - t0 < tokens_per_launch ? tokens - t0 : tokens_per_launch;
+    const int64_t q_off = t0 * q_heads * head_dim * act_bytes, kv_off = t0 * kv_heads * head_dim * act_bytes;
+    r.q = static_cast<const char*>(q) + q_off;
+    r.k = static_cast<const char*>(k) + kv_off;
+    r.v = static_cast<const char*>(v) + kv_off;
+    r.q_out = static_cast<char*>(q_out) + q_off;
+    r.k_out = k_out == nullptr ? nullptr : static_cast<char*>(k_out) + kv_off;
+    r.positions = positions + t0;
+    r.block_ids = block_ids == nullptr ? nullptr : block_ids + t0;
+    r.block_offsets = block_offsets == nullptr ? nullptr : block_offsets + t0;
+    const int64_t rows = r.tokens * heads;
+    const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+    hipLaunchKernelGGL(fn, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), r);
+    if (int rc = check_launch(op)) return rc;
+  }
+  return ARENO_OK;
+}
+
+// Test hook: caps the tokens one launch of the fused front step takes (0 = only the kernel's own limit), so that the
+// walk over token ranges can be exercised at sizes a test can afford.  Returns the previous value.
+extern "C" int64_t areno_hip_debug_set_rope_tokens_per_launch(int64_t tokens) {
+  const int64_t before = areno::g_rope_tokens_per_launch;
+  areno::g_rope_tokens_per_launch = tokens > 0 ? tokens : 0;
+  return before;
 }

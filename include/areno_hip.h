@@ -210,9 +210,9 @@ int areno_hip_paged_varlen_prefill(const areno_paged_cache* cache, const void* q
  *   cos, sin      device [max_pos, head_dim] float32 (the doubled-frequency tables of RotaryEmbedding)
  *   q_weight, k_weight  device [head_dim] float32, NULL = no norm on that tensor
  *   cache         NULL = no cache write (then block_ids / block_offsets are ignored)
- * head_dim 64, 128, 256 or 512; every tensor 16-byte aligned.  The kernel indexes with 32 bits: tokens < 2^24,
- * tokens * (q_heads + 2 kv_heads) * head_dim < 2^31, max_pos * head_dim < 2^30, num_blocks * block_size < 2^32;
- * anything larger returns ARENO_ERR_UNSUPPORTED before a launch (run it in token ranges).
+ * head_dim 64, 128, 256 or 512; every tensor 16-byte aligned.  The kernel indexes with 32 bits: a call with more
+ * tokens than that allows (2^24, or 2^31 elements of q, k and v together) runs as consecutive launches over token
+ * ranges; max_pos * head_dim >= 2^30 or num_blocks * block_size >= 2^32 return ARENO_ERR_UNSUPPORTED.
  */
 int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache, const void* q, const void* k, const void* v,
                                        void* q_out, void* k_out, int32_t dtype, int64_t tokens, int32_t q_heads,
@@ -338,6 +338,13 @@ int areno_hip_attention_backward(const void* grad_out, const void* q, const void
                                  const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* context_lens,
                                  int32_t num_seqs, int32_t window_left, float softmax_scale, void* workspace,
                                  size_t workspace_bytes, void* stream);
+
+/*
+ * Test hook, no counterpart in the reference: caps the tokens one launch of areno_hip_qk_norm_rope_cache_write takes
+ * (0 = only the kernel's own limit) so that its walk over token ranges can be tested at small sizes.  Returns the
+ * previous cap.  Process-wide; not for production callers.
+ */
+int64_t areno_hip_debug_set_rope_tokens_per_launch(int64_t tokens);
 
 /*
  * Measurement aid, no counterpart in the reference: reads `pages` runs of page_bytes bytes from one pool or from two

@@ -83,6 +83,43 @@ def test_pages_hold_the_quantized_outputs(kv):
     assert float(err.max()) < 0.1
 
 
+def test_token_ranges_give_what_one_launch_gives():
+    """A call whose token count is past the kernel's 32-bit indexing runs as consecutive launches over token ranges;
+    with the range capped at 5 tokens (the library's test hook) a 53-token call must leave the same outputs and pages,
+    bit for bit, as one launch."""
+    import ctypes
+
+    from areno_amd.accel import cabi
+
+    lib = cabi.lib()
+    lib.areno_hip_debug_set_rope_tokens_per_launch.restype = ctypes.c_int64
+    lib.areno_hip_debug_set_rope_tokens_per_launch.argtypes = [ctypes.c_int64]
+    t, hq, hkv, d, bs, nb = 53, 16, 4, 128, 16, 8
+    dtype = torch.bfloat16
+    q, k, v, pos, cos, sin, qw, kw = _inputs(t, hq, hkv, d, dtype, seed=11)
+    g = torch.Generator().manual_seed(4)
+    slots = torch.randperm(nb * bs, generator=g)[:t]
+    ids, offs = (slots // bs).to(DEV), (slots % bs).to(DEV)
+    results = []
+    for cap in (0, 5):
+        layer = allocate_kv_caches(1, nb, bs, hkv, d, DEV, dtype, "fp8")[0]
+        layer.k_cache.view(torch.uint8).fill_(0x11)
+        layer.v_cache.view(torch.uint8).fill_(0x11)
+        before = lib.areno_hip_debug_set_rope_tokens_per_launch(cap)
+        try:
+            q_out, k_out = ops.areno_qk_norm_rope_cache_write(
+                q.to(DEV), k.to(DEV), v.to(DEV), pos.to(DEV), cos.to(DEV), sin.to(DEV), q_norm_weight=qw.to(DEV),
+                k_norm_weight=kw.to(DEV), eps=1e-6, k_cache=layer.k_cache, v_cache=layer.v_cache, cache_block_ids=ids,
+                cache_block_offsets=offs, k_scale=layer.k_scale, v_scale=layer.v_scale,
+            )  # fmt: skip
+            torch.cuda.synchronize()
+        finally:
+            lib.areno_hip_debug_set_rope_tokens_per_launch(before)
+        results.append((q_out, k_out, layer.k_cache, layer.v_cache, layer.k_scale, layer.v_scale))
+    for a, b, name in zip(results[0], results[1], ("q_out", "k_out", "k pages", "v pages", "k scales", "v scales")):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"{name} differ between one launch and eleven"
+
+
 def test_argument_checks():
     q, k, v, pos, cos, sin, qw, kw = _inputs(4, 4, 2, 128, torch.bfloat16, seed=1)
     with pytest.raises(RuntimeError, match="requires CUDA"):
