@@ -52,12 +52,11 @@ def _contig(t: torch.Tensor | None) -> torch.Tensor | None:
 
 
 def _no_autograd(op: str, *tensors: torch.Tensor | None) -> None:
-    """The paged ops have no backward here (the reference's decode backward recomputes with its PyTorch reference,
-    ``accel/attention.py:245-264`` there; the paged prefill op is this build's own).  Rather than hand back an output
-    that silently carries no gradient, a call that autograd would have to record is refused."""
+    """The paged prefill op (this build's own; the reference has none) has no backward.  Rather than hand back an
+    output that silently carries no gradient, a call that autograd would have to record is refused."""
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
         raise RuntimeError(
-            f"{op}: backward is not implemented for the paged ops; call it under torch.no_grad() / "
+            f"{op}: backward is not implemented for the paged prefill op; call it under torch.no_grad() / "
             "torch.inference_mode() or detach the inputs"
         )
 
@@ -96,6 +95,57 @@ class _VarlenCausalAttention(torch.autograd.Function):
             cu_seqlens.contiguous(), None, None, ctx.window_left, ctx.softmax_scale,
         )  # fmt: skip
         return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None
+
+
+class _PagedDecode(torch.autograd.Function):
+    """The decode op under autograd.  As in the reference (``_ArenoPagedCausalAttentionDecode``,
+    ``areno/accel/attention.py:212-264`` there) the forward is the kernel and the backward recomputes the attention
+    densely in fp32 with tensor ops and lets autograd differentiate that: gradients for ``q`` and for the (unquantized)
+    cache tensors as they stand after the append, none for the update rows.  A training-side convenience, not a fast
+    path: it gathers every row's pages into one ``(batch, tokens, kv_heads, head_dim)`` tensor."""
+
+    @staticmethod
+    def forward(ctx, call, q, k_cache, v_cache, k_scale, v_scale, block_table, cache_seqlens, window_left, softmax_scale):
+        out = call()
+        ctx.save_for_backward(q, k_cache, v_cache, k_scale, v_scale, block_table, cache_seqlens)
+        ctx.window_left = window_left
+        ctx.softmax_scale = softmax_scale
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        q, k_cache, v_cache, k_scale, v_scale, block_table, cache_seqlens = ctx.saved_tensors
+        quantized = k_scale is not None
+        bs = k_cache.shape[1]
+        group = q.shape[1] // k_cache.shape[2]
+        lengths = cache_seqlens.long() + 1  # the appended token is visible
+        cols = (int(lengths.max()) + bs - 1) // bs
+        table = block_table[:, :cols].long().clamp(0, k_cache.shape[0] - 1)  # (columns past a row's length are masked)
+        with torch.enable_grad():
+            q32 = q.detach().float().requires_grad_(True)
+            if quantized:
+                k32 = k_cache.float() * k_scale.float().unsqueeze(-1)
+                v32 = v_cache.float() * v_scale.float().unsqueeze(-1)
+            else:
+                k32 = k_cache.detach().float().requires_grad_(True)
+                v32 = v_cache.detach().float().requires_grad_(True)
+            keys = k32[table].flatten(1, 2).repeat_interleave(group, dim=2)  # (batch, tokens, q heads, head_dim)
+            values = v32[table].flatten(1, 2).repeat_interleave(group, dim=2)
+            t = torch.arange(keys.shape[1], device=q.device)
+            visible = t[None, :] < lengths[:, None]
+            if ctx.window_left >= 0:
+                visible &= t[None, :] >= (lengths[:, None] - 1 - ctx.window_left)
+            # slots no query sees may hold anything (never written, or poisoned): keep them out of the arithmetic
+            keys = torch.where(visible[:, :, None, None], keys, 0.0)
+            values = torch.where(visible[:, :, None, None], values, 0.0)
+            scores = torch.einsum("bhd,bthd->bht", q32, keys) * ctx.softmax_scale
+            probs = torch.softmax(scores.masked_fill(~visible[:, None, :], float("-inf")), dim=-1)
+            out = torch.einsum("bht,bthd->bhd", probs, values)
+            wanted = (q32,) if quantized else (q32, k32, v32)
+            grads = torch.autograd.grad(out, wanted, grad_output.float())
+        dq = grads[0].to(q.dtype)
+        dk, dv = (None, None) if quantized else (grads[1].to(k_cache.dtype), grads[2].to(v_cache.dtype))
+        return None, dq, dk, dv, None, None, None, None, None, None
 
 
 def _rows_of(x: torch.Tensor) -> torch.Tensor:
@@ -178,7 +228,6 @@ def areno_paged_causal_attention_decode(
     several rows instead of once per row.  The result is the same.
     """
     op = "areno_paged_causal_attention_decode"
-    _no_autograd(op, q, k_update, v_update)
     if not _all_on_gpu(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, k_scale, v_scale):
         raise RuntimeError(f"{op} requires CUDA tensors")
     if q.dim() != 3:
@@ -212,12 +261,24 @@ def areno_paged_causal_attention_decode(
             raise ValueError(f"{op} expects the batch to be a multiple of prefix_group_rows")
         if shared_prefix_lens.dtype != torch.int32 or shared_prefix_lens.shape != (q.shape[0] // int(prefix_group_rows),):
             raise ValueError(f"{op} expects int32 shared_prefix_lens shaped (batch / prefix_group_rows,)")
-        return ext.areno_paged_causal_attention_decode_forward_scaled(
-            *args, k_scale, v_scale, int(prefix_group_rows), shared_prefix_lens.contiguous()
-        )
-    if k_scale is None:
-        return ext.areno_paged_causal_attention_decode_forward(*args)
-    return ext.areno_paged_causal_attention_decode_forward_scaled(*args, k_scale, v_scale, 0, None)
+        groups = (int(prefix_group_rows), shared_prefix_lens.contiguous())
+
+        def call():
+            return ext.areno_paged_causal_attention_decode_forward_scaled(*args, k_scale, v_scale, *groups)
+    elif k_scale is None:
+
+        def call():
+            return ext.areno_paged_causal_attention_decode_forward(*args)
+    else:
+
+        def call():
+            return ext.areno_paged_causal_attention_decode_forward_scaled(*args, k_scale, v_scale, 0, None)
+
+    differentiable = (q, k_cache, v_cache) if k_scale is None else (q,)
+    if torch.is_grad_enabled() and any(t.requires_grad for t in differentiable):
+        return _PagedDecode.apply(call, q, k_cache, v_cache, k_scale, v_scale, block_table, cache_seqlens,
+                                  _window_left(window_left), _scale(q, softmax_scale))  # fmt: skip
+    return call()
 
 
 @torch._dynamo.disable

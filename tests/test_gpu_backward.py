@@ -90,3 +90,48 @@ def test_backward_is_deterministic_and_refuses_other_head_dims():
         out = ops.areno_varlen_causal_attention(qx, qx.detach(), qx.detach(), cux)
         with pytest.raises(RuntimeError, match=f"head_dim {d}"):
             out.sum().backward()
+
+
+@pytest.mark.parametrize("kv,window_left", [("bf16", None), ("bf16", 11), ("fp32", None), ("int8", None)])
+def test_decode_backward_recomputes_like_the_reference(kv, window_left):
+    """The decode op under autograd (``_ArenoPagedCausalAttentionDecode.backward``, areno/accel/attention.py:245-264 in
+    the reference): gradients of q and of the cache tensors as they stand after the append, none for the update rows;
+    compared with autograd through the CPU oracle's decode on the same (appended) cache.  Quantized caches (this
+    build's own) give a gradient for q only."""
+    from areno_amd import workloads
+    from tests.gpu_util import dequant_cpu, gpu_quantize
+
+    act = torch.float32 if kv == "fp32" else torch.bfloat16
+    lengths = torch.tensor([0, 5, 16, 37, 70])
+    w = workloads.make_decode_workload("decode-backward", seed=61, batch=5, hq=8, hkv=2, d=64, bs=16, kv=kv, lengths=lengths,
+                                       device=DEV, act_dtype=act, quantize_fn=gpu_quantize, pool_slack=0.5)  # fmt: skip
+    q = w.q.clone().requires_grad_(True)
+    quantized = w.k_scale is not None
+    kc, vc = w.k_cache, w.v_cache
+    if not quantized:
+        kc, vc = kc.clone().requires_grad_(True), vc.clone().requires_grad_(True)
+    out = ops.areno_paged_causal_attention_decode(q, w.k_update, w.v_update, kc, vc, w.block_table, w.cache_seqlens,
+                                                  window_left=window_left, softmax_scale=w.softmax_scale,
+                                                  k_scale=w.k_scale, v_scale=w.v_scale)  # fmt: skip
+    assert out.requires_grad
+    g = torch.Generator().manual_seed(9)
+    grad_out = torch.randn(out.shape, generator=g).to(out.dtype)
+    out.backward(grad_out.to(DEV))
+
+    # the oracle on the cache after the append, in fp32 on the CPU
+    k_ref, v_ref = (dequant_cpu(kc.detach(), w.k_scale), dequant_cpu(vc.detach(), w.v_scale))
+    q_ref = w.q.detach().cpu().float().requires_grad_(True)
+    k_ref, v_ref = k_ref.requires_grad_(True), v_ref.requires_grad_(True)
+    want = ar.ref_paged_decode(q_ref, k_ref, v_ref, w.block_table.cpu(), w.cache_seqlens.cpu(),
+                               -1 if window_left is None else window_left, w.softmax_scale)  # fmt: skip
+    want.backward(grad_out.float())
+    rel = REL[act]
+    _close(q.grad, q_ref.grad, rel, "dq")
+    if quantized:
+        assert w.k_update.grad is None
+    else:
+        _close(kc.grad, k_ref.grad, rel, "dk_cache")
+        _close(vc.grad, v_ref.grad, rel, "dv_cache")
+        live = set(w.block_table.cpu().flatten().tolist())
+        untouched = [b for b in range(kc.shape[0]) if b not in live]
+        assert float(kc.grad[untouched].abs().max()) == 0.0, "pages no row lists must get no gradient"
