@@ -451,6 +451,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   };
   V8 qop[NS];
   float qbias = 0.0f;
+  float4_t score_init = {0.0f, 0.0f, 0.0f, 0.0f};  // what the score products accumulate onto: -qbias for int8, else 0
   auto adopt_q = [&]() {
     float qsum = 0.0f;
 #pragma unroll
@@ -480,17 +481,24 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       }
       qop[sl] = __builtin_bit_cast(V8, w);
     }
-    if constexpr (KIND == KV_I8) qbias = kI8Offset * rows_sum(qsum);
+    if constexpr (KIND == KV_I8) {
+      qbias = kI8Offset * rows_sum(qsum);
+      score_init = float4_t{-qbias, -qbias, -qbias, -qbias};
+    }
   };
 
   float4_t acc[NB];
-  float m_run = kNegInf, l_run = 0.0f, p_sum = 0.0f;
+  float m_run = kNegInf, l_run = 0.0f;
+  // int8: sum over the item's tokens of the probabilities as rounded for P . V, which the offset of the V operands is
+  // taken out with; from the matrix cores (an all-ones A operand puts the column's sum over the tile's 32 tokens, all
+  // four k groups included, into every element), like the products it corrects
+  float4_t p_sum = {0.0f, 0.0f, 0.0f, 0.0f};
   auto reset_state = [&]() {
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) acc[nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     m_run = kNegInf;
     l_run = 0.0f;
-    p_sum = 0.0f;
+    p_sum = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   };
 
   int unit = 0;
@@ -498,7 +506,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     // combine the four k-groups' row sums; every lane of a head ends with the head's totals
     const float l_tot = rows_sum(l_run);
     float off = 0.0f;
-    if constexpr (KIND == KV_I8) off = kI8Offset * rows_sum(p_sum);
+    if constexpr (KIND == KV_I8) off = kI8Offset * p_sum[0];
     const bool shared = is_shared(v);
     const bool live = shared ? col_seq < nseq : lr < p.group;
     if (live) {
@@ -647,7 +655,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       const float pn = fast_exp2(s_new - m_new);
       m_run = m_new;
       l_run = l_run * alpha + (lk == 0 ? pn : 0.0f);
-      p_sum *= alpha;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) p_sum[j] *= alpha;
       const float pv = pn * kPScale;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
@@ -695,7 +704,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     float s[2][4];
 #pragma unroll
     for (int tg = 0; tg < 2; ++tg) {
-      float4_t c = {0.0f, 0.0f, 0.0f, 0.0f};
+      // int8: the products start from -1152 * sum(q) (score_init), which takes the offset of the operands out again
+      float4_t c = score_init;
 #pragma unroll
       for (int sl = 0; sl < NS; ++sl) {
         uint32_t w[WPS];
@@ -708,7 +718,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
         c = Ops::mfma(to_operand<KIND>(w), qop[sl], c);
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) s[tg][j] = c[j] - qbias;  // (this wave's part of) the dot products
+      for (int j = 0; j < 4; ++j) s[tg][j] = c[j];  // (this wave's part of) the dot products
     }
     between_k();
     if constexpr (DSPLIT > 1) {
@@ -758,24 +768,42 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
         for (int j = 0; j < 4; ++j) s[tg][j] = total[tg][j];
       }
     }
-    // the per-token K scale (softmax scale and log2 e folded in); tokens past the end stay exactly -inf
+    // the per-token K scale (softmax scale and log2 e folded in); tokens past the end become exactly -inf, which only
+    // an item's last tile has: every other tile takes the branch with one multiply per score
     float vs[2][4];
+    const bool whole_tile = t.tok + TK <= t.end;  // (scalar)
 #pragma unroll
     for (int tg = 0; tg < 2; ++tg) {
       if constexpr (T::kQuant) {
-        const float4_t ks = *reinterpret_cast<const float4_t*>(sc_lds + 16 * tg + 4 * lk);
         const float4_t vv = *reinterpret_cast<const float4_t*>(sc_lds + 32 + 16 * tg + 4 * lk);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          s[tg][j] = ks[j] == kNegInf ? kNegInf : s[tg][j] * ks[j];
-          vs[tg][j] = vv[j];
-        }
+        for (int j = 0; j < 4; ++j) vs[tg][j] = vv[j];
       } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const bool ok = t.tok + 16 * tg + 4 * lk + j < t.end;
-          s[tg][j] = ok ? s[tg][j] * p.scale_log2e : kNegInf;
-          vs[tg][j] = 1.0f;
+        for (int j = 0; j < 4; ++j) vs[tg][j] = 1.0f;
+      }
+    }
+    if (whole_tile) {
+#pragma unroll
+      for (int tg = 0; tg < 2; ++tg) {
+        float4_t ks = {p.scale_log2e, p.scale_log2e, p.scale_log2e, p.scale_log2e};
+        if constexpr (T::kQuant) ks = *reinterpret_cast<const float4_t*>(sc_lds + 16 * tg + 4 * lk);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[tg][j] *= ks[j];
+      }
+    } else {
+#pragma unroll
+      for (int tg = 0; tg < 2; ++tg) {
+        if constexpr (T::kQuant) {
+          const float4_t ks = *reinterpret_cast<const float4_t*>(sc_lds + 16 * tg + 4 * lk);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) s[tg][j] = ks[j] == kNegInf ? kNegInf : s[tg][j] * ks[j];
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const bool ok = t.tok + 16 * tg + 4 * lk + j < t.end;
+            s[tg][j] = ok ? s[tg][j] * p.scale_log2e : kNegInf;
+          }
         }
       }
     }
@@ -790,7 +818,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     m_run = m_new;
     if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
       l_run *= alpha;
-      p_sum *= alpha;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) p_sum[j] *= alpha;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
@@ -811,13 +840,13 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         pw[j] = pack_pair<KIND>(pe[2 * j], pe[2 * j + 1]);
-        if constexpr (KIND == KV_I8) {
-          const Pair pr = __builtin_bit_cast(Pair, pw[j]);
-          p_sum += static_cast<float>(pr.x) + static_cast<float>(pr.y);
-        }
       }
     }
     const V8 pop = __builtin_bit_cast(V8, uint4_t{pw[0], pw[1], pw[2], pw[3]});
+    if constexpr (KIND == KV_I8) {
+      constexpr uint32_t kOnes = 0x3c003c00u;  // two fp16 1.0
+      p_sum = Ops::mfma(__builtin_bit_cast(V8, uint4_t{kOnes, kOnes, kOnes, kOnes}), pop, p_sum);
+    }
 
     // -- O^T += V^T . P^T, one MFMA per 16-dim block -----------------------------------------------------------------
 #pragma unroll
