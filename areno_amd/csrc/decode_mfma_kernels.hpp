@@ -34,10 +34,11 @@
 // One tile is in flight per wave: the loads of tile x + 1 go out while tile x is computed (V registers are free once
 // the tile is staged, K registers once the scores are issued), the block ids of tile x + 2 in front of them.  The
 // loop over the regular tiles of an item has no branches around loads, so every wait the compiler places counts
-// exactly the loads younger than the one needed.  Measured on the part: with every wave holding a tile in flight the
-// memory system is saturated (a tile takes ~2.6 us to arrive at 6.4 TB/s aggregate), more tiles or waves in flight
-// only lengthen the queues; what a launch loses is its start (work list, block ids, first tile: ~4.5 us) and the
-// spread of the waves' finish times.
+// exactly the loads younger than the one needed.  Measured on the part: with one workgroup per CU and every wave
+// holding a tile in flight the memory system is saturated (an 8 KB tile takes ~1.45 us to arrive, 5.7-5.9 TB/s
+// aggregate; with two workgroups per CU 2.6 us), more tiles or waves in flight only lengthen the queues, and fewer
+// instructions per step change nothing; what a launch loses is its start (work list, block ids, first tile: ~3.7 us)
+// and the spread of the waves' finish times.
 // int8 codes become fp16 by placing (code ^ 0x80) under the exponent byte 0x64 (v_perm): 1152 + code exactly;
 // the offsets are removed algebraically (1152 * sum(q) per head, 1152 * sum(p) per head).  fp8 uses
 // v_cvt_scalef32_pk_f16_fp8 with scale 1 (exact).  bf16 / fp16 caches feed the MFMA directly.
@@ -46,7 +47,8 @@
 // each row's item: the wave that owns it reads the row of k_update / v_update (8 bytes per lane), quantizes it with
 // the cache writer's closed form, stores codes and scales into the page and folds the token into its running
 // softmax on the vector ALU (one token is not worth a matrix product).  The cached tokens in front of it never touch
-// the unwritten slot.
+// the unwritten slot.  That tile streams nothing: the regular tile in front of it fetches only the update rows, and the
+// tile behind it is requested at the start of the token's own step.
 //
 // GROUPED instantiation (batches whose rows come in prefix groups, e.g. the samples of one prompt): the item list is
 // [shared prefix of every sub-group of rows that fits side by side in the 16 MFMA columns] + [the rest of every
