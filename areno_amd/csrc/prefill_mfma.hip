@@ -16,9 +16,10 @@
 //     -- slot 2u for the first item of unit u, slot 2u + 1 for its last -- and prefill_merge_kernel combines them.
 //
 // One segment, per 32-key tile t (all waves share the K/V tiles in LDS):
-//   * the threads fetch K three tiles and V two tiles ahead with 16-byte coalesced loads (block ids one more
-//     tile ahead) and publish them into double-buffered LDS tiles one iteration before their first use, so one
-//     barrier per tile is enough (padded rows, conflict free).  8-bit codes are dequantized (times the per-token
+//   * the threads fetch K four tiles and V three tiles ahead with 16-byte coalesced loads (block ids two more
+//     tiles ahead; two register sets alternate, so a fetch has two tile steps to arrive) and publish them into
+//     double-buffered LDS tiles one iteration before their first use, so one barrier per tile is enough (padded
+//     rows, conflict free).  8-bit codes are dequantized (times the per-token
 //     scale) by the thread that stages them, once per workgroup: the tiles in LDS are always 16-bit.  When a tile
 //     has at most one chunk per thread (8-bit tiles, 16-bit tiles at head dim 64) the first four waves stage K and
 //     the last four V, one chunk each;
@@ -33,9 +34,11 @@
 //   * O^T[dim][row] += V^T . P^T : A = V^T through the LDS transpose reads, B = P^T (= the C layout of S^T); one
 //     more product with an all-ones A operand accumulates the row sums of P.
 // The tile loop is unrolled by two with the roles of the two score arrays swapped, so the scores of tile t + 1 are
-// computed where the next step reads them.  Vector-ALU and matrix-core time add up more than they overlap here: with
-// two waves per SIMD a plain VALU instruction issues every ~5.7 cycles (4 with more waves), v_exp_f32 every ~9, the
-// 34 MFMAs of a wave's tile step need 18 cycles each, and a wave's tile step has ~110 VALU instructions.
+// computed where the next step reads them (and the fetch register sets alternate with them).  Matrix-core, vector-ALU
+// and LDS time add up more than they overlap here: per pair of tile steps on a SIMD (two waves) the 68 products keep
+// the matrix core busy for 1 088 cycles and the vector ALU from issuing for about half of that, the ~104 plain
+// vector instructions and 16 v_exp_f32 (~9 cycles) of each wave take ~1 230, and the CU's LDS, at one instruction
+// per ~6 cycles whatever its width, ~1 050 for the 26 reads and stores per wave; the pair takes ~2 600.
 // The LDS layouts are the 16-bit ones of the decode kernel (decode_mfma_kernels.hpp).  Semantics:
 // _reference_attention with query_start = context_lens[s] (areno/accel/attention.py:25-41 in the reference); with
 // context 0 it is the reference's varlen kernel (areno/accel/csrc/attention.cu:145-242).
