@@ -13,9 +13,13 @@
 //
 // A (token, head) row is a q head (norm + rope -> q_out), a k head (norm + rope -> k_out and the page) or a v head
 // (-> the page).  D / 8 adjacent lanes hold a row, 16 bytes each, so a wave64 carries 64 / (D / 8) rows and every
-// global access is 16 bytes wide; the rotary partner i +- D/2 is the same slot of the lane D/16 away.  The cache rows
-// use the closed forms of areno_hip_cache_write's quantizer, so the pages hold exactly quantize(k_out) and
-// quantize(v).  Bound: HBM streaming, T * (Hq + 2 Hkv) * D elements in, T * (Hq + Hkv) * D out plus the pages.
+// global access is 16 bytes wide; the rotary partner i +- D/2 is the same slot of the lane D/16 away.  The grid is
+// three runs of workgroups, one per kind of row, so a wave's rows are all of one kind and each kind runs code of its
+// own: a q row computes no abs-max and no codes, a v row no norm and no rotation, and which tensor a row comes from
+// is a scalar.  The cache rows use the closed forms of areno_hip_cache_write's quantizer, so the pages hold exactly
+// quantize(k_out) and quantize(v).  Bound: HBM streaming, T * (Hq + 2 Hkv) * D elements in, T * (Hq + Hkv) * D out
+// plus the pages; the vector ALU is what the kernel actually waits for (the roundings of every product to the
+// activation dtype, which the eager ops of the reference imply, are most of its instructions).
 
 #include "cache_row_quant.hpp"
 
@@ -51,6 +55,8 @@ struct RopeWriteParams {
   int32_t cache_dtype;
   int32_t scale_dtype;
   float eps;
+  uint32_t q_blocks;   // workgroups of q rows; they come first in the grid
+  uint32_t kv_blocks;  // workgroups of k rows, then as many of v rows
 };
 
 // x rounded to the activation dtype, as float
@@ -58,18 +64,23 @@ __device__ __forceinline__ float round_to(float x, int dtype) {
   return dtype == ARENO_DT_BF16 ? bf16_bits_to_float(float_to_bf16_bits(x)) : f16_bits_to_float(float_to_f16_bits(x));
 }
 
-// Two values rounded to the activation dtype, as floats: one packed conversion and two unpacking steps for bf16
+// Two values rounded to the activation dtype: the packed pair is returned and the floats are replaced by the rounded
+// values (one packed conversion and two unpacking steps for bf16; a caller that only stores the pair pays for the
+// conversion alone)
 template <int ACT>
-__device__ __forceinline__ void round_pair(float& a, float& b) {
+__device__ __forceinline__ uint32_t round_pair(float& a, float& b) {
   if constexpr (ACT == ARENO_DT_BF16) {
     typedef float float2_t __attribute__((ext_vector_type(2)));
     typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
     const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{a, b}, bf16x2_t));
     a = __builtin_bit_cast(float, w << 16);
     b = __builtin_bit_cast(float, w & 0xffff0000u);
+    return w;
   } else {
-    a = round_to(a, ACT);
-    b = round_to(b, ACT);
+    const uint32_t lo = float_to_f16_bits(a), hi = float_to_f16_bits(b);
+    a = f16_bits_to_float(lo);
+    b = f16_bits_to_float(hi);
+    return lo | (hi << 16);
   }
 }
 
@@ -114,46 +125,43 @@ __device__ __forceinline__ float rotary_partner(float x) {
   }
 }
 
+// The rows of one kind (KIND 0: q heads, 1: k heads, 2: v heads) that workgroup `block` of that kind's run takes.
 // ACT: the activation dtype (ARENO_DT_F16 / ARENO_DT_BF16): no rounding step branches on it.  The launcher checks that
-// rows, element offsets of q / k / v and page rows fit 32 bits, so the index arithmetic is 32-bit: one division per
-// wave (rows of a wave are consecutive) and multiply-adds of 24-bit factors.
-template <int LPR, int ACT>
-__global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
+// rows, element offsets of q / k / v and page rows fit 32 bits, so the index arithmetic is 32-bit, with one division
+// per wave (the rows of a wave are consecutive).
+template <int LPR, int ACT, int KIND>
+__device__ __forceinline__ void rope_write_rows(const RopeWriteParams& p, uint32_t block) {
   constexpr int D = LPR * 8;
   constexpr int kRowsPerWave = kWave / LPR;
   const int lane = threadIdx.x & (kWave - 1);
   const int sub = lane % LPR;  // which 8 elements of the row
-  const uint32_t heads = static_cast<uint32_t>(p.q_heads + 2 * p.kv_heads);
+  const uint32_t heads = static_cast<uint32_t>(KIND == 0 ? p.q_heads : p.kv_heads);
   const uint32_t total = static_cast<uint32_t>(p.tokens) * heads;
-  const uint32_t wave_row =
-      (blockIdx.x * (blockDim.x / kWave) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) * kRowsPerWave;
+  const uint32_t wave_row = (block * (blockDim.x / kWave) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) * kRowsPerWave;
 
-  // ---- which row: (token, head slot) of the wave's first row by one scalar division, the lane group's from there ---
-  const uint32_t row_raw = wave_row + lane / LPR;
-  const bool live = row_raw < total;
+  // ---- which row: (token, head) of the wave's first row by one scalar division, the lane group's from there --------
+  const bool live = wave_row + lane / LPR < total;
   const uint32_t first = min(wave_row, total - 1);  // idle lane groups shadow the last row and store nothing
+  const uint32_t ahead = min(static_cast<uint32_t>(lane / LPR), total - 1 - first);
+  const uint32_t row = first + ahead;
   uint32_t token = first / heads;
-  uint32_t slot = first - token * heads + min(static_cast<uint32_t>(lane / LPR), total - 1 - first);
+  uint32_t head = first - token * heads + ahead;
 #pragma unroll
-  for (int i = 0; i < 3; ++i) {  // heads >= 3 and at most 7 rows further on: at most three tokens further
-    const bool wrap = slot >= heads;
-    slot -= wrap ? heads : 0u;
+  for (int i = 0; i < kRowsPerWave - 1; ++i) {  // at most kRowsPerWave - 1 rows further on, a head or more per token
+    const bool wrap = head >= heads;
+    head -= wrap ? heads : 0u;
     token += wrap ? 1u : 0u;
   }
-  const int kind = slot < static_cast<uint32_t>(p.q_heads) ? 0 : (slot < static_cast<uint32_t>(p.q_heads + p.kv_heads) ? 1 : 2);
-  const uint32_t head = kind == 0 ? slot : (kind == 1 ? slot - p.q_heads : slot - p.q_heads - p.kv_heads);
-  const void* src = kind == 0 ? p.q : (kind == 1 ? p.k : p.v);
-  const uint32_t src_heads = kind == 0 ? p.q_heads : p.kv_heads;
-  const uint32_t src_elem = (__umul24(token, src_heads) + head) * D + sub * 8;
-  const uint4_t raw = *reinterpret_cast<const uint4_t*>(static_cast<const char*>(src) + static_cast<uint64_t>(src_elem) * 2);
-  const int64_t pos = p.positions[token];
-  const uint32_t pc = pos < 0 ? 0u : (pos >= p.max_pos ? static_cast<uint32_t>(p.max_pos - 1) : static_cast<uint32_t>(pos));
-  const float* cos_row = p.cos + static_cast<uint64_t>(pc * D + sub * 8);
-  const float* sin_row = p.sin + static_cast<uint64_t>(pc * D + sub * 8);
-  const float4_t c0 = *reinterpret_cast<const float4_t*>(cos_row);
-  const float4_t c1 = *reinterpret_cast<const float4_t*>(cos_row + 4);
-  const float4_t s0 = *reinterpret_cast<const float4_t*>(sin_row);
-  const float4_t s1 = *reinterpret_cast<const float4_t*>(sin_row + 4);
+  const char* src = static_cast<const char*>(KIND == 0 ? p.q : (KIND == 1 ? p.k : p.v));
+  const uint64_t row_bytes = static_cast<uint64_t>(row * D + sub * 8) * 2;
+  const uint4_t raw = *reinterpret_cast<const uint4_t*>(src + row_bytes);
+
+  void* const cache = KIND == 0 ? nullptr : p.cache[KIND == 2 ? 1 : 0];
+  int64_t blk = -1, off = 0;
+  if (KIND != 0 && cache != nullptr) {
+    blk = p.block_ids[token];
+    off = p.block_offsets[token];
+  }
 
   float x[8];
 #pragma unroll
@@ -168,14 +176,23 @@ __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
     }
   }
 
-  // ---- q and k rows: norm and rotary (selects, not branches, keep every lane in the cross-lane steps) --------------
-  const float* weight = kind == 0 ? p.q_weight : (kind == 1 ? p.k_weight : nullptr);
-  {
-    float sum_sq = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) sum_sq += x[j] * x[j];
-    sum_sq = group_reduce<LPR>(sum_sq, [](float a, float b) { return a + b; });
+  if constexpr (KIND != 2) {
+    // ---- q and k rows: norm and rotary ----------------------------------------------------------------------------
+    const int64_t pos = p.positions[token];
+    const uint32_t pc =
+        pos < 0 ? 0u : (pos >= p.max_pos ? static_cast<uint32_t>(p.max_pos - 1) : static_cast<uint32_t>(pos));
+    const float* cos_row = p.cos + static_cast<uint64_t>(pc * D + sub * 8);
+    const float* sin_row = p.sin + static_cast<uint64_t>(pc * D + sub * 8);
+    const float4_t c0 = *reinterpret_cast<const float4_t*>(cos_row);
+    const float4_t c1 = *reinterpret_cast<const float4_t*>(cos_row + 4);
+    const float4_t s0 = *reinterpret_cast<const float4_t*>(sin_row);
+    const float4_t s1 = *reinterpret_cast<const float4_t*>(sin_row + 4);
+    const float* weight = KIND == 0 ? p.q_weight : p.k_weight;
     if (weight != nullptr) {
+      float sum_sq = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sum_sq += x[j] * x[j];
+      sum_sq = group_reduce<LPR>(sum_sq, [](float a, float b) { return a + b; });
       const float inv = rsqrtf(sum_sq / static_cast<float>(D) + p.eps);
       const float4_t w0 = *reinterpret_cast<const float4_t*>(weight + sub * 8);
       const float4_t w1 = *reinterpret_cast<const float4_t*>(weight + sub * 8 + 4);
@@ -188,53 +205,57 @@ __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
         x[j + 1] = b;
       }
     }
-  }
-  float partner[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) partner[j] = rotary_partner<LPR>(x[j]);
-  if (kind != 2) {
     // rotate_half: -x[i + D/2] below D/2, x[i - D/2] above; the sign goes onto the (rounded) sine, which leaves every
     // rounded product what it was
     const uint32_t sign = sub < LPR / 2 ? 0x80000000u : 0u;
+    uint32_t packed[4];
 #pragma unroll
     for (int j = 0; j < 8; j += 2) {
       float ca = j < 4 ? c0[j & 3] : c1[j & 3], cb = j < 4 ? c0[(j + 1) & 3] : c1[(j + 1) & 3];
       float sa = j < 4 ? s0[j & 3] : s1[j & 3], sb = j < 4 ? s0[(j + 1) & 3] : s1[(j + 1) & 3];
-      round_pair<ACT>(ca, cb);
+      round_pair<ACT>(ca, cb);  // the tables are cast to the activation dtype first, as the eager ops do
       round_pair<ACT>(sa, sb);
       sa = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, sa) ^ sign);
       sb = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, sb) ^ sign);
       float xa = x[j] * ca, xb = x[j + 1] * cb;
       round_pair<ACT>(xa, xb);
-      float ra = partner[j] * sa, rb = partner[j + 1] * sb;
+      float ra = rotary_partner<LPR>(x[j]) * sa, rb = rotary_partner<LPR>(x[j + 1]) * sb;
       round_pair<ACT>(ra, rb);
       float ya = xa + ra, yb = xb + rb;
-      round_pair<ACT>(ya, yb);
-      x[j] = ya;
+      packed[j / 2] = round_pair<ACT>(ya, yb);
+      x[j] = ya;  // read again only by the page store of a k row
       x[j + 1] = yb;
     }
-    void* out = kind == 0 ? p.q_out : p.k_out;
-    if (out != nullptr && live) {
-      const uint4_t packed = {pack_two_16(x[0], x[1], ACT), pack_two_16(x[2], x[3], ACT),
-                              pack_two_16(x[4], x[5], ACT), pack_two_16(x[6], x[7], ACT)};
-      *reinterpret_cast<uint4_t*>(static_cast<char*>(out) + static_cast<uint64_t>(src_elem) * 2) = packed;
-    }
+    void* out = KIND == 0 ? p.q_out : p.k_out;
+    if (out != nullptr && live)
+      *reinterpret_cast<uint4_t*>(static_cast<char*>(out) + row_bytes) = uint4_t{packed[0], packed[1], packed[2], packed[3]};
   }
 
-  // ---- k and v rows: into the page, through the cache writer's closed forms ------------------------------------------
-  float amax = 0.0f;
+  if constexpr (KIND != 0) {
+    // ---- k and v rows: into the page, through the cache writer's closed forms ------------------------------------
+    if (cache == nullptr) return;
+    float amax = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(x[j]));
-  amax = group_reduce<LPR>(amax, [](float a, float b) { return fmaxf(a, b); });
-  if (kind == 0 || !live) return;
-  void* cache = p.cache[kind - 1];
-  if (cache == nullptr) return;
-  const int64_t blk = p.block_ids[token];
-  const int64_t off = p.block_offsets[token];
-  if (blk < 0 || blk >= p.num_blocks || off < 0 || off >= p.block_size) return;
-  const uint32_t page_row = static_cast<uint32_t>(blk) * static_cast<uint32_t>(p.block_size) + static_cast<uint32_t>(off);
-  const int64_t dst_row = static_cast<int64_t>(static_cast<uint64_t>(page_row) * static_cast<uint32_t>(p.kv_heads) + head);
-  store_row_slice(x, amax, sub, dst_row, D, cache, p.scale[kind - 1], p.cache_dtype, p.scale_dtype);
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(x[j]));
+    amax = group_reduce<LPR>(amax, [](float a, float b) { return fmaxf(a, b); });
+    if (!live || blk < 0 || blk >= p.num_blocks || off < 0 || off >= p.block_size) return;
+    const uint32_t page_row =
+        static_cast<uint32_t>(blk) * static_cast<uint32_t>(p.block_size) + static_cast<uint32_t>(off);
+    const int64_t dst_row = static_cast<int64_t>(static_cast<uint64_t>(page_row) * heads + head);
+    store_row_slice(x, amax, sub, dst_row, D, cache, p.scale[KIND == 2 ? 1 : 0], p.cache_dtype, p.scale_dtype);
+  }
+}
+
+template <int LPR, int ACT>
+__global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
+  const uint32_t block = blockIdx.x;
+  if (block < p.q_blocks) {
+    rope_write_rows<LPR, ACT, 0>(p, block);
+  } else if (block < p.q_blocks + p.kv_blocks) {
+    rope_write_rows<LPR, ACT, 1>(p, block - p.q_blocks);
+  } else {
+    rope_write_rows<LPR, ACT, 2>(p, block - p.q_blocks - p.kv_blocks);
+  }
 }
 
 typedef void (*rope_write_fn)(RopeWriteParams);
@@ -312,9 +333,9 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
   p.eps = eps;
   const rope_write_fn fn = rope_write_lookup(head_dim, dtype);
   if (fn == nullptr) return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim must be 64, 128, 256 or 512, got %d", op, head_dim);
-  // The kernel's index arithmetic is 32-bit (rows, element offsets of q / k / v, rotary table offsets, page rows), with
-  // 24-bit factors in its multiply-adds.  The table and the pool must fit as they are; a token count past the limits
-  // runs as consecutive launches over token ranges.
+  // The kernel's index arithmetic is 32-bit (rows, element offsets of q / k / v, rotary table offsets, page rows).
+  // The table and the pool must fit as they are; a token count past the limits runs as consecutive launches over
+  // token ranges.
   const int heads = q_heads + 2 * kv_heads;
   if (heads >= (1 << 16) || static_cast<int64_t>(max_pos) * head_dim >= 0x3fffffffLL)
     return fail(ARENO_ERR_UNSUPPORTED, "%s: %d heads, %d positions x %d are past the kernel's 32-bit indexing", op, heads,
@@ -340,9 +361,9 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
     r.positions = positions + t0;
     r.block_ids = block_ids == nullptr ? nullptr : block_ids + t0;
     r.block_offsets = block_offsets == nullptr ? nullptr : block_offsets + t0;
-    const int64_t rows = r.tokens * heads;
-    const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-    hipLaunchKernelGGL(fn, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), r);
+    r.q_blocks = static_cast<uint32_t>((r.tokens * q_heads + rows_per_block - 1) / rows_per_block);
+    r.kv_blocks = static_cast<uint32_t>((r.tokens * kv_heads + rows_per_block - 1) / rows_per_block);
+    hipLaunchKernelGGL(fn, dim3(r.q_blocks + 2 * r.kv_blocks), dim3(256), 0, static_cast<hipStream_t>(stream), r);
     if (int rc = check_launch(op)) return rc;
   }
   return ARENO_OK;

@@ -32,7 +32,7 @@ def _inputs(t, hq, hkv, d, dtype, seed, max_pos=4096):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (28, 4, 128), (4, 4, 256), (2, 2, 512), (1, 1, 64), (3, 1, 128)])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (28, 4, 128), (4, 4, 256), (2, 2, 512), (1, 1, 64), (3, 1, 128), (32, 8, 128), (2, 1, 64), (6, 2, 128)])
 @pytest.mark.parametrize("norm", [True, False])
 def test_norm_rope_outputs(dtype, hq, hkv, d, norm):
     q, k, v, pos, cos, sin, qw, kw = _inputs(37, hq, hkv, d, dtype, seed=d + hq)
