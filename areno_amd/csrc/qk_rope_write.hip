@@ -94,8 +94,9 @@ __device__ __forceinline__ uint32_t round_pair(float& a, float& b) {
 // by 8 is lane ^ 8 exactly.
 template <int CTRL>
 __device__ __forceinline__ float row_permute(float x) {
-  const int v = __builtin_bit_cast(int, x);
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(v, v, CTRL, 0xf, 0xf, false));
+  // every lane has a source lane in these permutes, so the value for lanes without one is never used; saying so
+  // (bound_ctrl) lets the compiler fold the permute into the instruction that consumes it
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
 }
 constexpr int kDppQuadXor1 = 0xB1;     // quad_perm:[1,0,3,2]
 constexpr int kDppQuadXor2 = 0x4E;     // quad_perm:[2,3,0,1]
@@ -146,21 +147,23 @@ __device__ __forceinline__ void rope_write_rows(const RopeWriteParams& p, uint32
   const uint32_t row = first + ahead;
   uint32_t token = first / heads;
   uint32_t head = first - token * heads + ahead;
-#pragma unroll
-  for (int i = 0; i < kRowsPerWave - 1; ++i) {  // at most kRowsPerWave - 1 rows further on, a head or more per token
+  // at most kRowsPerWave - 1 rows further on: one token further when a token has that many heads or more
+  const int wraps = heads >= static_cast<uint32_t>(kRowsPerWave) ? 1 : kRowsPerWave - 1;
+  for (int i = 0; i < wraps; ++i) {
     const bool wrap = head >= heads;
     head -= wrap ? heads : 0u;
     token += wrap ? 1u : 0u;
   }
+  // byte offsets are 32-bit (the launcher's limits), so an access is a scalar base plus a lane's 32-bit offset
   const char* src = static_cast<const char*>(KIND == 0 ? p.q : (KIND == 1 ? p.k : p.v));
-  const uint64_t row_bytes = static_cast<uint64_t>(row * D + sub * 8) * 2;
+  const uint32_t row_bytes = (row * D + sub * 8) * 2u;
   const uint4_t raw = *reinterpret_cast<const uint4_t*>(src + row_bytes);
 
   void* const cache = KIND == 0 ? nullptr : p.cache[KIND == 2 ? 1 : 0];
   int64_t blk = -1, off = 0;
   if (KIND != 0 && cache != nullptr) {
-    blk = p.block_ids[token];
-    off = p.block_offsets[token];
+    blk = *reinterpret_cast<const int64_t*>(reinterpret_cast<const char*>(p.block_ids) + token * 8u);
+    off = *reinterpret_cast<const int64_t*>(reinterpret_cast<const char*>(p.block_offsets) + token * 8u);
   }
 
   float x[8];
@@ -178,11 +181,12 @@ __device__ __forceinline__ void rope_write_rows(const RopeWriteParams& p, uint32
 
   if constexpr (KIND != 2) {
     // ---- q and k rows: norm and rotary ----------------------------------------------------------------------------
-    const int64_t pos = p.positions[token];
+    const int64_t pos = *reinterpret_cast<const int64_t*>(reinterpret_cast<const char*>(p.positions) + token * 8u);
     const uint32_t pc =
         pos < 0 ? 0u : (pos >= p.max_pos ? static_cast<uint32_t>(p.max_pos - 1) : static_cast<uint32_t>(pos));
-    const float* cos_row = p.cos + static_cast<uint64_t>(pc * D + sub * 8);
-    const float* sin_row = p.sin + static_cast<uint64_t>(pc * D + sub * 8);
+    const uint32_t table_bytes = (pc * D + sub * 8) * 4u;
+    const float* cos_row = reinterpret_cast<const float*>(reinterpret_cast<const char*>(p.cos) + table_bytes);
+    const float* sin_row = reinterpret_cast<const float*>(reinterpret_cast<const char*>(p.sin) + table_bytes);
     const float4_t c0 = *reinterpret_cast<const float4_t*>(cos_row);
     const float4_t c1 = *reinterpret_cast<const float4_t*>(cos_row + 4);
     const float4_t s0 = *reinterpret_cast<const float4_t*>(sin_row);
