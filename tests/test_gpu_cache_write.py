@@ -119,6 +119,46 @@ def test_int8_rounding_ties_and_clamp():
     assert torch.equal(vc.cpu().view(4, 1, 128), codes)
 
 
+@pytest.mark.parametrize("cache_dtype,scale_dtype", [(torch.int8, torch.float16), (torch.float8_e4m3fn, torch.float32)])
+def test_quantizer_divisions_over_the_range_of_scales(cache_dtype, scale_dtype):
+    """bf16 rows whose abs-max runs from 2^-120 to 2^100: the lane-group kernel divides a row by its scale through one
+    shared reciprocal when the scale lies in 2^-60 .. 2^60 and by the plain division outside; both must give the
+    oracle's codes, with negative zeros, exact halves and denormal elements among the values."""
+    exps = [-120, -100, -70, -62, -61, -60, -59, -45, -20, -3, 0, 7, 30, 58, 59, 60, 61, 62, 70, 100]
+    hkv, d, bs = 2, 128, 16
+    t = len(exps) * 3
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(2, t, hkv, d, generator=g)
+    x[torch.rand(x.shape, generator=g) < 0.05] = -0.0
+    x[torch.rand(x.shape, generator=g) < 0.05] *= 2.0 ** -20
+    scale = torch.tensor([2.0**e for e in exps for _ in range(3)], dtype=torch.float64).view(1, t, 1, 1)
+    x = (x.double() * scale).to(torch.bfloat16)
+    x[:, :, :, 0] = (448.0 * scale[..., 0]).to(torch.bfloat16)  # an abs-max of exactly 448 x 2^e: fp8 scale 2^e
+    x[:, :, :, 1] = (0.5 * 2.0**-6 * scale[..., 0]).to(torch.bfloat16)  # half of fp8's smallest normal step: a tie
+    k, v = x[0], x[1]
+    nb = (t + bs - 1) // bs + 1
+    ids, offs = _addresses(t, nb, bs, seed=8)
+    kc = torch.zeros(nb, bs, hkv, d, dtype=torch.uint8).view(cache_dtype)
+    vc = torch.zeros_like(kc)
+    ks = torch.zeros(nb, bs, hkv, dtype=scale_dtype)
+    vs = torch.zeros_like(ks)
+    ref = [t_.clone() for t_ in (kc, vc, ks, vs)]
+    qr.ref_quantized_cache_write(k, v, *ref, ids, offs)
+    dev = [t_.to(DEV) for t_ in (kc, vc, ks, vs)]
+    ops.areno_paged_cache_write(k.to(DEV), v.to(DEV), dev[0], dev[1], ids.to(DEV), offs.to(DEV), k_scale=dev[2], v_scale=dev[3])
+    for name, got, want in zip(("k codes", "v codes", "k scale", "v scale"), dev, ref):
+        got = got.cpu()
+        if got.dtype in (torch.int8, torch.float8_e4m3fn):
+            gb, wb = got.view(torch.uint8), want.view(torch.uint8)
+            if cache_dtype == torch.float8_e4m3fn:  # +0 and -0 are one value
+                gb = torch.where(gb == 0x80, torch.zeros_like(gb), gb)
+                wb = torch.where(wb == 0x80, torch.zeros_like(wb), wb)
+            bad = (gb != wb).nonzero()
+            assert bad.numel() == 0, f"{name}: {bad.shape[0]} bytes differ, first at {bad[0].tolist()}"
+        else:
+            assert torch.equal(got, want), name
+
+
 def test_out_of_pool_addresses_are_skipped_and_empty_write_is_a_noop():
     kc = torch.zeros(2, 4, 1, 64, dtype=torch.bfloat16, device=DEV)
     vc = torch.zeros_like(kc)
