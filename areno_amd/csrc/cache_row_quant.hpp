@@ -16,12 +16,17 @@ __host__ __device__ inline bool is_quantized_dtype(int dtype) {
   return dtype == ARENO_DT_I8 || dtype == ARENO_DT_FP8_E4M3;
 }
 
-__device__ __forceinline__ void quantize_store_row(const float (&x)[kMaxPerLane], int lane, int d, int64_t dst_row,
-                                                   void* cache, void* scale, int cache_dtype, int scale_dtype) {
+// One row of EPW elements per lane (element idx = lane + 64 e, zeros behind the head's end): codes and scale by the
+// closed forms above, stored at cache row dst_row when `store` is set; xhat[e] receives what a reader of the page
+// sees for the element (code times the scale as stored).
+template <int EPW>
+__device__ __forceinline__ void quantize_row(const float (&x)[EPW], int lane, int d, int64_t dst_row, void* cache,
+                                             void* scale, int cache_dtype, int scale_dtype, bool store,
+                                             float (&xhat)[EPW]) {
   const int64_t dst_base = dst_row * d;
   float amax = 0.0f;
 #pragma unroll
-  for (int e = 0; e < kMaxPerLane; ++e) amax = fmaxf(amax, fabsf(x[e]));
+  for (int e = 0; e < EPW; ++e) amax = fmaxf(amax, fabsf(x[e]));
   amax = wave_max(amax);
   if (cache_dtype == ARENO_DT_I8) {
     const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
@@ -29,14 +34,13 @@ __device__ __forceinline__ void quantize_store_row(const float (&x)[kMaxPerLane]
     const float s = static_cast<float>(s16_fixed);
     int8_t* out = static_cast<int8_t*>(cache);
 #pragma unroll
-    for (int e = 0; e < kMaxPerLane; ++e) {
+    for (int e = 0; e < EPW; ++e) {
       const int idx = lane + e * kWave;
-      if (idx < d) {
-        const float code = fminf(fmaxf(rintf(x[e] / s), -127.0f), 127.0f);
-        out[dst_base + idx] = static_cast<int8_t>(static_cast<int>(code));
-      }
+      const float code = fminf(fmaxf(rintf(x[e] / s), -127.0f), 127.0f);
+      xhat[e] = code * s;
+      if (store && idx < d) out[dst_base + idx] = static_cast<int8_t>(static_cast<int>(code));
     }
-    if (lane == 0) {
+    if (store && lane == 0) {
       if (scale_dtype == ARENO_DT_F16) {
         static_cast<uint16_t*>(scale)[dst_row] = __builtin_bit_cast(uint16_t, s16_fixed);
       } else {
@@ -46,16 +50,17 @@ __device__ __forceinline__ void quantize_store_row(const float (&x)[kMaxPerLane]
   } else {
     float s = amax / 448.0f;
     if (s == 0.0f) s = 1.0f;
+    const float s_stored = scale_dtype == ARENO_DT_F16 ? f16_bits_to_float(float_to_f16_bits(s)) : s;
     uint8_t* out = static_cast<uint8_t*>(cache);
 #pragma unroll
-    for (int e = 0; e < kMaxPerLane; ++e) {
+    for (int e = 0; e < EPW; ++e) {
       const int idx = lane + e * kWave;
-      if (idx < d) {
-        const float y = fminf(fmaxf(x[e] / s, -448.0f), 448.0f);
-        out[dst_base + idx] = static_cast<uint8_t>(float_to_fp8_byte(y));
-      }
+      const float y = fminf(fmaxf(x[e] / s, -448.0f), 448.0f);
+      const uint32_t byte = float_to_fp8_byte(y);
+      xhat[e] = fp8_byte_to_float(byte) * s_stored;
+      if (store && idx < d) out[dst_base + idx] = static_cast<uint8_t>(byte);
     }
-    if (lane == 0) {
+    if (store && lane == 0) {
       if (scale_dtype == ARENO_DT_F16) {
         static_cast<uint16_t*>(scale)[dst_row] = static_cast<uint16_t>(float_to_f16_bits(s));
       } else {
@@ -63,6 +68,12 @@ __device__ __forceinline__ void quantize_store_row(const float (&x)[kMaxPerLane]
       }
     }
   }
+}
+
+__device__ __forceinline__ void quantize_store_row(const float (&x)[kMaxPerLane], int lane, int d, int64_t dst_row,
+                                                   void* cache, void* scale, int cache_dtype, int scale_dtype) {
+  float unused[kMaxPerLane];
+  quantize_row<kMaxPerLane>(x, lane, d, dst_row, cache, scale, cache_dtype, scale_dtype, true, unused);
 }
 
 // The same closed forms for a row held by a group of LPR adjacent lanes, 8 consecutive elements per lane (lane `sub`
@@ -84,11 +95,12 @@ __device__ __forceinline__ float lane_group_max(float x) {
 // x[j] / s for the eight elements a lane holds and the row's one divisor, rounded as the IEEE division rounds: the
 // steps of the correctly rounded sequence (reciprocal, one Newton step on it, quotient, two residual corrections;
 // what the compiler emits per division, less the rescaling of extreme operands) with the reciprocal's part done
-// once for the row: 5 instructions per element instead of 12.  Divisors outside 2^-60 .. 2^60, infinities and NaN
-// take the plain division.  Quotients below 2^-20 in magnitude may differ from the plain division's in their last
+// once for the row: 5 instructions per element instead of 12.  Divisors outside 2^-60 .. 2^60, infinities and NaN, and
+// rows with an infinite element (`amax` is the row's abs-max) take the plain division.  Quotients below 2^-20 in magnitude may differ from the plain division's in their last
 // bits; every code below rounds them to a zero of the right sign.
-__device__ __forceinline__ void divide_row_slice(const float (&x)[8], float s, float (&q)[8]) {
-  if (s >= 0x1p-60f && s <= 0x1p60f) {
+__device__ __forceinline__ void divide_row_slice(const float (&x)[8], float s, float amax, float (&q)[8]) {
+  // (an infinite element would come out of the corrections as NaN: a row that holds one takes the plain division)
+  if (s >= 0x1p-60f && s <= 0x1p60f && amax <= 0x1.fffffep127f) {
     const float r0 = __builtin_amdgcn_rcpf(s);
     const float r = fmaf(fmaf(-s, r0, 1.0f), r0, r0);
 #pragma unroll
@@ -112,7 +124,7 @@ __device__ __forceinline__ void store_row_slice(const float (&x)[8], float amax,
     const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
     const float s = static_cast<float>(s16_fixed);
     float q[8];
-    divide_row_slice(x, s, q);
+    divide_row_slice(x, s, amax, q);
     uint32_t words[2] = {0u, 0u};
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -131,7 +143,7 @@ __device__ __forceinline__ void store_row_slice(const float (&x)[8], float amax,
     float s = amax / 448.0f;
     if (s == 0.0f) s = 1.0f;
     float q[8];
-    divide_row_slice(x, s, q);
+    divide_row_slice(x, s, amax, q);
 #pragma unroll
     for (int j = 0; j < 8; ++j) q[j] = fminf(fmaxf(q[j], -448.0f), 448.0f);
     // two codes per conversion, into the low or the high half of the word

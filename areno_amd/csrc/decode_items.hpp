@@ -1,17 +1,22 @@
-// Work list of the matrix-core decode kernel: how a batch becomes items, items become 32-token tiles, and the
-// tile range is cut into equal units, one per wave.  Plain C++ shared by the split kernel, the merge kernel and the
-// host (the launcher sizes the workspace with it, and a CPU test walks every unit of a workload through the same
-// functions and checks each index they produce before anything is loaded through it).
+// Work list of the matrix-core decode kernel: how a batch becomes items, items become quanta of 16 tokens, and the
+// quantum range is cut into units of equal cost, one per wave.  Plain C++ shared by the split kernel, the merge
+// kernel, the plan kernel and the host (the launcher sizes the workspace with it, and a CPU test walks every unit of
+// a workload through the same functions and checks each index they produce before anything is loaded through it).
 //
-// Items.  Without prefix groups item v is row v: its visible keys [first_allowed, L_v] (the reference's range,
-// areno/accel/csrc/attention.cu:588-604).  With prefix groups the list is
+// Items.  Without prefix groups item v is row v: the cached keys the row's query may see, [first_allowed, end), the
+// reference's range (areno/accel/csrc/attention.cu:588-604) with end = L_v + 1 when the token being appended is in
+// its page already and end = L_v when the merge launch folds that token in (it is not in the page yet).  With
+// prefix groups the list is
 //   [shared prefix of every sub-group of rows that sit side by side in the 16 matrix-core columns]
 //   + [the rest of every row],
-// a shared item being read once for all rows of its sub-group.
-// Tiles.  An item is ceil((end - lo) / 32) regular tiles of cached tokens; when the append rides along (the newest
-// token's K / V row is not in the page yet) a per-row item ends in one more tile that holds only that token, taken
-// from the update row.
-// Units.  Unit u owns tiles [u * total / units, (u + 1) * total / units).
+// a shared item being read once for all rows of its sub-group.  An item may be empty (a row without cached keys).
+// Quanta.  An item is ceil((end - lo) / 16) quanta of 16 tokens, the last one possibly short.
+// Cost line.  The items lie one behind the other on a line of cost positions: a non-empty item takes
+// switch_quanta positions that carry no tokens (what it costs a wave to change items: a partial, the next Q, the
+// softmax state) and then one position per quantum.  Unit u owns positions [u * total / units, (u + 1) * total /
+// units): every unit has the same cost to within one position.  The part of an item inside a unit is a segment; a
+// wave goes through a segment in tile steps of 32 or 64 tokens counted from the segment's first token, the last step
+// masked at the segment's end.
 #pragma once
 
 #include <stdint.h>
@@ -24,7 +29,8 @@
 
 namespace areno {
 
-constexpr int kTileTokens = 32;
+constexpr int kTileTokens = 32;      // key tile of the prefill kernel; shared prefix lengths are cut to multiples of it
+constexpr int kQuantumTokens = 16;   // granularity of the decode kernel's unit borders
 constexpr int kMfmaMaxBatch = 1024;  // rows one launch indexes: the prefix sum over the items lives in LDS
 
 // first key a query at position length - 1 may see (window_left < 0: no window)
@@ -35,33 +41,32 @@ ARENO_HD int first_visible_key(int length, int window_left) {
 }
 
 struct UnitGeometry {
-  int total_tiles;
+  int total;  // cost positions of the launch
   int units;
   bool narrow;  // the products below fit 32 bits: 32-bit divisions are a fifth of the instructions of 64-bit ones
 
   ARENO_HD int unit_start(int u) const {
     if (narrow)
-      return static_cast<int>(static_cast<uint32_t>(u) * static_cast<uint32_t>(total_tiles) /
-                              static_cast<uint32_t>(units));
-    return static_cast<int>(static_cast<long long>(u) * total_tiles / units);
+      return static_cast<int>(static_cast<uint32_t>(u) * static_cast<uint32_t>(total) / static_cast<uint32_t>(units));
+    return static_cast<int>(static_cast<long long>(u) * total / units);
   }
-  // unit that owns tile x, 0 <= x < total_tiles: the largest u with unit_start(u) <= x
+  // unit that owns position x, 0 <= x < total: the largest u with unit_start(u) <= x
   ARENO_HD int unit_of(int x) const {
     if (narrow)
       return static_cast<int>((static_cast<uint32_t>(x + 1) * static_cast<uint32_t>(units) +
-                               static_cast<uint32_t>(total_tiles) - 1u) /
-                              static_cast<uint32_t>(total_tiles)) -
+                               static_cast<uint32_t>(total) - 1u) /
+                              static_cast<uint32_t>(total)) -
              1;
-    return static_cast<int>((static_cast<long long>(x + 1) * units + total_tiles - 1) / total_tiles - 1);
+    return static_cast<int>((static_cast<long long>(x + 1) * units + total - 1) / total - 1);
   }
 };
 
-ARENO_HD UnitGeometry make_unit_geometry(int total_tiles, int units) {
+ARENO_HD UnitGeometry make_unit_geometry(int total, int units) {
   UnitGeometry g;
-  g.total_tiles = total_tiles;
+  g.total = total;
   g.units = units;
-  // largest product in unit_start / unit_of: (total_tiles + 1) * units + total_tiles
-  g.narrow = (static_cast<long long>(total_tiles) + 2) * (static_cast<long long>(units) + 1) < (1LL << 31);
+  // largest product in unit_start / unit_of: (total + 1) * units + total
+  g.narrow = (static_cast<long long>(total) + 2) * (static_cast<long long>(units) + 1) < (1LL << 31);
   return g;
 }
 
@@ -69,7 +74,8 @@ ARENO_HD UnitGeometry make_unit_geometry(int total_tiles, int units) {
 struct ItemShape {
   int batch;
   int window_left;
-  int new_token_tile;  // 1: per-row items end in a tile of their own for the token being appended
+  int append_in_merge;  // 1: the token being appended is not in its page; items end in front of it (the merge adds it)
+  int switch_quanta;    // cost positions in front of a non-empty item's quanta
   // prefix groups; num_shared = 0 and the other three = 1 without them
   int num_shared;      // shared items, listed in front of the per-row items
   int group_rows;      // rows per prefix group
@@ -81,17 +87,18 @@ struct ItemShape {
 };
 
 struct ItemInfo {
-  int lo;       // first token
-  int end;      // end of the cached tokens the item reads through the block table of `row`
-  int row;      // block-table / query row (first row of the sub-group for a shared item)
-  int nseq;     // rows served side by side (1 for a per-row item)
-  int has_new;  // a tile for the newest token follows the cached ones
-  ARENO_HD int tiles() const { return (end - lo + kTileTokens - 1) / kTileTokens + has_new; }
+  int lo;    // first token
+  int end;   // end of the cached tokens the item reads through the block table of `row`
+  int row;   // block-table / query row (first row of the sub-group for a shared item)
+  int nseq;  // rows served side by side (1 for a per-row item)
+  ARENO_HD int quanta() const { return end > lo ? (end - lo + kQuantumTokens - 1) / kQuantumTokens : 0; }
+  // positions on the cost line
+  ARENO_HD int extent(int switch_quanta) const { return end > lo ? quanta() + switch_quanta : 0; }
 };
 
 // Lens supplies  int row_len(int row)  (cache_seqlens)  and  int group_len(int group)  (shared_prefix_lens).
 // Tokens of a sub-group's shared prefix: the caller's figure, clipped to what every member has cached and cut to a
-// whole number of tiles.
+// whole number of 32-token tiles.
 template <class Lens>
 ARENO_HD int shared_prefix_tokens(const ItemShape& s, const Lens& lens, int sub, int& row0, int& count) {
   const int gi = sub / s.subs_per_group;
@@ -109,7 +116,7 @@ ARENO_HD int shared_prefix_tokens(const ItemShape& s, const Lens& lens, int sub,
 
 template <bool GROUPED, class Lens>
 ARENO_HD ItemInfo item_info(const ItemShape& s, const Lens& lens, int v) {
-  ItemInfo it = {0, 0, 0, 1, 0};
+  ItemInfo it = {0, 0, 0, 1};
   if constexpr (GROUPED) {
     if (v < s.num_shared) {
       it.end = shared_prefix_tokens(s, lens, v, it.row, it.nseq);
@@ -119,67 +126,90 @@ ARENO_HD ItemInfo item_info(const ItemShape& s, const Lens& lens, int v) {
     const int gi = b / s.group_rows;
     int row0, count;
     it.lo = shared_prefix_tokens(s, lens, gi * s.subs_per_group + (b - gi * s.group_rows) / s.cols_seqs, row0, count);
-    it.end = lens.row_len(b) + 1 - s.new_token_tile;
+    it.end = lens.row_len(b) + 1 - s.append_in_merge;
     it.row = b;
-    it.has_new = s.new_token_tile;
     return it;
   } else {
     const int len = lens.row_len(v);
     it.lo = first_visible_key(len + 1, s.window_left);
-    it.end = len + 1 - s.new_token_tile;
+    it.end = len + 1 - s.append_in_merge;
     it.row = v;
-    it.has_new = s.new_token_tile;
     return it;
   }
 }
 
-// Position of a tile stream: item, first token of the tile, the global index of the item's last tile + 1.
+// Position of a wave's tile stream: the item, the first token of the tile, and where the segment (the part of the
+// item that belongs to the wave's unit) ends.
 struct TileCursor {
   int b;
   int tok;
-  int x_end;  // cum[b + 1]
+  int seg_end;  // end of the segment in tokens (<= it.end)
+  int q_end;    // end of the segment on the cost line: min(cum(b + 1), end of the unit)
   ItemInfo it;
-  // the tile holds only the token being appended (no cached tokens left in the item)
-  ARENO_HD bool on_new_token() const { return tok >= it.end; }
 };
 
-// Cum supplies  int at(int i)  = tiles of items [0, i), 0 <= i <= num_items.
-// Put the cursor on global tile x (0 <= x < cum.at(num_items)).
-template <bool GROUPED, class Lens, class Cum>
-ARENO_HD void cursor_seek(TileCursor& c, const ItemShape& s, const Lens& lens, const Cum& cum, int x) {
-  int lo = 0, hi = s.num_items();
-  while (lo + 1 < hi) {  // the largest item index with cum <= x; items without tiles in front of it are skipped
+enum CursorMove { kCursorSameSegment = 0, kCursorOpensItem = 1, kCursorUnitDone = 2 };
+
+// Table supplies  ItemInfo info(int b)  and  int cum(int i)  = cost positions of items [0, i), 0 <= i <= num_items.
+// Put the cursor on the part of item b (non-empty, cum(b) <= from < cum(b + 1)) that lies in [from, c1); false when
+// that part holds no quantum (c1 does not reach past the item's switch positions).
+template <class Table>
+ARENO_HD bool cursor_open(TileCursor& c, const Table& t, int switch_quanta, int b, int from, int c1) {
+  const int first = t.cum(b) + switch_quanta;  // position of the item's first quantum
+  if (c1 <= first) return false;
+  c.b = b;
+  c.it = t.info(b);
+  const int ce = t.cum(b + 1);
+  c.q_end = ce < c1 ? ce : c1;
+  const int start = from > first ? from : first;
+  c.tok = c.it.lo + (start - first) * kQuantumTokens;
+  const int e = c.it.lo + (c.q_end - first) * kQuantumTokens;
+  c.seg_end = e < c.it.end ? e : c.it.end;
+  return true;
+}
+
+// Put the cursor on the first tile of the unit [c0, c1), 0 <= c0 < c1 <= cum(num_items); false when the unit holds
+// no quantum.
+template <class Table>
+ARENO_HD bool cursor_seek(TileCursor& c, const Table& t, int switch_quanta, int num_items, int c0, int c1) {
+  int lo = 0, hi = num_items;
+  while (lo + 1 < hi) {  // the largest item index with cum <= c0; empty items in front of it are skipped
     const int mid = (lo + hi) >> 1;
-    if (cum.at(mid) <= x) {
+    if (t.cum(mid) <= c0) {
       lo = mid;
     } else {
       hi = mid;
     }
   }
-  c.b = lo;
-  c.it = item_info<GROUPED>(s, lens, lo);
-  c.tok = c.it.lo + (x - cum.at(lo)) * kTileTokens;
-  c.x_end = cum.at(lo + 1);
+  return cursor_open(c, t, switch_quanta, lo, c0, c1);
 }
 
-// Move the cursor from tile x_next - 1 to tile x_next (x_next < cum.at(num_items)); true when that tile opens an item.
-template <bool GROUPED, class Lens, class Cum>
-ARENO_HD bool cursor_advance(TileCursor& c, const ItemShape& s, const Lens& lens, const Cum& cum, int x_next) {
-  if (x_next != c.x_end) {
-    c.tok += kTileTokens;
-    return false;
-  }
-  int b = c.b + 1;
-  int end = cum.at(b + 1);
-  while (end == x_next) {  // items without tiles (a group with no shared prefix); ends before num_items because
-    ++b;                   // x_next is a tile of some item
-    end = cum.at(b + 1);
-  }
-  c.b = b;
-  c.x_end = end;
-  c.it = item_info<GROUPED>(s, lens, b);
-  c.tok = c.it.lo;
-  return true;
+// The next non-empty item behind position q = cum(b + 1) of item b, when the unit [.., c1) reaches its quanta;
+// -1 otherwise.  (q < c1 <= cum(num_items), so a non-empty item follows.)
+template <class Table>
+ARENO_HD int next_item_in_unit(const Table& t, int switch_quanta, int b, int q, int c1) {
+  if (q >= c1) return -1;
+  int n = b + 1;
+  while (t.cum(n + 1) == q) ++n;  // empty items
+  return c1 > q + switch_quanta ? n : -1;
+}
+
+// Move the cursor one tile step of `tile_tokens` tokens on inside the unit that ends at position c1.
+template <class Table>
+ARENO_HD CursorMove cursor_advance(TileCursor& c, const Table& t, int switch_quanta, int c1, int tile_tokens) {
+  c.tok += tile_tokens;
+  if (c.tok < c.seg_end) return kCursorSameSegment;
+  const int q = c.q_end;
+  const int n = next_item_in_unit(t, switch_quanta, c.b, q, c1);
+  if (n < 0) return kCursorUnitDone;
+  cursor_open(c, t, switch_quanta, n, q, c1);
+  return kCursorOpensItem;
+}
+
+// Units that hold quanta of an item with cost positions [cb, ce) (ce > cb): the first and the last.
+ARENO_HD void item_units(const UnitGeometry& geo, int switch_quanta, int cb, int ce, int& first, int& last) {
+  first = geo.unit_of(cb + switch_quanta);
+  last = geo.unit_of(ce - 1);
 }
 
 // Sub-groups of a prefix group that sit side by side in the 16 matrix-core columns, or 0 when grouping does not apply.

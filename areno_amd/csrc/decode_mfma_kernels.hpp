@@ -7,17 +7,22 @@
 // form the (zero padded) 16-wide N side of v_mfma_f32_16x16x32 tiles; the vector ALU only dequantizes
 // (<= 0.75 op per element) and runs the softmax.
 //
-// Work decomposition (decode_items.hpp; exactly balanced, no host knowledge of the lengths):
-//   * a sequence contributes ceil(visible_keys / 32) tiles of 32 tokens; every workgroup computes the
-//     prefix sum of tile counts over the batch in LDS and takes an equal share of the global tile range
-//     (a "unit" per wave), so all waves stream the same number of bytes whatever the length distribution;
+// Work decomposition (decode_items.hpp; balanced to within 16 tokens, no host knowledge of the lengths):
+//   * a sequence contributes ceil(visible cached keys / 16) quanta; the quanta of all sequences are cut into equal
+//     ranges, one "unit" per wave, so all waves stream the same number of bytes whatever the length distribution;
+//     a wave walks its unit in tile steps of TK tokens (32 for 16-bit pages, 64 for 8-bit pages: 16 KB in flight
+//     per wave either way), the last step of a segment masked;
+//   * the list of items (first token, end, row) and the prefix sums of their quanta live in LDS: every workgroup
+//     computes them from the sequence lengths, or copies them from a plan that areno_hip_paged_decode_plan left in
+//     device memory once for all layers of a step; with a plan a wave finds its unit's first tile (item, token, block
+//     ids) in one record, fetched next to the copy, instead of a prefix sum, a search and a block-table fetch;
 //   * a unit that crosses a sequence boundary emits one partial per sequence it touches, into slot
-//     (unit index + sequence index), which is unique and contiguous per sequence; the reduce kernel merges
-//     the slots of each sequence;
+//     (unit index + sequence index), which is unique and contiguous per sequence; the merge kernel merges
+//     the slots of each sequence and folds in the token being appended;
 //   * block = 4 wave64; wave w owns KV head z*HW + w % HW, so with kv_heads >= 4 the four waves of a
 //     workgroup read whole pages ([slot][kv_head][D] is contiguous).  Waves never synchronise after the
-//     prefix sum.
-// Data path per 32-token tile and wave (lane = (lr, lk) = (lane % 16, lane / 16); token group tg = 0, 1):
+//     prologue.
+// Data path per tile and wave (lane = (lr, lk) = (lane % 16, lane / 16); token group tg = 0 .. TK / 16 - 1):
 //   K  global --16 B/lane--> registers --> MFMA A operand, no LDS: lane (lr, lk) fetches from token 16 tg + lr the
 //      16-byte chunks lk, lk + 4, ... of the head's row, i.e. 64 contiguous bytes per token and load instruction.
 //      The k index of the products is whatever dims those chunks hold; Q^T (B operand, in registers for the whole
@@ -25,30 +30,24 @@
 //   V  global --same lane / chunk assignment--> registers --ds_write_b128--> LDS, chunk-major
 //      ([token group][chunk][16 tokens][16 B]; 256 contiguous bytes per 16 lanes) --ds_read_b64_tr_b8 / _tr_b16-->
 //      A operand V^T (the LDS transpose read gives each lane 8 tokens of one dim).  So that the 32 lanes of one pass of
-//      the transpose read cover all 64 banks once, the second token group starts 128 bytes off a multiple of 256 and,
+//      the transpose read cover all 64 banks once, every odd token group starts 128 bytes off a multiple of 256 and,
 //      for 16-bit elements (one read touches an even and an odd chunk), an odd chunk keeps its token rows 8..15 in
 //      front of rows 0..7.
-//   online softmax in the log2 domain on the C layout of S^T (head = lane % 16, 4 tokens per lane and group); the
-//      per-token K scale multiplies S, the V scale multiplies P (scales travel through 64 floats of LDS per tile).
-//   O^T[dim][head] += V^T . P^T, where P^T *is* the C layout of S^T, so no cross-lane movement of P is needed.
+//   online softmax in the log2 domain on the C layout of S^T (head = lane % 16, 4 tokens per lane and group), once
+//      per tile; the per-token K scale multiplies S, the V scale multiplies P (scales travel through LDS).
+//   O^T[dim][head] += V^T . P^T per pair of token groups, where P^T *is* the C layout of S^T, so no cross-lane
+//      movement of P is needed.
 // One tile is in flight per wave: the loads of tile x + 1 go out while tile x is computed (V registers are free once
 // the tile is staged, K registers once the scores are issued), the block ids of tile x + 2 in front of them.  The
-// loop over the regular tiles of an item has no branches around loads, so every wait the compiler places counts
-// exactly the loads younger than the one needed.  Measured on the part: with one workgroup per CU and every wave
-// holding a tile in flight the memory system is saturated (an 8 KB tile takes ~1.45 us to arrive, 5.7-5.9 TB/s
-// aggregate; with two workgroups per CU 2.6 us), more tiles or waves in flight only lengthen the queues, and fewer
-// instructions per step change nothing; what a launch loses is its start (work list, block ids, first tile: ~3.7 us)
-// and the spread of the waves' finish times.
+// loop over the tiles of a segment has no branches around loads, so every wait the compiler places counts
+// exactly the loads younger than the one needed.
 // int8 codes become fp16 by placing (code ^ 0x80) under the exponent byte 0x64 (v_perm): 1152 + code exactly;
 // the offsets are removed algebraically (1152 * sum(q) per head, 1152 * sum(p) per head).  fp8 uses
 // v_cvt_scalef32_pk_f16_fp8 with scale 1 (exact).  bf16 / fp16 caches feed the MFMA directly.
 //
-// The single-token append (areno/accel/csrc/attention.cu:526-553) rides along as a tile of its own at the end of
-// each row's item: the wave that owns it reads the row of k_update / v_update (8 bytes per lane), quantizes it with
-// the cache writer's closed form, stores codes and scales into the page and folds the token into its running
-// softmax on the vector ALU (one token is not worth a matrix product).  The cached tokens in front of it never touch
-// the unwritten slot.  That tile streams nothing: the regular tile in front of it fetches only the update rows, and the
-// tile behind it is requested at the start of the token's own step.
+// The single-token append (areno/accel/csrc/attention.cu:526-553) is not part of this kernel: the streaming waves
+// read the tokens that are in the pages, and the merge launch, which owns each (row, head) anyway, quantizes the
+// new row, stores it and folds it in as one more partial (paged_decode.hip).
 //
 // GROUPED instantiation (batches whose rows come in prefix groups, e.g. the samples of one prompt): the item list is
 // [shared prefix of every sub-group of rows that fits side by side in the 16 MFMA columns] + [the rest of every
@@ -76,27 +75,67 @@ namespace areno {
 #ifndef ARENO_MFMA_WIDE_OCC
 #define ARENO_MFMA_WIDE_OCC 2
 #endif
+// tokens per tile step: a wave keeps one tile (K and V) in flight, 16 KB at head dim 128 with either setting
+#ifndef ARENO_MFMA_QUANT_TK
+#define ARENO_MFMA_QUANT_TK 32
+#endif
+#ifndef ARENO_MFMA_WIDE_TK
+#define ARENO_MFMA_WIDE_TK 32
+#endif
 
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) short short4_t;
 typedef __attribute__((ext_vector_type(2))) int int2_t;
+typedef __attribute__((ext_vector_type(4))) int int4_t;
+
+// Tokens per tile step of the kernel that serves a cache kind.
+constexpr int decode_tile_tokens(bool quantized) { return quantized ? ARENO_MFMA_QUANT_TK : ARENO_MFMA_WIDE_TK; }
+
+// What a plan (areno_hip_paged_decode_plan) holds for the split and merge kernels, all int32 in device memory:
+//   cum    [items + 1]   exclusive prefix sums of the items' extents on the cost line (decode_items.hpp)
+//   items  [items][4]    lo, end, row, nseq of every item
+//   units  [units][16]   where a wave's unit starts (layout below)
+constexpr int kDecodeDumpFloats = 16 * 512 + 2 * kWave;  // 16 columns of the widest head, and an (m, l) pair per lane
+constexpr int kDecodeHold = 2;  // partials a wave parks in LDS before it stores them
+constexpr int kPlanUnitWords = 16;
+constexpr int kPlanUnitIds = 6;  // block ids of the first tile's columns that a unit record can hold
+enum PlanUnitWord {
+  kPuItem = 0,
+  kPuTok = 1,
+  kPuSegEnd = 2,
+  kPuQEnd = 3,
+  kPuQ0 = 4,  // the unit's positions on the cost line; q0 == q1: it holds no quantum
+  kPuQ1 = 5,
+  kPuLo = 6,
+  kPuEnd = 7,
+  kPuRow = 8,
+  kPuNseq = 9,
+  kPuIds = 10  // .. 15: block ids of columns (tok >> bs_shift) + 0 .. 5 of the item's row (clamped)
+};
 
 struct MfmaDecodeParams {
   DecodeParams d;      // part_ml / part_acc are indexed [slot][q_head] here
-  int32_t* plan;       // [items + 1]: exclusive prefix sums of tiles per item (written by workgroup 0)
+  int32_t* cum_out;    // [items + 1]: the prefix sums, written by workgroup 0 for the merge kernel (launches without a plan)
   int32_t tok_splits;  // waves of a workgroup that share a KV head (waves per workgroup / heads_per_wg / head split)
   int32_t num_units;   // gridDim.x * tok_splits
-  ItemShape items;     // rows -> items (prefix groups, window, whether the append rides along)
-  // Fused append: per-row items end in a tile for the newest token, whose K / V row comes from here
-  // ([batch, kv_heads, head_dim], dtype q_dtype), is quantized like the cache writer does and stored into the page.
+  ItemShape items;     // rows -> items (prefix groups, window, whether the merge folds in the token being appended)
+  // A plan built once for all layers of a step (NULL: every workgroup derives the work list from the lengths).
+  const int32_t* plan_cum;
+  const int32_t* plan_items;
+  const int32_t* plan_units;
+  // The token being appended, for the merge kernel when items.append_in_merge: [batch, kv_heads, head_dim], dtype
+  // q_dtype; quantized like the cache writer does and stored into the page.
   const void* k_update;
   const void* v_update;
+  int32_t write_append;  // 1: the merge stores the row into its page; 0: it only folds it in (the page holds it already)
+  int64_t num_blocks;    // pages of the pool (the append skips a row whose page id lies outside)
   // Prefix groups (GROUPED kernels only): rows [i * group_rows, (i + 1) * group_rows) share the pages of their first
   // shared_lens[i] tokens.  Shared items leave their partials in a second region (16 columns per kv head and slot).
   const int32_t* shared_lens;  // [batch / group_rows]
   float* shared_ml;            // [slot][kv_head][16][2]
   float* shared_acc;           // [slot][kv_head][16][head_dim]
+  float* dump;                 // kDecodeDumpFloats floats that the lanes without a partial row store to; never read
   unsigned long long* trace;   // [wave][8] timestamps; NULL outside tuning runs (ARENO_TRACE builds only read it)
 };
 
@@ -152,36 +191,64 @@ __device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, make_pair<P>(lo, hi));
 }
 
+// maximum of N values in ceil((N - 1) / 2) instructions (v_max3_f32)
+template <int N>
+__device__ __forceinline__ float max_all(const float (&v)[N]) {
+  if constexpr (N == 1) {
+    return v[0];
+  } else if constexpr (N == 2) {
+    return max_f32(v[0], v[1]);
+  } else {
+    constexpr int M = (N + 2) / 3;
+    float r[M];
+#pragma unroll
+    for (int i = 0; i < N / 3; ++i) r[i] = max3_f32(v[3 * i], v[3 * i + 1], v[3 * i + 2]);
+    if constexpr (N % 3 == 2) r[M - 1] = max_f32(v[N - 2], v[N - 1]);
+    if constexpr (N % 3 == 1) r[M - 1] = v[N - 1];
+    return max_all<M>(r);
+  }
+}
+
 // a wave-uniform value that the compiler cannot prove uniform (it came out of LDS): move it to a scalar register
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
-// The length arrays and the tile prefix sums in LDS, as the item functions of decode_items.hpp want them.  The
-// "uniform" flavour is for lookups whose index is the same in all lanes of a wave (the tile cursors): the values
-// then live in scalar registers.
-template <bool UNIFORM>
+// The item table in LDS as the cursor functions of decode_items.hpp want it; the lookups' indices are the same in
+// all lanes of a wave, so the values end up in scalar registers.
+struct LdsItemTable {
+  const int4_t* item;  // lo, end, row, nseq
+  const int* cum_;
+  __device__ __forceinline__ ItemInfo info(int b) const {
+    const int4_t r = item[b];
+    ItemInfo it;
+    it.lo = uniform(r[0]);
+    it.end = uniform(r[1]);
+    it.row = uniform(r[2]);
+    it.nseq = uniform(r[3]);
+    return it;
+  }
+  __device__ __forceinline__ int cum(int i) const { return uniform(cum_[i]); }
+};
+
+// The sequence lengths in LDS (grouped launches) or in device memory, for item_info in the prologue.
 struct LdsLens {
   const int* len;
   const int* glen;
-  __device__ __forceinline__ int row_len(int b) const { return UNIFORM ? uniform(len[b]) : len[b]; }
-  __device__ __forceinline__ int group_len(int g) const { return UNIFORM ? uniform(glen[g]) : glen[g]; }
-};
-struct LdsCum {
-  const int* cum;
-  __device__ __forceinline__ int at(int i) const { return uniform(cum[i]); }
+  __device__ __forceinline__ int row_len(int b) const { return len[b]; }
+  __device__ __forceinline__ int group_len(int g) const { return glen[g]; }
 };
 
 // What the pipeline remembers of a tile between the moment its block ids are requested and the moment it is computed
 // (all wave-uniform).
 struct TileDesc {
-  int tok;   // first token of the tile inside its sequence
-  int end;   // end of the item's cached tokens
-  int row;   // block-table / query row
-  int nseq;  // rows side by side (shared items), else 1
-  int b;     // item index
-  int x_end; // global index of the item's last tile + 1
-  int kind;  // bit 0: the tile opens its item; bit 1: it holds only the token being appended; bit 2: past the unit
+  int tok;    // first token of the tile inside its sequence
+  int end;    // end of the segment the tile belongs to (tokens at and behind it are masked)
+  int row;    // block-table / query row
+  int nseq;   // rows side by side (shared items), else 1
+  int b;      // item index
+  int q_end;  // where the segment ends on the cost line
+  int kind;   // kTilePhantom: past the unit's end
 };
-constexpr int kTileOpens = 1, kTileNewToken = 2, kTilePhantom = 4;
+constexpr int kTilePhantom = 4;
 
 // DSPLIT > 1 serves heads of DSPLIT * D elements (256 = 2 x 128, 192 = 3 x 64, 512 = 4 x 128): DSPLIT adjacent waves
 // of the workgroup take one part of the head dimension each.  Every wave computes the part of S = K . Q^T over its
@@ -189,7 +256,8 @@ constexpr int kTileOpens = 1, kTileNewToken = 2, kTilePhantom = 4;
 // the same softmax in all, P . V over the wave's own part of V, the wave's part of the partial row.  The waves of a
 // head synchronise through two counters each in LDS (part ready / parts consumed); no workgroup barrier is involved,
 // so the heads of one workgroup may run different units.
-template <int KIND, int D, bool SCALE16, int NW, bool GROUPED = false, int DSPLIT = 1>
+template <int KIND, int D, bool SCALE16, int NW, bool GROUPED = false, int DSPLIT = 1,
+          int TK = decode_tile_tokens(KVTraits<KIND>::kQuant)>
 __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUANT_OCC : ARENO_MFMA_WIDE_OCC) void decode_mfma_kernel(
     MfmaDecodeParams mp) {
   using T = KVTraits<KIND>;
@@ -198,29 +266,32 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   using Pair = typename T::pair_t;
   const DecodeParams& p = mp.d;
   constexpr int ES = T::kBytes;
-  constexpr int TK = kTileTokens;
+  constexpr int NTG = TK / 16;         // token groups of 16 per tile
+  constexpr int NPP = NTG / 2;         // pairs of token groups: one P.V product per pair and dim block
   constexpr int CPT = D * ES / 16;     // 16-byte chunks per token row
   constexpr int CPL = CPT / 4;         // chunks per lane and token: lk, lk + 4, ...
   constexpr int NS = D / 32;           // QK^T k-slices
   constexpr int NB = D / 16;           // P.V dim blocks
   constexpr int WPS = 8 * ES / 4;      // dwords per k-slice of 8 elements
   constexpr int TGS = CPT * 256 + 128;    // bytes of one token group of the V tile in LDS (128 of padding behind it)
+  constexpr int SPL = 2 * TK / kWave;  // scale entries (K scales of the tile's tokens, then V scales) per lane
   constexpr float kPScale = T::kQuant ? 256.0f : 1.0f;
-  constexpr int kParkFloats = DSPLIT > 1 ? 8 * kWave : 0;
-  constexpr int kWaveLds = 2 * TGS + 2 * TK * 4 + kParkFloats * 4;
-  constexpr int UPW = D / 64;          // dwords per lane of an update row pair (K row in lanes 0..31, V row in 32..63)
+  constexpr int kParkFloats = DSPLIT > 1 ? 4 * NTG * kWave : 0;
+  constexpr int kWaveLds = NTG * TGS + 2 * TK * 4 + kParkFloats * 4;
   static_assert(CPL >= 1 && CPL <= 4 && (D == 64 || D == 128), "unsupported head_dim");
-  static_assert(2 * TGS >= 2 * D * 4, "the new token's rows borrow the V tile");
+  static_assert(TK == 32 || TK == 64, "a tile is two or four groups of 16 tokens");
   static_assert(DSPLIT == 1 || (DSPLIT >= 2 && DSPLIT <= 4 && !GROUPED && NW % DSPLIT == 0), "unsupported head split");
   constexpr int DFULL = D * DSPLIT;  // elements of a whole head (row of Q, of a cache page, of a partial)
 
   __shared__ __attribute__((aligned(16))) char s_tiles[NW][kWaveLds];
   constexpr int kMaxItems = (GROUPED ? 2 : 1) * kMfmaMaxBatch;  // at most one shared item per row on top of the rows
+  __shared__ __attribute__((aligned(16))) int4_t s_item[kMaxItems];
   __shared__ int s_cum[kMaxItems + 1];
   __shared__ int s_wave_tot[NW];
-  __shared__ int s_len[kMfmaMaxBatch];                          // sequence lengths of the rows
+  __shared__ int s_len[GROUPED ? kMfmaMaxBatch : 1];            // sequence lengths of the rows
   constexpr int kMaxGroups = kMfmaMaxBatch / 2;                 // groups have at least two rows
   __shared__ int s_group_len[GROUPED ? kMaxGroups : 1];         // shared prefix length of each group
+  __shared__ __attribute__((aligned(16))) float s_hold[NW][kDecodeHold][kWave * 4 * (NB + 1)];  // parked partials
   __shared__ int s_pair_flags[2][NW];  // [0]: score parts this wave has published, [1]: steps whose parts it has read
   constexpr int SPT = (kMaxItems + NW * kWave - 1) / (NW * kWave);  // items per thread in the prefix sum
 
@@ -244,13 +315,44 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   const int lr = lane & 15;  // MFMA row / column index
   const int lk = lane >> 4;  // MFMA k group
 
-  // ---- the item list: lengths into LDS, tiles per item, exclusive prefix sum over the items ------------------------
   const ItemShape& shape = mp.items;
   const int num_items = shape.num_items();
-  const LdsLens<false> lens_any = {s_len, s_group_len};
-  const LdsLens<true> lens = {s_len, s_group_len};
-  const LdsCum cum = {s_cum};
-  {
+  const LdsItemTable table = {s_item, s_cum};
+  const bool planned = mp.plan_units != nullptr;  // (scalar)
+
+  const int hw_count = p.heads_per_wg;
+  const int half = wave % DSPLIT;  // which part of the head dimension this wave owns
+  const int hw = (wave / DSPLIT) % hw_count;
+  const int ts = (wave / DSPLIT) / hw_count;
+  const int kvh = blockIdx.y * hw_count + hw;
+  const int unit = blockIdx.x * mp.tok_splits + ts;
+
+  // ---- the item table: (lo, end, row, nseq) of every item and the exclusive prefix sum of their quanta, in LDS -----
+  int q0 = 0, q1 = 0;       // this wave's unit
+  TileCursor cur;           // the furthest tile requested so far
+  int first_ids[kPlanUnitIds];  // with a plan: block ids of the first tile's columns
+  if (planned) {
+    // the wave's unit record (one 64-byte scalar fetch), and the workgroup's copy of the plan's tables
+    const int32_t* rec = mp.plan_units + static_cast<int64_t>(unit) * kPlanUnitWords;
+    q0 = rec[kPuQ0];
+    q1 = rec[kPuQ1];
+    cur.b = rec[kPuItem];
+    cur.tok = rec[kPuTok];
+    cur.seg_end = rec[kPuSegEnd];
+    cur.q_end = rec[kPuQEnd];
+    cur.it.lo = rec[kPuLo];
+    cur.it.end = rec[kPuEnd];
+    cur.it.row = rec[kPuRow];
+    cur.it.nseq = rec[kPuNseq];
+#pragma unroll
+    for (int i = 0; i < kPlanUnitIds; ++i) first_ids[i] = rec[kPuIds + i];
+    for (int v = tid; v <= num_items; v += NW * kWave) {
+      if (v < num_items) s_item[v] = *reinterpret_cast<const int4_t*>(mp.plan_items + 4 * static_cast<int64_t>(v));
+      s_cum[v] = mp.plan_cum[v];
+    }
+    if (lane == 0) s_pair_flags[0][wave] = s_pair_flags[1][wave] = 0;
+    __syncthreads();
+  } else {
     int nt[SPT];
     int local = 0;
     if constexpr (GROUPED) {
@@ -259,10 +361,16 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       for (int i = tid; i < shape.batch; i += NW * kWave) s_len[i] = p.cache_seqlens[i];
       for (int i = tid; i < shape.num_groups(); i += NW * kWave) s_group_len[i] = mp.shared_lens[i];
       __syncthreads();
+      const LdsLens lens = {s_len, s_group_len};
 #pragma unroll
       for (int j = 0; j < SPT; ++j) {
         const int v = SPT * tid + j;
-        nt[j] = v < num_items ? item_info<true>(shape, lens_any, v).tiles() : 0;
+        nt[j] = 0;
+        if (v < num_items) {
+          const ItemInfo it = item_info<true>(shape, lens, v);
+          s_item[v] = int4_t{it.lo, it.end, it.row, it.nseq};
+          nt[j] = it.extent(shape.switch_quanta);
+        }
         local += nt[j];
       }
     } else {
@@ -275,12 +383,13 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
         const int v = SPT * tid + j;
         nt[j] = 0;
         if (v < num_items) {
-          s_len[v] = len[j];
           ItemInfo it;
           it.lo = first_visible_key(len[j] + 1, shape.window_left);
-          it.end = len[j] + 1 - shape.new_token_tile;
-          it.has_new = shape.new_token_tile;
-          nt[j] = it.tiles();
+          it.end = len[j] + 1 - shape.append_in_merge;
+          it.row = v;
+          it.nseq = 1;
+          s_item[v] = int4_t{it.lo, it.end, it.row, it.nseq};
+          nt[j] = it.extent(shape.switch_quanta);
         }
         local += nt[j];
       }
@@ -305,22 +414,19 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     // the entry behind the last thread's items has no owner of its own: it is the total when the list is full
     if (tid == NW * kWave - 1 && SPT * (tid + 1) <= num_items) s_cum[SPT * (tid + 1)] = excl;
     __syncthreads();
-  }
-  const int total_tiles = cum.at(num_items);
-  const UnitGeometry geo = make_unit_geometry(total_tiles, mp.num_units);
-  if (blockIdx.x == 0 && blockIdx.y == 0) {
-    for (int v = tid; v <= num_items; v += NW * kWave) mp.plan[v] = s_cum[v];
+    const UnitGeometry geo = make_unit_geometry(table.cum(num_items), mp.num_units);
+    if (blockIdx.x == 0 && blockIdx.y == 0) {
+      for (int v = tid; v <= num_items; v += NW * kWave) mp.cum_out[v] = s_cum[v];
+    }
+    q0 = geo.unit_start(unit);
+    q1 = geo.unit_start(unit + 1);
+    if (q0 < q1 && !cursor_seek(cur, table, shape.switch_quanta, num_items, q0, q1)) q1 = q0;  // no quantum in the unit
   }
   ARENO_TRACE_POINT();
 
-  const int hw_count = p.heads_per_wg;
-  const int half = wave % DSPLIT;  // which part of the head dimension this wave owns
-  const int hw = (wave / DSPLIT) % hw_count;
-  const int ts = (wave / DSPLIT) / hw_count;
-  const int kvh = blockIdx.y * hw_count + hw;
   char* const v_tile = &s_tiles[wave][0];
-  float* const sc_lds = reinterpret_cast<float*>(&s_tiles[wave][2 * TGS]);  // [0, 32): K scales, [32, 64): V scales
-  float* const park = reinterpret_cast<float*>(&s_tiles[wave][2 * TGS + 2 * TK * 4]);
+  float* const sc_lds = reinterpret_cast<float*>(&s_tiles[wave][NTG * TGS]);  // [0, TK): K scales, [TK, 2 TK): V scales
+  float* const park = reinterpret_cast<float*>(&s_tiles[wave][NTG * TGS + 2 * TK * 4]);
 
   constexpr int64_t row_bytes = static_cast<int64_t>(DFULL) * ES;
   const int64_t half_bytes = static_cast<int64_t>(half) * D * ES;  // of this wave's part inside a cache / update row
@@ -333,91 +439,82 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   // byte offset of token row r (0..15) of chunk c inside a token group of the V tile: 16-bit tiles keep the two
   // halves of an odd chunk's rows swapped (see the layout note above)
   auto chunk_row_pos = [](int c, int r) { return c * 256 + ((ES == 2 && (c & 1)) ? (r ^ 8) : r) * 16; };
+  // byte offset of token group tg inside the V tile: odd groups 128 bytes off a multiple of 256
+  auto group_pos = [](int tg) { return tg * TGS; };
 
   // ---- the pipeline's registers ------------------------------------------------------------------------------------
-  // Every step issues the same loads in the same order whatever the kinds of the tiles involved (only their addresses
-  // differ), so that the waits the compiler places count exactly the loads that are younger than the one needed and
-  // the tiles behind it stay in flight.  Loads that depend on a tile's kind (the update rows of an appended token, the
-  // Q of the next item) are extra loads on rare paths.
+  // Every step issues the same loads in the same order whatever the tiles involved (only their addresses differ), so
+  // that the waits the compiler places count exactly the loads that are younger than the one needed and the tiles
+  // behind it stay in flight.  The Q of the next item is an extra load at the start of a segment.
   typedef typename std::conditional<SCALE16, uint16_t, float>::type scale_raw_t;
-  uint4_t kreg[2 * CPL], vreg[2 * CPL];
-  scale_raw_t sreg;   // lane l < 32: K scale of tile token l; else V scale of token l - 32
-  uint32_t upd[UPW];  // a new-token tile: the update rows, K in lanes 0..31, V in 32..63
-  uint32_t new_row = 0;   // a new-token tile: cache row (block, slot, head) the token goes to
+  uint4_t kreg[NTG * CPL], vreg[NTG * CPL];
+  scale_raw_t sreg[SPL];  // entry lane + 64 i of [K scales of the tile's tokens, V scales of the tile's tokens]
   TileDesc desc0;      // the tile whose loads are in the registers
-  TileCursor cur;      // the furthest tile requested so far (its block ids are on their way)
-  TileDesc desc_ids;   // = that tile
+  TileDesc desc_ids;   // the furthest tile requested so far (its block ids are on their way)
 
-  auto describe = [&](const TileCursor& c, bool opens) {
+  auto describe = [&](const TileCursor& c) {
     TileDesc t;
     t.tok = c.tok;
-    t.end = c.it.end;
+    t.end = c.seg_end;
     t.row = c.it.row;
     t.nseq = c.it.nseq;
     t.b = c.b;
-    t.x_end = c.x_end;
-    t.kind = (opens ? kTileOpens : 0) | (c.on_new_token() ? kTileNewToken : 0);
+    t.q_end = c.q_end;
+    t.kind = 0;
     return t;
   };
   // (the launcher sends only page sizes that are powers of two here)
   auto column_of = [&](int t) { return t >> p.bs_shift; };
   auto slot_of = [&](int t) { return t & (p.block_size - 1); };
-  // The token whose cache row this lane fetches for group tg: its own token of a regular tile (clamped to the last
-  // cached one); the position being appended for a new-token tile (the row is not used, it only has to exist); one
-  // token for all lanes of a phantom tile (a tile past the unit's end: its loads keep the pipeline's shape and hit
-  // one cache line each).
+  // The token whose cache row this lane fetches for group tg: its own token of the tile, clamped to the segment's
+  // last one; one token for all lanes of a phantom tile (a tile past the unit's end: its loads keep the pipeline's
+  // shape and hit one cache line each).
   auto lane_token = [&](const TileDesc& t, int tg) {
     const int own = (t.kind & kTilePhantom) ? 0 : 16 * tg + lr;
-    return (t.kind & kTileNewToken) ? t.end : min(t.tok + own, t.end - 1);
+    return min(t.tok + own, t.end - 1);
   };
-  // (block ids and cache rows are pairs of scalars, one per token group, not arrays: an array indexed by a lane-dependent
+  // (block ids and cache rows are indexed with compile-time constants only: an array indexed by a lane-dependent
   // value would live in scratch memory, and scratch loads count with the global loads and drain the pipeline)
-  struct IdPair {
-    int g0, g1;
+  struct IdSet {
+    int g[NTG];
   };
   auto issue_id_loads = [&](const TileDesc& t) {
     const int32_t* table_row = p.block_table + static_cast<int64_t>(t.row) * p.max_blocks;
-    IdPair r;
-    r.g0 = table_row[column_of(lane_token(t, 0))];
-    r.g1 = table_row[column_of(lane_token(t, 1))];
+    IdSet r;
+#pragma unroll
+    for (int tg = 0; tg < NTG; ++tg) r.g[tg] = table_row[column_of(lane_token(t, tg))];
     return r;
   };
   // cache row (block, slot, head) of this lane's token of each group, from the block ids that have arrived
-  uint32_t row_g0 = 0, row_g1 = 0;
-  auto rows_from_ids = [&](const TileDesc& t, const IdPair& src) {
-    row_g0 = (static_cast<uint32_t>(src.g0) * p.block_size + slot_of(lane_token(t, 0))) * p.kv_heads + kvh;
-    row_g1 = (static_cast<uint32_t>(src.g1) * p.block_size + slot_of(lane_token(t, 1))) * p.kv_heads + kvh;
-  };
-  // what an appended token's tile needs: the update rows (first 32 lanes K, the others V) and the cache row they go to
-  auto issue_update_loads = [&](const TileDesc& t) {
-    if constexpr (DSPLIT == 1) {
-      if ((t.kind & (kTileNewToken | kTilePhantom)) == kTileNewToken) {
-        const void* src = lane < 32 ? mp.k_update : mp.v_update;
-        const int64_t off = (static_cast<int64_t>(t.row) * p.kv_heads + kvh) * D * 2 + (lane & 31) * (UPW * 4);
+  uint32_t row_g[NTG];
+  auto rows_from_ids = [&](const TileDesc& t, const IdSet& src) {
 #pragma unroll
-        for (int w = 0; w < UPW; ++w) upd[w] = *reinterpret_cast<const uint32_t*>(static_cast<const char*>(src) + off + 4 * w);
-      }
-      new_row = row_g0;
-    }
+    for (int tg = 0; tg < NTG; ++tg)
+      row_g[tg] = (static_cast<uint32_t>(src.g[tg]) * p.block_size + slot_of(lane_token(t, tg))) * p.kv_heads + kvh;
   };
-  auto issue_v_loads = [&](const TileDesc& t) {
-    issue_update_loads(t);
+  auto issue_v_loads = [&]() {
 #pragma unroll
-    for (int tg = 0; tg < 2; ++tg) {
-      const char* va = static_cast<const char*>(p.v_cache) + (tg ? row_g1 : row_g0) * row_bytes + half_bytes + lk * 16;
+    for (int tg = 0; tg < NTG; ++tg) {
+      const char* va = static_cast<const char*>(p.v_cache) + row_g[tg] * row_bytes + half_bytes + lk * 16;
 #pragma unroll
       for (int j = 0; j < CPL; ++j) vreg[tg * CPL + j] = *reinterpret_cast<const uint4_t*>(va + 64 * j);
     }
     if constexpr (T::kQuant) {
-      const uint32_t r = (lk & 1) ? row_g1 : row_g0;
-      const void* sp = lk < 2 ? p.k_scale : p.v_scale;
-      sreg = static_cast<const scale_raw_t*>(sp)[r];
+      // entry e = lane + 64 i is the scale of token e % TK = 16 (lk % NTG) + lr, whose cache row this lane holds
+      uint32_t r = row_g[0];
+#pragma unroll
+      for (int tg = 1; tg < NTG; ++tg) r = (lk % NTG) == tg ? row_g[tg] : r;
+#pragma unroll
+      for (int i = 0; i < SPL; ++i) {
+        const bool is_v = (lane + kWave * i) >= TK;
+        sreg[i] = static_cast<const scale_raw_t*>(is_v ? p.v_scale : p.k_scale)[r];
+      }
     }
   };
-  auto issue_k_loads = [&](const TileDesc& t) {
+  auto issue_k_loads = [&]() {
 #pragma unroll
-    for (int tg = 0; tg < 2; ++tg) {
-      const char* ka = static_cast<const char*>(p.k_cache) + (tg ? row_g1 : row_g0) * row_bytes + half_bytes + lk * 16;
+    for (int tg = 0; tg < NTG; ++tg) {
+      const char* ka = static_cast<const char*>(p.k_cache) + row_g[tg] * row_bytes + half_bytes + lk * 16;
 #pragma unroll
       for (int j = 0; j < CPL; ++j) kreg[tg * CPL + j] = *reinterpret_cast<const uint4_t*>(ka + 64 * j);
     }
@@ -431,25 +528,28 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   };
 
   // Q of an item: lane (lr = column, lk) needs, per k-slice, the 8 elements the K loads put there; 16 raw bytes per
-  // slice for 16-bit queries.  Requested one step before the item's first tile is computed, converted when compute
-  // gets there.  Column lr of the MFMA tiles: head lr of the row in a per-row item, (row lr / G, head lr % G) in a
-  // shared item.
+  // slice for 16-bit queries.  Column lr of the MFMA tiles: head lr of the row in a per-row item, (row lr / G, head
+  // lr % G) in a shared item.  The first step of a segment fetches the Q of the item that follows the segment; the
+  // next item adopts it when the segment is done.  (A column without a head fetches the row of the item's first head,
+  // which adopt_q drops.)
   uint4_t qraw[NS];
+  bool q_live = false;          // whether this lane's column has a head in the item q_src points into
+  const char* q_src = nullptr;  // this lane's part of the Q row that the steps fetch
   const int col_seq = GROUPED ? lr / p.group : 0;
   const int col_head = GROUPED ? lr - col_seq * p.group : lr;
-  auto issue_q_loads = [&](int item, int row, int nseq) {
+  auto set_q_source = [&](int item, int row, int nseq) {
     const bool shared = is_shared(item);
     const int m = shared ? col_seq : 0;
     const int g = shared ? col_head : lr;
     const bool live = shared ? m < nseq : lr < p.group;
+    const int64_t head_row = live ? static_cast<int64_t>(row + m) * p.q_heads + h0 + g
+                                  : static_cast<int64_t>(row) * p.q_heads + h0;
+    q_live = live;
+    q_src = static_cast<const char*>(p.q) + (head_row * DFULL + half * D) * 2;
+  };
+  auto issue_q_loads = [&]() {
 #pragma unroll
-    for (int sl = 0; sl < NS; ++sl) {
-      qraw[sl] = uint4_t{0u, 0u, 0u, 0u};
-      if (live) {
-        const int64_t idx = (static_cast<int64_t>(row + m) * p.q_heads + h0 + g) * DFULL + half * D + slice_base(sl);
-        qraw[sl] = load16(p.q, idx * 2);
-      }
-    }
+    for (int sl = 0; sl < NS; ++sl) qraw[sl] = load16(q_src, slice_base(sl) * 2);
   };
   V8 qop[NS];
   float qbias = 0.0f;
@@ -459,6 +559,8 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
 #pragma unroll
     for (int sl = 0; sl < NS; ++sl) {
       uint4_t w = qraw[sl];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = q_live ? w[j] : 0u;
       if (!q_is_operand_type) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -492,7 +594,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   float4_t acc[NB];
   float m_run = kNegInf, l_run = 0.0f;
   // int8: sum over the item's tokens of the probabilities as rounded for P . V, which the offset of the V operands is
-  // taken out with; from the matrix cores (an all-ones A operand puts the column's sum over the tile's 32 tokens, all
+  // taken out with; from the matrix cores (an all-ones A operand puts the column's sum over a pair's 32 tokens, all
   // four k groups included, into every element), like the products it corrects
   float4_t p_sum = {0.0f, 0.0f, 0.0f, 0.0f};
   auto reset_state = [&]() {
@@ -503,32 +605,78 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     p_sum = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
   };
 
-  int unit = 0;
-  auto write_partial = [&](int v, int row, int nseq) {
-    // combine the four k-groups' row sums; every lane of a head ends with the head's totals
-    const float l_tot = rows_sum(l_run);
-    float off = 0.0f;
-    if constexpr (KIND == KV_I8) off = kI8Offset * p_sum[0];
+  auto lds_fence = [&]() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+
+  // A finished segment's partial: the un-normalised accumulator rows and (m, l) of every column.  Per-row items go to
+  // slot unit + row, one row per q head; shared items to slot unit + item, 16 columns per kv head.  Every lane stores
+  // (no branch): columns without a head, and the (m, l) pair of the lanes that do not own it, go to a dump row that
+  // nothing reads.
+  auto store_partial = [&](int v, int row, int nseq, const float4_t (&o)[NB], float m_val, float l_val) {
     const bool shared = is_shared(v);
     const bool live = shared ? col_seq < nseq : lr < p.group;
-    if (live) {
-      // per-row items: slot unit + row, one row per q head; shared items: slot unit + item, 16 columns per kv head
-      const int64_t prow = shared ? (static_cast<int64_t>(unit + v) * p.kv_heads + kvh) * 16 + lr
-                                  : static_cast<int64_t>(unit + row) * p.q_heads + h0 + lr;
-      float* ml = shared ? mp.shared_ml : p.part_ml;
-      float* dst = (shared ? mp.shared_acc : p.part_acc) + prow * DFULL + half * D + 4 * lk;
+    const int64_t prow = shared ? (static_cast<int64_t>(unit + v) * p.kv_heads + kvh) * 16 + lr
+                                : static_cast<int64_t>(unit + row) * p.q_heads + h0 + lr;
+    float* const ml = shared ? mp.shared_ml : p.part_ml;
+    float* const rows = shared ? mp.shared_acc : p.part_acc;
+    float* dst = (live ? rows + prow * DFULL : mp.dump + lr * DFULL) + half * D + 4 * lk;
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        float4_t o = acc[nb];
+    for (int nb = 0; nb < NB; ++nb) *reinterpret_cast<float4_t*>(dst + 16 * nb) = o[nb];
+    float* const ml_dst = (live && lk == 0) ? ml + prow * 2 : mp.dump + 16 * DFULL + 2 * lane;
+    *reinterpret_cast<float2_t*>(ml_dst) = float2_t{m_val, l_val};
+  };
+  auto partial_values = [&](float4_t (&o)[NB], float& l_tot) {
+    // combine the four k-groups' row sums; every lane of a head ends with the head's totals
+    l_tot = rows_sum(l_run);
+    float off = 0.0f;
+    if constexpr (KIND == KV_I8) off = kI8Offset * p_sum[0];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) o[j] = (o[j] - off) * (1.0f / kPScale);
-        *reinterpret_cast<float4_t*>(dst + 16 * nb) = o;
-      }
-      if (lk == 0) {
-        ml[prow * 2] = m_run;
-        ml[prow * 2 + 1] = l_tot;
-      }
+    for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[nb][j] = (acc[nb][j] - off) * (1.0f / kPScale);
     }
+  };
+  // The partial of a segment behind which the unit goes on is parked in LDS and stored when the unit is done.  A
+  // store in the middle of the tile stream would sit in front of every later load in the wave's memory queue, which
+  // retires in order: each wait for a tile behind it would also wait for the stores' acknowledgement (measured: 2.4 us
+  // of a 32.7 us launch on units with two segments).  kDecodeHold partials fit; a unit with more segments stores the
+  // parked ones when the space is full.
+  int held = 0;
+  auto hold_slot = [&](int k) { return reinterpret_cast<float4_t*>(&s_hold[wave][k][0]) + lane; };
+  auto park_partial = [&](int v, int row, int nseq) {
+    float4_t o[NB];
+    float l_tot;
+    partial_values(o, l_tot);
+    float4_t* slot = hold_slot(held);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) slot[nb * kWave] = o[nb];
+    slot[NB * kWave] = float4_t{m_run, l_tot, __builtin_bit_cast(float, v), __builtin_bit_cast(float, (row << 5) | nseq)};
+    ++held;
+  };
+  auto flush_parked = [&]() {
+    lds_fence();
+    for (int k = 0; k < held; ++k) {
+      const float4_t* slot = hold_slot(k);
+      float4_t o[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) o[nb] = slot[nb * kWave];
+      const float4_t tail = slot[NB * kWave];
+      // (copies first: a bit_cast straight from a vector-element lvalue reads element 0)
+      const float item_bits = tail[2], rows_bits = tail[3];
+      const int v = uniform(__builtin_bit_cast(int, item_bits));
+      const int rn = uniform(__builtin_bit_cast(int, rows_bits));
+      store_partial(v, rn >> 5, rn & 31, o, tail[0], tail[1]);
+    }
+    held = 0;
+  };
+  auto write_partial = [&](int v, int row, int nseq) {
+    float4_t o[NB];
+    float l_tot;
+    partial_values(o, l_tot);
+    store_partial(v, row, nseq, o, m_run, l_tot);
   };
 
   // ---- pair synchronisation of the split-head variant ----------------------------------------------------------------
@@ -540,140 +688,9 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       __builtin_amdgcn_s_sleep(1);
     }
   };
-  auto lds_fence = [&]() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  };
 
-  // ---- the token being appended: quantize, store into the page, fold into the running softmax (vector ALU) ---------
-  // `after_read` runs once the update rows are out of their load registers: the next tile's loads go out there, ahead
-  // of the arithmetic, which is long for a step that streams nothing (the next tile may be an appended token's as well
-  // and load into the same registers).
-  auto new_token_step = [&](const TileDesc& t, auto&& after_read) {
-    if constexpr (DSPLIT == 1) {
-      constexpr int EPU = 2 * UPW;  // elements of the row this lane holds: (lane % 32) * EPU ...
-      const int sub = lane & 31;
-      const bool is_v = lane >= 32;
-      float x[EPU];
-      uint32_t raw_row[UPW];
-#pragma unroll
-      for (int w = 0; w < UPW; ++w) raw_row[w] = upd[w];
-      const int64_t dst_row = new_row;  // (the loads of the next tile replace it with theirs)
-      after_read();
-#pragma unroll
-      for (int w = 0; w < UPW; ++w) {
-        const uint32_t word = raw_row[w];
-        if (p.q_dtype == ARENO_DT_BF16) {
-          x[2 * w] = bf16_bits_to_float(word & 0xffffu);
-          x[2 * w + 1] = bf16_bits_to_float(word >> 16);
-        } else {
-          x[2 * w] = f16_bits_to_float(word & 0xffffu);
-          x[2 * w + 1] = f16_bits_to_float(word >> 16);
-        }
-      }
-      char* cache = static_cast<char*>(const_cast<void*>(is_v ? p.v_cache : p.k_cache));
-      float xhat[EPU];  // what a reader of the page sees
-      if constexpr (T::kQuant) {
-        float amax = 0.0f;
-#pragma unroll
-        for (int e = 0; e < EPU; ++e) amax = fmaxf(amax, fabsf(x[e]));
-#pragma unroll
-        for (int m = 1; m < 32; m <<= 1) amax = fmaxf(amax, wave_xor(amax, m));
-        float s, s_stored;
-        scale_raw_t raw;
-        if constexpr (KIND == KV_I8) {
-          const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
-          const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;
-          s = static_cast<float>(s16_fixed);
-          s_stored = s;
-          if constexpr (SCALE16) {
-            raw = __builtin_bit_cast(uint16_t, s16_fixed);
-          } else {
-            raw = s;
-          }
-        } else {
-          s = amax / 448.0f;
-          if (s == 0.0f) s = 1.0f;
-          if constexpr (SCALE16) {
-            raw = static_cast<uint16_t>(float_to_f16_bits(s));
-            s_stored = f16_bits_to_float(raw);
-          } else {
-            raw = s;
-            s_stored = s;
-          }
-        }
-        uint32_t word = 0;
-#pragma unroll
-        for (int e = 0; e < EPU; ++e) {
-          uint32_t byte;
-          float code_value;
-          if constexpr (KIND == KV_I8) {
-            const float code = fminf(fmaxf(rintf(x[e] / s), -127.0f), 127.0f);
-            byte = static_cast<uint32_t>(static_cast<int>(code)) & 0xffu;
-            code_value = code;
-          } else {
-            byte = float_to_fp8_byte(fminf(fmaxf(x[e] / s, -448.0f), 448.0f));
-            code_value = fp8_byte_to_float(byte);
-          }
-          word |= byte << (8 * e);
-          xhat[e] = code_value * s_stored;
-        }
-        char* dst = cache + dst_row * row_bytes + sub * EPU;
-        if constexpr (EPU == 4) {
-          *reinterpret_cast<uint32_t*>(dst) = word;
-        } else {
-          *reinterpret_cast<uint16_t*>(dst) = static_cast<uint16_t>(word);
-        }
-        if (sub == 0) static_cast<scale_raw_t*>(const_cast<void*>(is_v ? p.v_scale : p.k_scale))[dst_row] = raw;
-      } else {
-        // 16-bit pages hold the update row as it is (the launcher only fuses when the dtypes agree)
-        char* dst = cache + dst_row * row_bytes + sub * (EPU * 2);
-#pragma unroll
-        for (int w = 0; w < UPW; ++w) *reinterpret_cast<uint32_t*>(dst + 4 * w) = raw_row[w];
-#pragma unroll
-        for (int e = 0; e < EPU; ++e) xhat[e] = x[e];
-      }
-      // both rows as floats where the V tile is (no tile is staged at this point): K row, then V row
-      float* rowbuf = reinterpret_cast<float*>(v_tile);
-#pragma unroll
-      for (int e = 0; e < EPU; ++e) rowbuf[(is_v ? D : 0) + sub * EPU + e] = xhat[e];
-      lds_fence();
-      // score of the token for column lr: this lane's 8 elements of every k-slice, then the four lanes of the column
-      float dot = 0.0f;
-#pragma unroll
-      for (int sl = 0; sl < NS; ++sl) {
-        const float* kk = rowbuf + slice_base(sl);
-        const uint4_t qw = __builtin_bit_cast(uint4_t, qop[sl]);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const Pair pr = __builtin_bit_cast(Pair, static_cast<uint32_t>(qw[j]));
-          dot += static_cast<float>(pr.x) * kk[2 * j] + static_cast<float>(pr.y) * kk[2 * j + 1];
-        }
-      }
-      const float s_new = rows_sum(dot) * p.scale_log2e;
-      const float m_new = max_f32(m_run, s_new);
-      const float alpha = fast_exp2(m_run - m_new);  // m_run = -inf for a row without cached tokens -> 0
-      const float pn = fast_exp2(s_new - m_new);
-      m_run = m_new;
-      l_run = l_run * alpha + (lk == 0 ? pn : 0.0f);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) p_sum[j] *= alpha;
-      const float pv = pn * kPScale;
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        const float4_t vv = *reinterpret_cast<const float4_t*>(rowbuf + D + 16 * nb + 4 * lk);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[nb][j] = acc[nb][j] * alpha + pv * vv[j];
-      }
-      lds_fence();
-    } else {
-      after_read();  // (the split-head variant appends in a launch of its own and never gets here)
-    }
-  };
-
-  // ---- one regular tile: stage V and the scales, scores, softmax, P.V ----------------------------------------------
-  // `between_v` runs once the V registers of the set are free, `between_k` once the K registers are.
+  // ---- one tile: stage V and the scales, scores, softmax, P.V ------------------------------------------------------
+  // `between_v` runs once the V registers are free, `between_k` once the K registers are.
   auto tile_step = [&](const TileDesc& t, auto&& between_v, auto&& between_k) {
     if constexpr (DSPLIT > 1) {
       // the other waves of the head must have read the score part this wave parked in the previous step
@@ -683,7 +700,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       }
     }
 #pragma unroll
-    for (int tg = 0; tg < 2; ++tg) {
+    for (int tg = 0; tg < NTG; ++tg) {
 #pragma unroll
       for (int j = 0; j < CPL; ++j) {
         uint4_t vv = vreg[tg * CPL + j];
@@ -691,21 +708,26 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
 #pragma unroll
           for (int w = 0; w < 4; ++w) vv[w] ^= kI8Flip;
         }
-        *reinterpret_cast<uint4_t*>(v_tile + tg * TGS + chunk_row_pos(lk + 4 * j, lr)) = vv;
+        *reinterpret_cast<uint4_t*>(v_tile + group_pos(tg) + chunk_row_pos(lk + 4 * j, lr)) = vv;
       }
     }
     if constexpr (T::kQuant) {
-      const bool ok = t.tok + (lane & 31) < t.end;
-      const float s = scale_value(sreg);
-      sc_lds[lane] = lane < 32 ? (ok ? s * p.scale_log2e : kNegInf) : (ok ? s * kPScale : 0.0f);
+#pragma unroll
+      for (int i = 0; i < SPL; ++i) {
+        const int e = lane + kWave * i;
+        const bool is_v = e >= TK;
+        const bool ok = t.tok + (e & (TK - 1)) < t.end;
+        const float s = scale_value(sreg[i]);
+        sc_lds[e] = is_v ? (ok ? s * kPScale : 0.0f) : (ok ? s * p.scale_log2e : kNegInf);
+      }
     }
     lds_fence();
-    between_v();  // the V registers of the set are free
+    between_v();  // the V registers are free
 
-    // -- S^T = K . Q^T for the two 16-token groups ------------------------------------------------------------------
-    float s[2][4];
+    // -- S^T = K . Q^T for the 16-token groups ----------------------------------------------------------------------
+    float s[NTG][4];
 #pragma unroll
-    for (int tg = 0; tg < 2; ++tg) {
+    for (int tg = 0; tg < NTG; ++tg) {
       // int8: the products start from -1152 * sum(q) (score_init), which takes the offset of the operands out again
       float4_t c = score_init;
 #pragma unroll
@@ -725,9 +747,9 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     between_k();
     if constexpr (DSPLIT > 1) {
       // Park the part, tell the other waves of the head, wait for their parts, add all parts in the order of the head
-      // dimension.  Every wave of the head ends up with the same eight sums.
+      // dimension.  Every wave of the head ends up with the same sums.
 #pragma unroll
-      for (int tg = 0; tg < 2; ++tg) {
+      for (int tg = 0; tg < NTG; ++tg) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) park[(4 * tg + j) * kWave + lane] = s[tg][j];
       }
@@ -736,9 +758,9 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       if (lane == 0)
         __hip_atomic_store(&s_pair_flags[0][wave], pair_step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       const int first_wave = wave - half;
-      float total[2][4];
+      float total[NTG][4];
 #pragma unroll
-      for (int tg = 0; tg < 2; ++tg) {
+      for (int tg = 0; tg < NTG; ++tg) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) total[tg][j] = 0.0f;
       }
@@ -746,16 +768,16 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       for (int part = 0; part < DSPLIT; ++part) {
         if (part == half) {
 #pragma unroll
-          for (int tg = 0; tg < 2; ++tg) {
+          for (int tg = 0; tg < NTG; ++tg) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) total[tg][j] += s[tg][j];
           }
         } else {
           pair_wait(&s_pair_flags[0][first_wave + part], pair_step);
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-          const float* theirs = reinterpret_cast<const float*>(&s_tiles[first_wave + part][2 * TGS + 2 * TK * 4]);
+          const float* theirs = reinterpret_cast<const float*>(&s_tiles[first_wave + part][NTG * TGS + 2 * TK * 4]);
 #pragma unroll
-          for (int tg = 0; tg < 2; ++tg) {
+          for (int tg = 0; tg < NTG; ++tg) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) total[tg][j] += theirs[(4 * tg + j) * kWave + lane];
           }
@@ -765,19 +787,19 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       if (lane == 0)
         __hip_atomic_store(&s_pair_flags[1][wave], pair_step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 #pragma unroll
-      for (int tg = 0; tg < 2; ++tg) {
+      for (int tg = 0; tg < NTG; ++tg) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) s[tg][j] = total[tg][j];
       }
     }
     // the per-token K scale (softmax scale and log2 e folded in); tokens past the end become exactly -inf, which only
-    // an item's last tile has: every other tile takes the branch with one multiply per score
-    float vs[2][4];
+    // a segment's last tile has: every other tile takes the branch with one multiply per score
+    float vs[NTG][4];
     const bool whole_tile = t.tok + TK <= t.end;  // (scalar)
 #pragma unroll
-    for (int tg = 0; tg < 2; ++tg) {
+    for (int tg = 0; tg < NTG; ++tg) {
       if constexpr (T::kQuant) {
-        const float4_t vv = *reinterpret_cast<const float4_t*>(sc_lds + 32 + 16 * tg + 4 * lk);
+        const float4_t vv = *reinterpret_cast<const float4_t*>(sc_lds + TK + 16 * tg + 4 * lk);
 #pragma unroll
         for (int j = 0; j < 4; ++j) vs[tg][j] = vv[j];
       } else {
@@ -787,7 +809,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     }
     if (whole_tile) {
 #pragma unroll
-      for (int tg = 0; tg < 2; ++tg) {
+      for (int tg = 0; tg < NTG; ++tg) {
         float4_t ks = {p.scale_log2e, p.scale_log2e, p.scale_log2e, p.scale_log2e};
         if constexpr (T::kQuant) ks = *reinterpret_cast<const float4_t*>(sc_lds + 16 * tg + 4 * lk);
 #pragma unroll
@@ -795,7 +817,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       }
     } else {
 #pragma unroll
-      for (int tg = 0; tg < 2; ++tg) {
+      for (int tg = 0; tg < NTG; ++tg) {
         if constexpr (T::kQuant) {
           const float4_t ks = *reinterpret_cast<const float4_t*>(sc_lds + 16 * tg + 4 * lk);
 #pragma unroll
@@ -810,10 +832,14 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
       }
     }
 
-    // -- online softmax for column lr over the tile's 32 tokens ------------------------------------------------------
-    float mt = max3_f32(max3_f32(s[0][0], s[0][1], s[0][2]), max3_f32(s[0][3], s[1][0], s[1][1]),
-                        max_f32(s[1][2], s[1][3]));
-    mt = rows_max(mt);
+    // -- online softmax for column lr over the tile's tokens ---------------------------------------------------------
+    float flat[4 * NTG];
+#pragma unroll
+    for (int tg = 0; tg < NTG; ++tg) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) flat[4 * tg + j] = s[tg][j];
+    }
+    const float mt = rows_max(max_all<4 * NTG>(flat));
     const float m_new = max_f32(m_run, mt);
     const float m_safe = m_new == kNegInf ? 0.0f : m_new;
     const float alpha = fast_exp2(m_run - m_safe);
@@ -828,57 +854,60 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
         for (int j = 0; j < 4; ++j) acc[nb][j] *= alpha;
       }
     }
-    uint32_t pw[4];
-    {
+    V8 pop[NPP];
+#pragma unroll
+    for (int pp = 0; pp < NPP; ++pp) {
       float pe[8];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float e0 = fast_exp2(s[0][j] - m_safe);
-        const float e1 = fast_exp2(s[1][j] - m_safe);
+        const float e0 = fast_exp2(s[2 * pp][j] - m_safe);
+        const float e1 = fast_exp2(s[2 * pp + 1][j] - m_safe);
         l_run += e0 + e1;
-        pe[j] = T::kQuant ? e0 * vs[0][j] : e0;
-        pe[4 + j] = T::kQuant ? e1 * vs[1][j] : e1;
+        pe[j] = T::kQuant ? e0 * vs[2 * pp][j] : e0;
+        pe[4 + j] = T::kQuant ? e1 * vs[2 * pp + 1][j] : e1;
       }
+      uint32_t pw[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        pw[j] = pack_pair<KIND>(pe[2 * j], pe[2 * j + 1]);
+      for (int j = 0; j < 4; ++j) pw[j] = pack_pair<KIND>(pe[2 * j], pe[2 * j + 1]);
+      pop[pp] = __builtin_bit_cast(V8, uint4_t{pw[0], pw[1], pw[2], pw[3]});
+      if constexpr (KIND == KV_I8) {
+        constexpr uint32_t kOnes = 0x3c003c00u;  // two fp16 1.0
+        p_sum = Ops::mfma(__builtin_bit_cast(V8, uint4_t{kOnes, kOnes, kOnes, kOnes}), pop[pp], p_sum);
       }
-    }
-    const V8 pop = __builtin_bit_cast(V8, uint4_t{pw[0], pw[1], pw[2], pw[3]});
-    if constexpr (KIND == KV_I8) {
-      constexpr uint32_t kOnes = 0x3c003c00u;  // two fp16 1.0
-      p_sum = Ops::mfma(__builtin_bit_cast(V8, uint4_t{kOnes, kOnes, kOnes, kOnes}), pop, p_sum);
     }
 
-    // -- O^T += V^T . P^T, one MFMA per 16-dim block -----------------------------------------------------------------
+    // -- O^T += V^T . P^T, one MFMA per 16-dim block and pair of token groups ----------------------------------------
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      uint32_t vw[4];
-      if constexpr (ES == 1) {
-        // lane i of a 16-lane group supplies token row (i / 2), 8 bytes at column 8 (i % 2) of chunk nb: rows 0..3 are
-        // tokens 4 lk .. 4 lk + 3 of group 0, rows 4..7 the same tokens of group 1
-        const int r8 = lr >> 1;
-        const int tg = r8 >> 2;
-        const int tok = 4 * lk + (r8 & 3);
-        char* a = v_tile + tg * TGS + chunk_row_pos(nb, tok) + 8 * (lr & 1);
-        const int2_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_int2*)a);
-        vw[0] = static_cast<uint32_t>(r[0]);
-        vw[1] = static_cast<uint32_t>(r[1]);
-      } else {
-        // lane i supplies token row (i / 4), 4 elements at column 4 (i % 4) of the 16-dim block: chunk 2 nb + (i % 4) / 2,
-        // byte 8 ((i % 4) % 2); two reads of 4 tokens, one per token group
-        const int r4 = lr >> 2;
-        const int c4 = lr & 3;
+    for (int pp = 0; pp < NPP; ++pp) {
 #pragma unroll
-        for (int tg = 0; tg < 2; ++tg) {
-          char* a = v_tile + tg * TGS + chunk_row_pos(2 * nb + (c4 >> 1), 4 * lk + r4) + 8 * (c4 & 1);
-          const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
-          const uint2_t u = __builtin_bit_cast(uint2_t, r);
-          vw[2 * tg] = u[0];
-          vw[2 * tg + 1] = u[1];
+      for (int nb = 0; nb < NB; ++nb) {
+        uint32_t vw[4];
+        if constexpr (ES == 1) {
+          // lane i of a 16-lane group supplies token row (i / 2), 8 bytes at column 8 (i % 2) of chunk nb: rows 0..3 are
+          // tokens 4 lk .. 4 lk + 3 of the pair's first group, rows 4..7 the same tokens of its second group
+          const int r8 = lr >> 1;
+          const int tg = 2 * pp + (r8 >> 2);
+          const int tok = 4 * lk + (r8 & 3);
+          char* a = v_tile + group_pos(tg) + chunk_row_pos(nb, tok) + 8 * (lr & 1);
+          const int2_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_int2*)a);
+          vw[0] = static_cast<uint32_t>(r[0]);
+          vw[1] = static_cast<uint32_t>(r[1]);
+        } else {
+          // lane i supplies token row (i / 4), 4 elements at column 4 (i % 4) of the 16-dim block: chunk 2 nb + (i % 4) / 2,
+          // byte 8 ((i % 4) % 2); two reads of 4 tokens, one per token group
+          const int r4 = lr >> 2;
+          const int c4 = lr & 3;
+#pragma unroll
+          for (int g2 = 0; g2 < 2; ++g2) {
+            char* a = v_tile + group_pos(2 * pp + g2) + chunk_row_pos(2 * nb + (c4 >> 1), 4 * lk + r4) + 8 * (c4 & 1);
+            const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
+            const uint2_t u = __builtin_bit_cast(uint2_t, r);
+            vw[2 * g2] = u[0];
+            vw[2 * g2 + 1] = u[1];
+          }
         }
+        acc[nb] = Ops::mfma(to_operand<KIND>(vw), pop[pp], acc[nb]);
       }
-      acc[nb] = Ops::mfma(to_operand<KIND>(vw), pop, acc[nb]);
     }
     // all LDS reads of this tile are done before the next step overwrites it
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -886,109 +915,105 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   };
 
   // ---- this wave's unit --------------------------------------------------------------------------------------------
-  unit = blockIdx.x * mp.tok_splits + ts;
-  const int x0 = geo.unit_start(unit);
-  const int x1 = geo.unit_start(unit + 1);
-  if (x0 < x1) {
-    // move the request cursor to tile x (a phantom past the unit's end) and ask for its block ids
-    IdPair ids;  // block ids of the tile the request cursor is on
-    auto request = [&](int x) {
-      if (x < x1) {
-        const bool opens = cursor_advance<GROUPED>(cur, shape, lens, cum, x);
-        desc_ids = describe(cur, opens);
-      } else {
-        desc_ids.kind = (desc_ids.kind & kTileNewToken) | kTilePhantom;
+  if (q0 < q1) {
+    // move the request cursor one tile on (to a phantom past the unit's end) and ask for that tile's block ids
+    IdSet ids;  // block ids of the tile the request cursor is on
+    auto request_next = [&]() {
+      if (!(desc_ids.kind & kTilePhantom)) {
+        const CursorMove mv = cursor_advance(cur, table, shape.switch_quanta, q1, TK);
+        if (mv == kCursorUnitDone) {
+          desc_ids.kind = kTilePhantom;
+        } else {
+          desc_ids = describe(cur);
+        }
       }
       ids = issue_id_loads(desc_ids);
     };
-    // ---- prologue: block ids of the first two tiles one behind the other, Q of the first item, the first tile's
-    // loads ------------------------------------------------------------------------------------------------------------
-    cursor_seek<GROUPED>(cur, shape, lens, cum, x0);
-    desc_ids = describe(cur, true);
-    const IdPair ids_first = issue_id_loads(desc_ids);
-    issue_q_loads(desc_ids.b, desc_ids.row, desc_ids.nseq);
+    // ---- prologue: block ids of the first tile (from the unit record when there is a plan), Q of the first item,
+    // the first tile's loads, block ids of the second tile ------------------------------------------------------------
+    desc_ids = describe(cur);
     desc0 = desc_ids;
-    request(x0 + 1);
+    IdSet ids_first;
+    // a record's ids cover kPlanUnitIds columns from the first token's: enough unless pages are very small
+    const bool ids_from_plan = planned && column_of(desc0.tok + TK - 1) - column_of(desc0.tok) < kPlanUnitIds;
+    if (ids_from_plan) {
+      const int col0 = column_of(desc0.tok);
+#pragma unroll
+      for (int tg = 0; tg < NTG; ++tg) {
+        const int c = column_of(lane_token(desc0, tg)) - col0;
+        int id = first_ids[0];
+#pragma unroll
+        for (int i = 1; i < kPlanUnitIds; ++i) id = c == i ? first_ids[i] : id;
+        ids_first.g[tg] = id;
+      }
+    } else {
+      ids_first = issue_id_loads(desc0);
+    }
+    set_q_source(desc0.b, desc0.row, desc0.nseq);
+    issue_q_loads();
+    request_next();  // the second tile's ids right behind the first tile's
     rows_from_ids(desc0, ids_first);
-    issue_v_loads(desc0);
-    issue_k_loads(desc0);
+    issue_v_loads();
+    issue_k_loads();
     adopt_q();
     reset_state();
 
     // One step of the pipeline on the tile in the registers (tile x): the ids of tile x + 1 have arrived (requested a
-    // step ago), those of tile x + 2 are requested, and tile x + 1's loads go out as `work` frees the V registers
+    // step ago), those of tile x + 2 are requested, and tile x + 1's loads go out as the step frees the V registers
     // (`between_v`) and the K registers (`between_k`).
-    auto step = [&](int x, auto&& work, auto stream_next) {
+    auto step = [&](auto first_of_segment) {
       ARENO_TRACE_POINT();
       const TileDesc t = desc0;
       const TileDesc nt = desc_ids;
       rows_from_ids(nt, ids);
       // the ids are consumed before the next ones are requested into the same registers
       __builtin_amdgcn_sched_barrier(0);
-      request(x + 2);
+      request_next();
+      if constexpr (decltype(first_of_segment)::value) issue_q_loads();
       // (scheduling barriers: a load of the next tile must not move in front of the last use of the registers it
       // fills, or the two values would need different registers and a copy of a value still in flight)
-      work(
+      tile_step(
           t,
           [&]() {
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (decltype(stream_next)::value) {
-              issue_v_loads(nt);
-            } else {
-              issue_update_loads(nt);  // the next tile is an appended token's: it streams nothing
-            }
+            issue_v_loads();
             __builtin_amdgcn_sched_barrier(0);
           },
           [&]() {
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (decltype(stream_next)::value) issue_k_loads(nt);
+            issue_k_loads();
             __builtin_amdgcn_sched_barrier(0);
           });
       desc0 = nt;
     };
-    using std::false_type;
-    using std::true_type;
 
-    // The unit as a sequence of item segments: the tiles of one item that fall into the unit.  The loop over a
-    // segment's regular tiles has no item logic in it (so nothing but the tile stream is carried around it); the
-    // appended token's tile, the partial and the switch to the next item's Q come behind it.
-    int x = x0;
+    // The unit as a sequence of segments: the tiles of one item that fall into the unit.  The loop over a segment's
+    // tiles has no item logic in it (so nothing but the tile stream is carried around it); the partial and the switch
+    // to the next item's Q come behind it.
     for (;;) {
       const TileDesc first = desc0;
-      const int seg_end = min(x1, first.x_end);
-      const bool appended = shape.new_token_tile && !is_shared(first.b) && seg_end == first.x_end;
-      const int regular_end = seg_end - (appended ? 1 : 0);
-      if (first.x_end < x1) {
-        // Q of the next item with tiles: requested now (qraw is free), adopted when this segment is done
-        int b2 = first.b + 1;
-        while (cum.at(b2 + 1) == first.x_end) ++b2;
-        const ItemInfo it2 = item_info<GROUPED>(shape, lens, b2);
-        issue_q_loads(b2, it2.row, it2.nseq);
+      const int steps = (first.end - first.tok + TK - 1) / TK;
+      // the next item the unit holds quanta of, if any: its Q is what this segment's first step fetches
+      const int b2 = next_item_in_unit(table, shape.switch_quanta, first.b, first.q_end, q1);
+      const bool more = b2 >= 0;
+      if (more) {
+        const ItemInfo it2 = table.info(b2);
+        set_q_source(b2, it2.row, it2.nseq);
       }
-      // An appended token's tile streams nothing, so the regular tile in front of it fetches only the update rows,
-      // and the tile behind it is requested at the start of the appended token's own step.
-      auto regular = [&](const TileDesc& t, auto&& between_v, auto&& between_k) { tile_step(t, between_v, between_k); };
-      const int streaming_end = regular_end - (appended ? 1 : 0);
-      for (; x < streaming_end; ++x) step(x, regular, true_type{});
-      if (appended) {
-        if (x < regular_end) {
-          step(x, regular, false_type{});
-          ++x;
-        }
-        step(
-            x,
-            [&](const TileDesc& t, auto&& between_v, auto&& between_k) {
-              new_token_step(t, [&]() {
-                between_v();
-                between_k();
-              });
-            },
-            true_type{});
-        ++x;
+      // The first step of a segment is a copy of its own that fetches the Q of the item that follows the segment (of
+      // the segment's own item when none follows) at a fixed place in its load sequence, so no load sits behind a
+      // branch and the waits the compiler places in either copy count exactly the loads that are in flight.
+      step(std::true_type{});
+      for (int i = 1; i < steps; ++i) step(std::false_type{});
+      // the next item's Q first (its loads are older than a tile's), the partial's stores behind it
+      if (!more) {
+        write_partial(first.b, first.row, first.nseq);
+        flush_parked();
+        break;
       }
-      write_partial(first.b, first.row, first.nseq);
-      if (x >= x1) break;
       adopt_q();
+      if (held == kDecodeHold) flush_parked();
+      park_partial(first.b, first.row, first.nseq);
       reset_state();
     }
   }

@@ -9,6 +9,7 @@
 
 #include <mutex>
 
+#include "cache_row_quant.hpp"
 #include "decode_mfma_kernels.hpp"
 
 namespace areno {
@@ -130,12 +131,20 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_kernel(Decod
   }
 }
 
-// Merge of the MFMA path's partials.  The units that own tiles of an item wrote one partial each: a per-row item
+// Merge of the MFMA path's partials.  The units that own quanta of an item wrote one partial each: a per-row item
 // into slot (unit + row) of the per-row region, a shared-prefix item (grouped mode) into slot (unit + item) of the
 // shared region, where the row's head sits in column (row - first row) * G + head of its kv head.  One wave per
 // (row, q head) gathers the candidates of both kinds: lanes first fetch up to 64 (m, l) pairs in parallel and agree
 // on the maximum, then every lane accumulates its share of the head dimension with the partial loads of a group of
 // four candidates in flight together (the loop has no loop-carried memory dependence).
+//
+// The token being appended (items.append_in_merge): the streaming waves of the split kernel read only what is in the
+// pages, and this kernel, which owns the (row, head) anyway, does what the reference's update kernel
+// (areno/accel/csrc/attention.cu:526-553) and the last key of its split kernel do: the wave reads the row of
+// k_update / v_update of its kv head, quantizes it with the cache writer's closed form, the wave of the kv head's
+// first q head stores codes and scale at (block_table[b, L / bs], L % bs) -- skipped, like the cache writer does, when
+// the column or the page id lies outside the table or the pool -- and the token enters the merge as a partial of its
+// own with m = q . k_new, l = 1, acc = v_new, both as a reader of the page would see them.
 template <int EPW>  // head-dimension elements per lane: head_dim <= 64 EPW
 __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel(MfmaDecodeParams mp) {
   const DecodeParams& p = mp.d;
@@ -147,14 +156,75 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   const int d = p.head_dim;
   const ItemShape& shape = mp.items;
   const int num_items = shape.num_items();
-  // the plan entries this row needs, fetched together (their indices follow from the row alone)
+  const int32_t* cum = mp.plan_cum != nullptr ? mp.plan_cum : mp.cum_out;
+  // the prefix sums this row needs, fetched together (their indices follow from the row alone)
   const int v_own = shape.num_shared + b;
-  const int plan_total = mp.plan[num_items], plan_own = mp.plan[v_own], plan_own_end = mp.plan[v_own + 1];
-  const UnitGeometry geo = make_unit_geometry(plan_total, mp.num_units);
-  // the row's own item (always at least one tile) ...
-  const int own_lo = geo.unit_of(plan_own);
-  const int own_n = geo.unit_of(plan_own_end - 1) - own_lo + 1;
-  // ... and the shared item of its sub-group, if it has tiles
+  const int cum_total = cum[num_items], cum_own = cum[v_own], cum_own_end = cum[v_own + 1];
+
+  float acc[EPW];
+#pragma unroll
+  for (int e = 0; e < EPW; ++e) acc[e] = 0.0f;
+  float m = kNegInf, l = 0.0f;
+  if (shape.append_in_merge) {
+    const int kvh = h / p.group;
+    const int64_t src_base = (static_cast<int64_t>(b) * p.kv_heads + kvh) * d;
+    float qv[EPW], kx[EPW], vx[EPW];
+    uint16_t kraw[EPW], vraw[EPW];
+#pragma unroll
+    for (int e = 0; e < EPW; ++e) {
+      const int idx = lane + e * kWave;
+      const bool in = idx < d;
+      kraw[e] = in ? static_cast<const uint16_t*>(mp.k_update)[src_base + idx] : 0;
+      vraw[e] = in ? static_cast<const uint16_t*>(mp.v_update)[src_base + idx] : 0;
+      qv[e] = in ? load_as_float(p.q, static_cast<int64_t>(row) * d + idx, p.q_dtype) : 0.0f;
+      kx[e] = p.q_dtype == ARENO_DT_BF16 ? bf16_bits_to_float(kraw[e]) : f16_bits_to_float(kraw[e]);
+      vx[e] = p.q_dtype == ARENO_DT_BF16 ? bf16_bits_to_float(vraw[e]) : f16_bits_to_float(vraw[e]);
+    }
+    const int64_t pos = p.cache_seqlens[b];
+    const int64_t col = pos / p.block_size;
+    const int64_t slot = pos - col * p.block_size;
+    bool ok = pos >= 0 && col < p.max_blocks;
+    const int64_t blk = ok ? p.block_table[static_cast<int64_t>(b) * p.max_blocks + col] : 0;
+    ok = ok && blk >= 0 && blk < mp.num_blocks;
+    const bool store = ok && mp.write_append != 0 && h == kvh * p.group;
+    const int64_t dst_row = (blk * p.block_size + slot) * p.kv_heads + kvh;
+    float khat[EPW], vhat[EPW];
+    if (is_quantized_dtype(p.cache_dtype)) {
+      quantize_row<EPW>(kx, lane, d, dst_row, const_cast<void*>(p.k_cache), const_cast<void*>(p.k_scale), p.cache_dtype,
+                        p.scale_dtype, store, khat);
+      quantize_row<EPW>(vx, lane, d, dst_row, const_cast<void*>(p.v_cache), const_cast<void*>(p.v_scale), p.cache_dtype,
+                        p.scale_dtype, store, vhat);
+    } else {
+      // 16-bit pages of the query's dtype hold the update row as it is
+#pragma unroll
+      for (int e = 0; e < EPW; ++e) {
+        const int idx = lane + e * kWave;
+        if (store && idx < d) {
+          static_cast<uint16_t*>(const_cast<void*>(p.k_cache))[dst_row * d + idx] = kraw[e];
+          static_cast<uint16_t*>(const_cast<void*>(p.v_cache))[dst_row * d + idx] = vraw[e];
+        }
+        khat[e] = kx[e];
+        vhat[e] = vx[e];
+      }
+    }
+    float dot = 0.0f;
+#pragma unroll
+    for (int e = 0; e < EPW; ++e) dot += qv[e] * khat[e];
+    m = wave_sum(dot) * p.scale_log2e;
+    l = 1.0f;
+#pragma unroll
+    for (int e = 0; e < EPW; ++e) acc[e] = vhat[e];
+  }
+
+  const UnitGeometry geo = make_unit_geometry(cum_total, mp.num_units);
+  // the row's own item, if it has quanta ...
+  int own_lo = 0, own_n = 0;
+  if (cum_own_end > cum_own) {
+    int last;
+    item_units(geo, shape.switch_quanta, cum_own, cum_own_end, own_lo, last);
+    own_n = last - own_lo + 1;
+  }
+  // ... and the shared item of its sub-group, if it has quanta
   int sh_lo = 0, sh_n = 0, sh_item = 0, sh_col = 0;
   if (shape.num_shared > 0) {
     const int gi = b / shape.group_rows;
@@ -163,9 +233,10 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
     const int first_row = gi * shape.group_rows + j * shape.cols_seqs;
     const int kvh = h / p.group;
     sh_col = kvh * 16 + (b - first_row) * p.group + (h - kvh * p.group);
-    if (mp.plan[sh_item + 1] > mp.plan[sh_item]) {
-      sh_lo = geo.unit_of(mp.plan[sh_item]);
-      sh_n = geo.unit_of(mp.plan[sh_item + 1] - 1) - sh_lo + 1;
+    if (cum[sh_item + 1] > cum[sh_item]) {
+      int last;
+      item_units(geo, shape.switch_quanta, cum[sh_item], cum[sh_item + 1], sh_lo, last);
+      sh_n = last - sh_lo + 1;
     }
   }
   const int total = own_n + sh_n;
@@ -184,15 +255,11 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
     }
   };
 
-  float acc[EPW];
-#pragma unroll
-  for (int e = 0; e < EPW; ++e) acc[e] = 0.0f;
-  float m = kNegInf, l = 0.0f;
   for (int base = 0; base < total; base += kWave) {
     // lane j looks at candidate base + j
     float part_m = kNegInf, part_l = 0.0f;
     if (base + lane < total) {
-      // a unit without tiles wrote nothing: its candidate is absent (weight 0 below)
+      // a unit without quanta wrote nothing: its candidate is absent (weight 0 below)
       const int u = unit_of_candidate(base + lane);
       if (geo.unit_start(u) != geo.unit_start(u + 1)) {
         const float* ml = nullptr;
@@ -226,7 +293,7 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
 #pragma unroll
         for (int e = 0; e < EPW; ++e) {
           const int idx = lane + e * kWave;
-          // partials of units without tiles were never written: read only what carries a non-zero weight
+          // partials of units without quanta were never written: read only what carries a non-zero weight
           v[jj][e] = (idx < d && present) ? part[idx] : 0.0f;
         }
       }
@@ -265,8 +332,9 @@ constexpr int kComputeUnits = 256;
 constexpr int kMfmaWorkgroups = kComputeUnits;
 constexpr int kMfmaMaxUnits = kMfmaWorkgroups * kMfmaWaves;  // one kv head, every wave a unit of its own
 
+// partials of `slots` slots, and behind them the dump row of the lanes that own no partial row
 size_t mfma_partial_bytes(size_t slots, int q_heads, int head_dim) {
-  const size_t bytes = slots * q_heads * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
+  const size_t bytes = (slots * q_heads * (static_cast<size_t>(head_dim) + 2) + kDecodeDumpFloats) * sizeof(float);
   return (bytes + 255) / 256 * 256;
 }
 
@@ -362,7 +430,7 @@ MfmaGrid mfma_grid_for(int kv_heads, int head_dim) {
   return g;
 }
 
-// plan of the grouped item list (up to one shared item per row on top of the rows), kept 256-byte granular
+// cum entries of the grouped item list (up to one shared item per row on top of the rows), kept 256-byte granular
 size_t grouped_plan_bytes(int batch) { return ((2 * static_cast<size_t>(batch) + 64) * sizeof(int32_t) + 255) / 256 * 256; }
 
 size_t shared_region_bytes(int kv_heads, int head_dim, int num_shared) {
@@ -370,11 +438,201 @@ size_t shared_region_bytes(int kv_heads, int head_dim, int num_shared) {
   return slots * kv_heads * 16 * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
 }
 
+decode_mfma_fn mfma_lookup(const areno_paged_cache* cache, bool grouped) {
+  const bool s16 = cache->scale_dtype == ARENO_DT_F16;
+  switch (cache->cache_dtype) {
+    case ARENO_DT_BF16: return decode_mfma_lookup_bf16(cache->head_dim, s16, grouped);
+    case ARENO_DT_F16: return decode_mfma_lookup_f16(cache->head_dim, s16, grouped);
+    case ARENO_DT_I8: return decode_mfma_lookup_i8(cache->head_dim, s16, grouped);
+    case ARENO_DT_FP8_E4M3: return decode_mfma_lookup_fp8(cache->head_dim, s16, grouped);
+    default: return nullptr;
+  }
+}
+
+// Whether (and how) the matrix-core kernel serves a call: 16-bit or 8-bit caches, head_dim 64 / 128 / 192 / 256 / 512,
+// up to 16 q heads per kv head, page sizes that are powers of two, at most kMfmaMaxBatch rows.  Shared by the decode
+// launcher and the plan builder, which must agree on the item list and the units.
+struct MfmaChoice {
+  decode_mfma_fn fn;  // NULL: another kernel takes the call
+  MfmaGrid grid;
+  ItemShape items;
+  int tile_tokens;
+};
+MfmaChoice choose_mfma(const areno_paged_cache* cache, int q_dtype, int batch, int q_heads, int window_left,
+                       bool with_update, int group_rows, bool has_shared_lens) {
+  MfmaChoice c;
+  c.fn = nullptr;
+  c.grid = mfma_grid_for(cache->kv_heads, cache->head_dim);
+  // what changing items costs a wave, in 16-token quanta of streaming (measured: ~1.4 us against ~1.4 us per 32-token
+  // tile of 8-bit pages, ~2.6 us per tile of 16-bit pages)
+  c.items = ItemShape{batch, window_left, 0, is_quantized(cache->cache_dtype) ? 3 : 1, 0, 1, 1, 1};
+  c.tile_tokens = decode_tile_tokens(is_quantized(cache->cache_dtype));
+  const int group = q_heads / cache->kv_heads;
+  const bool aligned = (reinterpret_cast<uintptr_t>(cache->k) % 16 == 0) && (reinterpret_cast<uintptr_t>(cache->v) % 16 == 0);
+  // the kernel indexes cache rows (block, slot, head) with 32 bits
+  const bool rows_fit = static_cast<double>(cache->num_blocks) * cache->block_size * cache->kv_heads < 4294967296.0;
+  if (!aligned || q_dtype == ARENO_DT_F32 || !prefer_mfma() || group > 16 || batch > kMfmaMaxBatch || !rows_fit ||
+      log2_exact(cache->block_size) < 0)
+    return c;
+  // prefix groups: only without a window, when at least two rows fit side by side
+  int cols_seqs = 0, subs_per_group = 0, num_shared = 0;
+  if (has_shared_lens && window_left < 0) num_shared = shared_items_for(batch, group, group_rows, &cols_seqs, &subs_per_group);
+  c.fn = mfma_lookup(cache, num_shared > 0);
+  if (c.fn == nullptr && num_shared > 0) {
+    // no grouped kernel for this shape: the plain matrix-core kernel, every row reading its own pages
+    num_shared = 0;
+    c.fn = mfma_lookup(cache, false);
+  }
+  if (c.fn == nullptr) return c;
+  // The token being appended is folded in by the merge launch when its row can go into the page as it is (16-bit
+  // pages of the query's dtype) or through the quantizer (8-bit pages); the streaming waves then read the cached
+  // tokens only.
+  c.items.append_in_merge = (with_update && (is_quantized(cache->cache_dtype) || q_dtype == cache->cache_dtype)) ? 1 : 0;
+  if (num_shared > 0) {
+    c.items.num_shared = num_shared;
+    c.items.group_rows = group_rows;
+    c.items.cols_seqs = cols_seqs;
+    c.items.subs_per_group = subs_per_group;
+  }
+  return c;
+}
+
+// ---- the plan: item table, prefix sums and one record per unit, built once for all layers of a decode step ----------
+struct PlanParams {
+  const int32_t* cache_seqlens;
+  const int32_t* shared_lens;
+  const int32_t* block_table;
+  int32_t* cum;
+  int32_t* items;
+  int32_t* units;
+  ItemShape shape;
+  int32_t num_units;
+  int32_t bs_shift;
+  int32_t max_blocks;
+};
+
+struct GlobalLens {
+  const int32_t* len;
+  const int32_t* glen;
+  __device__ int row_len(int b) const { return len[b]; }
+  __device__ int group_len(int g) const { return glen[g]; }
+};
+struct PlainItemTable {
+  const int4_t* item;
+  const int* cum_;
+  __device__ ItemInfo info(int b) const {
+    const int4_t r = item[b];
+    return ItemInfo{r[0], r[1], r[2], r[3]};
+  }
+  __device__ int cum(int i) const { return cum_[i]; }
+};
+
+constexpr int kPlanThreads = 1024;
+
+template <bool GROUPED>
+__global__ __launch_bounds__(kPlanThreads) void decode_plan_kernel(PlanParams pp) {
+  constexpr int kMaxItems = (GROUPED ? 2 : 1) * kMfmaMaxBatch;
+  constexpr int SPT = kMaxItems / kPlanThreads;
+  constexpr int kWaves = kPlanThreads / kWave;
+  __shared__ __attribute__((aligned(16))) int4_t s_item[kMaxItems];
+  __shared__ int s_cum[kMaxItems + 1];
+  __shared__ int s_wave_tot[kWaves];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const ItemShape& shape = pp.shape;
+  const int num_items = shape.num_items();
+  const GlobalLens lens = {pp.cache_seqlens, pp.shared_lens};
+  int nt[SPT];
+  int local = 0;
+#pragma unroll
+  for (int j = 0; j < SPT; ++j) {
+    const int v = SPT * tid + j;
+    nt[j] = 0;
+    if (v < num_items) {
+      const ItemInfo it = item_info<GROUPED>(shape, lens, v);
+      const int4_t r = {it.lo, it.end, it.row, it.nseq};
+      s_item[v] = r;
+      *reinterpret_cast<int4_t*>(pp.items + 4 * static_cast<int64_t>(v)) = r;
+      nt[j] = it.extent(shape.switch_quanta);
+    }
+    local += nt[j];
+  }
+  int incl = local;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int v = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += v;
+  }
+  if (lane == kWave - 1) s_wave_tot[wave] = incl;
+  __syncthreads();
+  int excl = incl - local;
+  for (int w2 = 0; w2 < wave; ++w2) excl += s_wave_tot[w2];
+#pragma unroll
+  for (int j = 0; j < SPT; ++j) {
+    const int v = SPT * tid + j;
+    if (v <= num_items) {
+      s_cum[v] = excl;
+      pp.cum[v] = excl;
+    }
+    excl += nt[j];
+  }
+  if (tid == kPlanThreads - 1 && SPT * (tid + 1) <= num_items) {
+    s_cum[SPT * (tid + 1)] = excl;
+    pp.cum[SPT * (tid + 1)] = excl;
+  }
+  __syncthreads();
+  const PlainItemTable table = {s_item, s_cum};
+  const UnitGeometry geo = make_unit_geometry(s_cum[num_items], pp.num_units);
+  for (int u = tid; u < pp.num_units; u += kPlanThreads) {
+    int rec[kPlanUnitWords];
+#pragma unroll
+    for (int i = 0; i < kPlanUnitWords; ++i) rec[i] = 0;
+    const int q0 = geo.unit_start(u), q1 = geo.unit_start(u + 1);
+    TileCursor c;
+    if (q0 < q1 && cursor_seek(c, table, shape.switch_quanta, num_items, q0, q1)) {
+      rec[kPuQ0] = q0;
+      rec[kPuQ1] = q1;
+      rec[kPuItem] = c.b;
+      rec[kPuTok] = c.tok;
+      rec[kPuSegEnd] = c.seg_end;
+      rec[kPuQEnd] = c.q_end;
+      rec[kPuLo] = c.it.lo;
+      rec[kPuEnd] = c.it.end;
+      rec[kPuRow] = c.it.row;
+      rec[kPuNseq] = c.it.nseq;
+      // block ids of the first tile's columns; columns behind the segment's last one repeat it
+      const int col0 = c.tok >> pp.bs_shift;
+      int last = (c.seg_end - 1) >> pp.bs_shift;
+      last = last < pp.max_blocks - 1 ? last : pp.max_blocks - 1;
+      const int32_t* table_row = pp.block_table + static_cast<int64_t>(c.it.row) * pp.max_blocks;
+#pragma unroll
+      for (int i = 0; i < kPlanUnitIds; ++i) rec[kPuIds + i] = table_row[col0 + i < last ? col0 + i : last];
+    }
+    int4_t* dst = reinterpret_cast<int4_t*>(pp.units + static_cast<int64_t>(u) * kPlanUnitWords);
+#pragma unroll
+    for (int i = 0; i < kPlanUnitWords / 4; ++i) dst[i] = int4_t{rec[4 * i], rec[4 * i + 1], rec[4 * i + 2], rec[4 * i + 3]};
+  }
+}
+
+// layout of a plan buffer for an item list of `items` entries and `units` units, in int32 words
+struct PlanLayout {
+  size_t cum, items, units, words;
+};
+PlanLayout plan_layout(size_t items, size_t units) {
+  PlanLayout l;
+  l.cum = 0;
+  l.items = (items + 1 + 3) / 4 * 4;  // 16-byte aligned
+  l.units = l.items + 4 * items;
+  l.words = l.units + kPlanUnitWords * units;
+  return l;
+}
+
 int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_update, const void* v_update, void* out,
                 int32_t q_dtype, int32_t batch, int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
                 const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits, float softmax_scale,
-                int32_t group_rows, const int32_t* shared_lens, void* workspace, size_t workspace_bytes,
-                int32_t stages, void* stream) {
+                int32_t group_rows, const int32_t* shared_lens, const areno_decode_plan* plan, void* workspace,
+                size_t workspace_bytes, int32_t stages, void* stream) {
   const char* op = "areno_hip_paged_decode";
   if (int rc = validate_paged_cache(cache, op)) return rc;
   if (q == nullptr || out == nullptr || block_table == nullptr || cache_seqlens == nullptr)
@@ -399,16 +657,30 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: block_size * max_blocks out of range", op);
   const size_t base_need = areno_hip_paged_decode_workspace_bytes(batch, q_heads, cache->head_dim, cache->block_size,
                                                                   max_blocks, num_splits);
-  // prefix groups: only without a window, on the matrix-core path, when at least two rows fit side by side
-  int cols_seqs = 0, subs_per_group = 0;
-  int num_shared = 0;
-  if (shared_lens != nullptr && window_left < 0)
-    num_shared = shared_items_for(batch, q_heads / cache->kv_heads, group_rows, &cols_seqs, &subs_per_group);
+  MfmaChoice choice = choose_mfma(cache, q_dtype, batch, q_heads, window_left, k_update != nullptr, group_rows,
+                                  shared_lens != nullptr);
+  if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) choice.fn = nullptr;
+  const int num_shared = choice.fn != nullptr ? choice.items.num_shared : 0;
   const size_t plan_extra = num_shared > 0 ? grouped_plan_bytes(batch) : 0;
   const size_t need =
       base_need + plan_extra + (num_shared > 0 ? shared_region_bytes(cache->kv_heads, cache->head_dim, num_shared) : 0);
   if (workspace == nullptr || workspace_bytes < need)
     return fail(ARENO_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", op, need, workspace_bytes);
+
+  // a plan must have been built for exactly this call's shapes (its tables are read without further checks)
+  const bool planned = plan != nullptr && plan->units > 0;
+  if (planned) {
+    const int32_t eff_group_rows = num_shared > 0 ? group_rows : 0;
+    if (choice.fn == nullptr || plan->buffer == nullptr || plan->batch != batch || plan->q_heads != q_heads ||
+        plan->kv_heads != cache->kv_heads || plan->head_dim != cache->head_dim || plan->block_size != cache->block_size ||
+        plan->max_blocks != max_blocks || plan->window_left != window_left || plan->cache_dtype != cache->cache_dtype ||
+        plan->q_dtype != q_dtype || plan->with_update != (k_update != nullptr ? 1 : 0) ||
+        plan->group_rows != eff_group_rows || plan->units != choice.grid.units ||
+        plan->items != choice.items.num_items() || plan->tile_tokens != choice.tile_tokens)
+      return fail(ARENO_ERR_INVALID_ARGUMENT,
+                  "%s: the plan was built for other shapes (batch, heads, head_dim, page size, table width, window, "
+                  "cache / query dtype, update rows or prefix groups differ)", op);
+  }
 
   DecodeParams p;
   p.q = q;
@@ -439,63 +711,15 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
   p.heads_per_wg = cache->kv_heads % 4 == 0 ? 4 : (cache->kv_heads % 2 == 0 ? 2 : 1);
   p.scale_log2e = softmax_scale * kLog2e;
 
-  decode_split_fn fast = nullptr;
-  const bool aligned = (reinterpret_cast<uintptr_t>(cache->k) % 16 == 0) &&
-                       (reinterpret_cast<uintptr_t>(cache->v) % 16 == 0) &&
-                       (reinterpret_cast<uintptr_t>(workspace) % 16 == 0);
-  if (aligned && q_dtype != ARENO_DT_F32) {
-    switch (cache->cache_dtype) {
-      case ARENO_DT_BF16: fast = decode_split_lookup_bf16(p.head_dim, p.group); break;
-      case ARENO_DT_F16: fast = decode_split_lookup_f16(p.head_dim, p.group); break;
-      case ARENO_DT_I8: fast = decode_split_lookup_i8(p.head_dim, p.group); break;
-      case ARENO_DT_FP8_E4M3: fast = decode_split_lookup_fp8(p.head_dim, p.group); break;
-      default: break;
-    }
-  }
   hipStream_t s = static_cast<hipStream_t>(stream);
-
-  // ---- matrix-core path: 16-bit or 8-bit caches, head_dim 64/128/256, up to 16 q heads per kv head --------
-  decode_mfma_fn mfma = nullptr;
-  // the kernel indexes cache rows (block, slot, head) with 32 bits
-  const bool rows_fit = static_cast<double>(cache->num_blocks) * cache->block_size * cache->kv_heads < 4294967296.0;
-  const bool mfma_ok = aligned && q_dtype != ARENO_DT_F32 && prefer_mfma() && p.group <= 16 &&
-                       batch <= kMfmaMaxBatch && rows_fit && p.bs_shift >= 0;
-  if (mfma_ok) {
-    const bool s16 = cache->scale_dtype == ARENO_DT_F16;
-    const bool grouped = num_shared > 0;
-    switch (cache->cache_dtype) {
-      case ARENO_DT_BF16: mfma = decode_mfma_lookup_bf16(p.head_dim, s16, grouped); break;
-      case ARENO_DT_F16: mfma = decode_mfma_lookup_f16(p.head_dim, s16, grouped); break;
-      case ARENO_DT_I8: mfma = decode_mfma_lookup_i8(p.head_dim, s16, grouped); break;
-      case ARENO_DT_FP8_E4M3: mfma = decode_mfma_lookup_fp8(p.head_dim, s16, grouped); break;
-      default: break;
-    }
-  }
-  if (mfma == nullptr && num_shared > 0) {
-    // no grouped kernel for this shape: the plain matrix-core kernel, every row reading its own pages
-    num_shared = 0;
-    const bool s16 = cache->scale_dtype == ARENO_DT_F16;
-    if (mfma_ok) {
-      switch (cache->cache_dtype) {
-        case ARENO_DT_BF16: mfma = decode_mfma_lookup_bf16(p.head_dim, s16, false); break;
-        case ARENO_DT_F16: mfma = decode_mfma_lookup_f16(p.head_dim, s16, false); break;
-        case ARENO_DT_I8: mfma = decode_mfma_lookup_i8(p.head_dim, s16, false); break;
-        case ARENO_DT_FP8_E4M3: mfma = decode_mfma_lookup_fp8(p.head_dim, s16, false); break;
-        default: break;
-      }
-    }
-  }
-  if (mfma == nullptr) num_shared = 0;  // the other kernels read every row's pages on their own
-  const MfmaGrid grid = mfma_grid_for(cache->kv_heads, p.head_dim);
-  // ---- append: rides along in the matrix-core split kernel as a tile of its own per row when the kernel can take the
-  // new rows as they are (one wave per head, 16-bit pages of the query's dtype or 8-bit pages), else a launch of its
-  // own in front ------------------------------------------------------------------------------------------------------
-  const bool fuse_append =
-      mfma != nullptr && k_update != nullptr && v_update != nullptr && (stages & ARENO_STAGE_APPEND) &&
-      (stages & ARENO_STAGE_SPLIT) && grid.head_split == 1 &&
-      (is_quantized(cache->cache_dtype) || q_dtype == cache->cache_dtype) &&
-      reinterpret_cast<uintptr_t>(k_update) % 8 == 0 && reinterpret_cast<uintptr_t>(v_update) % 8 == 0;
-  if (k_update != nullptr && (stages & ARENO_STAGE_APPEND) && !fuse_append) {
+  const decode_mfma_fn mfma = choice.fn;
+  const MfmaGrid& grid = choice.grid;
+  // ---- append: the merge launch of the matrix-core path does it (append_in_merge); a launch of its own in front of
+  // the other kernels, and for a staged call that asks for the append without the merge ------------------------------
+  const bool merge_appends = mfma != nullptr && choice.items.append_in_merge != 0;
+  const bool append_in_front = k_update != nullptr && (stages & ARENO_STAGE_APPEND) &&
+                               (!merge_appends || !(stages & ARENO_STAGE_REDUCE));
+  if (append_in_front) {
     if (int rc = areno_hip_cache_write_decode(cache, k_update, v_update, q_dtype, batch, block_table, max_blocks,
                                               cache_seqlens, stream))
       return rc;
@@ -507,31 +731,38 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     mp.d.heads_per_wg = grid.heads_per_wg;
     mp.tok_splits = grid.tok_splits;
     mp.num_units = grid.units;
-    mp.items.batch = batch;
-    mp.items.window_left = window_left;
-    mp.items.new_token_tile = fuse_append ? 1 : 0;
-    mp.items.num_shared = num_shared;
-    mp.items.group_rows = num_shared > 0 ? group_rows : 1;
-    mp.items.cols_seqs = num_shared > 0 ? cols_seqs : 1;
-    mp.items.subs_per_group = num_shared > 0 ? subs_per_group : 1;
-    mp.k_update = fuse_append ? k_update : nullptr;
-    mp.v_update = fuse_append ? v_update : nullptr;
+    mp.items = choice.items;
+    mp.k_update = merge_appends ? k_update : nullptr;
+    mp.v_update = merge_appends ? v_update : nullptr;
+    mp.write_append = (merge_appends && (stages & ARENO_STAGE_APPEND) && !append_in_front) ? 1 : 0;
+    mp.num_blocks = cache->num_blocks;
     mp.trace = g_trace_buffer;
     const size_t slots = static_cast<size_t>(grid.units) + batch;
     const size_t part_bytes = mfma_partial_bytes(slots, q_heads, p.head_dim);
     mp.d.part_ml = static_cast<float*>(workspace);
     mp.d.part_acc = mp.d.part_ml + slots * q_heads * 2;
-    mp.plan = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + part_bytes);
+    mp.dump = mp.d.part_acc + slots * q_heads * p.head_dim;
+    mp.cum_out = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + part_bytes);
     mp.shared_lens = shared_lens;
     mp.shared_ml = nullptr;
     mp.shared_acc = nullptr;
     if (num_shared > 0) {
-      // behind the ungrouped layout: the (longer) plan of the item list, then the shared partial region
-      mp.plan = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + base_need);
+      // behind the ungrouped layout: the (longer) prefix sums of the item list, then the shared partial region
+      mp.cum_out = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + base_need);
       char* region = static_cast<char*>(workspace) + base_need + plan_extra;
       const size_t shared_slots = static_cast<size_t>(grid.units) + num_shared;
       mp.shared_ml = reinterpret_cast<float*>(region);
       mp.shared_acc = mp.shared_ml + shared_slots * cache->kv_heads * 16 * 2;
+    }
+    mp.plan_cum = nullptr;
+    mp.plan_items = nullptr;
+    mp.plan_units = nullptr;
+    if (planned) {
+      const PlanLayout l = plan_layout(plan->items, plan->units);
+      const int32_t* words = static_cast<const int32_t*>(plan->buffer);
+      mp.plan_cum = words + l.cum;
+      mp.plan_items = words + l.items;
+      mp.plan_units = words + l.units;
     }
     if (stages & ARENO_STAGE_SPLIT) {
       hipLaunchKernelGGL(mfma, dim3(grid.workgroups, grid.head_groups), dim3(grid.waves * kWave), 0, s, mp);
@@ -545,14 +776,27 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     return ARENO_OK;
   }
 
+  decode_split_fn fast = nullptr;
+  const bool aligned = (reinterpret_cast<uintptr_t>(cache->k) % 16 == 0) &&
+                       (reinterpret_cast<uintptr_t>(cache->v) % 16 == 0) &&
+                       (reinterpret_cast<uintptr_t>(workspace) % 16 == 0);
+  if (aligned && q_dtype != ARENO_DT_F32) {
+    switch (cache->cache_dtype) {
+      case ARENO_DT_BF16: fast = decode_split_lookup_bf16(p.head_dim, p.group); break;
+      case ARENO_DT_F16: fast = decode_split_lookup_f16(p.head_dim, p.group); break;
+      case ARENO_DT_I8: fast = decode_split_lookup_i8(p.head_dim, p.group); break;
+      case ARENO_DT_FP8_E4M3: fast = decode_split_lookup_fp8(p.head_dim, p.group); break;
+      default: break;
+    }
+  }
   if (!(stages & ARENO_STAGE_SPLIT)) {
     // skip
   } else if (fast != nullptr) {
-    const dim3 grid(ch.max_parts, batch, cache->kv_heads / p.heads_per_wg);
-    hipLaunchKernelGGL(fast, grid, dim3(kDecodeThreads), 0, s, p);
+    const dim3 grid3(ch.max_parts, batch, cache->kv_heads / p.heads_per_wg);
+    hipLaunchKernelGGL(fast, grid3, dim3(kDecodeThreads), 0, s, p);
   } else {
-    const dim3 grid(batch * q_heads, ch.max_parts);
-    hipLaunchKernelGGL(decode_split_generic_kernel, grid, dim3(kWave), 0, s, p);
+    const dim3 grid3(batch * q_heads, ch.max_parts);
+    hipLaunchKernelGGL(decode_split_generic_kernel, grid3, dim3(kWave), 0, s, p);
   }
   if (int rc = check_launch(op)) return rc;
   if (!(stages & ARENO_STAGE_REDUCE)) return ARENO_OK;
@@ -572,13 +816,15 @@ namespace {
 int decode_in_row_ranges(const areno_paged_cache* cache, const void* q, const void* k_update, const void* v_update,
                          void* out, int32_t q_dtype, int32_t batch, int32_t q_heads, const int32_t* block_table,
                          int32_t max_blocks, const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
-                         float softmax_scale, int32_t group_rows, const int32_t* shared_lens, void* workspace,
-                         size_t workspace_bytes, int32_t stages, void* stream) {
+                         float softmax_scale, int32_t group_rows, const int32_t* shared_lens,
+                         const areno_decode_plan* plan, void* workspace, size_t workspace_bytes, int32_t stages,
+                         void* stream) {
   if (batch <= kMfmaMaxBatch || cache == nullptr || q == nullptr || out == nullptr || block_table == nullptr ||
       cache_seqlens == nullptr || q_heads <= 0 || max_blocks <= 0 || cache->kv_heads <= 0 || cache->head_dim <= 0)
     return decode_impl(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
-                       cache_seqlens, window_left, num_splits, softmax_scale, group_rows, shared_lens, workspace,
+                       cache_seqlens, window_left, num_splits, softmax_scale, group_rows, shared_lens, plan, workspace,
                        workspace_bytes, stages, stream);
+  // (a plan covers one launch: areno_hip_paged_decode_plan leaves units = 0 for batches this large)
   int rows_per_launch = kMfmaMaxBatch;
   if (shared_lens != nullptr && group_rows > 1) rows_per_launch = kMfmaMaxBatch / group_rows * group_rows;
   if (rows_per_launch <= 0) rows_per_launch = kMfmaMaxBatch;  // groups wider than a launch: decode_impl drops the hint
@@ -594,7 +840,7 @@ int decode_in_row_ranges(const areno_paged_cache* cache, const void* q, const vo
         v_update != nullptr ? static_cast<const char*>(v_update) + r0 * kv_row : nullptr,
         static_cast<char*>(out) + r0 * q_row, q_dtype, rows, q_heads, block_table + static_cast<size_t>(r0) * max_blocks,
         max_blocks, cache_seqlens + r0, window_left, num_splits, softmax_scale, grouped ? group_rows : 1,
-        grouped ? shared_lens + r0 / group_rows : nullptr, workspace, workspace_bytes, stages, stream);
+        grouped ? shared_lens + r0 / group_rows : nullptr, nullptr, workspace, workspace_bytes, stages, stream);
     if (rc != ARENO_OK) return rc;
   }
   return ARENO_OK;
@@ -610,7 +856,7 @@ extern "C" int areno_hip_paged_decode_stages(const areno_paged_cache* cache, con
                                              float softmax_scale, void* workspace, size_t workspace_bytes,
                                              int32_t stages, void* stream) {
   return areno::decode_in_row_ranges(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
-                            cache_seqlens, window_left, num_splits, softmax_scale, 0, nullptr, workspace,
+                            cache_seqlens, window_left, num_splits, softmax_scale, 0, nullptr, nullptr, workspace,
                             workspace_bytes, stages, stream);
 }
 
@@ -636,8 +882,93 @@ extern "C" int areno_hip_paged_decode_grouped(const areno_paged_cache* cache, co
     return areno::fail(ARENO_ERR_INVALID_ARGUMENT,
                        "areno_hip_paged_decode_grouped: batch %d is not a multiple of group_rows %d", batch, group_rows);
   return areno::decode_in_row_ranges(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
-                            cache_seqlens, window_left, num_splits, softmax_scale, group_rows, shared_lens, workspace,
-                            workspace_bytes, stages, stream);
+                            cache_seqlens, window_left, num_splits, softmax_scale, group_rows, shared_lens, nullptr,
+                            workspace, workspace_bytes, stages, stream);
+}
+
+extern "C" size_t areno_hip_paged_decode_plan_bytes(int32_t batch) {
+  if (batch <= 0) return 0;
+  const size_t items = 2 * static_cast<size_t>(batch < areno::kMfmaMaxBatch ? batch : areno::kMfmaMaxBatch);
+  return areno::plan_layout(items, areno::kMfmaMaxUnits).words * sizeof(int32_t);
+}
+
+extern "C" int areno_hip_paged_decode_plan(areno_decode_plan* plan, void* buffer, size_t buffer_bytes,
+                                           const areno_paged_cache* cache, int32_t q_dtype, int32_t batch,
+                                           int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
+                                           const int32_t* cache_seqlens, int32_t window_left, int32_t with_update,
+                                           int32_t group_rows, const int32_t* shared_lens, void* stream) {
+  using namespace areno;
+  const char* op = "areno_hip_paged_decode_plan";
+  if (plan == nullptr) return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: plan is NULL", op);
+  if (int rc = validate_paged_cache(cache, op)) return rc;
+  if (block_table == nullptr || cache_seqlens == nullptr || batch < 0 || q_heads <= 0 || max_blocks <= 0 ||
+      q_heads % cache->kv_heads != 0)
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: NULL block_table / cache_seqlens or sizes out of range", op);
+  if (shared_lens != nullptr && (group_rows < 1 || (batch > 0 && batch % group_rows != 0)))
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: batch %d is not a multiple of group_rows %d", op, batch, group_rows);
+  const MfmaChoice choice = batch > 0 ? choose_mfma(cache, q_dtype, batch, q_heads, window_left, with_update != 0,
+                                                    group_rows, shared_lens != nullptr)
+                                      : MfmaChoice{};
+  plan->buffer = buffer;
+  plan->buffer_bytes = buffer_bytes;
+  plan->batch = batch;
+  plan->q_heads = q_heads;
+  plan->kv_heads = cache->kv_heads;
+  plan->head_dim = cache->head_dim;
+  plan->block_size = cache->block_size;
+  plan->max_blocks = max_blocks;
+  plan->window_left = window_left;
+  plan->cache_dtype = cache->cache_dtype;
+  plan->q_dtype = q_dtype;
+  plan->with_update = with_update != 0 ? 1 : 0;
+  plan->group_rows = 0;
+  plan->units = 0;
+  plan->items = 0;
+  plan->tile_tokens = 0;
+  if (batch == 0 || choice.fn == nullptr) return ARENO_OK;  // a kernel that takes no plan serves these shapes
+  const PlanLayout l = plan_layout(choice.items.num_items(), choice.grid.units);
+  if (buffer == nullptr || reinterpret_cast<uintptr_t>(buffer) % 16 != 0 || buffer_bytes < l.words * sizeof(int32_t))
+    return fail(ARENO_ERR_WORKSPACE, "%s: a 16-byte aligned buffer of %zu bytes is needed, %zu given", op,
+                l.words * sizeof(int32_t), buffer_bytes);
+  PlanParams pp;
+  pp.cache_seqlens = cache_seqlens;
+  pp.shared_lens = shared_lens;
+  pp.block_table = block_table;
+  int32_t* words = static_cast<int32_t*>(buffer);
+  pp.cum = words + l.cum;
+  pp.items = words + l.items;
+  pp.units = words + l.units;
+  pp.shape = choice.items;
+  pp.num_units = choice.grid.units;
+  pp.bs_shift = log2_exact(cache->block_size);
+  pp.max_blocks = max_blocks;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (choice.items.num_shared > 0) {
+    hipLaunchKernelGGL(decode_plan_kernel<true>, dim3(1), dim3(kPlanThreads), 0, s, pp);
+  } else {
+    hipLaunchKernelGGL(decode_plan_kernel<false>, dim3(1), dim3(kPlanThreads), 0, s, pp);
+  }
+  if (int rc = check_launch(op)) return rc;
+  plan->group_rows = choice.items.num_shared > 0 ? group_rows : 0;
+  plan->units = choice.grid.units;
+  plan->items = choice.items.num_items();
+  plan->tile_tokens = choice.tile_tokens;
+  return ARENO_OK;
+}
+
+extern "C" int areno_hip_paged_decode_planned(const areno_paged_cache* cache, const void* q, const void* k_update,
+                                              const void* v_update, void* out, int32_t q_dtype, int32_t batch,
+                                              int32_t q_heads, const int32_t* block_table, int32_t max_blocks,
+                                              const int32_t* cache_seqlens, int32_t window_left, int32_t num_splits,
+                                              float softmax_scale, int32_t group_rows, const int32_t* shared_lens,
+                                              const areno_decode_plan* plan, void* workspace, size_t workspace_bytes,
+                                              int32_t stages, void* stream) {
+  if (shared_lens != nullptr && (group_rows < 1 || (batch > 0 && batch % group_rows != 0)))
+    return areno::fail(ARENO_ERR_INVALID_ARGUMENT,
+                       "areno_hip_paged_decode_planned: batch %d is not a multiple of group_rows %d", batch, group_rows);
+  return areno::decode_in_row_ranges(cache, q, k_update, v_update, out, q_dtype, batch, q_heads, block_table, max_blocks,
+                            cache_seqlens, window_left, num_splits, softmax_scale, group_rows, shared_lens, plan,
+                            workspace, workspace_bytes, stages, stream);
 }
 
 // ---- the decode op for callers that cannot allocate -----------------------------------------------------------------

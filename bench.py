@@ -185,9 +185,9 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
 
     spread = {}
 
-    # the op folds the append into the split kernel; the stand-alone append launch is timed for reference only
-    us_split = time_stage(cabi.STAGE_APPEND | cabi.STAGE_SPLIT)
-    us_reduce = time_stage(cabi.STAGE_REDUCE)
+    # the op folds the append into the merge launch; the stand-alone append launch is timed for reference only
+    us_split = time_stage(cabi.STAGE_SPLIT)
+    us_reduce = time_stage(cabi.STAGE_APPEND | cabi.STAGE_REDUCE)
     us_append = time_stage(cabi.STAGE_APPEND)
     torch.cuda.synchronize()
     assert torch.equal(out2, out), "C-ABI staged run disagrees with the op"
@@ -199,9 +199,9 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
         "workload": w.name,
         "us_per_step": us_graph,
         "us_per_step_eager": us_eager,
-        "kernel_us": {"split_with_append": us_split, "reduce": us_reduce, "append_alone_not_in_op": us_append},
+        "kernel_us": {"split": us_split, "merge_with_append": us_reduce, "append_alone_not_in_op": us_append},
         # 10th / 90th percentile of the split kernel's samples (each the mean of back-to-back launches)
-        "split_us_p10_p90": list(spread[cabi.STAGE_APPEND | cabi.STAGE_SPLIT]),
+        "split_us_p10_p90": list(spread[cabi.STAGE_SPLIT]),
         "tokens_per_s": w.q.shape[0] / (us_graph * 1e-6),
         "algorithmic_bytes": alg_bytes,
         "op_gbps": alg_bytes / (us_graph * 1e-6) / 1e9,
@@ -448,7 +448,7 @@ def wave_trace(w, launches=12):
     for it in range(launches):
         buf.zero_()
         cabi.paged_decode(cabi.describe_cache(*pools[it % len(pools)]), w.q, w.k_update, w.v_update, out, w.block_table,
-                          w.cache_seqlens, workspace, softmax_scale=w.softmax_scale, stages=cabi.STAGE_APPEND | cabi.STAGE_SPLIT)  # fmt: skip
+                          w.cache_seqlens, workspace, softmax_scale=w.softmax_scale, stages=cabi.STAGE_SPLIT)  # fmt: skip
         torch.cuda.synchronize()
         runs.append(buf.cpu().view(-1, 8).numpy().copy())
     lib.areno_hip_debug_set_trace(None)

@@ -167,6 +167,52 @@ int areno_hip_paged_decode_grouped(const areno_paged_cache* cache, const void* q
                                    int32_t stages, void* stream);
 
 /*
+ * A per-step plan for the decode op.  block_table and cache_seqlens are the same for every layer of a decode step (the
+ * reference builds one InferMeta per step and all layers reuse it: areno/engine/inference.py:935,
+ * areno/engine/runtime/decode_graph.py:96,140-178), so the work list the split kernel derives from them -- the item
+ * table, the prefix sums of the items' 16-token quanta, where every wave's share starts and the block ids of its
+ * first tile -- can be built once per step instead of once per layer.  No counterpart in the reference, whose split
+ * kernel uses a fixed chunk per thread block (areno/accel/csrc/attention.cu:588-594).
+ *   areno_hip_paged_decode_plan_bytes(batch)   bytes of device memory a plan for `batch` rows needs at most
+ *   areno_hip_paged_decode_plan(...)           one small launch on `stream` that fills `buffer` (16-byte aligned, the
+ *                                              caller's) and describes it in *plan (host memory, the caller's); legal
+ *                                              inside stream capture.  `cache` gives the pool geometry and dtypes (its
+ *                                              pointers only have to be aligned like the pools the decode calls will
+ *                                              pass); with_update = the decode calls will pass k_update / v_update;
+ *                                              group_rows / shared_lens as in areno_hip_paged_decode_grouped (0 / NULL:
+ *                                              no prefix groups).
+ *   areno_hip_paged_decode_planned(...)        areno_hip_paged_decode_grouped with the plan; plan = NULL or a plan with
+ *                                              units == 0 (shapes that a kernel without a work list serves) is exactly
+ *                                              that call.  Every argument the plan was built from must be the same
+ *                                              (shapes and dtypes are checked: ARENO_ERR_INVALID_ARGUMENT; the contents
+ *                                              of block_table, cache_seqlens and shared_lens at the time of the plan
+ *                                              launch must still be what the decode call sees).  Same results, bit for
+ *                                              bit, as the call without a plan.
+ * A plan may be reused by any number of decode calls (the layers of a step) and is rebuilt when the tables change.
+ */
+typedef struct areno_decode_plan {
+  void* buffer; /* device memory the plan's tables live in */
+  size_t buffer_bytes;
+  int32_t batch, q_heads, kv_heads, head_dim, block_size, max_blocks, window_left;
+  int32_t cache_dtype, q_dtype, with_update, group_rows;
+  int32_t units;       /* waves that share the work; 0: the shapes take a kernel that uses no plan */
+  int32_t items;       /* entries of the item list */
+  int32_t tile_tokens; /* tokens per tile step of the kernel the plan is for */
+} areno_decode_plan;
+size_t areno_hip_paged_decode_plan_bytes(int32_t batch);
+int areno_hip_paged_decode_plan(areno_decode_plan* plan, void* buffer, size_t buffer_bytes,
+                                const areno_paged_cache* cache, int32_t q_dtype, int32_t batch, int32_t q_heads,
+                                const int32_t* block_table, int32_t max_blocks, const int32_t* cache_seqlens,
+                                int32_t window_left, int32_t with_update, int32_t group_rows,
+                                const int32_t* shared_lens, void* stream);
+int areno_hip_paged_decode_planned(const areno_paged_cache* cache, const void* q, const void* k_update,
+                                   const void* v_update, void* out, int32_t q_dtype, int32_t batch, int32_t q_heads,
+                                   const int32_t* block_table, int32_t max_blocks, const int32_t* cache_seqlens,
+                                   int32_t window_left, int32_t num_splits, float softmax_scale, int32_t group_rows,
+                                   const int32_t* shared_lens, const areno_decode_plan* plan, void* workspace,
+                                   size_t workspace_bytes, int32_t stages, void* stream);
+
+/*
  * Packed causal self-attention over new tokens only, GQA without expanding KV:
  * areno_varlen_causal_attention_forward_cuda (areno/accel/csrc/attention.cu:813-861; pybind name
  * areno_varlen_causal_attention_forward, extension.cpp:182).  Token t of the sequence starting at

@@ -1,7 +1,7 @@
 """Every unit of the matrix-core decode kernel's work list, walked on the CPU through the kernel's own item and cursor
 functions (``areno_amd/csrc/decode_items.hpp`` compiled by g++ into ``tests/native/decode_walk.cpp``) with accessors
-that check each index before use: length-array and prefix-sum indices, block-table columns, cached positions, partial
-slots, and that the units cover every tile exactly once.  Workloads: the benchmark configurations at full size and the
+that check each index before use: item-table and prefix-sum indices, block-table columns, cached positions, partial
+slots, and that the units read every cached token exactly once, in tile steps of 32 and of 64 tokens.  Workloads: the benchmark configurations at full size and the
 shapes of the GPU parity tests that exercise prefix groups (32 / 8 heads x 8 samples, 400 groups of 3, overstated and
 zero shared lengths), windows, empty rows and the largest batch."""
 
@@ -24,52 +24,56 @@ def walker():
     subprocess.run(["g++", "-O1", "-std=c++17", "-shared", "-fPIC", "-Wall", "-Werror", "-o", out,
                     os.path.join(ROOT, "tests", "native", "decode_walk.cpp")], check=True)  # fmt: skip
     lib = ctypes.CDLL(out)
-    lib.decode_walk.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p] + [ctypes.c_int] * 7 + [
-        ctypes.POINTER(ctypes.c_longlong), ctypes.POINTER(ctypes.c_longlong), ctypes.c_char_p, ctypes.c_int]  # fmt: skip
+    lib.decode_walk.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p] + [ctypes.c_int] * 9 + [
+        ctypes.POINTER(ctypes.c_longlong)] * 3 + [ctypes.c_char_p, ctypes.c_int]  # fmt: skip
 
-    def walk(lengths, *, q_per_kv, units, shared=None, group_rows=1, window_left=-1, new_token_tile=1, block_size=16,
-             max_blocks=None):  # fmt: skip
+    def walk(lengths, *, q_per_kv, units, shared=None, group_rows=1, window_left=-1, append_in_merge=1, tile_tokens=32,
+             block_size=16, max_blocks=None, switch_quanta=3):  # fmt: skip
         lens = torch.as_tensor(lengths, dtype=torch.int32).contiguous()
         sh = None if shared is None else torch.as_tensor(shared, dtype=torch.int32).contiguous()
         if max_blocks is None:
             max_blocks = int(lens.max()) // block_size + 1
-        tiles, partials = ctypes.c_longlong(0), ctypes.c_longlong(0)
+        quanta, partials, steps = ctypes.c_longlong(0), ctypes.c_longlong(0), ctypes.c_longlong(0)
         msg = ctypes.create_string_buffer(256)
         rc = lib.decode_walk(lens.data_ptr(), lens.numel(), None if sh is None else sh.data_ptr(), group_rows, q_per_kv,
-                             window_left, new_token_tile, units, block_size, max_blocks, ctypes.byref(tiles),
-                             ctypes.byref(partials), msg, 256)  # fmt: skip
+                             window_left, append_in_merge, switch_quanta, units, tile_tokens, block_size, max_blocks,
+                             ctypes.byref(quanta), ctypes.byref(partials), ctypes.byref(steps), msg, 256)  # fmt: skip
         assert rc == 0, msg.value.decode()
-        return tiles.value, partials.value
+        return quanta.value, partials.value, steps.value
 
     return walk
 
 
-def _expected_tiles(lengths, new_token_tile, window_left=-1):
+def _expected_quanta(lengths, append_in_merge, window_left=-1):
     total = 0
     for n in [int(x) for x in lengths]:
         lo = 0 if window_left < 0 else max(0, n - window_left)
-        total += -(-(n + 1 - new_token_tile - lo) // 32) + new_token_tile
+        total += max(0, -(-(n + 1 - append_in_merge - lo) // 16))
     return total
 
 
-@pytest.mark.parametrize("new_token_tile", [0, 1])
-def test_cfg1_cfg2_units(walker, new_token_tile):
+@pytest.mark.parametrize("append_in_merge", [0, 1])
+@pytest.mark.parametrize("tile_tokens", [32, 64])
+def test_cfg1_cfg2_units(walker, append_in_merge, tile_tokens):
     g = workloads._gen(1002 + 1)
     lengths = workloads._randint(g, 512, 4096, 64)
-    tiles, partials = walker(lengths, q_per_kv=7, units=512, new_token_tile=new_token_tile)
-    assert tiles == _expected_tiles(lengths, new_token_tile)
-    assert 512 <= partials <= 512 + 64 * (1 + new_token_tile)
+    quanta, partials, steps = walker(lengths, q_per_kv=7, units=256, append_in_merge=append_in_merge, tile_tokens=tile_tokens)
+    assert quanta == _expected_quanta(lengths, append_in_merge)
+    assert 256 <= partials <= 256 + 64
+    # a unit's steps: its quanta in whole tiles, one more per segment border
+    per_tile = tile_tokens // 16
+    assert steps <= quanta // per_tile + 256 + 64 + 64
 
 
-@pytest.mark.parametrize("new_token_tile", [0, 1])
-def test_cfg3_full_size_with_and_without_groups(walker, new_token_tile):
+@pytest.mark.parametrize("append_in_merge", [0, 1])
+def test_cfg3_full_size_with_and_without_groups(walker, append_in_merge):
     prefix, lengths = workloads.cfg3_lengths()
     shared = (prefix // 16) * 16
-    plain, _ = walker(lengths, q_per_kv=4, units=512, new_token_tile=new_token_tile)
-    grouped, _ = walker(lengths, q_per_kv=4, units=512, shared=shared, group_rows=8, new_token_tile=new_token_tile)
-    assert plain == _expected_tiles(lengths, new_token_tile)
-    # a prompt's shared tiles are read once per sub-group of 4 rows instead of once per row
-    saved = sum(int(s) // 32 * (8 - 2) for s in shared)
+    plain, _, _ = walker(lengths, q_per_kv=4, units=512, append_in_merge=append_in_merge)
+    grouped, _, _ = walker(lengths, q_per_kv=4, units=512, shared=shared, group_rows=8, append_in_merge=append_in_merge)
+    assert plain == _expected_quanta(lengths, append_in_merge)
+    # a prompt's shared tokens (cut to whole 32-token tiles) are read once per sub-group of 4 rows instead of once per row
+    saved = sum(int(s) // 32 * 2 * (8 - 2) for s in shared)
     assert grouped == plain - saved
 
 
@@ -79,7 +83,7 @@ def test_reduced_rollouts_of_the_gpu_tests(walker, hq, hkv, samples, units):
     prefix, lengths = workloads.cfg3_lengths(77, 6, samples, 8, 700, 120.0, 1.0, 900)
     shared = (prefix // 16) * 16
     walker(lengths, q_per_kv=hq // hkv, units=units, shared=shared, group_rows=samples)
-    walker(lengths, q_per_kv=hq // hkv, units=units, shared=shared, group_rows=samples, new_token_tile=0)
+    walker(lengths, q_per_kv=hq // hkv, units=units, shared=shared, group_rows=samples, append_in_merge=0, tile_tokens=32)
 
 
 def test_groups_of_three_at_the_largest_launch(walker):
@@ -100,12 +104,29 @@ def test_overstated_and_zero_shared_lengths(walker):
 
 
 @pytest.mark.parametrize("window_left", [-1, 0, 40, 5000])
-@pytest.mark.parametrize("new_token_tile", [0, 1])
-def test_windows_empty_rows_and_page_borders(walker, window_left, new_token_tile):
-    lengths = [0, 15, 16, 17, 31, 32, 33, 300, 0, 1, 4095]
-    tiles, _ = walker(lengths, q_per_kv=4, units=2048, window_left=window_left, new_token_tile=new_token_tile)
-    assert tiles == _expected_tiles(lengths, new_token_tile, window_left)
-    walker(lengths, q_per_kv=1, units=512, window_left=window_left, new_token_tile=new_token_tile, block_size=48)
+@pytest.mark.parametrize("append_in_merge", [0, 1])
+@pytest.mark.parametrize("tile_tokens,switch_quanta", [(32, 3), (64, 3), (32, 0), (32, 1), (32, 7)])
+def test_windows_empty_rows_and_page_borders(walker, window_left, append_in_merge, tile_tokens, switch_quanta):
+    lengths = [0, 15, 16, 17, 31, 32, 33, 300, 0, 1, 4095, 0]
+    kw = dict(window_left=window_left, append_in_merge=append_in_merge, tile_tokens=tile_tokens, switch_quanta=switch_quanta)
+    quanta, _, _ = walker(lengths, q_per_kv=4, units=2048, **kw)
+    assert quanta == _expected_quanta(lengths, append_in_merge, window_left)
+    walker(lengths, q_per_kv=1, units=512, block_size=48, **kw)
+    walker(lengths, q_per_kv=1, units=3, **kw)
+    walker(lengths, q_per_kv=1, units=40, **kw)  # units of a few positions: some hold nothing but switch positions
+
+
+def test_rows_at_the_end_of_their_block_table(walker):
+    """A row whose next position has no column left (length = max_blocks * block_size): with the append folded into the
+    merge launch the streaming waves read columns below max_blocks only."""
+    walker([64, 32, 64], q_per_kv=4, units=64, block_size=16, max_blocks=4, append_in_merge=1)
+    with pytest.raises(AssertionError, match="columns"):
+        walker([64, 32, 64], q_per_kv=4, units=64, block_size=16, max_blocks=4, append_in_merge=0)
+
+
+def test_batches_of_empty_rows(walker):
+    assert walker([0, 0, 0], q_per_kv=4, units=1024)[0] == 0
+    assert walker([0, 0, 5, 0], q_per_kv=4, units=1024)[0] == 1
 
 
 def test_full_item_list(walker):
