@@ -54,9 +54,10 @@ def test_version_status_strings_and_workspace_size(lib):
     ws.restype = ctypes.c_size_t
     ws.argtypes = [ctypes.c_int32] * 6
     # two layouts share the workspace: fixed chunks (B * Hq * chunks rows) and the balanced-piece layout
-    # ((256 workgroups * 4 waves + B) * Hq rows plus the B + 1 prefix sums); the size is the larger of the two
+    # ((256 workgroups * 4 waves + B) * Hq rows, the dump row of the lanes that own no partial -- 16 columns of the widest
+    # head and an (m, l) pair per lane -- plus the B + 1 prefix sums); the size is the larger of the two
     def pieces(b, hq, d):
-        rows = (1024 + b) * hq * (d + 2) * 4
+        rows = ((1024 + b) * hq * (d + 2) + 16 * 512 + 2 * 64) * 4
         return (rows + 255) // 256 * 256 + (b + 1 + 63) // 64 * 64 * 4
 
     # B=64, Hq=28, D=128, bs=16, MB=257: 4112 tokens -> 17 chunks of 256
