@@ -1,14 +1,15 @@
 """Paged / quantized KV-cache attention ops (the hot path of ``areno.accel`` in the reference).
 
 Re-exports the op surface the reference's inference backend imports
-(``areno/accel/__init__.py:17-21`` there) plus this build's additions (cache write, paged prefill, and the fused
-QK-norm + rotary + cache-write step in front of the path).
+(``areno/accel/__init__.py:17-21`` there) plus this build's additions (cache write, paged prefill, the fused
+QK-norm + rotary + cache-write step in front of the path, and the per-step plan of the decode op).
 """
 
 from areno_amd.accel.attention import (
     areno_causal_attention,
     areno_paged_cache_write,
     areno_paged_causal_attention_decode,
+    areno_paged_decode_plan,
     areno_paged_varlen_causal_attention,
     areno_qk_norm_rope_cache_write,
     areno_varlen_causal_attention,
@@ -18,6 +19,7 @@ __all__ = [
     "areno_causal_attention",
     "areno_paged_cache_write",
     "areno_paged_causal_attention_decode",
+    "areno_paged_decode_plan",
     "areno_paged_varlen_causal_attention",
     "areno_qk_norm_rope_cache_write",
     "areno_varlen_causal_attention",

@@ -197,6 +197,56 @@ class _CausalAttention(torch.autograd.Function):
         return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None
 
 
+_PLAN_DTYPE_CODES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+@torch._dynamo.disable
+def areno_paged_decode_plan(
+    block_table: torch.Tensor,
+    cache_seqlens: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    *,
+    q_heads: int,
+    q_dtype: torch.dtype = torch.bfloat16,
+    window_left: int | None = None,
+    with_update: bool = True,
+    k_scale: torch.Tensor | None = None,
+    v_scale: torch.Tensor | None = None,
+    prefix_group_rows: int | None = None,
+    shared_prefix_lens: torch.Tensor | None = None,
+    buffer: torch.Tensor | None = None,
+):
+    """Build the work list of one decode step once, for all layers of the step.
+
+    ``block_table`` and ``cache_seqlens`` are the same for every layer of a decode step (the reference builds one
+    ``InferMeta`` per step, ``areno/engine/inference.py:935`` there), so what the decode kernel derives from them --
+    which wave reads which tokens, where it starts and the block ids of its first tile -- is computed by one small
+    launch here and handed to every layer's :func:`areno_paged_causal_attention_decode` call as ``plan=``.  The caches
+    are any layer's (their shape, dtype and alignment are what matters); ``with_update`` says whether those calls pass
+    update rows.  ``buffer`` (optional uint8 CUDA tensor) makes the plan reuse caller memory, e.g. inside a captured
+    graph that rebuilds the plan from static tables on every replay.  Legal inside stream capture.
+    """
+    op = "areno_paged_decode_plan"
+    if not _all_on_gpu(block_table, cache_seqlens, k_cache, v_cache, k_scale, v_scale, shared_prefix_lens, buffer):
+        raise RuntimeError(f"{op} requires CUDA tensors")
+    if block_table.dim() != 2 or cache_seqlens.dim() != 1:
+        raise ValueError(f"{op} expects block_table 2D and cache_seqlens 1D")
+    if block_table.dtype != torch.int32 or cache_seqlens.dtype != torch.int32:
+        raise ValueError(f"{op} expects int32 block_table and cache_seqlens")
+    if q_dtype not in _PLAN_DTYPE_CODES:
+        raise ValueError(f"{op} expects q_dtype float32, float16 or bfloat16")
+    if (prefix_group_rows is None) != (shared_prefix_lens is None):
+        raise ValueError(f"{op} expects prefix_group_rows and shared_prefix_lens together")
+    _check_scales(op, k_cache, k_scale, v_scale)
+    return _extension().areno_paged_decode_plan(
+        block_table.contiguous(), cache_seqlens.contiguous(), k_cache, v_cache, k_scale, v_scale,
+        _PLAN_DTYPE_CODES[q_dtype], int(q_heads), _window_left(window_left), bool(with_update),
+        0 if prefix_group_rows is None else int(prefix_group_rows),
+        None if shared_prefix_lens is None else shared_prefix_lens.contiguous(), buffer,
+    )  # fmt: skip
+
+
 @torch._dynamo.disable
 def areno_paged_causal_attention_decode(
     q: torch.Tensor,
@@ -214,6 +264,7 @@ def areno_paged_causal_attention_decode(
     v_scale: torch.Tensor | None = None,
     prefix_group_rows: int | None = None,
     shared_prefix_lens: torch.Tensor | None = None,
+    plan=None,
 ) -> torch.Tensor:
     """Apply single-token paged-cache causal attention to ``(batch, heads, dim)`` Q.
 
@@ -226,6 +277,10 @@ def areno_paged_causal_attention_decode(
     ``[i * prefix_group_rows, (i + 1) * prefix_group_rows)`` list the same block ids for their first
     ``shared_prefix_lens[i]`` tokens (the samples of one prompt in a rollout); those pages are then read once for
     several rows instead of once per row.  The result is the same.
+
+    ``plan`` (optional): what :func:`areno_paged_decode_plan` built from the same ``block_table``, ``cache_seqlens``,
+    window and prefix groups.  The tables are the same for every layer of a decode step, so one plan serves all of
+    them; the result is bit-identical to the call without a plan.
     """
     op = "areno_paged_causal_attention_decode"
     if not _all_on_gpu(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, k_scale, v_scale):
@@ -262,6 +317,13 @@ def areno_paged_causal_attention_decode(
         if shared_prefix_lens.dtype != torch.int32 or shared_prefix_lens.shape != (q.shape[0] // int(prefix_group_rows),):
             raise ValueError(f"{op} expects int32 shared_prefix_lens shaped (batch / prefix_group_rows,)")
         groups = (int(prefix_group_rows), shared_prefix_lens.contiguous())
+    else:
+        groups = (0, None)
+    if plan is not None:
+
+        def call():
+            return ext.areno_paged_causal_attention_decode_forward_planned(*args, k_scale, v_scale, *groups, plan)
+    elif shared_prefix_lens is not None:
 
         def call():
             return ext.areno_paged_causal_attention_decode_forward_scaled(*args, k_scale, v_scale, *groups)

@@ -43,6 +43,16 @@ class PagedCache(ctypes.Structure):
     ]
 
 
+class DecodePlan(ctypes.Structure):
+    """``struct areno_decode_plan``."""
+
+    _fields_ = [("buffer", ctypes.c_void_p), ("buffer_bytes", ctypes.c_size_t)] + [
+        (name, ctypes.c_int32)
+        for name in ("batch", "q_heads", "kv_heads", "head_dim", "block_size", "max_blocks", "window_left", "cache_dtype",
+                     "q_dtype", "with_update", "group_rows", "units", "items", "tile_tokens")
+    ]  # fmt: skip
+
+
 class BlockTables(ctypes.Structure):
     """``struct areno_block_tables``."""
 
@@ -88,6 +98,10 @@ def lib() -> ctypes.CDLL:
         handle.areno_hip_paged_decode_grouped.argtypes = decode_args[:-2] + [_I32, _P, _P, _SZ, _I32, _P]
         handle.areno_hip_paged_decode_grouped_workspace_bytes.restype = _SZ
         handle.areno_hip_paged_decode_grouped_workspace_bytes.argtypes = [_I32] * 8
+        handle.areno_hip_paged_decode_plan_bytes.restype = _SZ
+        handle.areno_hip_paged_decode_plan_bytes.argtypes = [_I32]
+        handle.areno_hip_paged_decode_plan.argtypes = [_P, _P, _SZ, _P, _I32, _I32, _I32, _P, _I32, _P, _I32, _I32, _I32, _P, _P]
+        handle.areno_hip_paged_decode_planned.argtypes = decode_args[:-2] + [_I32, _P, _P, _P, _SZ, _I32, _P]
         handle.areno_hip_varlen_attention.argtypes = [_P, _P, _P, _P, _I32, _I64, _I32, _I32, _I32, _P, _I32, _I32, _F, _P, _SZ, _P]  # fmt: skip
         handle.areno_hip_paged_varlen_prefill.argtypes = [_P, _P, _P, _I32, _I64, _I32, _I32, _P, _I32, _P, _P, _I32, _F, _P, _SZ, _P]  # fmt: skip
         handle.areno_hip_prefill_workspace_bytes.restype = _SZ
@@ -140,12 +154,41 @@ def decode_grouped_workspace_bytes(batch, q_heads, kv_heads, head_dim, block_siz
                                                                     max_blocks, num_splits, group_rows))  # fmt: skip
 
 
+def decode_plan_bytes(batch: int) -> int:
+    return int(lib().areno_hip_paged_decode_plan_bytes(int(batch)))
+
+
+def paged_decode_plan(cache: PagedCache, q_dtype: torch.dtype, q_heads: int, block_table, cache_seqlens, buffer, *,
+                      window_left=-1, with_update=True, group_rows=None, shared_lens=None, stream=None) -> DecodePlan:  # fmt: skip
+    """``areno_hip_paged_decode_plan`` on raw pointers: fills ``buffer`` (a uint8 device tensor of at least
+    ``decode_plan_bytes(batch)`` bytes, which must outlive the plan) and returns the host-side description."""
+    plan = DecodePlan()
+    check(lib().areno_hip_paged_decode_plan(
+        ctypes.byref(plan), buffer.data_ptr(), buffer.numel(), ctypes.byref(cache), _DTYPE_CODES[q_dtype],
+        block_table.shape[0], int(q_heads), block_table.data_ptr(), block_table.shape[1], cache_seqlens.data_ptr(),
+        int(window_left), 1 if with_update else 0, 0 if shared_lens is None else int(group_rows),
+        None if shared_lens is None else shared_lens.data_ptr(), current_stream_ptr() if stream is None else stream,
+    ), "areno_hip_paged_decode_plan")  # fmt: skip
+    return plan
+
+
 def paged_decode(cache: PagedCache, q, k_update, v_update, out, block_table, cache_seqlens, workspace, *,
                  window_left=-1, num_splits=8, softmax_scale=None, stages=STAGE_ALL, stream=None,
-                 group_rows=None, shared_lens=None) -> None:  # fmt: skip
-    """``areno_hip_paged_decode_stages`` (or ``_grouped`` when ``shared_lens`` is given) on raw pointers;
-    ``workspace`` is a uint8 device tensor."""
+                 group_rows=None, shared_lens=None, plan: DecodePlan | None = None) -> None:  # fmt: skip
+    """``areno_hip_paged_decode_stages`` (``_grouped`` when ``shared_lens`` is given, ``_planned`` with a plan) on raw
+    pointers; ``workspace`` is a uint8 device tensor."""
     scale = float(softmax_scale if softmax_scale is not None else q.shape[-1] ** -0.5)
+    if plan is not None:
+        status = lib().areno_hip_paged_decode_planned(
+            ctypes.byref(cache), q.data_ptr(), None if k_update is None else k_update.data_ptr(),
+            None if v_update is None else v_update.data_ptr(), out.data_ptr(), dtype_code(q), q.shape[0], q.shape[1],
+            block_table.data_ptr(), block_table.shape[1], cache_seqlens.data_ptr(), int(window_left), int(num_splits),
+            scale, 0 if shared_lens is None else int(group_rows), None if shared_lens is None else shared_lens.data_ptr(),
+            ctypes.byref(plan), workspace.data_ptr(), workspace.numel(), int(stages),
+            current_stream_ptr() if stream is None else stream,
+        )  # fmt: skip
+        check(status, "areno_hip_paged_decode_planned")
+        return
     if shared_lens is not None:
         status = lib().areno_hip_paged_decode_grouped(
             ctypes.byref(cache), q.data_ptr(), None if k_update is None else k_update.data_ptr(),

@@ -87,7 +87,8 @@ at::Tensor paged_decode_forward_impl(at::Tensor q, at::Tensor k_update, at::Tens
                                      at::Tensor v_cache, at::Tensor block_table, at::Tensor cache_seqlens,
                                      int64_t window_left, int64_t num_splits, double softmax_scale,
                                      c10::optional<at::Tensor> k_scale, c10::optional<at::Tensor> v_scale,
-                                     int64_t prefix_group_rows, c10::optional<at::Tensor> shared_prefix_lens) {
+                                     int64_t prefix_group_rows, c10::optional<at::Tensor> shared_prefix_lens,
+                                     const areno_decode_plan* plan) {
   const char* op = "areno_paged_causal_attention_decode";
   TORCH_CHECK(q.is_cuda(), op, " q must be CUDA");
   TORCH_CHECK(k_update.is_cuda(), op, " k_update must be CUDA");
@@ -144,14 +145,93 @@ at::Tensor paged_decode_forward_impl(at::Tensor q, at::Tensor k_update, at::Tens
       cache.block_size, static_cast<int32_t>(block_table.size(1)), static_cast<int32_t>(num_splits), group_rows);
   TORCH_CHECK(ws_bytes > 0, op, " invalid shapes for the split-KV workspace");
   auto workspace = at::empty({static_cast<int64_t>(ws_bytes)}, q.options().dtype(at::kByte));
-  const int status = areno_hip_paged_decode_grouped(
+  const int status = areno_hip_paged_decode_planned(
       &cache, q.data_ptr(), k_update.data_ptr(), v_update.data_ptr(), out.data_ptr(), dtype_code(q, op, "q"),
       static_cast<int32_t>(q.size(0)), static_cast<int32_t>(q.size(1)), block_table.data_ptr<int32_t>(),
       static_cast<int32_t>(block_table.size(1)), cache_seqlens.data_ptr<int32_t>(), static_cast<int32_t>(window_left),
-      static_cast<int32_t>(num_splits), static_cast<float>(softmax_scale), group_rows, shared_ptr,
+      static_cast<int32_t>(num_splits), static_cast<float>(softmax_scale), group_rows, shared_ptr, plan,
       workspace.data_ptr(), ws_bytes, ARENO_STAGE_ALL, current_stream(q));
   check_status(status, op);
   return out;
+}
+
+at::Tensor paged_decode_forward_scaled(at::Tensor q, at::Tensor k_update, at::Tensor v_update, at::Tensor k_cache,
+                                       at::Tensor v_cache, at::Tensor block_table, at::Tensor cache_seqlens,
+                                       int64_t window_left, int64_t num_splits, double softmax_scale,
+                                       c10::optional<at::Tensor> k_scale, c10::optional<at::Tensor> v_scale,
+                                       int64_t prefix_group_rows, c10::optional<at::Tensor> shared_prefix_lens) {
+  return paged_decode_forward_impl(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, window_left,
+                                   num_splits, softmax_scale, k_scale, v_scale, prefix_group_rows, shared_prefix_lens,
+                                   nullptr);
+}
+
+// A per-step plan of the decode op (areno_hip_paged_decode_plan): the host-side description and the device buffer it
+// points into, kept alive together.
+struct DecodePlan {
+  areno_decode_plan plan;
+  at::Tensor buffer;
+};
+
+std::shared_ptr<DecodePlan> paged_decode_plan(at::Tensor block_table, at::Tensor cache_seqlens, at::Tensor k_cache,
+                                              at::Tensor v_cache, c10::optional<at::Tensor> k_scale,
+                                              c10::optional<at::Tensor> v_scale, int64_t q_dtype_code, int64_t q_heads,
+                                              int64_t window_left, bool with_update, int64_t prefix_group_rows,
+                                              c10::optional<at::Tensor> shared_prefix_lens,
+                                              c10::optional<at::Tensor> buffer) {
+  const char* op = "areno_paged_decode_plan";
+  TORCH_CHECK(block_table.is_cuda() && cache_seqlens.is_cuda(), op, " block_table and cache_seqlens must be CUDA");
+  TORCH_CHECK(block_table.is_contiguous() && cache_seqlens.is_contiguous(), op, " tensors must be contiguous");
+  TORCH_CHECK(block_table.dim() == 2 && cache_seqlens.dim() == 1, op, " expects block_table 2D and cache_seqlens 1D");
+  TORCH_CHECK(block_table.scalar_type() == at::kInt && cache_seqlens.scalar_type() == at::kInt, op,
+              " block_table and cache_seqlens must be int32");
+  TORCH_CHECK(block_table.size(0) == cache_seqlens.size(0), op, " batch mismatch");
+  TORCH_CHECK(q_dtype_code == ARENO_DT_F16 || q_dtype_code == ARENO_DT_BF16 || q_dtype_code == ARENO_DT_F32, op,
+              " q dtype must be fp16, bf16 or fp32");
+  const areno_paged_cache cache = describe_cache(k_cache, v_cache, k_scale, v_scale, op);
+  TORCH_CHECK(q_heads > 0 && q_heads % cache.kv_heads == 0, op, " q heads must be divisible by kv heads");
+  const int32_t batch = static_cast<int32_t>(block_table.size(0));
+  const int32_t* shared_ptr = nullptr;
+  int32_t group_rows = 0;
+  if (shared_prefix_lens.has_value()) {
+    const at::Tensor& sl = *shared_prefix_lens;
+    TORCH_CHECK(prefix_group_rows >= 1 && batch % prefix_group_rows == 0, op,
+                " batch must be a multiple of prefix_group_rows");
+    TORCH_CHECK(sl.is_cuda() && sl.is_contiguous() && sl.scalar_type() == at::kInt && sl.dim() == 1 &&
+                    sl.size(0) == batch / prefix_group_rows,
+                op, " shared_prefix_lens must be a CUDA int32 (batch / prefix_group_rows,) tensor");
+    shared_ptr = sl.data_ptr<int32_t>();
+    group_rows = static_cast<int32_t>(prefix_group_rows);
+  }
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(block_table));
+  auto holder = std::make_shared<DecodePlan>();
+  const size_t bytes = areno_hip_paged_decode_plan_bytes(batch > 0 ? batch : 1);
+  if (buffer.has_value()) {
+    TORCH_CHECK(buffer->is_cuda() && buffer->is_contiguous() && buffer->scalar_type() == at::kByte &&
+                    static_cast<size_t>(buffer->numel()) >= bytes,
+                op, " buffer must be a contiguous CUDA uint8 tensor of at least ", bytes, " bytes");
+    holder->buffer = *buffer;
+  } else {
+    holder->buffer = at::empty({static_cast<int64_t>(bytes)}, block_table.options().dtype(at::kByte));
+  }
+  const int status = areno_hip_paged_decode_plan(
+      &holder->plan, holder->buffer.data_ptr(), static_cast<size_t>(holder->buffer.numel()), &cache,
+      static_cast<int32_t>(q_dtype_code), batch, static_cast<int32_t>(q_heads), block_table.data_ptr<int32_t>(),
+      static_cast<int32_t>(block_table.size(1)), cache_seqlens.data_ptr<int32_t>(), static_cast<int32_t>(window_left),
+      with_update ? 1 : 0, group_rows, shared_ptr, current_stream(block_table));
+  check_status(status, op);
+  return holder;
+}
+
+at::Tensor paged_decode_forward_planned(at::Tensor q, at::Tensor k_update, at::Tensor v_update, at::Tensor k_cache,
+                                        at::Tensor v_cache, at::Tensor block_table, at::Tensor cache_seqlens,
+                                        int64_t window_left, int64_t num_splits, double softmax_scale,
+                                        c10::optional<at::Tensor> k_scale, c10::optional<at::Tensor> v_scale,
+                                        int64_t prefix_group_rows, c10::optional<at::Tensor> shared_prefix_lens,
+                                        std::shared_ptr<DecodePlan> plan) {
+  TORCH_CHECK(plan != nullptr, "areno_paged_causal_attention_decode: plan is None");
+  return paged_decode_forward_impl(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, window_left,
+                                   num_splits, softmax_scale, k_scale, v_scale, prefix_group_rows, shared_prefix_lens,
+                                   &plan->plan);
 }
 
 // Reference signature (extension.cpp:184 in the reference).
@@ -159,7 +239,7 @@ at::Tensor paged_decode_forward(at::Tensor q, at::Tensor k_update, at::Tensor v_
                                 at::Tensor v_cache, at::Tensor block_table, at::Tensor cache_seqlens,
                                 int64_t window_left, int64_t num_splits, double softmax_scale) {
   return paged_decode_forward_impl(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, window_left,
-                                   num_splits, softmax_scale, c10::nullopt, c10::nullopt, 0, c10::nullopt);
+                                   num_splits, softmax_scale, c10::nullopt, c10::nullopt, 0, c10::nullopt, nullptr);
 }
 
 at::Tensor varlen_forward(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor cu_seqlens, int64_t window_left,
@@ -507,8 +587,16 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("areno_paged_causal_attention_decode_forward", &paged_decode_forward,
         "ARENO paged causal attention decode forward");
   m.def("areno_varlen_causal_attention_forward", &varlen_forward, "ARENO varlen causal attention forward");
-  m.def("areno_paged_causal_attention_decode_forward_scaled", &paged_decode_forward_impl,
+  m.def("areno_paged_causal_attention_decode_forward_scaled", &paged_decode_forward_scaled,
         "paged decode forward with optional int8/fp8 cache scales");
+  pybind11::class_<DecodePlan, std::shared_ptr<DecodePlan>>(m, "DecodePlan")
+      .def_property_readonly("units", [](const DecodePlan& p) { return p.plan.units; })
+      .def_property_readonly("items", [](const DecodePlan& p) { return p.plan.items; })
+      .def_property_readonly("batch", [](const DecodePlan& p) { return p.plan.batch; })
+      .def_property_readonly("buffer", [](const DecodePlan& p) { return p.buffer; });
+  m.def("areno_paged_decode_plan", &paged_decode_plan, "work list of a decode step, built once for all its layers");
+  m.def("areno_paged_causal_attention_decode_forward_planned", &paged_decode_forward_planned,
+        "paged decode forward with a per-step plan");
   m.def("areno_paged_cache_write", &cache_write, "quantize-and-scatter KV cache write");
   m.def("areno_paged_varlen_causal_attention_forward", &paged_varlen_forward,
         "causal varlen prefill over paged (optionally quantized) KV");

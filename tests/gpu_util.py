@@ -36,11 +36,24 @@ def dequant_cpu(cache: torch.Tensor, scale: torch.Tensor | None) -> torch.Tensor
     return out
 
 
-def run_decode(w: workloads.DecodeWorkload, *, window_left=None, num_splits=8):
+def build_plan(w: workloads.DecodeWorkload, *, window_left=None, grouped=False, buffer=None):
+    """The per-step plan of the decode op for a workload's tables."""
+    groups = {}
+    if grouped:
+        groups = dict(prefix_group_rows=w.meta["prefix_group_rows"], shared_prefix_lens=w.meta["shared_prefix_lens"])
+    return ops.areno_paged_decode_plan(
+        w.block_table, w.cache_seqlens, w.k_cache, w.v_cache, q_heads=w.q.shape[1], q_dtype=w.q.dtype,
+        window_left=window_left, k_scale=w.k_scale, v_scale=w.v_scale, buffer=buffer, **groups,
+    )  # fmt: skip
+
+
+def run_decode(w: workloads.DecodeWorkload, *, window_left=None, num_splits=8, planned=False):
+    """The decode op on a workload; ``planned`` runs it with a per-step plan built from the same tables."""
+    plan = build_plan(w, window_left=window_left) if planned else None
     return ops.areno_paged_causal_attention_decode(
         w.q, w.k_update, w.v_update, w.k_cache, w.v_cache, w.block_table, w.cache_seqlens,
         window_left=window_left, num_splits=num_splits, softmax_scale=w.softmax_scale,
-        k_scale=w.k_scale, v_scale=w.v_scale,
+        k_scale=w.k_scale, v_scale=w.v_scale, plan=plan,
     )  # fmt: skip
 
 

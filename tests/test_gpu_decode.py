@@ -11,8 +11,8 @@ import torch
 from areno_amd import workloads
 from areno_amd.accel import attention as ops
 from oracle import quant_ref as qr
-from tests.gpu_util import (DEV, assert_close, expected_decode, expected_decode_rows, gpu_quantize, run_decode,
-                            tolerances)
+from tests.gpu_util import (DEV, assert_close, build_plan, expected_decode, expected_decode_rows, gpu_quantize,
+                            run_decode, tolerances)
 
 pytestmark = pytest.mark.gpu
 
@@ -49,11 +49,12 @@ def _snapshot(w):
 
 @pytest.mark.parametrize("kv", ["fp32", "bf16", "fp16", "int8", "fp8"])
 @pytest.mark.parametrize("window_left", [None, 40, 0])
-def test_cfg0_tiny(kv, window_left):
+@pytest.mark.parametrize("planned", [False, True])
+def test_cfg0_tiny(kv, window_left, planned):
     w = workloads.cfg0_tiny(kv, device=DEV, quantize_fn=gpu_quantize, poison=True,
                             act_dtype=torch.bfloat16)  # fmt: skip
     before = _snapshot(w)
-    out = run_decode(w, window_left=window_left)
+    out = run_decode(w, window_left=window_left, planned=planned)
     assert out.shape == w.q.shape and out.dtype == w.q.dtype
     _check_append(w, before)
     assert_close(out, expected_decode(w, window_left=window_left), *tolerances(kv), what=f"cfg0 {kv} w={window_left}")
@@ -113,6 +114,8 @@ def test_head_dims_192_256_512_on_the_matrix_core_kernel(kv, d, hq, hkv, window_
     out = run_decode(w, window_left=window_left)
     assert_close(out, expected_decode(w, window_left=window_left), *tolerances(kv), what=f"D={d} {kv} {hq}/{hkv}")
     _check_append(w, before)
+    # the same step through a plan: the same bits (the second append rewrites the slot with the same values)
+    assert torch.equal(run_decode(w, window_left=window_left, planned=True), out)
 
 
 def test_graph_padded_rows_on_a_scratch_block_are_harmless():
@@ -139,6 +142,7 @@ def test_cfg1_cfg2_full_size(kv):
     before = _snapshot(w)
     out = run_decode(w)
     _check_append(w, before)
+    assert torch.equal(run_decode(w, planned=True), out), "the planned step differs from the plain one"
     mx, mean = assert_close(out, expected_decode(w), *tolerances(kv), what=f"cfg {kv} full")
     print(f"cfg1/2 {kv}: max-abs {mx:.3e} mean-abs {mean:.3e}")
     # size-independent property: appending the same token again at L_b + 1 ... is a different op; instead
@@ -211,6 +215,7 @@ def test_prefix_groups_match_the_plain_op_and_the_oracle(kv, hq, hkv, samples):
             dst.copy_(src)
     grouped = _grouped_decode(w)
     assert_close(grouped, expected_decode(w), *tolerances(kv), what=f"grouped {kv} vs oracle")
+    assert torch.equal(_grouped_decode(w, plan=build_plan(w, grouped=True)), grouped), "planned grouped step differs"
     # same math in another summation order: the outputs may differ by one unit of the 16-bit output format
     assert_close(grouped, plain.cpu().float(), 8e-3, what=f"grouped {kv} vs plain op")
     for a, b, name in zip((w.k_cache, w.v_cache, w.k_scale, w.v_scale), after_plain, ("k", "v", "k_scale", "v_scale")):
@@ -243,6 +248,7 @@ def test_cfg3_full_size_grouped():
     mx, mean = assert_close(grouped[rows], want, *tolerances("fp8"), what="cfg3 full size, grouped kernel vs oracle")
     print(f"cfg3 full grouped: max-abs {mx:.3e} mean-abs {mean:.3e} on {len(rows)} rows")
     after_grouped = tuple(t.clone() for t in pools)
+    assert torch.equal(_grouped_decode(w, plan=build_plan(w, grouped=True)), grouped), "planned grouped step differs"
     for dst, src in zip(pools, on_device):
         dst.copy_(src)
     plain = run_decode(w)
@@ -262,6 +268,9 @@ def test_batches_beyond_one_launch_run_in_row_ranges():
     out = run_decode(w)
     assert_close(out, expected_decode(w), *tolerances("int8"), what="1500 rows")
     _check_append(w, before)
+    plan = build_plan(w)
+    assert plan.units == 0  # a plan covers one launch; the op then runs as without one
+    assert torch.equal(run_decode(w, planned=True), out)
     r = workloads.cfg3_rollout("fp8", device=DEV, prompts=400, samples=3, prefix_lo=40, prefix_hi=120, median=30.0,
                                cap=100, quantize_fn=gpu_quantize, seed=83, hq=8, hkv=2)  # fmt: skip
     grouped = _grouped_decode(r)
@@ -328,3 +337,35 @@ def test_random_draws_of_shape_length_window_and_cache_type(seed):
     what = f"draw {seed}: {kv} {hkv * group}/{hkv} d={d} bs={bs} batch={batch} {profile} window={window}"
     assert_close(out, expected_decode(w, window_left=window), *tolerances(kv), what=what)
     _check_append(w, before)
+    assert torch.equal(run_decode(w, window_left=window, planned=True), out), f"{what}: the planned step differs"
+
+
+def test_a_plan_for_other_shapes_is_refused():
+    w = workloads.cfg0_tiny("int8", device=DEV, quantize_fn=gpu_quantize)
+    plan = build_plan(w)
+    assert plan.units > 0 and plan.batch == w.q.shape[0]
+    args = (w.q, w.k_update, w.v_update, w.k_cache, w.v_cache, w.block_table, w.cache_seqlens)
+    kw = dict(softmax_scale=w.softmax_scale, k_scale=w.k_scale, v_scale=w.v_scale, plan=plan)
+    with pytest.raises(RuntimeError, match="plan was built for other shapes"):
+        ops.areno_paged_causal_attention_decode(*args, window_left=5, **kw)
+    with pytest.raises(RuntimeError, match="plan was built for other shapes"):
+        ops.areno_paged_causal_attention_decode(w.q[:3], w.k_update[:3], w.v_update[:3], w.k_cache, w.v_cache,
+                                                w.block_table[:3].contiguous(), w.cache_seqlens[:3], **kw)  # fmt: skip
+    with pytest.raises(ValueError, match="int32 block_table"):
+        ops.areno_paged_decode_plan(w.block_table.long(), w.cache_seqlens, w.k_cache, w.v_cache, q_heads=8,
+                                    k_scale=w.k_scale, v_scale=w.v_scale)  # fmt: skip
+
+
+def test_one_plan_serves_the_layers_of_a_step():
+    """Two layers (two cache pools) of one decode step share block table, lengths and one plan."""
+    layers = [workloads.cfg0_tiny("fp8", device=DEV, quantize_fn=gpu_quantize, seed=s) for s in (1000, 1000)]
+    a, b = layers
+    b.k_cache.copy_(torch.flip(a.k_cache.view(torch.uint8), dims=(3,)).view(b.k_cache.dtype))  # other contents, same tables
+    plan = build_plan(a)
+    for w in layers:
+        plain = run_decode(w)
+        with_plan = ops.areno_paged_causal_attention_decode(
+            w.q, w.k_update, w.v_update, w.k_cache, w.v_cache, a.block_table, a.cache_seqlens,
+            softmax_scale=w.softmax_scale, k_scale=w.k_scale, v_scale=w.v_scale, plan=plan)  # fmt: skip
+        assert torch.equal(with_plan, plain)
+        assert_close(with_plan, expected_decode(w), *tolerances("fp8"), what="layer through the shared plan")

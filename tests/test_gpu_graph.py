@@ -20,13 +20,16 @@ BUCKET = 8
 STEPS = 4
 
 
-def _decode(q, ku, vu, kc, vc, table, lens, ks, vs, scale):
+def _decode(q, ku, vu, kc, vc, table, lens, ks, vs, scale, plan=None):
     return ops.areno_paged_causal_attention_decode(q, ku, vu, kc, vc, table, lens, num_splits=8, softmax_scale=scale,
-                                                   k_scale=ks, v_scale=vs)  # fmt: skip
+                                                   k_scale=ks, v_scale=vs, plan=plan)  # fmt: skip
 
 
 @pytest.mark.parametrize("kv,hq,hkv,d", [("bf16", 8, 2, 64), ("int8", 28, 4, 128), ("fp8", 8, 8, 128)])
-def test_decode_graph_replays_match_eager_and_oracle(kv, hq, hkv, d):
+@pytest.mark.parametrize("planned", [False, True])
+def test_decode_graph_replays_match_eager_and_oracle(kv, hq, hkv, d, planned):
+    """``planned``: the captured step rebuilds the per-step plan from the static tables (into a static buffer) in front
+    of the decode call, so every replay plans for the values copied in before it."""
     actual = len(LENGTHS)
     w = workloads.make_decode_workload(
         f"graph-{kv}", seed=31, batch=actual, hq=hq, hkv=hkv, d=d, bs=16, kv=kv, lengths=torch.tensor(LENGTHS),
@@ -49,8 +52,15 @@ def test_decode_graph_replays_match_eager_and_oracle(kv, hq, hkv, d):
     s_table = torch.full((BUCKET, cols), scratch, dtype=torch.int32, device=DEV)
     s_lens = torch.zeros(BUCKET, dtype=torch.int32, device=DEV)
 
+    s_plan = torch.empty(1 << 20, dtype=torch.uint8, device=DEV) if planned else None
+
     def run_static():
-        return _decode(s_q, s_ku, s_vu, g_kc, g_vc, s_table, s_lens, g_ks, g_vs, w.softmax_scale)
+        plan = None
+        if planned:
+            plan = ops.areno_paged_decode_plan(s_table, s_lens, g_kc, g_vc, q_heads=hq, q_dtype=w.q.dtype, k_scale=g_ks,
+                                               v_scale=g_vs, buffer=s_plan)  # fmt: skip
+            assert plan.units > 0
+        return _decode(s_q, s_ku, s_vu, g_kc, g_vc, s_table, s_lens, g_ks, g_vs, w.softmax_scale, plan)
 
     # warm-up on a side stream with everything parked (touches only the scratch block), then capture
     side = torch.cuda.Stream()
