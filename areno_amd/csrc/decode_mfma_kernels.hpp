@@ -38,7 +38,9 @@
 //   O^T[dim][head] += V^T . P^T per pair of token groups, where P^T *is* the C layout of S^T, so no cross-lane
 //      movement of P is needed.
 // One tile is in flight per wave: the loads of tile x + 1 go out while tile x is computed (V registers are free once
-// the tile is staged, K registers once the scores are issued), the block ids of tile x + 2 in front of them.  The
+// the tile is staged, K registers once the scores are issued), the block ids of tile x + 2 in front of them.  (Moving
+// the K tile to registers of its own so that its successor's loads go out at the start of the step was measured and
+// changed nothing: the memory system, not the moment of issue, sets a tile's time.)  The
 // loop over the tiles of a segment has no branches around loads, so every wait the compiler places counts
 // exactly the loads younger than the one needed.
 // int8 codes become fp16 by placing (code ^ 0x80) under the exponent byte 0x64 (v_perm): 1152 + code exactly;
@@ -96,6 +98,8 @@ constexpr int decode_tile_tokens(bool quantized) { return quantized ? ARENO_MFMA
 //   cum    [items + 1]   exclusive prefix sums of the items' extents on the cost line (decode_items.hpp)
 //   items  [items][4]    lo, end, row, nseq of every item
 //   units  [units][16]   where a wave's unit starts (layout below)
+//   rows   [batch][4]    for the merge kernel: first unit and number of units of the row's own item, and of its
+//                        sub-group's shared item
 constexpr int kDecodeDumpFloats = 16 * 512 + 2 * kWave;  // 16 columns of the widest head, and an (m, l) pair per lane
 constexpr int kDecodeHold = 2;  // partials a wave parks in LDS before it stores them
 constexpr int kPlanUnitWords = 16;
@@ -124,6 +128,7 @@ struct MfmaDecodeParams {
   const int32_t* plan_cum;
   const int32_t* plan_items;
   const int32_t* plan_units;
+  const int32_t* plan_rows;
   // The token being appended, for the merge kernel when items.append_in_merge: [batch, kv_heads, head_dim], dtype
   // q_dtype; quantized like the cache writer does and stored into the page.
   const void* k_update;

@@ -134,9 +134,8 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_kernel(Decod
 // Merge of the MFMA path's partials.  The units that own quanta of an item wrote one partial each: a per-row item
 // into slot (unit + row) of the per-row region, a shared-prefix item (grouped mode) into slot (unit + item) of the
 // shared region, where the row's head sits in column (row - first row) * G + head of its kv head.  One wave per
-// (row, q head) gathers the candidates of both kinds: lanes first fetch up to 64 (m, l) pairs in parallel and agree
-// on the maximum, then every lane accumulates its share of the head dimension with the partial loads of a group of
-// four candidates in flight together (the loop has no loop-carried memory dependence).
+// (row, q head) gathers the candidates of both kinds, kMergeChunk at a time, and merges them with the log-sum-exp
+// recurrence of the reference's reduce kernel (areno/accel/csrc/attention.cu:656-702).
 //
 // The token being appended (items.append_in_merge): the streaming waves of the split kernel read only what is in the
 // pages, and this kernel, which owns the (row, head) anyway, does what the reference's update kernel
@@ -145,6 +144,13 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_kernel(Decod
 // first q head stores codes and scale at (block_table[b, L / bs], L % bs) -- skipped, like the cache writer does, when
 // the column or the page id lies outside the table or the pool -- and the token enters the merge as a partial of its
 // own with m = q . k_new, l = 1, acc = v_new, both as a reader of the page would see them.
+//
+// Memory round trips, which are what this kernel's time is made of: (1) the row's entry of the plan (or the prefix
+// sums its units follow from), its length and the q / k_update / v_update rows; (2) the append's block id and, for up
+// to kMergeChunk candidates at once, (m, l) and the accumulator row together -- a candidate's row is fetched before
+// its weight is known, rows of absent candidates are dropped after the fact; (3) the stores.
+constexpr int kMergeChunk = 8;
+
 template <int EPW>  // head-dimension elements per lane: head_dim <= 64 EPW
 __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel(MfmaDecodeParams mp) {
   const DecodeParams& p = mp.d;
@@ -153,23 +159,44 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   if (row >= p.batch * p.q_heads) return;
   const int b = row / p.q_heads;
   const int h = row - b * p.q_heads;
+  const int kvh = h / p.group;
   const int d = p.head_dim;
   const ItemShape& shape = mp.items;
   const int num_items = shape.num_items();
-  const int32_t* cum = mp.plan_cum != nullptr ? mp.plan_cum : mp.cum_out;
-  // the prefix sums this row needs, fetched together (their indices follow from the row alone)
-  const int v_own = shape.num_shared + b;
-  const int cum_total = cum[num_items], cum_own = cum[v_own], cum_own_end = cum[v_own + 1];
+  const bool append = shape.append_in_merge != 0;
 
-  float acc[EPW];
-#pragma unroll
-  for (int e = 0; e < EPW; ++e) acc[e] = 0.0f;
-  float m = kNegInf, l = 0.0f;
-  if (shape.append_in_merge) {
-    const int kvh = h / p.group;
+  // ---- round trip 1 ---------------------------------------------------------------------------------------------------
+  // units that hold partials of the row: its own item's and, with prefix groups, its sub-group's shared item's
+  int own_lo = 0, own_n = 0, sh_lo = 0, sh_n = 0, sh_item = 0, sh_col = 0;
+  int4_t planned_units = {0, 0, 0, 0};
+  int cum_total = 0, cum_own = 0, cum_own_end = 0, cum_sh = 0, cum_sh_end = 0;
+  if (shape.num_shared > 0) {
+    const int gi = b / shape.group_rows;
+    const int j = (b - gi * shape.group_rows) / shape.cols_seqs;
+    sh_item = gi * shape.subs_per_group + j;
+    const int first_row = gi * shape.group_rows + j * shape.cols_seqs;
+    sh_col = kvh * 16 + (b - first_row) * p.group + (h - kvh * p.group);
+  }
+  if (mp.plan_rows != nullptr) {
+    planned_units = *reinterpret_cast<const int4_t*>(mp.plan_rows + 4 * static_cast<int64_t>(b));
+    cum_total = mp.plan_rows[-4];
+  } else {
+    const int32_t* cum = mp.cum_out;
+    const int v_own = shape.num_shared + b;
+    cum_total = cum[num_items];
+    cum_own = cum[v_own];
+    cum_own_end = cum[v_own + 1];
+    if (shape.num_shared > 0) {
+      cum_sh = cum[sh_item];
+      cum_sh_end = cum[sh_item + 1];
+    }
+  }
+  float qv[EPW], kx[EPW], vx[EPW];
+  uint16_t kraw[EPW], vraw[EPW];
+  int64_t pos = 0;
+  if (append) {
     const int64_t src_base = (static_cast<int64_t>(b) * p.kv_heads + kvh) * d;
-    float qv[EPW], kx[EPW], vx[EPW];
-    uint16_t kraw[EPW], vraw[EPW];
+    pos = p.cache_seqlens[b];
 #pragma unroll
     for (int e = 0; e < EPW; ++e) {
       const int idx = lane + e * kWave;
@@ -177,17 +204,95 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
       kraw[e] = in ? static_cast<const uint16_t*>(mp.k_update)[src_base + idx] : 0;
       vraw[e] = in ? static_cast<const uint16_t*>(mp.v_update)[src_base + idx] : 0;
       qv[e] = in ? load_as_float(p.q, static_cast<int64_t>(row) * d + idx, p.q_dtype) : 0.0f;
-      kx[e] = p.q_dtype == ARENO_DT_BF16 ? bf16_bits_to_float(kraw[e]) : f16_bits_to_float(kraw[e]);
-      vx[e] = p.q_dtype == ARENO_DT_BF16 ? bf16_bits_to_float(vraw[e]) : f16_bits_to_float(vraw[e]);
     }
-    const int64_t pos = p.cache_seqlens[b];
+  }
+  // (with fewer cost positions than units a candidate's unit may be empty and have written nothing)
+  const bool every_unit_has_quanta = cum_total >= mp.num_units;
+  const UnitGeometry geo = make_unit_geometry(cum_total, mp.num_units);
+  if (mp.plan_rows != nullptr) {
+    own_lo = planned_units[0];
+    own_n = planned_units[1];
+    sh_lo = planned_units[2];
+    sh_n = planned_units[3];
+  } else {
+    if (cum_own_end > cum_own) {
+      int last;
+      item_units(geo, shape.switch_quanta, cum_own, cum_own_end, own_lo, last);
+      own_n = last - own_lo + 1;
+    }
+    if (cum_sh_end > cum_sh) {
+      int last;
+      item_units(geo, shape.switch_quanta, cum_sh, cum_sh_end, sh_lo, last);
+      sh_n = last - sh_lo + 1;
+    }
+  }
+  const int total = own_n + sh_n;
+
+  // ---- round trip 2: candidates, and the page the new token goes to -------------------------------------------------
+  // candidate c: where its (m, l) pair and its accumulator row are; absent when its unit wrote nothing
+  auto locate = [&](int c, const float*& ml, const float*& acc_row) {
+    bool present = c < total;
+    const int cc = present ? c : 0;
+    const int u = cc < own_n ? own_lo + cc : sh_lo + (cc - own_n);
+    if (!every_unit_has_quanta) present = present && geo.unit_start(u) != geo.unit_start(u + 1);
+    if (cc < own_n) {
+      const int64_t prow = static_cast<int64_t>(u + b) * p.q_heads + h;
+      ml = p.part_ml + prow * 2;
+      acc_row = p.part_acc + prow * d;
+    } else {
+      const int64_t prow = static_cast<int64_t>(u + sh_item) * p.kv_heads * 16 + sh_col;
+      ml = mp.shared_ml + prow * 2;
+      acc_row = mp.shared_acc + prow * d;
+    }
+    return present;
+  };
+  struct Chunk {
+    float m[kMergeChunk], l[kMergeChunk];
+    float v[kMergeChunk][EPW];
+  };
+  auto load_chunk = [&](int base, Chunk& ch) {
+#pragma unroll
+    for (int j = 0; j < kMergeChunk; ++j) {
+      const float* ml = nullptr;
+      const float* part = nullptr;
+      const bool present = total > 0 && locate(base + j, ml, part);  // (total == 0: nothing was located)
+      float2_t pair = {kNegInf, 0.0f};
+      if (present) pair = *reinterpret_cast<const float2_t*>(ml);
+      // a partial without keys contributes nothing (attention.cu:680-682 in the reference)
+      ch.m[j] = (present && pair[1] != 0.0f) ? pair[0] : kNegInf;
+      ch.l[j] = present ? pair[1] : 0.0f;
+#pragma unroll
+      for (int e = 0; e < EPW; ++e) {
+        const int idx = lane + e * kWave;
+        ch.v[j][e] = (present && idx < d) ? part[idx] : 0.0f;
+      }
+    }
+  };
+  Chunk first;
+  load_chunk(0, first);
+  bool store = false;
+  int64_t dst_row = 0;
+  if (append) {
     const int64_t col = pos / p.block_size;
     const int64_t slot = pos - col * p.block_size;
     bool ok = pos >= 0 && col < p.max_blocks;
     const int64_t blk = ok ? p.block_table[static_cast<int64_t>(b) * p.max_blocks + col] : 0;
     ok = ok && blk >= 0 && blk < mp.num_blocks;
-    const bool store = ok && mp.write_append != 0 && h == kvh * p.group;
-    const int64_t dst_row = (blk * p.block_size + slot) * p.kv_heads + kvh;
+    store = ok && mp.write_append != 0 && h == kvh * p.group;
+    dst_row = (blk * p.block_size + slot) * p.kv_heads + kvh;
+  }
+
+  // ---- the new token: quantize, store, m = q . k_new, l = 1, acc = v_new ----------------------------------------------
+  float acc[EPW];
+#pragma unroll
+  for (int e = 0; e < EPW; ++e) acc[e] = 0.0f;
+  float m = kNegInf, l = 0.0f;
+  if (append) {
+#pragma unroll
+    for (int e = 0; e < EPW; ++e) {
+      kx[e] = p.q_dtype == ARENO_DT_BF16 ? bf16_bits_to_float(kraw[e]) : f16_bits_to_float(kraw[e]);
+      vx[e] = p.q_dtype == ARENO_DT_BF16 ? bf16_bits_to_float(vraw[e]) : f16_bits_to_float(vraw[e]);
+    }
     float khat[EPW], vhat[EPW];
     if (is_quantized_dtype(p.cache_dtype)) {
       quantize_row<EPW>(kx, lane, d, dst_row, const_cast<void*>(p.k_cache), const_cast<void*>(p.k_scale), p.cache_dtype,
@@ -216,93 +321,30 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
     for (int e = 0; e < EPW; ++e) acc[e] = vhat[e];
   }
 
-  const UnitGeometry geo = make_unit_geometry(cum_total, mp.num_units);
-  // the row's own item, if it has quanta ...
-  int own_lo = 0, own_n = 0;
-  if (cum_own_end > cum_own) {
-    int last;
-    item_units(geo, shape.switch_quanta, cum_own, cum_own_end, own_lo, last);
-    own_n = last - own_lo + 1;
-  }
-  // ... and the shared item of its sub-group, if it has quanta
-  int sh_lo = 0, sh_n = 0, sh_item = 0, sh_col = 0;
-  if (shape.num_shared > 0) {
-    const int gi = b / shape.group_rows;
-    const int j = (b - gi * shape.group_rows) / shape.cols_seqs;
-    sh_item = gi * shape.subs_per_group + j;
-    const int first_row = gi * shape.group_rows + j * shape.cols_seqs;
-    const int kvh = h / p.group;
-    sh_col = kvh * 16 + (b - first_row) * p.group + (h - kvh * p.group);
-    if (cum[sh_item + 1] > cum[sh_item]) {
-      int last;
-      item_units(geo, shape.switch_quanta, cum[sh_item], cum[sh_item + 1], sh_lo, last);
-      sh_n = last - sh_lo + 1;
-    }
-  }
-  const int total = own_n + sh_n;
-  // candidate c: the unit it belongs to, and where its (m, l) pair and its accumulator row are
-  auto unit_of_candidate = [&](int c) { return c < own_n ? own_lo + c : sh_lo + (c - own_n); };
-  auto locate = [&](int c, const float*& ml, const float*& acc_row) {
-    const int u = unit_of_candidate(c);
-    if (c < own_n) {
-      const int64_t prow = static_cast<int64_t>(u + b) * p.q_heads + h;
-      ml = p.part_ml + prow * 2;
-      acc_row = p.part_acc + prow * d;
-    } else {
-      const int64_t prow = static_cast<int64_t>(u + sh_item) * p.kv_heads * 16 + sh_col;
-      ml = mp.shared_ml + prow * 2;
-      acc_row = mp.shared_acc + prow * d;
-    }
-  };
-
-  for (int base = 0; base < total; base += kWave) {
-    // lane j looks at candidate base + j
-    float part_m = kNegInf, part_l = 0.0f;
-    if (base + lane < total) {
-      // a unit without quanta wrote nothing: its candidate is absent (weight 0 below)
-      const int u = unit_of_candidate(base + lane);
-      if (geo.unit_start(u) != geo.unit_start(u + 1)) {
-        const float* ml = nullptr;
-        const float* unused = nullptr;
-        locate(base + lane, ml, unused);
-        part_m = ml[0];
-        part_l = ml[1];
-        if (part_l == 0.0f) part_m = kNegInf;  // a partial without keys contributes nothing
-      }
-    }
-    const float m_new = fmaxf(m, wave_max(part_m));
+  // ---- merge ----------------------------------------------------------------------------------------------------------
+  auto merge_chunk = [&](const Chunk& ch) {
+    float m_new = m;
+#pragma unroll
+    for (int j = 0; j < kMergeChunk; ++j) m_new = fmaxf(m_new, ch.m[j]);
     const float m_safe = m_new == kNegInf ? 0.0f : m_new;
     const float alpha = fast_exp2(m - m_safe);
-    const float w = fast_exp2(part_m - m_safe);  // 0 for absent candidates
-    l = l * alpha + wave_sum(w * part_l);
-    m = m_new;
+    l *= alpha;
 #pragma unroll
     for (int e = 0; e < EPW; ++e) acc[e] *= alpha;
-    const int count = min(kWave, total - base);
-    for (int j0 = 0; j0 < count; j0 += 4) {
-      float wj[4];
-      float v[4][EPW];
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const int j = min(j0 + jj, count - 1);
-        wj[jj] = j0 + jj < count ? __shfl(w, j, kWave) : 0.0f;
-        const float* ml = nullptr;
-        const float* part = nullptr;
-        locate(base + j, ml, part);
-        const bool present = wj[jj] != 0.0f;
+    for (int j = 0; j < kMergeChunk; ++j) {
+      const float w = fast_exp2(ch.m[j] - m_safe);  // 0 for absent candidates
+      l += w * ch.l[j];
 #pragma unroll
-        for (int e = 0; e < EPW; ++e) {
-          const int idx = lane + e * kWave;
-          // partials of units without quanta were never written: read only what carries a non-zero weight
-          v[jj][e] = (idx < d && present) ? part[idx] : 0.0f;
-        }
-      }
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-#pragma unroll
-        for (int e = 0; e < EPW; ++e) acc[e] += wj[jj] * v[jj][e];
-      }
+      for (int e = 0; e < EPW; ++e) acc[e] += w * ch.v[j][e];
     }
+    m = m_new;
+  };
+  merge_chunk(first);
+  for (int base = kMergeChunk; base < total; base += kMergeChunk) {
+    Chunk more;
+    load_chunk(base, more);
+    merge_chunk(more);
   }
 #pragma unroll
   for (int e = 0; e < EPW; ++e) {
@@ -505,6 +547,7 @@ struct PlanParams {
   int32_t* cum;
   int32_t* items;
   int32_t* units;
+  int32_t* rows;
   ItemShape shape;
   int32_t num_units;
   int32_t bs_shift;
@@ -584,6 +627,30 @@ __global__ __launch_bounds__(kPlanThreads) void decode_plan_kernel(PlanParams pp
   __syncthreads();
   const PlainItemTable table = {s_item, s_cum};
   const UnitGeometry geo = make_unit_geometry(s_cum[num_items], pp.num_units);
+  // per row, for the merge kernel: first unit and number of units of its own item and of its sub-group's shared item;
+  // in front of the rows the total of the cost line
+  if (tid == 0) *reinterpret_cast<int4_t*>(pp.rows - 4) = int4_t{s_cum[num_items], 0, 0, 0};
+  for (int b = tid; b < shape.batch; b += kPlanThreads) {
+    int4_t r = {0, 0, 0, 0};
+    const int v_own = shape.num_shared + b;
+    if (s_cum[v_own + 1] > s_cum[v_own]) {
+      int first, last;
+      item_units(geo, shape.switch_quanta, s_cum[v_own], s_cum[v_own + 1], first, last);
+      r[0] = first;
+      r[1] = last - first + 1;
+    }
+    if (GROUPED) {
+      const int gi = b / shape.group_rows;
+      const int sh_item = gi * shape.subs_per_group + (b - gi * shape.group_rows) / shape.cols_seqs;
+      if (s_cum[sh_item + 1] > s_cum[sh_item]) {
+        int first, last;
+        item_units(geo, shape.switch_quanta, s_cum[sh_item], s_cum[sh_item + 1], first, last);
+        r[2] = first;
+        r[3] = last - first + 1;
+      }
+    }
+    *reinterpret_cast<int4_t*>(pp.rows + 4 * static_cast<int64_t>(b)) = r;
+  }
   for (int u = tid; u < pp.num_units; u += kPlanThreads) {
     int rec[kPlanUnitWords];
 #pragma unroll
@@ -617,14 +684,15 @@ __global__ __launch_bounds__(kPlanThreads) void decode_plan_kernel(PlanParams pp
 
 // layout of a plan buffer for an item list of `items` entries and `units` units, in int32 words
 struct PlanLayout {
-  size_t cum, items, units, words;
+  size_t cum, items, units, rows, words;
 };
-PlanLayout plan_layout(size_t items, size_t units) {
+PlanLayout plan_layout(size_t items, size_t units, size_t batch) {
   PlanLayout l;
   l.cum = 0;
   l.items = (items + 1 + 3) / 4 * 4;  // 16-byte aligned
   l.units = l.items + 4 * items;
-  l.words = l.units + kPlanUnitWords * units;
+  l.rows = l.units + kPlanUnitWords * units + 4;  // (the four words in front of the rows: total cost positions, 0, 0, 0)
+  l.words = l.rows + 4 * batch;
   return l;
 }
 
@@ -757,12 +825,14 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     mp.plan_cum = nullptr;
     mp.plan_items = nullptr;
     mp.plan_units = nullptr;
+    mp.plan_rows = nullptr;
     if (planned) {
-      const PlanLayout l = plan_layout(plan->items, plan->units);
+      const PlanLayout l = plan_layout(plan->items, plan->units, plan->batch);
       const int32_t* words = static_cast<const int32_t*>(plan->buffer);
       mp.plan_cum = words + l.cum;
       mp.plan_items = words + l.items;
       mp.plan_units = words + l.units;
+      mp.plan_rows = words + l.rows;
     }
     if (stages & ARENO_STAGE_SPLIT) {
       hipLaunchKernelGGL(mfma, dim3(grid.workgroups, grid.head_groups), dim3(grid.waves * kWave), 0, s, mp);
@@ -889,7 +959,7 @@ extern "C" int areno_hip_paged_decode_grouped(const areno_paged_cache* cache, co
 extern "C" size_t areno_hip_paged_decode_plan_bytes(int32_t batch) {
   if (batch <= 0) return 0;
   const size_t items = 2 * static_cast<size_t>(batch < areno::kMfmaMaxBatch ? batch : areno::kMfmaMaxBatch);
-  return areno::plan_layout(items, areno::kMfmaMaxUnits).words * sizeof(int32_t);
+  return areno::plan_layout(items, areno::kMfmaMaxUnits, items / 2).words * sizeof(int32_t);
 }
 
 extern "C" int areno_hip_paged_decode_plan(areno_decode_plan* plan, void* buffer, size_t buffer_bytes,
@@ -926,7 +996,7 @@ extern "C" int areno_hip_paged_decode_plan(areno_decode_plan* plan, void* buffer
   plan->items = 0;
   plan->tile_tokens = 0;
   if (batch == 0 || choice.fn == nullptr) return ARENO_OK;  // a kernel that takes no plan serves these shapes
-  const PlanLayout l = plan_layout(choice.items.num_items(), choice.grid.units);
+  const PlanLayout l = plan_layout(choice.items.num_items(), choice.grid.units, batch);
   if (buffer == nullptr || reinterpret_cast<uintptr_t>(buffer) % 16 != 0 || buffer_bytes < l.words * sizeof(int32_t))
     return fail(ARENO_ERR_WORKSPACE, "%s: a 16-byte aligned buffer of %zu bytes is needed, %zu given", op,
                 l.words * sizeof(int32_t), buffer_bytes);
@@ -938,6 +1008,7 @@ extern "C" int areno_hip_paged_decode_plan(areno_decode_plan* plan, void* buffer
   pp.cum = words + l.cum;
   pp.items = words + l.items;
   pp.units = words + l.units;
+  pp.rows = words + l.rows;
   pp.shape = choice.items;
   pp.num_units = choice.grid.units;
   pp.bs_shift = log2_exact(cache->block_size);

@@ -62,16 +62,30 @@ def _gpu_quantize(x, cache_dtype):
     return kc.view(n, hkv, d), ks.view(n, hkv)
 
 
-def _step(w, pool):
+LAYERS_PER_PLAN = 28  # layers of the Qwen2.5-7B-like model the shapes come from: one plan serves the layers of a step
+
+
+def _groups(w):
+    if "shared_prefix_lens" in w.meta:  # what the rollout scheduler knows: rows per prompt, shared tokens per prompt
+        return dict(prefix_group_rows=w.meta["prefix_group_rows"], shared_prefix_lens=w.meta["shared_prefix_lens"])
+    return {}
+
+
+def _plan(w, pool, buffer=None):
     from areno_amd.accel import attention as ops
 
     kc, vc, ks, vs = pool
-    groups = {}
-    if "shared_prefix_lens" in w.meta:  # what the rollout scheduler knows: rows per prompt, shared tokens per prompt
-        groups = dict(prefix_group_rows=w.meta["prefix_group_rows"], shared_prefix_lens=w.meta["shared_prefix_lens"])
+    return ops.areno_paged_decode_plan(w.block_table, w.cache_seqlens, kc, vc, q_heads=w.q.shape[1], q_dtype=w.q.dtype,
+                                       k_scale=ks, v_scale=vs, buffer=buffer, **_groups(w))  # fmt: skip
+
+
+def _step(w, pool, plan=None):
+    from areno_amd.accel import attention as ops
+
+    kc, vc, ks, vs = pool
     return ops.areno_paged_causal_attention_decode(
         w.q, w.k_update, w.v_update, kc, vc, w.block_table, w.cache_seqlens,
-        softmax_scale=w.softmax_scale, k_scale=ks, v_scale=vs, **groups,
+        softmax_scale=w.softmax_scale, k_scale=ks, v_scale=vs, plan=plan, **_groups(w),
     )  # fmt: skip
 
 
@@ -90,8 +104,13 @@ def _parity_sample(w, out, rows=4):
     return float((out[:rows].cpu().float() - want).abs().max())
 
 
-def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
-    """Time the whole op (graph replay and eager) and each kernel of it; returns a dict of numbers."""
+def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repeats=15):
+    """Time the whole op (graph replay and eager) and each kernel of it; returns a dict of numbers.
+
+    A step is one layer's decode op.  The layers of a model's decode step share block table and lengths, so the timed
+    sequence is what an engine runs: one plan launch, then LAYERS_PER_PLAN ops that use it, each on another layer's
+    pools, replayed from HIP graphs; the plan launch is inside the timed region and its cost is spread over the steps
+    it serves.  The same sequence without plans is timed next to it."""
     import torch
 
     from areno_amd.accel import cabi
@@ -104,48 +123,69 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
     out = _step(w, pools[0])
     torch.cuda.synchronize()
     parity = _parity_sample(w, out)
+    planned_equal = bool(torch.equal(_step(w, pools[0], _plan(w, pools[0])), out))
 
-    # ---- whole op, replayed from HIP graphs (one graph = one pass over all pool copies) --------------
+    # ---- whole op, replayed from HIP graphs ---------------------------------------------------------------------------
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         for pool in pools:
-            _step(w, pool)
+            _step(w, pool, _plan(w, pool))
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
+    plan_buffer = torch.empty(cabi.decode_plan_bytes(w.q.shape[0]), dtype=torch.uint8, device=w.q.device)
 
-    def capture(n):
+    def capture(n, planned, first_pool=0):
+        """A graph of n steps: with plans, a plan launch in front of every LAYERS_PER_PLAN steps."""
         g = torch.cuda.CUDAGraph()
         keep = []
         with torch.cuda.graph(g):
+            plan = None
             for i in range(n):
-                keep.append(_step(w, pools[i % copies]))
+                pool = pools[(first_pool + i) % copies]
+                if planned and i % LAYERS_PER_PLAN == 0:
+                    plan = _plan(w, pool, plan_buffer)
+                keep.append(_step(w, pool, plan))
         return g, keep
 
-    full, keep_full = capture(copies)
-    rem_n = steps % copies
-    rem, keep_rem = capture(rem_n) if rem_n else (None, None)
-    for _ in range(max(1, -(-warmup // copies))):
-        full.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps // copies):
-        full.replay()
-    if rem is not None:
-        rem.replay()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    us_graph = (t1 - t0) / steps * 1e6
-    # graph replays must reproduce the eager result (checked on the first pool)
-    graph_ok = bool(torch.equal(keep_full[0], out))
+    def timed_replays(planned):
+        """us/step over exactly `steps` steps, `repeats` times."""
+        full_n = min(steps, LAYERS_PER_PLAN * max(1, copies // LAYERS_PER_PLAN + 1))
+        full_n -= full_n % LAYERS_PER_PLAN if full_n >= LAYERS_PER_PLAN else 0
+        full, keep_full = capture(full_n, planned)
+        rem_n = steps % full_n
+        rem, _ = capture(rem_n, planned) if rem_n else (None, None)
+        for _ in range(max(1, -(-warmup // full_n))):
+            full.replay()
+        torch.cuda.synchronize()
+        samples = []
+        for _ in range(repeats):
+            t0 = time.perf_counter()
+            for _ in range(steps // full_n):
+                full.replay()
+            if rem is not None:
+                rem.replay()
+            torch.cuda.synchronize()
+            samples.append((time.perf_counter() - t0) / steps * 1e6)
+        samples.sort()
+        # graph replays must reproduce the eager result (checked on the first pool)
+        return statistics.median(samples), [samples[len(samples) // 10], samples[(len(samples) * 9) // 10]], bool(torch.equal(keep_full[0], out))
 
-    # ---- whole op, eager launches (host launch overhead included) ----------------------------------------
-    for i in range(warmup):
-        _step(w, pools[i % copies])
+    us_graph, us_graph_spread, graph_ok = timed_replays(True)
+    us_graph_plain, us_graph_plain_spread, graph_plain_ok = timed_replays(False)
+
+    # ---- whole op, eager launches (host launch overhead included), a plan per LAYERS_PER_PLAN steps ------------------
+    def eager(n):
+        plan = None
+        for i in range(n):
+            if i % LAYERS_PER_PLAN == 0:
+                plan = _plan(w, pools[i % copies], plan_buffer)
+            _step(w, pools[i % copies], plan)
+
+    eager(warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(steps):
-        _step(w, pools[i % copies])
+    eager(steps)
     torch.cuda.synchronize()
     us_eager = (time.perf_counter() - t0) / steps * 1e6
 
@@ -160,13 +200,13 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=w.q.device)
     caches = [cabi.describe_cache(*pool) for pool in pools]
     out2 = torch.empty_like(w.q)
+    spread = {}
 
-    def time_stage(stage):
-        def launch(i):
-            cabi.paged_decode(caches[i % copies], w.q, w.k_update, w.v_update, out2, w.block_table, w.cache_seqlens,
-                              workspace, softmax_scale=w.softmax_scale, stages=stage, group_rows=group_rows,
-                              shared_lens=shared_lens)  # fmt: skip
+    def build_plan():
+        return cabi.paged_decode_plan(caches[0], w.q.dtype, hq, w.block_table, w.cache_seqlens, plan_buffer,
+                                      group_rows=group_rows, shared_lens=shared_lens)  # fmt: skip
 
+    def time_launches(launch, name):
         for i in range(max(copies, 20)):
             launch(i)
         torch.cuda.synchronize()
@@ -180,35 +220,51 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
             e1.synchronize()
             samples.append(e0.elapsed_time(e1) * 1e3 / kernel_iters)
         samples.sort()
-        spread[stage] = (samples[len(samples) // 10], samples[(len(samples) * 9) // 10])
+        spread[name] = [samples[len(samples) // 10], samples[(len(samples) * 9) // 10]]
         return statistics.median(samples)
 
-    spread = {}
+    def time_stage(stage, plan, name):
+        def launch(i):
+            cabi.paged_decode(caches[i % copies], w.q, w.k_update, w.v_update, out2, w.block_table, w.cache_seqlens,
+                              workspace, softmax_scale=w.softmax_scale, stages=stage, group_rows=group_rows,
+                              shared_lens=shared_lens, plan=plan)  # fmt: skip
 
+        return time_launches(launch, name)
+
+    plan = build_plan()
     # the op folds the append into the merge launch; the stand-alone append launch is timed for reference only
-    us_split = time_stage(cabi.STAGE_SPLIT)
-    us_reduce = time_stage(cabi.STAGE_APPEND | cabi.STAGE_REDUCE)
-    us_append = time_stage(cabi.STAGE_APPEND)
+    us_split_plain = time_stage(cabi.STAGE_SPLIT, None, "split_plain")
+    us_split = time_stage(cabi.STAGE_SPLIT, plan, "split")
+    us_reduce = time_stage(cabi.STAGE_APPEND | cabi.STAGE_REDUCE, plan, "merge")
+    us_append = time_stage(cabi.STAGE_APPEND, None, "append")
+    us_plan = time_launches(lambda i: build_plan(), "plan")
     torch.cuda.synchronize()
     assert torch.equal(out2, out), "C-ABI staged run disagrees with the op"
 
     gbps = alg_bytes / (us_split * 1e-6) / 1e9
-    traffic = PROFILED_TRAFFIC_BYTES.get(w.name)
     ceiling = measure_stream_ceiling(w, pools)
     return {
         "workload": w.name,
         "us_per_step": us_graph,
+        "us_per_step_p10_p90": us_graph_spread,
+        "us_per_step_without_plan": us_graph_plain,
+        "us_per_step_without_plan_p10_p90": us_graph_plain_spread,
         "us_per_step_eager": us_eager,
-        "kernel_us": {"split": us_split, "merge_with_append": us_reduce, "append_alone_not_in_op": us_append},
-        # 10th / 90th percentile of the split kernel's samples (each the mean of back-to-back launches)
-        "split_us_p10_p90": list(spread[cabi.STAGE_SPLIT]),
+        "plan": {"layers_per_plan": LAYERS_PER_PLAN, "plan_kernel_us": us_plan,
+                 "plan_us_per_step": us_plan / LAYERS_PER_PLAN, "planned_equals_plain_bitwise": planned_equal},
+        "kernel_us": {"split": us_split, "split_without_plan": us_split_plain, "merge_with_append": us_reduce,
+                      "append_alone_not_in_op": us_append, "plan": us_plan},
+        # 10th / 90th percentile of the kernels' samples (each the mean of back-to-back launches)
+        "split_us_p10_p90": spread["split"],
+        "split_without_plan_us_p10_p90": spread["split_plain"],
         "tokens_per_s": w.q.shape[0] / (us_graph * 1e-6),
         "algorithmic_bytes": alg_bytes,
         "op_gbps": alg_bytes / (us_graph * 1e-6) / 1e9,
         "roofline": {
             "bound": "hbm", "kernel": "decode_mfma_kernel", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic, "traffic_profiled": traffic,
-            "traffic_source": PROFILED_TRAFFIC_SOURCE["decode"],
+            "frac": gbps / HBM_PEAK_GBPS, "traffic": PROFILED_TRAFFIC_BYTES.get(w.name),
+            "traffic_source": PROFILED_TRAFFIC_SOURCE["decode"] if w.name in PROFILED_TRAFFIC_BYTES else None,
+            "frac_without_plan": alg_bytes / (us_split_plain * 1e-6) / 1e9 / HBM_PEAK_GBPS,
             # what a reader that computes nothing reaches over the same pools (all pages in address order / the distinct
             # pages of the block table in random order), and the split kernel against the latter
             "stream_ceiling_gbps": ceiling["linear_gbps"], "stream_ceiling_paged_gbps": ceiling["paged_gbps"],
@@ -216,7 +272,7 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15):
         },  # fmt: skip
         "pool_copies": copies,
         "parity_max_abs_4rows": parity,
-        "graph_replay_matches_eager": graph_ok,
+        "graph_replay_matches_eager": graph_ok and graph_plain_ok,
         "kv_tokens": {"logical": w.logical_tokens, "unique": w.unique_tokens},
         "block_tables": measure_block_tables(w),
     }
@@ -418,7 +474,7 @@ def measure_prefill(w, iters=20):
         "roofline": {
             "bound": "mfma", "kernel": "prefill_mfma_kernel", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": PROFILED_TRAFFIC_BYTES.get(w.name),
-            "traffic_profiled": PROFILED_TRAFFIC_BYTES.get(w.name), "traffic_source": PROFILED_TRAFFIC_SOURCE["prefill"],
+            "traffic_source": PROFILED_TRAFFIC_SOURCE["prefill"],
         },  # fmt: skip
     }
 
