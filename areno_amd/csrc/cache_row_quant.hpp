@@ -27,7 +27,7 @@ __device__ __forceinline__ void quantize_row(const float (&x)[EPW], int lane, in
   float amax = 0.0f;
 #pragma unroll
   for (int e = 0; e < EPW; ++e) amax = fmaxf(amax, fabsf(x[e]));
-  amax = wave_max(amax);
+  amax = wave_max_fast(amax);
   if (cache_dtype == ARENO_DT_I8) {
     const _Float16 s16 = static_cast<_Float16>(fminf(amax / 127.0f, 65504.0f));
     const _Float16 s16_fixed = (s16 == static_cast<_Float16>(0.0f)) ? static_cast<_Float16>(1.0f) : s16;

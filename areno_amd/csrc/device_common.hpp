@@ -147,6 +147,35 @@ __device__ __forceinline__ float rows_sum(float x) {
   return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
 }
 
+// Reductions over the whole wave, result in every lane, without the LDS crossbar (ds_bpermute) that __shfl_xor
+// compiles to: four data-parallel-primitive steps inside each row of 16 lanes (quad permutes, then the row's half and
+// full mirror), then the two row swaps above.  A third of the latency of six ds_bpermute round trips, which is what a
+// kernel made of a few dependent steps per wave (the merge launch) consists of.
+template <int CTRL>
+__device__ __forceinline__ float dpp_lanes(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+constexpr int kDppQuadSwap1 = 0xb1;      // quad_perm [1, 0, 3, 2]
+constexpr int kDppQuadSwap2 = 0x4e;      // quad_perm [2, 3, 0, 1]
+constexpr int kDppRowHalfMirror = 0x141;  // lane i of a half row <- lane 7 - i
+constexpr int kDppRowMirror = 0x140;      // lane i of a row <- lane 15 - i
+
+__device__ __forceinline__ float wave_max_fast(float x) {
+  x = max_f32(x, dpp_lanes<kDppQuadSwap1>(x));
+  x = max_f32(x, dpp_lanes<kDppQuadSwap2>(x));
+  x = max_f32(x, dpp_lanes<kDppRowHalfMirror>(x));
+  x = max_f32(x, dpp_lanes<kDppRowMirror>(x));
+  return rows_max(x);
+}
+
+__device__ __forceinline__ float wave_sum_fast(float x) {
+  x += dpp_lanes<kDppQuadSwap1>(x);
+  x += dpp_lanes<kDppQuadSwap2>(x);
+  x += dpp_lanes<kDppRowHalfMirror>(x);
+  x += dpp_lanes<kDppRowMirror>(x);
+  return rows_sum(x);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 constexpr float kLog2e = 1.4426950408889634f;

@@ -315,7 +315,7 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
     float dot = 0.0f;
 #pragma unroll
     for (int e = 0; e < EPW; ++e) dot += qv[e] * khat[e];
-    m = wave_sum(dot) * p.scale_log2e;
+    m = wave_sum_fast(dot) * p.scale_log2e;
     l = 1.0f;
 #pragma unroll
     for (int e = 0; e < EPW; ++e) acc[e] = vhat[e];

@@ -479,10 +479,12 @@ def measure_prefill(w, iters=20):
     }
 
 
-def wave_trace(w, launches=12):
+def wave_trace(w, launches=18):
     """Per-wave timeline of the split kernel (tuning builds only: ``ARENO_TRACE=1 python setup.py build_ext --inplace``
     makes the kernel stamp its waves with the 100 MHz wall clock): when waves start, have the work list, start their
-    first four tiles and finish, relative to the first wave's start, over the last launches of a warm sequence."""
+    first four tiles and finish, relative to the first wave's start, over the last launches of a warm sequence; with a
+    per-step plan and without one.  The finish times are also set against what the work list gives each unit: tile
+    steps, segments (items it holds quanta of) and 16-token quanta."""
     import ctypes
 
     import numpy as np
@@ -499,57 +501,65 @@ def wave_trace(w, launches=12):
     workspace = torch.empty(cabi.decode_workspace_bytes(b, hq, d, bs, w.block_table.shape[1]), dtype=torch.uint8, device=w.q.device)
     out = torch.empty_like(w.q)
     buf = torch.zeros(8192 * 8, dtype=torch.int64, device=w.q.device)
-    lib.areno_hip_debug_set_trace(buf.data_ptr())
-    runs = []
-    for it in range(launches):
-        buf.zero_()
-        cabi.paged_decode(cabi.describe_cache(*pools[it % len(pools)]), w.q, w.k_update, w.v_update, out, w.block_table,
-                          w.cache_seqlens, workspace, softmax_scale=w.softmax_scale, stages=cabi.STAGE_SPLIT)  # fmt: skip
-        torch.cuda.synchronize()
-        runs.append(buf.cpu().view(-1, 8).numpy().copy())
-    lib.areno_hip_debug_set_trace(None)
+    plan_buffer = torch.empty(cabi.decode_plan_bytes(b), dtype=torch.uint8, device=w.q.device)
+    plan = cabi.paged_decode_plan(cabi.describe_cache(*pools[0]), w.q.dtype, hq, w.block_table, w.cache_seqlens, plan_buffer)
+    keys = ("start", "work_list_ready", "tile0", "tile1", "tile2", "tile3", "finish")
 
     def pct(a, q):
         return float(np.percentile(a, q))
 
-    summary = []
-    for t in runs[launches // 2:]:
-        t = t[t[:, 6] != 0].astype(np.float64)
-        t0 = t[:, 0].min()
-        us = lambda col: (t[:, col] - t0) / 100.0  # noqa: E731
-        rec = {"waves": int(len(t))}
-        for name, col in (("start", 0), ("work_list_ready", 1), ("tile0", 2), ("tile1", 3), ("tile2", 4), ("tile3", 5), ("finish", 6)):
-            v = us(col)[t[:, col] != 0]
-            rec[name] = {"mean": float(v.mean()), "p10": pct(v, 10), "p50": pct(v, 50), "p90": pct(v, 90), "max": float(v.max())}
-        summary.append(rec)
-    keys = ("start", "work_list_ready", "tile0", "tile1", "tile2", "tile3", "finish")
-    mean = {k: {s: float(np.mean([r[k][s] for r in summary])) for s in ("mean", "p10", "p50", "p90", "max")} for k in keys}
-    out = {"workload": w.name, "launches_averaged": len(summary), "waves": summary[-1]["waves"], "us_since_first_wave_start": mean}
+    def timeline(use_plan):
+        lib.areno_hip_debug_set_trace(buf.data_ptr())
+        runs = []
+        for it in range(launches):
+            buf.zero_()
+            cabi.paged_decode(cabi.describe_cache(*pools[it % len(pools)]), w.q, w.k_update, w.v_update, out, w.block_table,
+                              w.cache_seqlens, workspace, softmax_scale=w.softmax_scale, stages=cabi.STAGE_SPLIT,
+                              plan=plan if use_plan else None)  # fmt: skip
+            torch.cuda.synchronize()
+            runs.append(buf.cpu().view(-1, 8).numpy().copy())
+        lib.areno_hip_debug_set_trace(None)
+        runs = runs[launches // 3:]
+        waves = int((runs[0][:, 6] != 0).sum())
+        us = {k: np.stack([(r[:waves, col] - r[:waves, 0].min()) / 100.0 for r in runs]) for col, k in enumerate(keys)}
+        table = {k: {"mean": float(v.mean()), "p10": pct(v, 10), "p50": pct(v, 50), "p90": pct(v, 90),
+                     "max": float(v.max(1).mean())} for k, v in us.items()}  # fmt: skip
+        fin = us["finish"]
+        return waves, table, fin
 
-    # Who finishes last: waves by whether a row ends in their unit (plain launches of one workgroup row, where wave i
-    # belongs to unit i // 4: the tile range [u T / U, (u + 1) T / U) of the list "cached tiles + 1 per row").
-    waves = summary[-1]["waves"]
-    if hkv <= 4 and waves % 4 == 0:
+    waves, planned, fin = timeline(True)
+    _, plain, _ = timeline(False)
+    result = {"workload": w.name, "launches_averaged": launches - launches // 3, "waves": waves,
+              "us_since_first_wave_start": {"with_plan": planned, "without_plan": plain}}  # fmt: skip
+    # the finish times of the planned launches against the units' work (plain launches of one workgroup row: wave i
+    # belongs to unit i // 4); the same arithmetic as areno_amd/csrc/decode_items.hpp
+    if hkv <= 4 and waves % 4 == 0 and w.k_scale is not None:
         lens = w.cache_seqlens.cpu().numpy().astype(np.int64)
-        cum = np.concatenate([[0], np.cumsum((lens + 31) // 32 + 1)])
+        switch, tile = 3, 32
+        quanta = (lens + 15) // 16
+        extent = np.where(quanta > 0, quanta + switch, 0)
+        cum = np.concatenate([[0], np.cumsum(extent)])
         units = waves // 4
-        starts = np.arange(units + 1) * cum[-1] // units
-        ends_in_unit = np.array([((cum[1:] > a) & (cum[1:] <= e)).sum() for a, e in zip(starts[:-1], starts[1:])])
-        has_end = ends_in_unit[np.arange(waves) // 4] > 0
-        groups = {"no_row_ends_in_unit": [], "a_row_ends_in_unit": []}
-        for t in runs[launches // 2:]:
-            t = t[:waves].astype(np.float64)
-            finish = (t[:, 6] - t[:, 0].min()) / 100.0
-            for name, sel in (("no_row_ends_in_unit", ~has_end), ("a_row_ends_in_unit", has_end)):
-                if sel.any():
-                    groups[name].append((int(sel.sum()), float(finish[sel].mean()), pct(finish[sel], 90), float(finish[sel].max())))
-        out["finish_by_row_end"] = {
-            name: {"waves": v[0][0], "mean": [min(x[1] for x in v), max(x[1] for x in v)],
-                   "p90": [min(x[2] for x in v), max(x[2] for x in v)], "max": [min(x[3] for x in v), max(x[3] for x in v)]}
-            for name, v in groups.items() if v
-        }  # fmt: skip
-        out["tiles_per_unit"] = [int((starts[1:] - starts[:-1]).min()), int((starts[1:] - starts[:-1]).max())]
-    return out
+        borders = np.arange(units + 1) * cum[-1] // units
+        steps, segments = np.zeros(units), np.zeros(units)
+        for u in range(units):
+            for v in range(len(lens)):
+                lo, hi = max(borders[u], cum[v] + switch), min(borders[u + 1], cum[v + 1])
+                if hi > lo:
+                    tokens = min(lens[v], (hi - cum[v] - switch) * 16) - (lo - cum[v] - switch) * 16
+                    steps[u] += -(-tokens // tile)
+                    segments[u] += 1
+        unit_finish = fin.mean(0).reshape(units, 4).mean(1)
+        result["finish_by_segments_in_unit"] = {
+            int(k): {"units": int((segments == k).sum()), "mean_finish_us": float(unit_finish[segments == k].mean())}
+            for k in sorted(set(segments.tolist()))
+        }
+        result["finish_by_steps_in_unit"] = {
+            int(k): {"units": int((steps == k).sum()), "mean_finish_us": float(unit_finish[steps == k].mean())}
+            for k in sorted(set(steps.tolist()))
+        }
+        result["finish_spread"] = {"std_of_unit_means_us": float(fin.mean(0).std()), "std_within_unit_over_launches_us": float(fin.std(0).mean())}
+    return result
 
 
 def cpu_baseline(w, warmups=3, repeats=7):
