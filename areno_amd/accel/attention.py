@@ -22,8 +22,10 @@ defaulting to the reference behaviour:
 
 Everything runs as HIP kernels through ``areno_amd.accel._areno_accel``; there is no Python
 fallback.  The varlen and dense ops are autograd functions with HIP backward kernels like the
-reference's; the paged ops (decode, paged prefill) are inference-only and refuse inputs that require
-gradients while gradients are being recorded, instead of returning an output without a graph.
+reference's; the decode op's backward recomputes densely, as the reference's does; the paged prefill op (this
+build's own) is inference-only and refuses inputs that require gradients while gradients are being recorded,
+instead of returning an output without a graph.  float64 tensors are accepted as in the reference, whose kernels
+read doubles and compute in fp32: the ops run on fp32 copies and cast the result back.
 """
 
 from __future__ import annotations
@@ -105,7 +107,10 @@ class _PagedDecode(torch.autograd.Function):
     path: it gathers every row's pages into one ``(batch, tokens, kv_heads, head_dim)`` tensor."""
 
     @staticmethod
-    def forward(ctx, call, q, k_cache, v_cache, k_scale, v_scale, block_table, cache_seqlens, window_left, softmax_scale):
+    def forward(ctx, call, q, k_update, v_update, k_cache, v_cache, k_scale, v_scale, block_table, cache_seqlens,
+                window_left, softmax_scale):
+        # (k_update / v_update are inputs so that an output whose only differentiable inputs are the update rows stays
+        # in the graph; their gradient is None)
         out = call()
         ctx.save_for_backward(q, k_cache, v_cache, k_scale, v_scale, block_table, cache_seqlens)
         ctx.window_left = window_left
@@ -145,7 +150,7 @@ class _PagedDecode(torch.autograd.Function):
             grads = torch.autograd.grad(out, wanted, grad_output.float())
         dq = grads[0].to(q.dtype)
         dk, dv = (None, None) if quantized else (grads[1].to(k_cache.dtype), grads[2].to(v_cache.dtype))
-        return None, dq, dk, dv, None, None, None, None, None, None
+        return None, dq, None, None, dk, dv, None, None, None, None, None, None
 
 
 def _rows_of(x: torch.Tensor) -> torch.Tensor:
@@ -198,6 +203,28 @@ class _CausalAttention(torch.autograd.Function):
 
 
 _PLAN_DTYPE_CODES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def _decode_in_double(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, window_left, num_splits,
+                      softmax_scale):
+    """float64 tensors: the reference's kernels read doubles, compute in fp32 and write doubles
+    (``AT_DISPATCH_FLOATING_TYPES_AND2`` with float accumulators, ``areno/accel/csrc/attention.cu:979`` there), so
+    the op runs on fp32 copies and the result is cast back; the update rows go into the float64 pages as they are."""
+    bs, max_blocks = k_cache.shape[1], block_table.shape[1]
+    with torch.no_grad():
+        pos = cache_seqlens.long()
+        col = torch.div(pos, bs, rounding_mode="floor")
+        ok = (pos >= 0) & (col < max_blocks)
+        blk = block_table.long().gather(1, col.clamp(0, max_blocks - 1).unsqueeze(1)).squeeze(1)
+        ok &= (blk >= 0) & (blk < k_cache.shape[0])
+        rows = ok.nonzero().squeeze(1)
+        k_cache[blk[rows], (pos - col * bs)[rows]] = k_update.detach()[rows]
+        v_cache[blk[rows], (pos - col * bs)[rows]] = v_update.detach()[rows]
+    out = areno_paged_causal_attention_decode(
+        q.float(), k_update.float(), v_update.float(), k_cache.float(), v_cache.float(), block_table, cache_seqlens,
+        window_left=window_left, num_splits=num_splits, softmax_scale=_scale(q, softmax_scale),
+    )  # fmt: skip
+    return out.double()
 
 
 @torch._dynamo.disable
@@ -301,6 +328,9 @@ def areno_paged_causal_attention_decode(
         raise ValueError(f"{op} expects contiguous cache tensors (they are updated in place)")
     if k_scale is not None and not (k_scale.is_contiguous() and v_scale.is_contiguous()):
         raise ValueError(f"{op} expects contiguous scale tensors (they are updated in place)")
+    if q.dtype == torch.float64 and k_cache.dtype == torch.float64:
+        return _decode_in_double(q, k_update, v_update, k_cache, v_cache, block_table, cache_seqlens, window_left,
+                                 num_splits, softmax_scale)  # fmt: skip
     ext = _extension()
     args = (
         q.contiguous(), k_update.contiguous(), v_update.contiguous(), k_cache, v_cache,
@@ -336,10 +366,12 @@ def areno_paged_causal_attention_decode(
         def call():
             return ext.areno_paged_causal_attention_decode_forward_scaled(*args, k_scale, v_scale, 0, None)
 
-    differentiable = (q, k_cache, v_cache) if k_scale is None else (q,)
+    # the update rows are in the graph like q and the caches (their gradient is None, as in the reference: the
+    # output reaches them only through the in-place cache write, which autograd does not see)
+    differentiable = (q, k_update, v_update, k_cache, v_cache) if k_scale is None else (q, k_update, v_update)
     if torch.is_grad_enabled() and any(t.requires_grad for t in differentiable):
-        return _PagedDecode.apply(call, q, k_cache, v_cache, k_scale, v_scale, block_table, cache_seqlens,
-                                  _window_left(window_left), _scale(q, softmax_scale))  # fmt: skip
+        return _PagedDecode.apply(call, q, k_update, v_update, k_cache, v_cache, k_scale, v_scale, block_table,
+                                  cache_seqlens, _window_left(window_left), _scale(q, softmax_scale))  # fmt: skip
     return call()
 
 
@@ -367,6 +399,10 @@ def areno_varlen_causal_attention(
         raise ValueError(f"{op} expects q heads to be divisible by kv heads")
     if q.shape[2] != k.shape[2] or q.shape[2] != v.shape[2]:
         raise ValueError(f"{op} head dim mismatch")
+    if q.dtype == torch.float64 and k.dtype == torch.float64 and v.dtype == torch.float64:
+        # the reference's kernels read doubles and compute in fp32 (attention.cu:846 there): the same through casts
+        return _VarlenCausalAttention.apply(q.float(), k.float(), v.float(), cu_seqlens, _window_left(window_left),
+                                            _scale(q, softmax_scale)).double()  # fmt: skip
     return _VarlenCausalAttention.apply(q, k, v, cu_seqlens, _window_left(window_left), _scale(q, softmax_scale))
 
 
@@ -401,6 +437,9 @@ def areno_causal_attention(
     sk = k.shape[2]
     if sk < int(query_start) + q.shape[2]:
         raise ValueError(f"{op} needs at least query_start + q_len = {int(query_start) + q.shape[2]} keys, got {sk}")
+    if q.dtype == torch.float64 and k.dtype == torch.float64 and v.dtype == torch.float64:
+        return _CausalAttention.apply(q.float(), k.float(), v.float(), int(query_start), _window_left(window_left),
+                                      _scale(q, softmax_scale)).double()  # fmt: skip
     return _CausalAttention.apply(q, k, v, int(query_start), _window_left(window_left), _scale(q, softmax_scale))
 
 

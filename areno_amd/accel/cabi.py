@@ -106,7 +106,7 @@ def lib() -> ctypes.CDLL:
         handle.areno_hip_paged_varlen_prefill.argtypes = [_P, _P, _P, _I32, _I64, _I32, _I32, _P, _I32, _P, _P, _I32, _F, _P, _SZ, _P]  # fmt: skip
         handle.areno_hip_prefill_workspace_bytes.restype = _SZ
         handle.areno_hip_prefill_workspace_bytes.argtypes = [_I32, _I32]
-        handle.areno_hip_probe_stream_read.argtypes = [_P, _P, _P, _I64, _I32, _P, _P]
+        handle.areno_hip_probe_stream_read.argtypes = [_P, _P, _P, _I64, _I32, _I32, _P, _P]
         handle.areno_hip_block_tables_init.argtypes = [_P, _P]
         handle.areno_hip_block_tables_reserve.argtypes = [_P, _P, _P, _I32, _P]
         handle.areno_hip_block_tables_ensure_decode.argtypes = [_P, _P, _P, _I32, _P]
@@ -222,13 +222,15 @@ def paged_decode_static(cache: PagedCache, q, k_update, v_update, out, block_tab
     ))  # fmt: skip
 
 
-def probe_stream_read(pool_a, pool_b, page_bytes: int, sink, page_ids=None, stream=None) -> int:
+def probe_stream_read(pool_a, pool_b, page_bytes: int, sink, page_ids=None, stream=None, prefetch_ids=False) -> int:
     """``areno_hip_probe_stream_read`` over two device tensors (K and V pool) cut into runs of ``page_bytes``: all of
-    them, in order, or the runs an int32 tensor of ids names.  Returns the bytes one call reads."""
+    them, in order, or the runs an int32 tensor of ids names (``prefetch_ids``: each wave fetches its next id a run
+    ahead).  Returns the bytes one call reads."""
     pages = (pool_a.numel() * pool_a.element_size()) // page_bytes if page_ids is None else page_ids.numel()
     check(lib().areno_hip_probe_stream_read(pool_a.data_ptr(), None if pool_b is None else pool_b.data_ptr(),
                                             None if page_ids is None else page_ids.data_ptr(), pages, page_bytes,
-                                            sink.data_ptr(), current_stream_ptr() if stream is None else stream),
+                                            1 if prefetch_ids else 0, sink.data_ptr(),
+                                            current_stream_ptr() if stream is None else stream),
           "areno_hip_probe_stream_read")  # fmt: skip
     return pages * page_bytes * (1 if pool_b is None else 2)
 

@@ -268,7 +268,9 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
             # what a reader that computes nothing reaches over the same pools (all pages in address order / the distinct
             # pages of the block table in random order), and the split kernel against the latter
             "stream_ceiling_gbps": ceiling["linear_gbps"], "stream_ceiling_paged_gbps": ceiling["paged_gbps"],
-            "frac_of_stream_ceiling": gbps / ceiling["paged_gbps"],
+            "stream_ceiling_paged_prefetch_gbps": ceiling["paged_prefetch_gbps"],
+            "stream_ceiling_paged_kv_adjacent_gbps": ceiling["paged_kv_adjacent_gbps"],
+            "frac_of_stream_ceiling": gbps / max(ceiling["paged_gbps"], ceiling["paged_prefetch_gbps"]),
         },  # fmt: skip
         "pool_copies": copies,
         "parity_max_abs_4rows": parity,
@@ -280,7 +282,11 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
 
 def measure_stream_ceiling(w, pools, iters=10, samples=9):
     """GB/s of `areno_hip_probe_stream_read` (16-byte loads, a page per wave at a time, nothing computed; one launch
-    reads a page set from the K and the V pool, as a decode launch does) over the K and V pools of all pool copies: every page in address order, and the distinct pages the block table names in a random order."""
+    reads a page set from the K and the V pool, as a decode launch does) over the K and V pools of all pool copies:
+    every page in address order (`linear`); the distinct pages the block table names in a random order, each wave
+    fetching a page's id when it gets there (`paged`) or one page ahead, as the decode kernel does
+    (`paged_prefetch`); and the same number of bytes as runs of two pages from one pool in random order
+    (`paged_kv_adjacent`: what a layout that keeps a block's K and V pages side by side would offer)."""
     import torch
 
     from areno_amd.accel import cabi
@@ -293,10 +299,15 @@ def measure_stream_ceiling(w, pools, iters=10, samples=9):
     used = torch.unique(torch.cat([table[b, : (int(lens[b]) + bs) // bs] for b in range(table.shape[0])]))
     # every page once (rows of a rollout share pages), in a fixed random order as the shuffled pools give it to the kernel
     used = used[torch.randperm(used.numel(), generator=torch.Generator().manual_seed(7))].to(torch.int32).to(w.q.device)
+    # runs of two pages inside one pool: half as many ids, drawn over the pool's page pairs
+    pairs = (used[: used.numel() // 2] // 2).contiguous()
 
-    def timed(ids):
+    def timed(ids, **kw):
         def once():
-            return sum(cabi.probe_stream_read(pool[0], pool[1], page_bytes, sink, ids) for pool in pools)
+            if kw.get("adjacent"):
+                return sum(cabi.probe_stream_read(pool[0], pool[1], 2 * page_bytes, sink, ids, prefetch_ids=True) for pool in pools)
+            return sum(cabi.probe_stream_read(pool[0], pool[1], page_bytes, sink, ids, prefetch_ids=kw.get("prefetch", False))
+                       for pool in pools)  # fmt: skip
 
         nbytes = once()
         torch.cuda.synchronize()
@@ -311,7 +322,8 @@ def measure_stream_ceiling(w, pools, iters=10, samples=9):
             out.append(e0.elapsed_time(e1) * 1e-3 / iters)
         return nbytes / statistics.median(out) / 1e9
 
-    return {"linear_gbps": timed(None), "paged_gbps": timed(used), "page_bytes": page_bytes}
+    return {"linear_gbps": timed(None), "paged_gbps": timed(used), "paged_prefetch_gbps": timed(used, prefetch=True),
+            "paged_kv_adjacent_gbps": timed(pairs, adjacent=True), "page_bytes": page_bytes}  # fmt: skip
 
 
 def measure_block_tables(w, inner=20, repeats=5):

@@ -386,23 +386,28 @@ int areno_hip_attention_backward(const void* grad_out, const void* q, const void
                                  size_t workspace_bytes, void* stream);
 
 /*
- * Test hook, no counterpart in the reference: caps the tokens one launch of areno_hip_qk_norm_rope_cache_write takes
+ * ---- Diagnostics: not part of any caller's contract -------------------------------------------------------------------
+ * The two entry points below have no counterpart in the reference and no production caller: the first exists for a
+ * test of this library, the second for its benchmark.
+ *
+ * areno_hip_debug_set_rope_tokens_per_launch: caps the tokens one launch of areno_hip_qk_norm_rope_cache_write takes
  * (0 = only the kernel's own limit) so that its walk over token ranges can be tested at small sizes.  Returns the
- * previous cap.  Process-wide; not for production callers.
- */
-int64_t areno_hip_debug_set_rope_tokens_per_launch(int64_t tokens);
-
-/*
- * Measurement aid, no counterpart in the reference: reads `pages` runs of page_bytes bytes from one pool or from two
- * (page i starts at base + page_ids[i] * page_bytes, or at base + i * page_bytes when page_ids is NULL; base_b NULL =
- * one pool) with 16-byte loads, one workgroup of four waves per CU, one page per wave at a time, and computes nothing.
- * What this reaches over the K and V pools of a workload is the streaming ceiling the decode kernels' bandwidth is
- * compared with (bench.py): same pages, same bytes per launch.
+ * previous cap.  Process-wide.
+ *
+ * areno_hip_probe_stream_read: reads `pages` runs of page_bytes bytes from one pool or from two (page i starts at
+ * base + page_ids[i] * page_bytes, or at base + i * page_bytes when page_ids is NULL; base_b NULL = one pool) and
+ * computes nothing: 512 workgroups of four waves (two per CU), a wave takes one run at a time with eight 16-byte
+ * loads per lane in flight.  prefetch_ids != 0: a wave fetches the id of its next run in front of the current run's
+ * loads (as the decode kernel fetches block ids a tile ahead) instead of when it gets there.  What this reaches over
+ * the K and V pools of a workload is the streaming ceiling the decode kernels' bandwidth is compared with (bench.py):
+ * same pages, same bytes per launch; with page_bytes doubled and one pool it reads what a layout with a block's K and
+ * V pages side by side would offer.
  *   base_a, base_b  device, 16-byte aligned;  page_bytes a multiple of 1024;  sink  device, >= 4 bytes (written
  *                   practically never)
  */
+int64_t areno_hip_debug_set_rope_tokens_per_launch(int64_t tokens);
 int areno_hip_probe_stream_read(const void* base_a, const void* base_b, const int32_t* page_ids, int64_t pages,
-                                int32_t page_bytes, void* sink, void* stream);
+                                int32_t page_bytes, int32_t prefetch_ids, void* sink, void* stream);
 
 #ifdef __cplusplus
 }

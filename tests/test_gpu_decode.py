@@ -190,6 +190,39 @@ def test_error_behaviour_matches_the_reference_shim():
     assert ops.areno_paged_causal_attention_decode(q_grad, *args[1:]).requires_grad
     with torch.no_grad():
         assert not ops.areno_paged_causal_attention_decode(q_grad, *args[1:]).requires_grad
+    # update rows that require grad keep the output in the graph; their gradient is None, as in the reference
+    ku = w.k_update.clone().requires_grad_(True)
+    out = ops.areno_paged_causal_attention_decode(w.q, ku, *args[2:])
+    assert out.requires_grad
+    out.float().sum().backward()
+    assert ku.grad is None
+
+
+def test_float64_tensors_compute_in_fp32_like_the_reference():
+    """The reference's launchers take double tensors and accumulate in float (attention.cu:846,979 there)."""
+    w = workloads.cfg0_tiny("fp32", device=DEV, poison=True, act_dtype=torch.float32)
+    q, ku, vu = w.q.double(), w.k_update.double() + 1e-12, w.v_update.double() - 1e-12
+    kc, vc = w.k_cache.double(), w.v_cache.double()
+    out = ops.areno_paged_causal_attention_decode(q, ku, vu, kc, vc, w.block_table, w.cache_seqlens,
+                                                  softmax_scale=w.softmax_scale)  # fmt: skip
+    assert out.dtype == torch.float64
+    ids, offs = qr.decode_addresses(w.block_table.cpu(), w.cache_seqlens.cpu(), w.k_cache.shape[1])
+    assert torch.equal(kc.cpu()[ids, offs], ku.cpu()) and torch.equal(vc.cpu()[ids, offs], vu.cpu())  # the doubles as they are
+    w.k_cache, w.v_cache = kc.float(), vc.float()
+    assert_close(out, expected_decode(w), 1e-4, what="float64 decode")
+    # varlen and dense ops
+    g = torch.Generator(device=DEV).manual_seed(3)
+    qv = torch.randn(40, 4, 64, generator=g, device=DEV, dtype=torch.float64)
+    kv = torch.randn(40, 2, 64, generator=g, device=DEV, dtype=torch.float64)
+    vv = torch.randn(40, 2, 64, generator=g, device=DEV, dtype=torch.float64)
+    cu = torch.tensor([0, 7, 40], dtype=torch.int32, device=DEV)
+    got = ops.areno_varlen_causal_attention(qv, kv, vv, cu)
+    want = ops.areno_varlen_causal_attention(qv.float(), kv.float(), vv.float(), cu)
+    assert got.dtype == torch.float64 and torch.equal(got.float(), want)
+    qd = qv[:32].view(2, 16, 4, 64).transpose(1, 2).contiguous()
+    kd = kv[:32].view(2, 16, 2, 64).transpose(1, 2).repeat_interleave(2, dim=1).contiguous()
+    got = ops.areno_causal_attention(qd, kd, kd)
+    assert got.dtype == torch.float64 and torch.equal(got.float(), ops.areno_causal_attention(qd.float(), kd.float(), kd.float()))
 
 
 # ---- prefix groups: shared pages read once for several rows --------------------------------------------------------

@@ -75,3 +75,38 @@ def test_static_scratch_decode_refuses_shapes_beyond_its_buffer():
     assert "built-in buffer holds 67108864" in message and "areno_hip_paged_decode" in message
     torch.cuda.synchronize()
     assert torch.equal(before, w.k_cache)
+
+
+def test_static_scratch_decode_allocates_nothing_and_replays_from_a_graph():
+    """What the entry point exists for: no device memory is allocated by a call (free bytes unchanged), and it can be
+    recorded into a HIP graph; every replay must give the eager result."""
+    w = workloads.cfg0_tiny("int8", device=DEV, quantize_fn=gpu_quantize)
+    cache = cabi.describe_cache(w.k_cache, w.v_cache, w.k_scale, w.v_scale)
+    out = torch.empty_like(w.q)
+
+    def call(stream=None):
+        return cabi.paged_decode_static(cache, w.q, w.k_update, w.v_update, out, w.block_table, w.cache_seqlens,
+                                        softmax_scale=w.softmax_scale, stream=stream)  # fmt: skip
+
+    cabi.check(call(), "warm call")  # the first call on a device looks the buffer's address up
+    torch.cuda.synchronize()
+    eager = out.clone()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        cabi.check(call(), "static call")
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "a static call changed the device's free memory"
+    assert torch.equal(out, eager)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        cabi.check(call(torch.cuda.current_stream().cuda_stream), "static call under capture")
+    for replay in range(3):
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {replay} differs from the eager call"
+        cabi.check(call(), "eager call between replays")  # the program's own work between the replays
+        torch.cuda.synchronize()
