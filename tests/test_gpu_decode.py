@@ -402,3 +402,31 @@ def test_one_plan_serves_the_layers_of_a_step():
             softmax_scale=w.softmax_scale, k_scale=w.k_scale, v_scale=w.v_scale, plan=plan)  # fmt: skip
         assert torch.equal(with_plan, plain)
         assert_close(with_plan, expected_decode(w), *tolerances("fp8"), what="layer through the shared plan")
+
+
+@pytest.mark.parametrize("kv", ["bf16", "int8"])
+def test_a_row_at_the_end_of_its_block_table_writes_nothing(kv):
+    """A row whose length equals the table's capacity (no column for the next position: the page bookkeeping reports
+    it as full) must not have its new token stored anywhere -- the cache writer skips such rows -- and no kernel may
+    read a column behind the table; the other rows decode as usual."""
+    bs, cols = 16, 6
+    lengths = torch.tensor([cols * bs, 40, cols * bs, 7])
+    w = workloads.make_decode_workload("full-rows", seed=91, batch=4, hq=8, hkv=2, d=128, bs=bs, kv=kv, lengths=lengths,
+                                       device=DEV, quantize_fn=gpu_quantize, poison=True)  # fmt: skip
+    w.block_table = w.block_table[:, :cols].contiguous()  # rows 0 and 2 fill their six columns
+    before = _snapshot(w)
+    for planned in (False, True):
+        out = run_decode(w, planned=planned)
+        torch.cuda.synchronize()
+        assert torch.isfinite(out.float()).all()
+        live = [1, 3]
+        ids, offs = qr.decode_addresses(w.block_table[live].cpu(), w.cache_seqlens[live].cpu(), bs)
+        touched = torch.zeros(w.k_cache.shape[:2], dtype=torch.bool)
+        touched[ids, offs] = True
+        for name, old in zip(("k_cache", "v_cache", "k_scale", "v_scale"), before):
+            if old is None:
+                continue
+            new = getattr(w, name).cpu()
+            same = new.view(torch.uint8)[~touched] == old.view(torch.uint8)[~touched]
+            assert same.all(), f"{name}: a slot other than the two served rows' targets changed"
+        assert_close(out[live], expected_decode(w, rows=live), *tolerances(kv), what=f"served rows, planned={planned}")
