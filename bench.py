@@ -1,16 +1,19 @@
 """Benchmark of the paged decode-attention hot path on one MI355X.
 
-A step is one call of the decode op (fused cache append + split-KV GQA attention + merge) for one layer over
-one batch of synthetic sequences.  The headline workload is the Qwen2.5-7B-like shape (B=64, 28 q heads /
+A step is one call of the decode op (split-KV GQA attention, then the merge launch that also appends the new token)
+for one layer over one batch of synthetic sequences.  The headline workload is the Qwen2.5-7B-like shape (B=64, 28 q heads /
 4 kv heads, D=128, page 16, contexts uniform in [512, 4096]) with an int8 KV cache (quantizing append included), the
 configuration the bandwidth target is stated on; the same shape with a bf16 cache, the fp8 rollout shape and the fp8
 prefill shape are measured too and reported under "workloads".  Inputs are resident in HBM before timing starts.  Steps rotate over several copies of the KV
 pools so that the working set exceeds the 256 MB Infinity Cache and the reads really come from HBM.
 
-Prints ONE JSON line.  `value` is microseconds per step measured over exactly `--steps` steps replayed from
-HIP graphs (how the engine runs decode); `roofline` is for the split-KV kernel alone: algorithmic bytes of one
-launch divided by its mean duration measured with events on the launch stream, next to what a plain reader of the
-same pools reaches (`stream_ceiling_gbps`); `cpu_baseline` is the CPU oracle timed on the host cores.
+Prints ONE JSON line.  `value` is microseconds per step: the median of 15 timings of exactly `--steps` steps replayed
+from HIP graphs (how the engine runs decode), `value_p10_p90` their spread.  The steps run as an engine runs the
+layers of a model: block table and lengths are the same for every layer of a decode step, so one plan launch
+(`areno_hip_paged_decode_plan`) serves 28 steps; it is part of the timed sequence.  `value_without_plan` is the same
+sequence with every step deriving its work list by itself.  `roofline` is for the split-KV kernel alone: algorithmic
+bytes of one launch divided by its mean duration measured with events on the launch stream, next to what a plain reader
+of the same pools reaches (`stream_ceiling_*`); `cpu_baseline` is the CPU oracle timed on the host cores.
 """
 
 from __future__ import annotations
@@ -104,13 +107,14 @@ def _parity_sample(w, out, rows=4):
     return float((out[:rows].cpu().float() - want).abs().max())
 
 
-def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repeats=15):
+def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repeats=15, plan_mode="both"):
     """Time the whole op (graph replay and eager) and each kernel of it; returns a dict of numbers.
 
     A step is one layer's decode op.  The layers of a model's decode step share block table and lengths, so the timed
     sequence is what an engine runs: one plan launch, then LAYERS_PER_PLAN ops that use it, each on another layer's
     pools, replayed from HIP graphs; the plan launch is inside the timed region and its cost is spread over the steps
-    it serves.  The same sequence without plans is timed next to it."""
+    it serves.  The same sequence without plans is timed next to it (`plan_mode` "only" / "off" leave one of the two
+    out, so that a profiler's per-kernel averages belong to one of them)."""
     import torch
 
     from areno_amd.accel import cabi
@@ -124,6 +128,7 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
     torch.cuda.synchronize()
     parity = _parity_sample(w, out)
     planned_equal = bool(torch.equal(_step(w, pools[0], _plan(w, pools[0])), out))
+    plan_mode = plan_mode if plan_mode in ("both", "only", "off") else "both"
 
     # ---- whole op, replayed from HIP graphs ---------------------------------------------------------------------------
     side = torch.cuda.Stream()
@@ -171,14 +176,16 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
         # graph replays must reproduce the eager result (checked on the first pool)
         return statistics.median(samples), [samples[len(samples) // 10], samples[(len(samples) * 9) // 10]], bool(torch.equal(keep_full[0], out))
 
-    us_graph, us_graph_spread, graph_ok = timed_replays(True)
-    us_graph_plain, us_graph_plain_spread, graph_plain_ok = timed_replays(False)
+    with_plan, without_plan = plan_mode != "off", plan_mode != "only"
+    nan = float("nan")
+    us_graph, us_graph_spread, graph_ok = timed_replays(True) if with_plan else (nan, [nan, nan], True)
+    us_graph_plain, us_graph_plain_spread, graph_plain_ok = timed_replays(False) if without_plan else (nan, [nan, nan], True)
 
     # ---- whole op, eager launches (host launch overhead included), a plan per LAYERS_PER_PLAN steps ------------------
     def eager(n):
         plan = None
         for i in range(n):
-            if i % LAYERS_PER_PLAN == 0:
+            if with_plan and i % LAYERS_PER_PLAN == 0:
                 plan = _plan(w, pools[i % copies], plan_buffer)
             _step(w, pools[i % copies], plan)
 
@@ -231,13 +238,15 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
 
         return time_launches(launch, name)
 
-    plan = build_plan()
+    plan = build_plan() if with_plan else None
     # the op folds the append into the merge launch; the stand-alone append launch is timed for reference only
-    us_split_plain = time_stage(cabi.STAGE_SPLIT, None, "split_plain")
-    us_split = time_stage(cabi.STAGE_SPLIT, plan, "split")
+    us_split_plain = time_stage(cabi.STAGE_SPLIT, None, "split_plain") if without_plan else nan
+    us_split = time_stage(cabi.STAGE_SPLIT, plan, "split") if with_plan else nan
     us_reduce = time_stage(cabi.STAGE_APPEND | cabi.STAGE_REDUCE, plan, "merge")
     us_append = time_stage(cabi.STAGE_APPEND, None, "append")
-    us_plan = time_launches(lambda i: build_plan(), "plan")
+    us_plan = time_launches(lambda i: build_plan(), "plan") if with_plan else nan
+    if not with_plan:  # a run without plans reports the plain figures in the headline fields
+        us_graph, us_graph_spread, us_split, spread["split"] = us_graph_plain, us_graph_plain_spread, us_split_plain, spread["split_plain"]
     torch.cuda.synchronize()
     assert torch.equal(out2, out), "C-ABI staged run disagrees with the op"
 
@@ -256,7 +265,7 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
                       "append_alone_not_in_op": us_append, "plan": us_plan},
         # 10th / 90th percentile of the kernels' samples (each the mean of back-to-back launches)
         "split_us_p10_p90": spread["split"],
-        "split_without_plan_us_p10_p90": spread["split_plain"],
+        "split_without_plan_us_p10_p90": spread.get("split_plain"),
         "tokens_per_s": w.q.shape[0] / (us_graph * 1e-6),
         "algorithmic_bytes": alg_bytes,
         "op_gbps": alg_bytes / (us_graph * 1e-6) / 1e9,
@@ -617,6 +626,9 @@ def main() -> int:
     ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg2_b256"], default=None,
                     help="measure a single workload")  # fmt: skip
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--plan", choices=["both", "only", "off"], default="both",
+                    help="decode workloads: time the steps with a per-step plan and without one (both), or only one of the "
+                         "two (for profiler runs whose per-kernel averages should belong to one of them)")  # fmt: skip
     ap.add_argument("--wave-trace", choices=["cfg1", "cfg2", "cfg3"], default=None,
                     help="print the split kernel's per-wave timeline for a workload (needs an ARENO_TRACE=1 build) and exit")  # fmt: skip
     args = ap.parse_args()
@@ -657,7 +669,7 @@ def main() -> int:
     baseline = None
     for name in names:
         w = builders[name]()
-        results[name] = measure_prefill(w) if name == "cfg4" else measure_decode(w, args.steps, args.warmup)
+        results[name] = measure_prefill(w) if name == "cfg4" else measure_decode(w, args.steps, args.warmup, plan_mode=args.plan)
         if name == names[0] and not args.no_cpu and name != "cfg4":
             baseline = cpu_baseline(w)
         del w
@@ -682,7 +694,11 @@ def main() -> int:
             "workload": head["workload"],
             "shape": "B=64 Hq=28 Hkv=4 D=128 page=16 ctx~U[512,4096]" if names[0] != "cfg3" else "B=256 Hq=32 Hkv=8 D=128",
             "launch": "HIP graph replay, KV pools rotated over >1.3 GB",
+            "step": "one layer's decode op (split + merge launch); per-step plan: one plan launch per "
+                    f"{LAYERS_PER_PLAN} steps, inside the timed region" if "plan" in head else "one paged prefill",
         },
+        "value_p10_p90": head.get("us_per_step_p10_p90"),
+        "value_without_plan": head.get("us_per_step_without_plan"),
         "tokens_per_s": head["tokens_per_s"],
         "hbm_gbps_op": head.get("op_gbps"),
         "roofline": head["roofline"],
