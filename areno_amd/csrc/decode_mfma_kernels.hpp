@@ -10,8 +10,8 @@
 // Work decomposition (decode_items.hpp; balanced to within 16 tokens, no host knowledge of the lengths):
 //   * a sequence contributes ceil(visible cached keys / 16) quanta; the quanta of all sequences are cut into equal
 //     ranges, one "unit" per wave, so all waves stream the same number of bytes whatever the length distribution;
-//     a wave walks its unit in tile steps of TK tokens (32 for 16-bit pages, 64 for 8-bit pages: 16 KB in flight
-//     per wave either way), the last step of a segment masked;
+//     a wave walks its unit in tile steps of TK tokens (32; the step is generic in TK, and 64-token steps for 8-bit
+//     pages, 16 KB in flight per wave like a 16-bit tile, measured slower), the last step of a segment masked;
 //   * the list of items (first token, end, row) and the prefix sums of their quanta live in LDS: every workgroup
 //     computes them from the sequence lengths, or copies them from a plan that areno_hip_paged_decode_plan left in
 //     device memory once for all layers of a step; with a plan a wave finds its unit's first tile (item, token, block
@@ -77,7 +77,7 @@ namespace areno {
 #ifndef ARENO_MFMA_WIDE_OCC
 #define ARENO_MFMA_WIDE_OCC 2
 #endif
-// tokens per tile step: a wave keeps one tile (K and V) in flight, 16 KB at head dim 128 with either setting
+// tokens per tile step: a wave keeps one tile (K and V) in flight, 8 KB (8-bit) / 16 KB (16-bit) at head dim 128
 #ifndef ARENO_MFMA_QUANT_TK
 #define ARENO_MFMA_QUANT_TK 32
 #endif

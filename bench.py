@@ -34,8 +34,8 @@ POOL_TARGET_BYTES = 1.3e9  # rotate over at least this much distinct KV
 # HBM bytes per launch of the dominant kernel as two rocprofv3 counter runs of this script recorded them (FETCH_SIZE,
 # scaled by the factor 2.0 that a copy of known size gives for it, plus WRITE_SIZE).  Recorded constants, not
 # measurements of the present run: the summaries they come from are under profiles/.
-PROFILED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 310.91e6, "cfg2-qwen7b-int8": 153.71e6, "cfg3-rollout-fp8": 1065.34e6,
-                          "cfg4-prefill-fp8": 1624.88e6}
+PROFILED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 311.02e6, "cfg2-qwen7b-int8": 153.95e6, "cfg3-rollout-fp8": 1066.22e6,
+                          "cfg4-prefill-fp8": 1624.94e6}
 PROFILED_TRAFFIC_SOURCE = {
     "decode": "recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script: profiles/decode_mfma_kernel_hbm_traffic_cfg1_cfg2_cfg3.md",
     "prefill": "recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script: profiles/prefill_mfma_kernel_hbm_traffic_cfg4.md",
@@ -250,6 +250,8 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
     torch.cuda.synchronize()
     assert torch.equal(out2, out), "C-ABI staged run disagrees with the op"
 
+    if not with_plan:  # a run without plans reports the plain launches as the step and as the kernel
+        us_graph, us_graph_spread, us_split = us_graph_plain, us_graph_plain_spread, us_split_plain
     gbps = alg_bytes / (us_split * 1e-6) / 1e9
     ceiling = measure_stream_ceiling(w, pools)
     return {
@@ -618,6 +620,15 @@ def cpu_baseline(w, warmups=3, repeats=7):
     }  # fmt: skip
 
 
+def _without_nan(x):
+    """Figures a run did not measure (`--plan only` / `off`) as null instead of NaN, which JSON has no literal for."""
+    if isinstance(x, dict):
+        return {k: _without_nan(v) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [_without_nan(v) for v in x]
+    return None if isinstance(x, float) and x != x else x
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--gpus", type=int, default=1)
@@ -706,7 +717,7 @@ def main() -> int:
         "workloads": results,
         "device": torch.cuda.get_device_name(0),
     }
-    print(json.dumps(line))
+    print(json.dumps(_without_nan(line)))
     return 0
 
 

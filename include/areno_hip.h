@@ -100,6 +100,11 @@ size_t areno_hip_paged_decode_workspace_bytes(int32_t batch, int32_t q_heads, in
  *   2. split-KV pass over keys [first_allowed, L_b], first_allowed = max(0, L_b - window_left) when
  *      window_left >= 0 else 0; query head h reads kv head h / (q_heads / kv_heads);
  *   3. log-sum-exp merge of the partials, normalise, cast to q_dtype.
+ * Same results as those three steps in that order; the launches are two on the matrix-core path: the split pass
+ * reads the cached keys [first_allowed, L_b), and the merge launch quantizes the update rows, writes them into
+ * their page slots and folds key L_b into the result from the update rows' stored values (what a reader of the page
+ * would see).  The other kernels, and 16-bit pages of another dtype than the query's, append in a launch in front.
+ * k_update / v_update must not alias the pages they are written to.
  *   q, out        device [batch, q_heads, head_dim], q_dtype (F16/BF16; F32 with an F32 cache)
  *   workspace     device, at least areno_hip_paged_decode_workspace_bytes(...) bytes, 256-byte aligned
  */
@@ -112,8 +117,11 @@ int areno_hip_paged_decode(const areno_paged_cache* cache, const void* q, const 
  * The same op with a stage mask, for profilers and benchmarks that time one kernel at a time:
  * ARENO_STAGE_APPEND (cache write of the update rows), ARENO_STAGE_SPLIT (split-KV pass into the workspace),
  * ARENO_STAGE_REDUCE (merge of the workspace partials into `out`).  areno_hip_paged_decode is
- * stages = ARENO_STAGE_ALL.  No counterpart in the reference, whose launcher always runs its three
- * kernels (areno/accel/csrc/attention.cu:979-1018).
+ * stages = ARENO_STAGE_ALL.  On the matrix-core path the merge launch is the one that appends: REDUCE with APPEND
+ * writes the update rows and counts their key, REDUCE without APPEND counts the key from the update rows and leaves
+ * the pages alone (for timing loops that replay a step on an unchanged cache), APPEND without REDUCE runs the
+ * stand-alone cache write.  No counterpart in the reference, whose launcher always runs its three kernels
+ * (areno/accel/csrc/attention.cu:979-1018).
  */
 #define ARENO_STAGE_APPEND 1
 #define ARENO_STAGE_SPLIT 2
