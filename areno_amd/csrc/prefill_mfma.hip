@@ -4,7 +4,7 @@
 // query-row axis: row r of the block is (token r / GP, head r % GP) with GP = G rounded up to a power of two, so one
 // 16-row MFMA tile holds 16 / GP tokens of all heads and K/V are read once for the whole group (GQA without
 // expanding KV, as areno/accel/csrc/attention.cu:170-171 does per row).  A block is 256 rows: each of the 8 waves
-// owns 32 (two 16-row tiles).  One such workgroup per CU (the registers allow two waves per SIMD either way; eight
+// owns 32 (two 16-row tiles; one at head dims 192 and 256, and at 512 two waves share one).  One such workgroup per CU (the registers allow two waves per SIMD either way; eight
 // waves behind one set of K/V tiles halve the staging work per wave against two workgroups of four).
 //
 // Balance: an item costs one "tile step" per 32-key tile it may see, and items differ by orders of magnitude (a
@@ -230,11 +230,15 @@ __device__ __forceinline__ void dequant_chunk(uint4_t codes, float scale, uint4_
   hi = uint4_t{out[4], out[5], out[6], out[7]};
 }
 
-template <int KIND, int D, bool SCALE16, int RT>
+// DS > 1 (head dim 512): DS adjacent waves share a row tile, each with D / DS of the head's elements -- its part of
+// K . Q^T, which the waves of the tile exchange through LDS and add in the same order, and its columns of O.
+template <int KIND, int D, bool SCALE16, int RT, int DS = 1>
 __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) void prefill_mfma_kernel(PrefillParams p) {
+  static_assert(DS == 1 || RT == 1, "a split head has one row tile per wave group");
   constexpr int kRowTiles = RT;
-  constexpr int kRowsPerWave = 16 * RT;
-  constexpr int kRowsPerWg = kRowsPerWave * kPrefillWaves;
+  constexpr int kRowsPerWave = 16 * RT;  // rows of one wave (DS = 1) or of the DS waves that share them
+  constexpr int kRowsPerWg = kRowsPerWave * kPrefillWaves / DS;
+  constexpr int DW = D / DS;  // head-dim elements one wave multiplies and accumulates
   using T = KVTraits<KIND>;
   // The tiles in LDS are 16-bit whatever the cache holds: 8-bit codes are dequantized (times the per-token scale)
   // once, by the thread that stages them, instead of by every wave that reads them.
@@ -250,18 +254,23 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
   constexpr int NLD = (CHUNKS + kPrefillThreads - 1) / kPrefillThreads;  // loads per thread per tensor per tile
   constexpr int RSK = D * 2 + 16;
   constexpr int RSV = 2 * D + 32;
-  constexpr int NS = D / 32;
-  constexpr int NB = D / 16;
+  constexpr int NS = DW / 32;
+  constexpr int NB = DW / 16;
   typedef typename std::conditional<SCALE16, uint16_t, float>::type scale_raw_t;
 
   __shared__ __attribute__((aligned(16))) char s_k[2][TK * RSK];
   __shared__ __attribute__((aligned(16))) char s_v[2][TK * RSV];
   __shared__ int s_cum[kMaxPrefillSeqs + 1];
   __shared__ int s_wave_tot[kPrefillWaves];
+  // score parts of a split head: [wave][tg][j][lane]
+  __shared__ float s_part[DS > 1 ? kPrefillWaves : 1][2][4][DS > 1 ? kWave : 1];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lets the tile-level decisions stay scalar
+  const int row_wave = wave / DS;  // which rows of the block the wave works on
+  const int dpart = wave % DS;     // which part of the head dim
+  const int d0 = dpart * DW;
   const int lr = lane & 15;
   const int lk = lane >> 4;
   const int kvh = blockIdx.y;
@@ -327,7 +336,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
     V8 qop[kRowTiles][NS];
 #pragma unroll
     for (int nq = 0; nq < kRowTiles; ++nq) {
-      const int r = wave * kRowsPerWave + 16 * nq + lr;
+      const int r = row_wave * kRowsPerWave + 16 * nq + lr;
       const int t = r >> p.group_shift;
       const int hh = r & (p.group_pad - 1);
       const bool live = t < tok_cnt && hh < p.group;
@@ -336,7 +345,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
 #pragma unroll
       for (int sl = 0; sl < NS; ++sl) {
         uint4_t w = {0u, 0u, 0u, 0u};
-        if (live) w = load16(p.q, (row_elem[nq] + (D / 4) * lk + 8 * sl) * 2);
+        if (live) w = load16(p.q, (row_elem[nq] + d0 + (DW / 4) * lk + 8 * sl) * 2);
         if (!q_is_operand_type) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
@@ -356,9 +365,9 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
       }
     }
     // rows of this wave: which query positions they span (wave-uniform), for skipping the mask on interior tiles
-    const bool wave_live = wave * kRowsPerWave < (tok_cnt << p.group_shift);
-    const int wave_qmin = ctx + tok0 + ((wave * kRowsPerWave) >> p.group_shift);
-    const int wave_qmax = ctx + tok0 + min(tok_cnt - 1, ((wave + 1) * kRowsPerWave - 1) >> p.group_shift);
+    const bool wave_live = row_wave * kRowsPerWave < (tok_cnt << p.group_shift);
+    const int wave_qmin = ctx + tok0 + ((row_wave * kRowsPerWave) >> p.group_shift);
+    const int wave_qmax = ctx + tok0 + min(tok_cnt - 1, ((row_wave + 1) * kRowsPerWave - 1) >> p.group_shift);
 
     float4_t acc[kRowTiles][NB];
     // Row sums of the probabilities come from the matrix cores as well: one more product per key tile with an
@@ -525,7 +534,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
       const char* kt = s_k[tile & 1];
 #pragma unroll
       for (int tg = 0; tg < 2; ++tg) {
-        const char* krow = kt + (16 * tg + lr) * RSK + (D / 4) * 2 * lk;
+        const char* krow = kt + (16 * tg + lr) * RSK + (d0 + (DW / 4) * lk) * 2;
         V8 kop[NS];
 #pragma unroll
         for (int sl = 0; sl < NS; ++sl) kop[sl] = *reinterpret_cast<const V8*>(krow + 16 * sl);
@@ -548,7 +557,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
       stage(t + 1, set_b, set_a);
     }
     __syncthreads();
-    if (wave_live) scores(ta, s_cur);
+    if (DS == 1 && wave_live) scores(ta, s_cur);
 
     // ---- iteration t: staging first, then the scores of tile t + 1 go to the matrix cores in the same block as the row
     // maxima of tile t ---------------------------------------------------------------------------------------------------
@@ -559,7 +568,37 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
     auto tile_step = [&](int t, float (&s_cur)[kRowTiles][2][4], float (&s_next)[kRowTiles][2][4], FetchSet& mine,
                          FetchSet& other) {
       __syncthreads();
-      stage(t, mine, other);
+      if constexpr (DS == 1) stage(t, mine, other);
+      if constexpr (DS > 1) {
+        // A split head computes the scores of tile t here (K[t] was published two steps ago), hands its part to the
+        // other waves of its rows and adds all parts in index order, so that those waves go on with identical scores.
+        // The staging step, which overwrites K[t] with K[t + 2], comes behind the second barrier, when every wave has
+        // read K[t]; the parts are read before the next step's barrier, which is what lets one buffer do.  (No
+        // overlap of these products with the previous tile's softmax, and a second barrier per tile: the price of
+        // the wide head.)
+        if (wave_live) {
+          scores(t, s_cur);
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s_part[wave][tg][j][lane] = s_cur[0][tg][j];
+          }
+        }
+        __syncthreads();
+        stage(t, mine, other);
+        if (wave_live) {
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              float sum = s_part[row_wave * DS][tg][j][lane];
+#pragma unroll
+              for (int part = 1; part < DS; ++part) sum += s_part[row_wave * DS + part][tg][j][lane];
+              s_cur[0][tg][j] = sum;
+            }
+          }
+        }
+      }
       if (!wave_live) return;
       const int k0 = t * TK;
       const bool need_mask = k0 + TK - 1 > wave_qmin || (p.window_left >= 0 && k0 < wave_qmax - p.window_left);
@@ -588,7 +627,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
           }
         }
       }
-      scores(t + 1, s_next);  // past tb this reads a buffer of clamped or stale keys; the result is dropped
+      if constexpr (DS == 1) scores(t + 1, s_next);  // past tb this reads a buffer of clamped or stale keys; the result is dropped
       // -- online softmax in the log2 domain; the (positive) softmax scale is applied to the row maximum and inside
       // the exponent's multiply-add -----------------------------------------------------------------------------------
       // The reference value m of a row only has to be the same for all its keys and to bound the scores well enough
@@ -660,7 +699,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
           const int tok = 16 * half + 4 * lk + r4;
-          char* a = vt + v_row_of(tok) * RSV + (16 * nb + 4 * (lr & 3)) * 2;
+          char* a = vt + v_row_of(tok) * RSV + (d0 + 16 * nb + 4 * (lr & 3)) * 2;
           const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
           const uint2_t u = __builtin_bit_cast(uint2_t, r);
           vw[2 * half] = u[0];
@@ -687,7 +726,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
         const float inv = 1.0f / l_tot;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-          const int64_t e0 = row_elem[nq] + 16 * nb + 4 * lk;
+          const int64_t e0 = row_elem[nq] + d0 + 16 * nb + 4 * lk;
           uint32_t lo, hi;
           const float o0 = acc[nq][nb][0] * inv, o1 = acc[nq][nb][1] * inv;
           const float o2 = acc[nq][nb][2] * inv, o3 = acc[nq][nb][3] * inv;
@@ -701,12 +740,12 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
           *reinterpret_cast<uint2_t*>(static_cast<char*>(p.out) + e0 * 2) = uint2_t{lo, hi};
         }
       } else {
-        const int r = wave * kRowsPerWave + 16 * nq + lr;
+        const int r = row_wave * kRowsPerWave + 16 * nq + lr;
         const int64_t prow = (static_cast<int64_t>(slot) * p.kv_heads + kvh) * kRowsPerWg + r;
-        float* dst = p.part_acc + prow * D + 4 * lk;
+        float* dst = p.part_acc + prow * D + d0 + 4 * lk;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) *reinterpret_cast<float4_t*>(dst + 16 * nb) = acc[nq][nb];
-        if (lk == 0) {
+        if (lk == 0 && dpart == 0) {
           p.part_ml[prow * 2] = m_run[nq];
           p.part_ml[prow * 2 + 1] = l_tot;
         }
@@ -857,13 +896,22 @@ prefill_fn prefill_lookup_rt(int head_dim, bool scale16) {
       }
       return prefill_mfma_kernel<KIND, 192, false, 1>;
     }
+    if (head_dim == 512) {
+      if constexpr (kQuant) {
+        if (scale16) return prefill_mfma_kernel<KIND, 512, true, 1, 2>;
+      }
+      return prefill_mfma_kernel<KIND, 512, false, 1, 2>;
+    }
   }
   return nullptr;
 }
 
 // 16-row tiles per wave: two up to head dim 128 (four need more registers than a wave has), one at head dims 192 and
-// 256, where the accumulators and the Q operands of one tile take the registers two take at 128.
+// 256, where the accumulators and the Q operands of one tile take the registers two take at 128; at 512 two waves
+// share a tile, 256 elements each.
 int prefill_row_tiles(int head_dim) { return head_dim > 128 ? 1 : 2; }
+int prefill_head_split(int head_dim) { return head_dim > 256 ? 2 : 1; }
+int prefill_rows_per_wg(int head_dim) { return 16 * prefill_row_tiles(head_dim) * kPrefillWaves / prefill_head_split(head_dim); }
 
 template <int KIND>
 prefill_fn prefill_lookup(int head_dim, bool scale16, int row_tiles) {
@@ -894,7 +942,7 @@ size_t prefill_mfma_workspace_bytes(int32_t kv_heads, int32_t head_dim) {
   if (kv_heads <= 0 || head_dim <= 0) return 0;
   const int units = prefill_units(kv_heads);
   return prefill_ml_bytes(units, kv_heads) +
-         static_cast<size_t>(2) * units * kv_heads * kMaxRowsPerWg * head_dim * sizeof(float);
+         static_cast<size_t>(2) * units * kv_heads * prefill_rows_per_wg(head_dim) * head_dim * sizeof(float);
 }
 
 // block_table == nullptr selects packed K/V: cache->k / cache->v then point at (tokens, kv_heads, D) tensors and
@@ -917,7 +965,7 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
     return ARENO_ERR_UNSUPPORTED;
   const bool scale16 = cache->scale_dtype == ARENO_DT_F16;
   const int row_tiles = prefill_row_tiles(cache->head_dim);
-  const int rows_per_wg = 16 * row_tiles * kPrefillWaves;
+  const int rows_per_wg = prefill_rows_per_wg(cache->head_dim);
   prefill_fn fn = nullptr;
   switch (cache->cache_dtype) {
     case ARENO_DT_BF16: fn = prefill_lookup<KV_BF16>(cache->head_dim, scale16, row_tiles); break;

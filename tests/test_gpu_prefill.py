@@ -22,7 +22,7 @@ def _packed(lens, hq, hkv, d, dtype, seed=0):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("window_left", [None, 0, 7])
-@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (28, 4, 128), (4, 4, 80), (8, 2, 256), (6, 6, 192)])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (28, 4, 128), (4, 4, 80), (8, 2, 256), (6, 6, 192), (8, 2, 512)])
 def test_varlen_new_tokens_only(dtype, window_left, hq, hkv, d):
     q, k, v, cu = _packed([5, 1, 130, 0, 67], hq, hkv, d, dtype)
     out = ops.areno_varlen_causal_attention(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), window_left=window_left)
@@ -32,7 +32,7 @@ def test_varlen_new_tokens_only(dtype, window_left, hq, hkv, d):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("d", [64, 128, 192, 256])
+@pytest.mark.parametrize("d", [64, 128, 192, 256, 512])
 @pytest.mark.parametrize("profile", ["climb", "jump", "fall", "wide"])
 def test_varlen_score_ranges_that_move_along_the_keys(dtype, d, profile):
     """The matrix-core kernel keeps a softmax reference value per row that it raises only when a key tile exceeds it
@@ -92,11 +92,12 @@ def test_paged_prefill_shapes(hq, hkv, d, bs):
 
 
 @pytest.mark.parametrize("kv", ["bf16", "fp16", "int8", "fp8"])
-@pytest.mark.parametrize("d", [256, 192])
+@pytest.mark.parametrize("d", [256, 192, 512])
 @pytest.mark.parametrize("hq,hkv,window_left", [(16, 8, None), (8, 1, 40), (12, 4, None)])
-def test_paged_prefill_head_dims_192_256(kv, d, hq, hkv, window_left):
-    """Head dims 256 (the sliding-attention layers of the Gemma family, Qwen3.5) and 192 (128 + 64 rotary channels of
-    the MLA-style layers) on the matrix-core kernel: one 16-row tile per wave; a query block cut by many shares goes
+def test_paged_prefill_head_dims_192_256_512(kv, d, hq, hkv, window_left):
+    """Head dims 256 (the sliding-attention layers of the Gemma family, Qwen3.5), 192 (128 + 64 rotary channels of
+    the MLA-style layers) and 512 (the Gemma family's full-attention layers) on the matrix-core kernel: one 16-row
+    tile per wave, at 512 shared by two waves with half of the head each; a query block cut by many shares goes
     through the merge of the wide partials."""
     new = torch.tensor([3, 150, 64, 1, 33])
     ctx = torch.tensor([900, 0, 77, 2500, 310])
