@@ -4,8 +4,9 @@
 // query-row axis: row r of the block is (token r / GP, head r % GP) with GP = G rounded up to a power of two, so one
 // 16-row MFMA tile holds 16 / GP tokens of all heads and K/V are read once for the whole group (GQA without
 // expanding KV, as areno/accel/csrc/attention.cu:170-171 does per row).  A block is 256 rows: each of the 8 waves
-// owns 32 (two 16-row tiles; one at head dims 192 and 256, and at 512 two waves share one).  One such workgroup per CU (the registers allow two waves per SIMD either way; eight
-// waves behind one set of K/V tiles halve the staging work per wave against two workgroups of four).
+// owns 32 (two 16-row tiles; one at head dims 192 and 256, and at 512 two waves share one).  One such workgroup per
+// CU (the registers allow two waves per SIMD either way; eight waves behind one set of K/V tiles halve the staging
+// work per wave against two workgroups of four).
 //
 // Balance: an item costs one "tile step" per 32-key tile it may see, and items differ by orders of magnitude (a
 // query block on a 16k context next to one on an empty context).  Every workgroup computes the prefix sum of tile
