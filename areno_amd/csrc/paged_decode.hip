@@ -151,19 +151,25 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_kernel(Decod
 // its weight is known, rows of absent candidates are dropped after the fact; (3) the stores.
 constexpr int kMergeChunk = 8;
 
+// The arguments in front of the parameter block are what the kernel's first loads are addressed with: as leading
+// scalar arguments they reach the wave in registers at its start (kernel-argument preload, at most 16 words), while
+// the block behind them takes a fetch of its own.
 template <int EPW>  // head-dimension elements per lane: head_dim <= 64 EPW
-__global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel(MfmaDecodeParams mp) {
+__global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel(
+    const int32_t* plan_rows, const int32_t* cache_seqlens, const void* q_rows, const void* k_update,
+    const void* v_update, int32_t total_rows, int32_t q_heads, int32_t kv_heads, int32_t group, int32_t head_dim,
+    int32_t q_dtype, MfmaDecodeParams mp) {
   const DecodeParams& p = mp.d;
   const int lane = threadIdx.x & (kWave - 1);
   const int row = blockIdx.x * kReduceRows + (threadIdx.x >> 6);
-  if (row >= p.batch * p.q_heads) return;
-  const int b = row / p.q_heads;
-  const int h = row - b * p.q_heads;
-  const int kvh = h / p.group;
-  const int d = p.head_dim;
+  if (row >= total_rows) return;
+  const int b = row / q_heads;
+  const int h = row - b * q_heads;
+  const int kvh = h / group;
+  const int d = head_dim;
   const ItemShape& shape = mp.items;
   const int num_items = shape.num_items();
-  const bool append = shape.append_in_merge != 0;
+  const bool append = k_update != nullptr;  // (the launcher passes the update rows only when this launch folds them in)
 
   // ---- round trip 1 ---------------------------------------------------------------------------------------------------
   // units that hold partials of the row: its own item's and, with prefix groups, its sub-group's shared item's
@@ -177,9 +183,9 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
     const int first_row = gi * shape.group_rows + j * shape.cols_seqs;
     sh_col = kvh * 16 + (b - first_row) * p.group + (h - kvh * p.group);
   }
-  if (mp.plan_rows != nullptr) {
-    planned_units = *reinterpret_cast<const int4_t*>(mp.plan_rows + 4 * static_cast<int64_t>(b));
-    cum_total = mp.plan_rows[-4];
+  if (plan_rows != nullptr) {
+    planned_units = *reinterpret_cast<const int4_t*>(plan_rows + 4 * static_cast<int64_t>(b));
+    cum_total = plan_rows[-4];
   } else {
     const int32_t* cum = mp.cum_out;
     const int v_own = shape.num_shared + b;
@@ -195,21 +201,21 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   uint16_t kraw[EPW], vraw[EPW];
   int64_t pos = 0;
   if (append) {
-    const int64_t src_base = (static_cast<int64_t>(b) * p.kv_heads + kvh) * d;
-    pos = p.cache_seqlens[b];
+    const int64_t src_base = (static_cast<int64_t>(b) * kv_heads + kvh) * d;
+    pos = cache_seqlens[b];
 #pragma unroll
     for (int e = 0; e < EPW; ++e) {
       const int idx = lane + e * kWave;
       const bool in = idx < d;
-      kraw[e] = in ? static_cast<const uint16_t*>(mp.k_update)[src_base + idx] : 0;
-      vraw[e] = in ? static_cast<const uint16_t*>(mp.v_update)[src_base + idx] : 0;
-      qv[e] = in ? load_as_float(p.q, static_cast<int64_t>(row) * d + idx, p.q_dtype) : 0.0f;
+      kraw[e] = in ? static_cast<const uint16_t*>(k_update)[src_base + idx] : 0;
+      vraw[e] = in ? static_cast<const uint16_t*>(v_update)[src_base + idx] : 0;
+      qv[e] = in ? load_as_float(q_rows, static_cast<int64_t>(row) * d + idx, q_dtype) : 0.0f;
     }
   }
   // (with fewer cost positions than units a candidate's unit may be empty and have written nothing)
   const bool every_unit_has_quanta = cum_total >= mp.num_units;
   const UnitGeometry geo = make_unit_geometry(cum_total, mp.num_units);
-  if (mp.plan_rows != nullptr) {
+  if (plan_rows != nullptr) {
     own_lo = planned_units[0];
     own_n = planned_units[1];
     sh_lo = planned_units[2];
@@ -353,7 +359,8 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   }
 }
 
-typedef void (*reduce_slots_fn)(MfmaDecodeParams);
+typedef void (*reduce_slots_fn)(const int32_t*, const int32_t*, const void*, const void*, const void*, int32_t, int32_t,
+                                int32_t, int32_t, int32_t, int32_t, MfmaDecodeParams);
 // the narrowest instantiation that covers the head: the kernel is a few hundred instructions per wave and mostly
 // launch latency, so slots that would only be predicated off are worth leaving out
 reduce_slots_fn reduce_slots_kernel_for(int head_dim) {
@@ -835,12 +842,16 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
       mp.plan_rows = words + l.rows;
     }
     if (stages & ARENO_STAGE_SPLIT) {
-      hipLaunchKernelGGL(mfma, dim3(grid.workgroups, grid.head_groups), dim3(grid.waves * kWave), 0, s, mp);
+      hipLaunchKernelGGL(mfma, dim3(grid.workgroups, grid.head_groups), dim3(grid.waves * kWave), 0, s, mp.plan_units,
+                         mp.plan_items, mp.plan_cum, p.cache_seqlens, mp.tok_splits, mp.d.heads_per_wg,
+                         mp.items.num_items(), mp);
       if (int rc = check_launch(op)) return rc;
     }
     if (stages & ARENO_STAGE_REDUCE) {
       const int rblocks = (batch * q_heads + kReduceRows - 1) / kReduceRows;
-      hipLaunchKernelGGL(reduce_slots_kernel_for(mp.d.head_dim), dim3(rblocks), dim3(kReduceRows * kWave), 0, s, mp);
+      hipLaunchKernelGGL(reduce_slots_kernel_for(mp.d.head_dim), dim3(rblocks), dim3(kReduceRows * kWave), 0, s,
+                         mp.plan_rows, p.cache_seqlens, p.q, mp.k_update, mp.v_update, batch * q_heads, q_heads,
+                         p.kv_heads, p.group, p.head_dim, p.q_dtype, mp);
       if (int rc = check_launch(op)) return rc;
     }
     return ARENO_OK;

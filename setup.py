@@ -37,6 +37,9 @@ HIP_DEVICE_FLAGS = [
     f"--offload-arch={GPU_ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-Wall", "-Wno-unused-function",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-fno-honor-nans",  # fmaxf as a bare v_max_f32 / v_max3_f32 (no canonicalising self-max); nothing here relies on NaN
+    # leading scalar kernel arguments (up to 16 words) arrive in registers at wave start instead of through a fetch of
+    # the argument block: the decode kernels put what their first loads are addressed with there
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-DARENO_DEVICE_FLAGS_OK=1",  # device_common.hpp refuses to compile without the two flags above
 ] + [f"-D{name}={os.environ[name]}" for name in ("ARENO_MFMA_NW", "ARENO_TRACE", "ARENO_MFMA_QUANT_OCC", "ARENO_MFMA_WIDE_OCC", "ARENO_PREFILL_WAVES") if os.environ.get(name)]  # fmt: skip
 
