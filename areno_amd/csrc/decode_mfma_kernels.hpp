@@ -123,6 +123,7 @@ struct MfmaDecodeParams {
   int32_t* cum_out;    // [items + 1]: the prefix sums, written by workgroup 0 for the merge kernel (launches without a plan)
   int32_t tok_splits;  // waves of a workgroup that share a KV head (waves per workgroup / heads_per_wg / head split)
   int32_t num_units;   // gridDim.x * tok_splits
+  int32_t head_parts;  // column tiles per kv head: ceil(q heads per kv head / 16); a wave serves one (kv head, part)
   ItemShape items;     // rows -> items (prefix groups, window, whether the merge folds in the token being appended)
   // A plan built once for all layers of a step (NULL: every workgroup derives the work list from the lengths).
   const int32_t* plan_cum;
@@ -333,7 +334,12 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   const int half = wave % DSPLIT;  // which part of the head dimension this wave owns
   const int hw = (wave / DSPLIT) % hw_count;
   const int ts = (wave / DSPLIT) / hw_count;
-  const int kvh = blockIdx.y * hw_count + hw;
+  // more than 16 query heads per kv head take several column tiles: the "heads" the grid is laid out over are
+  // (kv head, part) pairs, the parts of a kv head next to each other so that they stream its pages at the same time
+  const int vhead = blockIdx.y * hw_count + hw;
+  const int kvh = mp.head_parts > 1 ? vhead / mp.head_parts : vhead;
+  const int part = vhead - kvh * mp.head_parts;
+  const int group_here = min(16, p.group - 16 * part);  // query heads of this wave's column tile
   const int unit = blockIdx.x * tok_splits + ts;
 
   // ---- the item table: (lo, end, row, nseq) of every item and the exclusive prefix sum of their quanta, in LDS -----
@@ -439,7 +445,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
 
   constexpr int64_t row_bytes = static_cast<int64_t>(DFULL) * ES;
   const int64_t half_bytes = static_cast<int64_t>(half) * D * ES;  // of this wave's part inside a cache / update row
-  const int h0 = kvh * p.group;
+  const int h0 = kvh * p.group + 16 * part;
   const bool q_is_operand_type = (KIND == KV_BF16 && p.q_dtype == ARENO_DT_BF16) ||
                                  (KIND != KV_BF16 && p.q_dtype == ARENO_DT_F16);
   auto is_shared = [&](int v) { return GROUPED && v < shape.num_shared; };
@@ -550,7 +556,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     const bool shared = is_shared(item);
     const int m = shared ? col_seq : 0;
     const int g = shared ? col_head : lr;
-    const bool live = shared ? m < nseq : lr < p.group;
+    const bool live = shared ? m < nseq : lr < group_here;
     const int64_t head_row = live ? static_cast<int64_t>(row + m) * p.q_heads + h0 + g
                                   : static_cast<int64_t>(row) * p.q_heads + h0;
     q_live = live;
@@ -626,7 +632,7 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
   // nothing reads.
   auto store_partial = [&](int v, int row, int nseq, const float4_t (&o)[NB], float m_val, float l_val) {
     const bool shared = is_shared(v);
-    const bool live = shared ? col_seq < nseq : lr < p.group;
+    const bool live = shared ? col_seq < nseq : lr < group_here;
     const int64_t prow = shared ? (static_cast<int64_t>(unit + v) * p.kv_heads + kvh) * 16 + lr
                                 : static_cast<int64_t>(unit + row) * p.q_heads + h0 + lr;
     float* const ml = shared ? mp.shared_ml : p.part_ml;

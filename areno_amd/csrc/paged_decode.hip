@@ -499,28 +499,32 @@ decode_mfma_fn mfma_lookup(const areno_paged_cache* cache, bool grouped) {
 }
 
 // Whether (and how) the matrix-core kernel serves a call: 16-bit or 8-bit caches, head_dim 64 / 128 / 192 / 256 / 512,
-// up to 16 q heads per kv head, page sizes that are powers of two, at most kMfmaMaxBatch rows.  Shared by the decode
+// up to 16 * kMaxHeadParts q heads per kv head (16 per column tile; further tiles of a kv head run as heads of their
+// own that read the same pages), page sizes that are powers of two, at most kMfmaMaxBatch rows.  Shared by the decode
 // launcher and the plan builder, which must agree on the item list and the units.
+constexpr int kMaxHeadParts = 8;
 struct MfmaChoice {
   decode_mfma_fn fn;  // NULL: another kernel takes the call
   MfmaGrid grid;
   ItemShape items;
   int tile_tokens;
+  int head_parts;  // column tiles per kv head
 };
 MfmaChoice choose_mfma(const areno_paged_cache* cache, int q_dtype, int batch, int q_heads, int window_left,
                        bool with_update, int group_rows, bool has_shared_lens) {
   MfmaChoice c;
   c.fn = nullptr;
-  c.grid = mfma_grid_for(cache->kv_heads, cache->head_dim);
+  const int group = q_heads / cache->kv_heads;
+  c.head_parts = (group + 15) / 16;
+  c.grid = mfma_grid_for(cache->kv_heads * c.head_parts, cache->head_dim);
   // what changing items costs a wave, in 16-token quanta of streaming (measured: ~1.4 us against ~1.4 us per 32-token
   // tile of 8-bit pages, ~2.6 us per tile of 16-bit pages)
   c.items = ItemShape{batch, window_left, 0, is_quantized(cache->cache_dtype) ? 3 : 1, 0, 1, 1, 1};
   c.tile_tokens = decode_tile_tokens(is_quantized(cache->cache_dtype));
-  const int group = q_heads / cache->kv_heads;
   const bool aligned = (reinterpret_cast<uintptr_t>(cache->k) % 16 == 0) && (reinterpret_cast<uintptr_t>(cache->v) % 16 == 0);
   // the kernel indexes cache rows (block, slot, head) with 32 bits
   const bool rows_fit = static_cast<double>(cache->num_blocks) * cache->block_size * cache->kv_heads < 4294967296.0;
-  if (!aligned || q_dtype == ARENO_DT_F32 || !prefer_mfma() || group > 16 || batch > kMfmaMaxBatch || !rows_fit ||
+  if (!aligned || q_dtype == ARENO_DT_F32 || !prefer_mfma() || c.head_parts > kMaxHeadParts || batch > kMfmaMaxBatch || !rows_fit ||
       log2_exact(cache->block_size) < 0)
     return c;
   // prefix groups: only without a window, when at least two rows fit side by side
@@ -806,6 +810,7 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     mp.d.heads_per_wg = grid.heads_per_wg;
     mp.tok_splits = grid.tok_splits;
     mp.num_units = grid.units;
+    mp.head_parts = choice.head_parts;
     mp.items = choice.items;
     mp.k_update = merge_appends ? k_update : nullptr;
     mp.v_update = merge_appends ? v_update : nullptr;

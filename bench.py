@@ -291,6 +291,61 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
     }
 
 
+def measure_other_shapes(device, steps=56, repeats=7):
+    """us/step (graph replay, a plan per LAYERS_PER_PLAN steps where the shape takes one) of decode shapes next to the
+    benchmark's: cfg 2's rows with more than 16 query heads per KV head (several column tiles per KV head on the
+    matrix-core kernel) and on pages whose size is no power of two (the vector-ALU kernels).  Two pool copies only,
+    so part of the int8 working set may sit in the Infinity Cache: these are orders of magnitude, not roofline figures."""
+    import torch
+
+    from areno_amd import workloads
+    from areno_amd.accel import cabi
+
+    shapes = {
+        "mqa_32q_1kv_int8": dict(hq=32, hkv=1, bs=16, kv="int8"),
+        "gqa_64q_2kv_bf16": dict(hq=64, hkv=2, bs=16, kv="bf16"),
+        "cfg2_rows_page48_int8": dict(hq=28, hkv=4, bs=48, kv="int8"),
+    }
+    g = torch.Generator().manual_seed(2002)
+    lengths = torch.randint(512, 4097, (64,), generator=g)
+    result = {}
+    for name, sh in shapes.items():
+        w = workloads.make_decode_workload(name, seed=7, batch=64, hq=sh["hq"], hkv=sh["hkv"], d=128, bs=sh["bs"], kv=sh["kv"],
+                                           lengths=lengths, device=device, quantize_fn=_gpu_quantize)  # fmt: skip
+        pools = _clone_pools(w, 2)
+        plan_buffer = torch.empty(max(16, cabi.decode_plan_bytes(64)), dtype=torch.uint8, device=device)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for pool in pools:
+                _step(w, pool, _plan(w, pool))
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        keep = []
+        with torch.cuda.graph(graph):
+            plan = None
+            for i in range(steps):
+                if i % LAYERS_PER_PLAN == 0:
+                    plan = _plan(w, pools[0], plan_buffer)
+                keep.append(_step(w, pools[i % 2], plan))
+        graph.replay()
+        torch.cuda.synchronize()
+        samples = []
+        for _ in range(repeats):
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize()
+            samples.append((time.perf_counter() - t0) / steps * 1e6)
+        us = statistics.median(samples)
+        result[name] = {"us_per_step": us, "algorithmic_gbps": w.algorithmic_bytes() / (us * 1e-6) / 1e9,
+                        "kernel": "matrix cores" if plan is not None and plan.units > 0 else "vector ALU",
+                        "parity_max_abs_4rows": _parity_sample(w, keep[0])}  # fmt: skip
+        del w, pools, keep, graph
+        torch.cuda.empty_cache()
+    return result
+
+
 def measure_stream_ceiling(w, pools, iters=10, samples=9):
     """GB/s of `areno_hip_probe_stream_read` (16-byte loads, a page per wave at a time, nothing computed; one launch
     reads a page set from the K and the V pool, as a decode launch does) over the K and V pools of all pool copies:
@@ -685,6 +740,9 @@ def main() -> int:
             baseline = cpu_baseline(w)
         del w
         torch.cuda.empty_cache()
+
+    if not args.only:
+        results["other_shapes"] = measure_other_shapes(dev)
 
     head = results[names[0]]
     dtype = {"cfg1": "bf16", "cfg2": "int8", "cfg3": "fp8", "cfg4": "fp8", "cfg2_b256": "int8"}[names[0]]

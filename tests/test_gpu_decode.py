@@ -81,7 +81,10 @@ def test_fp16_query_with_quantized_cache():
     ("bf16", 28, 4, 128, 16), ("int8", 28, 4, 128, 16), ("fp8", 32, 8, 128, 16), ("bf16", 16, 2, 128, 256),
     ("int8", 4, 4, 64, 16), ("bf16", 6, 2, 128, 16), ("fp16", 12, 1, 64, 32), ("int8", 5, 1, 128, 8),
     ("bf16", 8, 2, 96, 16), ("bf16", 24, 2, 128, 16), ("fp8", 8, 8, 128, 48), ("fp32", 8, 2, 128, 16),
-    ("int8", 32, 1, 128, 16), ("bf16", 40, 2, 64, 16),  # more than 16 q heads per kv head: the vector-ALU kernels
+    # more than 16 q heads per kv head: several 16-column tiles per kv head (2 x 16, 16 + 4, 16 + 16 + 8, 8 x 16)
+    ("int8", 32, 1, 128, 16), ("bf16", 40, 2, 64, 16), ("fp8", 40, 1, 128, 16), ("bf16", 128, 1, 128, 16),
+    ("int8", 136, 1, 64, 16),  # more than 128: the vector-ALU kernels
+    ("bf16", 24, 4, 128, 12),  # a page size that is no power of two: the vector-ALU kernels
 ])  # fmt: skip
 def test_shapes_head_ratios_and_block_sizes(kv, hq, hkv, d, bs):
     g = torch.Generator().manual_seed(hq * 131 + d)
@@ -92,8 +95,12 @@ def test_shapes_head_ratios_and_block_sizes(kv, hq, hkv, d, bs):
     lengths[2] = bs  # ...and the first slot of a fresh page
     w = workloads.make_decode_workload("shapes", seed=77, batch=batch, hq=hq, hkv=hkv, d=d, bs=bs, kv=kv,
                                        lengths=lengths, device=DEV, quantize_fn=gpu_quantize, poison=True)  # fmt: skip
+    before = _snapshot(w)
     out = run_decode(w)
     assert_close(out, expected_decode(w), *tolerances(kv), what=f"{kv} {hq}/{hkv} d={d} bs={bs}")
+    _check_append(w, before)
+    if kv != "fp32":  # through a plan: the same bits (the second append rewrites the slot with the same values)
+        assert torch.equal(run_decode(w, planned=True), out)
 
 
 @pytest.mark.parametrize("kv", ["bf16", "fp16", "int8", "fp8"])
