@@ -124,6 +124,10 @@ struct MfmaDecodeParams {
   int32_t tok_splits;  // waves of a workgroup that share a KV head (waves per workgroup / heads_per_wg / head split)
   int32_t num_units;   // gridDim.x * tok_splits
   int32_t head_parts;  // column tiles per kv head: ceil(q heads per kv head / 16); a wave serves one (kv head, part)
+  // token -> block-table column for any page size: (token * bs_magic) >> (32 + bs_post), exact for tokens below 2^30
+  // (page_division() in paged_decode.hip)
+  uint32_t bs_magic;
+  int32_t bs_post;
   ItemShape items;     // rows -> items (prefix groups, window, whether the merge folds in the token being appended)
   // A plan built once for all layers of a step (NULL: every workgroup derives the work list from the lengths).
   const int32_t* plan_cum;
@@ -478,15 +482,15 @@ __global__ __launch_bounds__(NW * kWave, KVTraits<KIND>::kQuant ? ARENO_MFMA_QUA
     t.kind = 0;
     return t;
   };
-  // (the launcher sends only page sizes that are powers of two here)
-  auto column_of = [&](int t) { return t >> p.bs_shift; };
-  auto slot_of = [&](int t) { return t & (p.block_size - 1); };
+  // block-table column and slot of a token, for any page size: a division by multiply and shift
+  auto column_of = [&](int t) { return static_cast<int>(__umulhi(static_cast<uint32_t>(t), mp.bs_magic) >> mp.bs_post); };
+  auto slot_of = [&](int t) { return t - column_of(t) * p.block_size; };
   // The token whose cache row this lane fetches for group tg: its own token of the tile, clamped to the segment's
   // last one; one token for all lanes of a phantom tile (a tile past the unit's end: its loads keep the pipeline's
   // shape and hit one cache line each).
   auto lane_token = [&](const TileDesc& t, int tg) {
     const int own = (t.kind & kTilePhantom) ? 0 : 16 * tg + lr;
-    return min(t.tok + own, t.end - 1);
+    return max(min(t.tok + own, t.end - 1), 0);  // (never negative: the page division below takes it as unsigned)
   };
   // (block ids and cache rows are indexed with compile-time constants only: an array indexed by a lane-dependent
   // value would live in scratch memory, and scratch loads count with the global loads and drain the pipeline)

@@ -500,9 +500,27 @@ decode_mfma_fn mfma_lookup(const areno_paged_cache* cache, bool grouped) {
 
 // Whether (and how) the matrix-core kernel serves a call: 16-bit or 8-bit caches, head_dim 64 / 128 / 192 / 256 / 512,
 // up to 16 * kMaxHeadParts q heads per kv head (16 per column tile; further tiles of a kv head run as heads of their
-// own that read the same pages), page sizes that are powers of two, at most kMfmaMaxBatch rows.  Shared by the decode
+// own that read the same pages), pages of at least 4 tokens, at most kMfmaMaxBatch rows.  Shared by the decode
 // launcher and the plan builder, which must agree on the item list and the units.
 constexpr int kMaxHeadParts = 8;
+
+// Division of a token index by the page size as a multiply and a shift: with s = ceil(log2(bs)) and
+// magic = floor(2^(30 + s) / bs) + 1, (t * magic) >> (30 + s) == t / bs for every 0 <= t < 2^30 (the error of the
+// product is below t / 2^(30 + s) <= 1 / 2^s, which cannot carry a quotient over while (bs - 1) / bs + 1 / 2^s <= 1).
+// The kernel takes the high word of the product, so the shift left over is s - 2 and pages of fewer than 4 tokens are
+// not served this way.
+struct PageDivision {
+  uint32_t magic;
+  int32_t post;
+};
+bool page_division(int64_t block_size, PageDivision* out) {
+  if (block_size < 4 || block_size > (1 << 24)) return false;
+  int s = 0;
+  while ((int64_t{1} << s) < block_size) ++s;
+  out->magic = static_cast<uint32_t>((uint64_t{1} << (30 + s)) / static_cast<uint64_t>(block_size) + 1);
+  out->post = s - 2;
+  return true;
+}
 struct MfmaChoice {
   decode_mfma_fn fn;  // NULL: another kernel takes the call
   MfmaGrid grid;
@@ -524,8 +542,9 @@ MfmaChoice choose_mfma(const areno_paged_cache* cache, int q_dtype, int batch, i
   const bool aligned = (reinterpret_cast<uintptr_t>(cache->k) % 16 == 0) && (reinterpret_cast<uintptr_t>(cache->v) % 16 == 0);
   // the kernel indexes cache rows (block, slot, head) with 32 bits
   const bool rows_fit = static_cast<double>(cache->num_blocks) * cache->block_size * cache->kv_heads < 4294967296.0;
+  PageDivision division;
   if (!aligned || q_dtype == ARENO_DT_F32 || !prefer_mfma() || c.head_parts > kMaxHeadParts || batch > kMfmaMaxBatch || !rows_fit ||
-      log2_exact(cache->block_size) < 0)
+      !page_division(cache->block_size, &division))
     return c;
   // prefix groups: only without a window, when at least two rows fit side by side
   int cols_seqs = 0, subs_per_group = 0, num_shared = 0;
@@ -561,7 +580,7 @@ struct PlanParams {
   int32_t* rows;
   ItemShape shape;
   int32_t num_units;
-  int32_t bs_shift;
+  int32_t block_size;
   int32_t max_blocks;
 };
 
@@ -680,8 +699,8 @@ __global__ __launch_bounds__(kPlanThreads) void decode_plan_kernel(PlanParams pp
       rec[kPuRow] = c.it.row;
       rec[kPuNseq] = c.it.nseq;
       // block ids of the first tile's columns; columns behind the segment's last one repeat it
-      const int col0 = c.tok >> pp.bs_shift;
-      int last = (c.seg_end - 1) >> pp.bs_shift;
+      const int col0 = c.tok / pp.block_size;
+      int last = (c.seg_end - 1) / pp.block_size;
       last = last < pp.max_blocks - 1 ? last : pp.max_blocks - 1;
       const int32_t* table_row = pp.block_table + static_cast<int64_t>(c.it.row) * pp.max_blocks;
 #pragma unroll
@@ -811,6 +830,12 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
     mp.tok_splits = grid.tok_splits;
     mp.num_units = grid.units;
     mp.head_parts = choice.head_parts;
+    {
+      PageDivision division = {0, 0};
+      page_division(cache->block_size, &division);  // (checked by choose_mfma)
+      mp.bs_magic = division.magic;
+      mp.bs_post = division.post;
+    }
     mp.items = choice.items;
     mp.k_update = merge_appends ? k_update : nullptr;
     mp.v_update = merge_appends ? v_update : nullptr;
@@ -1027,7 +1052,7 @@ extern "C" int areno_hip_paged_decode_plan(areno_decode_plan* plan, void* buffer
   pp.rows = words + l.rows;
   pp.shape = choice.items;
   pp.num_units = choice.grid.units;
-  pp.bs_shift = log2_exact(cache->block_size);
+  pp.block_size = cache->block_size;
   pp.max_blocks = max_blocks;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (choice.items.num_shared > 0) {

@@ -294,7 +294,8 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
 def measure_other_shapes(device, steps=56, repeats=7):
     """us/step (graph replay, a plan per LAYERS_PER_PLAN steps where the shape takes one) of decode shapes next to the
     benchmark's: cfg 2's rows with more than 16 query heads per KV head (several column tiles per KV head on the
-    matrix-core kernel) and on pages whose size is no power of two (the vector-ALU kernels).  Two pool copies only,
+    matrix-core kernel) and on pages whose size is no power of two (a multiply-shift division in the kernel's page
+    arithmetic).  Two pool copies only,
     so part of the int8 working set may sit in the Infinity Cache: these are orders of magnitude, not roofline figures."""
     import torch
 

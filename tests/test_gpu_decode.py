@@ -84,7 +84,8 @@ def test_fp16_query_with_quantized_cache():
     # more than 16 q heads per kv head: several 16-column tiles per kv head (2 x 16, 16 + 4, 16 + 16 + 8, 8 x 16)
     ("int8", 32, 1, 128, 16), ("bf16", 40, 2, 64, 16), ("fp8", 40, 1, 128, 16), ("bf16", 128, 1, 128, 16),
     ("int8", 136, 1, 64, 16),  # more than 128: the vector-ALU kernels
-    ("bf16", 24, 4, 128, 12),  # a page size that is no power of two: the vector-ALU kernels
+    ("bf16", 24, 4, 128, 12), ("int8", 8, 2, 128, 768),  # page sizes that are no power of two
+    ("bf16", 4, 2, 64, 2),  # pages of fewer than 4 tokens: the vector-ALU kernels
 ])  # fmt: skip
 def test_shapes_head_ratios_and_block_sizes(kv, hq, hkv, d, bs):
     g = torch.Generator().manual_seed(hq * 131 + d)
