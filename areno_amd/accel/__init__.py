@@ -2,7 +2,8 @@
 
 Re-exports the op surface the reference's inference backend imports
 (``areno/accel/__init__.py:17-21`` there) plus this build's additions (cache write, paged prefill, the fused
-QK-norm + rotary + cache-write step in front of the path, and the per-step plan of the decode op).
+QK-norm + rotary + cache-write step in front of the path, and what a decode step prepares once for all its layers:
+the plan of the decode op and the rotary rows of the fused step).
 """
 
 from areno_amd.accel.attention import (
@@ -12,6 +13,7 @@ from areno_amd.accel.attention import (
     areno_paged_decode_plan,
     areno_paged_varlen_causal_attention,
     areno_qk_norm_rope_cache_write,
+    areno_rope_rows,
     areno_varlen_causal_attention,
 )
 
@@ -22,5 +24,6 @@ __all__ = [
     "areno_paged_decode_plan",
     "areno_paged_varlen_causal_attention",
     "areno_qk_norm_rope_cache_write",
+    "areno_rope_rows",
     "areno_varlen_causal_attention",
 ]

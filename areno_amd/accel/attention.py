@@ -539,6 +539,7 @@ def areno_qk_norm_rope_cache_write(
     cache_block_offsets: torch.Tensor | None = None,
     k_scale: torch.Tensor | None = None,
     v_scale: torch.Tensor | None = None,
+    rope_rows: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """The layer's steps in front of attention in one kernel: ``q_norm`` / ``k_norm`` (per-head RMSNorm, fp32
     weights), rotary embedding from the ``(max_position, head_dim)`` float32 tables of ``RotaryEmbedding``, and,
@@ -546,10 +547,15 @@ def areno_qk_norm_rope_cache_write(
 
     ``q (T, Hq, D)``, ``k`` / ``v (T, Hkv, D)`` fp16 or bf16; returns ``(q, k)`` after norm and rotary.  The pages
     receive exactly what ``areno_paged_cache_write(k_out, v, ...)`` would store.
+
+    ``rope_rows``: what :func:`areno_rope_rows` made of ``position_ids`` and the tables for this dtype, once per step
+    for all layers; the kernel then reads a token's prepared cosines and sines instead of fetching its position and
+    table rows and rounding them for every (token, head) row.  Same results, bit for bit; ``position_ids`` and the
+    tables are not looked at.
     """
     op = "areno_qk_norm_rope_cache_write"
     tensors = (q, k, v, position_ids, cos_cached, sin_cached, q_norm_weight, k_norm_weight, k_cache, v_cache,
-               cache_block_ids, cache_block_offsets, k_scale, v_scale)  # fmt: skip
+               cache_block_ids, cache_block_offsets, k_scale, v_scale, rope_rows)  # fmt: skip
     if not _all_on_gpu(*tensors):
         raise RuntimeError(f"{op} requires CUDA tensors")
     if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
@@ -564,11 +570,36 @@ def areno_qk_norm_rope_cache_write(
         _check_scales(op, k_cache, k_scale, v_scale)
         if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
             raise ValueError(f"{op} expects contiguous cache tensors (they are updated in place)")
+    weights = (None if q_norm_weight is None else q_norm_weight.to(torch.float32).contiguous(),
+               None if k_norm_weight is None else k_norm_weight.to(torch.float32).contiguous())  # fmt: skip
+    if rope_rows is not None:
+        if rope_rows.dtype != torch.float32 or rope_rows.shape != (q.shape[0], 2, q.shape[2]):
+            raise ValueError(f"{op} expects rope_rows from areno_rope_rows for these tokens: float32 (tokens, 2, head_dim)")
+        return tuple(_extension().areno_qk_norm_rope_cache_write_rows(
+            q.contiguous(), k.contiguous(), v.contiguous(), rope_rows.contiguous(), *weights, float(eps), k_cache, v_cache,
+            _contig(cache_block_ids), _contig(cache_block_offsets), k_scale, v_scale,
+        ))  # fmt: skip
     q_out, k_out = _extension().areno_qk_norm_rope_cache_write(
         q.contiguous(), k.contiguous(), v.contiguous(), position_ids.reshape(-1).to(torch.int64).contiguous(),
-        cos_cached.to(torch.float32).contiguous(), sin_cached.to(torch.float32).contiguous(),
-        None if q_norm_weight is None else q_norm_weight.to(torch.float32).contiguous(),
-        None if k_norm_weight is None else k_norm_weight.to(torch.float32).contiguous(),
+        cos_cached.to(torch.float32).contiguous(), sin_cached.to(torch.float32).contiguous(), *weights,
         float(eps), k_cache, v_cache, _contig(cache_block_ids), _contig(cache_block_offsets), k_scale, v_scale,
     )  # fmt: skip
     return q_out, k_out
+
+
+def areno_rope_rows(position_ids: torch.Tensor, cos_cached: torch.Tensor, sin_cached: torch.Tensor,
+                    dtype: torch.dtype) -> torch.Tensor:  # fmt: skip
+    """The rotary rows of a step's tokens for activations of ``dtype`` (fp16 / bf16): float32 ``(tokens, 2, head_dim)``,
+    row ``t`` holding ``cos_cached[position_ids[t]]`` cast to ``dtype`` and ``sin_cached[position_ids[t]]`` cast to
+    ``dtype`` with rotate_half's sign (minus on the first half of the head).  ``position_ids`` are the same for every
+    layer of a step (``layers/attention.py:94-96`` in the reference hands one tensor down), so this runs once per step
+    and every layer's :func:`areno_qk_norm_rope_cache_write` takes the result as ``rope_rows``."""
+    op = "areno_rope_rows"
+    if not _all_on_gpu(position_ids, cos_cached, sin_cached):
+        raise RuntimeError(f"{op} requires CUDA tensors")
+    if dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError(f"{op} expects an fp16 or bf16 activation dtype")
+    like = torch.empty(0, dtype=dtype, device=position_ids.device)
+    return _extension().areno_rope_rows(position_ids.reshape(-1).to(torch.int64).contiguous(),
+                                        cos_cached.to(torch.float32).contiguous(),
+                                        sin_cached.to(torch.float32).contiguous(), like)  # fmt: skip

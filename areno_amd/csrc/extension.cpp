@@ -343,29 +343,45 @@ at::Tensor paged_varlen_forward(at::Tensor q, at::Tensor k_cache, at::Tensor v_c
   return out;
 }
 
-std::vector<at::Tensor> qk_norm_rope_cache_write(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor positions,
-                                                 at::Tensor cos, at::Tensor sin, c10::optional<at::Tensor> q_weight,
-                                                 c10::optional<at::Tensor> k_weight, double eps,
-                                                 c10::optional<at::Tensor> k_cache, c10::optional<at::Tensor> v_cache,
-                                                 c10::optional<at::Tensor> block_ids,
-                                                 c10::optional<at::Tensor> block_offsets,
-                                                 c10::optional<at::Tensor> k_scale, c10::optional<at::Tensor> v_scale) {
-  const char* op = "areno_qk_norm_rope_cache_write";
-  TORCH_CHECK(q.is_cuda() && k.is_cuda() && v.is_cuda() && positions.is_cuda() && cos.is_cuda() && sin.is_cuda(), op,
-              " tensors must be CUDA");
-  TORCH_CHECK(q.is_contiguous() && k.is_contiguous() && v.is_contiguous() && positions.is_contiguous() &&
-                  cos.is_contiguous() && sin.is_contiguous(),
-              op, " tensors must be contiguous");
-  TORCH_CHECK(q.dim() == 3 && k.dim() == 3 && v.dim() == 3, op, " expects q/k/v shaped (tokens, heads, head_dim)");
-  TORCH_CHECK(q.scalar_type() == k.scalar_type() && q.scalar_type() == v.scalar_type(), op, " dtype mismatch");
-  TORCH_CHECK(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, op, " q/k/v must be fp16 or bf16");
-  TORCH_CHECK(k.sizes() == v.sizes(), op, " k/v shape mismatch");
-  TORCH_CHECK(q.size(0) == k.size(0) && q.size(2) == k.size(2), op, " q and k/v disagree on tokens or head_dim");
-  TORCH_CHECK(positions.dim() == 1 && positions.size(0) == q.size(0) && positions.scalar_type() == at::kLong, op,
-              " positions must be int64 (tokens,)");
-  TORCH_CHECK(cos.dim() == 2 && cos.sizes() == sin.sizes() && cos.size(1) == q.size(2) &&
-                  cos.scalar_type() == at::kFloat && sin.scalar_type() == at::kFloat,
+// The rotary rows of a step's tokens (areno_hip_rope_rows): float32 (tokens, 2, head_dim), rounded for `like`'s dtype.
+at::Tensor rope_rows(at::Tensor positions, at::Tensor cos, at::Tensor sin, at::Tensor like) {
+  const char* op = "areno_rope_rows";
+  TORCH_CHECK(positions.is_cuda() && cos.is_cuda() && sin.is_cuda(), op, " tensors must be CUDA");
+  TORCH_CHECK(positions.is_contiguous() && cos.is_contiguous() && sin.is_contiguous(), op, " tensors must be contiguous");
+  TORCH_CHECK(positions.dim() == 1 && positions.scalar_type() == at::kLong, op, " positions must be int64 (tokens,)");
+  TORCH_CHECK(cos.dim() == 2 && cos.sizes() == sin.sizes() && cos.scalar_type() == at::kFloat &&
+                  sin.scalar_type() == at::kFloat,
               op, " cos/sin must be float32 (max_position, head_dim)");
+  TORCH_CHECK(like.scalar_type() == at::kHalf || like.scalar_type() == at::kBFloat16, op,
+              " the activation dtype must be fp16 or bf16");
+  const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(positions));
+  auto rows = at::empty({positions.size(0), 2, cos.size(1)}, cos.options());
+  const int status = areno_hip_rope_rows(rows.data_ptr<float>(), positions.data_ptr<int64_t>(), cos.data_ptr<float>(),
+                                         sin.data_ptr<float>(), positions.size(0), static_cast<int32_t>(cos.size(1)),
+                                         static_cast<int32_t>(cos.size(0)), dtype_code(like, op, "like"),
+                                         current_stream(positions));
+  check_status(status, op);
+  return rows;
+}
+
+// Where the fused front step takes its rotary values from: the tables and the tokens' positions, or the prepared rows.
+struct RotarySource {
+  const int64_t* positions = nullptr;
+  const float* cos = nullptr;
+  const float* sin = nullptr;
+  int32_t max_pos = 0;
+  const float* rows = nullptr;
+};
+
+std::vector<at::Tensor> qk_rope_write_common(const char* op, const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                                             const RotarySource& rotary, const c10::optional<at::Tensor>& q_weight,
+                                             const c10::optional<at::Tensor>& k_weight, double eps,
+                                             const c10::optional<at::Tensor>& k_cache,
+                                             const c10::optional<at::Tensor>& v_cache,
+                                             const c10::optional<at::Tensor>& block_ids,
+                                             const c10::optional<at::Tensor>& block_offsets,
+                                             const c10::optional<at::Tensor>& k_scale,
+                                             const c10::optional<at::Tensor>& v_scale) {
   auto weight_ptr = [&](const c10::optional<at::Tensor>& w, const char* name) -> const float* {
     if (!w.has_value()) return nullptr;
     TORCH_CHECK(w->is_cuda() && w->is_contiguous() && w->scalar_type() == at::kFloat && w->dim() == 1 &&
@@ -396,13 +412,76 @@ std::vector<at::Tensor> qk_norm_rope_cache_write(at::Tensor q, at::Tensor k, at:
     ids = block_ids->data_ptr<int64_t>();
     offs = block_offsets->data_ptr<int64_t>();
   }
-  const int status = areno_hip_qk_norm_rope_cache_write(
-      cache_ptr, q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(), k_out.data_ptr(), dtype_code(q, op, "q"),
-      q.size(0), static_cast<int32_t>(q.size(1)), static_cast<int32_t>(k.size(1)), static_cast<int32_t>(q.size(2)),
-      positions.data_ptr<int64_t>(), cos.data_ptr<float>(), sin.data_ptr<float>(), static_cast<int32_t>(cos.size(0)), qw,
-      kw, static_cast<float>(eps), ids, offs, current_stream(q));
+  const int32_t dtype = dtype_code(q, op, "q");
+  const int32_t hq = static_cast<int32_t>(q.size(1)), hkv = static_cast<int32_t>(k.size(1));
+  const int32_t d = static_cast<int32_t>(q.size(2));
+  const int status =
+      rotary.rows != nullptr
+          ? areno_hip_qk_norm_rope_cache_write_rows(cache_ptr, q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(),
+                                                    k_out.data_ptr(), dtype, q.size(0), hq, hkv, d, rotary.rows, qw, kw,
+                                                    static_cast<float>(eps), ids, offs, current_stream(q))
+          : areno_hip_qk_norm_rope_cache_write(cache_ptr, q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(),
+                                               k_out.data_ptr(), dtype, q.size(0), hq, hkv, d, rotary.positions,
+                                               rotary.cos, rotary.sin, rotary.max_pos, qw, kw, static_cast<float>(eps),
+                                               ids, offs, current_stream(q));
   check_status(status, op);
   return {q_out, k_out};
+}
+
+void check_qkv_rows(const char* op, const at::Tensor& q, const at::Tensor& k, const at::Tensor& v) {
+  TORCH_CHECK(q.is_cuda() && k.is_cuda() && v.is_cuda(), op, " tensors must be CUDA");
+  TORCH_CHECK(q.is_contiguous() && k.is_contiguous() && v.is_contiguous(), op, " tensors must be contiguous");
+  TORCH_CHECK(q.dim() == 3 && k.dim() == 3 && v.dim() == 3, op, " expects q/k/v shaped (tokens, heads, head_dim)");
+  TORCH_CHECK(q.scalar_type() == k.scalar_type() && q.scalar_type() == v.scalar_type(), op, " dtype mismatch");
+  TORCH_CHECK(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, op, " q/k/v must be fp16 or bf16");
+  TORCH_CHECK(k.sizes() == v.sizes(), op, " k/v shape mismatch");
+  TORCH_CHECK(q.size(0) == k.size(0) && q.size(2) == k.size(2), op, " q and k/v disagree on tokens or head_dim");
+}
+
+std::vector<at::Tensor> qk_norm_rope_cache_write(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor positions,
+                                                 at::Tensor cos, at::Tensor sin, c10::optional<at::Tensor> q_weight,
+                                                 c10::optional<at::Tensor> k_weight, double eps,
+                                                 c10::optional<at::Tensor> k_cache, c10::optional<at::Tensor> v_cache,
+                                                 c10::optional<at::Tensor> block_ids,
+                                                 c10::optional<at::Tensor> block_offsets,
+                                                 c10::optional<at::Tensor> k_scale, c10::optional<at::Tensor> v_scale) {
+  const char* op = "areno_qk_norm_rope_cache_write";
+  check_qkv_rows(op, q, k, v);
+  TORCH_CHECK(positions.is_cuda() && cos.is_cuda() && sin.is_cuda(), op, " tensors must be CUDA");
+  TORCH_CHECK(positions.is_contiguous() && cos.is_contiguous() && sin.is_contiguous(), op, " tensors must be contiguous");
+  TORCH_CHECK(positions.dim() == 1 && positions.size(0) == q.size(0) && positions.scalar_type() == at::kLong, op,
+              " positions must be int64 (tokens,)");
+  TORCH_CHECK(cos.dim() == 2 && cos.sizes() == sin.sizes() && cos.size(1) == q.size(2) &&
+                  cos.scalar_type() == at::kFloat && sin.scalar_type() == at::kFloat,
+              op, " cos/sin must be float32 (max_position, head_dim)");
+  RotarySource rotary;
+  rotary.positions = positions.data_ptr<int64_t>();
+  rotary.cos = cos.data_ptr<float>();
+  rotary.sin = sin.data_ptr<float>();
+  rotary.max_pos = static_cast<int32_t>(cos.size(0));
+  return qk_rope_write_common(op, q, k, v, rotary, q_weight, k_weight, eps, k_cache, v_cache, block_ids, block_offsets,
+                              k_scale, v_scale);
+}
+
+std::vector<at::Tensor> qk_norm_rope_cache_write_rows(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor rope_rows,
+                                                      c10::optional<at::Tensor> q_weight,
+                                                      c10::optional<at::Tensor> k_weight, double eps,
+                                                      c10::optional<at::Tensor> k_cache,
+                                                      c10::optional<at::Tensor> v_cache,
+                                                      c10::optional<at::Tensor> block_ids,
+                                                      c10::optional<at::Tensor> block_offsets,
+                                                      c10::optional<at::Tensor> k_scale,
+                                                      c10::optional<at::Tensor> v_scale) {
+  const char* op = "areno_qk_norm_rope_cache_write";
+  check_qkv_rows(op, q, k, v);
+  TORCH_CHECK(rope_rows.is_cuda() && rope_rows.is_contiguous() && rope_rows.scalar_type() == at::kFloat &&
+                  rope_rows.dim() == 3 && rope_rows.size(0) == q.size(0) && rope_rows.size(1) == 2 &&
+                  rope_rows.size(2) == q.size(2),
+              op, " rope_rows must be a contiguous CUDA float32 (tokens, 2, head_dim) tensor");
+  RotarySource rotary;
+  rotary.rows = rope_rows.data_ptr<float>();
+  return qk_rope_write_common(op, q, k, v, rotary, q_weight, k_weight, eps, k_cache, v_cache, block_ids, block_offsets,
+                              k_scale, v_scale);
 }
 
 // ---- device-resident block tables ------------------------------------------------------------------------------------
@@ -598,6 +677,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("areno_paged_causal_attention_decode_forward_planned", &paged_decode_forward_planned,
         "paged decode forward with a per-step plan");
   m.def("areno_paged_cache_write", &cache_write, "quantize-and-scatter KV cache write");
+  m.def("areno_rope_rows", &rope_rows, "rotary rows of a step's tokens, rounded for an activation dtype");
+  m.def("areno_qk_norm_rope_cache_write_rows", &qk_norm_rope_cache_write_rows,
+        "QK norm + rotary + cache write from prepared rotary rows");
   m.def("areno_paged_varlen_causal_attention_forward", &paged_varlen_forward,
         "causal varlen prefill over paged (optionally quantized) KV");
   m.def("areno_qk_norm_rope_cache_write", &qk_norm_rope_cache_write,

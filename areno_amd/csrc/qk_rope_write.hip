@@ -40,6 +40,10 @@ struct RopeWriteParams {
   const float* cos;       // [max_pos, D]
   const float* sin;
   const int64_t* positions;  // [tokens]
+  // Per-token rotary rows from areno_hip_rope_rows ([tokens][2][D] float: the cosines rounded to the activation dtype,
+  // then the sines, rounded and with rotate_half's sign on them), or null: the kernel then takes a token's position,
+  // fetches its rows of the tables and rounds them itself, once per (token, head) row.
+  const float* rope_rows;
   void* cache[2];            // k, v pools; null pools: no cache write
   void* scale[2];
   const int64_t* block_ids;
@@ -130,7 +134,7 @@ __device__ __forceinline__ float rotary_partner(float x) {
 // ACT: the activation dtype (ARENO_DT_F16 / ARENO_DT_BF16): no rounding step branches on it.  The launcher checks that
 // rows, element offsets of q / k / v and page rows fit 32 bits, so the index arithmetic is 32-bit, with one division
 // per wave (the rows of a wave are consecutive).
-template <int LPR, int ACT, int KIND>
+template <int LPR, int ACT, int KIND, bool ROWS>
 __device__ __forceinline__ void rope_write_rows(const RopeWriteParams& p, uint32_t block) {
   constexpr int D = LPR * 8;
   constexpr int kRowsPerWave = kWave / LPR;
@@ -181,12 +185,20 @@ __device__ __forceinline__ void rope_write_rows(const RopeWriteParams& p, uint32
 
   if constexpr (KIND != 2) {
     // ---- q and k rows: norm and rotary ----------------------------------------------------------------------------
-    const int64_t pos = *reinterpret_cast<const int64_t*>(reinterpret_cast<const char*>(p.positions) + token * 8u);
-    const uint32_t pc =
-        pos < 0 ? 0u : (pos >= p.max_pos ? static_cast<uint32_t>(p.max_pos - 1) : static_cast<uint32_t>(pos));
-    const uint32_t table_bytes = (pc * D + sub * 8) * 4u;
-    const float* cos_row = reinterpret_cast<const float*>(reinterpret_cast<const char*>(p.cos) + table_bytes);
-    const float* sin_row = reinterpret_cast<const float*>(reinterpret_cast<const char*>(p.sin) + table_bytes);
+    const float* cos_row;
+    const float* sin_row;
+    if constexpr (ROWS) {
+      const uint32_t rows_bytes = (token * (2 * D) + sub * 8) * 4u;
+      cos_row = reinterpret_cast<const float*>(reinterpret_cast<const char*>(p.rope_rows) + rows_bytes);
+      sin_row = cos_row + D;
+    } else {
+      const int64_t pos = *reinterpret_cast<const int64_t*>(reinterpret_cast<const char*>(p.positions) + token * 8u);
+      const uint32_t pc =
+          pos < 0 ? 0u : (pos >= p.max_pos ? static_cast<uint32_t>(p.max_pos - 1) : static_cast<uint32_t>(pos));
+      const uint32_t table_bytes = (pc * D + sub * 8) * 4u;
+      cos_row = reinterpret_cast<const float*>(reinterpret_cast<const char*>(p.cos) + table_bytes);
+      sin_row = reinterpret_cast<const float*>(reinterpret_cast<const char*>(p.sin) + table_bytes);
+    }
     const float4_t c0 = *reinterpret_cast<const float4_t*>(cos_row);
     const float4_t c1 = *reinterpret_cast<const float4_t*>(cos_row + 4);
     const float4_t s0 = *reinterpret_cast<const float4_t*>(sin_row);
@@ -217,10 +229,12 @@ __device__ __forceinline__ void rope_write_rows(const RopeWriteParams& p, uint32
     for (int j = 0; j < 8; j += 2) {
       float ca = j < 4 ? c0[j & 3] : c1[j & 3], cb = j < 4 ? c0[(j + 1) & 3] : c1[(j + 1) & 3];
       float sa = j < 4 ? s0[j & 3] : s1[j & 3], sb = j < 4 ? s0[(j + 1) & 3] : s1[(j + 1) & 3];
-      round_pair<ACT>(ca, cb);  // the tables are cast to the activation dtype first, as the eager ops do
-      round_pair<ACT>(sa, sb);
-      sa = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, sa) ^ sign);
-      sb = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, sb) ^ sign);
+      if constexpr (!ROWS) {  // (prepared rows come rounded and signed)
+        round_pair<ACT>(ca, cb);  // the tables are cast to the activation dtype first, as the eager ops do
+        round_pair<ACT>(sa, sb);
+        sa = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, sa) ^ sign);
+        sb = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, sb) ^ sign);
+      }
       float xa = x[j] * ca, xb = x[j + 1] * cb;
       round_pair<ACT>(xa, xb);
       float ra = rotary_partner<LPR>(x[j]) * sa, rb = rotary_partner<LPR>(x[j + 1]) * sb;
@@ -250,28 +264,64 @@ __device__ __forceinline__ void rope_write_rows(const RopeWriteParams& p, uint32
   }
 }
 
-template <int LPR, int ACT>
+template <int LPR, int ACT, bool ROWS>
 __global__ __launch_bounds__(256) void qk_rope_write_kernel(RopeWriteParams p) {
   const uint32_t block = blockIdx.x;
   if (block < p.q_blocks) {
-    rope_write_rows<LPR, ACT, 0>(p, block);
+    rope_write_rows<LPR, ACT, 0, ROWS>(p, block);
   } else if (block < p.q_blocks + p.kv_blocks) {
-    rope_write_rows<LPR, ACT, 1>(p, block - p.q_blocks);
+    rope_write_rows<LPR, ACT, 1, ROWS>(p, block - p.q_blocks);
   } else {
-    rope_write_rows<LPR, ACT, 2>(p, block - p.q_blocks - p.kv_blocks);
+    rope_write_rows<LPR, ACT, 2, ROWS>(p, block - p.q_blocks - p.kv_blocks);
   }
 }
 
 typedef void (*rope_write_fn)(RopeWriteParams);
+template <bool ROWS>
 rope_write_fn rope_write_lookup(int head_dim, int dtype) {
   const bool bf16 = dtype == ARENO_DT_BF16;
   switch (head_dim) {
-    case 64: return bf16 ? qk_rope_write_kernel<8, ARENO_DT_BF16> : qk_rope_write_kernel<8, ARENO_DT_F16>;
-    case 128: return bf16 ? qk_rope_write_kernel<16, ARENO_DT_BF16> : qk_rope_write_kernel<16, ARENO_DT_F16>;
-    case 256: return bf16 ? qk_rope_write_kernel<32, ARENO_DT_BF16> : qk_rope_write_kernel<32, ARENO_DT_F16>;
-    case 512: return bf16 ? qk_rope_write_kernel<64, ARENO_DT_BF16> : qk_rope_write_kernel<64, ARENO_DT_F16>;
+    case 64: return bf16 ? qk_rope_write_kernel<8, ARENO_DT_BF16, ROWS> : qk_rope_write_kernel<8, ARENO_DT_F16, ROWS>;
+    case 128: return bf16 ? qk_rope_write_kernel<16, ARENO_DT_BF16, ROWS> : qk_rope_write_kernel<16, ARENO_DT_F16, ROWS>;
+    case 256: return bf16 ? qk_rope_write_kernel<32, ARENO_DT_BF16, ROWS> : qk_rope_write_kernel<32, ARENO_DT_F16, ROWS>;
+    case 512: return bf16 ? qk_rope_write_kernel<64, ARENO_DT_BF16, ROWS> : qk_rope_write_kernel<64, ARENO_DT_F16, ROWS>;
     default: return nullptr;
   }
+}
+
+// The rotary rows of a step's tokens, prepared once for all layers: thread (token, 4 elements) fetches the token's
+// position, its four cosines and sines, rounds them to the activation dtype (the cast the eager ops make, rotary.py:
+// 46-52 in the reference) and puts rotate_half's sign on the sines of the row's first half.
+struct RopeRowsParams {
+  float* rows;
+  const int64_t* positions;
+  const float* cos;
+  const float* sin;
+  int64_t tokens;
+  int32_t head_dim;
+  int32_t max_pos;
+  int32_t dtype;
+};
+__global__ __launch_bounds__(256) void rope_rows_kernel(RopeRowsParams p) {
+  const int64_t quads_per_row = p.head_dim / 4;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= p.tokens * quads_per_row) return;
+  const int64_t token = idx / quads_per_row;
+  const int e0 = static_cast<int>(idx - token * quads_per_row) * 4;
+  const int64_t pos = p.positions[token];
+  const int64_t pc = pos < 0 ? 0 : (pos >= p.max_pos ? p.max_pos - 1 : pos);
+  const float4_t c = *reinterpret_cast<const float4_t*>(p.cos + pc * p.head_dim + e0);
+  const float4_t s = *reinterpret_cast<const float4_t*>(p.sin + pc * p.head_dim + e0);
+  const float sign = e0 < p.head_dim / 2 ? -1.0f : 1.0f;
+  float4_t cr, sr;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    cr[j] = round_to(c[j], p.dtype);
+    sr[j] = sign * round_to(s[j], p.dtype);
+  }
+  float* dst = p.rows + token * (2 * p.head_dim) + e0;
+  *reinterpret_cast<float4_t*>(dst) = cr;
+  *reinterpret_cast<float4_t*>(dst + p.head_dim) = sr;
 }
 
 }  // namespace
@@ -279,15 +329,14 @@ rope_write_fn rope_write_lookup(int head_dim, int dtype) {
 int64_t g_rope_tokens_per_launch = 0;  // test hook, see areno_hip_debug_set_rope_tokens_per_launch
 }  // namespace areno
 
-extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache, const void* q, const void* k,
-                                                  const void* v, void* q_out, void* k_out, int32_t dtype,
-                                                  int64_t tokens, int32_t q_heads, int32_t kv_heads, int32_t head_dim,
-                                                  const int64_t* positions, const float* cos, const float* sin,
-                                                  int32_t max_pos, const float* q_weight, const float* k_weight,
-                                                  float eps, const int64_t* block_ids, const int64_t* block_offsets,
-                                                  void* stream) {
-  using namespace areno;
-  const char* op = "areno_hip_qk_norm_rope_cache_write";
+namespace areno {
+namespace {
+// rope_rows != nullptr: the prepared rows of the call's tokens stand in for positions / cos / sin / max_pos
+int rope_write_impl(const char* op, const areno_paged_cache* cache, const void* q, const void* k, const void* v,
+                    void* q_out, void* k_out, int32_t dtype, int64_t tokens, int32_t q_heads, int32_t kv_heads,
+                    int32_t head_dim, const int64_t* positions, const float* cos, const float* sin, int32_t max_pos,
+                    const float* rope_rows, const float* q_weight, const float* k_weight, float eps,
+                    const int64_t* block_ids, const int64_t* block_offsets, void* stream) {
   if (dtype != ARENO_DT_F16 && dtype != ARENO_DT_BF16)
     return fail(ARENO_ERR_UNSUPPORTED, "%s: activations must be f16 or bf16", op);
   if (tokens < 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || max_pos <= 0)
@@ -295,9 +344,11 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
   if (head_dim != 64 && head_dim != 128 && head_dim != 256 && head_dim != 512)
     return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim must be 64, 128, 256 or 512, got %d", op, head_dim);
   if (tokens == 0) return ARENO_OK;
-  if (q == nullptr || k == nullptr || v == nullptr || q_out == nullptr || positions == nullptr || cos == nullptr ||
-      sin == nullptr)
+  if (q == nullptr || k == nullptr || v == nullptr || q_out == nullptr ||
+      (rope_rows == nullptr && (positions == nullptr || cos == nullptr || sin == nullptr)))
     return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", op);
+  if (rope_rows != nullptr && reinterpret_cast<uintptr_t>(rope_rows) % 16 != 0)
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: rope_rows must be 16-byte aligned", op);
   RopeWriteParams p = {};
   if (cache != nullptr) {
     if (int rc = validate_paged_cache(cache, op)) return rc;
@@ -326,6 +377,7 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
   p.cos = cos;
   p.sin = sin;
   p.positions = positions;
+  p.rope_rows = rope_rows;
   p.block_ids = block_ids;
   p.block_offsets = block_offsets;
   p.tokens = tokens;
@@ -335,7 +387,7 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
   p.max_pos = max_pos;
   p.dtype = dtype;
   p.eps = eps;
-  const rope_write_fn fn = rope_write_lookup(head_dim, dtype);
+  const rope_write_fn fn = rope_rows != nullptr ? rope_write_lookup<true>(head_dim, dtype) : rope_write_lookup<false>(head_dim, dtype);
   if (fn == nullptr) return fail(ARENO_ERR_UNSUPPORTED, "%s: head_dim must be 64, 128, 256 or 512, got %d", op, head_dim);
   // The kernel's index arithmetic is 32-bit (rows, element offsets of q / k / v, rotary table offsets, page rows).
   // The table and the pool must fit as they are; a token count past the limits runs as consecutive launches over
@@ -348,6 +400,8 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
     return fail(ARENO_ERR_UNSUPPORTED, "%s: the pool's page rows do not fit 32 bits", op);
   int64_t tokens_per_launch = 0x7fffffffLL / (static_cast<int64_t>(heads) * head_dim) - 1;
   if (tokens_per_launch > (1 << 24) - 1) tokens_per_launch = (1 << 24) - 1;
+  // (byte offsets into the prepared rows: 8 * head_dim bytes per token)
+  if (rope_rows != nullptr && tokens_per_launch > 0xffffffffLL / (8 * head_dim) - 1) tokens_per_launch = 0xffffffffLL / (8 * head_dim) - 1;
   if (g_rope_tokens_per_launch > 0 && g_rope_tokens_per_launch < tokens_per_launch)
     tokens_per_launch = g_rope_tokens_per_launch;
   if (tokens_per_launch < 1) return fail(ARENO_ERR_UNSUPPORTED, "%s: one token's rows are past 32-bit indexing", op);
@@ -362,7 +416,8 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
     r.v = static_cast<const char*>(v) + kv_off;
     r.q_out = static_cast<char*>(q_out) + q_off;
     r.k_out = k_out == nullptr ? nullptr : static_cast<char*>(k_out) + kv_off;
-    r.positions = positions + t0;
+    r.positions = positions == nullptr ? nullptr : positions + t0;
+    r.rope_rows = rope_rows == nullptr ? nullptr : rope_rows + t0 * 2 * head_dim;
     r.block_ids = block_ids == nullptr ? nullptr : block_ids + t0;
     r.block_offsets = block_offsets == nullptr ? nullptr : block_offsets + t0;
     r.q_blocks = static_cast<uint32_t>((r.tokens * q_heads + rows_per_block - 1) / rows_per_block);
@@ -371,6 +426,59 @@ extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache
     if (int rc = check_launch(op)) return rc;
   }
   return ARENO_OK;
+}
+}  // namespace
+}  // namespace areno
+
+extern "C" int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache, const void* q, const void* k,
+                                                  const void* v, void* q_out, void* k_out, int32_t dtype,
+                                                  int64_t tokens, int32_t q_heads, int32_t kv_heads, int32_t head_dim,
+                                                  const int64_t* positions, const float* cos, const float* sin,
+                                                  int32_t max_pos, const float* q_weight, const float* k_weight,
+                                                  float eps, const int64_t* block_ids, const int64_t* block_offsets,
+                                                  void* stream) {
+  return areno::rope_write_impl("areno_hip_qk_norm_rope_cache_write", cache, q, k, v, q_out, k_out, dtype, tokens, q_heads,
+                                kv_heads, head_dim, positions, cos, sin, max_pos, nullptr, q_weight, k_weight, eps,
+                                block_ids, block_offsets, stream);
+}
+
+extern "C" int areno_hip_qk_norm_rope_cache_write_rows(const areno_paged_cache* cache, const void* q, const void* k,
+                                                       const void* v, void* q_out, void* k_out, int32_t dtype,
+                                                       int64_t tokens, int32_t q_heads, int32_t kv_heads,
+                                                       int32_t head_dim, const float* rope_rows, const float* q_weight,
+                                                       const float* k_weight, float eps, const int64_t* block_ids,
+                                                       const int64_t* block_offsets, void* stream) {
+  const char* op = "areno_hip_qk_norm_rope_cache_write_rows";
+  if (rope_rows == nullptr && tokens > 0) return areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: rope_rows is NULL", op);
+  return areno::rope_write_impl(op, cache, q, k, v, q_out, k_out, dtype, tokens, q_heads, kv_heads, head_dim, nullptr,
+                                nullptr, nullptr, 1, rope_rows, q_weight, k_weight, eps, block_ids, block_offsets, stream);
+}
+
+extern "C" size_t areno_hip_rope_rows_bytes(int64_t tokens, int32_t head_dim) {
+  if (tokens < 0 || head_dim <= 0) return 0;
+  return static_cast<size_t>(tokens) * 2 * static_cast<size_t>(head_dim) * sizeof(float);
+}
+
+extern "C" int areno_hip_rope_rows(float* rows, const int64_t* positions, const float* cos, const float* sin,
+                                   int64_t tokens, int32_t head_dim, int32_t max_pos, int32_t dtype, void* stream) {
+  using namespace areno;
+  const char* op = "areno_hip_rope_rows";
+  if (dtype != ARENO_DT_F16 && dtype != ARENO_DT_BF16)
+    return fail(ARENO_ERR_UNSUPPORTED, "%s: activations must be f16 or bf16", op);
+  if (tokens < 0 || head_dim <= 0 || head_dim % 8 != 0 || max_pos <= 0)
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: sizes out of range (head_dim must be a multiple of 8)", op);
+  if (tokens == 0) return ARENO_OK;
+  if (rows == nullptr || positions == nullptr || cos == nullptr || sin == nullptr)
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", op);
+  if (reinterpret_cast<uintptr_t>(rows) % 16 != 0 || reinterpret_cast<uintptr_t>(cos) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(sin) % 16 != 0)
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: rows / cos / sin must be 16-byte aligned", op);
+  RopeRowsParams p = {rows, positions, cos, sin, tokens, head_dim, max_pos, dtype};
+  const int64_t threads = tokens * (head_dim / 4);
+  const int64_t blocks = (threads + 255) / 256;
+  if (blocks > 0x7fffffffLL) return fail(ARENO_ERR_UNSUPPORTED, "%s: too many tokens for one launch", op);
+  hipLaunchKernelGGL(rope_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+  return check_launch(op);
 }
 
 // Test hook: caps the tokens one launch of the fused front step takes (0 = only the kernel's own limit), so that the

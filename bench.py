@@ -532,20 +532,40 @@ def measure_prefill(w, iters=20):
         )  # fmt: skip
 
     us_front = timed_graph(front)
+    # the same step with the rotary rows of the step's tokens prepared once for all layers (positions are the same in
+    # every layer): the rows kernel's time is spread over the layers it serves
+    rows = ops.areno_rope_rows(positions, cos, sin, w.q.dtype)
+
+    def front_rows():
+        return ops.areno_qk_norm_rope_cache_write(
+            w.q, w.k_new, w.v_new, positions, cos, sin, q_norm_weight=ones, k_norm_weight=ones, eps=1e-6,
+            k_cache=w.k_cache, v_cache=w.v_cache, cache_block_ids=w.cache_block_ids,
+            cache_block_offsets=w.cache_block_offsets, k_scale=w.k_scale, v_scale=w.v_scale, rope_rows=rows,
+        )  # fmt: skip
+
+    rows_equal = all(bool(torch.equal(a, b)) for a, b in zip(front(), front_rows()))
+    us_front_rows = timed_graph(front_rows)
+    us_rows = timed_graph(lambda: ops.areno_rope_rows(positions, cos, sin, w.q.dtype))
     act = w.q.element_size()
     scale_bytes = 0 if w.k_scale is None else 2 * w.k_scale.element_size()
     front_bytes = t * ((hq + 2 * hkv) * d * act + (hq + hkv) * d * act + hkv * (2 * d * w.k_cache.element_size() + scale_bytes))
+    us_front_step = us_front_rows + us_rows / LAYERS_PER_PLAN
     write()  # leave the pages as the attention measurement expects them
     flops = w.flops()
     tflops = flops / (us_attend * 1e-6) / 1e12
     return {
         "workload": w.name,
         "us_per_step": us_attend + us_write,
-        "kernel_us": {"cache_write": us_write, "prefill": us_attend, "qk_norm_rope_cache_write": us_front},
+        "kernel_us": {"cache_write": us_write, "prefill": us_attend, "qk_norm_rope_cache_write": us_front,
+                      "qk_norm_rope_cache_write_from_rows": us_front_rows, "rope_rows": us_rows},
         "prefill_us_p10_p90": spread["prefill"],
         "qk_norm_rope_cache_write": {
             "us": us_front, "algorithmic_bytes": front_bytes, "gbps": front_bytes / (us_front * 1e-6) / 1e9,
             "frac_of_hbm_peak": front_bytes / (us_front * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+            # with the step's rotary rows prepared once per LAYERS_PER_PLAN layers (their share of that launch included)
+            "us_from_rows": us_front_step, "rows_kernel_us": us_rows, "layers_per_rows": LAYERS_PER_PLAN,
+            "frac_of_hbm_peak_from_rows": front_bytes / (us_front_step * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+            "rows_equal_tables_bitwise": rows_equal,
         },  # fmt: skip
         "new_tokens": int(w.q.shape[0]),
         "tokens_per_s": w.q.shape[0] / ((us_attend + us_write) * 1e-6),

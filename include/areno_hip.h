@@ -276,6 +276,30 @@ int areno_hip_qk_norm_rope_cache_write(const areno_paged_cache* cache, const voi
                                        const int64_t* block_offsets, void* stream);
 
 /*
+ * The rotary rows of a step's tokens, prepared once for all layers.  position_ids are the same for every layer of a
+ * step (the reference passes one tensor down the stack, areno/engine/layers/attention.py:94-96), and what the fused
+ * step above does with them -- fetch the token's cosines and sines, cast them to the activation dtype as the eager
+ * ops do (areno/engine/layers/rotary.py:46-52) -- it otherwise repeats for every (token, head) row of every layer.
+ * No counterpart in the reference, whose RotaryEmbedding indexes and casts the tables per call.
+ *   areno_hip_rope_rows_bytes(tokens, head_dim)   bytes of the rows: tokens * 2 * head_dim floats
+ *   areno_hip_rope_rows(...)                      one launch: rows[t] = { dtype(cos[pos_t]) , +-dtype(sin[pos_t]) } as
+ *                                                 floats, the sign of rotate_half on the sines (minus for the first
+ *                                                 half of the head); positions clamped into [0, max_pos); head_dim a
+ *                                                 multiple of 8; rows, cos and sin 16-byte aligned
+ *   areno_hip_qk_norm_rope_cache_write_rows(...)  areno_hip_qk_norm_rope_cache_write with rope_rows (for the same
+ *                                                 tokens in the same order, built for the same dtype) in place of
+ *                                                 positions, cos, sin and max_pos; same results, bit for bit
+ */
+size_t areno_hip_rope_rows_bytes(int64_t tokens, int32_t head_dim);
+int areno_hip_rope_rows(float* rows, const int64_t* positions, const float* cos, const float* sin, int64_t tokens,
+                        int32_t head_dim, int32_t max_pos, int32_t dtype, void* stream);
+int areno_hip_qk_norm_rope_cache_write_rows(const areno_paged_cache* cache, const void* q, const void* k, const void* v,
+                                            void* q_out, void* k_out, int32_t dtype, int64_t tokens, int32_t q_heads,
+                                            int32_t kv_heads, int32_t head_dim, const float* rope_rows,
+                                            const float* q_weight, const float* k_weight, float eps,
+                                            const int64_t* block_ids, const int64_t* block_offsets, void* stream);
+
+/*
  * Bytes of device workspace the two prefill entry points above need (the reference allocates nothing here: its
  * varlen kernel keeps one query row per thread block, areno/accel/csrc/attention.cu:145-242).  The matrix-core
  * kernels cut the work into equal shares of key tiles whatever the length distribution, and a query block cut by a

@@ -120,6 +120,54 @@ def test_token_ranges_give_what_one_launch_gives():
         assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"{name} differ between one launch and eleven"
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (28, 4, 128), (4, 4, 256), (2, 2, 512)])
+def test_prepared_rotary_rows_give_the_same_bits(dtype, hq, hkv, d):
+    """areno_rope_rows prepares a step's cosines and sines once (rounded to the activation dtype, rotate_half's sign
+    on the sines); every layer's fused call then takes them as rope_rows.  Outputs and pages must be what the call
+    with positions and tables gives, bit for bit -- with positions outside the table (clamped by both), with and
+    without the norm, and when the call runs as several launches over token ranges."""
+    import ctypes
+
+    from areno_amd.accel import cabi
+
+    t, bs, nb = 61, 16, 8
+    q, k, v, pos, cos, sin, qw, kw = _inputs(t, hq, hkv, d, dtype, seed=3 * d + hq, max_pos=512)
+    pos[1], pos[2] = -5, 100_000  # clamped into the table by both paths
+    rows = ops.areno_rope_rows(pos.to(DEV), cos.to(DEV), sin.to(DEV), dtype)
+    assert rows.shape == (t, 2, d) and rows.dtype == torch.float32
+    pc = pos.clamp(0, 511)
+    assert torch.equal(rows[:, 0].cpu(), cos[pc].to(dtype).float())
+    sign = torch.cat([-torch.ones(d // 2), torch.ones(d // 2)])
+    assert torch.equal(rows[:, 1].cpu(), sin[pc].to(dtype).float() * sign)
+    g = torch.Generator().manual_seed(9)
+    slots = torch.randperm(nb * bs, generator=g)[:t]
+    ids, offs = (slots // bs).to(DEV), (slots % bs).to(DEV)
+    lib = cabi.lib()
+    lib.areno_hip_debug_set_rope_tokens_per_launch.restype = ctypes.c_int64
+    lib.areno_hip_debug_set_rope_tokens_per_launch.argtypes = [ctypes.c_int64]
+    for norm, cap in ((True, 0), (False, 0), (True, 7)):
+        weights = dict(q_norm_weight=qw.to(DEV), k_norm_weight=kw.to(DEV)) if norm else {}
+        results = []
+        for use_rows in (False, True):
+            layer = allocate_kv_caches(1, nb, bs, hkv, d, DEV, dtype, "int8")[0]
+            layer.k_cache.view(torch.uint8).fill_(0x11)
+            layer.v_cache.view(torch.uint8).fill_(0x11)
+            before = lib.areno_hip_debug_set_rope_tokens_per_launch(cap)
+            try:
+                q_out, k_out = ops.areno_qk_norm_rope_cache_write(
+                    q.to(DEV), k.to(DEV), v.to(DEV), pos.to(DEV), cos.to(DEV), sin.to(DEV), eps=1e-6,
+                    k_cache=layer.k_cache, v_cache=layer.v_cache, cache_block_ids=ids, cache_block_offsets=offs,
+                    k_scale=layer.k_scale, v_scale=layer.v_scale, rope_rows=rows if use_rows else None, **weights,
+                )  # fmt: skip
+                torch.cuda.synchronize()
+            finally:
+                lib.areno_hip_debug_set_rope_tokens_per_launch(before)
+            results.append((q_out, k_out, layer.k_cache, layer.v_cache, layer.k_scale, layer.v_scale))
+        for a, b, name in zip(results[0], results[1], ("q_out", "k_out", "k pages", "v pages", "k scales", "v scales")):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"{name} differ (norm={norm}, cap={cap})"
+
+
 def test_argument_checks():
     q, k, v, pos, cos, sin, qw, kw = _inputs(4, 4, 2, 128, torch.bfloat16, seed=1)
     with pytest.raises(RuntimeError, match="requires CUDA"):
