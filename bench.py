@@ -34,8 +34,8 @@ POOL_TARGET_BYTES = 1.3e9  # rotate over at least this much distinct KV
 # HBM bytes per launch of the dominant kernel as two rocprofv3 counter runs of this script recorded them (FETCH_SIZE,
 # scaled by the factor 2.0 that a copy of known size gives for it, plus WRITE_SIZE).  Recorded constants, not
 # measurements of the present run: the summaries they come from are under profiles/.
-PROFILED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 311.02e6, "cfg2-qwen7b-int8": 153.95e6, "cfg3-rollout-fp8": 1066.22e6,
-                          "cfg4-prefill-fp8": 1624.94e6}
+PROFILED_TRAFFIC_BYTES = {"cfg1-qwen7b-bf16": 311.03e6, "cfg2-qwen7b-int8": 153.97e6, "cfg3-rollout-fp8": 1065.92e6,
+                          "cfg4-prefill-fp8": 1624.87e6}
 PROFILED_TRAFFIC_SOURCE = {
     "decode": "recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script: profiles/decode_mfma_kernel_hbm_traffic_cfg1_cfg2_cfg3.md",
     "prefill": "recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script: profiles/prefill_mfma_kernel_hbm_traffic_cfg4.md",
@@ -713,6 +713,9 @@ def main() -> int:
     ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg2_b256"], default=None,
                     help="measure a single workload")  # fmt: skip
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--skip-other-shapes", action="store_true",
+                    help="leave out the probe of decode shapes next to the benchmark's (for profiler runs, whose per-kernel "
+                         "averages should belong to the benchmark's workloads)")
     ap.add_argument("--plan", choices=["both", "only", "off"], default="both",
                     help="decode workloads: time the steps with a per-step plan and without one (both), or only one of the "
                          "two (for profiler runs whose per-kernel averages should belong to one of them)")  # fmt: skip
@@ -762,7 +765,7 @@ def main() -> int:
         del w
         torch.cuda.empty_cache()
 
-    if not args.only:
+    if not args.only and not args.skip_other_shapes:
         results["other_shapes"] = measure_other_shapes(dev)
 
     head = results[names[0]]
