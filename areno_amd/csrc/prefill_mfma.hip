@@ -3,7 +3,8 @@
 // Work item = (sequence, kv head, block of query tokens).  The G query heads of the kv head are folded into the
 // query-row axis: row r of the block is (token r / GP, head r % GP) with GP = G rounded up to a power of two, so one
 // 16-row MFMA tile holds 16 / GP tokens of all heads and K/V are read once for the whole group (GQA without
-// expanding KV, as areno/accel/csrc/attention.cu:170-171 does per row).  A block is 256 rows: each of the 8 waves
+// expanding KV, as areno/accel/csrc/attention.cu:170-171 does per row; a kv head with more than 16 q heads runs as
+// several workgroup rows, 16 q heads each).  A block is 256 rows: each of the 8 waves
 // owns 32 (two 16-row tiles; one at head dims 192 and 256, and at 512 two waves share one).  One such workgroup per
 // CU (the registers allow two waves per SIMD either way; eight waves behind one set of K/V tiles halve the staging
 // work per wave against two workgroups of four).
@@ -81,21 +82,22 @@ struct PrefillParams {
   const int32_t* block_table;
   const int32_t* cu_seqlens_q;
   const int32_t* context_lens;
-  float* part_ml;   // [2 * units][kv_heads][rows_per_wg][2]
-  float* part_acc;  // [2 * units][kv_heads][rows_per_wg][head_dim]
+  float* part_ml;   // [2 * units][kv_heads * head_parts][rows_per_wg][2]
+  float* part_acc;  // [2 * units][kv_heads * head_parts][rows_per_wg][head_dim]
   int32_t num_seqs;
   int32_t q_heads;
   int32_t kv_heads;
   int32_t head_dim;
   int32_t group;        // q heads per kv head
-  int32_t group_pad;    // rounded up to a power of two (<= 16)
+  int32_t head_parts;   // workgroup rows (blockIdx.y) per kv head: ceil(group / 16); each takes up to 16 of its q heads
+  int32_t group_pad;    // q heads of one part rounded up to a power of two (<= 16)
   int32_t group_shift;  // log2(group_pad)
   int32_t block_size;
   int32_t bs_shift;
   int32_t max_blocks;
   int32_t window_left;
   int32_t q_dtype;
-  int32_t units;        // per kv head
+  int32_t units;        // per (kv head, part)
   int32_t rows_per_wg;  // query rows of one item: 64 per 16-row tile a wave owns
   float scale_log2e;
 };
@@ -274,7 +276,12 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
   const int d0 = dpart * DW;
   const int lr = lane & 15;
   const int lk = lane >> 4;
-  const int kvh = blockIdx.y;
+  // a kv head with more than 16 q heads runs as several "heads", each with up to 16 of them, that read the same K/V
+  const int vhead = blockIdx.y;
+  const int kvh = p.head_parts > 1 ? vhead / p.head_parts : vhead;
+  const int head0 = kvh * p.group + 16 * (vhead - kvh * p.head_parts);   // first q head of this part
+  const int group_here = min(16, (kvh + 1) * p.group - head0);           // q heads of this part
+  const int vheads = p.kv_heads * p.head_parts;
   const int unit = blockIdx.x;
   const int tq = kRowsPerWg >> p.group_shift;  // query tokens per item
 
@@ -340,9 +347,9 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
       const int r = row_wave * kRowsPerWave + 16 * nq + lr;
       const int t = r >> p.group_shift;
       const int hh = r & (p.group_pad - 1);
-      const bool live = t < tok_cnt && hh < p.group;
+      const bool live = t < tok_cnt && hh < group_here;
       q_pos[nq] = live ? ctx + tok0 + t : -1;
-      row_elem[nq] = (static_cast<int64_t>(q_begin + tok0 + t) * p.q_heads + kvh * p.group + hh) * D;
+      row_elem[nq] = (static_cast<int64_t>(q_begin + tok0 + t) * p.q_heads + head0 + hh) * D;
 #pragma unroll
       for (int sl = 0; sl < NS; ++sl) {
         uint4_t w = {0u, 0u, 0u, 0u};
@@ -742,7 +749,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
         }
       } else {
         const int r = row_wave * kRowsPerWave + 16 * nq + lr;
-        const int64_t prow = (static_cast<int64_t>(slot) * p.kv_heads + kvh) * kRowsPerWg + r;
+        const int64_t prow = (static_cast<int64_t>(slot) * vheads + vhead) * kRowsPerWg + r;
         float* dst = p.part_acc + prow * D + d0 + 4 * lk;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) *reinterpret_cast<float4_t*>(dst + 16 * nb) = acc[nq][nb];
@@ -783,7 +790,11 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
   __shared__ int s_wave_tot[kPrefillWaves];
   const int tid = threadIdx.x;
   const int unit = blockIdx.x;
-  const int kvh = blockIdx.y;
+  const int vhead = blockIdx.y;
+  const int kvh = p.head_parts > 1 ? vhead / p.head_parts : vhead;
+  const int head0 = kvh * p.group + 16 * (vhead - kvh * p.head_parts);
+  const int group_here = min(16, (kvh + 1) * p.group - head0);
+  const int vheads = p.kv_heads * p.head_parts;
   const int kRowsPerWg = p.rows_per_wg;
   const int tq = kRowsPerWg >> p.group_shift;
   const int d = p.head_dim;
@@ -814,12 +825,12 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
   for (int r = tid / parts; r < kRowsPerWg && tid < rows_per_pass * parts; r += rows_per_pass) {
     const int t = r >> p.group_shift;
     const int hh = r & (p.group_pad - 1);
-    if (t >= item.cnt || hh >= p.group) continue;
+    if (t >= item.cnt || hh >= group_here) continue;
     float m = kNegInf;
     for (int u = unit; u <= u_hi; ++u) {
       if (unit_start_step(total, u, p.units) == unit_start_step(total, u + 1, p.units)) continue;  // empty unit
       const int slot = 2 * u + ((u == unit && pos.item_x0 > x_begin) ? 1 : 0);
-      const int64_t prow = (static_cast<int64_t>(slot) * p.kv_heads + kvh) * kRowsPerWg + r;
+      const int64_t prow = (static_cast<int64_t>(slot) * vheads + vhead) * kRowsPerWg + r;
       const float pm = p.part_ml[prow * 2];
       const float pl = p.part_ml[prow * 2 + 1];
       if (pl != 0.0f) m = fmaxf(m, pm);
@@ -832,7 +843,7 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
     for (int u = unit; u <= u_hi; ++u) {
       if (unit_start_step(total, u, p.units) == unit_start_step(total, u + 1, p.units)) continue;
       const int slot = 2 * u + ((u == unit && pos.item_x0 > x_begin) ? 1 : 0);
-      const int64_t prow = (static_cast<int64_t>(slot) * p.kv_heads + kvh) * kRowsPerWg + r;
+      const int64_t prow = (static_cast<int64_t>(slot) * vheads + vhead) * kRowsPerWg + r;
       const float pl = p.part_ml[prow * 2 + 1];
       if (pl == 0.0f) continue;  // a partial without visible keys
       const float w = fast_exp2(p.part_ml[prow * 2] - m_safe);
@@ -849,7 +860,7 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
     }
     const float inv = 1.0f / lsum;
     const int64_t out_elem =
-        (static_cast<int64_t>(q_begin + item.tok0 + t) * p.q_heads + kvh * p.group + hh) * d + half * dh;
+        (static_cast<int64_t>(q_begin + item.tok0 + t) * p.q_heads + head0 + hh) * d + half * dh;
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c) {
       if (c >= chunks) continue;
@@ -957,8 +968,10 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   if (q_dtype != ARENO_DT_F16 && q_dtype != ARENO_DT_BF16) return ARENO_ERR_UNSUPPORTED;
   if (!(softmax_scale > 0.0f)) return ARENO_ERR_UNSUPPORTED;  // the kernel takes row maxima before scaling
   if (log2_exact_i(cache->block_size) < 0) return ARENO_ERR_UNSUPPORTED;  // page addressing by shift and mask
-  if (group > 16 || num_seqs > kMaxPrefillSeqs || tokens > 0x3fffffff) return ARENO_ERR_UNSUPPORTED;
-  if (cache->kv_heads > 65535) return ARENO_ERR_UNSUPPORTED;
+  const int head_parts = (group + 15) / 16;
+  const int vheads = cache->kv_heads * head_parts;
+  if (head_parts > 8 || num_seqs > kMaxPrefillSeqs || tokens > 0x3fffffff) return ARENO_ERR_UNSUPPORTED;
+  if (vheads > 65535) return ARENO_ERR_UNSUPPORTED;
   // page rows (block id * page size + slot, or token rows of packed K/V) are 32-bit in the kernel's address arithmetic
   if (block_table != nullptr && cache->num_blocks * cache->block_size > 0xffffffffLL) return ARENO_ERR_UNSUPPORTED;
   if (reinterpret_cast<uintptr_t>(cache->k) % 16 != 0 || reinterpret_cast<uintptr_t>(cache->v) % 16 != 0 ||
@@ -981,11 +994,14 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   const int64_t max_keys = block_table != nullptr ? static_cast<int64_t>(max_blocks) * cache->block_size : tokens;
   {
     int gp = 1;
-    while (gp < group) gp <<= 1;
+    while (gp < (head_parts > 1 ? 16 : group)) gp <<= 1;
     const int64_t items = tokens / (rows_per_wg / gp) + num_seqs;
     if (items * (max_keys / kTileTokens + 1) > 0x7fffffffLL) return ARENO_ERR_UNSUPPORTED;
   }
+  // (the partials of a launch laid out over (kv head, part) pairs never need more than the kv heads alone would,
+  // except when the pairs outnumber the launch's workgroups: then the generic kernel takes the call)
   const size_t need = prefill_mfma_workspace_bytes(cache->kv_heads, cache->head_dim);
+  if (head_parts > 1 && prefill_mfma_workspace_bytes(vheads, cache->head_dim) > need) return ARENO_ERR_UNSUPPORTED;
   if (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
     return fail(ARENO_ERR_WORKSPACE, "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", op, need,
                 workspace_bytes);
@@ -1005,20 +1021,21 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   p.kv_heads = cache->kv_heads;
   p.head_dim = cache->head_dim;
   p.group = group;
+  p.head_parts = head_parts;
   p.group_pad = 1;
-  while (p.group_pad < group) p.group_pad <<= 1;
+  while (p.group_pad < (head_parts > 1 ? 16 : group)) p.group_pad <<= 1;
   p.group_shift = log2_exact_i(p.group_pad);
   p.block_size = cache->block_size;
   p.bs_shift = log2_exact_i(cache->block_size);
   p.max_blocks = max_blocks;
   p.window_left = window_left;
   p.q_dtype = q_dtype;
-  p.units = prefill_units(cache->kv_heads);
+  p.units = prefill_units(vheads);
   p.rows_per_wg = rows_per_wg;
   p.scale_log2e = softmax_scale * kLog2e;
   p.part_ml = static_cast<float*>(workspace);
-  p.part_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + prefill_ml_bytes(p.units, cache->kv_heads));
-  const dim3 grid(p.units, cache->kv_heads);
+  p.part_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + prefill_ml_bytes(p.units, vheads));
+  const dim3 grid(p.units, vheads);
   hipLaunchKernelGGL(fn, grid, dim3(kPrefillThreads), 0, static_cast<hipStream_t>(stream), p);
   if (int rc = check_launch(op)) return rc;
   hipLaunchKernelGGL(prefill_merge_kernel, grid, dim3(kPrefillThreads), 0, static_cast<hipStream_t>(stream), p);

@@ -22,7 +22,7 @@ def _packed(lens, hq, hkv, d, dtype, seed=0):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("window_left", [None, 0, 7])
-@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (28, 4, 128), (4, 4, 80), (8, 2, 256), (6, 6, 192), (8, 2, 512)])
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (28, 4, 128), (4, 4, 80), (8, 2, 256), (6, 6, 192), (8, 2, 512), (40, 2, 128)])
 def test_varlen_new_tokens_only(dtype, window_left, hq, hkv, d):
     q, k, v, cu = _packed([5, 1, 130, 0, 67], hq, hkv, d, dtype)
     out = ops.areno_varlen_causal_attention(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), window_left=window_left)
@@ -81,7 +81,12 @@ def test_paged_prefill_small(kv, window_left):
     assert_close(out, _expected_prefill(w, window_left), *tolerances(kv), what=f"paged prefill {kv}")
 
 
-@pytest.mark.parametrize("hq,hkv,d,bs", [(28, 4, 128, 16), (8, 8, 64, 32), (6, 2, 128, 256), (4, 1, 96, 16)])
+@pytest.mark.parametrize("hq,hkv,d,bs", [
+    (28, 4, 128, 16), (8, 8, 64, 32), (6, 2, 128, 256), (4, 1, 96, 16),
+    # more than 16 q heads per kv head: several workgroup rows per kv head, 16 q heads each (16 + 16, 16 + 4, 16 + 8 at
+    # head dim 256, 16 + 16 + 1)
+    (32, 1, 128, 16), (40, 2, 64, 32), (24, 1, 256, 16), (33, 1, 128, 16),
+])  # fmt: skip
 def test_paged_prefill_shapes(hq, hkv, d, bs):
     g = torch.Generator().manual_seed(d + hq)
     new = torch.tensor([1, 64, 17, 129])
