@@ -106,7 +106,7 @@ def test_shapes_head_ratios_and_block_sizes(kv, hq, hkv, d, bs):
 
 @pytest.mark.parametrize("kv", ["bf16", "fp16", "int8", "fp8"])
 @pytest.mark.parametrize("d", [256, 192, 512])
-@pytest.mark.parametrize("hq,hkv,window_left", [(16, 8, None), (8, 2, None), (4, 1, 300), (24, 4, None)])
+@pytest.mark.parametrize("hq,hkv,window_left", [(16, 8, None), (8, 2, None), (4, 1, 300), (24, 4, None), (40, 2, None)])
 def test_head_dims_192_256_512_on_the_matrix_core_kernel(kv, d, hq, hkv, window_left):
     """Head dims 256 (Gemma-family sliding layers, Qwen3.5), 192 (128 + 64 rotary channels of MLA-style layers) and
     512 (Gemma-family full-attention layers): two, three resp. four waves share a head, each with a part of the head dimension, and exchange their parts of the
