@@ -11,7 +11,10 @@ Prints ONE JSON line.  `value` is microseconds per step: the median of 15 timing
 from HIP graphs (how the engine runs decode), `value_p10_p90` their spread.  The steps run as an engine runs the
 layers of a model: block table and lengths are the same for every layer of a decode step, so one plan launch
 (`areno_hip_paged_decode_plan`) serves 28 steps; it is part of the timed sequence.  `value_without_plan` is the same
-sequence with every step deriving its work list by itself.  `roofline` is for the split-KV kernel alone: algorithmic
+sequence with every step deriving its work list by itself.  Every timing is bracketed by `torch.cuda.synchronize()`,
+so it carries the host's launch of the first graph and its wake-up once (`host_bracket_us`, timed by itself on a
+graph of one tiny kernel: 30-45 us, i.e. ~0.2 us per step at the default 200 steps and ~1.5 us at 20);
+`value_on_device` is the same samples by events on the stream, without that.  `roofline` is for the split-KV kernel alone: algorithmic
 bytes of one launch divided by its mean duration measured with events on the launch stream, next to what a plain reader
 of the same pools reaches (`stream_ceiling_*`); `cpu_baseline` is the CPU oracle timed on the host cores.
 """
@@ -163,23 +166,51 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
         for _ in range(max(1, -(-warmup // full_n))):
             full.replay()
         torch.cuda.synchronize()
-        samples = []
+        samples, on_device = [], []
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         for _ in range(repeats):
             t0 = time.perf_counter()
+            first.record()
             for _ in range(steps // full_n):
                 full.replay()
             if rem is not None:
                 rem.replay()
+            last.record()
             torch.cuda.synchronize()
             samples.append((time.perf_counter() - t0) / steps * 1e6)
+            on_device.append(first.elapsed_time(last) * 1e3 / steps)
         samples.sort()
         # graph replays must reproduce the eager result (checked on the first pool)
-        return statistics.median(samples), [samples[len(samples) // 10], samples[(len(samples) * 9) // 10]], bool(torch.equal(keep_full[0], out))
+        return (statistics.median(samples), [samples[len(samples) // 10], samples[(len(samples) * 9) // 10]],
+                bool(torch.equal(keep_full[0], out)), statistics.median(on_device))  # fmt: skip
+
+    def host_bracket():
+        """What the bracket around a timed sample costs by itself: the host's launch of one graph and its wake-up from
+        torch.cuda.synchronize(), on a graph of one tiny kernel.  A sample of `steps` steps carries it once."""
+        flag = torch.zeros(1, device=w.q.device)
+        side2 = torch.cuda.Stream()
+        side2.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side2):
+            flag.zero_()
+        torch.cuda.current_stream().wait_stream(side2)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            flag.zero_()
+        times = []
+        for _ in range(31):
+            t0 = time.perf_counter()
+            g.replay()
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e6)
+        return statistics.median(times[1:])
 
     with_plan, without_plan = plan_mode != "off", plan_mode != "only"
     nan = float("nan")
-    us_graph, us_graph_spread, graph_ok = timed_replays(True) if with_plan else (nan, [nan, nan], True)
-    us_graph_plain, us_graph_plain_spread, graph_plain_ok = timed_replays(False) if without_plan else (nan, [nan, nan], True)
+    us_graph, us_graph_spread, graph_ok, us_graph_device = timed_replays(True) if with_plan else (nan, [nan, nan], True, nan)
+    us_graph_plain, us_graph_plain_spread, graph_plain_ok, us_graph_plain_device = (
+        timed_replays(False) if without_plan else (nan, [nan, nan], True, nan))  # fmt: skip
+    us_bracket = host_bracket()
 
     # ---- whole op, eager launches (host launch overhead included), a plan per LAYERS_PER_PLAN steps ------------------
     def eager(n):
@@ -252,12 +283,18 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
 
     if not with_plan:  # a run without plans reports the plain launches as the step and as the kernel
         us_graph, us_graph_spread, us_split = us_graph_plain, us_graph_plain_spread, us_split_plain
+        us_graph_device = us_graph_plain_device
     gbps = alg_bytes / (us_split * 1e-6) / 1e9
     ceiling = measure_stream_ceiling(w, pools)
     return {
         "workload": w.name,
         "us_per_step": us_graph,
         "us_per_step_p10_p90": us_graph_spread,
+        # the same samples by events on the stream (first replay's start to last replay's end): without the host's
+        # launch of the first graph and its wake-up from the synchronize, which `host_bracket_us` times on a graph of
+        # one tiny kernel and which a sample of `steps` steps carries once
+        "us_per_step_on_device": us_graph_device,
+        "host_bracket_us": us_bracket,
         "us_per_step_without_plan": us_graph_plain,
         "us_per_step_without_plan_p10_p90": us_graph_plain_spread,
         "us_per_step_eager": us_eager,
@@ -791,6 +828,8 @@ def main() -> int:
                     f"{LAYERS_PER_PLAN} steps, inside the timed region" if "plan" in head else "one paged prefill",
         },
         "value_p10_p90": head.get("us_per_step_p10_p90"),
+        "value_on_device": head.get("us_per_step_on_device"),
+        "host_bracket_us": head.get("host_bracket_us"),
         "value_without_plan": head.get("us_per_step_without_plan"),
         "tokens_per_s": head["tokens_per_s"],
         "hbm_gbps_op": head.get("op_gbps"),
