@@ -148,28 +148,67 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_kernel(Decod
 // Memory round trips, which are what this kernel's time is made of: (1) the row's entry of the plan (or the prefix
 // sums its units follow from), its length and the q / k_update / v_update rows; (2) the append's block id and, for up
 // to kMergeChunk candidates at once, (m, l) and the accumulator row together -- a candidate's row is fetched before
-// its weight is known, rows of absent candidates are dropped after the fact; (3) the stores.
+// its weight is known; (3) the stores.
 constexpr int kMergeChunk = 8;
 
 // The arguments in front of the parameter block are what the kernel's first loads are addressed with: as leading
 // scalar arguments they reach the wave in registers at its start (kernel-argument preload, at most 16 words), while
 // the block behind them takes a fetch of its own.
-template <int EPW>  // head-dimension elements per lane: head_dim <= 64 EPW
-__global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel(
+//
+// The kernel's time is those round trips plus what a wave issues in between, and with seven waves on a CU nothing
+// hides a wave's own instructions, so the kernel is instantiated for what would otherwise be decided at run time --
+// the query dtype (QDT), the cache dtype (CDT: QDT itself for 16-bit pages, ARENO_DT_I8, ARENO_DT_FP8_E4M3), whether
+// a plan brings the row's unit ranges (PLANNED) -- and its index arithmetic avoids divisions: the grid is (q heads /
+// kReduceRows, rows), the kv head of a q head and the page column of a position are multiplications by constants the
+// launcher derives; candidates of a kind sit a constant stride apart, so their addresses are a base plus a multiple.
+// Against a kernel that decided all of this at run time: a fifth of the instructions, 5.6 instead of 7.6 us per launch
+// at batch 64.
+
+// Candidates of one round trip: (m, l) and the lane's elements of the accumulator row.
+template <int N, int EPW>
+struct MergeChunk {
+  static constexpr int kSize = N;
+  float m[N], l[N];
+  float v[N][EPW];
+};
+
+// Whether unit u of a launch with fewer cost positions than units (total < units: tiny batches) holds none:
+// floor(u total / units) == floor((u + 1) total / units), i.e. (u total mod units) + total < units.  The product is
+// below 2^20 (at most 1 024 units), so the quotient comes from a float multiplication and one correction either way
+// instead of a division.
+__device__ __forceinline__ bool unit_is_empty(int total, int units, float units_rcp, int u) {
+  const int a = u * total;
+  int r = a - static_cast<int>(static_cast<float>(a) * units_rcp) * units;
+  r += r < 0 ? units : 0;
+  r -= r >= units ? units : 0;
+  return r + total < units;
+}
+
+// The kernel keeps to few registers (48 at head dim 128): a variant that fetched 32 candidates per round trip for rows
+// with many of them took 160 and every launch of it twice as long, whether or not a row had that many.  Rows with many
+// candidates -- a small batch spreads each row over all units: 256 candidates at batch 1 -- are served by more waves
+// instead: MW waves share a (row, head), wave w takes the chunks w, w + MW, ..., and wave 0 combines their results
+// through LDS (MW = 1: a workgroup of kReduceRows waves takes that many heads of a row, no LDS).  The launcher picks
+// MW from the batch size and the number of units, which is all it knows of the lengths.
+template <int EPW, int QDT, int CDT, bool PLANNED, int MW>  // EPW: head-dimension elements per lane, head_dim <= 64 EPW
+__global__ __launch_bounds__((MW == 1 ? kReduceRows : MW) * kWave) void decode_reduce_slots_kernel(
     const int32_t* plan_rows, const int32_t* cache_seqlens, const void* q_rows, const void* k_update,
-    const void* v_update, int32_t total_rows, int32_t q_heads, int32_t kv_heads, int32_t group, int32_t head_dim,
-    int32_t q_dtype, MfmaDecodeParams mp) {
+    const void* v_update, int32_t q_heads, int32_t kv_heads, int32_t group, uint32_t group_magic, int32_t head_dim,
+    MfmaDecodeParams mp) {
   const DecodeParams& p = mp.d;
   const int lane = threadIdx.x & (kWave - 1);
-  const int row = blockIdx.x * kReduceRows + (threadIdx.x >> 6);
-  if (row >= total_rows) return;
-  const int b = row / q_heads;
-  const int h = row - b * q_heads;
-  const int kvh = h / group;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // (in a scalar register)
+  const int b = blockIdx.y;
+  const int h = MW == 1 ? blockIdx.x * kReduceRows + wave : blockIdx.x;
+  const int part = MW == 1 ? 0 : wave;  // which share of the row's candidates this wave merges
+  if (h >= q_heads) return;
+  const int row = b * q_heads + h;
+  const int kvh = group == 1 ? h : static_cast<int>(__umulhi(static_cast<uint32_t>(h), group_magic));  // h / group
   const int d = head_dim;
   const ItemShape& shape = mp.items;
-  const int num_items = shape.num_items();
-  const bool append = k_update != nullptr;  // (the launcher passes the update rows only when this launch folds them in)
+  // (the launcher passes the update rows only when this launch folds them in; of the waves that share a row, the first
+  // one takes the new token)
+  const bool append = k_update != nullptr && part == 0;
 
   // ---- round trip 1 ---------------------------------------------------------------------------------------------------
   // units that hold partials of the row: its own item's and, with prefix groups, its sub-group's shared item's
@@ -181,52 +220,53 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
     const int j = (b - gi * shape.group_rows) / shape.cols_seqs;
     sh_item = gi * shape.subs_per_group + j;
     const int first_row = gi * shape.group_rows + j * shape.cols_seqs;
-    sh_col = kvh * 16 + (b - first_row) * p.group + (h - kvh * p.group);
+    sh_col = kvh * 16 + (b - first_row) * group + (h - kvh * group);
   }
-  if (plan_rows != nullptr) {
+  if constexpr (PLANNED) {
     planned_units = *reinterpret_cast<const int4_t*>(plan_rows + 4 * static_cast<int64_t>(b));
     cum_total = plan_rows[-4];
   } else {
     const int32_t* cum = mp.cum_out;
     const int v_own = shape.num_shared + b;
-    cum_total = cum[num_items];
+    cum_total = cum[shape.num_items()];
     cum_own = cum[v_own];
     cum_own_end = cum[v_own + 1];
-    if (shape.num_shared > 0) {
-      cum_sh = cum[sh_item];
-      cum_sh_end = cum[sh_item + 1];
-    }
+    cum_sh = cum[sh_item];  // (entry 0 and 1 when there are no shared items: read and not used)
+    cum_sh_end = cum[sh_item + 1];
   }
-  float qv[EPW], kx[EPW], vx[EPW];
-  uint16_t kraw[EPW], vraw[EPW];
-  int64_t pos = 0;
-  if (append) {
+  // the update rows and the query row (stand-ins from the query tensor when nothing is appended: read, not used)
+  uint16_t qraw[EPW], kraw[EPW], vraw[EPW];
+  const int pos = cache_seqlens[b];
+  {
+    const uint16_t* ksrc = static_cast<const uint16_t*>(append ? k_update : q_rows);
+    const uint16_t* vsrc = static_cast<const uint16_t*>(append ? v_update : q_rows);
     const int64_t src_base = (static_cast<int64_t>(b) * kv_heads + kvh) * d;
-    pos = cache_seqlens[b];
+    const int64_t q_base = static_cast<int64_t>(row) * d;
 #pragma unroll
     for (int e = 0; e < EPW; ++e) {
-      const int idx = lane + e * kWave;
-      const bool in = idx < d;
-      kraw[e] = in ? static_cast<const uint16_t*>(k_update)[src_base + idx] : 0;
-      vraw[e] = in ? static_cast<const uint16_t*>(v_update)[src_base + idx] : 0;
-      qv[e] = in ? load_as_float(q_rows, static_cast<int64_t>(row) * d + idx, q_dtype) : 0.0f;
+      const int idx = min(lane + e * kWave, d - 1);
+      kraw[e] = ksrc[src_base + idx];
+      vraw[e] = vsrc[src_base + idx];
+      qraw[e] = static_cast<const uint16_t*>(q_rows)[q_base + idx];
     }
   }
+  auto widen = [](uint16_t raw) { return QDT == ARENO_DT_BF16 ? bf16_bits_to_float(raw) : f16_bits_to_float(raw); };
   // (with fewer cost positions than units a candidate's unit may be empty and have written nothing)
   const bool every_unit_has_quanta = cum_total >= mp.num_units;
-  const UnitGeometry geo = make_unit_geometry(cum_total, mp.num_units);
-  if (plan_rows != nullptr) {
+  const float units_rcp = 1.0f / static_cast<float>(mp.num_units);
+  if constexpr (PLANNED) {
     own_lo = planned_units[0];
     own_n = planned_units[1];
     sh_lo = planned_units[2];
     sh_n = planned_units[3];
   } else {
+    const UnitGeometry geo = make_unit_geometry(cum_total, mp.num_units);
     if (cum_own_end > cum_own) {
       int last;
       item_units(geo, shape.switch_quanta, cum_own, cum_own_end, own_lo, last);
       own_n = last - own_lo + 1;
     }
-    if (cum_sh_end > cum_sh) {
+    if (shape.num_shared > 0 && cum_sh_end > cum_sh) {
       int last;
       item_units(geo, shape.switch_quanta, cum_sh, cum_sh_end, sh_lo, last);
       sh_n = last - sh_lo + 1;
@@ -234,59 +274,61 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   }
   const int total = own_n + sh_n;
 
-  // ---- round trip 2: candidates, and the page the new token goes to -------------------------------------------------
-  // candidate c: where its (m, l) pair and its accumulator row are; absent when its unit wrote nothing
-  auto locate = [&](int c, const float*& ml, const float*& acc_row) {
-    bool present = c < total;
-    const int cc = present ? c : 0;
-    const int u = cc < own_n ? own_lo + cc : sh_lo + (cc - own_n);
-    if (!every_unit_has_quanta) present = present && geo.unit_start(u) != geo.unit_start(u + 1);
-    if (cc < own_n) {
-      const int64_t prow = static_cast<int64_t>(u + b) * p.q_heads + h;
-      ml = p.part_ml + prow * 2;
-      acc_row = p.part_acc + prow * d;
-    } else {
-      const int64_t prow = static_cast<int64_t>(u + sh_item) * p.kv_heads * 16 + sh_col;
-      ml = mp.shared_ml + prow * 2;
-      acc_row = mp.shared_acc + prow * d;
-    }
-    return present;
-  };
-  struct Chunk {
-    float m[kMergeChunk], l[kMergeChunk];
-    float v[kMergeChunk][EPW];
-  };
-  auto load_chunk = [&](int base, Chunk& ch) {
-#pragma unroll
-    for (int j = 0; j < kMergeChunk; ++j) {
-      const float* ml = nullptr;
-      const float* part = nullptr;
-      const bool present = total > 0 && locate(base + j, ml, part);  // (total == 0: nothing was located)
-      float2_t pair = {kNegInf, 0.0f};
-      if (present) pair = *reinterpret_cast<const float2_t*>(ml);
-      // a partial without keys contributes nothing (attention.cu:680-682 in the reference)
-      ch.m[j] = (present && pair[1] != 0.0f) ? pair[0] : kNegInf;
-      ch.l[j] = present ? pair[1] : 0.0f;
-#pragma unroll
-      for (int e = 0; e < EPW; ++e) {
-        const int idx = lane + e * kWave;
-        ch.v[j][e] = (present && idx < d) ? part[idx] : 0.0f;
+  // ---- round trip 2: the page the new token goes to, and the candidates ------------------------------------------------
+  // position -> (block-table column, slot) by the launcher's multiply-shift constants (any page size); the id of a
+  // clamped column is read whatever the position and dropped when the position has no column
+  const int col = static_cast<int>(__umulhi(static_cast<uint32_t>(max(pos, 0)), mp.bs_magic) >> mp.bs_post);
+  const int slot = pos - col * p.block_size;
+  const int blk = p.block_table[static_cast<int64_t>(b) * p.max_blocks + min(col, p.max_blocks - 1)];
+  // Candidate c of the row is the partial of unit own_lo + c (c < own_n), then of unit sh_lo + c - own_n of the shared
+  // item: consecutive candidates of a kind sit a constant stride apart, so an address is a base plus a multiple.  A
+  // candidate past the row's last one reads the last one again (a line this wave fetches anyway) and is masked out;
+  // a row without candidates reads slot b of the per-row region, which nothing writes, and masks it out.
+  const int64_t own_row0 = static_cast<int64_t>(own_lo + b) * q_heads + h;
+  const int64_t sh_row0 = static_cast<int64_t>(sh_lo + sh_item) * kv_heads * 16 + sh_col;
+  const int64_t sh_row_stride = static_cast<int64_t>(kv_heads) * 16;
+  const float* const sh_ml = sh_n > 0 ? mp.shared_ml : p.part_ml;  // (never dereferenced without shared candidates)
+  const float* const sh_acc = sh_n > 0 ? mp.shared_acc : p.part_acc;
+  auto load_chunk = [&](int base, auto& ch) {
+    constexpr int N = std::remove_reference_t<decltype(ch)>::kSize;
+    // units without a quantum among the chunk's candidates (launches with fewer cost positions than units only)
+    uint32_t empty_mask = 0;
+    if (!every_unit_has_quanta) {
+      for (int j = 0; j < N && base + j < total; ++j) {
+        const int c = base + j;
+        const int u = c < own_n ? own_lo + c : sh_lo + (c - own_n);
+        empty_mask |= unit_is_empty(cum_total, mp.num_units, units_rcp, u) ? (1u << j) : 0u;
       }
     }
+    float2_t pair[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const int c = max(min(base + j, total - 1), 0);
+      const bool own = c < own_n || total == 0;
+      const int64_t prow = own ? own_row0 + static_cast<int64_t>(c) * q_heads : sh_row0 + (c - own_n) * sh_row_stride;
+      const float* ml = (own ? p.part_ml : sh_ml) + prow * 2;
+      const float* part = (own ? p.part_acc : sh_acc) + prow * d;
+      pair[j] = float2_t{kNegInf, 0.0f};
+#pragma unroll
+      for (int e = 0; e < EPW; ++e) ch.v[j][e] = 0.0f;
+      if (base + j < total) {
+        pair[j] = *reinterpret_cast<const float2_t*>(ml);
+#pragma unroll
+        for (int e = 0; e < EPW; ++e) ch.v[j][e] = part[min(lane + e * kWave, d - 1)];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const bool present = base + j < total && !((empty_mask >> j) & 1u);
+      // a partial without keys contributes nothing (attention.cu:680-682 in the reference)
+      ch.m[j] = (present && pair[j][1] != 0.0f) ? pair[j][0] : kNegInf;
+      ch.l[j] = present ? pair[j][1] : 0.0f;
+#pragma unroll
+      for (int e = 0; e < EPW; ++e) ch.v[j][e] = (present && lane + e * kWave < d) ? ch.v[j][e] : 0.0f;
+    }
   };
-  Chunk first;
-  load_chunk(0, first);
-  bool store = false;
-  int64_t dst_row = 0;
-  if (append) {
-    const int64_t col = pos / p.block_size;
-    const int64_t slot = pos - col * p.block_size;
-    bool ok = pos >= 0 && col < p.max_blocks;
-    const int64_t blk = ok ? p.block_table[static_cast<int64_t>(b) * p.max_blocks + col] : 0;
-    ok = ok && blk >= 0 && blk < mp.num_blocks;
-    store = ok && mp.write_append != 0 && h == kvh * p.group;
-    dst_row = (blk * p.block_size + slot) * p.kv_heads + kvh;
-  }
+  MergeChunk<kMergeChunk, EPW> first;
+  load_chunk(part * kMergeChunk, first);
 
   // ---- the new token: quantize, store, m = q . k_new, l = 1, acc = v_new ----------------------------------------------
   float acc[EPW];
@@ -294,16 +336,22 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   for (int e = 0; e < EPW; ++e) acc[e] = 0.0f;
   float m = kNegInf, l = 0.0f;
   if (append) {
+    const bool ok = pos >= 0 && col < p.max_blocks && blk >= 0 && blk < mp.num_blocks;
+    const bool store = ok && mp.write_append != 0 && h == kvh * group;
+    const int64_t dst_row = (static_cast<int64_t>(ok ? blk : 0) * p.block_size + slot) * kv_heads + kvh;
+    float kx[EPW], vx[EPW], qv[EPW];
 #pragma unroll
     for (int e = 0; e < EPW; ++e) {
-      kx[e] = p.q_dtype == ARENO_DT_BF16 ? bf16_bits_to_float(kraw[e]) : f16_bits_to_float(kraw[e]);
-      vx[e] = p.q_dtype == ARENO_DT_BF16 ? bf16_bits_to_float(vraw[e]) : f16_bits_to_float(vraw[e]);
+      const bool in = lane + e * kWave < d;
+      kx[e] = in ? widen(kraw[e]) : 0.0f;
+      vx[e] = in ? widen(vraw[e]) : 0.0f;
+      qv[e] = in ? widen(qraw[e]) : 0.0f;
     }
     float khat[EPW], vhat[EPW];
-    if (is_quantized_dtype(p.cache_dtype)) {
-      quantize_row<EPW>(kx, lane, d, dst_row, const_cast<void*>(p.k_cache), const_cast<void*>(p.k_scale), p.cache_dtype,
+    if constexpr (CDT == ARENO_DT_I8 || CDT == ARENO_DT_FP8_E4M3) {
+      quantize_row<EPW>(kx, lane, d, dst_row, const_cast<void*>(p.k_cache), const_cast<void*>(p.k_scale), CDT,
                         p.scale_dtype, store, khat);
-      quantize_row<EPW>(vx, lane, d, dst_row, const_cast<void*>(p.v_cache), const_cast<void*>(p.v_scale), p.cache_dtype,
+      quantize_row<EPW>(vx, lane, d, dst_row, const_cast<void*>(p.v_cache), const_cast<void*>(p.v_scale), CDT,
                         p.scale_dtype, store, vhat);
     } else {
       // 16-bit pages of the query's dtype hold the update row as it is
@@ -328,17 +376,18 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
   }
 
   // ---- merge ----------------------------------------------------------------------------------------------------------
-  auto merge_chunk = [&](const Chunk& ch) {
+  auto merge_chunk = [&](const auto& ch) {
+    constexpr int N = std::remove_reference_t<decltype(ch)>::kSize;
     float m_new = m;
 #pragma unroll
-    for (int j = 0; j < kMergeChunk; ++j) m_new = fmaxf(m_new, ch.m[j]);
+    for (int j = 0; j < N; ++j) m_new = fmaxf(m_new, ch.m[j]);
     const float m_safe = m_new == kNegInf ? 0.0f : m_new;
     const float alpha = fast_exp2(m - m_safe);
     l *= alpha;
 #pragma unroll
     for (int e = 0; e < EPW; ++e) acc[e] *= alpha;
 #pragma unroll
-    for (int j = 0; j < kMergeChunk; ++j) {
+    for (int j = 0; j < N; ++j) {
       const float w = fast_exp2(ch.m[j] - m_safe);  // 0 for absent candidates
       l += w * ch.l[j];
 #pragma unroll
@@ -347,27 +396,80 @@ __global__ __launch_bounds__(kReduceRows* kWave) void decode_reduce_slots_kernel
     m = m_new;
   };
   merge_chunk(first);
-  for (int base = kMergeChunk; base < total; base += kMergeChunk) {
-    Chunk more;
+  for (int base = (part + MW) * kMergeChunk; base < total; base += MW * kMergeChunk) {
+    MergeChunk<kMergeChunk, EPW> more;
     load_chunk(base, more);
     merge_chunk(more);
+  }
+  if constexpr (MW > 1) {
+    // the waves' (m, l, acc) meet in LDS; wave 0 combines them in wave order and writes the row
+    __shared__ float s_ml[MW][2];
+    __shared__ float s_acc[MW][EPW * kWave];
+    if (lane == 0) {
+      s_ml[part][0] = m;
+      s_ml[part][1] = l;
+    }
+#pragma unroll
+    for (int e = 0; e < EPW; ++e) s_acc[part][lane + e * kWave] = acc[e];
+    __syncthreads();
+    if (part != 0) return;
+    float m_all = kNegInf;
+#pragma unroll
+    for (int w2 = 0; w2 < MW; ++w2) m_all = fmaxf(m_all, s_ml[w2][0]);
+    const float m_safe = m_all == kNegInf ? 0.0f : m_all;
+    l = 0.0f;
+#pragma unroll
+    for (int e = 0; e < EPW; ++e) acc[e] = 0.0f;
+#pragma unroll
+    for (int w2 = 0; w2 < MW; ++w2) {
+      const float wgt = fast_exp2(s_ml[w2][0] - m_safe);  // 0 for a wave without candidates
+      l += wgt * s_ml[w2][1];
+#pragma unroll
+      for (int e = 0; e < EPW; ++e) acc[e] += wgt * s_acc[w2][lane + e * kWave];
+    }
   }
 #pragma unroll
   for (int e = 0; e < EPW; ++e) {
     const int idx = lane + e * kWave;
-    if (idx < d) store_from_float(p.out, static_cast<int64_t>(row) * d + idx, p.q_dtype, acc[e] / l);
+    if (idx < d) store_from_float(p.out, static_cast<int64_t>(row) * d + idx, QDT, acc[e] / l);
   }
 }
 
 typedef void (*reduce_slots_fn)(const int32_t*, const int32_t*, const void*, const void*, const void*, int32_t, int32_t,
-                                int32_t, int32_t, int32_t, int32_t, MfmaDecodeParams);
+                                int32_t, uint32_t, int32_t, MfmaDecodeParams);
 // the narrowest instantiation that covers the head: the kernel is a few hundred instructions per wave and mostly
 // launch latency, so slots that would only be predicated off are worth leaving out
-reduce_slots_fn reduce_slots_kernel_for(int head_dim) {
-  if (head_dim <= 64) return decode_reduce_slots_kernel<1>;
-  if (head_dim <= 128) return decode_reduce_slots_kernel<2>;
-  if (head_dim <= 256) return decode_reduce_slots_kernel<4>;
-  return decode_reduce_slots_kernel<kGenericMaxPerLane>;
+template <int QDT, int CDT, bool PLANNED, int MW>
+reduce_slots_fn reduce_slots_kernel_by_width(int head_dim) {
+  if (head_dim <= 64) return decode_reduce_slots_kernel<1, QDT, CDT, PLANNED, MW>;
+  if (head_dim <= 128) return decode_reduce_slots_kernel<2, QDT, CDT, PLANNED, MW>;
+  if (head_dim <= 256) return decode_reduce_slots_kernel<4, QDT, CDT, PLANNED, MW>;
+  return decode_reduce_slots_kernel<kGenericMaxPerLane, QDT, CDT, PLANNED, MW>;
+}
+template <int QDT, int CDT, bool PLANNED>
+reduce_slots_fn reduce_slots_kernel_by_waves(int head_dim, int waves) {
+  if (waves == 1) return reduce_slots_kernel_by_width<QDT, CDT, PLANNED, 1>(head_dim);
+  if (waves == 4) return reduce_slots_kernel_by_width<QDT, CDT, PLANNED, 4>(head_dim);
+  return reduce_slots_kernel_by_width<QDT, CDT, PLANNED, 16>(head_dim);
+}
+template <int QDT, bool PLANNED>
+reduce_slots_fn reduce_slots_kernel_by_cache(int head_dim, int cache_dtype, int waves) {
+  if (cache_dtype == ARENO_DT_I8) return reduce_slots_kernel_by_waves<QDT, ARENO_DT_I8, PLANNED>(head_dim, waves);
+  if (cache_dtype == ARENO_DT_FP8_E4M3) return reduce_slots_kernel_by_waves<QDT, ARENO_DT_FP8_E4M3, PLANNED>(head_dim, waves);
+  return reduce_slots_kernel_by_waves<QDT, QDT, PLANNED>(head_dim, waves);  // 16-bit pages (an append needs them in q's dtype)
+}
+reduce_slots_fn reduce_slots_kernel_for(int head_dim, int q_dtype, int cache_dtype, bool planned, int waves) {
+  if (q_dtype == ARENO_DT_BF16)
+    return planned ? reduce_slots_kernel_by_cache<ARENO_DT_BF16, true>(head_dim, cache_dtype, waves)
+                   : reduce_slots_kernel_by_cache<ARENO_DT_BF16, false>(head_dim, cache_dtype, waves);
+  return planned ? reduce_slots_kernel_by_cache<ARENO_DT_F16, true>(head_dim, cache_dtype, waves)
+                 : reduce_slots_kernel_by_cache<ARENO_DT_F16, false>(head_dim, cache_dtype, waves);
+}
+// Waves that share a (row, head) in the merge launch: a row has about units / batch + 2 candidates (the launcher knows
+// no lengths; a long row among short ones has more), and a wave takes kMergeChunk of them per round trip.
+int merge_waves_for(int units, int batch) {
+  const int chunks = (units / (batch > 0 ? batch : 1) + 2 + kMergeChunk - 1) / kMergeChunk;
+  return chunks <= 1 ? 1 : (chunks <= 4 ? 4 : 16);
 }
 
 // ---- geometry of the MFMA path ----------------------------------------------------------------------
@@ -544,6 +646,7 @@ MfmaChoice choose_mfma(const areno_paged_cache* cache, int q_dtype, int batch, i
   const bool rows_fit = static_cast<double>(cache->num_blocks) * cache->block_size * cache->kv_heads < 4294967296.0;
   PageDivision division;
   if (!aligned || q_dtype == ARENO_DT_F32 || !prefer_mfma() || c.head_parts > kMaxHeadParts || batch > kMfmaMaxBatch || !rows_fit ||
+      q_heads > 65535 ||
       !page_division(cache->block_size, &division))
     return c;
   // prefix groups: only without a window, when at least two rows fit side by side
@@ -878,10 +981,15 @@ int decode_impl(const areno_paged_cache* cache, const void* q, const void* k_upd
       if (int rc = check_launch(op)) return rc;
     }
     if (stages & ARENO_STAGE_REDUCE) {
-      const int rblocks = (batch * q_heads + kReduceRows - 1) / kReduceRows;
-      hipLaunchKernelGGL(reduce_slots_kernel_for(mp.d.head_dim), dim3(rblocks), dim3(kReduceRows * kWave), 0, s,
-                         mp.plan_rows, p.cache_seqlens, p.q, mp.k_update, mp.v_update, batch * q_heads, q_heads,
-                         p.kv_heads, p.group, p.head_dim, p.q_dtype, mp);
+      // (q_dtype is F16 or BF16 on this path; h / group as a multiplication: exact for h < 2^16)
+      const uint32_t group_magic = p.group > 1 ? static_cast<uint32_t>((uint64_t{1} << 32) / p.group + 1) : 0u;
+      const int merge_waves = merge_waves_for(grid.units, batch);
+      const reduce_slots_fn merge =
+          reduce_slots_kernel_for(p.head_dim, q_dtype, cache->cache_dtype, mp.plan_rows != nullptr, merge_waves);
+      const dim3 merge_grid(merge_waves == 1 ? (q_heads + kReduceRows - 1) / kReduceRows : q_heads, batch);
+      hipLaunchKernelGGL(merge, merge_grid, dim3((merge_waves == 1 ? kReduceRows : merge_waves) * kWave), 0, s,
+                         mp.plan_rows, p.cache_seqlens, p.q, mp.k_update, mp.v_update, q_heads, p.kv_heads, p.group,
+                         group_magic, p.head_dim, mp);
       if (int rc = check_launch(op)) return rc;
     }
     return ARENO_OK;

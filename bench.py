@@ -245,15 +245,27 @@ def measure_decode(w, steps, warmup, *, kernel_iters=20, kernel_samples=15, repe
                                       group_rows=group_rows, shared_lens=shared_lens)  # fmt: skip
 
     def time_launches(launch, name):
-        for i in range(max(copies, 20)):
-            launch(i)
+        """Mean duration of `kernel_iters` back-to-back launches, by events on the stream around one replay of a graph
+        that holds them (launched one by one from Python the host cannot keep up with kernels shorter than ~8 us, and
+        the figure would be its launch rate)."""
+        side3 = torch.cuda.Stream()
+        side3.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side3):
+            for i in range(max(copies, 20)):
+                launch(i)
+        torch.cuda.current_stream().wait_stream(side3)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(kernel_iters):
+                launch(i)
+        graph.replay()
         torch.cuda.synchronize()
         samples = []
         for _ in range(kernel_samples):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            for i in range(kernel_iters):
-                launch(i)
+            graph.replay()
             e1.record()
             e1.synchronize()
             samples.append(e0.elapsed_time(e1) * 1e3 / kernel_iters)
