@@ -126,6 +126,47 @@ def test_paged_prefill_staging_schemes(kv, d, bs):
     assert_close(_run_prefill(w), _expected_prefill(w), *tolerances(kv), what=f"prefill staging D={d} {kv} page {bs}")
 
 
+@pytest.mark.parametrize("seed", range(32))
+def test_random_draws_of_prefill_shape_length_window_and_cache_type(seed):
+    """Seeded random configurations through the paged prefill op: cache type, head counts (up to 33 q heads per kv
+    head: several workgroup rows per kv head), head dim (one tile or two per wave, the head split over two waves at
+    512, 96 on the one-wave-per-row kernel), page size (12 and 48: no power of two, the one-wave-per-row kernel),
+    number of sequences, new and cached lengths (sequences without new tokens, single tokens, blocks cut by many
+    shares) and window."""
+    import random
+
+    rng = random.Random(7000 + seed)
+    kv = rng.choice(["bf16", "fp16", "int8", "fp8"])
+    group = rng.choice([1, 2, 4, 7, 8, 16, 20, 33])
+    hkv = rng.choice([h for h in (1, 2, 4, 8) if h * group <= 64])
+    d = rng.choice([64, 128, 128, 192, 256, 512, 96])
+    bs = rng.choice([8, 16, 32, 64, 256, 12, 48])
+    slow = d == 96 or bs in (12, 48)  # one wave per (token, head): keep the work small
+    seqs = rng.choice([1, 3, 9] if slow else [1, 3, 9, 40])
+    g = torch.Generator().manual_seed(seed)
+    new_profile = rng.choice(["ones", "short", "mixed", "long"])
+    if new_profile == "ones":
+        new = torch.randint(0, 2, (seqs,), generator=g)
+    elif new_profile == "short":
+        new = torch.randint(0, 20, (seqs,), generator=g)
+    elif new_profile == "mixed":
+        new = torch.where(torch.rand(seqs, generator=g) < 0.6, torch.randint(0, 9, (seqs,), generator=g),
+                          torch.randint(60, 300, (seqs,), generator=g))  # fmt: skip
+    else:
+        new = torch.randint(100, 140 if slow else 400, (seqs,), generator=g)
+    if int(new.sum()) == 0:
+        new[0] = 1
+    ctx_hi = 300 if slow else rng.choice([1, 90, 700, 4000])
+    ctx = torch.where(torch.rand(seqs, generator=g) < 0.3, torch.zeros(seqs, dtype=torch.int64),
+                      torch.randint(0, ctx_hi, (seqs,), generator=g))  # fmt: skip
+    window = rng.choice([None, None, 0, 33, 700])
+    w = workloads.make_prefill_workload(f"draw-{seed}", seed=900 + seed, new_lens=new, ctx_lens=ctx, hq=hkv * group,
+                                        hkv=hkv, d=d, bs=bs, kv=kv, device=DEV, quantize_fn=gpu_quantize,
+                                        act_dtype=torch.float16 if kv == "fp16" else torch.bfloat16)  # fmt: skip
+    what = f"draw {seed}: {kv} {hkv * group}/{hkv} d={d} bs={bs} seqs={seqs} new={new_profile} ctx<{ctx_hi} window={window}"
+    assert_close(_run_prefill(w, window), _expected_prefill(w, window), *tolerances(kv), what=what)
+
+
 def test_prefill_with_a_full_sequence_list():
     """1024 sequences, the most one launch of the matrix-core kernel indexes: the prefix sum over the sequences must
     also produce its last entry, the total."""
