@@ -182,6 +182,23 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 // ---- host side ---------------------------------------------------------------------------
 
+// Division of a token index by the page size as a multiply and a shift: with s = ceil(log2(bs)) and
+// magic = floor(2^(30 + s) / bs) + 1, (t * magic) >> (30 + s) == t / bs for every 0 <= t < 2^30 (the error of the
+// product is below t / 2^(30 + s) <= 1 / 2^s, which cannot carry a quotient over while (bs - 1) / bs + 1 / 2^s <= 1).
+// A kernel takes the high word of the product (__umulhi), so the shift left over is s - 2 and pages of fewer than 4
+// tokens are not served this way.
+struct PageDivision {
+  uint32_t magic;
+  int32_t post;
+};
+inline bool page_division(int64_t block_size, PageDivision* out) {
+  if (block_size < 4 || block_size > (1 << 24)) return false;
+  int s = 0;
+  while ((int64_t{1} << s) < block_size) ++s;
+  out->magic = static_cast<uint32_t>((uint64_t{1} << (30 + s)) / static_cast<uint64_t>(block_size) + 1);
+  out->post = s - 2;
+  return true;
+}
 void set_error(const char* fmt, ...);
 int fail(int status, const char* fmt, ...);
 int check_launch(const char* what);

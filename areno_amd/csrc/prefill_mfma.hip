@@ -93,7 +93,9 @@ struct PrefillParams {
   int32_t group_pad;    // q heads of one part rounded up to a power of two (<= 16)
   int32_t group_shift;  // log2(group_pad)
   int32_t block_size;
-  int32_t bs_shift;
+  int32_t bs_shift;   // log2 of the page size, or -1: then a key's column is __umulhi(key, bs_magic) >> bs_post
+  uint32_t bs_magic;
+  int32_t bs_post;
   int32_t max_blocks;
   int32_t window_left;
   int32_t q_dtype;
@@ -235,7 +237,7 @@ __device__ __forceinline__ void dequant_chunk(uint4_t codes, float scale, uint4_
 
 // DS > 1 (head dim 512): DS adjacent waves share a row tile, each with D / DS of the head's elements -- its part of
 // K . Q^T, which the waves of the tile exchange through LDS and add in the same order, and its columns of O.
-template <int KIND, int D, bool SCALE16, int RT, int DS = 1>
+template <int KIND, int D, bool SCALE16, int RT, int DS = 1, bool ANYPAGE = false>
 __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) void prefill_mfma_kernel(PrefillParams p) {
   static_assert(DS == 1 || RT == 1, "a split head has one row tile per wave group");
   constexpr int kRowTiles = RT;
@@ -435,16 +437,31 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
     auto scale_at = [&](const char* base, uint32_t page_row) {
       return *reinterpret_cast<const scale_raw_t*>(base + static_cast<uint64_t>(page_row) * scale_stride);
     };
+    // Page sizes that are no power of two have instances of their own (ANYPAGE; a choice at run time cost the
+    // power-of-two instances 5 % of the launch): the key's column by a multiplication and a shift, the slot kept in
+    // place of the key, the page row as a 24-bit multiply-add (the launcher checks the ranges).
     auto load_ids = [&](FetchSet& f, int tile) {
+      int col[NLD];
+      if constexpr (ANYPAGE) {
 #pragma unroll
-      for (int i = 0; i < NLD; ++i) {
-        f.keys[i] = max(0, min(tile * TK + chunk_tok[i], key_hi));
-        f.ids[i] = table_row[packed ? 0 : (f.keys[i] >> p.bs_shift)];
+        for (int i = 0; i < NLD; ++i) {
+          const int key = max(0, min(tile * TK + chunk_tok[i], key_hi));
+          col[i] = static_cast<int>(__umulhi(static_cast<uint32_t>(key), p.bs_magic) >> p.bs_post);
+          f.keys[i] = key - __mul24(col[i], p.block_size);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+          f.keys[i] = max(0, min(tile * TK + chunk_tok[i], key_hi));
+          col[i] = packed ? 0 : (f.keys[i] >> p.bs_shift);
+        }
       }
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) f.ids[i] = table_row[col[i]];
     };
-    // page size is a power of two here (the launcher sends other sizes to the generic kernel); packed K/V run as one
-    // page per token with the token's row as its id
+    // packed K/V run as one page per token with the token's row as its id
     auto page_row_of = [&](const FetchSet& f, int i) -> uint32_t {
+      if constexpr (ANYPAGE) return static_cast<uint32_t>(__mul24(f.ids[i], p.block_size) + f.keys[i]);
       const uint32_t paged = (static_cast<uint32_t>(f.ids[i]) << p.bs_shift) + (static_cast<uint32_t>(f.keys[i]) & slot_mask);
       return packed ? static_cast<uint32_t>(q_begin + f.keys[i]) : paged;
     };
@@ -879,40 +896,40 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
 
 typedef void (*prefill_fn)(PrefillParams);
 
-template <int KIND, int RT>
+template <int KIND, int RT, bool ANYPAGE>
 prefill_fn prefill_lookup_rt(int head_dim, bool scale16) {
   constexpr bool kQuant = KVTraits<KIND>::kQuant;
   if constexpr (RT == 2) {
     if (head_dim == 128) {
       if constexpr (kQuant) {
-        if (scale16) return prefill_mfma_kernel<KIND, 128, true, 2>;
+        if (scale16) return prefill_mfma_kernel<KIND, 128, true, 2, 1, ANYPAGE>;
       }
-      return prefill_mfma_kernel<KIND, 128, false, 2>;
+      return prefill_mfma_kernel<KIND, 128, false, 2, 1, ANYPAGE>;
     }
     if (head_dim == 64) {
       if constexpr (kQuant) {
-        if (scale16) return prefill_mfma_kernel<KIND, 64, true, 2>;
+        if (scale16) return prefill_mfma_kernel<KIND, 64, true, 2, 1, ANYPAGE>;
       }
-      return prefill_mfma_kernel<KIND, 64, false, 2>;
+      return prefill_mfma_kernel<KIND, 64, false, 2, 1, ANYPAGE>;
     }
   } else {
     if (head_dim == 256) {
       if constexpr (kQuant) {
-        if (scale16) return prefill_mfma_kernel<KIND, 256, true, 1>;
+        if (scale16) return prefill_mfma_kernel<KIND, 256, true, 1, 1, ANYPAGE>;
       }
-      return prefill_mfma_kernel<KIND, 256, false, 1>;
+      return prefill_mfma_kernel<KIND, 256, false, 1, 1, ANYPAGE>;
     }
     if (head_dim == 192) {
       if constexpr (kQuant) {
-        if (scale16) return prefill_mfma_kernel<KIND, 192, true, 1>;
+        if (scale16) return prefill_mfma_kernel<KIND, 192, true, 1, 1, ANYPAGE>;
       }
-      return prefill_mfma_kernel<KIND, 192, false, 1>;
+      return prefill_mfma_kernel<KIND, 192, false, 1, 1, ANYPAGE>;
     }
     if (head_dim == 512) {
       if constexpr (kQuant) {
-        if (scale16) return prefill_mfma_kernel<KIND, 512, true, 1, 2>;
+        if (scale16) return prefill_mfma_kernel<KIND, 512, true, 1, 2, ANYPAGE>;
       }
-      return prefill_mfma_kernel<KIND, 512, false, 1, 2>;
+      return prefill_mfma_kernel<KIND, 512, false, 1, 2, ANYPAGE>;
     }
   }
   return nullptr;
@@ -926,8 +943,10 @@ int prefill_head_split(int head_dim) { return head_dim > 256 ? 2 : 1; }
 int prefill_rows_per_wg(int head_dim) { return 16 * prefill_row_tiles(head_dim) * kPrefillWaves / prefill_head_split(head_dim); }
 
 template <int KIND>
-prefill_fn prefill_lookup(int head_dim, bool scale16, int row_tiles) {
-  return row_tiles == 1 ? prefill_lookup_rt<KIND, 1>(head_dim, scale16) : prefill_lookup_rt<KIND, 2>(head_dim, scale16);
+prefill_fn prefill_lookup(int head_dim, bool scale16, int row_tiles, bool any_page_size) {
+  if (any_page_size)
+    return row_tiles == 1 ? prefill_lookup_rt<KIND, 1, true>(head_dim, scale16) : prefill_lookup_rt<KIND, 2, true>(head_dim, scale16);
+  return row_tiles == 1 ? prefill_lookup_rt<KIND, 1, false>(head_dim, scale16) : prefill_lookup_rt<KIND, 2, false>(head_dim, scale16);
 }
 
 int log2_exact_i(int x) {
@@ -967,7 +986,16 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   const int group = q_heads / cache->kv_heads;
   if (q_dtype != ARENO_DT_F16 && q_dtype != ARENO_DT_BF16) return ARENO_ERR_UNSUPPORTED;
   if (!(softmax_scale > 0.0f)) return ARENO_ERR_UNSUPPORTED;  // the kernel takes row maxima before scaling
-  if (log2_exact_i(cache->block_size) < 0) return ARENO_ERR_UNSUPPORTED;  // page addressing by shift and mask
+  // page addressing by shift and mask, or, for page sizes that are no power of two, by a multiplication and a shift
+  // (keys below 2^30) and 24-bit products (block ids, table columns and page sizes below 2^23)
+  const bool pow2_pages = log2_exact_i(cache->block_size) >= 0;
+  PageDivision division = {0, 0};
+  if (!pow2_pages) {
+    if (block_table == nullptr || !page_division(cache->block_size, &division)) return ARENO_ERR_UNSUPPORTED;
+    if (cache->num_blocks >= (1 << 23) || cache->block_size >= (1 << 23) || max_blocks >= (1 << 23) ||
+        static_cast<int64_t>(max_blocks) * cache->block_size > 0x3fffffffLL)
+      return ARENO_ERR_UNSUPPORTED;
+  }
   const int head_parts = (group + 15) / 16;
   const int vheads = cache->kv_heads * head_parts;
   if (head_parts > 8 || num_seqs > kMaxPrefillSeqs || tokens > 0x3fffffff) return ARENO_ERR_UNSUPPORTED;
@@ -982,10 +1010,10 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   const int rows_per_wg = prefill_rows_per_wg(cache->head_dim);
   prefill_fn fn = nullptr;
   switch (cache->cache_dtype) {
-    case ARENO_DT_BF16: fn = prefill_lookup<KV_BF16>(cache->head_dim, scale16, row_tiles); break;
-    case ARENO_DT_F16: fn = prefill_lookup<KV_F16>(cache->head_dim, scale16, row_tiles); break;
-    case ARENO_DT_I8: fn = prefill_lookup<KV_I8>(cache->head_dim, scale16, row_tiles); break;
-    case ARENO_DT_FP8_E4M3: fn = prefill_lookup<KV_FP8>(cache->head_dim, scale16, row_tiles); break;
+    case ARENO_DT_BF16: fn = prefill_lookup<KV_BF16>(cache->head_dim, scale16, row_tiles, !pow2_pages); break;
+    case ARENO_DT_F16: fn = prefill_lookup<KV_F16>(cache->head_dim, scale16, row_tiles, !pow2_pages); break;
+    case ARENO_DT_I8: fn = prefill_lookup<KV_I8>(cache->head_dim, scale16, row_tiles, !pow2_pages); break;
+    case ARENO_DT_FP8_E4M3: fn = prefill_lookup<KV_FP8>(cache->head_dim, scale16, row_tiles, !pow2_pages); break;
     default: break;
   }
   if (fn == nullptr) return ARENO_ERR_UNSUPPORTED;
@@ -1027,6 +1055,8 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   p.group_shift = log2_exact_i(p.group_pad);
   p.block_size = cache->block_size;
   p.bs_shift = log2_exact_i(cache->block_size);
+  p.bs_magic = division.magic;
+  p.bs_post = division.post;
   p.max_blocks = max_blocks;
   p.window_left = window_left;
   p.q_dtype = q_dtype;

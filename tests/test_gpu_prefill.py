@@ -86,6 +86,8 @@ def test_paged_prefill_small(kv, window_left):
     # more than 16 q heads per kv head: several workgroup rows per kv head, 16 q heads each (16 + 16, 16 + 4, 16 + 8 at
     # head dim 256, 16 + 16 + 1)
     (32, 1, 128, 16), (40, 2, 64, 32), (24, 1, 256, 16), (33, 1, 128, 16),
+    # page sizes that are no power of two: the key's page by a multiplication and a shift
+    (28, 4, 128, 12), (8, 2, 64, 48), (16, 8, 512, 80), (8, 8, 128, 1000),
 ])  # fmt: skip
 def test_paged_prefill_shapes(hq, hkv, d, bs):
     g = torch.Generator().manual_seed(d + hq)
@@ -113,12 +115,12 @@ def test_paged_prefill_head_dims_192_256_512(kv, d, hq, hkv, window_left):
 
 
 @pytest.mark.parametrize("kv", ["bf16", "fp16", "int8", "fp8"])
-@pytest.mark.parametrize("d,bs", [(64, 16), (64, 64), (128, 8), (128, 128)])
+@pytest.mark.parametrize("d,bs", [(64, 16), (64, 64), (128, 8), (128, 128), (64, 24), (128, 5), (128, 100)])
 def test_paged_prefill_staging_schemes(kv, d, bs):
     """The staging of a key tile has two schemes: one K and one V chunk per thread and round, or, when a tile has at
     most one chunk per thread (8-bit tiles up to head dim 128, 16-bit tiles at 64), K staged by the first half of
     the workgroup and V by the second.  8-bit tiles at head dim 64 leave half of each half without a live chunk.
-    Page sizes below, at and above the 32-key tile."""
+    Page sizes below, at and above the 32-key tile, powers of two and others."""
     new = torch.tensor([70, 1, 200, 33])
     ctx = torch.tensor([0, 1300, 95, 640])
     w = workloads.make_prefill_workload("staging", seed=d + bs, new_lens=new, ctx_lens=ctx, hq=8, hkv=2, d=d, bs=bs,
@@ -130,9 +132,8 @@ def test_paged_prefill_staging_schemes(kv, d, bs):
 def test_random_draws_of_prefill_shape_length_window_and_cache_type(seed):
     """Seeded random configurations through the paged prefill op: cache type, head counts (up to 33 q heads per kv
     head: several workgroup rows per kv head), head dim (one tile or two per wave, the head split over two waves at
-    512, 96 on the one-wave-per-row kernel), page size (12 and 48: no power of two, the one-wave-per-row kernel),
-    number of sequences, new and cached lengths (sequences without new tokens, single tokens, blocks cut by many
-    shares) and window."""
+    512, 96 on the one-wave-per-row kernel), page size (12 and 48: no power of two), number of sequences, new and
+    cached lengths (sequences without new tokens, single tokens, blocks cut by many shares) and window."""
     import random
 
     rng = random.Random(7000 + seed)
@@ -141,7 +142,7 @@ def test_random_draws_of_prefill_shape_length_window_and_cache_type(seed):
     hkv = rng.choice([h for h in (1, 2, 4, 8) if h * group <= 64])
     d = rng.choice([64, 128, 128, 192, 256, 512, 96])
     bs = rng.choice([8, 16, 32, 64, 256, 12, 48])
-    slow = d == 96 or bs in (12, 48)  # one wave per (token, head): keep the work small
+    slow = d == 96  # one wave per (token, head): keep the work small
     seqs = rng.choice([1, 3, 9] if slow else [1, 3, 9, 40])
     g = torch.Generator().manual_seed(seed)
     new_profile = rng.choice(["ones", "short", "mixed", "long"])
