@@ -46,6 +46,7 @@
 // context 0 it is the reference's varlen kernel (areno/accel/csrc/attention.cu:145-242).
 
 #include "decode_mfma_kernels.hpp"
+#include "prefill_steps.hpp"
 
 namespace areno {
 
@@ -104,23 +105,6 @@ struct PrefillParams {
   float scale_log2e;
 };
 
-// Key tiles query block j (tokens [j * tq, ...)) of a sequence may see: [tile_lo, tile_hi].
-struct BlockTiles {
-  int tok0, cnt, tile_lo, tile_hi;
-  __device__ int count() const { return tile_hi - tile_lo + 1; }
-};
-
-__device__ __forceinline__ BlockTiles block_tiles(int n_new, int ctx, int j, int tq, int window_left) {
-  BlockTiles b;
-  b.tok0 = j * tq;
-  b.cnt = min(tq, n_new - b.tok0);
-  const int key_hi = ctx + b.tok0 + b.cnt - 1;
-  const int key_lo = window_left >= 0 ? max(0, ctx + b.tok0 - window_left) : 0;
-  b.tile_lo = key_lo / kTileTokens;
-  b.tile_hi = key_hi / kTileTokens;
-  return b;
-}
-
 // Exclusive prefix sum of tile steps per sequence into s_cum[0 .. num_seqs] (all threads take part).
 __device__ __forceinline__ void prefix_tile_steps(const PrefillParams& p, int tq, int* s_cum, int* s_wave_tot) {
   constexpr int SPT = kMaxPrefillSeqs / kPrefillThreads;
@@ -136,7 +120,7 @@ __device__ __forceinline__ void prefix_tile_steps(const PrefillParams& p, int tq
     if (s < p.num_seqs) {
       const int n_new = p.cu_seqlens_q[s + 1] - p.cu_seqlens_q[s];
       const int ctx = p.context_lens != nullptr ? p.context_lens[s] : 0;
-      for (int j = 0; j * tq < n_new; ++j) steps[i] += block_tiles(n_new, ctx, j, tq, p.window_left).count();
+      steps[i] = sequence_steps(n_new, ctx, tq, p.window_left);
     }
     local += steps[i];
   }
@@ -182,24 +166,17 @@ __device__ __forceinline__ StepPos locate_step(const PrefillParams& p, const int
   r.seq = lo;
   r.n_new = p.cu_seqlens_q[lo + 1] - p.cu_seqlens_q[lo];
   r.ctx = p.context_lens != nullptr ? p.context_lens[lo] : 0;
-  int off = x - s_cum[lo];
-  r.item_x0 = s_cum[lo];
-  r.j = 0;
-  for (;;) {
-    const BlockTiles b = block_tiles(r.n_new, r.ctx, r.j, tq, p.window_left);
-    if (off < b.count()) {
-      r.tile = b.tile_lo + off;
-      break;
-    }
-    off -= b.count();
-    r.item_x0 += b.count();
-    ++r.j;
-    if (r.j * tq >= r.n_new) {  // x past the sequence's last step: callers never ask for it
-      r.j = 0;
-      r.tile = 0;
-      break;
-    }
+  const int off = x - s_cum[lo];
+  if (r.n_new <= 0 || off < 0) {  // x outside the sequence's steps: callers never ask for it
+    r.j = 0;
+    r.tile = 0;
+    r.item_x0 = s_cum[lo];
+    return r;
   }
+  r.j = block_of_step(r.n_new, r.ctx, tq, p.window_left, off);
+  const int before = steps_before_block(r.n_new, r.ctx, r.j, tq, p.window_left);
+  r.item_x0 = s_cum[lo] + before;
+  r.tile = block_tiles(r.n_new, r.ctx, r.j, tq, p.window_left).tile_lo + (off - before);
   return r;
 }
 
@@ -802,6 +779,8 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
 // starts in unit u and runs on into later units, it combines the partials of all units the item touches (slot
 // 2u' for a unit where the item comes first, 2u' + 1 where it comes last after other items), normalises and
 // writes the item's rows.
+constexpr int kMergeInFlight = 8;  // 16-byte chunks of each partial a thread of prefill_merge_kernel takes
+
 __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillParams p) {
   __shared__ int s_cum[kMaxPrefillSeqs + 1];
   __shared__ int s_wave_tot[kPrefillWaves];
@@ -831,65 +810,96 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
   while (u_hi + 1 < p.units && unit_start_step(total, u_hi + 1, p.units) <= item_x1 - 1) ++u_hi;
 
   const int q_begin = p.cu_seqlens_q[pos.seq];
-  // thread -> (row, 64-element part of the head dim).  Per unit all of a thread's accumulator loads are issued
-  // together (no store in between), the normalised row is written once at the end.
-  constexpr int kMaxChunks = 16;  // float4 chunks per thread: 64 elements of a row
-  const int parts = d > 64 ? d / 64 : 1;  // threads per row (head dim 64, 128, 192 or 256)
-  const int half = tid % parts;
-  const int dh = d / parts;
-  const int chunks = dh / 4;
-  const int rows_per_pass = kPrefillThreads / parts;  // threads beyond rows_per_pass * parts sit out (parts = 3)
-  for (int r = tid / parts; r < kRowsPerWg && tid < rows_per_pass * parts; r += rows_per_pass) {
-    const int t = r >> p.group_shift;
-    const int hh = r & (p.group_pad - 1);
-    if (t >= item.cnt || hh >= group_here) continue;
-    float m = kNegInf;
-    for (int u = unit; u <= u_hi; ++u) {
-      if (unit_start_step(total, u, p.units) == unit_start_step(total, u + 1, p.units)) continue;  // empty unit
-      const int slot = 2 * u + ((u == unit && pos.item_x0 > x_begin) ? 1 : 0);
-      const int64_t prow = (static_cast<int64_t>(slot) * vheads + vhead) * kRowsPerWg + r;
-      const float pm = p.part_ml[prow * 2];
-      const float pl = p.part_ml[prow * 2 + 1];
-      if (pl != 0.0f) m = fmaxf(m, pm);
+  // The partials of a slot are one contiguous block of rows x head_dim floats, walked as a flat array of 16-byte
+  // chunks, consecutive threads on consecutive chunks (a thread per row part left three quarters of every fetched
+  // line to a later instruction).  The kernel is a chain of dependent round trips on one workgroup per CU, so the
+  // chain is kept short: a workgroup takes kInFlight chunks per thread of every partial (blockIdx.z picks which; the
+  // launcher sizes the grid), the partials are combined in one pass with a running maximum, and the fetches of the
+  // next partial are issued before the current one is used.  (One workgroup per cut item walking all chunks in two
+  // passes took 32 us for the ~500 partials of a launch, 2.1 TB/s.)  The (m, l) pair of a chunk's row is the same
+  // for the lanes of the row and comes out of the cache.
+  const int chunks_per_row = d >> 2;
+  const int total_chunks = kRowsPerWg * chunks_per_row;
+  const float inv_chunks_per_row = 1.0f / static_cast<float>(chunks_per_row);
+  const int base = blockIdx.z * kMergeInFlight * kPrefillThreads + tid;
+  if (base >= total_chunks) return;
+  {
+    constexpr int kInFlight = kMergeInFlight;
+    int row[kInFlight];
+    bool live[kInFlight];
+    float m[kInFlight], lsum[kInFlight];
+    float4_t o[kInFlight];
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k) {
+      const int idx = min(base + k * kPrefillThreads, total_chunks - 1);
+      // idx / chunks_per_row: the product with the rounded reciprocal is exact here (idx + 0.5 is at least half a
+      // chunk away from a multiple of chunks_per_row, and idx < 2^16)
+      row[k] = static_cast<int>((static_cast<float>(idx) + 0.5f) * inv_chunks_per_row);
+      const int t = row[k] >> p.group_shift;
+      const int hh = row[k] & (p.group_pad - 1);
+      live[k] = base + k * kPrefillThreads < total_chunks && t < item.cnt && hh < group_here;
+      m[k] = kNegInf;
+      lsum[k] = 0.0f;
+      o[k] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     }
-    const float m_safe = m == kNegInf ? 0.0f : m;
-    float4_t o[kMaxChunks];
-#pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c) o[c] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    float lsum = 0.0f;
-    for (int u = unit; u <= u_hi; ++u) {
-      if (unit_start_step(total, u, p.units) == unit_start_step(total, u + 1, p.units)) continue;
+    struct Fetched {
+      float4_t a[kInFlight];
+      float2_t v[kInFlight];
+    };
+    auto next_unit = [&](int u) {  // the next unit from u on that owns steps, or u_hi + 1
+      while (u <= u_hi && unit_start_step(total, u, p.units) == unit_start_step(total, u + 1, p.units)) ++u;
+      return u;
+    };
+    auto fetch = [&](Fetched& f, int u) {
       const int slot = 2 * u + ((u == unit && pos.item_x0 > x_begin) ? 1 : 0);
-      const int64_t prow = (static_cast<int64_t>(slot) * vheads + vhead) * kRowsPerWg + r;
-      const float pl = p.part_ml[prow * 2 + 1];
-      if (pl == 0.0f) continue;  // a partial without visible keys
-      const float w = fast_exp2(p.part_ml[prow * 2] - m_safe);
-      lsum += w * pl;
-      const float4_t* src = reinterpret_cast<const float4_t*>(p.part_acc + prow * d + half * dh);
-      float4_t a[kMaxChunks];
+      const int64_t slot_row0 = (static_cast<int64_t>(slot) * vheads + vhead) * kRowsPerWg;
+      const float* ml = p.part_ml + slot_row0 * 2;
+      const float4_t* acc = reinterpret_cast<const float4_t*>(p.part_acc + slot_row0 * d);
 #pragma unroll
-      for (int c = 0; c < kMaxChunks; ++c) a[c] = c < chunks ? src[c] : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-      for (int c = 0; c < kMaxChunks; ++c) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) o[c][j] += w * a[c][j];
+      for (int k = 0; k < kInFlight; ++k) {
+        f.a[k] = acc[min(base + k * kPrefillThreads, total_chunks - 1)];
+        f.v[k] = *reinterpret_cast<const float2_t*>(ml + 2 * row[k]);
       }
-    }
-    const float inv = 1.0f / lsum;
-    const int64_t out_elem =
-        (static_cast<int64_t>(q_begin + item.tok0 + t) * p.q_heads + head0 + hh) * d + half * dh;
+    };
+    Fetched cur, nxt;
+    int u = next_unit(unit);  // (unit itself owns steps: checked above)
+    fetch(cur, u);
+    for (;;) {
+      const int u2 = next_unit(u + 1);
+      if (u2 <= u_hi) fetch(nxt, u2);
 #pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c) {
-      if (c >= chunks) continue;
+      for (int k = 0; k < kInFlight; ++k) {
+        if (cur.v[k][1] == 0.0f) continue;  // a partial without visible keys contributes nothing
+        const float m_new = fmaxf(m[k], cur.v[k][0]);
+        const float keep = fast_exp2(m[k] - m_new);  // 0 for the first partial (m = -inf)
+        const float w = fast_exp2(cur.v[k][0] - m_new);
+        lsum[k] = lsum[k] * keep + w * cur.v[k][1];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[k][j] = o[k][j] * keep + w * cur.a[k][j];
+        m[k] = m_new;
+      }
+      if (u2 > u_hi) break;
+      cur = nxt;
+      u = u2;
+    }
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k) {
+      if (!live[k]) continue;
+      const int idx = base + k * kPrefillThreads;
+      const int t = row[k] >> p.group_shift;
+      const int hh = row[k] & (p.group_pad - 1);
+      const float inv = 1.0f / lsum[k];
+      const int64_t out_elem = (static_cast<int64_t>(q_begin + item.tok0 + t) * p.q_heads + head0 + hh) * d +
+                               4 * (idx - row[k] * chunks_per_row);
       uint32_t lo, hi;
       if (p.q_dtype == ARENO_DT_BF16) {
-        lo = float_to_bf16_bits(o[c][0] * inv) | (float_to_bf16_bits(o[c][1] * inv) << 16);
-        hi = float_to_bf16_bits(o[c][2] * inv) | (float_to_bf16_bits(o[c][3] * inv) << 16);
+        lo = float_to_bf16_bits(o[k][0] * inv) | (float_to_bf16_bits(o[k][1] * inv) << 16);
+        hi = float_to_bf16_bits(o[k][2] * inv) | (float_to_bf16_bits(o[k][3] * inv) << 16);
       } else {
-        lo = float_to_f16_bits(o[c][0] * inv) | (float_to_f16_bits(o[c][1] * inv) << 16);
-        hi = float_to_f16_bits(o[c][2] * inv) | (float_to_f16_bits(o[c][3] * inv) << 16);
+        lo = float_to_f16_bits(o[k][0] * inv) | (float_to_f16_bits(o[k][1] * inv) << 16);
+        hi = float_to_f16_bits(o[k][2] * inv) | (float_to_f16_bits(o[k][3] * inv) << 16);
       }
-      *reinterpret_cast<uint2_t*>(static_cast<char*>(p.out) + (out_elem + 4 * c) * 2) = uint2_t{lo, hi};
+      *reinterpret_cast<uint2_t*>(static_cast<char*>(p.out) + out_elem * 2) = uint2_t{lo, hi};
     }
   }
 }
@@ -1068,7 +1078,9 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   const dim3 grid(p.units, vheads);
   hipLaunchKernelGGL(fn, grid, dim3(kPrefillThreads), 0, static_cast<hipStream_t>(stream), p);
   if (int rc = check_launch(op)) return rc;
-  hipLaunchKernelGGL(prefill_merge_kernel, grid, dim3(kPrefillThreads), 0, static_cast<hipStream_t>(stream), p);
+  const int merge_parts = (rows_per_wg * (cache->head_dim / 4) + kMergeInFlight * kPrefillThreads - 1) / (kMergeInFlight * kPrefillThreads);
+  hipLaunchKernelGGL(prefill_merge_kernel, dim3(p.units, vheads, merge_parts), dim3(kPrefillThreads), 0,
+                     static_cast<hipStream_t>(stream), p);
   return check_launch(op);
 }
 
