@@ -52,6 +52,13 @@ namespace areno {
 
 // LDS row that holds tile token t of the V tile: the second half is rotated by 4 rows so that the 8 tokens a
 // lane group reads through the transpose load ({4g..4g+3} and {16+4g..16+4g+3}) sit in rows distinct mod 16.
+// Workgroup barrier that orders LDS accesses only (no wait for outstanding global stores or loads).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 __device__ __forceinline__ int v_row_of(int t) { return t < 16 ? t : 16 + ((t + 4) & 15); }
 
 size_t prefill_mfma_workspace_bytes(int32_t kv_heads, int32_t head_dim);
@@ -149,6 +156,7 @@ __device__ __forceinline__ void prefix_tile_steps(const PrefillParams& p, int tq
 struct StepPos {
   int seq, j, tile;
   int n_new, ctx;
+  int q_begin;  // row of the sequence's first new token in q / out (cu_seqlens_q[seq])
   int item_x0;  // global step of the item's first tile
 };
 
@@ -164,7 +172,8 @@ __device__ __forceinline__ StepPos locate_step(const PrefillParams& p, const int
     }
   }
   r.seq = lo;
-  r.n_new = p.cu_seqlens_q[lo + 1] - p.cu_seqlens_q[lo];
+  r.q_begin = p.cu_seqlens_q[lo];
+  r.n_new = p.cu_seqlens_q[lo + 1] - r.q_begin;
   r.ctx = p.context_lens != nullptr ? p.context_lens[lo] : 0;
   const int off = x - s_cum[lo];
   if (r.n_new <= 0 || off < 0) {  // x outside the sequence's steps: callers never ask for it
@@ -307,7 +316,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
     const int ta = pos.tile;
     const int tb = min(item.tile_hi, ta + (x_end - x) - 1);
     const bool whole = ta == item.tile_lo && tb == item.tile_hi;
-    const int q_begin = p.cu_seqlens_q[pos.seq];
+    const int q_begin = pos.q_begin;
     const int ctx = pos.ctx;
     const int tok0 = item.tok0;
     const int tok_cnt = item.cnt;
@@ -331,23 +340,10 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
       row_elem[nq] = (static_cast<int64_t>(q_begin + tok0 + t) * p.q_heads + head0 + hh) * D;
 #pragma unroll
       for (int sl = 0; sl < NS; ++sl) {
+        // (as fetched: a query of the other 16-bit type is converted behind the pipeline's fill, so that its fetch
+        // and the fill's fetches are in flight together)
         uint4_t w = {0u, 0u, 0u, 0u};
         if (live) w = load16(p.q, (row_elem[nq] + d0 + (DW / 4) * lk + 8 * sl) * 2);
-        if (!q_is_operand_type) {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const uint32_t word = w[j];
-            float a, c;
-            if constexpr (OPK == KV_BF16) {
-              a = f16_bits_to_float(word & 0xffffu);
-              c = f16_bits_to_float(word >> 16);
-            } else {
-              a = bf16_bits_to_float(word & 0xffffu);
-              c = bf16_bits_to_float(word >> 16);
-            }
-            w[j] = __builtin_bit_cast(uint32_t, make_pair<Pair>(a, c));
-          }
-        }
         qop[nq][sl] = __builtin_bit_cast(V8, w);
       }
     }
@@ -559,6 +555,29 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
       stage(t + 1, set_b, set_a);
     }
     __syncthreads();
+    if (!q_is_operand_type) {
+#pragma unroll
+      for (int nq = 0; nq < kRowTiles; ++nq) {
+#pragma unroll
+        for (int sl = 0; sl < NS; ++sl) {
+          uint4_t w = __builtin_bit_cast(uint4_t, qop[nq][sl]);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const uint32_t word = w[j];
+            float a, c;
+            if constexpr (OPK == KV_BF16) {
+              a = f16_bits_to_float(word & 0xffffu);
+              c = f16_bits_to_float(word >> 16);
+            } else {
+              a = bf16_bits_to_float(word & 0xffffu);
+              c = bf16_bits_to_float(word >> 16);
+            }
+            w[j] = __builtin_bit_cast(uint32_t, make_pair<Pair>(a, c));
+          }
+          qop[nq][sl] = __builtin_bit_cast(V8, w);
+        }
+      }
+    }
     if (DS == 1 && wave_live) scores(ta, s_cur);
 
     // ---- iteration t: staging first, then the scores of tile t + 1 go to the matrix cores in the same block as the row
@@ -764,14 +783,17 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
         do {
           ++pos.seq;
           if (pos.seq >= p.num_seqs) break;
-          pos.n_new = p.cu_seqlens_q[pos.seq + 1] - p.cu_seqlens_q[pos.seq];
+          pos.q_begin = p.cu_seqlens_q[pos.seq];
+          pos.n_new = p.cu_seqlens_q[pos.seq + 1] - pos.q_begin;
         } while (pos.n_new == 0);
         if (pos.seq >= p.num_seqs) break;  // cannot happen while the prefix sums and this walk agree
         pos.ctx = p.context_lens != nullptr ? p.context_lens[pos.seq] : 0;
       }
       pos.tile = block_tiles(pos.n_new, pos.ctx, pos.j, tq, p.window_left).tile_lo;
     }
-    __syncthreads();  // every wave has left the segment before its LDS tiles are reused
+    // every wave has left the segment before its LDS tiles are reused.  Only LDS is ordered here: a barrier that also
+    // orders global memory waits for the acknowledgement of the output rows just stored, 3 us per item.
+    lds_barrier();
   }
 }
 
@@ -809,7 +831,7 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
   while (unit_start_step(total, u_hi, p.units) > item_x1 - 1) --u_hi;
   while (u_hi + 1 < p.units && unit_start_step(total, u_hi + 1, p.units) <= item_x1 - 1) ++u_hi;
 
-  const int q_begin = p.cu_seqlens_q[pos.seq];
+  const int q_begin = pos.q_begin;
   // The partials of a slot are one contiguous block of rows x head_dim floats, walked as a flat array of 16-byte
   // chunks, consecutive threads on consecutive chunks (a thread per row part left three quarters of every fetched
   // line to a later instruction).  The kernel is a chain of dependent round trips on one workgroup per CU, so the
