@@ -52,7 +52,9 @@ namespace areno {
 
 // LDS row that holds tile token t of the V tile: the second half is rotated by 4 rows so that the 8 tokens a
 // lane group reads through the transpose load ({4g..4g+3} and {16+4g..16+4g+3}) sit in rows distinct mod 16.
-// Workgroup barrier that orders LDS accesses only (no wait for outstanding global stores or loads).
+// Workgroup barrier that orders LDS accesses only.  The waves of this kernel exchange data through LDS alone, and a
+// barrier that also orders global memory waits for the acknowledgement of every output row stored before it (~3 us
+// behind an item's end), together with every fetch in front of those stores.
 __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
@@ -308,36 +310,227 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
   };
 
   StepPos pos = locate_step(p, s_cum, tq, x_begin);
-  int x = x_begin;
-  bool first_item = true;
-  while (x < x_end) {
-    // ---- one segment: key tiles [ta, tb] of item (pos.seq, pos.j) ------------------------------------------------
-    const BlockTiles item = block_tiles(pos.n_new, pos.ctx, pos.j, tq, p.window_left);
-    const int ta = pos.tile;
-    const int tb = min(item.tile_hi, ta + (x_end - x) - 1);
-    const bool whole = ta == item.tile_lo && tb == item.tile_hi;
-    const int q_begin = pos.q_begin;
-    const int ctx = pos.ctx;
-    const int tok0 = item.tok0;
-    const int tok_cnt = item.cnt;
-    const int key_hi = ctx + tok0 + tok_cnt - 1;
-    // packed K/V have no table: the id load then reads a valid dummy word and its value is ignored
-    const int32_t* table_row =
-        packed ? p.cu_seqlens_q : p.block_table + static_cast<int64_t>(pos.seq) * p.max_blocks;
 
-    // ---- this lane's query rows: row R = wave * 16 RT + 16 * nq + lr -> token tok0 + (R >> group_shift), head
-    // R & (group_pad - 1) --------------------------------------------------------------------------------------------
-    int q_pos[kRowTiles];         // absolute position of the row's query, or -1 for a padding row
-    int64_t row_elem[kRowTiles];  // element offset of the row in q / out
-    V8 qop[kRowTiles][NS];
+  // What the staging steps ask block ids for: the item whose tiles are being fetched.  It is switched to the next
+  // item before the current item's output is stored (see the end of the item loop).
+  int fc_key_hi = 0, fc_q_begin = 0;
+  const int32_t* fc_table_row = p.cu_seqlens_q;
+  // ---- the tile pipeline -----------------------------------------------------------------------------------------
+  // What one staging step fetches is published two steps later, so a fetch has two tile steps to arrive; block ids
+  // are fetched two steps ahead of the chunk they locate.  Two sets of fetch registers alternate from step to step
+  // (the tile loop is unrolled by two, so which set a step uses is fixed at compile time).
+  struct FetchSet {
+    int ids[NLD], keys[NLD];  // block id and key position of the tile to fetch next into this set
+    uint4_t kreg[NLD], vreg[NLD];
+    scale_raw_t ksreg[NLD], vsreg[NLD];
+    uint32_t k_row[NLD];  // page row of the K chunk in this set: the V chunk of the same tile is fetched a step later
+  };
+  FetchSet set_a, set_b;
+  {
+    FetchSet zero;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      zero.ids[i] = zero.keys[i] = 0;
+      zero.kreg[i] = zero.vreg[i] = uint4_t{0u, 0u, 0u, 0u};
+      zero.ksreg[i] = zero.vsreg[i] = scale_raw_t(0);
+      zero.k_row[i] = 0;
+    }
+    set_a = zero;
+    set_b = zero;
+  }
+  // Addresses.  The cache row of key t is page_row * kv_heads + kvh with page_row = (block id << bs_shift) + t's slot
+  // (packed K/V: q_begin + t), so a chunk's byte address is one 32 x 32 -> 64-bit multiply-add on a base that already
+  // holds the pool, the head and the chunk's column (the launcher checks that page rows fit 32 bits).  The key a
+  // block id was fetched for travels with the id.
+  const uint32_t row_stride = static_cast<uint32_t>(p.kv_heads) * static_cast<uint32_t>(row_bytes);
+  const uint32_t scale_stride = static_cast<uint32_t>(p.kv_heads) * static_cast<uint32_t>(sizeof(scale_raw_t));
+  const uint32_t slot_mask = static_cast<uint32_t>(p.block_size - 1);
+  auto chunk_base = [&](const void* pool, int i) {
+    return static_cast<const char*>(pool) + static_cast<int64_t>(kvh) * row_bytes + chunk_col[i] * 16;
+  };
+  auto scale_base = [&](const void* pool) {
+    return static_cast<const char*>(pool) + static_cast<int64_t>(kvh) * static_cast<int64_t>(sizeof(scale_raw_t));
+  };
+  auto chunk_at = [&](const char* base, uint32_t page_row) {
+    return *reinterpret_cast<const uint4_t*>(base + static_cast<uint64_t>(page_row) * row_stride);
+  };
+  auto scale_at = [&](const char* base, uint32_t page_row) {
+    return *reinterpret_cast<const scale_raw_t*>(base + static_cast<uint64_t>(page_row) * scale_stride);
+  };
+  // Page sizes that are no power of two have instances of their own (ANYPAGE; a choice at run time cost the
+  // power-of-two instances 5 % of the launch): the key's column by a multiplication and a shift, the slot kept in
+  // place of the key, the page row as a 24-bit multiply-add (the launcher checks the ranges).
+  auto load_ids = [&](FetchSet& f, int tile) {
+    int col[NLD];
+    if constexpr (ANYPAGE) {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const int key = max(0, min(tile * TK + chunk_tok[i], fc_key_hi));
+        col[i] = static_cast<int>(__umulhi(static_cast<uint32_t>(key), p.bs_magic) >> p.bs_post);
+        f.keys[i] = key - __mul24(col[i], p.block_size);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const int key = max(0, min(tile * TK + chunk_tok[i], fc_key_hi));
+        f.keys[i] = packed ? fc_q_begin + key : key;  // packed K/V: the key's row itself
+        col[i] = packed ? 0 : (key >> p.bs_shift);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) f.ids[i] = fc_table_row[col[i]];
+  };
+  // packed K/V run as one page per token with the token's row as its id
+  auto page_row_of = [&](const FetchSet& f, int i) -> uint32_t {
+    if constexpr (ANYPAGE) return static_cast<uint32_t>(__mul24(f.ids[i], p.block_size) + f.keys[i]);
+    const uint32_t paged = (static_cast<uint32_t>(f.ids[i]) << p.bs_shift) + (static_cast<uint32_t>(f.keys[i]) & slot_mask);
+    return packed ? static_cast<uint32_t>(f.keys[i]) : paged;
+  };
+  // The empty asm pins the use of a fetched chunk to this point of the iteration: without it the compiler converts
+  // the codes right at the top of the loop and every tile waits there for the loads it has just issued.
+  auto publish_k = [&](FetchSet& f, int tile) {
+    char* kd = s_k[tile & 1];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      asm volatile("" : "+v"(f.kreg[i]));
+      if (!chunk_live[i]) continue;
+      const int t = chunk_tok[i];
+      if constexpr (T::kQuant) {
+        uint4_t lo, hi;
+        dequant_chunk<KIND>(f.kreg[i], scale_value(f.ksreg[i]), lo, hi);
+        char* kdst = kd + t * RSK + chunk_col[i] * 32;
+        *reinterpret_cast<uint4_t*>(kdst) = lo;
+        *reinterpret_cast<uint4_t*>(kdst + 16) = hi;
+      } else {
+        *reinterpret_cast<uint4_t*>(kd + t * RSK + chunk_col[i] * 16) = f.kreg[i];
+      }
+    }
+  };
+  auto publish_v = [&](FetchSet& f, int tile) {
+    char* vd = s_v[tile & 1];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      asm volatile("" : "+v"(f.vreg[i]));
+      if (!chunk_live[i]) continue;
+      const int t = chunk_tok[i];
+      if constexpr (T::kQuant) {
+        uint4_t lo, hi;
+        dequant_chunk<KIND>(f.vreg[i], scale_value(f.vsreg[i]), lo, hi);
+        char* vdst = vd + v_row_of(t) * RSV + chunk_col[i] * 32;
+        *reinterpret_cast<uint4_t*>(vdst) = lo;
+        *reinterpret_cast<uint4_t*>(vdst + 16) = hi;
+      } else {
+        *reinterpret_cast<uint4_t*>(vd + v_row_of(t) * RSV + chunk_col[i] * 16) = f.vreg[i];
+      }
+    }
+  };
+  const char* const role_base = chunk_base(role_v ? p.v_cache : p.k_cache, 0);
+  const char* const role_scale_base = scale_base(role_v ? p.v_scale : p.k_scale);
+  // Staging step of iteration t with the fetch set `mine` of its parity (`other` is the previous and the next
+  // step's): K[t + 2] and V[t + 1], fetched two steps ago, go from the registers into the LDS buffers the previous
+  // iteration was the last to read; then K[t + 4] and V[t + 3] are fetched into the same registers, and the block
+  // ids of K[t + 6] / V[t + 5].  It runs for every t (key positions are clamped into the item's range): tiles
+  // outside [ta, tb] land in buffers nobody reads.
+  auto stage = [&](int t, FetchSet& mine, FetchSet& other) {
+    if constexpr (kRoleSplit) {
+      // one chunk per thread: kreg / ksreg / ids hold the K chunk in a K wave and the V chunk in a V wave.  V runs
+      // one tile behind K, as in the unsplit scheme.
+      const int behind = role_v ? 1 : 0;
+      asm volatile("" : "+v"(mine.kreg[0]));
+      if (chunk_live[0]) {
+        const int tk = chunk_tok[0];
+        const int pub = t + 2 - behind;
+        char* dst = role_v ? s_v[pub & 1] + v_row_of(tk) * RSV : s_k[pub & 1] + tk * RSK;
+        if constexpr (T::kQuant) {
+          uint4_t lo, hi;
+          dequant_chunk<KIND>(mine.kreg[0], scale_value(mine.ksreg[0]), lo, hi);
+          *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 32) = lo;
+          *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 32 + 16) = hi;
+        } else {
+          *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 16) = mine.kreg[0];
+        }
+      }
+      const uint32_t row = page_row_of(mine, 0);  // the ids of tile t + 4 - behind, fetched two steps ago
+      mine.kreg[0] = chunk_at(role_base, row);
+      if constexpr (T::kQuant) mine.ksreg[0] = scale_at(role_scale_base, row);
+      load_ids(mine, t + 6 - behind);
+    } else {
+      publish_k(mine, t + 2);
+      publish_v(mine, t + 1);
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        // V[t + 3]: the rows of K[t + 3], which the previous step fetched
+        mine.vreg[i] = chunk_at(chunk_base(p.v_cache, i), other.k_row[i]);
+        if constexpr (T::kQuant) mine.vsreg[i] = scale_at(scale_base(p.v_scale), other.k_row[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const uint32_t row = page_row_of(mine, i);  // the ids of tile t + 4, fetched two steps ago
+        mine.k_row[i] = row;
+        mine.kreg[i] = chunk_at(chunk_base(p.k_cache, i), row);
+        if constexpr (T::kQuant) mine.ksreg[i] = scale_at(scale_base(p.k_scale), row);
+      }
+      load_ids(mine, t + 6);
+    }
+  };
+
+
+  // ---- the unit's segments ---------------------------------------------------------------------------------------
+  // A segment is the part of an item (sequence, query block) inside the unit: key tiles [ta, tb].
+  struct Segment {
+    int seq, ta, tb, q_begin, ctx, tok0, tok_cnt;
+    bool whole;  // the item's first and last tile are both here: its rows are final
+  };
+  auto segment_at = [&](const StepPos& q, int x_at) {
+    const BlockTiles item = block_tiles(q.n_new, q.ctx, q.j, tq, p.window_left);
+    Segment g;
+    g.seq = q.seq;
+    g.ta = q.tile;
+    g.tb = min(item.tile_hi, q.tile + (x_end - x_at) - 1);
+    g.whole = g.ta == item.tile_lo && g.tb == item.tile_hi;
+    g.q_begin = q.q_begin;
+    g.ctx = q.ctx;
+    g.tok0 = item.tok0;
+    g.tok_cnt = item.cnt;
+    return g;
+  };
+  auto set_fetch_context = [&](const Segment& g) {
+    fc_key_hi = g.ctx + g.tok0 + g.tok_cnt - 1;
+    fc_q_begin = g.q_begin;
+    // packed K/V have no table: the id load then reads a valid dummy word and its value is ignored
+    fc_table_row = packed ? p.cu_seqlens_q : p.block_table + static_cast<int64_t>(g.seq) * p.max_blocks;
+  };
+  // the item behind q in the unit's order; false when the list is exhausted (cannot happen while the prefix sums and
+  // this walk agree)
+  auto next_position = [&](StepPos& q) -> bool {
+    ++q.j;
+    if (q.j * tq >= q.n_new) {
+      q.j = 0;
+      do {
+        ++q.seq;
+        if (q.seq >= p.num_seqs) return false;
+        q.q_begin = p.cu_seqlens_q[q.seq];
+        q.n_new = p.cu_seqlens_q[q.seq + 1] - q.q_begin;
+      } while (q.n_new == 0);
+      q.ctx = p.context_lens != nullptr ? p.context_lens[q.seq] : 0;
+    }
+    q.tile = block_tiles(q.n_new, q.ctx, q.j, tq, p.window_left).tile_lo;
+    return true;
+  };
+  // ---- this lane's query rows: row R = wave * 16 RT + 16 * nq + lr -> token tok0 + (R >> group_shift), head
+  // R & (group_pad - 1) ----------------------------------------------------------------------------------------------
+  int q_pos[kRowTiles];         // absolute position of the row's query, or -1 for a padding row
+  int64_t row_elem[kRowTiles];  // element offset of the row in q / out
+  V8 qop[kRowTiles][NS];
+  auto load_q = [&](const Segment& g) {
 #pragma unroll
     for (int nq = 0; nq < kRowTiles; ++nq) {
       const int r = row_wave * kRowsPerWave + 16 * nq + lr;
       const int t = r >> p.group_shift;
       const int hh = r & (p.group_pad - 1);
-      const bool live = t < tok_cnt && hh < group_here;
-      q_pos[nq] = live ? ctx + tok0 + t : -1;
-      row_elem[nq] = (static_cast<int64_t>(q_begin + tok0 + t) * p.q_heads + head0 + hh) * D;
+      const bool live = t < g.tok_cnt && hh < group_here;
+      q_pos[nq] = live ? g.ctx + g.tok0 + t : -1;
+      row_elem[nq] = (static_cast<int64_t>(g.q_begin + g.tok0 + t) * p.q_heads + head0 + hh) * D;
 #pragma unroll
       for (int sl = 0; sl < NS; ++sl) {
         // (as fetched: a query of the other 16-bit type is converted behind the pipeline's fill, so that its fetch
@@ -347,6 +540,20 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
         qop[nq][sl] = __builtin_bit_cast(V8, w);
       }
     }
+  };
+
+  int x = x_begin;
+  bool first_item = true;
+  Segment seg = segment_at(pos, x);
+  set_fetch_context(seg);
+  load_q(seg);
+  int prefilled = 0;  // staging steps of the segment's fill that ran before the previous segment's output was stored
+  for (;;) {
+    // ---- one segment: key tiles [ta, tb] of an item ------------------------------------------------------------------
+    const int ta = seg.ta, tb = seg.tb;
+    const bool whole = seg.whole;
+    const int ctx = seg.ctx, tok0 = seg.tok0, tok_cnt = seg.tok_cnt;
+
     // rows of this wave: which query positions they span (wave-uniform), for skipping the mask on interior tiles
     const bool wave_live = row_wave * kRowsPerWave < (tok_cnt << p.group_shift);
     const int wave_qmin = ctx + tok0 + ((row_wave * kRowsPerWave) >> p.group_shift);
@@ -367,164 +574,6 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) acc[nq][nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     }
-
-    // ---- the tile pipeline -----------------------------------------------------------------------------------------
-    // What one staging step fetches is published two steps later, so a fetch has two tile steps to arrive; block ids
-    // are fetched two steps ahead of the chunk they locate.  Two sets of fetch registers alternate from step to step
-    // (the tile loop is unrolled by two, so which set a step uses is fixed at compile time).
-    struct FetchSet {
-      int ids[NLD], keys[NLD];  // block id and key position of the tile to fetch next into this set
-      uint4_t kreg[NLD], vreg[NLD];
-      scale_raw_t ksreg[NLD], vsreg[NLD];
-      uint32_t k_row[NLD];  // page row of the K chunk in this set: the V chunk of the same tile is fetched a step later
-    };
-    FetchSet set_a, set_b;
-    {
-      FetchSet zero;
-#pragma unroll
-      for (int i = 0; i < NLD; ++i) {
-        zero.ids[i] = zero.keys[i] = 0;
-        zero.kreg[i] = zero.vreg[i] = uint4_t{0u, 0u, 0u, 0u};
-        zero.ksreg[i] = zero.vsreg[i] = scale_raw_t(0);
-        zero.k_row[i] = 0;
-      }
-      set_a = zero;
-      set_b = zero;
-    }
-    // Addresses.  The cache row of key t is page_row * kv_heads + kvh with page_row = (block id << bs_shift) + t's slot
-    // (packed K/V: q_begin + t), so a chunk's byte address is one 32 x 32 -> 64-bit multiply-add on a base that already
-    // holds the pool, the head and the chunk's column (the launcher checks that page rows fit 32 bits).  The key a
-    // block id was fetched for travels with the id.
-    const uint32_t row_stride = static_cast<uint32_t>(p.kv_heads) * static_cast<uint32_t>(row_bytes);
-    const uint32_t scale_stride = static_cast<uint32_t>(p.kv_heads) * static_cast<uint32_t>(sizeof(scale_raw_t));
-    const uint32_t slot_mask = static_cast<uint32_t>(p.block_size - 1);
-    auto chunk_base = [&](const void* pool, int i) {
-      return static_cast<const char*>(pool) + static_cast<int64_t>(kvh) * row_bytes + chunk_col[i] * 16;
-    };
-    auto scale_base = [&](const void* pool) {
-      return static_cast<const char*>(pool) + static_cast<int64_t>(kvh) * static_cast<int64_t>(sizeof(scale_raw_t));
-    };
-    auto chunk_at = [&](const char* base, uint32_t page_row) {
-      return *reinterpret_cast<const uint4_t*>(base + static_cast<uint64_t>(page_row) * row_stride);
-    };
-    auto scale_at = [&](const char* base, uint32_t page_row) {
-      return *reinterpret_cast<const scale_raw_t*>(base + static_cast<uint64_t>(page_row) * scale_stride);
-    };
-    // Page sizes that are no power of two have instances of their own (ANYPAGE; a choice at run time cost the
-    // power-of-two instances 5 % of the launch): the key's column by a multiplication and a shift, the slot kept in
-    // place of the key, the page row as a 24-bit multiply-add (the launcher checks the ranges).
-    auto load_ids = [&](FetchSet& f, int tile) {
-      int col[NLD];
-      if constexpr (ANYPAGE) {
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-          const int key = max(0, min(tile * TK + chunk_tok[i], key_hi));
-          col[i] = static_cast<int>(__umulhi(static_cast<uint32_t>(key), p.bs_magic) >> p.bs_post);
-          f.keys[i] = key - __mul24(col[i], p.block_size);
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-          f.keys[i] = max(0, min(tile * TK + chunk_tok[i], key_hi));
-          col[i] = packed ? 0 : (f.keys[i] >> p.bs_shift);
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < NLD; ++i) f.ids[i] = table_row[col[i]];
-    };
-    // packed K/V run as one page per token with the token's row as its id
-    auto page_row_of = [&](const FetchSet& f, int i) -> uint32_t {
-      if constexpr (ANYPAGE) return static_cast<uint32_t>(__mul24(f.ids[i], p.block_size) + f.keys[i]);
-      const uint32_t paged = (static_cast<uint32_t>(f.ids[i]) << p.bs_shift) + (static_cast<uint32_t>(f.keys[i]) & slot_mask);
-      return packed ? static_cast<uint32_t>(q_begin + f.keys[i]) : paged;
-    };
-    // The empty asm pins the use of a fetched chunk to this point of the iteration: without it the compiler converts
-    // the codes right at the top of the loop and every tile waits there for the loads it has just issued.
-    auto publish_k = [&](FetchSet& f, int tile) {
-      char* kd = s_k[tile & 1];
-#pragma unroll
-      for (int i = 0; i < NLD; ++i) {
-        asm volatile("" : "+v"(f.kreg[i]));
-        if (!chunk_live[i]) continue;
-        const int t = chunk_tok[i];
-        if constexpr (T::kQuant) {
-          uint4_t lo, hi;
-          dequant_chunk<KIND>(f.kreg[i], scale_value(f.ksreg[i]), lo, hi);
-          char* kdst = kd + t * RSK + chunk_col[i] * 32;
-          *reinterpret_cast<uint4_t*>(kdst) = lo;
-          *reinterpret_cast<uint4_t*>(kdst + 16) = hi;
-        } else {
-          *reinterpret_cast<uint4_t*>(kd + t * RSK + chunk_col[i] * 16) = f.kreg[i];
-        }
-      }
-    };
-    auto publish_v = [&](FetchSet& f, int tile) {
-      char* vd = s_v[tile & 1];
-#pragma unroll
-      for (int i = 0; i < NLD; ++i) {
-        asm volatile("" : "+v"(f.vreg[i]));
-        if (!chunk_live[i]) continue;
-        const int t = chunk_tok[i];
-        if constexpr (T::kQuant) {
-          uint4_t lo, hi;
-          dequant_chunk<KIND>(f.vreg[i], scale_value(f.vsreg[i]), lo, hi);
-          char* vdst = vd + v_row_of(t) * RSV + chunk_col[i] * 32;
-          *reinterpret_cast<uint4_t*>(vdst) = lo;
-          *reinterpret_cast<uint4_t*>(vdst + 16) = hi;
-        } else {
-          *reinterpret_cast<uint4_t*>(vd + v_row_of(t) * RSV + chunk_col[i] * 16) = f.vreg[i];
-        }
-      }
-    };
-    const char* const role_base = chunk_base(role_v ? p.v_cache : p.k_cache, 0);
-    const char* const role_scale_base = scale_base(role_v ? p.v_scale : p.k_scale);
-    // Staging step of iteration t with the fetch set `mine` of its parity (`other` is the previous and the next
-    // step's): K[t + 2] and V[t + 1], fetched two steps ago, go from the registers into the LDS buffers the previous
-    // iteration was the last to read; then K[t + 4] and V[t + 3] are fetched into the same registers, and the block
-    // ids of K[t + 6] / V[t + 5].  It runs for every t (key positions are clamped into the item's range): tiles
-    // outside [ta, tb] land in buffers nobody reads.
-    auto stage = [&](int t, FetchSet& mine, FetchSet& other) {
-      if constexpr (kRoleSplit) {
-        // one chunk per thread: kreg / ksreg / ids hold the K chunk in a K wave and the V chunk in a V wave.  V runs
-        // one tile behind K, as in the unsplit scheme.
-        const int behind = role_v ? 1 : 0;
-        asm volatile("" : "+v"(mine.kreg[0]));
-        if (chunk_live[0]) {
-          const int tk = chunk_tok[0];
-          const int pub = t + 2 - behind;
-          char* dst = role_v ? s_v[pub & 1] + v_row_of(tk) * RSV : s_k[pub & 1] + tk * RSK;
-          if constexpr (T::kQuant) {
-            uint4_t lo, hi;
-            dequant_chunk<KIND>(mine.kreg[0], scale_value(mine.ksreg[0]), lo, hi);
-            *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 32) = lo;
-            *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 32 + 16) = hi;
-          } else {
-            *reinterpret_cast<uint4_t*>(dst + chunk_col[0] * 16) = mine.kreg[0];
-          }
-        }
-        const uint32_t row = page_row_of(mine, 0);  // the ids of tile t + 4 - behind, fetched two steps ago
-        mine.kreg[0] = chunk_at(role_base, row);
-        if constexpr (T::kQuant) mine.ksreg[0] = scale_at(role_scale_base, row);
-        load_ids(mine, t + 6 - behind);
-      } else {
-        publish_k(mine, t + 2);
-        publish_v(mine, t + 1);
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-          // V[t + 3]: the rows of K[t + 3], which the previous step fetched
-          mine.vreg[i] = chunk_at(chunk_base(p.v_cache, i), other.k_row[i]);
-          if constexpr (T::kQuant) mine.vsreg[i] = scale_at(scale_base(p.v_scale), other.k_row[i]);
-        }
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-          const uint32_t row = page_row_of(mine, i);  // the ids of tile t + 4, fetched two steps ago
-          mine.k_row[i] = row;
-          mine.kreg[i] = chunk_at(chunk_base(p.k_cache, i), row);
-          if constexpr (T::kQuant) mine.ksreg[i] = scale_at(scale_base(p.k_scale), row);
-        }
-        load_ids(mine, t + 6);
-      }
-    };
 
     // raw scores of one key tile: S^T = K . Q^T
     float s_cur[kRowTiles][2][4];
@@ -548,13 +597,13 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
     };
 
     // ---- fill the pipe: after these iterations K[ta], K[ta + 1] and V[ta] are in LDS (the first ones only fetch) ------
-    for (int t = ta - 6; t < ta; t += 2) {
-      __syncthreads();
+    for (int t = ta - 6 + prefilled; t < ta; t += 2) {
+      lds_barrier();
       stage(t, set_a, set_b);
-      __syncthreads();
+      lds_barrier();
       stage(t + 1, set_b, set_a);
     }
-    __syncthreads();
+    lds_barrier();
     if (!q_is_operand_type) {
 #pragma unroll
       for (int nq = 0; nq < kRowTiles; ++nq) {
@@ -588,7 +637,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
     float s_alt[kRowTiles][2][4];
     auto tile_step = [&](int t, float (&s_cur)[kRowTiles][2][4], float (&s_next)[kRowTiles][2][4], FetchSet& mine,
                          FetchSet& other) {
-      __syncthreads();
+      lds_barrier();
       if constexpr (DS == 1) stage(t, mine, other);
       if constexpr (DS > 1) {
         // A split head computes the scores of tile t here (K[t] was published two steps ago), hands its part to the
@@ -605,7 +654,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
             for (int j = 0; j < 4; ++j) s_part[wave][tg][j][lane] = s_cur[0][tg][j];
           }
         }
-        __syncthreads();
+        lds_barrier();
         stage(t, mine, other);
         if (wave_live) {
 #pragma unroll
@@ -737,17 +786,40 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
       tile_step(t + 1, s_alt, s_cur, set_b, set_a);
     }
 
+    // ---- the next segment's first fetches go out in front of this segment's output -------------------------------
+    // The memory queue retires in order: whatever is fetched behind the output stores is waited for together with
+    // their acknowledgement (~3 us).  So the next segment's query rows and the block ids of its first two tiles (the
+    // first two steps of its fill) are requested here, and the rest of its fill runs while the stores drain.
+    x += tb - ta + 1;
+    const bool more = x < x_end && next_position(pos);
+    int done_q_pos[kRowTiles];
+    int64_t done_row_elem[kRowTiles];
+#pragma unroll
+    for (int nq = 0; nq < kRowTiles; ++nq) {
+      done_q_pos[nq] = q_pos[nq];
+      done_row_elem[nq] = row_elem[nq];
+    }
+    if (more) {
+      seg = segment_at(pos, x);
+      set_fetch_context(seg);
+      lds_barrier();  // every wave has left this segment's tiles (only LDS needs ordering here)
+      stage(seg.ta - 6, set_a, set_b);
+      lds_barrier();
+      stage(seg.ta - 5, set_b, set_a);
+      load_q(seg);
+    }
+
     // ---- finish the segment: final rows go to `out`, a cut item leaves its partial in the workspace ---------------
     const int slot = 2 * unit + (first_item ? 0 : 1);
 #pragma unroll
     for (int nq = 0; nq < kRowTiles; ++nq) {
       const float l_tot = l_acc[nq][0];
-      if (q_pos[nq] < 0) continue;
+      if (done_q_pos[nq] < 0) continue;
       if (whole) {
         const float inv = 1.0f / l_tot;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-          const int64_t e0 = row_elem[nq] + d0 + 16 * nb + 4 * lk;
+          const int64_t e0 = done_row_elem[nq] + d0 + 16 * nb + 4 * lk;
           uint32_t lo, hi;
           const float o0 = acc[nq][nb][0] * inv, o1 = acc[nq][nb][1] * inv;
           const float o2 = acc[nq][nb][2] * inv, o3 = acc[nq][nb][3] * inv;
@@ -773,27 +845,9 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
       }
     }
 
-    // ---- next item ---------------------------------------------------------------------------------------------------
-    x += tb - ta + 1;
     first_item = false;
-    if (x < x_end) {
-      ++pos.j;
-      if (pos.j * tq >= pos.n_new) {
-        pos.j = 0;
-        do {
-          ++pos.seq;
-          if (pos.seq >= p.num_seqs) break;
-          pos.q_begin = p.cu_seqlens_q[pos.seq];
-          pos.n_new = p.cu_seqlens_q[pos.seq + 1] - pos.q_begin;
-        } while (pos.n_new == 0);
-        if (pos.seq >= p.num_seqs) break;  // cannot happen while the prefix sums and this walk agree
-        pos.ctx = p.context_lens != nullptr ? p.context_lens[pos.seq] : 0;
-      }
-      pos.tile = block_tiles(pos.n_new, pos.ctx, pos.j, tq, p.window_left).tile_lo;
-    }
-    // every wave has left the segment before its LDS tiles are reused.  Only LDS is ordered here: a barrier that also
-    // orders global memory waits for the acknowledgement of the output rows just stored, 3 us per item.
-    lds_barrier();
+    if (!more) break;
+    prefilled = 2;
   }
 }
 
