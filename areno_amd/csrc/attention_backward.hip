@@ -19,35 +19,15 @@
 // elements wide (the smallest that covers the head; slices past the head's end read as zeros and are not stored);
 // 16-bit or fp32 inputs.
 
+#include <stdlib.h>
+#include <string.h>
+
 #include "device_common.hpp"
+#include "attention_backward.hpp"
 
 namespace areno {
 namespace {
 
-struct BwdParams {
-  const void* grad_out;
-  const void* q;
-  const void* k;
-  const void* v;
-  const void* out;
-  float* grad_q;
-  float* grad_k;
-  float* grad_v;
-  float* row_stats;  // [q_tokens * q_heads][2]: log2-domain log-sum-exp of the scaled scores, dO . O
-  const int32_t* cu_q;
-  const int32_t* cu_k;
-  const int32_t* ctx;  // may be nullptr: 0
-  int64_t q_tokens;
-  int64_t k_tokens;
-  int32_t num_seqs;
-  int32_t q_heads;
-  int32_t kv_heads;
-  int32_t window_left;
-  int32_t head_dim;
-  int32_t dtype;
-  float scale;
-  float scale_log2e;
-};
 
 constexpr int kBwdWaves = 4;
 constexpr int kLanesPerKey = 4;
@@ -362,6 +342,16 @@ extern "C" int areno_hip_attention_backward(const void* grad_out, const void* q,
   p.dtype = dtype;
   p.scale = softmax_scale;
   p.scale_log2e = softmax_scale * kLog2e;
+  // 16-bit inputs at head dims 64 and 128 run on the matrix cores (ARENO_BACKWARD_KERNEL=valu: a diagnosis switch
+  // that keeps them on the kernels below)
+  static const bool valu_only = [] {
+    const char* e = getenv("ARENO_BACKWARD_KERNEL");
+    return e != nullptr && strcmp(e, "valu") == 0;
+  }();
+  if (!valu_only) {
+    const int rc = launch_attention_backward_mfma(p, stream);
+    if (rc != ARENO_ERR_UNSUPPORTED) return rc;
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (q_rows > 0) {
     hipLaunchKernelGGL(rows, dim3(static_cast<unsigned>((q_rows + kBwdWaves - 1) / kBwdWaves)), dim3(kBwdWaves * kWave), 0,

@@ -1,0 +1,443 @@
+// Backward of the causal varlen / dense attention ops on the matrix cores (gfx950): 16-bit inputs, head dims 64 and
+// 128.  Same contract as the vector-ALU kernels of attention_backward.hip (fp32 dQ, dK, dV from dO, Q, K, V and the
+// saved output; areno/accel/csrc/attention.cu:244-524 in the reference), same two launches, no atomics:
+//
+//   dq kernel    a workgroup owns 64 packed query rows of one q head (four waves of 16 rows) and streams the keys its
+//                rows may see in tiles of 32 through LDS.  Per tile, with the keys as the rows of the products (the
+//                layout of the forward kernel):  S^T = K . Q^T  and  dP^T = V . dO^T  (two products per 16 keys and 32
+//                elements of the head), the online softmax of the forward on S^T, dS^T = P^T * (dP^T - dO . O), and
+//                dQ^T += K^T . dS^T  with the lane's own dS^T values as the B operand and K^T read transposed from the
+//                same LDS tile.  A row's softmax reference moves as in the forward (the accumulator is rescaled), so
+//                one pass over the keys gives dQ, the row's log-sum-exp and dO . O (left in the workspace).
+//   dkv kernel   a workgroup owns 64 packed key rows of one kv head and streams, for every q head of the group, the
+//                query rows that may see them in tiles of 32 (Q and dO tiles in LDS, the rows' statistics next to
+//                them):  S = Q . K^T,  dP = dO . V^T,  P = exp2(S - lse),  dS = P * (dP - dO . O),
+//                dV^T += dO^T . P  and  dK^T += Q^T . dS.  Every gradient element has one owner.
+//
+// The streamed index of a tile (keys in the dq kernel, queries in the dkv kernel) is the contraction index of the
+// second pair of products; a 16 x 16 product leaves element 4 g + j of that index in lane group g, which is exactly
+// how the next product wants its B operand, and the A operand comes from the LDS tile through transposing reads
+// (ds_read_b64_tr_b16), so nothing is shuffled between the products.
+// Geometry as in attention_backward.hip: sequence s has queries [cu_q[s], cu_q[s+1]) at positions ctx[s] + i and keys
+// [cu_k[s], cu_k[s+1]) at positions 0 ..; a query at position t sees keys max(0, t - window) .. t.  A block of 64
+// packed rows may hold rows of several sequences; it goes through them one after the other, the rows of the others
+// masked.
+
+#include "attention_backward.hpp"
+#include "decode_mfma_kernels.hpp"
+
+namespace areno {
+namespace {
+
+constexpr int kBmWaves = 4;
+constexpr int kBmThreads = kBmWaves * kWave;
+constexpr int kBmRows = 16 * kBmWaves;  // packed rows a workgroup owns
+constexpr int kBmTile = 32;             // streamed rows per step
+constexpr float kBmNegInf = -__builtin_huge_valf();
+
+// the last sequence that starts at or in front of `row` (the one that holds it, when the row exists)
+__device__ __forceinline__ int seq_of_row(const int32_t* cu, int num_seqs, int64_t row) {
+  int lo = 0, hi = num_seqs;
+  while (lo + 1 < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (static_cast<int64_t>(cu[mid]) <= row) {
+      lo = mid;
+    } else {
+      hi = mid;
+    }
+  }
+  return lo;
+}
+
+// A tile of 32 rows x D 16-bit elements in LDS, row stride RS bytes.  Staging: every thread moves kChunks 16-byte
+// chunks of a tensor through registers, fetched one tile ahead of their use.
+template <int D>
+struct BmTile {
+  static constexpr int RS = D * 2 + 16;
+  static constexpr int kChunksPerRow = D * 2 / 16;
+  static constexpr int kChunks = kBmTile * kChunksPerRow / kBmThreads;  // per thread: 1 (D = 64) or 2 (D = 128)
+  static_assert(kBmTile * kChunksPerRow % kBmThreads == 0, "tile chunks");
+};
+
+// Operand reads.  Row operand (A of the first pair of products): row 16 tg + lr of the tile, elements
+// (D / 4) lk + 8 sl .. + 8 -- the same split of the head over the four lane groups as the register operands.
+template <int KIND, int D>
+__device__ __forceinline__ typename MfmaOps<KIND>::vec8 tile_row_operand(const char* tile, int tg, int sl, int lr, int lk) {
+  using V8 = typename MfmaOps<KIND>::vec8;
+  return *reinterpret_cast<const V8*>(tile + (16 * tg + lr) * BmTile<D>::RS + ((D / 4) * lk + 8 * sl) * 2);
+}
+// Transposed operand (A of the second pair): head elements 16 nb + lr as rows, the tile's 32 rows as the contraction
+// index in the order lane group lk holds them after the first pair (rows 4 lk .. 4 lk + 3, then 16 + 4 lk .. + 3).
+template <int KIND, int D>
+__device__ __forceinline__ typename MfmaOps<KIND>::vec8 tile_transposed_operand(char* tile, int nb, int lr, int lk) {
+  using V8 = typename MfmaOps<KIND>::vec8;
+  uint32_t w[4];
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int row = 16 * half + 4 * lk + (lr >> 2);
+    char* a = tile + row * BmTile<D>::RS + (16 * nb + 4 * (lr & 3)) * 2;
+    const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
+    const uint2_t u = __builtin_bit_cast(uint2_t, r);
+    w[2 * half] = u[0];
+    w[2 * half + 1] = u[1];
+  }
+  return __builtin_bit_cast(V8, uint4_t{w[0], w[1], w[2], w[3]});
+}
+// eight values of the streamed index, as a lane holds them after the first pair of products ([tg][j]), as B operand
+template <int KIND>
+__device__ __forceinline__ typename MfmaOps<KIND>::vec8 streamed_operand(const float (&x)[2][4]) {
+  using V8 = typename MfmaOps<KIND>::vec8;
+  return __builtin_bit_cast(V8, uint4_t{pack_pair<KIND>(x[0][0], x[0][1]), pack_pair<KIND>(x[0][2], x[0][3]),
+                                        pack_pair<KIND>(x[1][0], x[1][1]), pack_pair<KIND>(x[1][2], x[1][3])});
+}
+template <int KIND>
+__device__ __forceinline__ float operand_element(uint32_t word, int hi) {
+  const uint32_t bits = hi ? word >> 16 : word & 0xffffu;
+  return KIND == KV_BF16 ? bf16_bits_to_float(bits) : f16_bits_to_float(bits);
+}
+
+// ---- dQ (and the rows' statistics) ------------------------------------------------------------------------------------
+template <int KIND, int D>
+__global__ __launch_bounds__(kBmThreads) void bwd_mfma_dq_kernel(BwdParams p) {
+  using Ops = MfmaOps<KIND>;
+  using V8 = typename Ops::vec8;
+  using T = BmTile<D>;
+  constexpr int NS = D / 32, NB = D / 16;
+  __shared__ __attribute__((aligned(16))) char s_k[kBmTile * T::RS];
+  __shared__ __attribute__((aligned(16))) char s_v[kBmTile * T::RS];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int lr = lane & 15, lk = lane >> 4;
+  const int h = blockIdx.y;
+  const int kvh = h / (p.q_heads / p.kv_heads);
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * kBmRows;
+  const int64_t block_end = r0 + kBmRows < p.q_tokens ? r0 + kBmRows : p.q_tokens;
+  const int64_t row = r0 + 16 * wave + lr;  // this lane's query row (a column of the products)
+
+  for (int s = seq_of_row(p.cu_q, p.num_seqs, r0); s < p.num_seqs; ++s) {
+    const int64_t sq0 = p.cu_q[s], sq1 = p.cu_q[s + 1];
+    if (sq0 >= block_end) break;
+    const int64_t q_lo = sq0 > r0 ? sq0 : r0, q_hi = sq1 < block_end ? sq1 : block_end;
+    if (q_lo >= q_hi) continue;
+    const int ctx = p.ctx != nullptr ? p.ctx[s] : 0;
+    const int64_t k_base = p.cu_k[s];
+    const int n_k = p.cu_k[s + 1] - p.cu_k[s];
+    const bool live = row >= q_lo && row < q_hi;
+    const int pos = live ? ctx + static_cast<int>(row - sq0) : -1;
+    const bool wave_live = __builtin_amdgcn_ballot_w64(live) != 0;
+    const int pos_min = ctx + static_cast<int>(q_lo - sq0), pos_max = ctx + static_cast<int>(q_hi - 1 - sq0);
+    const int key_lo = p.window_left >= 0 ? (pos_min - p.window_left > 0 ? pos_min - p.window_left : 0) : 0;
+    const int key_hi = pos_max < n_k - 1 ? pos_max : n_k - 1;
+
+    // this lane's parts of its row of Q and dO (B operands), and dO . O
+    const int64_t row_elem = (row * p.q_heads + h) * D;
+    V8 qop[NS], gop[NS];
+    float delta = 0.0f;
+#pragma unroll
+    for (int sl = 0; sl < NS; ++sl) {
+      uint4_t qw = {0u, 0u, 0u, 0u}, gw = qw, ow = qw;
+      if (live) {
+        const int64_t off = (row_elem + (D / 4) * lk + 8 * sl) * 2;
+        qw = load16(p.q, off);
+        gw = load16(p.grad_out, off);
+        ow = load16(p.out, off);
+      }
+      qop[sl] = __builtin_bit_cast(V8, qw);
+      gop[sl] = __builtin_bit_cast(V8, gw);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        delta += operand_element<KIND>(gw[j], 0) * operand_element<KIND>(ow[j], 0) +
+                 operand_element<KIND>(gw[j], 1) * operand_element<KIND>(ow[j], 1);
+      }
+    }
+    delta = rows_sum(delta);
+
+    float4_t acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = kBmNegInf, l_lane = 0.0f;
+
+    if (key_hi >= key_lo) {  // (the same for the whole workgroup)
+      const int t0 = key_lo / kBmTile, t1 = key_hi / kBmTile;
+      uint4_t kreg[T::kChunks], vreg[T::kChunks];
+      auto fetch = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < T::kChunks; ++i) {
+          const int c = tid + kBmThreads * i;
+          const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
+          const int key = kBmTile * t + r < n_k ? kBmTile * t + r : n_k - 1;  // rows past the end repeat the last key
+          const int64_t off = ((k_base + key) * p.kv_heads + kvh) * (D * 2) + col * 16;
+          kreg[i] = load16(p.k, off);
+          vreg[i] = load16(p.v, off);
+        }
+      };
+      auto publish = [&]() {
+#pragma unroll
+        for (int i = 0; i < T::kChunks; ++i) {
+          const int c = tid + kBmThreads * i;
+          const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
+          *reinterpret_cast<uint4_t*>(s_k + r * T::RS + col * 16) = kreg[i];
+          *reinterpret_cast<uint4_t*>(s_v + r * T::RS + col * 16) = vreg[i];
+        }
+      };
+      fetch(t0);
+      __syncthreads();  // the tiles' previous readers (an earlier sequence of this block) are done
+      publish();
+      __syncthreads();
+      for (int t = t0; t <= t1; ++t) {
+        if (t < t1) fetch(t + 1);
+        if (wave_live) {
+          float sc[2][4], dp[2][4];
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+            float4_t c1 = {0.0f, 0.0f, 0.0f, 0.0f}, c2 = c1;
+#pragma unroll
+            for (int sl = 0; sl < NS; ++sl) {
+              c1 = Ops::mfma(tile_row_operand<KIND, D>(s_k, tg, sl, lr, lk), qop[sl], c1);
+              c2 = Ops::mfma(tile_row_operand<KIND, D>(s_v, tg, sl, lr, lk), gop[sl], c2);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int key = kBmTile * t + 16 * tg + 4 * lk + j;
+              const bool ok = key <= pos && key < n_k && (p.window_left < 0 || key >= pos - p.window_left);
+              sc[tg][j] = ok ? c1[j] * p.scale_log2e : kBmNegInf;
+              dp[tg][j] = c2[j];
+            }
+          }
+          float mt = sc[0][0];
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) mt = fmaxf(mt, sc[tg][j]);
+          }
+          mt = rows_max(mt);
+          const float m_new = fmaxf(m_run, mt);
+          const float m_ref = m_new == kBmNegInf ? 0.0f : m_new;
+          const float alpha = fast_exp2(m_run - m_ref);  // 0 while the row has seen no key
+          m_run = m_new;
+          float ds[2][4], psum = 0.0f;
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float pe = fast_exp2(sc[tg][j] - m_ref);  // exp2(-inf) = 0 for masked keys
+              psum += pe;
+              ds[tg][j] = pe * (dp[tg][j] - delta);
+            }
+          }
+          l_lane = l_lane * alpha + psum;
+          const V8 dsop = streamed_operand<KIND>(ds);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[nb][j] *= alpha;
+            acc[nb] = Ops::mfma(tile_transposed_operand<KIND, D>(s_k, nb, lr, lk), dsop, acc[nb]);
+          }
+        }
+        __syncthreads();  // every wave has read tile t
+        if (t < t1) publish();
+        __syncthreads();
+      }
+    }
+
+    // dQ = scale / l * sum_k p_k (dP_k - dO . O) K_k; the row's log-sum-exp (log2 domain) and dO . O for the dkv kernel
+    const float l_tot = rows_sum(l_lane);
+    if (live) {
+      const float f = l_tot > 0.0f ? p.scale / l_tot : 0.0f;
+      float* dst = p.grad_q + row_elem + 4 * lk;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        *reinterpret_cast<float4_t*>(dst + 16 * nb) = float4_t{acc[nb][0] * f, acc[nb][1] * f, acc[nb][2] * f, acc[nb][3] * f};
+      }
+      if (lk == 0) {
+        float* st = p.row_stats + (row * p.q_heads + h) * 2;
+        // a row without visible keys gets a reference no score reaches: its probabilities come out as zeros
+        st[0] = l_tot > 0.0f ? m_run + __builtin_log2f(l_tot) : __builtin_huge_valf();
+        st[1] = delta;
+      }
+    }
+  }
+}
+
+// ---- dK, dV -------------------------------------------------------------------------------------------------------------
+template <int KIND, int D>
+__global__ __launch_bounds__(kBmThreads) void bwd_mfma_dkv_kernel(BwdParams p) {
+  using Ops = MfmaOps<KIND>;
+  using V8 = typename Ops::vec8;
+  using T = BmTile<D>;
+  constexpr int NS = D / 32, NB = D / 16;
+  __shared__ __attribute__((aligned(16))) char s_q[kBmTile * T::RS];
+  __shared__ __attribute__((aligned(16))) char s_g[kBmTile * T::RS];
+  __shared__ float s_stat[kBmTile][2];  // log-sum-exp and dO . O of the tile's query rows
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int lr = lane & 15, lk = lane >> 4;
+  const int kvh = blockIdx.y;
+  const int group = p.q_heads / p.kv_heads;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * kBmRows;
+  const int64_t block_end = r0 + kBmRows < p.k_tokens ? r0 + kBmRows : p.k_tokens;
+  const int64_t row = r0 + 16 * wave + lr;  // this lane's key row (a column of the products)
+  const bool row_exists = row < p.k_tokens;
+
+  // this lane's parts of its row of K and V (B operands)
+  const int64_t row_elem = (row * p.kv_heads + kvh) * D;
+  V8 kop[NS], vop[NS];
+#pragma unroll
+  for (int sl = 0; sl < NS; ++sl) {
+    uint4_t kw = {0u, 0u, 0u, 0u}, vw = kw;
+    if (row_exists) {
+      const int64_t off = (row_elem + (D / 4) * lk + 8 * sl) * 2;
+      kw = load16(p.k, off);
+      vw = load16(p.v, off);
+    }
+    kop[sl] = __builtin_bit_cast(V8, kw);
+    vop[sl] = __builtin_bit_cast(V8, vw);
+  }
+  float4_t acc_k[NB], acc_v[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) acc_k[nb] = acc_v[nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+  for (int s = seq_of_row(p.cu_k, p.num_seqs, r0); s < p.num_seqs; ++s) {
+    const int64_t sk0 = p.cu_k[s], sk1 = p.cu_k[s + 1];
+    if (sk0 >= block_end) break;
+    const int64_t k_lo = sk0 > r0 ? sk0 : r0, k_hi = sk1 < block_end ? sk1 : block_end;
+    if (k_lo >= k_hi) continue;
+    const int ctx = p.ctx != nullptr ? p.ctx[s] : 0;
+    const int64_t q_base = p.cu_q[s];
+    const int n_q = p.cu_q[s + 1] - p.cu_q[s];
+    const bool live = row >= k_lo && row < k_hi;
+    const int key = live ? static_cast<int>(row - sk0) : -1;  // this lane's key position in the sequence
+    const bool wave_live = __builtin_amdgcn_ballot_w64(live) != 0;
+    // queries i (position ctx + i) that see one of the block's keys: key <= ctx + i <= key + window
+    const int key_min = static_cast<int>(k_lo - sk0), key_max = static_cast<int>(k_hi - 1 - sk0);
+    const int i_lo = key_min - ctx > 0 ? key_min - ctx : 0;
+    int i_hi = n_q - 1;
+    if (p.window_left >= 0 && key_max + p.window_left - ctx < i_hi) i_hi = key_max + p.window_left - ctx;
+    if (i_hi < i_lo) continue;  // (the same for the whole workgroup)
+    const int t0 = i_lo / kBmTile, t1 = i_hi / kBmTile;
+    const int steps = (t1 - t0 + 1) * group;  // tiles of every q head of the group, head by head
+
+    uint4_t qreg[T::kChunks], greg[T::kChunks];
+    float2_t stat_reg = {0.0f, 0.0f};
+    auto fetch = [&](int step) {
+      const int hq = kvh * group + step / (t1 - t0 + 1);
+      const int t = t0 + step % (t1 - t0 + 1);
+#pragma unroll
+      for (int i = 0; i < T::kChunks; ++i) {
+        const int c = tid + kBmThreads * i;
+        const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
+        const int qi = kBmTile * t + r < n_q ? kBmTile * t + r : n_q - 1;  // rows past the end repeat the last query
+        const int64_t off = ((q_base + qi) * p.q_heads + hq) * (D * 2) + col * 16;
+        qreg[i] = load16(p.q, off);
+        greg[i] = load16(p.grad_out, off);
+      }
+      if (tid < kBmTile) {
+        const int qi = kBmTile * t + tid < n_q ? kBmTile * t + tid : n_q - 1;
+        stat_reg = *reinterpret_cast<const float2_t*>(p.row_stats + ((q_base + qi) * p.q_heads + hq) * 2);
+      }
+    };
+    auto publish = [&]() {
+#pragma unroll
+      for (int i = 0; i < T::kChunks; ++i) {
+        const int c = tid + kBmThreads * i;
+        const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
+        *reinterpret_cast<uint4_t*>(s_q + r * T::RS + col * 16) = qreg[i];
+        *reinterpret_cast<uint4_t*>(s_g + r * T::RS + col * 16) = greg[i];
+      }
+      if (tid < kBmTile) {
+        s_stat[tid][0] = stat_reg[0];
+        s_stat[tid][1] = stat_reg[1];
+      }
+    };
+    fetch(0);
+    __syncthreads();  // the tiles' previous readers (an earlier sequence of this block) are done
+    publish();
+    __syncthreads();
+    for (int step = 0; step < steps; ++step) {
+      if (step + 1 < steps) fetch(step + 1);
+      if (wave_live) {
+        const int t = t0 + step % (t1 - t0 + 1);
+        float pr[2][4], ds[2][4];
+#pragma unroll
+        for (int tg = 0; tg < 2; ++tg) {
+          float4_t c1 = {0.0f, 0.0f, 0.0f, 0.0f}, c2 = c1;
+#pragma unroll
+          for (int sl = 0; sl < NS; ++sl) {
+            c1 = Ops::mfma(tile_row_operand<KIND, D>(s_q, tg, sl, lr, lk), kop[sl], c1);
+            c2 = Ops::mfma(tile_row_operand<KIND, D>(s_g, tg, sl, lr, lk), vop[sl], c2);
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int r = 16 * tg + 4 * lk + j;  // query row of the tile
+            const int qi = kBmTile * t + r;
+            const int pos = ctx + qi;
+            const bool ok = live && qi < n_q && key <= pos && (p.window_left < 0 || key >= pos - p.window_left);
+            const float pe = ok ? fast_exp2(c1[j] * p.scale_log2e - s_stat[r][0]) : 0.0f;
+            pr[tg][j] = pe;
+            ds[tg][j] = pe * (c2[j] - s_stat[r][1]);
+          }
+        }
+        const V8 pop = streamed_operand<KIND>(pr);
+        const V8 dsop = streamed_operand<KIND>(ds);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          acc_v[nb] = Ops::mfma(tile_transposed_operand<KIND, D>(s_g, nb, lr, lk), pop, acc_v[nb]);
+          acc_k[nb] = Ops::mfma(tile_transposed_operand<KIND, D>(s_q, nb, lr, lk), dsop, acc_k[nb]);
+        }
+      }
+      __syncthreads();  // every wave has read this step's tiles
+      if (step + 1 < steps) publish();
+      __syncthreads();
+    }
+  }
+
+  // every gradient element is written, also the zeros of keys no query sees
+  if (row_exists) {
+    float* dk = p.grad_k + row_elem + 4 * lk;
+    float* dv = p.grad_v + row_elem + 4 * lk;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      *reinterpret_cast<float4_t*>(dk + 16 * nb) =
+          float4_t{acc_k[nb][0] * p.scale, acc_k[nb][1] * p.scale, acc_k[nb][2] * p.scale, acc_k[nb][3] * p.scale};
+      *reinterpret_cast<float4_t*>(dv + 16 * nb) = acc_v[nb];
+    }
+  }
+}
+
+typedef void (*bm_fn)(BwdParams);
+
+}  // namespace
+
+int launch_attention_backward_mfma(const BwdParams& p, void* stream) {
+  if (p.dtype != ARENO_DT_BF16 && p.dtype != ARENO_DT_F16) return ARENO_ERR_UNSUPPORTED;
+  if (p.head_dim != 64 && p.head_dim != 128) return ARENO_ERR_UNSUPPORTED;
+  if (p.q_heads > 65535 || p.kv_heads > 65535) return ARENO_ERR_UNSUPPORTED;
+  const int64_t q_blocks = (p.q_tokens + kBmRows - 1) / kBmRows, k_blocks = (p.k_tokens + kBmRows - 1) / kBmRows;
+  if (q_blocks > 0x7fffffffLL || k_blocks > 0x7fffffffLL) return ARENO_ERR_UNSUPPORTED;
+  const bool bf16 = p.dtype == ARENO_DT_BF16;
+  bm_fn dq, dkv;
+  if (p.head_dim == 64) {
+    dq = bf16 ? bwd_mfma_dq_kernel<KV_BF16, 64> : bwd_mfma_dq_kernel<KV_F16, 64>;
+    dkv = bf16 ? bwd_mfma_dkv_kernel<KV_BF16, 64> : bwd_mfma_dkv_kernel<KV_F16, 64>;
+  } else {
+    dq = bf16 ? bwd_mfma_dq_kernel<KV_BF16, 128> : bwd_mfma_dq_kernel<KV_F16, 128>;
+    dkv = bf16 ? bwd_mfma_dkv_kernel<KV_BF16, 128> : bwd_mfma_dkv_kernel<KV_F16, 128>;
+  }
+  const char* op = "areno_hip_attention_backward";
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (q_blocks > 0) {
+    hipLaunchKernelGGL(dq, dim3(static_cast<unsigned>(q_blocks), p.q_heads), dim3(kBmThreads), 0, s, p);
+    if (int rc = check_launch(op)) return rc;
+  }
+  if (k_blocks > 0) {
+    hipLaunchKernelGGL(dkv, dim3(static_cast<unsigned>(k_blocks), p.kv_heads), dim3(kBmThreads), 0, s, p);
+    if (int rc = check_launch(op)) return rc;
+  }
+  return ARENO_OK;
+}
+
+}  // namespace areno

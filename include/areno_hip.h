@@ -407,7 +407,8 @@ int areno_hip_block_tables_prefill_slots(const areno_block_tables* tables, const
  *   cu_seqlens_q      device [num_seqs + 1] int32;  cu_seqlens_k  the same for the keys, NULL = cu_seqlens_q (varlen op)
  *   context_lens      device [num_seqs] int32 position of each sequence's first query, NULL = 0 (dense op: query_start)
  *   workspace         areno_hip_attention_backward_workspace_bytes(q_tokens, q_heads) bytes: per-row log-sum-exp and dO . O
- * head_dim a multiple of 8 up to 256.  Two launches; deterministic (no atomics).
+ * head_dim a multiple of 8 up to 256 (F16 / BF16 at 64 and 128: matrix-core kernels).  Two launches; deterministic
+ * (no atomics).
  */
 size_t areno_hip_attention_backward_workspace_bytes(int64_t q_tokens, int32_t q_heads);
 int areno_hip_attention_backward(const void* grad_out, const void* q, const void* k, const void* v, const void* out,

@@ -51,6 +51,28 @@ def test_varlen_backward(dtype, window_left, hq, hkv, d):
         _close(got, ref, REL[dtype], f"{name} {dtype} d={d} window={window_left}")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hkv,d,window_left", [(8, 2, 128, None), (4, 4, 64, None), (6, 1, 64, 40), (4, 2, 128, 200), (2, 1, 128, 0)])
+def test_varlen_backward_long_sequences_on_the_matrix_core_kernels(dtype, hq, hkv, d, window_left):
+    """16-bit inputs at head dims 64 / 128 take the matrix-core backward: sequences longer than its blocks of 64 rows
+    and tiles of 32, blocks that hold several sequences (and empty ones), query groups, windows shorter and longer
+    than a tile."""
+    g = torch.Generator().manual_seed(hq * 31 + d)
+    lens = [300, 1, 0, 700, 5, 63, 64, 65, 129]
+    t = sum(lens)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    q = torch.randn(t, hq, d, generator=g).to(dtype)
+    k = torch.randn(t, hkv, d, generator=g).to(dtype)
+    v = torch.randn(t, hkv, d, generator=g).to(dtype)
+    go = torch.randn(t, hq, d, generator=g).to(dtype)
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    ops.areno_varlen_causal_attention(qd, kd, vd, cu.to(DEV), window_left=window_left).backward(go.to(DEV))
+    qf, kf, vf = (x.float().requires_grad_(True) for x in (q, k, v))
+    ar.ref_varlen(qf, kf, vf, cu, ar.window_left_arg(window_left), d**-0.5).backward(go.float())
+    for got, ref, name in ((qd.grad, qf.grad, "dq"), (kd.grad, kf.grad, "dk"), (vd.grad, vf.grad, "dv")):
+        _close(got, ref, REL[dtype], f"{name} {dtype} {hq}/{hkv} d={d} window={window_left}")
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("query_start,window_left", [(0, None), (7, None), (3, 5)])
 def test_dense_backward(dtype, query_start, window_left):
