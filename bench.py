@@ -4,8 +4,9 @@ A step is one call of the decode op (split-KV GQA attention, then the merge laun
 for one layer over one batch of synthetic sequences.  The headline workload is the Qwen2.5-7B-like shape (B=64, 28 q heads /
 4 kv heads, D=128, page 16, contexts uniform in [512, 4096]) with an int8 KV cache (quantizing append included), the
 configuration the bandwidth target is stated on; the same shape with a bf16 cache, the fp8 rollout shape and the fp8
-prefill shape are measured too and reported under "workloads".  Inputs are resident in HBM before timing starts.  Steps rotate over several copies of the KV
-pools so that the working set exceeds the 256 MB Infinity Cache and the reads really come from HBM.
+prefill shape are measured too and reported under "workloads" (next to a few decode shapes beside the benchmark's and
+the backward of the varlen op).  Inputs are resident in HBM before timing starts.  Steps rotate over several copies
+of the KV pools so that the working set exceeds the 256 MB Infinity Cache and the reads really come from HBM.
 
 Prints ONE JSON line.  `value` is microseconds per step: the median of 15 timings of exactly `--steps` steps replayed
 from HIP graphs (how the engine runs decode), `value_p10_p90` their spread.  The steps run as an engine runs the
@@ -394,6 +395,42 @@ def measure_other_shapes(device, steps=56, repeats=7):
         del w, pools, keep, graph
         torch.cuda.empty_cache()
     return result
+
+
+def measure_backward(device, seqs=2, new=2048, hq=28, hkv=4, d=128, iters=10):
+    """us per call of the varlen op's backward (dQ, dK, dV through autograd, bf16, the matrix-core kernels) and its
+    rate counted as 2.5 x the forward's FLOPs, next to the forward on the same inputs; the training-side companion of
+    the path, reported for completeness."""
+    import torch
+
+    from areno_amd.accel import attention as ops
+
+    g = torch.Generator().manual_seed(7)
+    t = seqs * new
+    cu = torch.arange(0, t + 1, new, dtype=torch.int32, device=device)
+    q, k, v, go = (torch.randn(t, h, d, generator=g).bfloat16().to(device) for h in (hq, hkv, hkv, hq))
+    q, k, v = (x.requires_grad_(True) for x in (q, k, v))
+    out = ops.areno_varlen_causal_attention(q, k, v, cu)
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        first.record()
+        for _ in range(iters):
+            fn()
+        last.record()
+        torch.cuda.synchronize()
+        return first.elapsed_time(last) / iters * 1e3
+
+    us_backward = timed(lambda: torch.autograd.grad(out, (q, k, v), go, retain_graph=True))
+    with torch.no_grad():
+        us_forward = timed(lambda: ops.areno_varlen_causal_attention(q, k, v, cu))
+    flops = seqs * 4 * hq * d * new * (new + 1) / 2
+    return {"shape": f"{seqs} x {new} tokens, {hq}/{hkv} heads, D = {d}, bf16", "backward_us": us_backward,
+            "backward_tflops_as_2.5x_forward": 2.5 * flops / us_backward / 1e6, "forward_us": us_forward,
+            "forward_tflops": flops / us_forward / 1e6}  # fmt: skip
 
 
 def measure_stream_ceiling(w, pools, iters=10, samples=9):
@@ -816,6 +853,7 @@ def main() -> int:
 
     if not args.only and not args.skip_other_shapes:
         results["other_shapes"] = measure_other_shapes(dev)
+        results["varlen_backward"] = measure_backward(dev)
 
     head = results[names[0]]
     dtype = {"cfg1": "bf16", "cfg2": "int8", "cfg3": "fp8", "cfg4": "fp8", "cfg2_b256": "int8"}[names[0]]
