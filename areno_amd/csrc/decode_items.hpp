@@ -42,10 +42,11 @@ ARENO_HD int first_visible_key(int length, int window_left) {
 
 struct UnitGeometry {
   int total;  // cost positions of the launch
-  int units;
+  int units;  // units that own positions: the launch's units, or only as many as there are positions (see below)
   bool narrow;  // the products below fit 32 bits: 32-bit divisions are a fifth of the instructions of 64-bit ones
 
   ARENO_HD int unit_start(int u) const {
+    if (u >= units) return total;  // a unit behind the last one that owns positions
     if (narrow)
       return static_cast<int>(static_cast<uint32_t>(u) * static_cast<uint32_t>(total) / static_cast<uint32_t>(units));
     return static_cast<int>(static_cast<long long>(u) * total / units);
@@ -61,10 +62,14 @@ struct UnitGeometry {
   }
 };
 
+// A launch with fewer than two cost positions per unit (a tiny batch) uses only its first total / 2 units, two
+// positions each (a tile step reads two quanta of tokens anyway), and leaves the others without work: spread over
+// all units, a row's positions would lie in units far apart with empty ones in between, and the merge would go
+// through the whole range (256 candidates for a single row of any length).
 ARENO_HD UnitGeometry make_unit_geometry(int total, int units) {
   UnitGeometry g;
   g.total = total;
-  g.units = units;
+  g.units = total < 2 * units ? (total > 1 ? total / 2 : 1) : units;
   // largest product in unit_start / unit_of: (total + 1) * units + total
   g.narrow = (static_cast<long long>(total) + 2) * (static_cast<long long>(units) + 1) < (1LL << 31);
   return g;

@@ -172,18 +172,6 @@ struct MergeChunk {
   float v[N][EPW];
 };
 
-// Whether unit u of a launch with fewer cost positions than units (total < units: tiny batches) holds none:
-// floor(u total / units) == floor((u + 1) total / units), i.e. (u total mod units) + total < units.  The product is
-// below 2^20 (at most 1 024 units), so the quotient comes from a float multiplication and one correction either way
-// instead of a division.
-__device__ __forceinline__ bool unit_is_empty(int total, int units, float units_rcp, int u) {
-  const int a = u * total;
-  int r = a - static_cast<int>(static_cast<float>(a) * units_rcp) * units;
-  r += r < 0 ? units : 0;
-  r -= r >= units ? units : 0;
-  return r + total < units;
-}
-
 // The kernel keeps to few registers (48 at head dim 128): a variant that fetched 32 candidates per round trip for rows
 // with many of them took 160 and every launch of it twice as long, whether or not a row had that many.  Rows with many
 // candidates -- a small batch spreads each row over all units: 256 candidates at batch 1 -- are served by more waves
@@ -251,9 +239,6 @@ __global__ __launch_bounds__((MW == 1 ? kReduceRows : MW) * kWave) void decode_r
     }
   }
   auto widen = [](uint16_t raw) { return QDT == ARENO_DT_BF16 ? bf16_bits_to_float(raw) : f16_bits_to_float(raw); };
-  // (with fewer cost positions than units a candidate's unit may be empty and have written nothing)
-  const bool every_unit_has_quanta = cum_total >= mp.num_units;
-  const float units_rcp = 1.0f / static_cast<float>(mp.num_units);
   if constexpr (PLANNED) {
     own_lo = planned_units[0];
     own_n = planned_units[1];
@@ -291,15 +276,6 @@ __global__ __launch_bounds__((MW == 1 ? kReduceRows : MW) * kWave) void decode_r
   const float* const sh_acc = sh_n > 0 ? mp.shared_acc : p.part_acc;
   auto load_chunk = [&](int base, auto& ch) {
     constexpr int N = std::remove_reference_t<decltype(ch)>::kSize;
-    // units without a quantum among the chunk's candidates (launches with fewer cost positions than units only)
-    uint32_t empty_mask = 0;
-    if (!every_unit_has_quanta) {
-      for (int j = 0; j < N && base + j < total; ++j) {
-        const int c = base + j;
-        const int u = c < own_n ? own_lo + c : sh_lo + (c - own_n);
-        empty_mask |= unit_is_empty(cum_total, mp.num_units, units_rcp, u) ? (1u << j) : 0u;
-      }
-    }
     float2_t pair[N];
 #pragma unroll
     for (int j = 0; j < N; ++j) {
@@ -319,7 +295,7 @@ __global__ __launch_bounds__((MW == 1 ? kReduceRows : MW) * kWave) void decode_r
     }
 #pragma unroll
     for (int j = 0; j < N; ++j) {
-      const bool present = base + j < total && !((empty_mask >> j) & 1u);
+      const bool present = base + j < total;  // (every unit of a row's range holds quanta of the row)
       // a partial without keys contributes nothing (attention.cu:680-682 in the reference)
       ch.m[j] = (present && pair[j][1] != 0.0f) ? pair[j][0] : kNegInf;
       ch.l[j] = present ? pair[j][1] : 0.0f;

@@ -86,6 +86,7 @@ int walk(const ItemShape& shape, const CheckedLens& lens, int units, int tile_to
   for (int v = 0; v < num_items; ++v) seen[v].assign(items[v].end > items[v].lo ? items[v].end - items[v].lo : 0, 0);
   *partials = 0;
   *steps = 0;
+  std::vector<int> written(num_items, 0);  // partials every item got
   for (int unit = 0; unit < units; ++unit) {
     const int q0 = geo.unit_start(unit), q1 = geo.unit_start(unit + 1);
     if (q0 < 0 || q1 > total || q0 > q1) {
@@ -162,6 +163,7 @@ int walk(const ItemShape& shape, const CheckedLens& lens, int units, int tile_to
           return 1;
         }
         ++*partials;
+        ++written[b_before];
         // the merge kernel finds the partial through unit_of over the item's quanta
         int u_lo, u_hi;
         item_units(geo, shape.switch_quanta, cum[b_before], cum[b_before + 1], u_lo, u_hi);
@@ -184,6 +186,19 @@ int walk(const ItemShape& shape, const CheckedLens& lens, int units, int tile_to
         snprintf(fail->msg, sizeof(fail->msg), "token %zu of item %d was never read", items[v].lo + i, v);
         return 1;
       }
+    }
+  }
+  // the merge kernel reads one partial from every unit of an item's range: each of them must have written one
+  for (int v = 0; v < num_items; ++v) {
+    int expected = 0;
+    if (items[v].quanta() > 0) {
+      int u_lo, u_hi;
+      item_units(geo, shape.switch_quanta, cum[v], cum[v + 1], u_lo, u_hi);
+      expected = u_hi - u_lo + 1;
+    }
+    if (written[v] != expected) {
+      snprintf(fail->msg, sizeof(fail->msg), "item %d got %d partials, the merge reads %d", v, written[v], expected);
+      return 1;
     }
   }
   *quanta_seen = 0;

@@ -124,6 +124,16 @@ def test_rows_at_the_end_of_their_block_table(walker):
         walker([64, 32, 64], q_per_kv=4, units=64, block_size=16, max_blocks=4, append_in_merge=0)
 
 
+@pytest.mark.parametrize("lengths", [[800], [15], [4096], [40, 0, 7, 130], [1]])
+@pytest.mark.parametrize("switch_quanta", [1, 3])
+def test_launches_with_fewer_cost_positions_than_units(walker, lengths, switch_quanta):
+    """A tiny batch has fewer cost positions than the launch has units: the first units take one position each and the
+    others none, so a row's units are neighbours (the merge reads one partial per unit of the row's range)."""
+    quanta, partials, _ = walker(lengths, q_per_kv=7, units=256, switch_quanta=switch_quanta)
+    assert quanta == _expected_quanta(lengths, 1)
+    assert partials <= quanta  # at most one partial per unit that holds a quantum
+
+
 def test_batches_of_empty_rows(walker):
     assert walker([0, 0, 0], q_per_kv=4, units=1024)[0] == 0
     assert walker([0, 0, 5, 0], q_per_kv=4, units=1024)[0] == 1
