@@ -345,8 +345,9 @@ def measure_other_shapes(device, steps=56, repeats=7):
     """us/step (graph replay, a plan per LAYERS_PER_PLAN steps where the shape takes one) of decode shapes next to the
     benchmark's: cfg 2's rows with more than 16 query heads per KV head (several column tiles per KV head on the
     matrix-core kernel) and on pages whose size is no power of two (a multiply-shift division in the kernel's page
-    arithmetic).  Two pool copies only,
-    so part of the int8 working set may sit in the Infinity Cache: these are orders of magnitude, not roofline figures."""
+    arithmetic), and a single sequence of 4 096 cached tokens (a launch with as many cost positions as units: the
+    latency of a decode step that has next to nothing to read).  Two pool copies only, so part of the working set may
+    sit in the Infinity Cache: these are orders of magnitude, not roofline figures."""
     import torch
 
     from areno_amd import workloads
@@ -356,15 +357,18 @@ def measure_other_shapes(device, steps=56, repeats=7):
         "mqa_32q_1kv_int8": dict(hq=32, hkv=1, bs=16, kv="int8"),
         "gqa_64q_2kv_bf16": dict(hq=64, hkv=2, bs=16, kv="bf16"),
         "cfg2_rows_page48_int8": dict(hq=28, hkv=4, bs=48, kv="int8"),
+        "one_sequence_4096_tokens_int8": dict(hq=28, hkv=4, bs=16, kv="int8", lengths=[4096]),
     }
     g = torch.Generator().manual_seed(2002)
-    lengths = torch.randint(512, 4097, (64,), generator=g)
+    cfg2_like_lengths = torch.randint(512, 4097, (64,), generator=g)
     result = {}
     for name, sh in shapes.items():
-        w = workloads.make_decode_workload(name, seed=7, batch=64, hq=sh["hq"], hkv=sh["hkv"], d=128, bs=sh["bs"], kv=sh["kv"],
-                                           lengths=lengths, device=device, quantize_fn=_gpu_quantize)  # fmt: skip
+        lengths = torch.tensor(sh["lengths"]) if "lengths" in sh else cfg2_like_lengths
+        batch = int(lengths.numel())
+        w = workloads.make_decode_workload(name, seed=7, batch=batch, hq=sh["hq"], hkv=sh["hkv"], d=128, bs=sh["bs"],
+                                           kv=sh["kv"], lengths=lengths, device=device, quantize_fn=_gpu_quantize)  # fmt: skip
         pools = _clone_pools(w, 2)
-        plan_buffer = torch.empty(max(16, cabi.decode_plan_bytes(64)), dtype=torch.uint8, device=device)
+        plan_buffer = torch.empty(max(16, cabi.decode_plan_bytes(batch)), dtype=torch.uint8, device=device)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
