@@ -1,10 +1,10 @@
 // Causal varlen prefill over paged (optionally quantized) KV on the matrix cores (gfx950).
 //
 // Work item = (sequence, kv head, block of query tokens).  The G query heads of the kv head are folded into the
-// query-row axis: row r of the block is (token r / GP, head r % GP) with GP = G rounded up to a power of two, so one
-// 16-row MFMA tile holds 16 / GP tokens of all heads and K/V are read once for the whole group (GQA without
-// expanding KV, as areno/accel/csrc/attention.cu:170-171 does per row; a kv head with more than 16 q heads runs as
-// several workgroup rows, 16 q heads each).  A block is 256 rows: each of the 8 waves
+// query-row axis: row r of the block is (token r / G, head r % G), so a block of 256 rows holds 256 / G tokens of
+// all heads (36 of them for 7 heads: 4 rows stay empty, where padding G to 8 left 32) and K/V are read once for the
+// whole group (GQA without expanding KV, as areno/accel/csrc/attention.cu:170-171 does per row; a kv head with more
+// than 16 q heads runs as several workgroup rows, 16 q heads each).  A block is 256 rows: each of the 8 waves
 // owns 32 (two 16-row tiles; one at head dims 192 and 256, and at 512 two waves share one).  One such workgroup per
 // CU (the registers allow two waves per SIMD either way; eight waves behind one set of K/V tiles halve the staging
 // work per wave against two workgroups of four).
@@ -100,8 +100,12 @@ struct PrefillParams {
   int32_t head_dim;
   int32_t group;        // q heads per kv head
   int32_t head_parts;   // workgroup rows (blockIdx.y) per kv head: ceil(group / 16); each takes up to 16 of its q heads
-  int32_t group_pad;    // q heads of one part rounded up to a power of two (<= 16)
-  int32_t group_shift;  // log2(group_pad)
+  // Row folding: row r of a query block is (token r / fold, q head r % fold of the part), fold = the q heads per kv
+  // head (16 when a kv head runs as several parts).  The quotient comes from a multiplication: r < 512, fold <= 16.
+  int32_t fold;
+  int32_t fold_magic;    // ceil(2^16 / fold): r / fold == (r * fold_magic) >> 16 for r < 2^12
+  int32_t block_tokens;  // rows_per_wg / fold: query tokens per item (the last rows of a block stay empty when fold
+                         // does not divide rows_per_wg)
   int32_t block_size;
   int32_t bs_shift;   // log2 of the page size, or -1: then a key's column is __umulhi(key, bs_magic) >> bs_post
   uint32_t bs_magic;
@@ -273,7 +277,7 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
   const int group_here = min(16, (kvh + 1) * p.group - head0);           // q heads of this part
   const int vheads = p.kv_heads * p.head_parts;
   const int unit = blockIdx.x;
-  const int tq = kRowsPerWg >> p.group_shift;  // query tokens per item
+  const int tq = p.block_tokens;  // query tokens per item
 
   prefix_tile_steps(p, tq, s_cum, s_wave_tot);
   const int total = s_cum[p.num_seqs];
@@ -517,8 +521,8 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
     q.tile = block_tiles(q.n_new, q.ctx, q.j, tq, p.window_left).tile_lo;
     return true;
   };
-  // ---- this lane's query rows: row R = wave * 16 RT + 16 * nq + lr -> token tok0 + (R >> group_shift), head
-  // R & (group_pad - 1) ----------------------------------------------------------------------------------------------
+  // ---- this lane's query rows: row R = wave * 16 RT + 16 * nq + lr -> token tok0 + R / fold, head R % fold ---------
+  auto token_of_row = [&](int r) { return (r * p.fold_magic) >> 16; };
   int q_pos[kRowTiles];         // absolute position of the row's query, or -1 for a padding row
   int64_t row_elem[kRowTiles];  // element offset of the row in q / out
   V8 qop[kRowTiles][NS];
@@ -526,8 +530,8 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
 #pragma unroll
     for (int nq = 0; nq < kRowTiles; ++nq) {
       const int r = row_wave * kRowsPerWave + 16 * nq + lr;
-      const int t = r >> p.group_shift;
-      const int hh = r & (p.group_pad - 1);
+      const int t = token_of_row(r);
+      const int hh = r - t * p.fold;
       const bool live = t < g.tok_cnt && hh < group_here;
       q_pos[nq] = live ? g.ctx + g.tok0 + t : -1;
       row_elem[nq] = (static_cast<int64_t>(g.q_begin + g.tok0 + t) * p.q_heads + head0 + hh) * D;
@@ -555,9 +559,9 @@ __global__ __launch_bounds__(kPrefillThreads, RT <= 2 ? 8 / kPrefillWaves : 1) v
     const int ctx = seg.ctx, tok0 = seg.tok0, tok_cnt = seg.tok_cnt;
 
     // rows of this wave: which query positions they span (wave-uniform), for skipping the mask on interior tiles
-    const bool wave_live = row_wave * kRowsPerWave < (tok_cnt << p.group_shift);
-    const int wave_qmin = ctx + tok0 + ((row_wave * kRowsPerWave) >> p.group_shift);
-    const int wave_qmax = ctx + tok0 + min(tok_cnt - 1, ((row_wave + 1) * kRowsPerWave - 1) >> p.group_shift);
+    const bool wave_live = row_wave * kRowsPerWave < tok_cnt * p.fold;
+    const int wave_qmin = ctx + tok0 + token_of_row(row_wave * kRowsPerWave);
+    const int wave_qmax = ctx + tok0 + min(tok_cnt - 1, token_of_row((row_wave + 1) * kRowsPerWave - 1));
 
     float4_t acc[kRowTiles][NB];
     // Row sums of the probabilities come from the matrix cores as well: one more product per key tile with an
@@ -868,7 +872,7 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
   const int group_here = min(16, (kvh + 1) * p.group - head0);
   const int vheads = p.kv_heads * p.head_parts;
   const int kRowsPerWg = p.rows_per_wg;
-  const int tq = kRowsPerWg >> p.group_shift;
+  const int tq = p.block_tokens;
   const int d = p.head_dim;
   prefix_tile_steps(p, tq, s_cum, s_wave_tot);
   const int total = s_cum[p.num_seqs];
@@ -911,8 +915,8 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
       // idx / chunks_per_row: the product with the rounded reciprocal is exact here (idx + 0.5 is at least half a
       // chunk away from a multiple of chunks_per_row, and idx < 2^16)
       row[k] = static_cast<int>((static_cast<float>(idx) + 0.5f) * inv_chunks_per_row);
-      const int t = row[k] >> p.group_shift;
-      const int hh = row[k] & (p.group_pad - 1);
+      const int t = (row[k] * p.fold_magic) >> 16;
+      const int hh = row[k] - t * p.fold;
       live[k] = base + k * kPrefillThreads < total_chunks && t < item.cnt && hh < group_here;
       m[k] = kNegInf;
       lsum[k] = 0.0f;
@@ -962,8 +966,8 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_merge_kernel(PrefillP
     for (int k = 0; k < kInFlight; ++k) {
       if (!live[k]) continue;
       const int idx = base + k * kPrefillThreads;
-      const int t = row[k] >> p.group_shift;
-      const int hh = row[k] & (p.group_pad - 1);
+      const int t = (row[k] * p.fold_magic) >> 16;
+      const int hh = row[k] - t * p.fold;
       const float inv = 1.0f / lsum[k];
       const int64_t out_elem = (static_cast<int64_t>(q_begin + item.tok0 + t) * p.q_heads + head0 + hh) * d +
                                4 * (idx - row[k] * chunks_per_row);
@@ -1106,10 +1110,10 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   // tile steps are counted in 32-bit: (tokens / query block + seqs) * (longest visible range / 32) must fit; the
   // paged case is bounded by the table width
   const int64_t max_keys = block_table != nullptr ? static_cast<int64_t>(max_blocks) * cache->block_size : tokens;
+  const int fold = head_parts > 1 ? 16 : group;  // rows of a token in a query block
+  const int block_tokens = rows_per_wg / fold;
   {
-    int gp = 1;
-    while (gp < (head_parts > 1 ? 16 : group)) gp <<= 1;
-    const int64_t items = tokens / (rows_per_wg / gp) + num_seqs;
+    const int64_t items = tokens / block_tokens + num_seqs;
     if (items * (max_keys / kTileTokens + 1) > 0x7fffffffLL) return ARENO_ERR_UNSUPPORTED;
   }
   // (the partials of a launch laid out over (kv head, part) pairs never need more than the kv heads alone would,
@@ -1136,9 +1140,9 @@ int launch_prefill_mfma(const areno_paged_cache* cache, const void* q, void* out
   p.head_dim = cache->head_dim;
   p.group = group;
   p.head_parts = head_parts;
-  p.group_pad = 1;
-  while (p.group_pad < (head_parts > 1 ? 16 : group)) p.group_pad <<= 1;
-  p.group_shift = log2_exact_i(p.group_pad);
+  p.fold = fold;
+  p.fold_magic = (65536 + fold - 1) / fold;
+  p.block_tokens = block_tokens;
   p.block_size = cache->block_size;
   p.bs_shift = log2_exact_i(cache->block_size);
   p.bs_magic = division.magic;

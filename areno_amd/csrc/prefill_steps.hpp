@@ -1,5 +1,5 @@
-// Tile steps of the prefill kernel's work list: a sequence's new tokens are cut into query blocks of tq tokens (a
-// power of two, at least 4), block j may see the key tiles [tile_lo, tile_hi] of kTileTokens keys, and the blocks'
+// Tile steps of the prefill kernel's work list: a sequence's new tokens are cut into query blocks of tq tokens
+// (at least 4; a power of two unless the q heads of a kv head are not), block j may see the key tiles [tile_lo, tile_hi] of kTileTokens keys, and the blocks'
 // tile steps lie one behind the other on the line the launch shares out in equal ranges.  Plain C++ shared by the
 // prefill kernel, its merge kernel and a CPU test that holds the closed forms below against a walk over the blocks.
 //
@@ -33,11 +33,13 @@ ARENO_HD BlockTiles block_tiles(int n_new, int ctx, int j, int tq, int window_le
   return b;
 }
 
-ARENO_HD int query_blocks(int n_new, int tq) { return (n_new + tq - 1) >> __builtin_ctz(static_cast<unsigned>(tq)); }
+// Division of a non-negative value by the block size: a shift for the usual power of two.
+ARENO_HD bool is_power_of_two(int x) { return (x & (x - 1)) == 0; }
+ARENO_HD int div_block(int x, int tq) {
+  return is_power_of_two(tq) ? x >> __builtin_ctz(static_cast<unsigned>(tq)) : x / tq;
+}
+ARENO_HD int query_blocks(int n_new, int tq) { return div_block(n_new + tq - 1, tq); }
 
-// Block sizes and the blocks per tile are powers of two, so every division below is a shift (a 64-bit division by a
-// run-time value costs a GPU thread some hundred instructions, and the bisection below evaluates several per step).
-ARENO_HD int log2_of_power_of_two(int x) { return __builtin_ctz(static_cast<unsigned>(x)); }
 constexpr int kTileShift = 5;
 static_assert((1 << kTileShift) == kTileTokens, "tile size");
 
@@ -47,15 +49,38 @@ ARENO_HD long long floor_ramp(long long n, int r_shift) {
   return ((q * (q - 1) / 2) << r_shift) + q * (n - (q << r_shift));
 }
 
-// sum over j in [0, n) of floor((a + j * tq) / kTileTokens) for a >= 0 and tq = 2^tq_shift: tq is either a multiple
-// of the tile (every block adds tq / kTileTokens whole tiles) or divides it (r = kTileTokens / tq blocks per tile:
-// floor((a + j * tq) / kTileTokens) = floor((floor(a / tq) + j) / r))
-ARENO_HD long long tile_index_sum(long long a, int tq_shift, long long n) {
+// sum over j in [0, n) of floor((a + j * tq) / kTileTokens) for a >= 0.
+// A power of two is either a multiple of the tile (every block adds tq / kTileTokens whole tiles) or divides it
+// (r = kTileTokens / tq blocks per tile: floor((a + j * tq) / kTileTokens) = floor((floor(a / tq) + j) / r)).
+// Any other block size (a group of q heads that is no power of two folds 256 / group tokens into a block): with
+// a = 32 A + a0 and tq = 32 W + r the term is A + j W + floor((a0 + j r) / 32), and the last part repeats, up to a
+// constant, with period P = 32 / gcd(r, 32) in j: term(j + P) = term(j) + P r / 32.  One period is summed in a loop of
+// at most 32 steps; no division by a run-time value anywhere (a 64-bit one costs a GPU thread some hundred
+// instructions, and the bisection below evaluates several sums per step).
+ARENO_HD long long tile_index_sum(long long a, int tq, long long n) {
   if (n <= 0) return 0;
-  if (tq_shift >= kTileShift) return n * (a >> kTileShift) + ((n * (n - 1) / 2) << (tq_shift - kTileShift));
-  const int r_shift = kTileShift - tq_shift;
-  const long long c = a >> tq_shift;
-  return floor_ramp(c + n, r_shift) - floor_ramp(c, r_shift);
+  if (is_power_of_two(tq)) {
+    const int tq_shift = __builtin_ctz(static_cast<unsigned>(tq));
+    if (tq_shift >= kTileShift) return n * (a >> kTileShift) + ((n * (n - 1) / 2) << (tq_shift - kTileShift));
+    const int r_shift = kTileShift - tq_shift;
+    const long long c = a >> tq_shift;
+    return floor_ramp(c + n, r_shift) - floor_ramp(c, r_shift);
+  }
+  const int r = tq & (kTileTokens - 1), a0 = static_cast<int>(a & (kTileTokens - 1));
+  long long sum = n * (a >> kTileShift) + (tq >> kTileShift) * (n * (n - 1) / 2);
+  if (r == 0) return sum;
+  const int g_shift = __builtin_ctz(static_cast<unsigned>(r));  // gcd(r, 32) = 2^g_shift, the lowest set bit of r
+  const int p_shift = kTileShift - g_shift;                     // period P = 2^p_shift
+  const int inc = r >> g_shift;                                 // P r / 32
+  const long long q = n >> p_shift;
+  const int rest = static_cast<int>(n - (q << p_shift));
+  int period_sum = 0, rest_sum = 0;
+  for (int j = 0; j < (1 << p_shift); ++j) {
+    const int term = (a0 + j * r) >> kTileShift;
+    period_sum += term;
+    if (j < rest) rest_sum += term;
+  }
+  return sum + q * period_sum + ((inc * (q * (q - 1) / 2)) << p_shift) + rest_sum + rest * q * inc;
 }
 
 // Tile steps of blocks [0, j) of a sequence, 0 <= j <= query_blocks(n_new, tq): the sum of block_tiles(...).count().
@@ -64,14 +89,15 @@ ARENO_HD long long tile_index_sum(long long a, int tq_shift, long long n) {
 // ctx + i * tq - window_left lies beyond key 0.
 ARENO_HD int steps_before_block(int n_new, int ctx, int j, int tq, int window_left) {
   if (j <= 0) return 0;
-  const int tq_shift = log2_of_power_of_two(tq);
-  const int blocks = (n_new + tq - 1) >> tq_shift;
+  const int blocks = query_blocks(n_new, tq);
   const int full = j < blocks ? j : blocks - 1;
-  long long sum = tile_index_sum(static_cast<long long>(ctx) + tq - 1, tq_shift, full);
+  long long sum = tile_index_sum(static_cast<long long>(ctx) + tq - 1, tq, full);
   if (j >= blocks) sum += (static_cast<long long>(ctx) + n_new - 1) >> kTileShift;
   if (window_left >= 0) {
-    const long long j0 = ctx > window_left ? 0 : ((static_cast<long long>(window_left) - ctx) >> tq_shift) + 1;
-    if (j0 < j) sum -= tile_index_sum(static_cast<long long>(ctx) - window_left + (j0 << tq_shift), tq_shift, j - j0);
+    const int j0 = ctx > window_left ? 0 : div_block(window_left - ctx, tq) + 1;
+    if (j0 < j) {
+      sum -= tile_index_sum(static_cast<long long>(ctx) - window_left + static_cast<long long>(j0) * tq, tq, j - j0);
+    }
   }
   return static_cast<int>(sum + j);
 }
