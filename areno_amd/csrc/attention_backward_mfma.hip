@@ -98,7 +98,7 @@ __device__ __forceinline__ float operand_element(uint32_t word, int hi) {
 
 // ---- dQ (and the rows' statistics) ------------------------------------------------------------------------------------
 template <int KIND, int D>
-__global__ __launch_bounds__(kBmThreads) void bwd_mfma_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p) {
   using Ops = MfmaOps<KIND>;
   using V8 = typename Ops::vec8;
   using T = BmTile<D>;
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(kBmThreads) void bwd_mfma_dq_kernel(BwdParams p) {
 
 // ---- dK, dV -------------------------------------------------------------------------------------------------------------
 template <int KIND, int D>
-__global__ __launch_bounds__(kBmThreads) void bwd_mfma_dkv_kernel(BwdParams p) {
+__global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p) {
   using Ops = MfmaOps<KIND>;
   using V8 = typename Ops::vec8;
   using T = BmTile<D>;
