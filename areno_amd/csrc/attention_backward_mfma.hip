@@ -270,7 +270,7 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
   constexpr int NS = D / 32, NB = D / 16;
   __shared__ __attribute__((aligned(16))) char s_q[kBmTile * T::RS];
   __shared__ __attribute__((aligned(16))) char s_g[kBmTile * T::RS];
-  __shared__ float s_stat[kBmTile][2];  // log-sum-exp and dO . O of the tile's query rows
+  __shared__ __attribute__((aligned(16))) float s_stat[kBmTile][2];  // log-sum-exp and dO . O of the tile's query rows
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -323,9 +323,13 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
 
     uint4_t qreg[T::kChunks], greg[T::kChunks];
     float2_t stat_reg = {0.0f, 0.0f};
-    auto fetch = [&](int step) {
-      const int hq = kvh * group + step / (t1 - t0 + 1);
-      const int t = t0 + step % (t1 - t0 + 1);
+    int fetch_head = kvh * group, fetch_tile = t0;  // the step the next fetch is for
+    auto fetch = [&]() {
+      const int hq = fetch_head, t = fetch_tile;
+      if (++fetch_tile > t1) {
+        fetch_tile = t0;
+        ++fetch_head;
+      }
 #pragma unroll
       for (int i = 0; i < T::kChunks; ++i) {
         const int c = tid + kBmThreads * i;
@@ -353,17 +357,23 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
         s_stat[tid][1] = stat_reg[1];
       }
     };
-    fetch(0);
+    fetch();
     __syncthreads();  // the tiles' previous readers (an earlier sequence of this block) are done
     publish();
     __syncthreads();
+    int t = t0 - 1;  // the query tile of the step
     for (int step = 0; step < steps; ++step) {
-      if (step + 1 < steps) fetch(step + 1);
+      if (step + 1 < steps) fetch();
+      t = t < t1 ? t + 1 : t0;
       if (wave_live) {
-        const int t = t0 + step % (t1 - t0 + 1);
         float pr[2][4], ds[2][4];
 #pragma unroll
         for (int tg = 0; tg < 2; ++tg) {
+          // the statistics of the four query rows this lane gets from the products: rows 16 tg + 4 lk .. + 3
+          const float4_t st01 = *reinterpret_cast<const float4_t*>(&s_stat[16 * tg + 4 * lk][0]);
+          const float4_t st23 = *reinterpret_cast<const float4_t*>(&s_stat[16 * tg + 4 * lk + 2][0]);
+          const float lse[4] = {st01[0], st01[2], st23[0], st23[2]};
+          const float dlt[4] = {st01[1], st01[3], st23[1], st23[3]};
           float4_t c1 = {0.0f, 0.0f, 0.0f, 0.0f}, c2 = c1;
 #pragma unroll
           for (int sl = 0; sl < NS; ++sl) {
@@ -372,13 +382,13 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
           }
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const int r = 16 * tg + 4 * lk + j;  // query row of the tile
-            const int qi = kBmTile * t + r;
+            const int qi = kBmTile * t + 16 * tg + 4 * lk + j;  // query of the sequence
             const int pos = ctx + qi;
             const bool ok = live && qi < n_q && key <= pos && (p.window_left < 0 || key >= pos - p.window_left);
-            const float pe = ok ? fast_exp2(c1[j] * p.scale_log2e - s_stat[r][0]) : 0.0f;
+            // (a query without visible keys has +inf as its log-sum-exp: exp2(-inf) = 0 either way)
+            const float pe = fast_exp2(ok ? c1[j] * p.scale_log2e - lse[j] : kBmNegInf);
             pr[tg][j] = pe;
-            ds[tg][j] = pe * (c2[j] - s_stat[r][1]);
+            ds[tg][j] = pe * (c2[j] - dlt[j]);
           }
         }
         const V8 pop = streamed_operand<KIND>(pr);
