@@ -23,6 +23,8 @@
 // packed rows may hold rows of several sequences; it goes through them one after the other, the rows of the others
 // masked.
 
+#include <type_traits>
+
 #include "attention_backward.hpp"
 #include "decode_mfma_kernels.hpp"
 
@@ -268,9 +270,9 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
   using V8 = typename Ops::vec8;
   using T = BmTile<D>;
   constexpr int NS = D / 32, NB = D / 16;
-  __shared__ __attribute__((aligned(16))) char s_q[kBmTile * T::RS];
-  __shared__ __attribute__((aligned(16))) char s_g[kBmTile * T::RS];
-  __shared__ __attribute__((aligned(16))) float s_stat[kBmTile][2];  // log-sum-exp and dO . O of the tile's query rows
+  __shared__ __attribute__((aligned(16))) char s_q[2][kBmTile * T::RS];  // (two buffers each: one in use, one filling)
+  __shared__ __attribute__((aligned(16))) char s_g[2][kBmTile * T::RS];
+  __shared__ __attribute__((aligned(16))) float s_stat[2][kBmTile][2];  // log-sum-exp and dO . O of the tile's query rows
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -311,7 +313,10 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
     const int n_q = p.cu_q[s + 1] - p.cu_q[s];
     const bool live = row >= k_lo && row < k_hi;
     const int key = live ? static_cast<int>(row - sk0) : -1;  // this lane's key position in the sequence
-    const bool wave_live = __builtin_amdgcn_ballot_w64(live) != 0;
+    const uint64_t live_lanes = __builtin_amdgcn_ballot_w64(live);
+    const bool wave_live = live_lanes != 0, wave_full = live_lanes == ~0ull;
+    // (the wave's 16 key rows, when all of them belong to this sequence)
+    const int wave_key_lo = static_cast<int>(r0 + 16 * wave - sk0), wave_key_hi = wave_key_lo + 15;
     // queries i (position ctx + i) that see one of the block's keys: key <= ctx + i <= key + window
     const int key_min = static_cast<int>(k_lo - sk0), key_max = static_cast<int>(k_hi - 1 - sk0);
     const int i_lo = key_min - ctx > 0 ? key_min - ctx : 0;
@@ -321,10 +326,17 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
     const int t0 = i_lo / kBmTile, t1 = i_hi / kBmTile;
     const int steps = (t1 - t0 + 1) * group;  // tiles of every q head of the group, head by head
 
-    uint4_t qreg[T::kChunks], greg[T::kChunks];
-    float2_t stat_reg = {0.0f, 0.0f};
-    int fetch_head = kvh * group, fetch_tile = t0;  // the step the next fetch is for
-    auto fetch = [&]() {
+    // Two register sets hold the tiles of the next two steps while they are in flight; a step computes on one of the
+    // two LDS buffers, moves the next step's tile into the other one and asks for the tile two steps further on.
+    struct Staged {
+      uint4_t q[T::kChunks], g[T::kChunks];
+      float2_t stat;
+    };
+    Staged set_a, set_b;
+    int fetch_head = kvh * group, fetch_tile = t0, fetched = 0;  // the step the next fetch is for
+    auto fetch = [&](Staged& st) {
+      if (fetched >= steps) return;
+      ++fetched;
       const int hq = fetch_head, t = fetch_tile;
       if (++fetch_tile > t1) {
         fetch_tile = t0;
@@ -336,72 +348,94 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
         const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
         const int qi = kBmTile * t + r < n_q ? kBmTile * t + r : n_q - 1;  // rows past the end repeat the last query
         const int64_t off = ((q_base + qi) * p.q_heads + hq) * (D * 2) + col * 16;
-        qreg[i] = load16(p.q, off);
-        greg[i] = load16(p.grad_out, off);
+        st.q[i] = load16(p.q, off);
+        st.g[i] = load16(p.grad_out, off);
       }
       if (tid < kBmTile) {
         const int qi = kBmTile * t + tid < n_q ? kBmTile * t + tid : n_q - 1;
-        stat_reg = *reinterpret_cast<const float2_t*>(p.row_stats + ((q_base + qi) * p.q_heads + hq) * 2);
+        st.stat = *reinterpret_cast<const float2_t*>(p.row_stats + ((q_base + qi) * p.q_heads + hq) * 2);
       }
     };
-    auto publish = [&]() {
+    auto publish = [&](const Staged& st, int buf) {
 #pragma unroll
       for (int i = 0; i < T::kChunks; ++i) {
         const int c = tid + kBmThreads * i;
         const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
-        *reinterpret_cast<uint4_t*>(s_q + r * T::RS + col * 16) = qreg[i];
-        *reinterpret_cast<uint4_t*>(s_g + r * T::RS + col * 16) = greg[i];
+        *reinterpret_cast<uint4_t*>(s_q[buf] + r * T::RS + col * 16) = st.q[i];
+        *reinterpret_cast<uint4_t*>(s_g[buf] + r * T::RS + col * 16) = st.g[i];
       }
-      if (tid < kBmTile) {
-        s_stat[tid][0] = stat_reg[0];
-        s_stat[tid][1] = stat_reg[1];
-      }
+      if (tid < kBmTile) *reinterpret_cast<float2_t*>(&s_stat[buf][tid][0]) = st.stat;
     };
-    fetch();
-    __syncthreads();  // the tiles' previous readers (an earlier sequence of this block) are done
-    publish();
-    __syncthreads();
     int t = t0 - 1;  // the query tile of the step
-    for (int step = 0; step < steps; ++step) {
-      if (step + 1 < steps) fetch();
+    // one step: the products of the tile in LDS buffer `buf`; between them the next step's tile goes from `next`
+    // into the other buffer and `next` is asked to fetch again
+    auto step_on = [&](int step, int buf, Staged& next) {
       t = t < t1 ? t + 1 : t0;
-      if (wave_live) {
-        float pr[2][4], ds[2][4];
+      float pr[2][4], ds[2][4];
+      auto first_products = [&](auto masked) {
 #pragma unroll
         for (int tg = 0; tg < 2; ++tg) {
           // the statistics of the four query rows this lane gets from the products: rows 16 tg + 4 lk .. + 3
-          const float4_t st01 = *reinterpret_cast<const float4_t*>(&s_stat[16 * tg + 4 * lk][0]);
-          const float4_t st23 = *reinterpret_cast<const float4_t*>(&s_stat[16 * tg + 4 * lk + 2][0]);
+          const float4_t st01 = *reinterpret_cast<const float4_t*>(&s_stat[buf][16 * tg + 4 * lk][0]);
+          const float4_t st23 = *reinterpret_cast<const float4_t*>(&s_stat[buf][16 * tg + 4 * lk + 2][0]);
           const float lse[4] = {st01[0], st01[2], st23[0], st23[2]};
           const float dlt[4] = {st01[1], st01[3], st23[1], st23[3]};
           float4_t c1 = {0.0f, 0.0f, 0.0f, 0.0f}, c2 = c1;
 #pragma unroll
           for (int sl = 0; sl < NS; ++sl) {
-            c1 = Ops::mfma(tile_row_operand<KIND, D>(s_q, tg, sl, lr, lk), kop[sl], c1);
-            c2 = Ops::mfma(tile_row_operand<KIND, D>(s_g, tg, sl, lr, lk), vop[sl], c2);
+            c1 = Ops::mfma(tile_row_operand<KIND, D>(s_q[buf], tg, sl, lr, lk), kop[sl], c1);
+            c2 = Ops::mfma(tile_row_operand<KIND, D>(s_g[buf], tg, sl, lr, lk), vop[sl], c2);
           }
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const int qi = kBmTile * t + 16 * tg + 4 * lk + j;  // query of the sequence
-            const int pos = ctx + qi;
-            const bool ok = live && qi < n_q && key <= pos && (p.window_left < 0 || key >= pos - p.window_left);
+            float x = c1[j] * p.scale_log2e - lse[j];
+            if constexpr (decltype(masked)::value) {
+              const int qi = kBmTile * t + 16 * tg + 4 * lk + j;  // query of the sequence
+              const int pos = ctx + qi;
+              const bool ok = live && qi < n_q && key <= pos && (p.window_left < 0 || key >= pos - p.window_left);
+              x = ok ? x : kBmNegInf;
+            }
             // (a query without visible keys has +inf as its log-sum-exp: exp2(-inf) = 0 either way)
-            const float pe = fast_exp2(ok ? c1[j] * p.scale_log2e - lse[j] : kBmNegInf);
+            const float pe = fast_exp2(x);
             pr[tg][j] = pe;
             ds[tg][j] = pe * (c2[j] - dlt[j]);
           }
         }
+      };
+      if (wave_live) {
+        // most tiles lie below the diagonal and inside the window as a whole: every query of the tile sees every key
+        // of this wave, and nothing needs a mask
+        const int pos_lo = ctx + kBmTile * t, pos_hi = pos_lo + kBmTile - 1;
+        const bool plain = wave_full && kBmTile * t + kBmTile <= n_q && pos_lo >= wave_key_hi &&
+                           (p.window_left < 0 || pos_hi - p.window_left <= wave_key_lo);
+        if (plain) {
+          first_products(std::false_type{});
+        } else {
+          first_products(std::true_type{});
+        }
+      }
+      if (step + 1 < steps) publish(next, buf ^ 1);
+      fetch(next);
+      if (wave_live) {
         const V8 pop = streamed_operand<KIND>(pr);
         const V8 dsop = streamed_operand<KIND>(ds);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-          acc_v[nb] = Ops::mfma(tile_transposed_operand<KIND, D>(s_g, nb, lr, lk), pop, acc_v[nb]);
-          acc_k[nb] = Ops::mfma(tile_transposed_operand<KIND, D>(s_q, nb, lr, lk), dsop, acc_k[nb]);
+          acc_v[nb] = Ops::mfma(tile_transposed_operand<KIND, D>(s_g[buf], nb, lr, lk), pop, acc_v[nb]);
+          acc_k[nb] = Ops::mfma(tile_transposed_operand<KIND, D>(s_q[buf], nb, lr, lk), dsop, acc_k[nb]);
         }
       }
-      __syncthreads();  // every wave has read this step's tiles
-      if (step + 1 < steps) publish();
-      __syncthreads();
+      __syncthreads();  // every wave has read this step's tile, the next one is in place
+    };
+    // (every wave has passed the barrier behind the last step of an earlier sequence of this block)
+    fetch(set_a);
+    fetch(set_b);
+    publish(set_a, 0);
+    fetch(set_a);
+    __syncthreads();
+    for (int step = 0; step < steps; step += 2) {
+      step_on(step, 0, set_b);
+      if (step + 1 < steps) step_on(step + 1, 1, set_a);
     }
   }
 
