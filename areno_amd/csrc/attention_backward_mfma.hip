@@ -128,7 +128,10 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
     const int n_k = p.cu_k[s + 1] - p.cu_k[s];
     const bool live = row >= q_lo && row < q_hi;
     const int pos = live ? ctx + static_cast<int>(row - sq0) : -1;
-    const bool wave_live = __builtin_amdgcn_ballot_w64(live) != 0;
+    const uint64_t live_lanes = __builtin_amdgcn_ballot_w64(live);
+    const bool wave_live = live_lanes != 0, wave_full = live_lanes == ~0ull;
+    // (the positions of the wave's 16 query rows, when all of them belong to this sequence)
+    const int wave_pos_lo = ctx + static_cast<int>(r0 + 16 * wave - sq0), wave_pos_hi = wave_pos_lo + 15;
     const int pos_min = ctx + static_cast<int>(q_lo - sq0), pos_max = ctx + static_cast<int>(q_hi - 1 - sq0);
     const int key_lo = p.window_left >= 0 ? (pos_min - p.window_left > 0 ? pos_min - p.window_left : 0) : 0;
     const int key_hi = pos_max < n_k - 1 ? pos_max : n_k - 1;
@@ -192,21 +195,36 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
         if (t < t1) fetch(t + 1);
         if (wave_live) {
           float sc[2][4], dp[2][4];
+          auto first_products = [&](auto masked) {
 #pragma unroll
-          for (int tg = 0; tg < 2; ++tg) {
-            float4_t c1 = {0.0f, 0.0f, 0.0f, 0.0f}, c2 = c1;
+            for (int tg = 0; tg < 2; ++tg) {
+              float4_t c1 = {0.0f, 0.0f, 0.0f, 0.0f}, c2 = c1;
 #pragma unroll
-            for (int sl = 0; sl < NS; ++sl) {
-              c1 = Ops::mfma(tile_row_operand<KIND, D>(s_k, tg, sl, lr, lk), qop[sl], c1);
-              c2 = Ops::mfma(tile_row_operand<KIND, D>(s_v, tg, sl, lr, lk), gop[sl], c2);
+              for (int sl = 0; sl < NS; ++sl) {
+                c1 = Ops::mfma(tile_row_operand<KIND, D>(s_k, tg, sl, lr, lk), qop[sl], c1);
+                c2 = Ops::mfma(tile_row_operand<KIND, D>(s_v, tg, sl, lr, lk), gop[sl], c2);
+              }
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                sc[tg][j] = c1[j] * p.scale_log2e;
+                if constexpr (decltype(masked)::value) {
+                  const int key = kBmTile * t + 16 * tg + 4 * lk + j;
+                  const bool ok = key <= pos && key < n_k && (p.window_left < 0 || key >= pos - p.window_left);
+                  sc[tg][j] = ok ? sc[tg][j] : kBmNegInf;
+                }
+                dp[tg][j] = c2[j];
+              }
             }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const int key = kBmTile * t + 16 * tg + 4 * lk + j;
-              const bool ok = key <= pos && key < n_k && (p.window_left < 0 || key >= pos - p.window_left);
-              sc[tg][j] = ok ? c1[j] * p.scale_log2e : kBmNegInf;
-              dp[tg][j] = c2[j];
-            }
+          };
+          // most tiles lie below the diagonal and inside the window as a whole: every query row of this wave sees
+          // every key of the tile, and nothing needs a mask
+          const int key_first = kBmTile * t, key_last = key_first + kBmTile - 1;
+          const bool plain = wave_full && key_last < n_k && key_last <= wave_pos_lo &&
+                             (p.window_left < 0 || key_first >= wave_pos_hi - p.window_left);
+          if (plain) {
+            first_products(std::false_type{});
+          } else {
+            first_products(std::true_type{});
           }
           float mt = sc[0][0];
 #pragma unroll
