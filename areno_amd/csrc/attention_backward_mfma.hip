@@ -114,7 +114,8 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
   const int lr = lane & 15, lk = lane >> 4;
   const int h = blockIdx.y;
   const int kvh = h / (p.q_heads / p.kv_heads);
-  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * kBmRows;
+  // (the last blocks first: in a long sequence they see the most keys, and the launch ends with the short ones)
+  const int64_t r0 = static_cast<int64_t>(gridDim.x - 1 - blockIdx.x) * kBmRows;
   const int64_t block_end = r0 + kBmRows < p.q_tokens ? r0 + kBmRows : p.q_tokens;
   const int64_t row = r0 + 16 * wave + lr;  // this lane's query row (a column of the products)
 
@@ -206,7 +207,7 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
               }
 #pragma unroll
               for (int j = 0; j < 4; ++j) {
-                sc[tg][j] = c1[j] * p.scale_log2e;
+                sc[tg][j] = c1[j];  // (the softmax scale goes in with the reference, below)
                 if constexpr (decltype(masked)::value) {
                   const int key = kBmTile * t + 16 * tg + 4 * lk + j;
                   const bool ok = key <= pos && key < n_k && (p.window_left < 0 || key >= pos - p.window_left);
@@ -233,7 +234,7 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
             for (int j = 0; j < 4; ++j) mt = fmaxf(mt, sc[tg][j]);
           }
           mt = rows_max(mt);
-          const float m_new = fmaxf(m_run, mt);
+          const float m_new = fmaxf(m_run, mt * p.scale_log2e);  // (the scale is positive)
           const float m_ref = m_new == kBmNegInf ? 0.0f : m_new;
           const float alpha = fast_exp2(m_run - m_ref);  // 0 while the row has seen no key
           m_run = m_new;
@@ -242,17 +243,22 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
           for (int tg = 0; tg < 2; ++tg) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-              const float pe = fast_exp2(sc[tg][j] - m_ref);  // exp2(-inf) = 0 for masked keys
+              const float pe = fast_exp2(__builtin_fmaf(sc[tg][j], p.scale_log2e, -m_ref));  // exp2(-inf) = 0: masked keys
               psum += pe;
               ds[tg][j] = pe * (dp[tg][j] - delta);
             }
           }
           l_lane = l_lane * alpha + psum;
           const V8 dsop = streamed_operand<KIND>(ds);
+          if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {  // (after the first tiles a new maximum is rare)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) acc[nb][j] *= alpha;
+            }
+          }
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[nb][j] *= alpha;
             acc[nb] = Ops::mfma(tile_transposed_operand<KIND, D>(s_k, nb, lr, lk), dsop, acc[nb]);
           }
         }
