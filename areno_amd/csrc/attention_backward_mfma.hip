@@ -54,6 +54,23 @@ __device__ __forceinline__ int seq_of_row(const int32_t* cu, int num_seqs, int64
   return lo;
 }
 
+// The block of 64 packed rows the i-th workgroup (of a head) takes.  Blocks differ in cost by their place in their
+// sequence (a query block late in a long sequence sees the most keys, a key block early in it is seen by the most
+// queries), and a launch ends soonest when the expensive blocks start first.  The lengths are not known on the host,
+// so the order assumes sequences of about equal length: the packed blocks are cut into num_seqs runs and taken run by
+// run in turn, the expensive end of every run first (`from_end`: the last block of a run).  Any order is correct.
+__device__ __forceinline__ int64_t block_in_cost_order(int64_t i, int64_t blocks, int num_seqs, bool from_end) {
+  const int64_t runs = num_seqs > 0 ? num_seqs : 1, per = blocks / runs, rest = blocks - per * runs;
+  if (per == 0) return from_end ? blocks - 1 - i : i;
+  if (from_end) {  // the blocks behind the last whole run belong to the end of the last sequence: first
+    if (i < rest) return blocks - 1 - i;
+    const int64_t j = i - rest;
+    return (j % runs) * per + (per - 1 - j / runs);
+  }
+  if (i >= per * runs) return i;
+  return (i % runs) * per + i / runs;
+}
+
 // A tile of 32 rows x D 16-bit elements in LDS, in one of two layouts.
 //   padded (SWZ = false)    row stride D * 2 + 16 bytes.  The row operands (16 lanes read the same 16-byte chunk of 16
 //                           rows) meet every bank once, the transposed ones (32 lanes read 32 bytes of 8 consecutive
@@ -134,10 +151,11 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
   const int lr = lane & 15, lk = lane >> 4;
-  const int h = blockIdx.y;
+  // workgroups in launch order: the heads of a block next to each other, the blocks by cost
+  const int h = static_cast<int>(blockIdx.x % static_cast<unsigned>(p.q_heads));
   const int kvh = h / (p.q_heads / p.kv_heads);
-  // (the last blocks first: in a long sequence they see the most keys, and the launch ends with the short ones)
-  const int64_t r0 = static_cast<int64_t>(gridDim.x - 1 - blockIdx.x) * kBmRows;
+  const int64_t q_blocks = (p.q_tokens + kBmRows - 1) / kBmRows;
+  const int64_t r0 = block_in_cost_order(blockIdx.x / static_cast<unsigned>(p.q_heads), q_blocks, p.num_seqs, true) * kBmRows;
   const int64_t block_end = r0 + kBmRows < p.q_tokens ? r0 + kBmRows : p.q_tokens;
   const int64_t row = r0 + 16 * wave + lr;  // this lane's query row (a column of the products)
 
@@ -310,23 +328,46 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
 }
 
 // ---- dK, dV -------------------------------------------------------------------------------------------------------------
-template <int KIND, int D, bool SWZ>
-__global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p) {
+// P = 1: four waves, one stream of tiles.  P = 2: eight waves in two parts of four; both parts own the same 64 key
+// rows and take every second step of the stream each (tiles and statistics of their own in LDS), and the second
+// part's sums go through LDS to the first at the end.  That halves the longest chain of steps of a launch too small
+// to give every compute unit two workgroups; the order of the sums stays fixed.
+template <int D, bool SWZ, int P>
+struct DkvLds {
+  using T = BmTile<D, SWZ>;
+  static constexpr int kTile = kBmTile * T::RS;
+  static constexpr int kStat = kBmTile * 2 * 4;
+  // per part and buffer: a Q tile, a dO tile, the rows' statistics
+  static constexpr int kBuffer = 2 * kTile + kStat;
+  static constexpr int kStream = P * 2 * kBuffer;
+  static constexpr int kSums = P > 1 ? kBmThreads * (D / 16) * 2 * 16 : 0;  // (P = 2: a float4 per lane, block and tensor)
+  static constexpr int kBytes = kStream > kSums ? kStream : kSums;
+};
+extern __shared__ __attribute__((aligned(16))) char bm_dkv_lds[];
+
+template <int KIND, int D, bool SWZ, int P>
+__global__ __launch_bounds__(kBmThreads* P, P == 1 ? 2 : 1) void bwd_mfma_dkv_kernel(BwdParams p) {
   using Ops = MfmaOps<KIND>;
   using V8 = typename Ops::vec8;
   using T = BmTile<D, SWZ>;
+  using L = DkvLds<D, SWZ, P>;
   constexpr int NS = D / 32, NB = D / 16;
-  __shared__ __attribute__((aligned(16))) char s_q[2][kBmTile * T::RS];  // (two buffers each: one in use, one filling)
-  __shared__ __attribute__((aligned(16))) char s_g[2][kBmTile * T::RS];
-  __shared__ __attribute__((aligned(16))) float s_stat[2][kBmTile][2];  // log-sum-exp and dO . O of the tile's query rows
 
-  const int tid = threadIdx.x;
+  const int part = P > 1 ? static_cast<int>(threadIdx.x) / kBmThreads : 0;  // (the same for a wave)
+  const int tid = P > 1 ? static_cast<int>(threadIdx.x) % kBmThreads : static_cast<int>(threadIdx.x);  // thread of the part
+  char* const lds = bm_dkv_lds + part * (2 * L::kBuffer);
+  auto s_q = [&](int buf) { return lds + buf * L::kBuffer; };
+  auto s_g = [&](int buf) { return lds + buf * L::kBuffer + L::kTile; };
+  auto s_stat = [&](int buf) { return reinterpret_cast<float*>(lds + buf * L::kBuffer + 2 * L::kTile); };  // [row][2]
+
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
   const int lr = lane & 15, lk = lane >> 4;
-  const int kvh = blockIdx.y;
+  // workgroups in launch order: the kv heads of a block next to each other, the blocks by cost
+  const int kvh = static_cast<int>(blockIdx.x % static_cast<unsigned>(p.kv_heads));
   const int group = p.q_heads / p.kv_heads;
-  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * kBmRows;
+  const int64_t k_blocks = (p.k_tokens + kBmRows - 1) / kBmRows;
+  const int64_t r0 = block_in_cost_order(blockIdx.x / static_cast<unsigned>(p.kv_heads), k_blocks, p.num_seqs, false) * kBmRows;
   const int64_t block_end = r0 + kBmRows < p.k_tokens ? r0 + kBmRows : p.k_tokens;
   const int64_t row = r0 + 16 * wave + lr;  // this lane's key row (a column of the products)
   const bool row_exists = row < p.k_tokens;
@@ -370,7 +411,27 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
     if (p.window_left >= 0 && key_max + p.window_left - ctx < i_hi) i_hi = key_max + p.window_left - ctx;
     if (i_hi < i_lo) continue;  // (the same for the whole workgroup)
     const int t0 = i_lo / kBmTile, t1 = i_hi / kBmTile;
-    const int steps = (t1 - t0 + 1) * group;  // tiles of every q head of the group, head by head
+    const int tiles = t1 - t0 + 1;
+    // the stream: tiles of every q head of the group, head by head; this part takes steps part, part + P, ...
+    const int stream_steps = tiles * group;
+    const int steps = (stream_steps - part + P - 1) / P;  // this part's
+    const int rounds = (stream_steps + P - 1) / P;        // the longest part's: every part keeps the barriers of all
+    // (head, tile) of a step of the stream, counted up by P steps at a time
+    struct Cursor {
+      int head, tile;
+    };
+    auto advance = [&](Cursor& c) {
+      c.tile += P;
+      while (c.tile > t1) {
+        c.tile -= tiles;
+        ++c.head;
+      }
+    };
+    Cursor first = {kvh * group, t0 + part};
+    while (first.tile > t1) {
+      first.tile -= tiles;
+      ++first.head;
+    }
 
     // Two register sets hold the tiles of the next two steps while they are in flight; a step computes on one of the
     // two LDS buffers, moves the next step's tile into the other one and asks for the tile two steps further on.
@@ -379,15 +440,13 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
       float2_t stat;
     };
     Staged set_a, set_b;
-    int fetch_head = kvh * group, fetch_tile = t0, fetched = 0;  // the step the next fetch is for
+    Cursor fetch_at = first;
+    int fetched = 0;
     auto fetch = [&](Staged& st) {
       if (fetched >= steps) return;
       ++fetched;
-      const int hq = fetch_head, t = fetch_tile;
-      if (++fetch_tile > t1) {
-        fetch_tile = t0;
-        ++fetch_head;
-      }
+      const int hq = fetch_at.head, t = fetch_at.tile;
+      advance(fetch_at);
 #pragma unroll
       for (int i = 0; i < T::kChunks; ++i) {
         const int c = tid + kBmThreads * i;
@@ -407,30 +466,32 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
       for (int i = 0; i < T::kChunks; ++i) {
         const int c = tid + kBmThreads * i;
         const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
-        *reinterpret_cast<uint4_t*>(s_q[buf] + T::chunk_pos(r, col)) = st.q[i];
-        *reinterpret_cast<uint4_t*>(s_g[buf] + T::chunk_pos(r, col)) = st.g[i];
+        *reinterpret_cast<uint4_t*>(s_q(buf) + T::chunk_pos(r, col)) = st.q[i];
+        *reinterpret_cast<uint4_t*>(s_g(buf) + T::chunk_pos(r, col)) = st.g[i];
       }
-      if (tid < kBmTile) *reinterpret_cast<float2_t*>(&s_stat[buf][tid][0]) = st.stat;
+      if (tid < kBmTile) *reinterpret_cast<float2_t*>(s_stat(buf) + 2 * tid) = st.stat;
     };
-    int t = t0 - 1;  // the query tile of the step
+    Cursor at = first;  // the step being computed
     // one step: the products of the tile in LDS buffer `buf`; between them the next step's tile goes from `next`
     // into the other buffer and `next` is asked to fetch again
     auto step_on = [&](int step, int buf, Staged& next) {
-      t = t < t1 ? t + 1 : t0;
+      const int t = at.tile;
+      advance(at);
+      const bool compute = wave_live && step < steps;
       float pr[2][4], ds[2][4];
       auto first_products = [&](auto masked) {
 #pragma unroll
         for (int tg = 0; tg < 2; ++tg) {
           // the statistics of the four query rows this lane gets from the products: rows 16 tg + 4 lk .. + 3
-          const float4_t st01 = *reinterpret_cast<const float4_t*>(&s_stat[buf][16 * tg + 4 * lk][0]);
-          const float4_t st23 = *reinterpret_cast<const float4_t*>(&s_stat[buf][16 * tg + 4 * lk + 2][0]);
+          const float4_t st01 = *reinterpret_cast<const float4_t*>(s_stat(buf) + 2 * (16 * tg + 4 * lk));
+          const float4_t st23 = *reinterpret_cast<const float4_t*>(s_stat(buf) + 2 * (16 * tg + 4 * lk + 2));
           const float lse[4] = {st01[0], st01[2], st23[0], st23[2]};
           const float dlt[4] = {st01[1], st01[3], st23[1], st23[3]};
           float4_t c1 = {0.0f, 0.0f, 0.0f, 0.0f}, c2 = c1;
 #pragma unroll
           for (int sl = 0; sl < NS; ++sl) {
-            c1 = Ops::mfma(tile_row_operand<KIND, T, D>(s_q[buf], tg, sl, lr, lk), kop[sl], c1);
-            c2 = Ops::mfma(tile_row_operand<KIND, T, D>(s_g[buf], tg, sl, lr, lk), vop[sl], c2);
+            c1 = Ops::mfma(tile_row_operand<KIND, T, D>(s_q(buf), tg, sl, lr, lk), kop[sl], c1);
+            c2 = Ops::mfma(tile_row_operand<KIND, T, D>(s_g(buf), tg, sl, lr, lk), vop[sl], c2);
           }
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
@@ -448,7 +509,7 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
           }
         }
       };
-      if (wave_live) {
+      if (compute) {
         // most tiles lie below the diagonal and inside the window as a whole: every query of the tile sees every key
         // of this wave, and nothing needs a mask
         const int pos_lo = ctx + kBmTile * t, pos_hi = pos_lo + kBmTile - 1;
@@ -462,13 +523,13 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
       }
       if (step + 1 < steps) publish(next, buf ^ 1);
       fetch(next);
-      if (wave_live) {
+      if (compute) {
         const V8 pop = streamed_operand<KIND>(pr);
         const V8 dsop = streamed_operand<KIND>(ds);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-          acc_v[nb] = Ops::mfma(tile_transposed_operand<KIND, T>(s_g[buf], nb, lr, lk), pop, acc_v[nb]);
-          acc_k[nb] = Ops::mfma(tile_transposed_operand<KIND, T>(s_q[buf], nb, lr, lk), dsop, acc_k[nb]);
+          acc_v[nb] = Ops::mfma(tile_transposed_operand<KIND, T>(s_g(buf), nb, lr, lk), pop, acc_v[nb]);
+          acc_k[nb] = Ops::mfma(tile_transposed_operand<KIND, T>(s_q(buf), nb, lr, lk), dsop, acc_k[nb]);
         }
       }
       __syncthreads();  // every wave has read this step's tile, the next one is in place
@@ -476,12 +537,36 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dkv_kernel(BwdParams p
     // (every wave has passed the barrier behind the last step of an earlier sequence of this block)
     fetch(set_a);
     fetch(set_b);
-    publish(set_a, 0);
+    if (steps > 0) publish(set_a, 0);
     fetch(set_a);
     __syncthreads();
-    for (int step = 0; step < steps; step += 2) {
+    for (int step = 0; step < rounds; step += 2) {
       step_on(step, 0, set_b);
-      if (step + 1 < steps) step_on(step + 1, 1, set_a);
+      if (step + 1 < rounds) step_on(step + 1, 1, set_a);
+    }
+  }
+
+  if constexpr (P > 1) {
+    // the second part's sums to the first: a float4 per lane, block and tensor, lanes next to each other
+    float4_t* sums = reinterpret_cast<float4_t*>(bm_dkv_lds);
+    // (the tiles' last readers have passed a barrier, or no step ran at all)
+    if (part == 1) {
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        sums[(2 * nb) * kBmThreads + tid] = acc_k[nb];
+        sums[(2 * nb + 1) * kBmThreads + tid] = acc_v[nb];
+      }
+    }
+    __syncthreads();
+    if (part != 0) return;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      const float4_t dk = sums[(2 * nb) * kBmThreads + tid], dv = sums[(2 * nb + 1) * kBmThreads + tid];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc_k[nb][j] += dk[j];
+        acc_v[nb][j] += dv[j];
+      }
     }
   }
 
@@ -504,6 +589,28 @@ inline bm_fn pick(bool bf16, bool swizzled, bm_fn bf16_padded, bm_fn f16_padded,
   return swizzled ? (bf16 ? bf16_swizzled : f16_swizzled) : (bf16 ? bf16_padded : f16_padded);
 }
 
+// the dkv kernel of a (type, head dim, layout, parts) with its LDS size; more than 64 KB has to be allowed once
+struct DkvLaunch {
+  bm_fn fn;
+  int lds_bytes, threads;
+};
+template <int KIND, int D, bool SWZ, int P>
+DkvLaunch dkv_launch() {
+  constexpr int kBytes = DkvLds<D, SWZ, P>::kBytes;
+  const bm_fn fn = bwd_mfma_dkv_kernel<KIND, D, SWZ, P>;
+  if constexpr (kBytes > 64 * 1024) {
+    static const hipError_t allowed =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
+    if (allowed != hipSuccess) return DkvLaunch{nullptr, 0, 0};
+  }
+  return DkvLaunch{fn, kBytes, kBmThreads * P};
+}
+template <int KIND, int D>
+DkvLaunch dkv_launch(bool swizzled, int parts) {
+  if (swizzled) return dkv_launch<KIND, D, true, 1>();
+  return parts == 2 ? dkv_launch<KIND, D, false, 2>() : dkv_launch<KIND, D, false, 1>();
+}
+
 }  // namespace
 
 int launch_attention_backward_mfma(const BwdParams& p, void* stream) {
@@ -511,37 +618,45 @@ int launch_attention_backward_mfma(const BwdParams& p, void* stream) {
   if (p.head_dim != 64 && p.head_dim != 128) return ARENO_ERR_UNSUPPORTED;
   if (p.q_heads > 65535 || p.kv_heads > 65535) return ARENO_ERR_UNSUPPORTED;
   const int64_t q_blocks = (p.q_tokens + kBmRows - 1) / kBmRows, k_blocks = (p.k_tokens + kBmRows - 1) / kBmRows;
-  if (q_blocks > 0x7fffffffLL || k_blocks > 0x7fffffffLL) return ARENO_ERR_UNSUPPORTED;
+  if (q_blocks * p.q_heads > 0x7fffffffLL || k_blocks * p.kv_heads > 0x7fffffffLL) return ARENO_ERR_UNSUPPORTED;
   const bool bf16 = p.dtype == ARENO_DT_BF16;
   // the swizzled tile layout once a compute unit (256 of them) gets workgroups in several rounds: 8 and 16 a unit
   // and more measured faster with it, 1 to 7 a unit faster without
   bool dq_swz = q_blocks * p.q_heads > 16 * kBmComputeUnits, dkv_swz = k_blocks * p.kv_heads > 4 * kBmComputeUnits;
-  // ARENO_BACKWARD_TILES=swizzled|padded (read at every launch) fixes the layout: both give the same bits, so this is
-  // for tests of the one a small launch would not take, and for timing
+  // the dkv kernel in two parts up to that size: 2 to 20 % faster from 1 to 4 workgroups per unit (the launch ends
+  // with its longest workgroups, and theirs is the chain that the split halves), no difference above
+  int dkv_parts = dkv_swz ? 1 : 2;
+  // ARENO_BACKWARD_TILES=swizzled|padded and ARENO_BACKWARD_PARTS=1|2 (read at every launch) fix these choices: all
+  // give the same dQ and, up to the order of one last sum, the same dK and dV, so this is for tests of the kernels
+  // a launch of the test's size would not take, and for timing
   if (const char* e = getenv("ARENO_BACKWARD_TILES")) {
     if (strcmp(e, "swizzled") == 0) dq_swz = dkv_swz = true;
     if (strcmp(e, "padded") == 0) dq_swz = dkv_swz = false;
   }
-  bm_fn dq, dkv;
+  if (const char* e = getenv("ARENO_BACKWARD_PARTS")) {
+    if (strcmp(e, "1") == 0) dkv_parts = 1;
+    if (strcmp(e, "2") == 0 && !dkv_swz) dkv_parts = 2;  // (the swizzled layout comes in one part only)
+  }
+  bm_fn dq;
+  DkvLaunch dkv;
   if (p.head_dim == 64) {
     dq = pick(bf16, dq_swz, bwd_mfma_dq_kernel<KV_BF16, 64, false>, bwd_mfma_dq_kernel<KV_F16, 64, false>,
               bwd_mfma_dq_kernel<KV_BF16, 64, true>, bwd_mfma_dq_kernel<KV_F16, 64, true>);
-    dkv = pick(bf16, dkv_swz, bwd_mfma_dkv_kernel<KV_BF16, 64, false>, bwd_mfma_dkv_kernel<KV_F16, 64, false>,
-               bwd_mfma_dkv_kernel<KV_BF16, 64, true>, bwd_mfma_dkv_kernel<KV_F16, 64, true>);
+    dkv = bf16 ? dkv_launch<KV_BF16, 64>(dkv_swz, dkv_parts) : dkv_launch<KV_F16, 64>(dkv_swz, dkv_parts);
   } else {
     dq = pick(bf16, dq_swz, bwd_mfma_dq_kernel<KV_BF16, 128, false>, bwd_mfma_dq_kernel<KV_F16, 128, false>,
               bwd_mfma_dq_kernel<KV_BF16, 128, true>, bwd_mfma_dq_kernel<KV_F16, 128, true>);
-    dkv = pick(bf16, dkv_swz, bwd_mfma_dkv_kernel<KV_BF16, 128, false>, bwd_mfma_dkv_kernel<KV_F16, 128, false>,
-               bwd_mfma_dkv_kernel<KV_BF16, 128, true>, bwd_mfma_dkv_kernel<KV_F16, 128, true>);
+    dkv = bf16 ? dkv_launch<KV_BF16, 128>(dkv_swz, dkv_parts) : dkv_launch<KV_F16, 128>(dkv_swz, dkv_parts);
   }
   const char* op = "areno_hip_attention_backward";
+  if (dkv.fn == nullptr) return fail(ARENO_ERR_LAUNCH, "%s: the dkv kernel's LDS size was refused", op);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (q_blocks > 0) {
-    hipLaunchKernelGGL(dq, dim3(static_cast<unsigned>(q_blocks), p.q_heads), dim3(kBmThreads), 0, s, p);
+    hipLaunchKernelGGL(dq, dim3(static_cast<unsigned>(q_blocks * p.q_heads)), dim3(kBmThreads), 0, s, p);
     if (int rc = check_launch(op)) return rc;
   }
   if (k_blocks > 0) {
-    hipLaunchKernelGGL(dkv, dim3(static_cast<unsigned>(k_blocks), p.kv_heads), dim3(kBmThreads), 0, s, p);
+    hipLaunchKernelGGL(dkv.fn, dim3(static_cast<unsigned>(k_blocks * p.kv_heads)), dim3(dkv.threads), dkv.lds_bytes, s, p);
     if (int rc = check_launch(op)) return rc;
   }
   return ARENO_OK;
