@@ -71,33 +71,19 @@ __device__ __forceinline__ int64_t block_in_cost_order(int64_t i, int64_t blocks
   return (i % runs) * per + i / runs;
 }
 
-// A tile of 32 rows x D 16-bit elements in LDS, in one of two layouts.
-//   padded (SWZ = false)    row stride D * 2 + 16 bytes.  The row operands (16 lanes read the same 16-byte chunk of 16
-//                           rows) meet every bank once, the transposed ones (32 lanes read 32 bytes of 8 consecutive
-//                           rows) meet every bank twice; all addresses are one base plus constants.
-//   swizzled (SWZ = true)   rows back to back, the 16-byte chunks of a row permuted: chunk c of row r lies at place
-//                           c ^ swizzle(r).  Both kinds of reads meet every bank once, at the price of an address
-//                           register per chunk.
-// Measured: without bank conflicts LDS is busy 40 % less, which pays once several workgroups share a compute unit's
-// LDS (3 % at 8 workgroups per unit), while a launch of one or two workgroups per unit is 3-8 % faster on the padded
-// layout; the launcher picks by the size of the grid.
-// Staging: every thread moves kChunks 16-byte chunks of a tensor through registers.
-template <int D, bool SWZ>
+// A tile of 32 rows x D 16-bit elements in LDS, row stride D * 2 + 16 bytes: the row operands (16 lanes read the same
+// 16-byte chunk of 16 rows) meet every bank once, the transposed ones (32 lanes read 32 bytes of 8 consecutive rows)
+// meet every bank twice.  (A layout without any bank conflict -- rows back to back, the chunks of a row permuted by
+// a function of the row -- was measured: LDS is busy 40 % less with it and no launch got faster, small ones 3-8 %
+// slower from the address registers it takes.)  Staging: every thread moves kChunks 16-byte chunks of a tensor
+// through registers.
+template <int D>
 struct BmTile {
-  static constexpr int RS = SWZ ? D * 2 : D * 2 + 16;
+  static constexpr int RS = D * 2 + 16;
   static constexpr int kChunksPerRow = D * 2 / 16;
   static constexpr int kChunks = kBmTile * kChunksPerRow / kBmThreads;  // per thread: 1 (D = 64) or 2 (D = 128)
   static_assert(kBmTile * kChunksPerRow % kBmThreads == 0, "tile chunks");
-  static_assert(D == 64 || D == 128, "the swizzle is written for rows of 128 and 256 bytes");
-  // D = 128 (a row spans all 64 banks): bits 1-3 from the row's low bits separate 8 consecutive rows' chunk pairs,
-  // bit 0 from row bit 3 separates rows r and r + 8.  D = 64 (two rows span the banks, row bit 0 picks the half):
-  // bits 1-2 from row bits 1-2, bit 0 from row bit 3.
-  static __device__ __forceinline__ int swizzle(int r) {
-    return D == 128 ? (((r & 7) << 1) ^ ((r >> 3) & 1)) : ((((r >> 1) & 3) << 1) ^ ((r >> 3) & 1));
-  }
-  static __device__ __forceinline__ int chunk_pos(int r, int c) {
-    return SWZ ? r * RS + ((c ^ swizzle(r)) << 4) : r * RS + (c << 4);
-  }
+  static __device__ __forceinline__ int chunk_pos(int r, int c) { return r * RS + (c << 4); }
 };
 
 // Operand reads.  Row operand (A of the first pair of products): row 16 tg + lr of the tile, elements
@@ -138,11 +124,11 @@ __device__ __forceinline__ float operand_element(uint32_t word, int hi) {
 }
 
 // ---- dQ (and the rows' statistics) ------------------------------------------------------------------------------------
-template <int KIND, int D, bool SWZ>
+template <int KIND, int D>
 __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p) {
   using Ops = MfmaOps<KIND>;
   using V8 = typename Ops::vec8;
-  using T = BmTile<D, SWZ>;
+  using T = BmTile<D>;
   constexpr int NS = D / 32, NB = D / 16;
   __shared__ __attribute__((aligned(16))) char s_k[kBmTile * T::RS];
   __shared__ __attribute__((aligned(16))) char s_v[kBmTile * T::RS];
@@ -332,9 +318,9 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
 // rows and take every second step of the stream each (tiles and statistics of their own in LDS), and the second
 // part's sums go through LDS to the first at the end.  That halves the longest chain of steps of a launch too small
 // to give every compute unit two workgroups; the order of the sums stays fixed.
-template <int D, bool SWZ, int P>
+template <int D, int P>
 struct DkvLds {
-  using T = BmTile<D, SWZ>;
+  using T = BmTile<D>;
   static constexpr int kTile = kBmTile * T::RS;
   static constexpr int kStat = kBmTile * 2 * 4;
   // per part and buffer: a Q tile, a dO tile, the rows' statistics
@@ -345,12 +331,12 @@ struct DkvLds {
 };
 extern __shared__ __attribute__((aligned(16))) char bm_dkv_lds[];
 
-template <int KIND, int D, bool SWZ, int P>
+template <int KIND, int D, int P>
 __global__ __launch_bounds__(kBmThreads* P, P == 1 ? 2 : 1) void bwd_mfma_dkv_kernel(BwdParams p) {
   using Ops = MfmaOps<KIND>;
   using V8 = typename Ops::vec8;
-  using T = BmTile<D, SWZ>;
-  using L = DkvLds<D, SWZ, P>;
+  using T = BmTile<D>;
+  using L = DkvLds<D, P>;
   constexpr int NS = D / 32, NB = D / 16;
 
   const int part = P > 1 ? static_cast<int>(threadIdx.x) / kBmThreads : 0;  // (the same for a wave)
@@ -585,19 +571,16 @@ __global__ __launch_bounds__(kBmThreads* P, P == 1 ? 2 : 1) void bwd_mfma_dkv_ke
 
 typedef void (*bm_fn)(BwdParams);
 constexpr int64_t kBmComputeUnits = 256;
-inline bm_fn pick(bool bf16, bool swizzled, bm_fn bf16_padded, bm_fn f16_padded, bm_fn bf16_swizzled, bm_fn f16_swizzled) {
-  return swizzled ? (bf16 ? bf16_swizzled : f16_swizzled) : (bf16 ? bf16_padded : f16_padded);
-}
 
-// the dkv kernel of a (type, head dim, layout, parts) with its LDS size; more than 64 KB has to be allowed once
+// the dkv kernel of a (type, head dim, parts) with its LDS size; more than 64 KB has to be allowed once
 struct DkvLaunch {
   bm_fn fn;
   int lds_bytes, threads;
 };
-template <int KIND, int D, bool SWZ, int P>
+template <int KIND, int D, int P>
 DkvLaunch dkv_launch() {
-  constexpr int kBytes = DkvLds<D, SWZ, P>::kBytes;
-  const bm_fn fn = bwd_mfma_dkv_kernel<KIND, D, SWZ, P>;
+  constexpr int kBytes = DkvLds<D, P>::kBytes;
+  const bm_fn fn = bwd_mfma_dkv_kernel<KIND, D, P>;
   if constexpr (kBytes > 64 * 1024) {
     static const hipError_t allowed =
         hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
@@ -606,9 +589,8 @@ DkvLaunch dkv_launch() {
   return DkvLaunch{fn, kBytes, kBmThreads * P};
 }
 template <int KIND, int D>
-DkvLaunch dkv_launch(bool swizzled, int parts) {
-  if (swizzled) return dkv_launch<KIND, D, true, 1>();
-  return parts == 2 ? dkv_launch<KIND, D, false, 2>() : dkv_launch<KIND, D, false, 1>();
+DkvLaunch dkv_launch(int parts) {
+  return parts == 2 ? dkv_launch<KIND, D, 2>() : dkv_launch<KIND, D, 1>();
 }
 
 }  // namespace
@@ -620,33 +602,29 @@ int launch_attention_backward_mfma(const BwdParams& p, void* stream) {
   const int64_t q_blocks = (p.q_tokens + kBmRows - 1) / kBmRows, k_blocks = (p.k_tokens + kBmRows - 1) / kBmRows;
   if (q_blocks * p.q_heads > 0x7fffffffLL || k_blocks * p.kv_heads > 0x7fffffffLL) return ARENO_ERR_UNSUPPORTED;
   const bool bf16 = p.dtype == ARENO_DT_BF16;
-  // the swizzled tile layout once a compute unit (256 of them) gets workgroups in several rounds: 8 and 16 a unit
-  // and more measured faster with it, 1 to 7 a unit faster without
-  bool dq_swz = q_blocks * p.q_heads > 16 * kBmComputeUnits, dkv_swz = k_blocks * p.kv_heads > 4 * kBmComputeUnits;
-  // the dkv kernel in two parts up to that size: 2 to 20 % faster from 1 to 4 workgroups per unit (the launch ends
-  // with its longest workgroups, and theirs is the chain that the split halves), no difference above
-  int dkv_parts = dkv_swz ? 1 : 2;
-  // ARENO_BACKWARD_TILES=swizzled|padded and ARENO_BACKWARD_PARTS=1|2 (read at every launch) fix these choices: all
-  // give the same dQ and, up to the order of one last sum, the same dK and dV, so this is for tests of the kernels
-  // a launch of the test's size would not take, and for timing
-  if (const char* e = getenv("ARENO_BACKWARD_TILES")) {
-    if (strcmp(e, "swizzled") == 0) dq_swz = dkv_swz = true;
-    if (strcmp(e, "padded") == 0) dq_swz = dkv_swz = false;
-  }
+  // The dkv kernel in two parts while the launch is small: it ends with its longest workgroups, and theirs is the
+  // chain of steps that the split halves (head dim 128: 2 to 20 % faster from 1 to 4 workgroups per compute unit, no
+  // difference above; head dim 64: 14 % faster at 2 per unit, 10 % slower at 4, 2.3 x slower at 8 -- there a
+  // two-part workgroup fills a unit's registers alone, while one-part ones share them four at a time).  Chains too
+  // short to matter stay in one part: the split wants about 64 steps in the longest chain, estimated from the mean
+  // sequence length.
+  const int64_t two_parts_up_to = (p.head_dim == 128 ? 4 : 2) * kBmComputeUnits;
+  const int64_t longest_chain = p.q_tokens / (p.num_seqs > 0 ? p.num_seqs : 1) / kBmTile * (p.q_heads / p.kv_heads);
+  int dkv_parts = k_blocks * p.kv_heads <= two_parts_up_to && longest_chain >= 64 ? 2 : 1;
+  // ARENO_BACKWARD_PARTS=1|2 (read at every launch) fixes the choice: the same dK and dV up to the order of one last
+  // sum, so this is for tests of the kernel a launch of the test's size would not take, and for timing
   if (const char* e = getenv("ARENO_BACKWARD_PARTS")) {
     if (strcmp(e, "1") == 0) dkv_parts = 1;
-    if (strcmp(e, "2") == 0 && !dkv_swz) dkv_parts = 2;  // (the swizzled layout comes in one part only)
+    if (strcmp(e, "2") == 0) dkv_parts = 2;
   }
   bm_fn dq;
   DkvLaunch dkv;
   if (p.head_dim == 64) {
-    dq = pick(bf16, dq_swz, bwd_mfma_dq_kernel<KV_BF16, 64, false>, bwd_mfma_dq_kernel<KV_F16, 64, false>,
-              bwd_mfma_dq_kernel<KV_BF16, 64, true>, bwd_mfma_dq_kernel<KV_F16, 64, true>);
-    dkv = bf16 ? dkv_launch<KV_BF16, 64>(dkv_swz, dkv_parts) : dkv_launch<KV_F16, 64>(dkv_swz, dkv_parts);
+    dq = bf16 ? bwd_mfma_dq_kernel<KV_BF16, 64> : bwd_mfma_dq_kernel<KV_F16, 64>;
+    dkv = bf16 ? dkv_launch<KV_BF16, 64>(dkv_parts) : dkv_launch<KV_F16, 64>(dkv_parts);
   } else {
-    dq = pick(bf16, dq_swz, bwd_mfma_dq_kernel<KV_BF16, 128, false>, bwd_mfma_dq_kernel<KV_F16, 128, false>,
-              bwd_mfma_dq_kernel<KV_BF16, 128, true>, bwd_mfma_dq_kernel<KV_F16, 128, true>);
-    dkv = bf16 ? dkv_launch<KV_BF16, 128>(dkv_swz, dkv_parts) : dkv_launch<KV_F16, 128>(dkv_swz, dkv_parts);
+    dq = bf16 ? bwd_mfma_dq_kernel<KV_BF16, 128> : bwd_mfma_dq_kernel<KV_F16, 128>;
+    dkv = bf16 ? dkv_launch<KV_BF16, 128>(dkv_parts) : dkv_launch<KV_F16, 128>(dkv_parts);
   }
   const char* op = "areno_hip_attention_backward";
   if (dkv.fn == nullptr) return fail(ARENO_ERR_LAUNCH, "%s: the dkv kernel's LDS size was refused", op);
