@@ -26,6 +26,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "attention_backward.hpp"
@@ -572,7 +573,7 @@ __global__ __launch_bounds__(kBmThreads* P, P == 1 ? 2 : 1) void bwd_mfma_dkv_ke
 typedef void (*bm_fn)(BwdParams);
 constexpr int64_t kBmComputeUnits = 256;
 
-// the dkv kernel of a (type, head dim, parts) with its LDS size; more than 64 KB has to be allowed once
+// the dkv kernel of a (type, head dim, parts) with its LDS size; more than 64 KB has to be allowed once per device
 struct DkvLaunch {
   bm_fn fn;
   int lds_bytes, threads;
@@ -582,9 +583,17 @@ DkvLaunch dkv_launch() {
   constexpr int kBytes = DkvLds<D, P>::kBytes;
   const bm_fn fn = bwd_mfma_dkv_kernel<KIND, D, P>;
   if constexpr (kBytes > 64 * 1024) {
-    static const hipError_t allowed =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
-    if (allowed != hipSuccess) return DkvLaunch{nullptr, 0, 0};
+    static std::atomic<uint64_t> allowed_on{0};  // one bit per device (the attribute belongs to the device's copy)
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return DkvLaunch{nullptr, 0, 0};
+    if ((allowed_on.load(std::memory_order_acquire) >> device & 1) == 0) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kBytes) !=
+          hipSuccess) {
+        (void)hipGetLastError();
+        return DkvLaunch{nullptr, 0, 0};
+      }
+      allowed_on.fetch_or(uint64_t{1} << device, std::memory_order_release);
+    }
   }
   return DkvLaunch{fn, kBytes, kBmThreads * P};
 }
