@@ -40,6 +40,10 @@ HIP_DEVICE_FLAGS = [
     # leading scalar kernel arguments (up to 16 words) arrive in registers at wave start instead of through a fetch of
     # the argument block: the decode kernels put what their first loads are addressed with there
     "-mllvm", "-amdgpu-kernarg-preload-count=16",
+    # matrix products accumulate in vector registers: left to itself the compiler puts the decode kernels'
+    # accumulators into accumulation registers and copies all 36 of them out and back around the rescaling of every
+    # tile step (117 copies per step at head dim 128); no kernel here needs more than the 256 vector registers
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-DARENO_DEVICE_FLAGS_OK=1",  # device_common.hpp refuses to compile without the two flags above
 ] + [f"-D{name}={os.environ[name]}" for name in ("ARENO_MFMA_NW", "ARENO_TRACE", "ARENO_MFMA_QUANT_OCC", "ARENO_MFMA_WIDE_OCC", "ARENO_PREFILL_WAVES") if os.environ.get(name)]  # fmt: skip
 
