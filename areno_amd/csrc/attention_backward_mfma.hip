@@ -315,33 +315,47 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
 }
 
 // ---- dK, dV -------------------------------------------------------------------------------------------------------------
-// P = 1: four waves, one stream of tiles.  P = 2: eight waves in two parts of four; both parts own the same 64 key
-// rows and take every second step of the stream each (tiles and statistics of their own in LDS), and the second
-// part's sums go through LDS to the first at the end.  That halves the longest chain of steps of a launch too small
-// to give every compute unit two workgroups; the order of the sums stays fixed.
-template <int D, int P>
-struct DkvLds {
-  using T = BmTile<D>;
-  static constexpr int kTile = kBmTile * T::RS;
+// A workgroup owns a block of KR packed key rows of one kv head, or two of them one after the other: block i and
+// block blocks - 1 - i.  A key block early in its sequence is seen by all later queries and one late in it by few.
+// A launch of many workgroups per compute unit evens that out by starting the expensive blocks first
+// (block_in_cost_order); in a launch of about one workgroup per unit nothing comes after the expensive block to
+// fill the gap, and there the pairs help: for sequences of about equal length the costs of such a pair add up to
+// the same for every i, so the workgroups end together.  (The launcher says which by the size of the grid.)
+// The workgroup has P parts of KR / 16 waves.  Every part owns all KR key rows (16 per wave) and takes every P-th
+// step of the stream of query tiles (tiles and statistics of its own in LDS); the sums of parts 1 .. P - 1 go to
+// part 0 through LDS at the end of a block, in a fixed order.  More parts shorten the chain of steps a block is:
+// (KR, P) = (64, 1) four waves, two workgroups per compute unit, for launches that fill the units several times;
+// (64, 2) and (32, 4) eight waves, for launches of about one workgroup per unit.
+template <int D, int KR, int P>
+struct DkvShape {
+  static constexpr int kKeyWaves = KR / 16;
+  static constexpr int kPartThreads = kKeyWaves * kWave;
+  static constexpr int kThreads = kPartThreads * P;
+  static constexpr int RS = BmTile<D>::RS;
+  static constexpr int kChunksPerRow = BmTile<D>::kChunksPerRow;
+  static constexpr int kChunks = kBmTile * kChunksPerRow / kPartThreads;  // 16-byte chunks of a tile per thread of a part
+  static_assert(kBmTile * kChunksPerRow % kPartThreads == 0, "tile chunks");
+  static constexpr int kTile = kBmTile * RS;
   static constexpr int kStat = kBmTile * 2 * 4;
   // per part and buffer: a Q tile, a dO tile, the rows' statistics
   static constexpr int kBuffer = 2 * kTile + kStat;
   static constexpr int kStream = P * 2 * kBuffer;
-  static constexpr int kSums = P > 1 ? kBmThreads * (D / 16) * 2 * 16 : 0;  // (P = 2: a float4 per lane, block and tensor)
-  static constexpr int kBytes = kStream > kSums ? kStream : kSums;
+  static constexpr int kSums = (P - 1) * kPartThreads * (D / 16) * 2 * 16;  // a float4 per lane, block of 16 and tensor
+  static constexpr int kLdsBytes = kStream > kSums ? kStream : kSums;
 };
 extern __shared__ __attribute__((aligned(16))) char bm_dkv_lds[];
 
-template <int KIND, int D, int P>
-__global__ __launch_bounds__(kBmThreads* P, P == 1 ? 2 : 1) void bwd_mfma_dkv_kernel(BwdParams p) {
+template <int KIND, int D, int KR, int P>
+__global__ __launch_bounds__((DkvShape<D, KR, P>::kThreads), (DkvShape<D, KR, P>::kThreads == 256 ? 2 : 1)) void bwd_mfma_dkv_kernel(
+    BwdParams p) {
   using Ops = MfmaOps<KIND>;
   using V8 = typename Ops::vec8;
   using T = BmTile<D>;
-  using L = DkvLds<D, P>;
+  using L = DkvShape<D, KR, P>;
   constexpr int NS = D / 32, NB = D / 16;
 
-  const int part = P > 1 ? static_cast<int>(threadIdx.x) / kBmThreads : 0;  // (the same for a wave)
-  const int tid = P > 1 ? static_cast<int>(threadIdx.x) % kBmThreads : static_cast<int>(threadIdx.x);  // thread of the part
+  const int part = P > 1 ? static_cast<int>(threadIdx.x) / L::kPartThreads : 0;  // (the same for a wave)
+  const int tid = P > 1 ? static_cast<int>(threadIdx.x) % L::kPartThreads : static_cast<int>(threadIdx.x);  // in the part
   char* const lds = bm_dkv_lds + part * (2 * L::kBuffer);
   auto s_q = [&](int buf) { return lds + buf * L::kBuffer; };
   auto s_g = [&](int buf) { return lds + buf * L::kBuffer + L::kTile; };
@@ -350,222 +364,239 @@ __global__ __launch_bounds__(kBmThreads* P, P == 1 ? 2 : 1) void bwd_mfma_dkv_ke
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
   const int lr = lane & 15, lk = lane >> 4;
-  // workgroups in launch order: the kv heads of a block next to each other, the blocks by cost
   const int kvh = static_cast<int>(blockIdx.x % static_cast<unsigned>(p.kv_heads));
   const int group = p.q_heads / p.kv_heads;
-  const int64_t k_blocks = (p.k_tokens + kBmRows - 1) / kBmRows;
-  const int64_t r0 = block_in_cost_order(blockIdx.x / static_cast<unsigned>(p.kv_heads), k_blocks, p.num_seqs, false) * kBmRows;
-  const int64_t block_end = r0 + kBmRows < p.k_tokens ? r0 + kBmRows : p.k_tokens;
-  const int64_t row = r0 + 16 * wave + lr;  // this lane's key row (a column of the products)
-  const bool row_exists = row < p.k_tokens;
+  const int64_t k_blocks = (p.k_tokens + KR - 1) / KR;
+  const int64_t wg = blockIdx.x / static_cast<unsigned>(p.kv_heads);
+  // (launched with a workgroup per pair of blocks, or with one per block: then in cost order, one block each)
+  const bool paired = gridDim.x / static_cast<unsigned>(p.kv_heads) < k_blocks;
+  const int64_t first_block = paired ? wg : block_in_cost_order(wg, k_blocks, p.num_seqs, false);
 
-  // this lane's parts of its row of K and V (B operands)
-  const int64_t row_elem = (row * p.kv_heads + kvh) * D;
-  V8 kop[NS], vop[NS];
+  for (int half = 0; half < 2; ++half) {
+    const int64_t block = half == 0 ? first_block : k_blocks - 1 - first_block;
+    // (no second block without pairs, and none for the middle one of an odd number of blocks)
+    if (half == 1 && (!paired || block <= first_block)) break;
+    const int64_t r0 = block * KR;
+    const int64_t block_end = r0 + KR < p.k_tokens ? r0 + KR : p.k_tokens;
+    const int64_t row = r0 + 16 * wave + lr;  // this lane's key row (a column of the products)
+    const bool row_exists = row < p.k_tokens;
+
+    // this lane's parts of its row of K and V (B operands)
+    const int64_t row_elem = (row * p.kv_heads + kvh) * D;
+    V8 kop[NS], vop[NS];
 #pragma unroll
-  for (int sl = 0; sl < NS; ++sl) {
-    uint4_t kw = {0u, 0u, 0u, 0u}, vw = kw;
-    if (row_exists) {
-      const int64_t off = (row_elem + (D / 4) * lk + 8 * sl) * 2;
-      kw = load16(p.k, off);
-      vw = load16(p.v, off);
+    for (int sl = 0; sl < NS; ++sl) {
+      uint4_t kw = {0u, 0u, 0u, 0u}, vw = kw;
+      if (row_exists) {
+        const int64_t off = (row_elem + (D / 4) * lk + 8 * sl) * 2;
+        kw = load16(p.k, off);
+        vw = load16(p.v, off);
+      }
+      kop[sl] = __builtin_bit_cast(V8, kw);
+      vop[sl] = __builtin_bit_cast(V8, vw);
     }
-    kop[sl] = __builtin_bit_cast(V8, kw);
-    vop[sl] = __builtin_bit_cast(V8, vw);
-  }
-  float4_t acc_k[NB], acc_v[NB];
+    float4_t acc_k[NB], acc_v[NB];
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) acc_k[nb] = acc_v[nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int nb = 0; nb < NB; ++nb) acc_k[nb] = acc_v[nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-  for (int s = seq_of_row(p.cu_k, p.num_seqs, r0); s < p.num_seqs; ++s) {
-    const int64_t sk0 = p.cu_k[s], sk1 = p.cu_k[s + 1];
-    if (sk0 >= block_end) break;
-    const int64_t k_lo = sk0 > r0 ? sk0 : r0, k_hi = sk1 < block_end ? sk1 : block_end;
-    if (k_lo >= k_hi) continue;
-    const int ctx = p.ctx != nullptr ? p.ctx[s] : 0;
-    const int64_t q_base = p.cu_q[s];
-    const int n_q = p.cu_q[s + 1] - p.cu_q[s];
-    const bool live = row >= k_lo && row < k_hi;
-    const int key = live ? static_cast<int>(row - sk0) : -1;  // this lane's key position in the sequence
-    const uint64_t live_lanes = __builtin_amdgcn_ballot_w64(live);
-    const bool wave_live = live_lanes != 0, wave_full = live_lanes == ~0ull;
-    // (the wave's 16 key rows, when all of them belong to this sequence)
-    const int wave_key_lo = static_cast<int>(r0 + 16 * wave - sk0), wave_key_hi = wave_key_lo + 15;
-    // queries i (position ctx + i) that see one of the block's keys: key <= ctx + i <= key + window
-    const int key_min = static_cast<int>(k_lo - sk0), key_max = static_cast<int>(k_hi - 1 - sk0);
-    const int i_lo = key_min - ctx > 0 ? key_min - ctx : 0;
-    int i_hi = n_q - 1;
-    if (p.window_left >= 0 && key_max + p.window_left - ctx < i_hi) i_hi = key_max + p.window_left - ctx;
-    if (i_hi < i_lo) continue;  // (the same for the whole workgroup)
-    const int t0 = i_lo / kBmTile, t1 = i_hi / kBmTile;
-    const int tiles = t1 - t0 + 1;
-    // the stream: tiles of every q head of the group, head by head; this part takes steps part, part + P, ...
-    const int stream_steps = tiles * group;
-    const int steps = (stream_steps - part + P - 1) / P;  // this part's
-    const int rounds = (stream_steps + P - 1) / P;        // the longest part's: every part keeps the barriers of all
-    // (head, tile) of a step of the stream, counted up by P steps at a time
-    struct Cursor {
-      int head, tile;
-    };
-    auto advance = [&](Cursor& c) {
-      c.tile += P;
-      while (c.tile > t1) {
-        c.tile -= tiles;
-        ++c.head;
-      }
-    };
-    Cursor first = {kvh * group, t0 + part};
-    while (first.tile > t1) {
-      first.tile -= tiles;
-      ++first.head;
-    }
-
-    // Two register sets hold the tiles of the next two steps while they are in flight; a step computes on one of the
-    // two LDS buffers, moves the next step's tile into the other one and asks for the tile two steps further on.
-    struct Staged {
-      uint4_t q[T::kChunks], g[T::kChunks];
-      float2_t stat;
-    };
-    Staged set_a, set_b;
-    Cursor fetch_at = first;
-    int fetched = 0;
-    auto fetch = [&](Staged& st) {
-      if (fetched >= steps) return;
-      ++fetched;
-      const int hq = fetch_at.head, t = fetch_at.tile;
-      advance(fetch_at);
-#pragma unroll
-      for (int i = 0; i < T::kChunks; ++i) {
-        const int c = tid + kBmThreads * i;
-        const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
-        const int qi = kBmTile * t + r < n_q ? kBmTile * t + r : n_q - 1;  // rows past the end repeat the last query
-        const int64_t off = ((q_base + qi) * p.q_heads + hq) * (D * 2) + col * 16;
-        st.q[i] = load16(p.q, off);
-        st.g[i] = load16(p.grad_out, off);
-      }
-      if (tid < kBmTile) {
-        const int qi = kBmTile * t + tid < n_q ? kBmTile * t + tid : n_q - 1;
-        st.stat = *reinterpret_cast<const float2_t*>(p.row_stats + ((q_base + qi) * p.q_heads + hq) * 2);
-      }
-    };
-    auto publish = [&](const Staged& st, int buf) {
-#pragma unroll
-      for (int i = 0; i < T::kChunks; ++i) {
-        const int c = tid + kBmThreads * i;
-        const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
-        *reinterpret_cast<uint4_t*>(s_q(buf) + T::chunk_pos(r, col)) = st.q[i];
-        *reinterpret_cast<uint4_t*>(s_g(buf) + T::chunk_pos(r, col)) = st.g[i];
-      }
-      if (tid < kBmTile) *reinterpret_cast<float2_t*>(s_stat(buf) + 2 * tid) = st.stat;
-    };
-    Cursor at = first;  // the step being computed
-    // one step: the products of the tile in LDS buffer `buf`; between them the next step's tile goes from `next`
-    // into the other buffer and `next` is asked to fetch again
-    auto step_on = [&](int step, int buf, Staged& next) {
-      const int t = at.tile;
-      advance(at);
-      const bool compute = wave_live && step < steps;
-      float pr[2][4], ds[2][4];
-      auto first_products = [&](auto masked) {
-#pragma unroll
-        for (int tg = 0; tg < 2; ++tg) {
-          // the statistics of the four query rows this lane gets from the products: rows 16 tg + 4 lk .. + 3
-          const float4_t st01 = *reinterpret_cast<const float4_t*>(s_stat(buf) + 2 * (16 * tg + 4 * lk));
-          const float4_t st23 = *reinterpret_cast<const float4_t*>(s_stat(buf) + 2 * (16 * tg + 4 * lk + 2));
-          const float lse[4] = {st01[0], st01[2], st23[0], st23[2]};
-          const float dlt[4] = {st01[1], st01[3], st23[1], st23[3]};
-          float4_t c1 = {0.0f, 0.0f, 0.0f, 0.0f}, c2 = c1;
-#pragma unroll
-          for (int sl = 0; sl < NS; ++sl) {
-            c1 = Ops::mfma(tile_row_operand<KIND, T, D>(s_q(buf), tg, sl, lr, lk), kop[sl], c1);
-            c2 = Ops::mfma(tile_row_operand<KIND, T, D>(s_g(buf), tg, sl, lr, lk), vop[sl], c2);
-          }
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            float x = c1[j] * p.scale_log2e - lse[j];
-            if constexpr (decltype(masked)::value) {
-              const int qi = kBmTile * t + 16 * tg + 4 * lk + j;  // query of the sequence
-              const int pos = ctx + qi;
-              const bool ok = live && qi < n_q && key <= pos && (p.window_left < 0 || key >= pos - p.window_left);
-              x = ok ? x : kBmNegInf;
-            }
-            // (a query without visible keys has +inf as its log-sum-exp: exp2(-inf) = 0 either way)
-            const float pe = fast_exp2(x);
-            pr[tg][j] = pe;
-            ds[tg][j] = pe * (c2[j] - dlt[j]);
-          }
+    for (int s = seq_of_row(p.cu_k, p.num_seqs, r0); s < p.num_seqs; ++s) {
+      const int64_t sk0 = p.cu_k[s], sk1 = p.cu_k[s + 1];
+      if (sk0 >= block_end) break;
+      const int64_t k_lo = sk0 > r0 ? sk0 : r0, k_hi = sk1 < block_end ? sk1 : block_end;
+      if (k_lo >= k_hi) continue;
+      const int ctx = p.ctx != nullptr ? p.ctx[s] : 0;
+      const int64_t q_base = p.cu_q[s];
+      const int n_q = p.cu_q[s + 1] - p.cu_q[s];
+      const bool live = row >= k_lo && row < k_hi;
+      const int key = live ? static_cast<int>(row - sk0) : -1;  // this lane's key position in the sequence
+      const uint64_t live_lanes = __builtin_amdgcn_ballot_w64(live);
+      const bool wave_live = live_lanes != 0, wave_full = live_lanes == ~0ull;
+      // (the wave's 16 key rows, when all of them belong to this sequence)
+      const int wave_key_lo = static_cast<int>(r0 + 16 * wave - sk0), wave_key_hi = wave_key_lo + 15;
+      // queries i (position ctx + i) that see one of the block's keys: key <= ctx + i <= key + window
+      const int key_min = static_cast<int>(k_lo - sk0), key_max = static_cast<int>(k_hi - 1 - sk0);
+      const int i_lo = key_min - ctx > 0 ? key_min - ctx : 0;
+      int i_hi = n_q - 1;
+      if (p.window_left >= 0 && key_max + p.window_left - ctx < i_hi) i_hi = key_max + p.window_left - ctx;
+      if (i_hi < i_lo) continue;  // (the same for the whole workgroup)
+      const int t0 = i_lo / kBmTile, t1 = i_hi / kBmTile;
+      const int tiles = t1 - t0 + 1;
+      // the stream: tiles of every q head of the group, head by head; this part takes steps part, part + P, ...
+      const int stream_steps = tiles * group;
+      const int steps = (stream_steps - part + P - 1) / P;  // this part's
+      const int rounds = (stream_steps + P - 1) / P;        // the longest part's: every part keeps the barriers of all
+      // (head, tile) of a step of the stream, counted up by P steps at a time
+      struct Cursor {
+        int head, tile;
+      };
+      auto advance = [&](Cursor& c) {
+        c.tile += P;
+        while (c.tile > t1) {
+          c.tile -= tiles;
+          ++c.head;
         }
       };
-      if (compute) {
-        // most tiles lie below the diagonal and inside the window as a whole: every query of the tile sees every key
-        // of this wave, and nothing needs a mask
-        const int pos_lo = ctx + kBmTile * t, pos_hi = pos_lo + kBmTile - 1;
-        const bool plain = wave_full && kBmTile * t + kBmTile <= n_q && pos_lo >= wave_key_hi &&
-                           (p.window_left < 0 || pos_hi - p.window_left <= wave_key_lo);
-        if (plain) {
-          first_products(std::false_type{});
-        } else {
-          first_products(std::true_type{});
-        }
+      Cursor first = {kvh * group, t0 + part};
+      while (first.tile > t1) {
+        first.tile -= tiles;
+        ++first.head;
       }
-      if (step + 1 < steps) publish(next, buf ^ 1);
-      fetch(next);
-      if (compute) {
-        const V8 pop = streamed_operand<KIND>(pr);
-        const V8 dsop = streamed_operand<KIND>(ds);
+
+      // Two register sets hold the tiles of the next two steps while they are in flight; a step computes on one of
+      // the two LDS buffers, moves the next step's tile into the other one and asks for the tile two steps further on.
+      struct Staged {
+        uint4_t q[L::kChunks], g[L::kChunks];
+        float2_t stat;
+      };
+      Staged set_a, set_b;
+      Cursor fetch_at = first;
+      int fetched = 0;
+      auto fetch = [&](Staged& st) {
+        if (fetched >= steps) return;
+        ++fetched;
+        const int hq = fetch_at.head, t = fetch_at.tile;
+        advance(fetch_at);
+#pragma unroll
+        for (int i = 0; i < L::kChunks; ++i) {
+          const int c = tid + L::kPartThreads * i;
+          const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
+          const int qi = kBmTile * t + r < n_q ? kBmTile * t + r : n_q - 1;  // rows past the end repeat the last query
+          const int64_t off = ((q_base + qi) * p.q_heads + hq) * (D * 2) + col * 16;
+          st.q[i] = load16(p.q, off);
+          st.g[i] = load16(p.grad_out, off);
+        }
+        if (tid < kBmTile) {
+          const int qi = kBmTile * t + tid < n_q ? kBmTile * t + tid : n_q - 1;
+          st.stat = *reinterpret_cast<const float2_t*>(p.row_stats + ((q_base + qi) * p.q_heads + hq) * 2);
+        }
+      };
+      auto publish = [&](const Staged& st, int buf) {
+#pragma unroll
+        for (int i = 0; i < L::kChunks; ++i) {
+          const int c = tid + L::kPartThreads * i;
+          const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
+          *reinterpret_cast<uint4_t*>(s_q(buf) + T::chunk_pos(r, col)) = st.q[i];
+          *reinterpret_cast<uint4_t*>(s_g(buf) + T::chunk_pos(r, col)) = st.g[i];
+        }
+        if (tid < kBmTile) *reinterpret_cast<float2_t*>(s_stat(buf) + 2 * tid) = st.stat;
+      };
+      Cursor at = first;  // the step being computed
+      // one step: the products of the tile in LDS buffer `buf`; between them the next step's tile goes from `next`
+      // into the other buffer and `next` is asked to fetch again
+      auto step_on = [&](int step, int buf, Staged& next) {
+        const int t = at.tile;
+        advance(at);
+        const bool compute = wave_live && step < steps;
+        float pr[2][4], ds[2][4];
+        auto first_products = [&](auto masked) {
+#pragma unroll
+          for (int tg = 0; tg < 2; ++tg) {
+            // the statistics of the four query rows this lane gets from the products: rows 16 tg + 4 lk .. + 3
+            const float4_t st01 = *reinterpret_cast<const float4_t*>(s_stat(buf) + 2 * (16 * tg + 4 * lk));
+            const float4_t st23 = *reinterpret_cast<const float4_t*>(s_stat(buf) + 2 * (16 * tg + 4 * lk + 2));
+            const float lse[4] = {st01[0], st01[2], st23[0], st23[2]};
+            const float dlt[4] = {st01[1], st01[3], st23[1], st23[3]};
+            float4_t c1 = {0.0f, 0.0f, 0.0f, 0.0f}, c2 = c1;
+#pragma unroll
+            for (int sl = 0; sl < NS; ++sl) {
+              c1 = Ops::mfma(tile_row_operand<KIND, T, D>(s_q(buf), tg, sl, lr, lk), kop[sl], c1);
+              c2 = Ops::mfma(tile_row_operand<KIND, T, D>(s_g(buf), tg, sl, lr, lk), vop[sl], c2);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              float x = c1[j] * p.scale_log2e - lse[j];
+              if constexpr (decltype(masked)::value) {
+                const int qi = kBmTile * t + 16 * tg + 4 * lk + j;  // query of the sequence
+                const int pos = ctx + qi;
+                const bool ok = live && qi < n_q && key <= pos && (p.window_left < 0 || key >= pos - p.window_left);
+                x = ok ? x : kBmNegInf;
+              }
+              // (a query without visible keys has +inf as its log-sum-exp: exp2(-inf) = 0 either way)
+              const float pe = fast_exp2(x);
+              pr[tg][j] = pe;
+              ds[tg][j] = pe * (c2[j] - dlt[j]);
+            }
+          }
+        };
+        if (compute) {
+          // most tiles lie below the diagonal and inside the window as a whole: every query of the tile sees every
+          // key of this wave, and nothing needs a mask
+          const int pos_lo = ctx + kBmTile * t, pos_hi = pos_lo + kBmTile - 1;
+          const bool plain = wave_full && kBmTile * t + kBmTile <= n_q && pos_lo >= wave_key_hi &&
+                             (p.window_left < 0 || pos_hi - p.window_left <= wave_key_lo);
+          if (plain) {
+            first_products(std::false_type{});
+          } else {
+            first_products(std::true_type{});
+          }
+        }
+        if (step + 1 < steps) publish(next, buf ^ 1);
+        fetch(next);
+        if (compute) {
+          const V8 pop = streamed_operand<KIND>(pr);
+          const V8 dsop = streamed_operand<KIND>(ds);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            acc_v[nb] = Ops::mfma(tile_transposed_operand<KIND, T>(s_g(buf), nb, lr, lk), pop, acc_v[nb]);
+            acc_k[nb] = Ops::mfma(tile_transposed_operand<KIND, T>(s_q(buf), nb, lr, lk), dsop, acc_k[nb]);
+          }
+        }
+        __syncthreads();  // every wave has read this step's tile, the next one is in place
+      };
+      // (every wave has passed a barrier behind the last use of the buffers: an earlier sequence's last step, or the
+      // hand-over of the block before)
+      fetch(set_a);
+      fetch(set_b);
+      if (steps > 0) publish(set_a, 0);
+      fetch(set_a);
+      __syncthreads();
+      for (int step = 0; step < rounds; step += 2) {
+        step_on(step, 0, set_b);
+        if (step + 1 < rounds) step_on(step + 1, 1, set_a);
+      }
+    }
+
+    if constexpr (P > 1) {
+      // the other parts' sums to part 0: a float4 per lane, block of 16 and tensor, lanes next to each other
+      // (the tiles' last readers have passed a barrier, or no step ran at all)
+      float4_t* sums = reinterpret_cast<float4_t*>(bm_dkv_lds);
+      if (part > 0) {
+        float4_t* mine = sums + (part - 1) * (2 * NB * L::kPartThreads);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-          acc_v[nb] = Ops::mfma(tile_transposed_operand<KIND, T>(s_g(buf), nb, lr, lk), pop, acc_v[nb]);
-          acc_k[nb] = Ops::mfma(tile_transposed_operand<KIND, T>(s_q(buf), nb, lr, lk), dsop, acc_k[nb]);
+          mine[(2 * nb) * L::kPartThreads + tid] = acc_k[nb];
+          mine[(2 * nb + 1) * L::kPartThreads + tid] = acc_v[nb];
         }
       }
-      __syncthreads();  // every wave has read this step's tile, the next one is in place
-    };
-    // (every wave has passed the barrier behind the last step of an earlier sequence of this block)
-    fetch(set_a);
-    fetch(set_b);
-    if (steps > 0) publish(set_a, 0);
-    fetch(set_a);
-    __syncthreads();
-    for (int step = 0; step < rounds; step += 2) {
-      step_on(step, 0, set_b);
-      if (step + 1 < rounds) step_on(step + 1, 1, set_a);
+      __syncthreads();
+      if (part == 0) {
+#pragma unroll
+        for (int other = 1; other < P; ++other) {
+          const float4_t* theirs = sums + (other - 1) * (2 * NB * L::kPartThreads);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            const float4_t dk = theirs[(2 * nb) * L::kPartThreads + tid], dv = theirs[(2 * nb + 1) * L::kPartThreads + tid];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              acc_k[nb][j] += dk[j];
+              acc_v[nb][j] += dv[j];
+            }
+          }
+        }
+      }
+      __syncthreads();  // the sums are read: the second block's tiles may overwrite them
     }
-  }
 
-  if constexpr (P > 1) {
-    // the second part's sums to the first: a float4 per lane, block and tensor, lanes next to each other
-    float4_t* sums = reinterpret_cast<float4_t*>(bm_dkv_lds);
-    // (the tiles' last readers have passed a barrier, or no step ran at all)
-    if (part == 1) {
+    // every gradient element is written, also the zeros of keys no query sees
+    if (part == 0 && row_exists) {
+      float* dk = p.grad_k + row_elem + 4 * lk;
+      float* dv = p.grad_v + row_elem + 4 * lk;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
-        sums[(2 * nb) * kBmThreads + tid] = acc_k[nb];
-        sums[(2 * nb + 1) * kBmThreads + tid] = acc_v[nb];
+        *reinterpret_cast<float4_t*>(dk + 16 * nb) =
+            float4_t{acc_k[nb][0] * p.scale, acc_k[nb][1] * p.scale, acc_k[nb][2] * p.scale, acc_k[nb][3] * p.scale};
+        *reinterpret_cast<float4_t*>(dv + 16 * nb) = acc_v[nb];
       }
-    }
-    __syncthreads();
-    if (part != 0) return;
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      const float4_t dk = sums[(2 * nb) * kBmThreads + tid], dv = sums[(2 * nb + 1) * kBmThreads + tid];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        acc_k[nb][j] += dk[j];
-        acc_v[nb][j] += dv[j];
-      }
-    }
-  }
-
-  // every gradient element is written, also the zeros of keys no query sees
-  if (row_exists) {
-    float* dk = p.grad_k + row_elem + 4 * lk;
-    float* dv = p.grad_v + row_elem + 4 * lk;
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      *reinterpret_cast<float4_t*>(dk + 16 * nb) =
-          float4_t{acc_k[nb][0] * p.scale, acc_k[nb][1] * p.scale, acc_k[nb][2] * p.scale, acc_k[nb][3] * p.scale};
-      *reinterpret_cast<float4_t*>(dv + 16 * nb) = acc_v[nb];
     }
   }
 }
@@ -573,33 +604,35 @@ __global__ __launch_bounds__(kBmThreads* P, P == 1 ? 2 : 1) void bwd_mfma_dkv_ke
 typedef void (*bm_fn)(BwdParams);
 constexpr int64_t kBmComputeUnits = 256;
 
-// the dkv kernel of a (type, head dim, parts) with its LDS size; more than 64 KB has to be allowed once per device
+// the dkv kernel of a (type, head dim, key rows per block, parts) with its launch shape; more than 64 KB of LDS has
+// to be allowed once per device
 struct DkvLaunch {
   bm_fn fn;
-  int lds_bytes, threads;
+  int lds_bytes, threads, key_rows;
 };
-template <int KIND, int D, int P>
+template <int KIND, int D, int KR, int P>
 DkvLaunch dkv_launch() {
-  constexpr int kBytes = DkvLds<D, P>::kBytes;
-  const bm_fn fn = bwd_mfma_dkv_kernel<KIND, D, P>;
-  if constexpr (kBytes > 64 * 1024) {
+  using L = DkvShape<D, KR, P>;
+  const bm_fn fn = bwd_mfma_dkv_kernel<KIND, D, KR, P>;
+  if constexpr (L::kLdsBytes > 64 * 1024) {
     static std::atomic<uint64_t> allowed_on{0};  // one bit per device (the attribute belongs to the device's copy)
     int device = 0;
-    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return DkvLaunch{nullptr, 0, 0};
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return DkvLaunch{nullptr, 0, 0, 0};
     if ((allowed_on.load(std::memory_order_acquire) >> device & 1) == 0) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kBytes) !=
-          hipSuccess) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              L::kLdsBytes) != hipSuccess) {
         (void)hipGetLastError();
-        return DkvLaunch{nullptr, 0, 0};
+        return DkvLaunch{nullptr, 0, 0, 0};
       }
       allowed_on.fetch_or(uint64_t{1} << device, std::memory_order_release);
     }
   }
-  return DkvLaunch{fn, kBytes, kBmThreads * P};
+  return DkvLaunch{fn, L::kLdsBytes, L::kThreads, KR};
 }
 template <int KIND, int D>
 DkvLaunch dkv_launch(int parts) {
-  return parts == 2 ? dkv_launch<KIND, D, 2>() : dkv_launch<KIND, D, 1>();
+  if (parts == 4) return dkv_launch<KIND, D, 32, 4>();
+  return parts == 2 ? dkv_launch<KIND, D, 64, 2>() : dkv_launch<KIND, D, 64, 1>();
 }
 
 }  // namespace
@@ -611,20 +644,29 @@ int launch_attention_backward_mfma(const BwdParams& p, void* stream) {
   const int64_t q_blocks = (p.q_tokens + kBmRows - 1) / kBmRows, k_blocks = (p.k_tokens + kBmRows - 1) / kBmRows;
   if (q_blocks * p.q_heads > 0x7fffffffLL || k_blocks * p.kv_heads > 0x7fffffffLL) return ARENO_ERR_UNSUPPORTED;
   const bool bf16 = p.dtype == ARENO_DT_BF16;
-  // The dkv kernel in two parts while the launch is small: it ends with its longest workgroups, and theirs is the
-  // chain of steps that the split halves (head dim 128: 2 to 20 % faster from 1 to 4 workgroups per compute unit, no
-  // difference above; head dim 64: 14 % faster at 2 per unit, 10 % slower at 4, 2.3 x slower at 8 -- there a
-  // two-part workgroup fills a unit's registers alone, while one-part ones share them four at a time).  Chains too
-  // short to matter stay in one part: the split wants about 64 steps in the longest chain, estimated from the mean
-  // sequence length.
-  const int64_t two_parts_up_to = (p.head_dim == 128 ? 4 : 2) * kBmComputeUnits;
+  // The dkv kernel's shape by the size of the launch.  About one workgroup per compute unit: pairs of blocks of 32
+  // key rows, eight waves in four parts (2 x 2 048 tokens, 28 / 4 heads: 527 -> 463 us for both launches; one
+  // sequence of 4 096: 975 -> 814 us).  Up to 4 per unit at head dim 128 and 2 at head dim 64: a block of 64 rows
+  // each, in cost order, eight waves in two parts (2 to 20 % faster than one part; above that the two are equal at
+  // 128, and at 64 a two-part workgroup fills a unit's registers alone where four one-part ones fit: 2.3 x slower at
+  // 8 per unit).  Else one part.  Chains too short to matter stay in one part: more parts want about 64 steps in
+  // the longest chain, estimated from the mean sequence length.
+  const int64_t blocks64 = (p.k_tokens + 63) / 64 * p.kv_heads, pairs32 = ((p.k_tokens + 31) / 32 + 1) / 2 * p.kv_heads;
   const int64_t longest_chain = p.q_tokens / (p.num_seqs > 0 ? p.num_seqs : 1) / kBmTile * (p.q_heads / p.kv_heads);
-  int dkv_parts = k_blocks * p.kv_heads <= two_parts_up_to && longest_chain >= 64 ? 2 : 1;
-  // ARENO_BACKWARD_PARTS=1|2 (read at every launch) fixes the choice: the same dK and dV up to the order of one last
-  // sum, so this is for tests of the kernel a launch of the test's size would not take, and for timing
+  int dkv_parts = 1;
+  if (longest_chain >= 64) {
+    if (pairs32 <= kBmComputeUnits * 5 / 4) {
+      dkv_parts = 4;
+    } else if (blocks64 <= (p.head_dim == 128 ? 4 : 2) * kBmComputeUnits) {
+      dkv_parts = 2;
+    }
+  }
+  // ARENO_BACKWARD_PARTS=1|2|4 (read at every launch) fixes the choice: the same dK and dV up to the order of the
+  // last sums, so this is for tests of the kernels a launch of the test's size would not take, and for timing
   if (const char* e = getenv("ARENO_BACKWARD_PARTS")) {
     if (strcmp(e, "1") == 0) dkv_parts = 1;
     if (strcmp(e, "2") == 0) dkv_parts = 2;
+    if (strcmp(e, "4") == 0) dkv_parts = 4;
   }
   bm_fn dq;
   DkvLaunch dkv;
@@ -643,7 +685,9 @@ int launch_attention_backward_mfma(const BwdParams& p, void* stream) {
     if (int rc = check_launch(op)) return rc;
   }
   if (k_blocks > 0) {
-    hipLaunchKernelGGL(dkv.fn, dim3(static_cast<unsigned>(k_blocks * p.kv_heads)), dim3(dkv.threads), dkv.lds_bytes, s, p);
+    const int64_t blocks = (p.k_tokens + dkv.key_rows - 1) / dkv.key_rows;
+    const int64_t groups = dkv_parts == 4 ? (blocks + 1) / 2 : blocks;  // (pairs with four parts, see above)
+    hipLaunchKernelGGL(dkv.fn, dim3(static_cast<unsigned>(groups * p.kv_heads)), dim3(dkv.threads), dkv.lds_bytes, s, p);
     if (int rc = check_launch(op)) return rc;
   }
   return ARENO_OK;
