@@ -75,8 +75,8 @@ __device__ __forceinline__ int64_t block_in_cost_order(int64_t i, int64_t blocks
 // A tile of 32 rows x D 16-bit elements in LDS, row stride D * 2 + 16 bytes: the row operands (16 lanes read the same
 // 16-byte chunk of 16 rows) meet every bank once, the transposed ones (32 lanes read 32 bytes of 8 consecutive rows)
 // meet every bank twice.  (A layout without any bank conflict -- rows back to back, the chunks of a row permuted by
-// a function of the row -- was measured: LDS is busy 40 % less with it and no launch got faster, small ones 3-8 %
-// slower from the address registers it takes.)  Staging: every thread moves kChunks 16-byte chunks of a tensor
+// a function of the row -- was measured, with four and with eight waves on a compute unit's LDS: LDS is busy 40 %
+// less with it and no launch got faster, small ones 3-8 % slower from the address registers it takes.)  Staging: every thread moves kChunks 16-byte chunks of a tensor
 // through registers.
 template <int D>
 struct BmTile {
