@@ -9,17 +9,20 @@
 //                dQ^T += K^T . dS^T  with the lane's own dS^T values as the B operand and K^T read transposed from the
 //                same LDS tile.  A row's softmax reference moves as in the forward (the accumulator is rescaled), so
 //                one pass over the keys gives dQ, the row's log-sum-exp and dO . O (left in the workspace).
-//   dkv kernel   a workgroup owns 64 packed key rows of one kv head and streams, for every q head of the group, the
-//                query rows that may see them in tiles of 32 (Q and dO tiles in LDS, the rows' statistics next to
-//                them):  S = Q . K^T,  dP = dO . V^T,  P = exp2(S - lse),  dS = P * (dP - dO . O),
-//                dV^T += dO^T . P  and  dK^T += Q^T . dS.  Every gradient element has one owner.
+//   dkv kernel   a workgroup owns 64 or 32 packed key rows of one kv head (16 per wave) and streams, for every q head
+//                of the group, the query rows that may see them in tiles of 32 (Q and dO tiles in LDS, the rows'
+//                statistics next to them):  S = Q . K^T,  dP = dO . V^T,  P = exp2(S - lse),  dS = P * (dP - dO . O),
+//                dV^T += dO^T . P  and  dK^T += Q^T . dS.  Every gradient element has one owner; in a small launch
+//                the stream of tiles is split over two or four sets of waves whose sums are added in a fixed order.
+// Both launches take their blocks in an order (or in pairs) that lets their workgroups end together: see
+// block_in_cost_order and the dkv kernel.
 //
 // The streamed index of a tile (keys in the dq kernel, queries in the dkv kernel) is the contraction index of the
 // second pair of products; a 16 x 16 product leaves element 4 g + j of that index in lane group g, which is exactly
 // how the next product wants its B operand, and the A operand comes from the LDS tile through transposing reads
 // (ds_read_b64_tr_b16), so nothing is shuffled between the products.
 // Geometry as in attention_backward.hip: sequence s has queries [cu_q[s], cu_q[s+1]) at positions ctx[s] + i and keys
-// [cu_k[s], cu_k[s+1]) at positions 0 ..; a query at position t sees keys max(0, t - window) .. t.  A block of 64
+// [cu_k[s], cu_k[s+1]) at positions 0 ..; a query at position t sees keys max(0, t - window) .. t.  A block of
 // packed rows may hold rows of several sequences; it goes through them one after the other, the rows of the others
 // masked.
 
