@@ -128,12 +128,17 @@ __device__ __forceinline__ float operand_element(uint32_t word, int hi) {
 }
 
 // ---- dQ (and the rows' statistics) ------------------------------------------------------------------------------------
-template <int KIND, int D>
+// CB = blocks of 16 query rows a wave owns: 1 (a workgroup of four waves owns 64 packed rows) or 2 (128 rows).  With
+// two, every operand read from the LDS tile serves two products (the tile's K and V rows in the first pair, K^T in
+// the second), at twice the registers for the rows' operands and sums.
+template <int KIND, int D, int CB>
 __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p) {
   using Ops = MfmaOps<KIND>;
   using V8 = typename Ops::vec8;
   using T = BmTile<D>;
   constexpr int NS = D / 32, NB = D / 16;
+  constexpr int kRows = kBmRows * CB;  // packed rows of the workgroup
+  constexpr int kWaveRows = 16 * CB;
   __shared__ __attribute__((aligned(16))) char s_k[kBmTile * T::RS];
   __shared__ __attribute__((aligned(16))) char s_v[kBmTile * T::RS];
 
@@ -144,10 +149,13 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
   // workgroups in launch order: the heads of a block next to each other, the blocks by cost
   const int h = static_cast<int>(blockIdx.x % static_cast<unsigned>(p.q_heads));
   const int kvh = h / (p.q_heads / p.kv_heads);
-  const int64_t q_blocks = (p.q_tokens + kBmRows - 1) / kBmRows;
-  const int64_t r0 = block_in_cost_order(blockIdx.x / static_cast<unsigned>(p.q_heads), q_blocks, p.num_seqs, true) * kBmRows;
-  const int64_t block_end = r0 + kBmRows < p.q_tokens ? r0 + kBmRows : p.q_tokens;
-  const int64_t row = r0 + 16 * wave + lr;  // this lane's query row (a column of the products)
+  const int64_t q_blocks = (p.q_tokens + kRows - 1) / kRows;
+  const int64_t r0 = block_in_cost_order(blockIdx.x / static_cast<unsigned>(p.q_heads), q_blocks, p.num_seqs, true) * kRows;
+  const int64_t block_end = r0 + kRows < p.q_tokens ? r0 + kRows : p.q_tokens;
+  const int64_t wave_row0 = r0 + kWaveRows * wave;
+  int64_t row[CB];  // this lane's query rows (columns of the products)
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) row[cb] = wave_row0 + 16 * cb + lr;
 
   for (int s = seq_of_row(p.cu_q, p.num_seqs, r0); s < p.num_seqs; ++s) {
     const int64_t sq0 = p.cu_q[s], sq1 = p.cu_q[s + 1];
@@ -157,43 +165,56 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
     const int ctx = p.ctx != nullptr ? p.ctx[s] : 0;
     const int64_t k_base = p.cu_k[s];
     const int n_k = p.cu_k[s + 1] - p.cu_k[s];
-    const bool live = row >= q_lo && row < q_hi;
-    const int pos = live ? ctx + static_cast<int>(row - sq0) : -1;
-    const uint64_t live_lanes = __builtin_amdgcn_ballot_w64(live);
-    const bool wave_live = live_lanes != 0, wave_full = live_lanes == ~0ull;
-    // (the positions of the wave's 16 query rows, when all of them belong to this sequence)
-    const int wave_pos_lo = ctx + static_cast<int>(r0 + 16 * wave - sq0), wave_pos_hi = wave_pos_lo + 15;
+    bool live[CB];
+    int pos[CB];
+    bool wave_live = false, wave_full = true;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+      live[cb] = row[cb] >= q_lo && row[cb] < q_hi;
+      pos[cb] = live[cb] ? ctx + static_cast<int>(row[cb] - sq0) : -1;
+      const uint64_t live_lanes = __builtin_amdgcn_ballot_w64(live[cb]);
+      wave_live = wave_live || live_lanes != 0;
+      wave_full = wave_full && live_lanes == ~0ull;
+    }
+    // (the positions of the wave's query rows, when all of them belong to this sequence)
+    const int wave_pos_lo = ctx + static_cast<int>(wave_row0 - sq0), wave_pos_hi = wave_pos_lo + kWaveRows - 1;
     const int pos_min = ctx + static_cast<int>(q_lo - sq0), pos_max = ctx + static_cast<int>(q_hi - 1 - sq0);
     const int key_lo = p.window_left >= 0 ? (pos_min - p.window_left > 0 ? pos_min - p.window_left : 0) : 0;
     const int key_hi = pos_max < n_k - 1 ? pos_max : n_k - 1;
 
-    // this lane's parts of its row of Q and dO (B operands), and dO . O
-    const int64_t row_elem = (row * p.q_heads + h) * D;
-    V8 qop[NS], gop[NS];
-    float delta = 0.0f;
+    // this lane's parts of its rows of Q and dO (B operands), and dO . O
+    int64_t row_elem[CB];
+    V8 qop[CB][NS], gop[CB][NS];
+    float delta[CB];
+    float4_t acc[CB][NB];
+    float m_run[CB], l_lane[CB];
 #pragma unroll
-    for (int sl = 0; sl < NS; ++sl) {
-      uint4_t qw = {0u, 0u, 0u, 0u}, gw = qw, ow = qw;
-      if (live) {
-        const int64_t off = (row_elem + (D / 4) * lk + 8 * sl) * 2;
-        qw = load16(p.q, off);
-        gw = load16(p.grad_out, off);
-        ow = load16(p.out, off);
-      }
-      qop[sl] = __builtin_bit_cast(V8, qw);
-      gop[sl] = __builtin_bit_cast(V8, gw);
+    for (int cb = 0; cb < CB; ++cb) {
+      row_elem[cb] = (row[cb] * p.q_heads + h) * D;
+      float d = 0.0f;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        delta += operand_element<KIND>(gw[j], 0) * operand_element<KIND>(ow[j], 0) +
-                 operand_element<KIND>(gw[j], 1) * operand_element<KIND>(ow[j], 1);
+      for (int sl = 0; sl < NS; ++sl) {
+        uint4_t qw = {0u, 0u, 0u, 0u}, gw = qw, ow = qw;
+        if (live[cb]) {
+          const int64_t off = (row_elem[cb] + (D / 4) * lk + 8 * sl) * 2;
+          qw = load16(p.q, off);
+          gw = load16(p.grad_out, off);
+          ow = load16(p.out, off);
+        }
+        qop[cb][sl] = __builtin_bit_cast(V8, qw);
+        gop[cb][sl] = __builtin_bit_cast(V8, gw);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          d += operand_element<KIND>(gw[j], 0) * operand_element<KIND>(ow[j], 0) +
+               operand_element<KIND>(gw[j], 1) * operand_element<KIND>(ow[j], 1);
+        }
       }
+      delta[cb] = rows_sum(d);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) acc[cb][nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      m_run[cb] = kBmNegInf;
+      l_lane[cb] = 0.0f;
     }
-    delta = rows_sum(delta);
-
-    float4_t acc[NB];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) acc[nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    float m_run = kBmNegInf, l_lane = 0.0f;
 
     if (key_hi >= key_lo) {  // (the same for the whole workgroup)
       const int t0 = key_lo / kBmTile, t1 = key_hi / kBmTile;
@@ -225,25 +246,36 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
       for (int t = t0; t <= t1; ++t) {
         if (t < t1) fetch(t + 1);
         if (wave_live) {
-          float sc[2][4], dp[2][4];
+          float sc[CB][2][4], dp[CB][2][4];
           auto first_products = [&](auto masked) {
 #pragma unroll
             for (int tg = 0; tg < 2; ++tg) {
-              float4_t c1 = {0.0f, 0.0f, 0.0f, 0.0f}, c2 = c1;
+              float4_t c1[CB], c2[CB];
+#pragma unroll
+              for (int cb = 0; cb < CB; ++cb) c1[cb] = c2[cb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
               for (int sl = 0; sl < NS; ++sl) {
-                c1 = Ops::mfma(tile_row_operand<KIND, T, D>(s_k, tg, sl, lr, lk), qop[sl], c1);
-                c2 = Ops::mfma(tile_row_operand<KIND, T, D>(s_v, tg, sl, lr, lk), gop[sl], c2);
+                const V8 k_rows = tile_row_operand<KIND, T, D>(s_k, tg, sl, lr, lk);
+                const V8 v_rows = tile_row_operand<KIND, T, D>(s_v, tg, sl, lr, lk);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                  c1[cb] = Ops::mfma(k_rows, qop[cb][sl], c1[cb]);
+                  c2[cb] = Ops::mfma(v_rows, gop[cb][sl], c2[cb]);
+                }
               }
 #pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                sc[tg][j] = c1[j];  // (the softmax scale goes in with the reference, below)
-                if constexpr (decltype(masked)::value) {
-                  const int key = kBmTile * t + 16 * tg + 4 * lk + j;
-                  const bool ok = key <= pos && key < n_k && (p.window_left < 0 || key >= pos - p.window_left);
-                  sc[tg][j] = ok ? sc[tg][j] : kBmNegInf;
+              for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                  sc[cb][tg][j] = c1[cb][j];  // (the softmax scale goes in with the reference, below)
+                  if constexpr (decltype(masked)::value) {
+                    const int key = kBmTile * t + 16 * tg + 4 * lk + j;
+                    const bool ok =
+                        key <= pos[cb] && key < n_k && (p.window_left < 0 || key >= pos[cb] - p.window_left);
+                    sc[cb][tg][j] = ok ? sc[cb][tg][j] : kBmNegInf;
+                  }
+                  dp[cb][tg][j] = c2[cb][j];
                 }
-                dp[tg][j] = c2[j];
               }
             }
           };
@@ -257,39 +289,52 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
           } else {
             first_products(std::true_type{});
           }
-          float mt = sc[0][0];
+          V8 dsop[CB];
+          bool moved = false;
+          float alpha[CB];
 #pragma unroll
-          for (int tg = 0; tg < 2; ++tg) {
+          for (int cb = 0; cb < CB; ++cb) {
+            float mt = sc[cb][0][0];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) mt = fmaxf(mt, sc[tg][j]);
-          }
-          mt = rows_max(mt);
-          const float m_new = fmaxf(m_run, mt * p.scale_log2e);  // (the scale is positive)
-          const float m_ref = m_new == kBmNegInf ? 0.0f : m_new;
-          const float alpha = fast_exp2(m_run - m_ref);  // 0 while the row has seen no key
-          m_run = m_new;
-          float ds[2][4], psum = 0.0f;
+            for (int tg = 0; tg < 2; ++tg) {
 #pragma unroll
-          for (int tg = 0; tg < 2; ++tg) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const float pe = fast_exp2(__builtin_fmaf(sc[tg][j], p.scale_log2e, -m_ref));  // exp2(-inf) = 0: masked keys
-              psum += pe;
-              ds[tg][j] = pe * (dp[tg][j] - delta);
+              for (int j = 0; j < 4; ++j) mt = fmaxf(mt, sc[cb][tg][j]);
             }
+            mt = rows_max(mt);
+            const float m_new = fmaxf(m_run[cb], mt * p.scale_log2e);  // (the scale is positive)
+            const float m_ref = m_new == kBmNegInf ? 0.0f : m_new;
+            alpha[cb] = fast_exp2(m_run[cb] - m_ref);  // 0 while the row has seen no key
+            m_run[cb] = m_new;
+            float ds[2][4], psum = 0.0f;
+#pragma unroll
+            for (int tg = 0; tg < 2; ++tg) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                // (exp2(-inf) = 0: masked keys)
+                const float pe = fast_exp2(__builtin_fmaf(sc[cb][tg][j], p.scale_log2e, -m_ref));
+                psum += pe;
+                ds[tg][j] = pe * (dp[cb][tg][j] - delta[cb]);
+              }
+            }
+            l_lane[cb] = l_lane[cb] * alpha[cb] + psum;
+            dsop[cb] = streamed_operand<KIND>(ds);
+            moved = moved || __builtin_amdgcn_ballot_w64(alpha[cb] != 1.0f) != 0;
           }
-          l_lane = l_lane * alpha + psum;
-          const V8 dsop = streamed_operand<KIND>(ds);
-          if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {  // (after the first tiles a new maximum is rare)
+          if (moved) {  // (after the first tiles a new maximum is rare)
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
+            for (int cb = 0; cb < CB; ++cb) {
 #pragma unroll
-              for (int j = 0; j < 4; ++j) acc[nb][j] *= alpha;
+              for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[cb][nb][j] *= alpha[cb];
+              }
             }
           }
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) {
-            acc[nb] = Ops::mfma(tile_transposed_operand<KIND, T>(s_k, nb, lr, lk), dsop, acc[nb]);
+            const V8 k_cols = tile_transposed_operand<KIND, T>(s_k, nb, lr, lk);
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) acc[cb][nb] = Ops::mfma(k_cols, dsop[cb], acc[cb][nb]);
           }
         }
         __syncthreads();  // every wave has read tile t
@@ -299,19 +344,23 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
     }
 
     // dQ = scale / l * sum_k p_k (dP_k - dO . O) K_k; the row's log-sum-exp (log2 domain) and dO . O for the dkv kernel
-    const float l_tot = rows_sum(l_lane);
-    if (live) {
-      const float f = l_tot > 0.0f ? p.scale / l_tot : 0.0f;
-      float* dst = p.grad_q + row_elem + 4 * lk;
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        *reinterpret_cast<float4_t*>(dst + 16 * nb) = float4_t{acc[nb][0] * f, acc[nb][1] * f, acc[nb][2] * f, acc[nb][3] * f};
-      }
-      if (lk == 0) {
-        float* st = p.row_stats + (row * p.q_heads + h) * 2;
-        // a row without visible keys gets a reference no score reaches: its probabilities come out as zeros
-        st[0] = l_tot > 0.0f ? m_run + __builtin_log2f(l_tot) : __builtin_huge_valf();
-        st[1] = delta;
+    for (int cb = 0; cb < CB; ++cb) {
+      const float l_tot = rows_sum(l_lane[cb]);
+      if (live[cb]) {
+        const float f = l_tot > 0.0f ? p.scale / l_tot : 0.0f;
+        float* dst = p.grad_q + row_elem[cb] + 4 * lk;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          *reinterpret_cast<float4_t*>(dst + 16 * nb) =
+              float4_t{acc[cb][nb][0] * f, acc[cb][nb][1] * f, acc[cb][nb][2] * f, acc[cb][nb][3] * f};
+        }
+        if (lk == 0) {
+          float* st = p.row_stats + (row[cb] * p.q_heads + h) * 2;
+          // a row without visible keys gets a reference no score reaches: its probabilities come out as zeros
+          st[0] = l_tot > 0.0f ? m_run[cb] + __builtin_log2f(l_tot) : __builtin_huge_valf();
+          st[1] = delta[cb];
+        }
       }
     }
   }
@@ -671,20 +720,33 @@ int launch_attention_backward_mfma(const BwdParams& p, void* stream) {
     if (strcmp(e, "2") == 0) dkv_parts = 2;
     if (strcmp(e, "4") == 0) dkv_parts = 4;
   }
+  // The dq kernel with 32 rows per wave at head dim 128 once the launch has 8 workgroups of 64 rows per compute unit:
+  // half the LDS reads per product (4 x 4 096 tokens, 32 / 8 heads: both launches 2 970 -> 2 760 us; 4 x 2 048
+  // tokens, 28 / 4 heads: 834 -> 807 us), but half the workgroups and two waves per SIMD instead of three, which
+  // costs small launches (8 x 512 tokens: +4 %) and head dim 64 (four waves per SIMD down to two: +5 %).
+  // ARENO_BACKWARD_DQ_ROWS=16|32 (read at every launch) fixes the choice, for tests and timing.
+  int dq_cb = p.head_dim == 128 && q_blocks * p.q_heads >= 8 * kBmComputeUnits ? 2 : 1;
+  if (const char* e = getenv("ARENO_BACKWARD_DQ_ROWS")) {
+    if (strcmp(e, "32") == 0) dq_cb = 2;
+    if (strcmp(e, "16") == 0) dq_cb = 1;
+  }
+  const int64_t dq_blocks = (p.q_tokens + kBmRows * dq_cb - 1) / (kBmRows * dq_cb);
   bm_fn dq;
   DkvLaunch dkv;
   if (p.head_dim == 64) {
-    dq = bf16 ? bwd_mfma_dq_kernel<KV_BF16, 64> : bwd_mfma_dq_kernel<KV_F16, 64>;
+    dq = dq_cb == 2 ? (bf16 ? bwd_mfma_dq_kernel<KV_BF16, 64, 2> : bwd_mfma_dq_kernel<KV_F16, 64, 2>)
+                    : (bf16 ? bwd_mfma_dq_kernel<KV_BF16, 64, 1> : bwd_mfma_dq_kernel<KV_F16, 64, 1>);
     dkv = bf16 ? dkv_launch<KV_BF16, 64>(dkv_parts) : dkv_launch<KV_F16, 64>(dkv_parts);
   } else {
-    dq = bf16 ? bwd_mfma_dq_kernel<KV_BF16, 128> : bwd_mfma_dq_kernel<KV_F16, 128>;
+    dq = dq_cb == 2 ? (bf16 ? bwd_mfma_dq_kernel<KV_BF16, 128, 2> : bwd_mfma_dq_kernel<KV_F16, 128, 2>)
+                    : (bf16 ? bwd_mfma_dq_kernel<KV_BF16, 128, 1> : bwd_mfma_dq_kernel<KV_F16, 128, 1>);
     dkv = bf16 ? dkv_launch<KV_BF16, 128>(dkv_parts) : dkv_launch<KV_F16, 128>(dkv_parts);
   }
   const char* op = "areno_hip_attention_backward";
   if (dkv.fn == nullptr) return fail(ARENO_ERR_LAUNCH, "%s: the dkv kernel's LDS size was refused", op);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (q_blocks > 0) {
-    hipLaunchKernelGGL(dq, dim3(static_cast<unsigned>(q_blocks * p.q_heads)), dim3(kBmThreads), 0, s, p);
+    hipLaunchKernelGGL(dq, dim3(static_cast<unsigned>(dq_blocks * p.q_heads)), dim3(kBmThreads), 0, s, p);
     if (int rc = check_launch(op)) return rc;
   }
   if (k_blocks > 0) {

@@ -52,10 +52,10 @@ def test_varlen_backward(dtype, window_left, hq, hkv, d):
 
 
 @pytest.mark.parametrize("last", [129, 161])
-@pytest.mark.parametrize("parts", ["1", "2", "4"])
+@pytest.mark.parametrize("parts,dq_rows", [("1", "16"), ("2", "32"), ("4", "16"), ("4", "32")])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("hq,hkv,d,window_left", [(8, 2, 128, None), (4, 4, 64, None), (6, 1, 64, 40), (4, 2, 128, 200), (2, 1, 128, 0)])
-def test_varlen_backward_long_sequences_on_the_matrix_core_kernels(dtype, hq, hkv, d, window_left, parts, last, monkeypatch):
+def test_varlen_backward_long_sequences_on_the_matrix_core_kernels(dtype, hq, hkv, d, window_left, parts, dq_rows, last, monkeypatch):
     """16-bit inputs at head dims 64 / 128 take the matrix-core backward: sequences longer than its blocks of 64 rows
     and tiles of 32, blocks that hold several sequences (and empty ones), query groups, windows shorter and longer
     than a tile.  The dkv kernel in each of its shapes: key blocks of 64 rows with the stream of query tiles in one
@@ -64,6 +64,7 @@ def test_varlen_backward_long_sequences_on_the_matrix_core_kernels(dtype, hq, hk
     even (1 327 tokens: every block has a partner in the four-part shape's pairs) or odd (1 359: the middle one has
     none)."""
     monkeypatch.setenv("ARENO_BACKWARD_PARTS", parts)
+    monkeypatch.setenv("ARENO_BACKWARD_DQ_ROWS", dq_rows)  # the dq kernel with 16 and with 32 query rows per wave
     g = torch.Generator().manual_seed(hq * 31 + d)
     lens = [300, 1, 0, 700, 5, 63, 64, 65, last]
     t = sum(lens)
