@@ -2,8 +2,8 @@
 // 128.  Same contract as the vector-ALU kernels of attention_backward.hip (fp32 dQ, dK, dV from dO, Q, K, V and the
 // saved output; areno/accel/csrc/attention.cu:244-524 in the reference), same two launches, no atomics:
 //
-//   dq kernel    a workgroup owns 64 packed query rows of one q head (four waves of 16 rows) and streams the keys its
-//                rows may see in tiles of 32 through LDS.  Per tile, with the keys as the rows of the products (the
+//   dq kernel    a workgroup owns 64 or 128 packed query rows of one q head (four waves of 16 or 32 rows) and streams
+//                the keys its rows may see in tiles of 32 through LDS.  Per tile, with the keys as the rows of the products (the
 //                layout of the forward kernel):  S^T = K . Q^T  and  dP^T = V . dO^T  (two products per 16 keys and 32
 //                elements of the head), the online softmax of the forward on S^T, dS^T = P^T * (dP^T - dO . O), and
 //                dQ^T += K^T . dS^T  with the lane's own dS^T values as the B operand and K^T read transposed from the
