@@ -858,6 +858,8 @@ def main() -> int:
     if not args.only and not args.skip_other_shapes:
         results["other_shapes"] = measure_other_shapes(dev)
         results["varlen_backward"] = measure_backward(dev)
+        # (a launch that fills the compute units many times over: the kernels' shapes for large launches)
+        results["varlen_backward_4x4096"] = measure_backward(dev, seqs=4, new=4096, hq=32, hkv=8, iters=5)
 
     head = results[names[0]]
     dtype = {"cfg1": "bf16", "cfg2": "int8", "cfg3": "fp8", "cfg4": "fp8", "cfg2_b256": "int8"}[names[0]]
