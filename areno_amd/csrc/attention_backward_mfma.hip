@@ -426,337 +426,6 @@ __global__ __launch_bounds__((DkvShape<D, KR, P>::kThreads), (DkvShape<D, KR, P>
   const int64_t first_block = paired ? wg : block_in_cost_order(wg, k_blocks, p.num_seqs, false);
 
   for (int half = 0; half < 2; ++half) {
-    const int row = 16 * half + 4 * lk + (lr >> 2);
-    char* a = tile + T::chunk_pos(row, 2 * nb + ((lr & 3) >> 1)) + 8 * (lr & 1);
-    const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)a);
-    const uint2_t u = __builtin_bit_cast(uint2_t, r);
-    w[2 * half] = u[0];
-    w[2 * half + 1] = u[1];
-  }
-  return __builtin_bit_cast(V8, uint4_t{w[0], w[1], w[2], w[3]});
-}
-// eight values of the streamed index, as a lane holds them after the first pair of products ([tg][j]), as B operand
-template <int KIND>
-__device__ __forceinline__ typename MfmaOps<KIND>::vec8 streamed_operand(const float (&x)[2][4]) {
-  using V8 = typename MfmaOps<KIND>::vec8;
-  return __builtin_bit_cast(V8, uint4_t{pack_pair<KIND>(x[0][0], x[0][1]), pack_pair<KIND>(x[0][2], x[0][3]),
-                                        pack_pair<KIND>(x[1][0], x[1][1]), pack_pair<KIND>(x[1][2], x[1][3])});
-}
-template <int KIND>
-__device__ __forceinline__ float operand_element(uint32_t word, int hi) {
-  const uint32_t bits = hi ? word >> 16 : word & 0xffffu;
-  return KIND == KV_BF16 ? bf16_bits_to_float(bits) : f16_bits_to_float(bits);
-}
-
-// ---- dQ (and the rows' statistics) ------------------------------------------------------------------------------------
-// CB = blocks of 16 query rows a wave owns: 1 (a workgroup of four waves owns 64 packed rows) or 2 (128 rows).  With
-// two, every operand read from the LDS tile serves two products (the tile's K and V rows in the first pair, K^T in
-// the second), at twice the registers for the rows' operands and sums.
-template <int KIND, int D, int CB>
-__global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p) {
-  using Ops = MfmaOps<KIND>;
-  using V8 = typename Ops::vec8;
-  using T = BmTile<D>;
-  constexpr int NS = D / 32, NB = D / 16;
-  constexpr int kRows = kBmRows * CB;  // packed rows of the workgroup
-  constexpr int kWaveRows = 16 * CB;
-  __shared__ __attribute__((aligned(16))) char s_k[kBmTile * T::RS];
-  __shared__ __attribute__((aligned(16))) char s_v[kBmTile * T::RS];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & (kWave - 1);
-  const int wave = uniform(tid >> 6);  // (in a scalar register: what follows from it is scalar work and scalar branches)
-  const int lr = lane & 15, lk = lane >> 4;
-  // workgroups in launch order: the heads of a block next to each other, the blocks by cost
-  const int h = static_cast<int>(blockIdx.x % static_cast<unsigned>(p.q_heads));
-  const int kvh = h / (p.q_heads / p.kv_heads);
-  const int64_t q_blocks = (p.q_tokens + kRows - 1) / kRows;
-  const int64_t r0 = block_in_cost_order(blockIdx.x / static_cast<unsigned>(p.q_heads), q_blocks, p.num_seqs, true) * kRows;
-  const int64_t block_end = r0 + kRows < p.q_tokens ? r0 + kRows : p.q_tokens;
-  const int64_t wave_row0 = r0 + kWaveRows * wave;
-  int64_t row[CB];  // this lane's query rows (columns of the products)
-#pragma unroll
-  for (int cb = 0; cb < CB; ++cb) row[cb] = wave_row0 + 16 * cb + lr;
-
-  for (int s = seq_of_row(p.cu_q, p.num_seqs, r0); s < p.num_seqs; ++s) {
-    const int64_t sq0 = p.cu_q[s], sq1 = p.cu_q[s + 1];
-    if (sq0 >= block_end) break;
-    const int64_t q_lo = sq0 > r0 ? sq0 : r0, q_hi = sq1 < block_end ? sq1 : block_end;
-    if (q_lo >= q_hi) continue;
-    const int ctx = p.ctx != nullptr ? p.ctx[s] : 0;
-    const int64_t k_base = p.cu_k[s];
-    const int n_k = p.cu_k[s + 1] - p.cu_k[s];
-    bool live[CB];
-    int pos[CB];
-    bool wave_live = false, wave_full = true;
-#pragma unroll
-    for (int cb = 0; cb < CB; ++cb) {
-      live[cb] = row[cb] >= q_lo && row[cb] < q_hi;
-      pos[cb] = live[cb] ? ctx + static_cast<int>(row[cb] - sq0) : -1;
-      const uint64_t live_lanes = __builtin_amdgcn_ballot_w64(live[cb]);
-      wave_live = wave_live || live_lanes != 0;
-      wave_full = wave_full && live_lanes == ~0ull;
-    }
-    // (the positions of the wave's query rows, when all of them belong to this sequence)
-    const int wave_pos_lo = ctx + static_cast<int>(wave_row0 - sq0), wave_pos_hi = wave_pos_lo + kWaveRows - 1;
-    const int pos_min = ctx + static_cast<int>(q_lo - sq0), pos_max = ctx + static_cast<int>(q_hi - 1 - sq0);
-    const int key_lo = p.window_left >= 0 ? (pos_min - p.window_left > 0 ? pos_min - p.window_left : 0) : 0;
-    const int key_hi = pos_max < n_k - 1 ? pos_max : n_k - 1;
-
-    // this lane's parts of its rows of Q and dO (B operands), and dO . O
-    int64_t row_elem[CB];
-    V8 qop[CB][NS], gop[CB][NS];
-    float delta[CB];
-    float4_t acc[CB][NB];
-    float m_run[CB], l_lane[CB];
-#pragma unroll
-    for (int cb = 0; cb < CB; ++cb) {
-      row_elem[cb] = (row[cb] * p.q_heads + h) * D;
-      float d = 0.0f;
-#pragma unroll
-      for (int sl = 0; sl < NS; ++sl) {
-        uint4_t qw = {0u, 0u, 0u, 0u}, gw = qw, ow = qw;
-        if (live[cb]) {
-          const int64_t off = (row_elem[cb] + (D / 4) * lk + 8 * sl) * 2;
-          qw = load16(p.q, off);
-          gw = load16(p.grad_out, off);
-          ow = load16(p.out, off);
-        }
-        qop[cb][sl] = __builtin_bit_cast(V8, qw);
-        gop[cb][sl] = __builtin_bit_cast(V8, gw);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          d += operand_element<KIND>(gw[j], 0) * operand_element<KIND>(ow[j], 0) +
-               operand_element<KIND>(gw[j], 1) * operand_element<KIND>(ow[j], 1);
-        }
-      }
-      delta[cb] = rows_sum(d);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) acc[cb][nb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-      m_run[cb] = kBmNegInf;
-      l_lane[cb] = 0.0f;
-    }
-
-    if (key_hi >= key_lo) {  // (the same for the whole workgroup)
-      const int t0 = key_lo / kBmTile, t1 = key_hi / kBmTile;
-      uint4_t kreg[T::kChunks], vreg[T::kChunks];
-      auto fetch = [&](int t) {
-#pragma unroll
-        for (int i = 0; i < T::kChunks; ++i) {
-          const int c = tid + kBmThreads * i;
-          const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
-          const int key = kBmTile * t + r < n_k ? kBmTile * t + r : n_k - 1;  // rows past the end repeat the last key
-          const int64_t off = ((k_base + key) * p.kv_heads + kvh) * (D * 2) + col * 16;
-          kreg[i] = load16(p.k, off);
-          vreg[i] = load16(p.v, off);
-        }
-      };
-      auto publish = [&]() {
-#pragma unroll
-        for (int i = 0; i < T::kChunks; ++i) {
-          const int c = tid + kBmThreads * i;
-          const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
-          *reinterpret_cast<uint4_t*>(s_k + T::chunk_pos(r, col)) = kreg[i];
-          *reinterpret_cast<uint4_t*>(s_v + T::chunk_pos(r, col)) = vreg[i];
-        }
-      };
-      fetch(t0);
-      __syncthreads();  // the tiles' previous readers (an earlier sequence of this block) are done
-      publish();
-      __syncthreads();
-      for (int t = t0; t <= t1; ++t) {
-        if (t < t1) fetch(t + 1);
-        if (wave_live) {
-          float sc[CB][2][4], dp[CB][2][4];
-          auto first_products = [&](auto masked) {
-#pragma unroll
-            for (int tg = 0; tg < 2; ++tg) {
-              float4_t c1[CB], c2[CB];
-#pragma unroll
-              for (int cb = 0; cb < CB; ++cb) c1[cb] = c2[cb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-              for (int sl = 0; sl < NS; ++sl) {
-                const V8 k_rows = tile_row_operand<KIND, T, D>(s_k, tg, sl, lr, lk);
-                const V8 v_rows = tile_row_operand<KIND, T, D>(s_v, tg, sl, lr, lk);
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                  c1[cb] = Ops::mfma(k_rows, qop[cb][sl], c1[cb]);
-                  c2[cb] = Ops::mfma(v_rows, gop[cb][sl], c2[cb]);
-                }
-              }
-#pragma unroll
-              for (int cb = 0; cb < CB; ++cb) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                  sc[cb][tg][j] = c1[cb][j];  // (the softmax scale goes in with the reference, below)
-                  if constexpr (decltype(masked)::value) {
-                    const int key = kBmTile * t + 16 * tg + 4 * lk + j;
-                    const bool ok =
-                        key <= pos[cb] && key < n_k && (p.window_left < 0 || key >= pos[cb] - p.window_left);
-                    sc[cb][tg][j] = ok ? sc[cb][tg][j] : kBmNegInf;
-                  }
-                  dp[cb][tg][j] = c2[cb][j];
-                }
-              }
-            }
-          };
-          // most tiles lie below the diagonal and inside the window as a whole: every query row of this wave sees
-          // every key of the tile, and nothing needs a mask
-          const int key_first = kBmTile * t, key_last = key_first + kBmTile - 1;
-          const bool plain = wave_full && key_last < n_k && key_last <= wave_pos_lo &&
-                             (p.window_left < 0 || key_first >= wave_pos_hi - p.window_left);
-          if (plain) {
-            first_products(std::false_type{});
-          } else {
-            first_products(std::true_type{});
-          }
-          V8 dsop[CB];
-          bool moved = false;
-          float alpha[CB];
-#pragma unroll
-          for (int cb = 0; cb < CB; ++cb) {
-            float mt = sc[cb][0][0];
-#pragma unroll
-            for (int tg = 0; tg < 2; ++tg) {
-#pragma unroll
-              for (int j = 0; j < 4; ++j) mt = fmaxf(mt, sc[cb][tg][j]);
-            }
-            mt = rows_max(mt);
-            const float m_new = fmaxf(m_run[cb], mt * p.scale_log2e);  // (the scale is positive)
-            const float m_ref = m_new == kBmNegInf ? 0.0f : m_new;
-            alpha[cb] = fast_exp2(m_run[cb] - m_ref);  // 0 while the row has seen no key
-            m_run[cb] = m_new;
-            float ds[2][4], psum = 0.0f;
-#pragma unroll
-            for (int tg = 0; tg < 2; ++tg) {
-#pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                // (exp2(-inf) = 0: masked keys)
-                const float pe = fast_exp2(__builtin_fmaf(sc[cb][tg][j], p.scale_log2e, -m_ref));
-                psum += pe;
-                ds[tg][j] = pe * (dp[cb][tg][j] - delta[cb]);
-              }
-            }
-            l_lane[cb] = l_lane[cb] * alpha[cb] + psum;
-            dsop[cb] = streamed_operand<KIND>(ds);
-            moved = moved || __builtin_amdgcn_ballot_w64(alpha[cb] != 1.0f) != 0;
-          }
-          if (moved) {  // (after the first tiles a new maximum is rare)
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) {
-#pragma unroll
-              for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[cb][nb][j] *= alpha[cb];
-              }
-            }
-          }
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) {
-            const V8 k_cols = tile_transposed_operand<KIND, T>(s_k, nb, lr, lk);
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) acc[cb][nb] = Ops::mfma(k_cols, dsop[cb], acc[cb][nb]);
-          }
-        }
-        __syncthreads();  // every wave has read tile t
-        if (t < t1) publish();
-        __syncthreads();
-      }
-    }
-
-    // dQ = scale / l * sum_k p_k (dP_k - dO . O) K_k; the row's log-sum-exp (log2 domain) and dO . O for the dkv kernel
-#pragma unroll
-    for (int cb = 0; cb < CB; ++cb) {
-      const float l_tot = rows_sum(l_lane[cb]);
-      if (live[cb]) {
-        const float f = l_tot > 0.0f ? p.scale / l_tot : 0.0f;
-        float* dst = p.grad_q + row_elem[cb] + 4 * lk;
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          *reinterpret_cast<float4_t*>(dst + 16 * nb) =
-              float4_t{acc[cb][nb][0] * f, acc[cb][nb][1] * f, acc[cb][nb][2] * f, acc[cb][nb][3] * f};
-        }
-        if (lk == 0) {
-          float* st = p.row_stats + (row[cb] * p.q_heads + h) * 2;
-          // a row without visible keys gets a reference no score reaches: its probabilities come out as zeros
-          st[0] = l_tot > 0.0f ? m_run[cb] + __builtin_log2f(l_tot) : __builtin_huge_valf();
-          st[1] = delta[cb];
-        }
-      }
-    }
-  }
-}
-
-// ---- dK, dV -------------------------------------------------------------------------------------------------------------
-// A workgroup owns a block of KR packed key rows of one kv head, or two of them one after the other: block i and
-// block blocks - 1 - i.  A key block early in its sequence is seen by all later queries and one late in it by few.
-// A launch of many workgroups per compute unit evens that out by starting the expensive blocks first
-// (block_in_cost_order); in a launch of about one workgroup per unit nothing comes after the expensive block to
-// fill the gap, and there the pairs help: for sequences of about equal length the costs of such a pair add up to
-// the same for every i, so the workgroups end together.  (The launcher says which by the size of the grid.)
-// The workgroup has P parts of KR / 16 waves.  Every part owns all KR key rows (16 per wave) and takes every P-th
-// step of the stream of query tiles (tiles and statistics of its own in LDS); the sums of parts 1 .. P - 1 go to
-// part 0 through LDS at the end of a block, in a fixed order.  More parts shorten the chain of steps a block is:
-// (KR, P) = (64, 1) four waves, two workgroups per compute unit, for launches that fill the units several times;
-// (64, 2) and (32, 4) eight waves, for launches of about one workgroup per unit.
-template <int D, int KR, int P>
-struct DkvShape {
-  static constexpr int kKeyWaves = KR / 16;
-  static constexpr int kPartThreads = kKeyWaves * kWave;
-  static constexpr int kThreads = kPartThreads * P;
-  static constexpr int RS = BmTile<D>::RS;
-  static constexpr int kChunksPerRow = BmTile<D>::kChunksPerRow;
-  static constexpr int kChunks = kBmTile * kChunksPerRow / kPartThreads;  // 16-byte chunks of a tile per thread of a part
-  static_assert(kBmTile * kChunksPerRow % kPartThreads == 0, "tile chunks");
-  static constexpr int kTile = kBmTile * RS;
-  static constexpr int kStat = kBmTile * 2 * 4;
-  // per part and buffer: a Q tile, a dO tile, the rows' statistics
-  static constexpr int kBuffer = 2 * kTile + kStat;
-  static constexpr int kStream = P * 2 * kBuffer;
-  static constexpr int kSums = (P - 1) * kPartThreads * (D / 16) * 2 * 16;  // a float4 per lane, block of 16 and tensor
-  static constexpr int kLdsBytes = kStream > kSums ? kStream : kSums;
-};
-extern __shared__ __attribute__((aligned(16))) char bm_dkv_lds[];
-
-template <int KIND, int D, int KR, int P>
-__global__ __launch_bounds__((DkvShape<D, KR, P>::kThreads), (DkvShape<D, KR, P>::kThreads == 256 ? 2 : 1)) void bwd_mfma_dkv_kernel(
-    BwdParams p) {
-  using Ops = MfmaOps<KIND>;
-  using V8 = typename Ops::vec8;
-  using T = BmTile<D>;
-  using L = DkvShape<D, KR, P>;
-  constexpr int NS = D / 32, NB = D / 16;
-
-  // (the same for a wave, and told so: the part's steps, cursors and loop counts then live in scalar registers)
-  const int part = P > 1 ? uniform(static_cast<int>(threadIdx.x) / L::kPartThreads) : 0;
-  const int tid = P > 1 ? static_cast<int>(threadIdx.x) % L::kPartThreads : static_cast<int>(threadIdx.x);  // in the part
-  char* const lds = bm_dkv_lds + part * (2 * L::kBuffer);
-  auto s_q = [&](int buf) { return lds + buf * L::kBuffer; };
-  auto s_g = [&](int buf) { return lds + buf * L::kBuffer + L::kTile; };
-  auto s_stat = [&](int buf) { return reinterpret_cast<float*>(lds + buf * L::kBuffer + 2 * L::kTile); };  // [row][2]
-
-  const int lane = tid & (kWave - 1);
-  const int wave = uniform(tid >> 6);
-  const int lr = lane & 15, lk = lane >> 4;
-  const int kvh = static_cast<int>(blockIdx.x % static_cast<unsigned>(p.kv_heads));
-  const int group = p.q_heads / p.kv_heads;
-  const int64_t k_blocks = (p.k_tokens + KR - 1) / KR;
-  const int64_t wg = blockIdx.x / static_cast<unsigned>(p.kv_heads);
-  // (launched with a workgroup per pair of blocks, or with one per block: then in cost order, one block each)
-  const bool paired = gridDim.x / static_cast<unsigned>(p.kv_heads) < k_blocks;
-  const int64_t first_block = paired ? wg : block_in_cost_order(wg, k_blocks, p.num_seqs, false);
-
-  // byte offsets of this thread's chunks inside a tile of 32 query rows of Q / dO, and of its row's statistics
-  uint32_t chunk_offset[L::kChunks];
-#pragma unroll
-  for (int i = 0; i < L::kChunks; ++i) {
-    const int c = tid + L::kPartThreads * i;
-    const int r = c / T::kChunksPerRow, col = c % T::kChunksPerRow;
-    chunk_offset[i] = static_cast<uint32_t>(r) * static_cast<uint32_t>(p.q_heads) * (D * 2) + col * 16;
-  }
-  const uint32_t stat_offset = static_cast<uint32_t>(tid & (kBmTile - 1)) * static_cast<uint32_t>(p.q_heads) * 2;
-
-  for (int half = 0; half < 2; ++half) {
     const int64_t block = half == 0 ? first_block : k_blocks - 1 - first_block;
     // (no second block without pairs, and none for the middle one of an odd number of blocks)
     if (half == 1 && (!paired || block <= first_block)) break;
