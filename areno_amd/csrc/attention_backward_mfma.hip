@@ -33,6 +33,7 @@
 #include <type_traits>
 
 #include "attention_backward.hpp"
+#include "backward_order.hpp"
 #include "decode_mfma_kernels.hpp"
 
 namespace areno {
@@ -56,23 +57,6 @@ __device__ __forceinline__ int seq_of_row(const int32_t* cu, int num_seqs, int64
     }
   }
   return lo;
-}
-
-// The block of 64 packed rows the i-th workgroup (of a head) takes.  Blocks differ in cost by their place in their
-// sequence (a query block late in a long sequence sees the most keys, a key block early in it is seen by the most
-// queries), and a launch ends soonest when the expensive blocks start first.  The lengths are not known on the host,
-// so the order assumes sequences of about equal length: the packed blocks are cut into num_seqs runs and taken run by
-// run in turn, the expensive end of every run first (`from_end`: the last block of a run).  Any order is correct.
-__device__ __forceinline__ int64_t block_in_cost_order(int64_t i, int64_t blocks, int num_seqs, bool from_end) {
-  const int64_t runs = num_seqs > 0 ? num_seqs : 1, per = blocks / runs, rest = blocks - per * runs;
-  if (per == 0) return from_end ? blocks - 1 - i : i;
-  if (from_end) {  // the blocks behind the last whole run belong to the end of the last sequence: first
-    if (i < rest) return blocks - 1 - i;
-    const int64_t j = i - rest;
-    return (j % runs) * per + (per - 1 - j / runs);
-  }
-  if (i >= per * runs) return i;
-  return (i % runs) * per + i / runs;
 }
 
 // A tile of 32 rows x D 16-bit elements in LDS, row stride D * 2 + 16 bytes: the row operands (16 lanes read the same
