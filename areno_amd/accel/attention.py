@@ -94,9 +94,11 @@ class _VarlenCausalAttention(torch.autograd.Function):
         q, k, v, out, cu_seqlens = ctx.saved_tensors
         dq, dk, dv = _extension().areno_attention_backward(
             grad_output.contiguous(), q.contiguous(), k.contiguous(), v.contiguous(), out.contiguous(),
-            cu_seqlens.contiguous(), None, None, ctx.window_left, ctx.softmax_scale,
+            cu_seqlens.contiguous(), None, None, ctx.window_left, ctx.softmax_scale, True,
         )  # fmt: skip
-        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None
+        # (the kernels round their fp32 sums to the inputs' dtype at the store: the casts of the reference's wrapper,
+        # ``areno/accel/attention.py:117-118`` there, without fp32 tensors in between)
+        return dq, dk, dv, None, None, None
 
 
 class _PagedDecode(torch.autograd.Function):
@@ -194,7 +196,7 @@ class _CausalAttention(torch.autograd.Function):
         start = torch.full((batch,), ctx.query_start, device=dev, dtype=torch.int32)
         dq, dk, dv = _extension().areno_attention_backward(
             _rows_of(grad_output), _rows_of(q), _rows_of(k), _rows_of(v), _rows_of(out), cu_q, cu_k, start,
-            ctx.window_left, ctx.softmax_scale,
+            ctx.window_left, ctx.softmax_scale, True,
         )  # fmt: skip
         dq = dq.view(batch, sq, heads, d).transpose(1, 2)
         dk = dk.view(batch, sk, heads, d).transpose(1, 2)

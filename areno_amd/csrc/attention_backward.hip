@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_rows_kern
   if (token >= p.cu_q[p.num_seqs]) {  // rows past the last sequence take part in nothing
 #pragma unroll
     for (int e = 0; e < EPL; ++e) {
-      if (grp == 0 && e < valid_e) p.grad_q[q_base + e] = 0.0f;
+      if (grp == 0 && e < valid_e) store_grad(p.grad_q, q_base + e, 0.0f, p.grad_dtype);
     }
     return;
   }
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_rows_kern
 #pragma unroll
   for (int e = 0; e < EPL; ++e) {
     const float total = groups_sum(acc[e]);
-    if (grp == 0 && e < valid_e) p.grad_q[q_base + e] = total * p.scale;
+    if (grp == 0 && e < valid_e) store_grad(p.grad_q, q_base + e, total * p.scale, p.grad_dtype);
   }
 }
 
@@ -254,8 +254,8 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void attention_backward_keys_kern
     const float tk = groups_sum(dk[e]);
     const float tv = groups_sum(dv[e]);
     if (grp == 0 && e < valid_e) {
-      p.grad_k[k_base + e] = tk * p.scale;
-      p.grad_v[k_base + e] = tv;
+      store_grad(p.grad_k, k_base + e, tk * p.scale, p.grad_dtype);
+      store_grad(p.grad_v, k_base + e, tv, p.grad_dtype);
     }
   }
 }
@@ -294,8 +294,24 @@ extern "C" int areno_hip_attention_backward(const void* grad_out, const void* q,
                                             const int32_t* cu_seqlens_k, const int32_t* context_lens, int32_t num_seqs,
                                             int32_t window_left, float softmax_scale, void* workspace,
                                             size_t workspace_bytes, void* stream) {
+  return areno_hip_attention_backward_typed(grad_out, q, k, v, out, grad_q, grad_k, grad_v, ARENO_DT_F32, dtype, q_tokens,
+                                            k_tokens, q_heads, kv_heads, head_dim, cu_seqlens_q, cu_seqlens_k,
+                                            context_lens, num_seqs, window_left, softmax_scale, workspace,
+                                            workspace_bytes, stream);
+}
+
+extern "C" int areno_hip_attention_backward_typed(const void* grad_out, const void* q, const void* k, const void* v,
+                                                  const void* out, void* grad_q, void* grad_k, void* grad_v,
+                                                  int32_t grad_dtype, int32_t dtype, int64_t q_tokens, int64_t k_tokens,
+                                                  int32_t q_heads, int32_t kv_heads, int32_t head_dim,
+                                                  const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                                  const int32_t* context_lens, int32_t num_seqs, int32_t window_left,
+                                                  float softmax_scale, void* workspace, size_t workspace_bytes,
+                                                  void* stream) {
   using namespace areno;
   const char* op = "areno_hip_attention_backward";
+  if (grad_dtype != ARENO_DT_F32 && grad_dtype != dtype)
+    return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: gradients come in f32 or in the inputs' type", op);
   if (q_tokens < 0 || k_tokens < 0 || num_seqs < 1 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0)
     return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: sizes out of range or q_heads not a multiple of kv_heads", op);
   if (dtype != ARENO_DT_F32 && dtype != ARENO_DT_F16 && dtype != ARENO_DT_BF16)
@@ -308,7 +324,8 @@ extern "C" int areno_hip_attention_backward(const void* grad_out, const void* q,
   if (grad_out == nullptr || q == nullptr || k == nullptr || v == nullptr || out == nullptr || grad_q == nullptr ||
       grad_k == nullptr || grad_v == nullptr || cu_seqlens_q == nullptr)
     return fail(ARENO_ERR_INVALID_ARGUMENT, "%s: tensor pointer is NULL", op);
-  for (const void* ptr : {grad_out, q, k, v, out}) {
+  for (const void* ptr : {grad_out, q, k, v, out, static_cast<const void*>(grad_q), static_cast<const void*>(grad_k),
+                          static_cast<const void*>(grad_v)}) {
     if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return fail(ARENO_ERR_UNSUPPORTED, "%s: tensors must be 16-byte aligned", op);
   }
   const size_t need = areno_hip_attention_backward_workspace_bytes(q_tokens, q_heads);
@@ -340,6 +357,7 @@ extern "C" int areno_hip_attention_backward(const void* grad_out, const void* q,
   p.window_left = window_left;
   p.head_dim = head_dim;
   p.dtype = dtype;
+  p.grad_dtype = grad_dtype;
   p.scale = softmax_scale;
   p.scale_log2e = softmax_scale * kLog2e;
   // 16-bit inputs at head dims 64 and 128 run on the matrix cores (ARENO_BACKWARD_KERNEL=valu: a diagnosis switch

@@ -333,11 +333,10 @@ __global__ __launch_bounds__(kBmThreads, 2) void bwd_mfma_dq_kernel(BwdParams p)
       const float l_tot = rows_sum(l_lane[cb]);
       if (live[cb]) {
         const float f = l_tot > 0.0f ? p.scale / l_tot : 0.0f;
-        float* dst = p.grad_q + row_elem[cb] + 4 * lk;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-          *reinterpret_cast<float4_t*>(dst + 16 * nb) =
-              float4_t{acc[cb][nb][0] * f, acc[cb][nb][1] * f, acc[cb][nb][2] * f, acc[cb][nb][3] * f};
+          store_grad4(p.grad_q, row_elem[cb] + 4 * lk + 16 * nb, acc[cb][nb][0] * f, acc[cb][nb][1] * f,
+                      acc[cb][nb][2] * f, acc[cb][nb][3] * f, p.grad_dtype);
         }
         if (lk == 0) {
           float* st = p.row_stats + (row[cb] * p.q_heads + h) * 2;
@@ -626,13 +625,12 @@ __global__ __launch_bounds__((DkvShape<D, KR, P>::kThreads), (DkvShape<D, KR, P>
 
     // every gradient element is written, also the zeros of keys no query sees
     if (part == 0 && row_exists) {
-      float* dk = p.grad_k + row_elem + 4 * lk;
-      float* dv = p.grad_v + row_elem + 4 * lk;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
-        *reinterpret_cast<float4_t*>(dk + 16 * nb) =
-            float4_t{acc_k[nb][0] * p.scale, acc_k[nb][1] * p.scale, acc_k[nb][2] * p.scale, acc_k[nb][3] * p.scale};
-        *reinterpret_cast<float4_t*>(dv + 16 * nb) = acc_v[nb];
+        const int64_t at_elem = row_elem + 4 * lk + 16 * nb;
+        store_grad4(p.grad_k, at_elem, acc_k[nb][0] * p.scale, acc_k[nb][1] * p.scale, acc_k[nb][2] * p.scale,
+                    acc_k[nb][3] * p.scale, p.grad_dtype);
+        store_grad4(p.grad_v, at_elem, acc_v[nb][0], acc_v[nb][1], acc_v[nb][2], acc_v[nb][3], p.grad_dtype);
       }
     }
   }

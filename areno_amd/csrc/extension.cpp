@@ -618,11 +618,13 @@ std::vector<at::Tensor> block_tables_prefill_slots(at::Tensor table, at::Tensor 
 }
 
 // Backward of the varlen / dense ops.  q / grad_out / out: (Tq, Hq, D); k / v: (Tk, Hkv, D); returns fp32 gradients
-// like the reference's launchers (attention.cu:786-811, 898-925 there).
+// like the reference's launchers (attention.cu:786-811, 898-925 there), or, with `grads_in_input_dtype`, the same
+// sums rounded once to the inputs' type by the kernels (what the reference's autograd functions make of the fp32
+// gradients with a cast each).
 std::vector<at::Tensor> attention_backward(at::Tensor grad_out, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor out,
                                            at::Tensor cu_q, c10::optional<at::Tensor> cu_k,
                                            c10::optional<at::Tensor> context_lens, int64_t window_left,
-                                           double softmax_scale) {
+                                           double softmax_scale, bool grads_in_input_dtype) {
   const char* op = "areno_attention_backward";
   for (const at::Tensor* t : {&grad_out, &q, &k, &v, &out}) {
     TORCH_CHECK(t->is_cuda(), op, " tensors must be CUDA");
@@ -644,13 +646,14 @@ std::vector<at::Tensor> attention_backward(at::Tensor grad_out, at::Tensor q, at
   if (cu_k.has_value()) check_i32(*cu_k, num_seqs + 1, "cu_seqlens_k");
   if (context_lens.has_value()) check_i32(*context_lens, num_seqs, "context_lens");
   const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(device_of(q));
-  const auto fopts = q.options().dtype(at::kFloat);
+  const auto fopts = grads_in_input_dtype ? q.options() : q.options().dtype(at::kFloat);
+  const int32_t grad_dtype = grads_in_input_dtype ? dtype_code(q, op, "q") : static_cast<int32_t>(ARENO_DT_F32);
   at::Tensor dq = at::empty(q.sizes(), fopts), dk = at::empty(k.sizes(), fopts), dv = at::empty(v.sizes(), fopts);
   const size_t ws_bytes = areno_hip_attention_backward_workspace_bytes(q.size(0), static_cast<int32_t>(q.size(1)));
   at::Tensor workspace = at::empty({static_cast<int64_t>(ws_bytes)}, q.options().dtype(at::kByte));
-  const int status = areno_hip_attention_backward(
-      grad_out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dq.data_ptr<float>(),
-      dk.data_ptr<float>(), dv.data_ptr<float>(), dtype_code(q, op, "q"), q.size(0), k.size(0),
+  const int status = areno_hip_attention_backward_typed(
+      grad_out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+      dv.data_ptr(), grad_dtype, dtype_code(q, op, "q"), q.size(0), k.size(0),
       static_cast<int32_t>(q.size(1)), static_cast<int32_t>(k.size(1)), static_cast<int32_t>(q.size(2)),
       cu_q.data_ptr<int32_t>(), cu_k.has_value() ? cu_k->data_ptr<int32_t>() : nullptr,
       context_lens.has_value() ? context_lens->data_ptr<int32_t>() : nullptr, static_cast<int32_t>(num_seqs),

@@ -417,6 +417,19 @@ int areno_hip_attention_backward(const void* grad_out, const void* q, const void
                                  const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* context_lens,
                                  int32_t num_seqs, int32_t window_left, float softmax_scale, void* workspace,
                                  size_t workspace_bytes, void* stream);
+/*
+ * The same with the gradients in a type of the caller's choice: grad_dtype = ARENO_DT_F32 (the call above), or
+ * = dtype for 16-bit inputs: the fp32 sums are rounded once, at the store, to what the reference's autograd
+ * functions produce by casting the fp32 gradients afterwards (areno/accel/attention.py:117-118,182-183) -- without the
+ * fp32 tensors and the three cast kernels.  grad_q, grad_k, grad_v: 16-byte aligned.  No counterpart in the
+ * reference's extension (there the cast is Python's).
+ */
+int areno_hip_attention_backward_typed(const void* grad_out, const void* q, const void* k, const void* v, const void* out,
+                                       void* grad_q, void* grad_k, void* grad_v, int32_t grad_dtype, int32_t dtype,
+                                       int64_t q_tokens, int64_t k_tokens, int32_t q_heads, int32_t kv_heads,
+                                       int32_t head_dim, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                       const int32_t* context_lens, int32_t num_seqs, int32_t window_left,
+                                       float softmax_scale, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * ---- Diagnostics: not part of any caller's contract -------------------------------------------------------------------
