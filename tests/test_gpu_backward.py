@@ -165,3 +165,24 @@ def test_decode_backward_recomputes_like_the_reference(kv, window_left):
         live = set(w.block_table.cpu().flatten().tolist())
         untouched = [b for b in range(kc.shape[0]) if b not in live]
         assert float(kc.grad[untouched].abs().max()) == 0.0, "pages no row lists must get no gradient"
+
+
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float16, 64), (torch.bfloat16, 96), (torch.float32, 64)])
+def test_gradients_in_the_input_dtype_are_the_fp32_gradients_rounded_once(dtype, d):
+    """The extension's backward with fp32 gradients (the reference launchers' contract) and with gradients in the
+    inputs' dtype (what the autograd functions ask for): the second is the first cast, bit for bit, on the
+    matrix-core kernels (head dims 64 / 128) and on the vector-ALU ones (96; fp32 inputs)."""
+    from areno_amd.accel.attention import _extension
+
+    g = torch.Generator().manual_seed(d)
+    lens = [70, 1, 129, 300]
+    t, hq, hkv = sum(lens), 6, 2
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=DEV)
+    q, go = (torch.randn(t, hq, d, generator=g).to(dtype).to(DEV) for _ in range(2))
+    k, v = (torch.randn(t, hkv, d, generator=g).to(dtype).to(DEV) for _ in range(2))
+    out = ops.areno_varlen_causal_attention(q, k, v, cu)
+    wide = _extension().areno_attention_backward(go, q, k, v, out, cu, None, None, -1, d**-0.5, False)
+    typed = _extension().areno_attention_backward(go, q, k, v, out, cu, None, None, -1, d**-0.5, True)
+    for a, b, name in zip(wide, typed, ("dq", "dk", "dv")):
+        assert a.dtype == torch.float32 and b.dtype == dtype
+        assert torch.equal(a.to(dtype), b), f"{name} {dtype} d={d}"
