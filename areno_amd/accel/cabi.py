@@ -107,6 +107,8 @@ def lib() -> ctypes.CDLL:
         handle.areno_hip_prefill_workspace_bytes.restype = _SZ
         handle.areno_hip_prefill_workspace_bytes.argtypes = [_I32, _I32]
         handle.areno_hip_probe_stream_read.argtypes = [_P, _P, _P, _I64, _I32, _I32, _P, _P]
+        handle.areno_hip_probe_mfma_rate.restype = _I64
+        handle.areno_hip_probe_mfma_rate.argtypes = [_I32, _I32, _P, _P]
         handle.areno_hip_block_tables_init.argtypes = [_P, _P]
         handle.areno_hip_block_tables_reserve.argtypes = [_P, _P, _P, _I32, _P]
         handle.areno_hip_block_tables_ensure_decode.argtypes = [_P, _P, _P, _I32, _P]
@@ -233,6 +235,16 @@ def probe_stream_read(pool_a, pool_b, page_bytes: int, sink, page_ids=None, stre
                                             current_stream_ptr() if stream is None else stream),
           "areno_hip_probe_stream_read")  # fmt: skip
     return pages * page_bytes * (1 if pool_b is None else 2)
+
+
+def probe_mfma_rate(shape: int, iters: int, sink, stream=None) -> int:
+    """``areno_hip_probe_mfma_rate``: one launch of independent matrix products of a shape (0: 16 x 16 x 32 bf16,
+    1: 32 x 32 x 16 bf16, 2 / 3: the same in f16); returns the launch's floating-point operations."""
+    flops = int(lib().areno_hip_probe_mfma_rate(int(shape), int(iters), sink.data_ptr(),
+                                                current_stream_ptr() if stream is None else stream))  # fmt: skip
+    if flops < 0:
+        check(-1, "areno_hip_probe_mfma_rate")
+    return flops
 
 
 def prefill_workspace_bytes(kv_heads: int, head_dim: int) -> int:

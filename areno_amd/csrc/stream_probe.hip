@@ -53,8 +53,74 @@ __global__ __launch_bounds__(kProbeWaves* kWave, 2) void stream_read_kernel(cons
   if (fold == 0x9e3779b9u) sink[0] = fold;  // practically never: the store only keeps the loads alive
 }
 
+// Measurement aid: the rate at which the matrix cores take one shape of product when nothing else is asked of them.
+// Every wave issues `iters` rounds of independent products on register operands (8 accumulators of 16 x 16, or 4 of
+// 32 x 32: the same 32 accumulation registers per lane); 1 024 workgroups of four waves.
+typedef __attribute__((ext_vector_type(8))) __bf16 probe_bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 probe_f16x8;
+typedef __attribute__((ext_vector_type(4))) float probe_f32x4;
+typedef __attribute__((ext_vector_type(16))) float probe_f32x16;
+constexpr int kRateWorkgroups = 1024;
+
+template <int SHAPE>  // 0: 16 x 16 x 32 bf16, 1: 32 x 32 x 16 bf16, 2: 16 x 16 x 32 f16, 3: 32 x 32 x 16 f16
+__global__ __launch_bounds__(kProbeWaves* kWave) void mfma_rate_kernel(int iters, float* sink) {
+  probe_bf16x8 a, b;
+  probe_f16x8 ah, bh;
+  for (int i = 0; i < 8; ++i) {
+    a[i] = static_cast<__bf16>(threadIdx.x * 0.001f + i);
+    b[i] = static_cast<__bf16>(threadIdx.x * 0.002f - i);
+    ah[i] = static_cast<_Float16>(threadIdx.x * 0.001f + i);
+    bh[i] = static_cast<_Float16>(threadIdx.x * 0.002f - i);
+  }
+  probe_f32x4 small[8];
+  probe_f32x16 big[4];
+  for (int i = 0; i < 8; ++i) small[i] = probe_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int i = 0; i < 4; ++i) {
+    for (int j = 0; j < 16; ++j) big[i][j] = 0.0f;
+  }
+  for (int it = 0; it < iters; ++it) {
+    if constexpr (SHAPE == 0) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) small[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, small[i], 0, 0, 0);
+    } else if constexpr (SHAPE == 1) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) big[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, big[i], 0, 0, 0);
+    } else if constexpr (SHAPE == 2) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) small[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bh, small[i], 0, 0, 0);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) big[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh, big[i], 0, 0, 0);
+    }
+  }
+  float fold = 0.0f;
+  for (int i = 0; i < 8; ++i) fold += small[i][0] + small[i][3];
+  for (int i = 0; i < 4; ++i) fold += big[i][0] + big[i][15];
+  if (fold == 12345.678f) sink[0] = fold;  // practically never: the store only keeps the products alive
+}
+
 }  // namespace
 }  // namespace areno
+
+extern "C" int64_t areno_hip_probe_mfma_rate(int32_t shape, int32_t iters, void* sink, void* stream) {
+  const char* op = "areno_hip_probe_mfma_rate";
+  if (shape < 0 || shape > 3 || iters < 1 || sink == nullptr) {
+    areno::fail(ARENO_ERR_INVALID_ARGUMENT, "%s: shape 0..3, iters >= 1 and a sink", op);
+    return -1;
+  }
+  const dim3 grid(areno::kRateWorkgroups), block(areno::kProbeWaves * areno::kWave);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* out = static_cast<float*>(sink);
+  switch (shape) {
+    case 0: hipLaunchKernelGGL(areno::mfma_rate_kernel<0>, grid, block, 0, s, iters, out); break;
+    case 1: hipLaunchKernelGGL(areno::mfma_rate_kernel<1>, grid, block, 0, s, iters, out); break;
+    case 2: hipLaunchKernelGGL(areno::mfma_rate_kernel<2>, grid, block, 0, s, iters, out); break;
+    default: hipLaunchKernelGGL(areno::mfma_rate_kernel<3>, grid, block, 0, s, iters, out); break;
+  }
+  if (areno::check_launch(op) != ARENO_OK) return -1;
+  // floating-point operations of the launch: 2 x 16 384 multiply-adds per round and wave in either shape
+  return static_cast<int64_t>(areno::kRateWorkgroups) * areno::kProbeWaves * iters * (8LL * 16 * 16 * 32 * 2);
+}
 
 extern "C" int areno_hip_probe_stream_read(const void* base_a, const void* base_b, const int32_t* page_ids, int64_t pages,
                                            int32_t page_bytes, int32_t prefetch_ids, void* sink, void* stream) {

@@ -664,8 +664,35 @@ def measure_prefill(w, iters=20):
             "bound": "mfma", "kernel": "prefill_mfma_kernel", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": PROFILED_TRAFFIC_BYTES.get(w.name),
             "traffic_source": PROFILED_TRAFFIC_SOURCE["prefill"],
+            # what the matrix cores sustain on this part when they are asked for nothing but products of one shape
+            # (areno_hip_probe_mfma_rate, timed here): the kernel's products are 16 x 16 x 32
+            **measure_mfma_ceilings(w.q.device, tflops),
         },  # fmt: skip
     }
+
+
+def measure_mfma_ceilings(device, kernel_tflops, iters=40000, samples=5):
+    """TFLOP/s of launches of independent matrix products on register operands, per shape of product (f16, the type
+    the prefill kernel computes fp8 pages in; bf16 next to it), median of a few launches."""
+    import torch
+
+    from areno_amd.accel import cabi
+
+    sink = torch.zeros(4, dtype=torch.float32, device=device)
+    rates = {}
+    for name, shape in (("16x16x32_f16", 2), ("32x32x16_f16", 3), ("16x16x32_bf16", 0), ("32x32x16_bf16", 1)):
+        cabi.probe_mfma_rate(shape, 1000, sink)
+        torch.cuda.synchronize()
+        got = []
+        for _ in range(samples):
+            first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            first.record()
+            flops = cabi.probe_mfma_rate(shape, iters, sink)
+            last.record()
+            torch.cuda.synchronize()
+            got.append(flops / (first.elapsed_time(last) * 1e-3) / 1e12)
+        rates[name] = statistics.median(got)
+    return {"mfma_ceiling_tflops": rates, "frac_of_16x16x32_f16_ceiling": kernel_tflops / rates["16x16x32_f16"]}
 
 
 def wave_trace(w, launches=18):

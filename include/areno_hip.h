@@ -433,8 +433,8 @@ int areno_hip_attention_backward_typed(const void* grad_out, const void* q, cons
 
 /*
  * ---- Diagnostics: not part of any caller's contract -------------------------------------------------------------------
- * The two entry points below have no counterpart in the reference and no production caller: the first exists for a
- * test of this library, the second for its benchmark.
+ * The entry points below have no counterpart in the reference and no production caller: the first exists for a
+ * test of this library, the others for its benchmark.
  *
  * areno_hip_debug_set_rope_tokens_per_launch: caps the tokens one launch of areno_hip_qk_norm_rope_cache_write takes
  * (0 = only the kernel's own limit) so that its walk over token ranges can be tested at small sizes.  Returns the
@@ -450,10 +450,17 @@ int areno_hip_attention_backward_typed(const void* grad_out, const void* q, cons
  * V pages side by side would offer.
  *   base_a, base_b  device, 16-byte aligned;  page_bytes a multiple of 1024;  sink  device, >= 4 bytes (written
  *                   practically never)
+ *
+ * areno_hip_probe_mfma_rate: 1 024 workgroups of four waves issue `iters` rounds of independent matrix products on
+ * register operands and nothing else: shape 0 = 16 x 16 x 32 bf16 (8 products a round), 1 = 32 x 32 x 16 bf16 (4 a
+ * round), 2 / 3 the same in f16.  Returns the floating-point operations of the launch (-1 on error); timed by the
+ * caller, that is the rate the matrix cores sustain for the shape, which the kernels' rates are compared with
+ * (bench.py).  sink as above.
  */
 int64_t areno_hip_debug_set_rope_tokens_per_launch(int64_t tokens);
 int areno_hip_probe_stream_read(const void* base_a, const void* base_b, const int32_t* page_ids, int64_t pages,
                                 int32_t page_bytes, int32_t prefetch_ids, void* sink, void* stream);
+int64_t areno_hip_probe_mfma_rate(int32_t shape, int32_t iters, void* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -35,7 +35,7 @@ def test_header_declares_the_expected_entry_points():
                      "areno_hip_block_tables_init", "areno_hip_block_tables_reserve",
                      "areno_hip_block_tables_ensure_decode", "areno_hip_block_tables_release",
                      "areno_hip_block_tables_gather", "areno_hip_block_tables_decode_step",
-                     "areno_hip_block_tables_prefill_slots", "areno_hip_attention_backward", "areno_hip_attention_backward_typed",
+                     "areno_hip_block_tables_prefill_slots", "areno_hip_attention_backward", "areno_hip_attention_backward_typed", "areno_hip_probe_mfma_rate",
                      "areno_hip_attention_backward_workspace_bytes", "areno_hip_paged_decode_plan",
                      "areno_hip_paged_decode_plan_bytes", "areno_hip_paged_decode_planned", "areno_hip_rope_rows",
                      "areno_hip_rope_rows_bytes", "areno_hip_qk_norm_rope_cache_write_rows"):  # fmt: skip
